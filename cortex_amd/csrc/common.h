@@ -1,0 +1,163 @@
+// common.h -- shared host/device helpers of libcortex_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <type_traits>
+
+#include "../../include/cortex_hip.h"
+
+namespace cthip {
+
+// ------------------------------------------------------------------ errors
+
+// Thread-local message read back by ct_last_error().
+char* err_buf();
+const char** last_kernel_slot();
+int set_error(int code, const char* fmt, ...);
+bool debug_sync();
+
+// Scratch memory owned by the library, one growing block per (device, stream).
+// Kernels of one stream run in order, so consecutive calls may reuse it.
+int stream_scratch(hipStream_t s, size_t bytes, void** out);
+void release_stream_scratch(hipStream_t s);
+
+inline void note_kernel(const char* name) { *last_kernel_slot() = name; }
+
+#define CT_HIP(expr)                                                                          \
+  do {                                                                                        \
+    hipError_t e__ = (expr);                                                                  \
+    if (e__ != hipSuccess)                                                                    \
+      return ::cthip::set_error(CT_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e__));  \
+  } while (0)
+
+#define CT_REQUIRE(cond, ...)                                              \
+  do {                                                                     \
+    if (!(cond)) return ::cthip::set_error(CT_ERR_INVALID, __VA_ARGS__);   \
+  } while (0)
+
+// Called after every kernel launch: surfaces launch errors and, in debug-sync
+// mode, faults of the kernel itself.
+inline int after_launch(hipStream_t s) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(CT_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+  if (debug_sync()) {
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return set_error(CT_ERR_HIP, "kernel failed: %s", hipGetErrorString(e));
+  }
+  return CT_OK;
+}
+
+// ------------------------------------------------------------------ datatypes
+
+inline int dtype_size(int dt) {
+  switch (dt) {
+    case CT_I8: case CT_U8: return 1;
+    case CT_I16: return 2;
+    case CT_I32: case CT_F32: return 4;
+    case CT_I64: case CT_F64: return 8;
+    default: return 0;
+  }
+}
+
+template <class T> struct acc_of {
+  using type = typename std::conditional<std::is_floating_point<T>::value, double, int64_t>::type;
+};
+
+// Runs `body` with T bound to the C type of datatype `dt`.
+#define CT_DISPATCH_DTYPE(dt, ...)                                              \
+  switch (dt) {                                                                 \
+    case CT_I8: { using T = int8_t; __VA_ARGS__; } break;                       \
+    case CT_I16: { using T = int16_t; __VA_ARGS__; } break;                     \
+    case CT_I32: { using T = int32_t; __VA_ARGS__; } break;                     \
+    case CT_I64: { using T = int64_t; __VA_ARGS__; } break;                     \
+    case CT_F32: { using T = float; __VA_ARGS__; } break;                       \
+    case CT_F64: { using T = double; __VA_ARGS__; } break;                      \
+    case CT_U8: { using T = uint8_t; __VA_ARGS__; } break;                      \
+    default: return ::cthip::set_error(CT_ERR_INVALID, "unknown datatype %d", (int)(dt)); \
+  }
+
+// ------------------------------------------------------------------ JVM value semantics
+// The CPU backend of the reference is JVM code compiled under *unchecked-math*
+// (src/cortex/compute/cpu/tensor_math.clj:28): its casts are Java primitive
+// conversions (src/cortex/compute/cpu/driver.clj:149-157).  These helpers give
+// the same results on the device and on the host.
+
+#define CT_HD __host__ __device__ __forceinline__
+
+CT_HD int32_t jvm_d2i(double v) {  // NaN -> 0, saturates, rounds toward zero
+  int32_t r = (int32_t)(v < 2147483647.0 ? (v > -2147483648.0 ? v : -2147483648.0) : 2147483647.0);
+  return (v != v) ? 0 : r;
+}
+CT_HD int64_t jvm_d2l(double v) {
+  const double hi = 9223372036854775808.0;
+  if (v != v) return 0;
+  if (v >= hi) return INT64_MAX;
+  if (v <= -hi) return INT64_MIN;
+  return (int64_t)v;
+}
+
+// Result of a long computation stored into T.
+template <class T> CT_HD T jvm_cast(int64_t v) {
+  if constexpr (std::is_floating_point<T>::value) return (T)v;
+  else return (T)(uint64_t)v;
+}
+// Result of a double computation stored into T; byte and short go through int.
+template <class T> CT_HD T jvm_cast(double v) {
+  if constexpr (std::is_same<T, double>::value) return v;
+  else if constexpr (std::is_same<T, float>::value) return (float)v;
+  else if constexpr (std::is_same<T, int64_t>::value) return jvm_d2l(v);
+  else return (T)(uint32_t)jvm_d2i(v);
+}
+template <class T, class S> CT_HD T jvm_convert(S s) {
+  if constexpr (std::is_same<T, S>::value) return s;
+  else if constexpr (std::is_floating_point<S>::value) return jvm_cast<T>((double)s);
+  else return jvm_cast<T>((int64_t)s);
+}
+
+// Wrapping long arithmetic / plain double arithmetic under one name.
+CT_HD int64_t w_mul(int64_t a, int64_t b) { return (int64_t)((uint64_t)a * (uint64_t)b); }
+CT_HD int64_t w_add(int64_t a, int64_t b) { return (int64_t)((uint64_t)a + (uint64_t)b); }
+CT_HD int64_t w_sub(int64_t a, int64_t b) { return (int64_t)((uint64_t)a - (uint64_t)b); }
+CT_HD int64_t w_neg(int64_t a) { return (int64_t)(0ull - (uint64_t)a); }
+CT_HD double w_mul(double a, double b) { return a * b; }
+CT_HD double w_add(double a, double b) { return a + b; }
+CT_HD double w_sub(double a, double b) { return a - b; }
+CT_HD double w_neg(double a) { return -a; }
+
+// Casting (/ a b) of two longs to T: exact quotients are Longs (truncating
+// cast); inexact ones are Ratios whose intValue saturates and whose longValue
+// truncates toward zero.  Division by zero yields 0 on the device (the
+// reference throws ArithmeticException; a kernel cannot).
+template <class T> CT_HD T jvm_ratio_cast(int64_t n, int64_t d) {
+  if (d == 0) return (T)0;
+  if (n == INT64_MIN && d == -1) return jvm_cast<T>(n);
+  const int64_t q = n / d;
+  if (std::is_same<T, int64_t>::value || q * d == n) return jvm_cast<T>(q);
+  return jvm_cast<T>((double)q);
+}
+
+// ------------------------------------------------------------------ 32-bit division by an invariant
+
+// q = n / d for 0 <= n < 2^31, 1 <= d < 2^31, with one multiply-high.
+struct FastDiv {
+  uint32_t d, m, s;
+  FastDiv() : d(1), m(0), s(0) {}
+  explicit FastDiv(uint32_t div) : d(div) {
+    for (s = 0; s < 32; ++s)
+      if ((1u << s) >= d) break;
+    const uint64_t one = 1;
+    m = (uint32_t)(((one << 32) * ((one << s) - d)) / d + 1);
+  }
+  __device__ __forceinline__ uint32_t div(uint32_t n) const { return (__umulhi(n, m) + n) >> s; }
+  __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
+    q = div(n);
+    r = n - q * d;
+  }
+};
+
+}  // namespace cthip

@@ -1,0 +1,240 @@
+// driver.hip -- device, memory, stream and event entry points (the
+// cortex.compute.driver protocols, src/cortex/compute/driver.clj:46-203) plus
+// the library's error state.
+#include <atomic>
+#include <map>
+#include <mutex>
+
+#include "elementwise.h"
+#include "functors.h"
+
+namespace cthip {
+
+namespace {
+thread_local char g_err[512] = "";
+thread_local const char* g_kernel = "";
+std::atomic<int> g_debug_sync{0};
+}  // namespace
+
+char* err_buf() { return g_err; }
+const char** last_kernel_slot() { return &g_kernel; }
+bool debug_sync() { return g_debug_sync.load(std::memory_order_relaxed) != 0; }
+
+namespace {
+struct ScratchKey {
+  int device;
+  hipStream_t stream;
+  bool operator<(const ScratchKey& o) const { return device != o.device ? device < o.device : stream < o.stream; }
+};
+struct ScratchBlock { void* ptr; size_t bytes; };
+std::mutex g_scratch_mutex;
+std::map<ScratchKey, ScratchBlock> g_scratch;
+}  // namespace
+
+int stream_scratch(hipStream_t s, size_t bytes, void** out) {
+  int dev = 0;
+  CT_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  ScratchBlock& b = g_scratch[ScratchKey{dev, s}];
+  if (b.bytes < bytes) {
+    if (b.ptr) {
+      // earlier kernels of this stream may still be reading the old block
+      CT_HIP(hipStreamSynchronize(s));
+      CT_HIP(hipFree(b.ptr));
+      b.ptr = nullptr;
+      b.bytes = 0;
+    }
+    size_t want = bytes < (size_t(1) << 20) ? (size_t(1) << 20) : bytes;
+    CT_HIP(hipMalloc(&b.ptr, want));
+    b.bytes = want;
+  }
+  *out = b.ptr;
+  return CT_OK;
+}
+
+void release_stream_scratch(hipStream_t s) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  auto it = g_scratch.find(ScratchKey{dev, s});
+  if (it == g_scratch.end()) return;
+  if (it->second.ptr) (void)hipFree(it->second.ptr);
+  g_scratch.erase(it);
+}
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+}  // namespace cthip
+
+using namespace cthip;
+
+extern "C" {
+
+const char* ct_last_error(void) { return err_buf(); }
+const char* ct_last_kernel(void) { return *last_kernel_slot(); }
+
+int ct_set_debug_sync(int on) {
+  g_debug_sync.store(on ? 1 : 0);
+  return CT_OK;
+}
+
+int ct_device_count(int* n) {
+  CT_REQUIRE(n != nullptr, "ct_device_count: null output");
+  CT_HIP(hipGetDeviceCount(n));
+  return CT_OK;
+}
+
+int ct_set_device(int device) {
+  CT_HIP(hipSetDevice(device));
+  return CT_OK;
+}
+
+int ct_get_device(int* device) {
+  CT_REQUIRE(device != nullptr, "ct_get_device: null output");
+  CT_HIP(hipGetDevice(device));
+  return CT_OK;
+}
+
+int ct_memory_info(size_t* free_bytes, size_t* total_bytes) {
+  CT_REQUIRE(free_bytes && total_bytes, "ct_memory_info: null output");
+  CT_HIP(hipMemGetInfo(free_bytes, total_bytes));
+  return CT_OK;
+}
+
+int ct_malloc(void** ptr, size_t bytes) {
+  CT_REQUIRE(ptr != nullptr, "ct_malloc: null output");
+  *ptr = nullptr;
+  CT_HIP(hipMalloc(ptr, bytes ? bytes : 1));
+  return CT_OK;
+}
+
+int ct_free(void* ptr) {
+  if (ptr) CT_HIP(hipFree(ptr));
+  return CT_OK;
+}
+
+int ct_host_alloc(void** ptr, size_t bytes) {
+  CT_REQUIRE(ptr != nullptr, "ct_host_alloc: null output");
+  *ptr = nullptr;
+  CT_HIP(hipHostMalloc(ptr, bytes ? bytes : 1, hipHostMallocDefault));
+  return CT_OK;
+}
+
+int ct_host_free(void* ptr) {
+  if (ptr) CT_HIP(hipHostFree(ptr));
+  return CT_OK;
+}
+
+int ct_stream_create(void** stream) {
+  CT_REQUIRE(stream != nullptr, "ct_stream_create: null output");
+  hipStream_t s = nullptr;
+  CT_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = (void*)s;
+  return CT_OK;
+}
+
+int ct_stream_destroy(void* stream) {
+  if (stream) {
+    CT_HIP(hipStreamSynchronize((hipStream_t)stream));
+    release_stream_scratch((hipStream_t)stream);
+    CT_HIP(hipStreamDestroy((hipStream_t)stream));
+  }
+  return CT_OK;
+}
+
+int ct_stream_sync(void* stream) {
+  CT_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return CT_OK;
+}
+
+int ct_event_record(void** event, void* stream) {
+  CT_REQUIRE(event != nullptr, "ct_event_record: null output");
+  hipEvent_t e = nullptr;
+  CT_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  hipError_t rc = hipEventRecord(e, (hipStream_t)stream);
+  if (rc != hipSuccess) {
+    (void)hipEventDestroy(e);
+    return set_error(CT_ERR_HIP, "hipEventRecord failed: %s", hipGetErrorString(rc));
+  }
+  *event = (void*)e;
+  return CT_OK;
+}
+
+int ct_event_record_timed(void** event, void* stream) {
+  CT_REQUIRE(event != nullptr, "ct_event_record_timed: null output");
+  hipEvent_t e = nullptr;
+  CT_HIP(hipEventCreate(&e));
+  hipError_t rc = hipEventRecord(e, (hipStream_t)stream);
+  if (rc != hipSuccess) {
+    (void)hipEventDestroy(e);
+    return set_error(CT_ERR_HIP, "hipEventRecord failed: %s", hipGetErrorString(rc));
+  }
+  *event = (void*)e;
+  return CT_OK;
+}
+
+int ct_stream_wait_event(void* stream, void* event) {
+  CT_REQUIRE(event != nullptr, "ct_stream_wait_event: null event");
+  CT_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0));
+  return CT_OK;
+}
+
+int ct_event_sync(void* event) {
+  CT_REQUIRE(event != nullptr, "ct_event_sync: null event");
+  CT_HIP(hipEventSynchronize((hipEvent_t)event));
+  return CT_OK;
+}
+
+int ct_event_destroy(void* event) {
+  if (event) CT_HIP(hipEventDestroy((hipEvent_t)event));
+  return CT_OK;
+}
+
+int ct_event_elapsed_ms(void* start_event, void* stop_event, float* ms) {
+  CT_REQUIRE(start_event && stop_event && ms, "ct_event_elapsed_ms: null argument");
+  CT_HIP(hipEventElapsedTime(ms, (hipEvent_t)start_event, (hipEvent_t)stop_event));
+  return CT_OK;
+}
+
+int ct_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream) {
+  if (bytes == 0) return CT_OK;
+  CT_REQUIRE(dst && src, "ct_memcpy_async: null pointer");
+  hipMemcpyKind k;
+  switch (kind) {
+    case CT_COPY_HOST_TO_DEVICE: k = hipMemcpyHostToDevice; break;
+    case CT_COPY_DEVICE_TO_HOST: k = hipMemcpyDeviceToHost; break;
+    case CT_COPY_DEVICE_TO_DEVICE: k = hipMemcpyDeviceToDevice; break;
+    default: return set_error(CT_ERR_INVALID, "ct_memcpy_async: unknown copy kind %d", kind);
+  }
+  CT_HIP(hipMemcpyAsync(dst, src, bytes, k, (hipStream_t)stream));
+  if (debug_sync()) CT_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return CT_OK;
+}
+
+// PStream memset (src/cortex/compute/cuda/driver.clj:1020-1032): a typed fill.
+// It runs as a fill kernel for every value, zero included, so that it can be
+// recorded into a captured graph.
+int ct_memset(void* stream, void* buffer, int dtype, double value, int64_t n) {
+  CT_REQUIRE(n >= 0, "ct_memset: negative count");
+  if (n == 0) return CT_OK;
+  CT_REQUIRE(buffer != nullptr, "ct_memset: null buffer");
+  ct_dims d;
+  std::memset(&d, 0, sizeof(d));
+  d.ndim = 1;
+  d.shape[0] = n;
+  d.strides[0] = 1;
+  CT_DISPATCH_DTYPE(dtype, {
+    ConstantF<T> f{jvm_cast<T>(value)};
+    EwOperand ops[1] = {{buffer, &d, (int)sizeof(T), 0}};
+    return launch_elementwise(static_cast<hipStream_t>(stream), f, ops, n);
+  });
+  return CT_OK;
+}
+
+}  // extern "C"

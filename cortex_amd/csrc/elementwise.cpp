@@ -1,0 +1,138 @@
+// elementwise.cpp -- turns a Plan into kernel argument blocks (host only).
+#include "elementwise.h"
+
+#include <algorithm>
+
+namespace cthip {
+
+namespace {
+constexpr int64_t kLim31 = int64_t(1) << 31;
+
+void common_vec(const Plan& plan, const EwOperand* ops, VecArgs* a) {
+  const Canon& c = plan.canon;
+  std::memset(a, 0, sizeof(*a));
+  a->n_outer = c.nd - 1;
+  for (int d = 0; d + 1 < c.nd; ++d) a->outer_fd[d] = FastDiv((uint32_t)c.size[d + 1]);
+  for (int k = 0; k < plan.n_ops; ++k) {
+    a->ptr[k] = (char*)ops[k].ptr;
+    a->cbits[k] = ops[k].cbits;
+    if (!ops[k].ptr) a->const_mask |= 1u << k;
+    else if (c.stride[k][0] == 1) a->unit_mask |= 1u << k;
+    for (int d = 0; d + 1 < c.nd; ++d) a->outer_stride[k][d] = c.stride[k][d + 1];
+  }
+}
+}  // namespace
+
+int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_args, int* main_vec,
+                VecArgs* tail_args, bool* has_tail) {
+  const Canon& c = plan.canon;
+  const int64_t inner = c.size[0];
+  int64_t rows = 1;
+  for (int d = 1; d < c.nd; ++d) rows *= c.size[d];
+  *has_tail = false;
+
+  bool aligned = vmax > 1;
+  for (int k = 0; aligned && k < plan.n_ops; ++k) {
+    if (!ops[k].ptr || c.stride[k][0] != 1) continue;
+    if (((uintptr_t)ops[k].ptr % (uintptr_t)(vmax * ops[k].elem_size)) != 0) aligned = false;
+    for (int d = 1; aligned && d < c.nd; ++d)
+      if (c.stride[k][d] % vmax != 0) aligned = false;
+  }
+  if (aligned && c.nd > 1 && inner % vmax != 0) aligned = false;
+  if (aligned && c.nd == 1 && inner < vmax) aligned = false;
+
+  common_vec(plan, ops, main_args);
+  if (!aligned) {
+    *main_vec = 1;
+    main_args->inner_vecs = (uint32_t)std::min<int64_t>(inner, kLim31 - 1);
+    main_args->inner_fd = FastDiv(main_args->inner_vecs);
+    main_args->total_vecs = (uint64_t)inner * (uint64_t)rows;
+    return CT_OK;
+  }
+  *main_vec = vmax;
+  const int64_t inner_vecs = inner / vmax;
+  main_args->inner_vecs = (uint32_t)std::min<int64_t>(inner_vecs, kLim31 - 1);
+  main_args->inner_fd = FastDiv(main_args->inner_vecs);
+  main_args->total_vecs = (uint64_t)inner_vecs * (uint64_t)rows;
+  const int64_t tail = inner - inner_vecs * vmax;  // only possible when flat
+  if (tail > 0) {
+    *has_tail = true;
+    common_vec(plan, ops, tail_args);
+    for (int k = 0; k < plan.n_ops; ++k)
+      if (ops[k].ptr && c.stride[k][0] == 1)
+        tail_args->ptr[k] = (char*)ops[k].ptr + (inner_vecs * vmax) * ops[k].elem_size;
+    tail_args->inner_vecs = (uint32_t)tail;
+    tail_args->inner_fd = FastDiv((uint32_t)tail);
+    tail_args->total_vecs = (uint64_t)tail;
+  }
+  return CT_OK;
+}
+
+int prepare_tile(const Plan& plan, const EwOperand* ops, int ts, TileArgs* a, size_t* lds_bytes,
+                 uint32_t* grid) {
+  const Canon& c = plan.canon;
+  const int b = plan.tile_b;
+  std::memset(a, 0, sizeof(*a));
+  a->sizeA = (uint32_t)c.size[0];
+  a->sizeB = (uint32_t)c.size[b];
+  a->tilesA = (a->sizeA + ts - 1) / ts;
+  a->tilesB = (a->sizeB + ts - 1) / ts;
+  a->tilesA_fd = FastDiv(a->tilesA);
+  a->tilesB_fd = FastDiv(a->tilesB);
+  int64_t blocks = (int64_t)a->tilesA * a->tilesB;
+  int no = 0;
+  for (int d = 1; d < c.nd; ++d) {
+    if (d == b) continue;
+    a->outer_fd[no] = FastDiv((uint32_t)c.size[d]);
+    for (int k = 0; k < plan.n_ops; ++k) a->outer_stride[k][no] = c.stride[k][d];
+    blocks *= c.size[d];
+    ++no;
+  }
+  a->n_outer = no;
+  CT_REQUIRE(blocks < kLim31, "internal: tile grid too large");
+  *grid = (uint32_t)blocks;
+  size_t lds = 0;
+  for (int k = 0; k < plan.n_ops; ++k) {
+    a->ptr[k] = (char*)ops[k].ptr;
+    a->cbits[k] = ops[k].cbits;
+    a->strideA[k] = c.stride[k][0];
+    a->strideB[k] = c.stride[k][b];
+    if (!ops[k].ptr) a->const_mask |= 1u << k;
+    if (plan.via_lds[k]) {
+      a->lds_mask |= 1u << k;
+      lds += tile_slot_bytes((size_t)ops[k].elem_size, ts);
+    }
+  }
+  *lds_bytes = lds;
+  return CT_OK;
+}
+
+int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* a, bool* use64, uint32_t* grid) {
+  const GenPlan& g = plan.gen;
+  std::memset(a, 0, sizeof(*a));
+  a->n = plan.n;
+  a->nd = g.nd;
+  bool big = plan.n >= kLim31;
+  for (int d = 0; d < CT_MAX_DIMS; ++d) {
+    a->rmax[d] = g.rmax[d];
+    if (g.rmax[d] >= kLim31) big = true;
+  }
+  for (int k = 0; k < plan.n_ops; ++k) {
+    a->op[k] = g.op[k];
+    a->ptr[k] = (char*)ops[k].ptr;
+    a->cbits[k] = ops[k].cbits;
+    if (g.op[k].mode == 3) a->need_coords = 1;
+    if (g.op[k].ec >= kLim31 || g.op[k].amt >= kLim31) big = true;
+    for (int d = 0; d < CT_MAX_DIMS; ++d)
+      if (g.op[k].shape[d] >= kLim31) big = true;
+  }
+  for (int k = plan.n_ops; k < kMaxOps; ++k) a->op[k].mode = 4;
+  if (!big)
+    for (int d = 0; d < CT_MAX_DIMS; ++d) a->rmax_fd[d] = FastDiv((uint32_t)g.rmax[d]);
+  *use64 = big;
+  const int64_t blocks = (plan.n + kBlock - 1) / kBlock;
+  *grid = (uint32_t)std::min<int64_t>(blocks, 16384);
+  return CT_OK;
+}
+
+}  // namespace cthip

@@ -1,0 +1,447 @@
+// elementwise.h -- the three elementwise kernel families and their launcher.
+//
+// A functor F describes one scalar operation:
+//   static constexpr int NIN;              number of inputs, 0..3
+//   using Out, In0, In1, In2;              element types (unused inputs: any type)
+//   __device__ Out operator()(In0, In1, In2) const;
+// The launcher analyses the operands' dimensions (plan.h) and runs F through
+//   ew_vec_kernel   128-bit coalesced accesses along the innermost axis;
+//                   broadcast operands are read as wave-uniform scalars;
+//                   address arithmetic is done once per vector, not per element
+//   ew_tile_kernel  transposed inputs staged through a padded LDS tile so both
+//                   the reads and the writes are coalesced
+//   ew_gen_kernel   per-element addressing with the reference's address objects
+#pragma once
+
+#include "common.h"
+#include "plan.h"
+
+namespace cthip {
+
+template <class T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
+
+constexpr int kBlock = 256;
+
+template <class T> __device__ __forceinline__ T const_from_bits(uint64_t bits) {
+  T c;
+  __builtin_memcpy(&c, &bits, sizeof(T));
+  return c;
+}
+template <class T> inline uint64_t bits_of(T c) {
+  uint64_t b = 0;
+  std::memcpy(&b, &c, sizeof(T));
+  return b;
+}
+
+// ------------------------------------------------------------------ VEC
+
+struct VecArgs {
+  uint64_t total_vecs;
+  uint32_t inner_vecs;
+  FastDiv inner_fd;
+  int32_t n_outer;
+  FastDiv outer_fd[CT_MAX_DIMS - 1];
+  char* ptr[kMaxOps];
+  int64_t outer_stride[kMaxOps][CT_MAX_DIMS - 1];
+  uint32_t unit_mask;   // bit k: operand k is unit-stride along the inner axis
+  uint32_t const_mask;  // bit k: operand k is a scalar constant
+  uint64_t cbits[kMaxOps];
+};
+
+template <class T, int VEC>
+__device__ __forceinline__ Vec<T, VEC> vec_load(const VecArgs& a, int k, int64_t base, int64_t col) {
+  Vec<T, VEC> r;
+  if ((a.const_mask >> k) & 1u) {
+    const T c = const_from_bits<T>(a.cbits[k]);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) r.v[i] = c;
+  } else if ((a.unit_mask >> k) & 1u) {
+    r = *reinterpret_cast<const Vec<T, VEC>*>(reinterpret_cast<const T*>(a.ptr[k]) + base + col);
+  } else {
+    const T c = reinterpret_cast<const T*>(a.ptr[k])[base];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) r.v[i] = c;
+  }
+  return r;
+}
+
+template <class F, int VEC, int UNROLL>
+__global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs a) {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+
+  const uint64_t first = (uint64_t)blockIdx.x * (uint64_t)(kBlock * UNROLL) + threadIdx.x;
+  Vec<In0, VEC> x0[UNROLL];
+  Vec<In1, VEC> x1[UNROLL];
+  Vec<In2, VEC> x2[UNROLL];
+  int64_t dst[UNROLL];
+  bool live[UNROLL];
+
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const uint64_t v = first + (uint64_t)u * kBlock;
+    live[u] = v < a.total_vecs;
+    if (!live[u]) continue;
+    int64_t off[kMaxOps] = {0, 0, 0, 0};
+    int64_t col;
+    if (a.n_outer == 0) {
+      col = (int64_t)v * VEC;
+    } else {
+      uint32_t row, cv;
+      a.inner_fd.divmod((uint32_t)v, row, cv);
+      col = (int64_t)cv * VEC;
+      for (int d = 0; d < a.n_outer; ++d) {
+        uint32_t q, r;
+        a.outer_fd[d].divmod(row, q, r);
+        row = q;
+#pragma unroll
+        for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
+      }
+    }
+    dst[u] = off[0] + col;
+    if constexpr (NIN >= 1) x0[u] = vec_load<In0, VEC>(a, 1, off[1], col);
+    if constexpr (NIN >= 2) x1[u] = vec_load<In1, VEC>(a, 2, off[2], col);
+    if constexpr (NIN >= 3) x2[u] = vec_load<In2, VEC>(a, 3, off[3], col);
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    if (!live[u]) continue;
+    Vec<Out, VEC> r;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      In0 p0{};
+      In1 p1{};
+      In2 p2{};
+      if constexpr (NIN >= 1) p0 = x0[u].v[i];
+      if constexpr (NIN >= 2) p1 = x1[u].v[i];
+      if constexpr (NIN >= 3) p2 = x2[u].v[i];
+      r.v[i] = f(p0, p1, p2);
+    }
+    *reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(a.ptr[0]) + dst[u]) = r;
+  }
+}
+
+// ------------------------------------------------------------------ TILE
+
+struct TileArgs {
+  uint32_t sizeA, sizeB, tilesA, tilesB;
+  FastDiv tilesA_fd, tilesB_fd;
+  int32_t n_outer;
+  FastDiv outer_fd[CT_MAX_DIMS - 2];
+  char* ptr[kMaxOps];
+  int64_t strideA[kMaxOps], strideB[kMaxOps];
+  int64_t outer_stride[kMaxOps][CT_MAX_DIMS - 2];
+  uint32_t lds_mask;    // bit k: operand k is unit-stride along B and goes through LDS
+  uint32_t const_mask;
+  uint64_t cbits[kMaxOps];
+};
+
+// Largest element size among a functor's types (unused inputs alias Out).
+template <class F> struct elem_sizes {
+  static constexpr size_t m01 = sizeof(typename F::In0) > sizeof(typename F::In1) ? sizeof(typename F::In0) : sizeof(typename F::In1);
+  static constexpr size_t m012 = m01 > sizeof(typename F::In2) ? m01 : sizeof(typename F::In2);
+  static constexpr size_t max_in = m012;
+  static constexpr size_t max_all = m012 > sizeof(typename F::Out) ? m012 : sizeof(typename F::Out);
+};
+// Tile edge: 64 elements for input types up to 4 bytes, 32 for 8-byte types,
+// so one tile row is at most a 256-byte contiguous segment.
+template <class F> struct tile_edge {
+  static constexpr int value = elem_sizes<F>::max_in > 4 ? 32 : 64;
+};
+constexpr size_t tile_slot_bytes(size_t elem, int ts) { return ((elem * ts * (ts + 1)) + 15) & ~size_t(15); }
+
+template <class T, int TS>
+__device__ __forceinline__ void tile_stage(const TileArgs& a, int k, T* lds, int64_t base, uint32_t a0,
+                                           uint32_t b0, int tx, int ty) {
+  // coalesced along B: lane tx walks B, rows of the tile walk A
+  constexpr int ROWS = kBlock / TS;
+  const T* p = reinterpret_cast<const T*>(a.ptr[k]) + base;
+  const uint32_t b = b0 + tx;
+#pragma unroll
+  for (int i = 0; i < TS / ROWS; ++i) {
+    const int row = ty + i * ROWS;
+    const uint32_t ai = a0 + row;
+    if (ai < a.sizeA && b < a.sizeB)
+      lds[row * (TS + 1) + tx] = p[(int64_t)ai * a.strideA[k] + (int64_t)b * a.strideB[k]];
+  }
+}
+
+template <class T, int TS>
+__device__ __forceinline__ T tile_fetch(const TileArgs& a, int k, const T* lds, int64_t base, uint32_t ai,
+                                        uint32_t bi, int tx, int row) {
+  if ((a.const_mask >> k) & 1u) return const_from_bits<T>(a.cbits[k]);
+  if ((a.lds_mask >> k) & 1u) return lds[tx * (TS + 1) + row];
+  return reinterpret_cast<const T*>(a.ptr[k])[base + (int64_t)ai * a.strideA[k] + (int64_t)bi * a.strideB[k]];
+}
+
+template <class F>
+__global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileArgs a) {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+  constexpr int TS = tile_edge<F>::value;
+  constexpr int ROWS = kBlock / TS;
+  extern __shared__ __align__(16) char smem[];
+
+  // LDS slots are handed out in operand order to the operands that need one.
+  In0* l0 = nullptr;
+  In1* l1 = nullptr;
+  In2* l2 = nullptr;
+  {
+    char* p = smem;
+    if (NIN >= 1 && ((a.lds_mask >> 1) & 1u)) { l0 = reinterpret_cast<In0*>(p); p += tile_slot_bytes(sizeof(In0), TS); }
+    if (NIN >= 2 && ((a.lds_mask >> 2) & 1u)) { l1 = reinterpret_cast<In1*>(p); p += tile_slot_bytes(sizeof(In1), TS); }
+    if (NIN >= 3 && ((a.lds_mask >> 3) & 1u)) { l2 = reinterpret_cast<In2*>(p); }
+  }
+
+  uint32_t bid, tb, ta, q0;
+  a.tilesB_fd.divmod(blockIdx.x, q0, tb);
+  a.tilesA_fd.divmod(q0, bid, ta);
+  int64_t off[kMaxOps] = {0, 0, 0, 0};
+  for (int d = 0; d < a.n_outer; ++d) {
+    uint32_t q, r;
+    a.outer_fd[d].divmod(bid, q, r);
+    bid = q;
+#pragma unroll
+    for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
+  }
+  const uint32_t a0 = ta * TS, b0 = tb * TS;
+  const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
+
+  if constexpr (NIN >= 1) if (l0) tile_stage<In0, TS>(a, 1, l0, off[1], a0, b0, tx, ty);
+  if constexpr (NIN >= 2) if (l1) tile_stage<In1, TS>(a, 2, l1, off[2], a0, b0, tx, ty);
+  if constexpr (NIN >= 3) if (l2) tile_stage<In2, TS>(a, 3, l2, off[3], a0, b0, tx, ty);
+  __syncthreads();
+
+  // coalesced along A: lane tx walks A, rows of the tile walk B
+  const uint32_t ai = a0 + tx;
+  Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + off[0];
+#pragma unroll
+  for (int i = 0; i < TS / ROWS; ++i) {
+    const int row = ty + i * ROWS;
+    const uint32_t bi = b0 + row;
+    if (ai < a.sizeA && bi < a.sizeB) {
+      In0 p0{};
+      In1 p1{};
+      In2 p2{};
+      if constexpr (NIN >= 1) p0 = tile_fetch<In0, TS>(a, 1, l0, off[1], ai, bi, tx, row);
+      if constexpr (NIN >= 2) p1 = tile_fetch<In1, TS>(a, 2, l1, off[2], ai, bi, tx, row);
+      if constexpr (NIN >= 3) p2 = tile_fetch<In2, TS>(a, 3, l2, off[3], ai, bi, tx, row);
+      dp[(int64_t)ai * a.strideA[0] + (int64_t)bi * a.strideB[0]] = f(p0, p1, p2);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ GENERAL
+
+struct GenArgs {
+  int64_t n;
+  int32_t nd;
+  int32_t need_coords;  // some operand is in per-dimension mode
+  FastDiv rmax_fd[CT_MAX_DIMS];
+  int64_t rmax[CT_MAX_DIMS];
+  GenOperand op[kMaxOps];
+  char* ptr[kMaxOps];
+  uint64_t cbits[kMaxOps];
+};
+
+template <class I>
+__device__ __forceinline__ int64_t gen_address(const GenArgs& a, int k, I e, const I* arg) {
+  const GenOperand& o = a.op[k];
+  switch (o.mode) {
+    case 0: return (int64_t)e;
+    case 1: return (int64_t)((e / (I)o.amt) % (I)o.ec);
+    case 2: return (int64_t)(e % (I)o.ec);
+    default: break;
+  }
+  int64_t off = 0;
+  for (int d = 0; d < a.nd; ++d) {
+    const int64_t s = o.shape[d];
+    if (s == 1) continue;
+    I c;
+    if (s == a.rmax[d]) c = arg[d] - arg[d + 1] * (I)a.rmax[d];
+    else c = arg[d] % (I)s;
+    const int64_t ci = o.index[d] ? (int64_t)o.index[d][c] : (int64_t)c;
+    off += ci * o.stride[d];
+  }
+  return off;
+}
+
+// Address of logical element e through one of the reference's address objects,
+// with plain 64-bit division (used off the hot paths: reductions' fallback and
+// the serial accumulate).
+__device__ __forceinline__ int64_t ref_address(const GenOperand& o, int nd, const int64_t* rmax, int64_t e) {
+  switch (o.mode) {
+    case 0: return e;
+    case 1: return (e / o.amt) % o.ec;
+    case 2: return e % o.ec;
+    default: break;
+  }
+  int64_t off = 0, arg = e;
+  for (int d = 0; d < nd; ++d) {
+    const int64_t c = arg % o.shape[d];
+    arg /= rmax[d];
+    off += (o.index[d] ? (int64_t)o.index[d][c] : c) * o.stride[d];
+  }
+  return off;
+}
+
+template <class F, class I>
+__global__ void __launch_bounds__(kBlock) ew_gen_kernel(const F f, const GenArgs a) {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+  const I n = (I)a.n;
+  const I step = (I)gridDim.x * kBlock;
+  for (I e = (I)blockIdx.x * kBlock + threadIdx.x; e < n; e += step) {
+    I arg[CT_MAX_DIMS + 1];
+    if (a.need_coords) {
+      arg[0] = e;
+      for (int d = 0; d < a.nd; ++d) {
+        if constexpr (sizeof(I) == 4) arg[d + 1] = a.rmax_fd[d].div(arg[d]);
+        else arg[d + 1] = arg[d] / (I)a.rmax[d];
+      }
+    }
+    In0 p0{};
+    In1 p1{};
+    In2 p2{};
+    if constexpr (NIN >= 1)
+      p0 = (a.op[1].mode == 4) ? const_from_bits<In0>(a.cbits[1])
+                               : reinterpret_cast<const In0*>(a.ptr[1])[gen_address<I>(a, 1, e, arg)];
+    if constexpr (NIN >= 2)
+      p1 = (a.op[2].mode == 4) ? const_from_bits<In1>(a.cbits[2])
+                               : reinterpret_cast<const In1*>(a.ptr[2])[gen_address<I>(a, 2, e, arg)];
+    if constexpr (NIN >= 3)
+      p2 = (a.op[3].mode == 4) ? const_from_bits<In2>(a.cbits[3])
+                               : reinterpret_cast<const In2*>(a.ptr[3])[gen_address<I>(a, 3, e, arg)];
+    reinterpret_cast<Out*>(a.ptr[0])[gen_address<I>(a, 0, e, arg)] = f(p0, p1, p2);
+  }
+}
+
+// One lane applies the updates for e = 0, 1, ... in order.  This is the
+// reference's serial accumulate loop (cpu/tensor_math.clj:234, 324, 399) kept
+// for the cases where several e hit one destination address in an order that
+// cannot be recovered from the dimensions (indirectly indexed destinations).
+template <class F>
+__global__ void ew_serial_kernel(const F f, const GenArgs a) {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  for (int64_t e = 0; e < a.n; ++e) {
+    In0 p0{};
+    In1 p1{};
+    In2 p2{};
+    if constexpr (NIN >= 1)
+      p0 = (a.op[1].mode == 4) ? const_from_bits<In0>(a.cbits[1])
+                               : reinterpret_cast<const In0*>(a.ptr[1])[ref_address(a.op[1], a.nd, a.rmax, e)];
+    if constexpr (NIN >= 2)
+      p1 = (a.op[2].mode == 4) ? const_from_bits<In1>(a.cbits[2])
+                               : reinterpret_cast<const In1*>(a.ptr[2])[ref_address(a.op[2], a.nd, a.rmax, e)];
+    if constexpr (NIN >= 3)
+      p2 = (a.op[3].mode == 4) ? const_from_bits<In2>(a.cbits[3])
+                               : reinterpret_cast<const In2*>(a.ptr[3])[ref_address(a.op[3], a.nd, a.rmax, e)];
+    reinterpret_cast<Out*>(a.ptr[0])[ref_address(a.op[0], a.nd, a.rmax, e)] = f(p0, p1, p2);
+  }
+}
+
+// ------------------------------------------------------------------ launcher
+
+struct EwOperand {
+  const void* ptr;      // nullptr: constant
+  const ct_dims* dims;
+  int elem_size;
+  uint64_t cbits;       // constant value, already in the operand's element type
+};
+
+int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_args, int* main_vec,
+                VecArgs* tail_args, bool* has_tail);
+int prepare_tile(const Plan& plan, const EwOperand* ops, int ts, TileArgs* args, size_t* lds_bytes,
+                 uint32_t* grid);
+int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use64, uint32_t* grid);
+
+template <class F, int VEC>
+inline void launch_vec(hipStream_t s, const F& f, const VecArgs& a) {
+  if (a.total_vecs == 0) return;
+  if (a.total_vecs >= (uint64_t)kBlock * 4 * 512) {
+    const uint64_t per = (uint64_t)kBlock * 4;
+    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 4>), dim3((uint32_t)((a.total_vecs + per - 1) / per)), dim3(kBlock), 0, s, f, a);
+  } else {
+    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 1>), dim3((uint32_t)((a.total_vecs + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, f, a);
+  }
+}
+
+// ops[0] is the destination; ops[1..NIN] the inputs in functor order.
+template <class F>
+int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t n) {
+  constexpr int NIN = F::NIN;
+  if (n == 0) return CT_OK;
+  OperandIn in[kMaxOps];
+  for (int k = 0; k <= NIN; ++k) in[k] = {ops[k].ptr, ops[k].dims, ops[k].elem_size};
+  Plan plan;
+  if (int rc = build_plan(in, NIN + 1, n, &plan)) return rc;
+
+  constexpr int VMAX = 16 / (int)elem_sizes<F>::max_all;
+
+  if (plan.kind == PK_VEC) {
+    VecArgs main_args, tail_args;
+    int vec = 1;
+    bool has_tail = false;
+    if (int rc = prepare_vec(plan, ops, VMAX, &main_args, &vec, &tail_args, &has_tail)) return rc;
+    if (vec == VMAX && VMAX > 1) {
+      note_kernel("vec");
+      launch_vec<F, VMAX>(s, f, main_args);
+      if (has_tail) launch_vec<F, 1>(s, f, tail_args);
+    } else {
+      note_kernel("vec1");
+      launch_vec<F, 1>(s, f, main_args);
+    }
+    return after_launch(s);
+  }
+  if (plan.kind == PK_TILE) {
+    TileArgs ta;
+    size_t lds = 0;
+    uint32_t grid = 0;
+    if (int rc = prepare_tile(plan, ops, tile_edge<F>::value, &ta, &lds, &grid)) return rc;
+    note_kernel("tile");
+    hipLaunchKernelGGL((ew_tile_kernel<F>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+    return after_launch(s);
+  }
+  GenArgs ga;
+  bool use64 = false;
+  uint32_t grid = 0;
+  if (int rc = prepare_gen(plan, ops, &ga, &use64, &grid)) return rc;
+  note_kernel(use64 ? "general64" : "general");
+  if (use64) hipLaunchKernelGGL((ew_gen_kernel<F, uint64_t>), dim3(grid), dim3(kBlock), 0, s, f, ga);
+  else hipLaunchKernelGGL((ew_gen_kernel<F, uint32_t>), dim3(grid), dim3(kBlock), 0, s, f, ga);
+  return after_launch(s);
+}
+
+// Serial, order-preserving execution of F (see ew_serial_kernel).
+template <class F>
+int launch_elementwise_serial(hipStream_t s, const F& f, const EwOperand* ops, int64_t n) {
+  constexpr int NIN = F::NIN;
+  if (n == 0) return CT_OK;
+  OperandIn in[kMaxOps];
+  for (int k = 0; k <= NIN; ++k) in[k] = {ops[k].ptr, ops[k].dims, ops[k].elem_size};
+  Plan plan;
+  if (int rc = build_plan(in, NIN + 1, n, &plan, true)) return rc;
+  GenArgs ga;
+  bool use64 = false;
+  uint32_t grid = 0;
+  if (int rc = prepare_gen(plan, ops, &ga, &use64, &grid)) return rc;
+  note_kernel("serial");
+  hipLaunchKernelGGL((ew_serial_kernel<F>), dim3(1), dim3(64), 0, s, f, ga);
+  return after_launch(s);
+}
+
+}  // namespace cthip

@@ -1,0 +1,168 @@
+// functors.h -- scalar operations of the tensor-math path with the value
+// semantics of the reference's CPU backend.
+//
+// For float tensors the CPU backend widens every operand to double, performs
+// the operation in double and rounds once at the store
+// (src/cortex/compute/cpu/tensor_math.clj:211-223, 278-304, 464-466); integer
+// tensors widen to long, wrap, and narrow by truncation.  The functors below
+// do the same on the device, one rounding per JVM operation (the library is
+// compiled with -ffp-contract=off so no multiply-add is fused).
+//
+// exp, tanh and logistic on float tensors with alpha == 1 are evaluated by the
+// single-precision device routines (about 1 ulp, far inside the 2e-6 relative
+// budget of a transcendental) because the double-precision routines would make
+// these kernels compute-bound; every other float operation takes the double
+// route and is bit-identical to the CPU backend.
+#pragma once
+
+#include "common.h"
+
+namespace cthip {
+
+// ------------------------------------------------------------------ assign
+
+template <class D, class S> struct AssignF {
+  static constexpr int NIN = 1;
+  using Out = D;
+  using In0 = S;
+  using In1 = D;
+  using In2 = D;
+  __device__ __forceinline__ D operator()(S s, D, D) const { return jvm_convert<D, S>(s); }
+};
+
+template <class T> struct ConstantF {
+  static constexpr int NIN = 0;
+  using Out = T;
+  using In0 = T;
+  using In1 = T;
+  using In2 = T;
+  T value;
+  __device__ __forceinline__ T operator()(T, T, T) const { return value; }
+};
+
+// ------------------------------------------------------------------ unary
+
+// java.lang.Math.round: nearest long, ties toward +infinity, NaN -> 0.
+__device__ __forceinline__ int64_t jvm_round(double v) {
+  if (v != v) return 0;
+  double r = floor(v);
+  if (v - r >= 0.5) r += 1.0;
+  return jvm_d2l(r);
+}
+
+// perform-unary-op-impl (cpu/tensor_math.clj:211-223) on v = x * alpha.
+template <class T, int OP, class A> __device__ __forceinline__ T unary_value(A v) {
+  if constexpr (OP == CT_UOP_FLOOR) return jvm_cast<T>(floor((double)v));
+  else if constexpr (OP == CT_UOP_CEIL) return jvm_cast<T>(ceil((double)v));
+  else if constexpr (OP == CT_UOP_ROUND) return jvm_cast<T>(jvm_round((double)v));
+  else if constexpr (OP == CT_UOP_NEGATE) return jvm_cast<T>(w_neg(v));
+  else if constexpr (OP == CT_UOP_TANH) return jvm_cast<T>(tanh((double)v));
+  else if constexpr (OP == CT_UOP_LOGISTIC) return jvm_cast<T>(1.0 / (1.0 + exp((double)w_neg(v))));
+  else if constexpr (OP == CT_UOP_EXP) return jvm_cast<T>(exp((double)v));
+  else if constexpr (OP == CT_UOP_SQRT) return jvm_cast<T>(sqrt((double)v));
+  else return jvm_cast<T>((double)v);
+}
+
+template <class T, int OP> struct UnaryF {
+  static constexpr int NIN = 1;
+  using Out = T;
+  using In0 = T;
+  using In1 = T;
+  using In2 = T;
+  using A = typename acc_of<T>::type;
+  A alpha;
+  int32_t single;  // float tensor, alpha == 1, transcendental op
+  __device__ __forceinline__ T operator()(T x, T, T) const {
+    if constexpr (std::is_same<T, float>::value &&
+                  (OP == CT_UOP_TANH || OP == CT_UOP_LOGISTIC || OP == CT_UOP_EXP)) {
+      if (single) {
+        if constexpr (OP == CT_UOP_TANH) return tanhf(x);
+        else if constexpr (OP == CT_UOP_EXP) return expf(x);
+        else return 1.0f / (1.0f + expf(-x));
+      }
+    }
+    return unary_value<T, OP, A>(w_mul((A)x, alpha));
+  }
+};
+
+// ------------------------------------------------------------------ binary
+
+__device__ __forceinline__ int32_t jvm_unchecked_int(int64_t v) { return (int32_t)(uint32_t)(uint64_t)v; }
+__device__ __forceinline__ int32_t jvm_unchecked_int(double v) { return jvm_d2i(v); }
+
+// perform-operation-impl (cpu/tensor_math.clj:278-304).
+template <class T, int OP, class A> __device__ __forceinline__ T binary_value(A x, A y) {
+  if constexpr (OP == CT_BOP_ADD) return jvm_cast<T>(w_add(x, y));
+  else if constexpr (OP == CT_BOP_SUB) return jvm_cast<T>(w_sub(x, y));
+  else if constexpr (OP == CT_BOP_MUL) return jvm_cast<T>(w_mul(x, y));
+  else if constexpr (OP == CT_BOP_DIV) {
+    if constexpr (std::is_same<A, double>::value) return jvm_cast<T>(x / y);
+    else return jvm_ratio_cast<T>(x, y);
+  }
+  else if constexpr (OP == CT_BOP_MAX) return jvm_cast<T>(x > y ? x : y);
+  else if constexpr (OP == CT_BOP_MIN) return jvm_cast<T>(x > y ? y : x);
+  else if constexpr (OP == CT_BOP_BIT_AND) return jvm_cast<T>((int64_t)(jvm_unchecked_int(x) & jvm_unchecked_int(y)));
+  else if constexpr (OP == CT_BOP_BIT_XOR) return jvm_cast<T>((int64_t)(jvm_unchecked_int(x) ^ jvm_unchecked_int(y)));
+  else if constexpr (OP == CT_BOP_EQ) return jvm_cast<T>((int64_t)(x == y ? 1 : 0));
+  else if constexpr (OP == CT_BOP_GT) return jvm_cast<T>((int64_t)(x > y ? 1 : 0));
+  else if constexpr (OP == CT_BOP_GE) return jvm_cast<T>((int64_t)(x >= y ? 1 : 0));
+  else if constexpr (OP == CT_BOP_LT) return jvm_cast<T>((int64_t)(x < y ? 1 : 0));
+  else return jvm_cast<T>((int64_t)(x <= y ? 1 : 0));
+}
+
+// dest = op(x * xa, y * ya).  A scalar operand is passed as a constant input
+// with alpha 1 (the caller has already folded its alpha, src/cortex/tensor.clj:680).
+template <class T, int OP> struct BinaryF {
+  static constexpr int NIN = 2;
+  using Out = T;
+  using In0 = T;
+  using In1 = T;
+  using In2 = T;
+  using A = typename acc_of<T>::type;
+  A xa, ya;
+  __device__ __forceinline__ T operator()(T x, T y, T) const {
+    return binary_value<T, OP, A>(w_mul((A)x, xa), w_mul((A)y, ya));
+  }
+};
+
+// ------------------------------------------------------------------ ternary select
+
+// Three tensors (cpu/tensor_math.clj:469-497): the comparison sees the
+// unrounded products.
+template <class T> struct SelectF {
+  static constexpr int NIN = 3;
+  using Out = T;
+  using In0 = T;
+  using In1 = T;
+  using In2 = T;
+  using A = typename acc_of<T>::type;
+  A xa, ya, za;
+  __device__ __forceinline__ T operator()(T x, T y, T z) const {
+    const A vx = w_mul(xa, (A)x);
+    return jvm_cast<T>(vx >= (A)0 ? w_mul(za, (A)z) : w_mul(ya, (A)y));
+  }
+};
+
+// One or two constants (cpu/tensor_math.clj:507-567): every argument is cast
+// to the tensor datatype before the comparison; arg_idx routes the three slots
+// (tensors first, then constants) to x, y, z.
+template <class T> struct SelectRoutedF {
+  static constexpr int NIN = 3;
+  using Out = T;
+  using In0 = T;
+  using In1 = T;
+  using In2 = T;
+  using A = typename acc_of<T>::type;
+  A alpha[3];  // 1 for constant slots
+  int8_t arg_idx[3];
+  __device__ __forceinline__ T operator()(T s0, T s1, T s2) const {
+    const T v0 = jvm_cast<T>(w_mul(alpha[0], (A)s0));
+    const T v1 = jvm_cast<T>(w_mul(alpha[1], (A)s1));
+    const T v2 = jvm_cast<T>(w_mul(alpha[2], (A)s2));
+    auto pick = [&](int i) { return i == 0 ? v0 : (i == 1 ? v1 : v2); };
+    const T x = pick(arg_idx[0]), y = pick(arg_idx[1]), z = pick(arg_idx[2]);
+    return ((A)x >= (A)0) ? z : y;
+  }
+};
+
+}  // namespace cthip

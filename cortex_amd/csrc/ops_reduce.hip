@@ -1,0 +1,461 @@
+// ops_reduce.hip -- unary-reduce! (src/cortex/tensor/math.clj:104-108;
+// src/cortex/compute/cpu/tensor_math.clj:582-663).
+//
+// Reference semantics: output element p (in the output's own logical order)
+// receives the reduction of input logical elements [p*k, (p+1)*k), where
+// k = ecount(input) / ecount(output); the accumulator is a double (a long for
+// integer tensors), seeded with the first element, and is rounded once at the
+// store.  max and min are java.lang.Math.max/min: NaN propagates and +0 > -0.
+//
+// Three kernels:
+//   reduce_row_kernel   the reduced axis is unit-stride in memory: a group of
+//                       16, 64 or 256 lanes owns one output, reads its row with
+//                       128-bit loads, accumulates in double and combines with
+//                       wavefront shuffles (and LDS across the 4 waves)
+//   reduce_col_kernel   the reduced axis is strided and another axis is
+//                       unit-stride (a transposed view): lanes own columns,
+//                       the 4 waves of a block stride down the rows so every
+//                       load stays coalesced; rows are split over blocks into
+//                       segments whose partial results go to scratch memory and
+//                       are combined by reduce_finish_kernel (deterministic, no
+//                       atomics)
+//   reduce_any_kernel   anything else (indirect dimensions, ragged segments):
+//                       one lane per output walking the reference's address
+//                       object
+// The double accumulator makes the summation order immaterial after the final
+// rounding to float (the tree order differs from the reference's sequential
+// order by about k * 2^-53 relative to the sum of magnitudes).
+#include <algorithm>
+
+#include "elementwise.h"
+
+using namespace cthip;
+
+namespace {
+
+enum RedKind { RK_MAX = 0, RK_MIN = 1, RK_SUM = 2, RK_SUMSQ = 3 };
+
+__device__ __forceinline__ double jmax(double a, double b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  if (a == 0.0 && b == 0.0) return (__double_as_longlong(a) < 0) ? b : a;
+  return a > b ? a : b;
+}
+__device__ __forceinline__ double jmin(double a, double b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  if (a == 0.0 && b == 0.0) return (__double_as_longlong(a) < 0) ? a : b;
+  return a < b ? a : b;
+}
+__device__ __forceinline__ int64_t jmax(int64_t a, int64_t b) { return a > b ? a : b; }
+__device__ __forceinline__ int64_t jmin(int64_t a, int64_t b) { return a < b ? a : b; }
+
+template <class A, int RK> __device__ __forceinline__ A red_identity() {
+  if constexpr (RK == RK_MAX) {
+    if constexpr (std::is_same<A, double>::value) return -__builtin_huge_val();
+    else return INT64_MIN;
+  } else if constexpr (RK == RK_MIN) {
+    if constexpr (std::is_same<A, double>::value) return __builtin_huge_val();
+    else return INT64_MAX;
+  } else {
+    return (A)0;
+  }
+}
+template <class A, int RK> __device__ __forceinline__ A red_combine(A a, A b) {
+  if constexpr (RK == RK_MAX) return jmax(a, b);
+  else if constexpr (RK == RK_MIN) return jmin(a, b);
+  else return w_add(a, b);
+}
+template <class T, class A, int RK> __device__ __forceinline__ A red_value(T x, A alpha) {
+  const A v = w_mul(alpha, (A)x);
+  if constexpr (RK == RK_SUMSQ) return w_mul(v, v);
+  else return v;
+}
+// Final cast, with mean and magnitude applied (cpu/tensor_math.clj:610-622).
+template <class T, class A> __device__ __forceinline__ T red_finish(A acc, int op, int64_t count) {
+  if (op == CT_ROP_MEAN) {
+    if constexpr (std::is_same<A, double>::value) return jvm_cast<T>(acc / (double)count);
+    else return jvm_ratio_cast<T>(acc, count);
+  }
+  if (op == CT_ROP_MAGNITUDE) return jvm_cast<T>(sqrt((double)acc));
+  return jvm_cast<T>(acc);
+}
+
+template <class A> __device__ __forceinline__ A shfl_xor_any(A v, int mask) {
+  if constexpr (std::is_same<A, double>::value) return __shfl_xor(v, mask, 64);
+  else return (A)__shfl_xor((long long)v, mask, 64);
+}
+
+struct OutAddr {
+  int32_t identity;  // output address == logical index
+  int32_t nd;
+  GenOperand op;
+  int64_t rmax[CT_MAX_DIMS];
+};
+__device__ __forceinline__ int64_t out_address(const OutAddr& o, int64_t p) {
+  return o.identity ? p : ref_address(o.op, o.nd, o.rmax, p);
+}
+
+struct RowArgs {
+  const void* in;
+  void* out;
+  int64_t k, n_out;
+  int32_t n_outer;
+  FastDiv osize[CT_MAX_DIMS];   // kept axes, fastest first
+  int64_t ostride[CT_MAX_DIMS];
+  OutAddr oa;
+  int32_t op;
+};
+
+// TPR lanes per output; kBlock / TPR outputs per block.
+template <class T, int RK, int VEC, int TPR>
+__global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, const typename acc_of<T>::type alpha) {
+  using A = typename acc_of<T>::type;
+  using V = Vec<T, VEC>;
+  constexpr int RPB = kBlock / TPR;
+  __shared__ A lds[kBlock / 64];
+  const int lane = threadIdx.x % TPR;
+  const int64_t p = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+  const bool live = p < a.n_out;
+  A acc0 = red_identity<A, RK>(), acc1 = red_identity<A, RK>();
+  if (live) {
+    int64_t base = 0;
+    uint32_t rem = (uint32_t)p;
+    for (int d = 0; d < a.n_outer; ++d) {
+      uint32_t q, r;
+      a.osize[d].divmod(rem, q, r);
+      rem = q;
+      base += (int64_t)r * a.ostride[d];
+    }
+    const V* row = reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.in) + base);
+    const int64_t nv = a.k / VEC;
+    int64_t i = lane;
+    for (; i + TPR < nv; i += 2 * TPR) {
+      const V x0 = row[i], x1 = row[i + TPR];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        acc0 = red_combine<A, RK>(acc0, red_value<T, A, RK>(x0.v[e], alpha));
+        acc1 = red_combine<A, RK>(acc1, red_value<T, A, RK>(x1.v[e], alpha));
+      }
+    }
+    if (i < nv) {
+      const V x0 = row[i];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc0 = red_combine<A, RK>(acc0, red_value<T, A, RK>(x0.v[e], alpha));
+    }
+  }
+  A acc = red_combine<A, RK>(acc0, acc1);
+  constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+  for (int m = W / 2; m >= 1; m >>= 1) acc = red_combine<A, RK>(acc, shfl_xor_any<A>(acc, m));
+  if constexpr (TPR > 64) {
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      acc = lds[0];
+#pragma unroll
+      for (int w = 1; w < kBlock / 64; ++w) acc = red_combine<A, RK>(acc, lds[w]);
+    }
+  }
+  if (live && lane == 0)
+    reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc, a.op, a.k);
+}
+
+struct ColArgs {
+  const void* in;
+  void* out;
+  void* partials;       // [n_seg][n_out] accumulators
+  int64_t k, n_out, rstride;
+  uint32_t u;           // size of the unit-stride kept axis
+  int64_t u_pmul;       // its multiplier in the output's logical index
+  uint32_t n_strips, n_seg, rows_per_seg;
+  FastDiv strips_fd, seg_fd;
+  int32_t n_rest;       // other kept axes, fastest first
+  FastDiv rsize[CT_MAX_DIMS];
+  int64_t rstride_in[CT_MAX_DIMS], r_pmul[CT_MAX_DIMS];
+  OutAddr oa;
+  int32_t op;
+};
+
+template <class T, int RK, int VEC>
+__global__ void __launch_bounds__(kBlock) reduce_col_kernel(const ColArgs a, const typename acc_of<T>::type alpha) {
+  using A = typename acc_of<T>::type;
+  using V = Vec<T, VEC>;
+  constexpr int WAVES = kBlock / 64;
+  __shared__ A lds[WAVES - 1][64 * VEC];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t q0, strip, seg, rest;
+  a.strips_fd.divmod(blockIdx.x, q0, strip);
+  a.seg_fd.divmod(q0, rest, seg);
+  int64_t base = 0, pbase = 0;
+  for (int d = 0; d < a.n_rest; ++d) {
+    uint32_t q, r;
+    a.rsize[d].divmod(rest, q, r);
+    rest = q;
+    base += (int64_t)r * a.rstride_in[d];
+    pbase += (int64_t)r * a.r_pmul[d];
+  }
+  const uint32_t col = (strip * 64 + lane) * VEC;
+  const bool live = col < a.u;
+  A acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = red_identity<A, RK>();
+  const int64_t r0 = (int64_t)seg * a.rows_per_seg;
+  int64_t r1 = r0 + a.rows_per_seg;
+  if (r1 > a.k) r1 = a.k;
+  if (live) {
+    const T* p = reinterpret_cast<const T*>(a.in) + base + col;
+    int64_t r = r0 + wave;
+    for (; r + WAVES < r1; r += 2 * WAVES) {
+      const V x0 = *reinterpret_cast<const V*>(p + r * a.rstride);
+      const V x1 = *reinterpret_cast<const V*>(p + (r + WAVES) * a.rstride);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x0.v[e], alpha));
+        acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x1.v[e], alpha));
+      }
+    }
+    if (r < r1) {
+      const V x0 = *reinterpret_cast<const V*>(p + r * a.rstride);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x0.v[e], alpha));
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) lds[wave - 1][e * 64 + lane] = acc[e];
+  }
+  __syncthreads();
+  if (wave == 0 && live) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+#pragma unroll
+      for (int w = 0; w < WAVES - 1; ++w) acc[e] = red_combine<A, RK>(acc[e], lds[w][e * 64 + lane]);
+      const int64_t p = pbase + (int64_t)(col + e) * a.u_pmul;
+      if (a.n_seg == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc[e], a.op, a.k);
+      else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc[e];
+    }
+  }
+}
+
+template <class T, int RK>
+__global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const ColArgs a) {
+  using A = typename acc_of<T>::type;
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p >= a.n_out) return;
+  const A* part = reinterpret_cast<const A*>(a.partials);
+  A acc = part[p];
+  for (uint32_t s = 1; s < a.n_seg; ++s) acc = red_combine<A, RK>(acc, part[(int64_t)s * a.n_out + p]);
+  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc, a.op, a.k);
+}
+
+struct AnyArgs {
+  const void* in;
+  void* out;
+  int64_t k, n_out;
+  int32_t in_nd;
+  GenOperand in_op;
+  int64_t in_rmax[CT_MAX_DIMS];
+  OutAddr oa;
+  int32_t op;
+};
+
+// One lane per output, in the reference's own order (sequential accumulation).
+template <class T, int RK>
+__global__ void __launch_bounds__(kBlock) reduce_any_kernel(const AnyArgs a, const typename acc_of<T>::type alpha) {
+  using A = typename acc_of<T>::type;
+  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p >= a.n_out) return;
+  const T* in = reinterpret_cast<const T*>(a.in);
+  const int64_t start = p * a.k;
+  A acc = red_value<T, A, RK>(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start)], alpha);
+  for (int64_t i = 1; i < a.k; ++i)
+    acc = red_combine<A, RK>(acc, red_value<T, A, RK>(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start + i)], alpha));
+  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc, a.op, a.k);
+}
+
+// ------------------------------------------------------------------ host planning
+
+struct RedShape {  // the input split into kept axes and one merged reduced axis
+  bool fast;       // direct, non-negative strides, segment = trailing axes, single reduced axis
+  int64_t k, rstride;
+  int n_kept;      // slowest first
+  int64_t ksize[CT_MAX_DIMS], kstride[CT_MAX_DIMS];
+};
+
+RedShape analyse(const ct_dims& in, int64_t k) {
+  RedShape r;
+  std::memset(&r, 0, sizeof(r));
+  r.k = k;
+  r.fast = dims_direct(in);
+  for (int i = 0; r.fast && i < in.ndim; ++i)
+    if (in.shape[i] > 1 && in.strides[i] < 0) r.fast = false;
+  if (!r.fast) return r;
+  int j = in.ndim;
+  int64_t prod = 1;
+  while (j > 0 && prod < k) prod *= in.shape[--j];
+  if (prod != k) { r.fast = false; return r; }
+  // merge the reduced axes j..nd-1 (size-1 axes dropped) into one
+  int64_t rsize = 1, rstr = 1;
+  bool have = false;
+  for (int i = in.ndim - 1; i >= j; --i) {
+    if (in.shape[i] == 1) continue;
+    if (!have) { rsize = in.shape[i]; rstr = in.strides[i]; have = true; }
+    else if (in.strides[i] == rstr * rsize) rsize *= in.shape[i];
+    else { r.fast = false; return r; }
+  }
+  r.rstride = have ? rstr : 1;
+  for (int i = 0; i < j; ++i) {
+    if (in.shape[i] == 1) continue;
+    r.ksize[r.n_kept] = in.shape[i];
+    r.kstride[r.n_kept] = in.strides[i];
+    ++r.n_kept;
+  }
+  return r;
+}
+
+template <class T> bool aligned_for(const void* p, int vec) { return ((uintptr_t)p % (uintptr_t)(vec * sizeof(T))) == 0; }
+
+template <class T, int RK>
+int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha_d, const void* in, const ct_dims* id,
+                 int op) {
+  using A = typename acc_of<T>::type;
+  const A alpha = (A)jvm_cast<T>(alpha_d);
+  const int64_t n_out = dims_ecount(*od), total = dims_ecount(*id);
+  const int64_t k = total / n_out;
+  CT_REQUIRE(k >= 1, "unary-reduce!: input (%lld elements) is smaller than output (%lld)", (long long)total,
+             (long long)n_out);
+
+  OutAddr oa;
+  std::memset(&oa, 0, sizeof(oa));
+  int out_rank = 0;
+  if (int rc = reference_operand_own(od, &oa.op, oa.rmax, &out_rank)) return rc;
+  oa.nd = out_rank;
+  oa.identity = oa.op.mode == 0;
+
+  constexpr int VMAX = 16 / (int)sizeof(T);
+  const RedShape rs = analyse(*id, k);
+  const bool small_idx = n_out < (int64_t(1) << 31) && k < (int64_t(1) << 31);
+
+  if (rs.fast && small_idx && rs.rstride == 1) {
+    RowArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.in = in; a.out = out; a.k = k; a.n_out = n_out; a.oa = oa; a.op = op;
+    a.n_outer = rs.n_kept;
+    bool vec_ok = VMAX > 1 && k % VMAX == 0 && aligned_for<T>(in, VMAX);
+    for (int d = 0; d < rs.n_kept; ++d) {  // fastest first
+      const int src = rs.n_kept - 1 - d;
+      a.osize[d] = FastDiv((uint32_t)rs.ksize[src]);
+      a.ostride[d] = rs.kstride[src];
+      if (rs.kstride[src] % VMAX != 0) vec_ok = false;
+    }
+    const int64_t row_bytes = k * (int64_t)sizeof(T);
+#define CT_ROW(VEC, TPR)                                                                                        \
+  hipLaunchKernelGGL((reduce_row_kernel<T, RK, VEC, TPR>), dim3((uint32_t)((n_out + (kBlock / TPR) - 1) / (kBlock / TPR))), \
+                     dim3(kBlock), 0, st, a, alpha)
+    if (row_bytes >= 4096) {
+      note_kernel(vec_ok ? "reduce_row256_vec" : "reduce_row256");
+      if (vec_ok) CT_ROW(VMAX, 256); else CT_ROW(1, 256);
+    } else if (row_bytes >= 512) {
+      note_kernel(vec_ok ? "reduce_row64_vec" : "reduce_row64");
+      if (vec_ok) CT_ROW(VMAX, 64); else CT_ROW(1, 64);
+    } else {
+      note_kernel("reduce_row16");
+      CT_ROW(1, 16);
+    }
+#undef CT_ROW
+    return after_launch(st);
+  }
+
+  int unit = -1;
+  if (rs.fast && small_idx)
+    for (int d = 0; d < rs.n_kept; ++d)
+      if (rs.kstride[d] == 1 && rs.ksize[d] >= 16) unit = d;
+  if (unit >= 0) {
+    ColArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.in = in; a.out = out; a.k = k; a.n_out = n_out; a.rstride = rs.rstride; a.oa = oa; a.op = op;
+    a.u = (uint32_t)rs.ksize[unit];
+    bool vec_ok = VMAX > 1 && a.u % VMAX == 0 && rs.rstride % VMAX == 0 && aligned_for<T>(in, VMAX);
+    // logical multipliers of the kept axes in the output index (row-major, slowest first)
+    int64_t pmul[CT_MAX_DIMS];
+    int64_t m = 1;
+    for (int d = rs.n_kept - 1; d >= 0; --d) { pmul[d] = m; m *= rs.ksize[d]; }
+    a.u_pmul = pmul[unit];
+    int64_t rest_count = 1;
+    for (int d = rs.n_kept - 1; d >= 0; --d) {  // fastest first
+      if (d == unit) continue;
+      a.rsize[a.n_rest] = FastDiv((uint32_t)rs.ksize[d]);
+      a.rstride_in[a.n_rest] = rs.kstride[d];
+      a.r_pmul[a.n_rest] = pmul[d];
+      if (rs.kstride[d] % VMAX != 0) vec_ok = false;
+      rest_count *= rs.ksize[d];
+      ++a.n_rest;
+    }
+    const int vec = vec_ok ? VMAX : 1;
+    a.n_strips = (a.u + 64 * vec - 1) / (64 * vec);
+    const int64_t base_blocks = (int64_t)a.n_strips * rest_count;
+    // enough blocks to fill 256 CUs several times over, at least 16 rows per segment,
+    // partials capped at 16 MiB
+    int64_t seg = (4096 + base_blocks - 1) / base_blocks;
+    seg = std::min<int64_t>(seg, std::max<int64_t>(1, k / 16));
+    seg = std::min<int64_t>(seg, std::max<int64_t>(1, (int64_t(16) << 20) / (n_out * (int64_t)sizeof(A))));
+    seg = std::max<int64_t>(seg, 1);
+    int64_t rows = (k + seg - 1) / seg;
+    seg = (k + rows - 1) / rows;
+    a.n_seg = (uint32_t)seg;
+    a.rows_per_seg = (uint32_t)rows;
+    a.strips_fd = FastDiv(a.n_strips);
+    a.seg_fd = FastDiv(a.n_seg);
+    const int64_t grid = base_blocks * seg;
+    if (grid < (int64_t(1) << 31)) {
+      if (seg > 1) {
+        if (int rc = stream_scratch(st, (size_t)(seg * n_out) * sizeof(A), &a.partials)) return rc;
+      }
+      note_kernel(vec_ok ? "reduce_col_vec" : "reduce_col");
+      if (vec_ok) hipLaunchKernelGGL((reduce_col_kernel<T, RK, VMAX>), dim3((uint32_t)grid), dim3(kBlock), 0, st, a, alpha);
+      else hipLaunchKernelGGL((reduce_col_kernel<T, RK, 1>), dim3((uint32_t)grid), dim3(kBlock), 0, st, a, alpha);
+      if (seg > 1)
+        hipLaunchKernelGGL((reduce_finish_kernel<T, RK>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock),
+                           0, st, a);
+      return after_launch(st);
+    }
+  }
+
+  AnyArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.in = in; a.out = out; a.k = k; a.n_out = n_out; a.oa = oa; a.op = op;
+  int in_rank = 0;
+  if (int rc = reference_operand_own(id, &a.in_op, a.in_rmax, &in_rank)) return rc;
+  a.in_nd = in_rank;
+  CT_REQUIRE((n_out + kBlock - 1) / kBlock < (int64_t(1) << 31), "unary-reduce!: too many outputs");
+  note_kernel("reduce_any");
+  hipLaunchKernelGGL((reduce_any_kernel<T, RK>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
+                     a, alpha);
+  return after_launch(st);
+}
+
+template <class T>
+int reduce_dispatch(hipStream_t st, void* out, const ct_dims* od, double alpha, const void* in, const ct_dims* id,
+                    int op) {
+  switch (op) {
+    case CT_ROP_MAX: return reduce_typed<T, RK_MAX>(st, out, od, alpha, in, id, op);
+    case CT_ROP_MIN: return reduce_typed<T, RK_MIN>(st, out, od, alpha, in, id, op);
+    case CT_ROP_SUM:
+    case CT_ROP_MEAN: return reduce_typed<T, RK_SUM>(st, out, od, alpha, in, id, op);
+    case CT_ROP_MAGNITUDE:
+    case CT_ROP_MAGNITUDE_SQUARED: return reduce_typed<T, RK_SUMSQ>(st, out, od, alpha, in, id, op);
+    default: return set_error(CT_ERR_INVALID, "unknown reduction operation %d", op);
+  }
+}
+
+}  // namespace
+
+extern "C" int ct_unary_reduce(void* stream, void* output, const ct_dims* output_dims, double input_alpha,
+                               const void* input, const ct_dims* input_dims, int op, int dtype) {
+  CT_REQUIRE(output && input, "ct_unary_reduce: null buffer");
+  if (int rc = check_dims(output_dims, "output")) return rc;
+  if (int rc = check_dims(input_dims, "input")) return rc;
+  CT_DISPATCH_DTYPE(dtype, return reduce_dispatch<T>(static_cast<hipStream_t>(stream), output, output_dims, input_alpha, input, input_dims, op));
+  return CT_OK;
+}

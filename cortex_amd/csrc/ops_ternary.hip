@@ -1,0 +1,89 @@
+// ops_ternary.hip -- ternary-op!, ternary-op-constant!, ternary-op-constant-constant!
+// (src/cortex/tensor/math.clj:75-102; src/cortex/compute/cpu/tensor_math.clj:464-580).
+#include "elementwise.h"
+#include "functors.h"
+
+using namespace cthip;
+
+namespace {
+bool valid_arg_idx(const int8_t* a) {
+  if (!a) return false;
+  int seen = 0;
+  for (int k = 0; k < 3; ++k) {
+    if (a[k] < 0 || a[k] > 2) return false;
+    seen |= 1 << a[k];
+  }
+  return seen == 7;
+}
+
+// slots 0..2: tensors first (with their alphas), then constants.
+template <class T>
+int routed_select(hipStream_t s, void* dest, const ct_dims* dd, const void* const* t, const ct_dims* const* td,
+                  const double* alpha, int n_tensors, const double* constants, const int8_t* arg_idx, int64_t n) {
+  using A = typename acc_of<T>::type;
+  SelectRoutedF<T> f;
+  EwOperand ops[4];
+  ops[0] = {dest, dd, (int)sizeof(T), 0};
+  for (int k = 0; k < 3; ++k) {
+    if (k < n_tensors) {
+      f.alpha[k] = (A)jvm_cast<T>(alpha[k]);
+      ops[k + 1] = {t[k], td[k], (int)sizeof(T), 0};
+    } else {
+      f.alpha[k] = (A)1;
+      ops[k + 1] = {nullptr, nullptr, (int)sizeof(T), bits_of<T>(jvm_cast<T>(constants[k - n_tensors]))};
+    }
+    f.arg_idx[k] = arg_idx[k];
+  }
+  return launch_elementwise(s, f, ops, n);
+}
+}  // namespace
+
+extern "C" {
+
+int ct_ternary_op(void* stream, void* dest, const ct_dims* dest_dims, const void* x, const ct_dims* x_dims,
+                  double x_alpha, const void* y, const ct_dims* y_dims, double y_alpha, const void* z,
+                  const ct_dims* z_dims, double z_alpha, int64_t n, int op, int dtype) {
+  CT_REQUIRE(dest && x && y && z, "ct_ternary_op: null buffer");
+  CT_REQUIRE(op == CT_TOP_SELECT, "unknown ternary operation %d", op);
+  CT_DISPATCH_DTYPE(dtype, {
+    using A = typename acc_of<T>::type;
+    SelectF<T> f{(A)jvm_cast<T>(x_alpha), (A)jvm_cast<T>(y_alpha), (A)jvm_cast<T>(z_alpha)};
+    EwOperand ops[4] = {{dest, dest_dims, (int)sizeof(T), 0},
+                        {x, x_dims, (int)sizeof(T), 0},
+                        {y, y_dims, (int)sizeof(T), 0},
+                        {z, z_dims, (int)sizeof(T), 0}};
+    return launch_elementwise(static_cast<hipStream_t>(stream), f, ops, n);
+  });
+  return CT_OK;
+}
+
+int ct_ternary_op_constant(void* stream, void* dest, const ct_dims* dest_dims, const void* a,
+                           const ct_dims* a_dims, double a_alpha, const void* b, const ct_dims* b_dims,
+                           double b_alpha, double constant, int64_t n, int op, const int8_t arg_idx[3],
+                           int dtype) {
+  CT_REQUIRE(dest && a && b, "ct_ternary_op_constant: null buffer");
+  CT_REQUIRE(op == CT_TOP_SELECT, "unknown ternary operation %d", op);
+  CT_REQUIRE(valid_arg_idx(arg_idx), "arg_idx must be a permutation of 0,1,2");
+  const void* t[2] = {a, b};
+  const ct_dims* td[2] = {a_dims, b_dims};
+  const double al[2] = {a_alpha, b_alpha};
+  const double cs[1] = {constant};
+  CT_DISPATCH_DTYPE(dtype, return routed_select<T>(static_cast<hipStream_t>(stream), dest, dest_dims, t, td, al, 2, cs, arg_idx, n));
+  return CT_OK;
+}
+
+int ct_ternary_op_constant_constant(void* stream, void* dest, const ct_dims* dest_dims, const void* a,
+                                    const ct_dims* a_dims, double a_alpha, double const_1, double const_2,
+                                    int64_t n, int op, const int8_t arg_idx[3], int dtype) {
+  CT_REQUIRE(dest && a, "ct_ternary_op_constant_constant: null buffer");
+  CT_REQUIRE(op == CT_TOP_SELECT, "unknown ternary operation %d", op);
+  CT_REQUIRE(valid_arg_idx(arg_idx), "arg_idx must be a permutation of 0,1,2");
+  const void* t[1] = {a};
+  const ct_dims* td[1] = {a_dims};
+  const double al[1] = {a_alpha};
+  const double cs[2] = {const_1, const_2};
+  CT_DISPATCH_DTYPE(dtype, return routed_select<T>(static_cast<hipStream_t>(stream), dest, dest_dims, t, td, al, 1, cs, arg_idx, n));
+  return CT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,255 @@
+/*
+ * cortex_hip.h -- C ABI of libcortex_hip.so, the gfx950 (MI355X) backend for
+ * the cortex tensor-math driver.
+ *
+ * Every entry point replaces one method of the reference's compute-driver or
+ * TensorMath protocols.  Paths cite /root/reference (originrose/cortex).
+ * A JVM caller binds these through JNA; a Python caller through ctypes.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and a non-zero ct_status otherwise;
+ *     ct_last_error() then returns a thread-local, human readable message.
+ *     (The reference throws on every failed native call,
+ *     src/cortex/compute/cuda/driver.clj:40-49.)
+ *   - A stream is an opaque handle; NULL selects the device's default stream.
+ *     Calls on one stream are ordered and asynchronous with respect to the
+ *     host, as on the reference's CUDA backend.
+ *   - Buffers are raw device pointers.  A sub-buffer is pointer arithmetic by
+ *     the caller (src/cortex/compute/cuda/driver.clj:502-506).
+ *   - Dimensions are given in ELEMENTS, slowest dimension first, exactly as the
+ *     reference's {:shape :strides} maps (src/cortex/tensor/dimensions.clj:95-118).
+ *   - Scalars (alphas, constants, optimizer hyper-parameters) cross as double
+ *     and are cast to the tensor datatype inside the library with JVM
+ *     primitive-conversion rules, mirroring drv/dtype-cast
+ *     (src/cortex/compute/driver.clj:17-43) followed by the CPU backend's
+ *     datatype->cast-fn (src/cortex/compute/cpu/driver.clj:149-157).
+ *   - Operation codes reuse the reference's enums
+ *     (resources/operations.h:27-45, 88-102; resources/tensor_unary_reduce.cu:9-20)
+ *     so the keyword->int tables of src/cortex/compute/cuda/tensor_math.clj:54-92
+ *     carry over unchanged.
+ */
+#ifndef CORTEX_HIP_H
+#define CORTEX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CT_MAX_DIMS 8
+
+/* {:shape :strides} of one operand.  index[d] != NULL marks dimension d as
+ * indirectly addressed: the element's coordinate c in [0, shape[d]) is looked
+ * up as index[d][c] (a DEVICE pointer to int32) before it is multiplied by the
+ * stride (src/cortex/tensor/dimensions.clj:7-9, 226-252). */
+typedef struct ct_dims {
+  int32_t ndim;
+  int64_t shape[CT_MAX_DIMS];
+  int64_t strides[CT_MAX_DIMS];
+  const int32_t* index[CT_MAX_DIMS];
+} ct_dims;
+
+/* Datatypes.  The first six are the reference's, in its order
+ * (src/cortex/compute/cuda/driver.clj:354-367; resources/datatypes.h:16-22).
+ * CT_U8 has no counterpart there: the reference's :byte is signed. */
+typedef enum ct_dtype {
+  CT_I8 = 0, CT_I16 = 1, CT_I32 = 2, CT_I64 = 3, CT_F32 = 4, CT_F64 = 5, CT_U8 = 6
+} ct_dtype;
+
+/* resources/operations.h:88-102 */
+typedef enum ct_unary_op_t {
+  CT_UOP_FLOOR = 0, CT_UOP_CEIL = 1, CT_UOP_ROUND = 2, CT_UOP_NEGATE = 3, CT_UOP_TANH = 4,
+  CT_UOP_LOGISTIC = 5, CT_UOP_EXP = 6, CT_UOP_SQRT = 7, CT_UOP_NOOP = 8
+} ct_unary_op_t;
+
+/* resources/operations.h:27-45 */
+typedef enum ct_binary_op_t {
+  CT_BOP_ADD = 0, CT_BOP_SUB = 1, CT_BOP_MUL = 2, CT_BOP_DIV = 3, CT_BOP_MIN = 4, CT_BOP_MAX = 5,
+  CT_BOP_BIT_AND = 6, CT_BOP_BIT_XOR = 7, CT_BOP_EQ = 8, CT_BOP_GT = 9, CT_BOP_GE = 10,
+  CT_BOP_LT = 11, CT_BOP_LE = 12
+} ct_binary_op_t;
+
+/* resources/operations.h:246-254: the only ternary op. */
+typedef enum ct_ternary_op_t { CT_TOP_SELECT = 0 } ct_ternary_op_t;
+
+/* resources/tensor_unary_reduce.cu:9-20 */
+typedef enum ct_reduce_op_t {
+  CT_ROP_MAX = 0, CT_ROP_MIN = 1, CT_ROP_SUM = 2, CT_ROP_MEAN = 3, CT_ROP_MAGNITUDE = 4,
+  CT_ROP_MAGNITUDE_SQUARED = 5
+} ct_reduce_op_t;
+
+typedef enum ct_status {
+  CT_OK = 0,
+  CT_ERR_INVALID = 1,     /* bad argument: rank, dtype, op code, null pointer, shape rule */
+  CT_ERR_HIP = 2,         /* a HIP runtime call failed; message carries hipGetErrorString */
+  CT_ERR_UNSUPPORTED = 3  /* valid in the reference but not provided by this backend */
+} ct_status;
+
+typedef enum ct_copy_kind {
+  CT_COPY_HOST_TO_DEVICE = 0, CT_COPY_DEVICE_TO_HOST = 1, CT_COPY_DEVICE_TO_DEVICE = 2
+} ct_copy_kind;
+
+/* ------------------------------------------------------------------ errors */
+
+/* Message of the last failed call on the calling thread ("" if none).
+ * Stands in for the exception text of cuda/driver.clj:40-49. */
+const char* ct_last_error(void);
+
+/* When on, every entry point synchronises its stream before returning so an
+ * asynchronous fault surfaces at the call that caused it.  Mirrors
+ * *cuda-library-debug-execution* (src/cortex/compute/cuda/driver.clj:88-93). */
+int ct_set_debug_sync(int on);
+
+/* Name of the kernel family chosen by the most recent tensor call on this
+ * thread ("vec", "tile", "general", ...).  Diagnostic only; no reference
+ * counterpart. */
+const char* ct_last_kernel(void);
+
+/* ------------------------------------------------- driver / device (PDriver, PDevice) */
+
+/* PDriver get-devices (src/cortex/compute/driver.clj:46-61;
+ * cuda/driver.clj:725-762). */
+int ct_device_count(int* n);
+/* Select the calling thread's device; the reference re-selects on every call
+ * because JVM threads migrate (cuda/driver.clj:63-85). */
+int ct_set_device(int device);
+int ct_get_device(int* device);
+/* PDevice memory-info-impl (compute/driver.clj:74-84). */
+int ct_memory_info(size_t* free_bytes, size_t* total_bytes);
+/* PDevice allocate-device-buffer-impl (cuda/driver.clj:888-895). */
+int ct_malloc(void** ptr, size_t bytes);
+int ct_free(void* ptr);
+/* PDriver allocate-host-buffer-impl: pinned host memory (cuda/driver.clj:849-887). */
+int ct_host_alloc(void** ptr, size_t bytes);
+int ct_host_free(void* ptr);
+
+/* ------------------------------------------------- streams / events (PStream, PEvent) */
+
+/* PDevice create-stream-impl (cuda/driver.clj:589-600). */
+int ct_stream_create(void** stream);
+int ct_stream_destroy(void* stream);
+/* Blocks the host until the stream drains: sync-stream
+ * (compute/driver.clj:217-221). */
+int ct_stream_sync(void* stream);
+/* PStream create-event: creates an event and records it on the stream
+ * (cuda/driver.clj:1033-1040). */
+int ct_event_record(void** event, void* stream);
+/* PStream sync-event: make `stream` wait for `event` (cuda/driver.clj:1041-1043). */
+int ct_stream_wait_event(void* stream, void* event);
+/* PEvent wait-for-event: block the host (cuda/driver.clj:1009-1018). */
+int ct_event_sync(void* event);
+int ct_event_destroy(void* event);
+/* Milliseconds between two recorded events; used for timing. No reference counterpart. */
+int ct_event_elapsed_ms(void* start_event, void* stop_event, float* ms);
+/* Like ct_event_record but the event keeps timestamps (for ct_event_elapsed_ms). */
+int ct_event_record_timed(void** event, void* stream);
+
+/* PStream copy-host->device / copy-device->host / copy-device->device
+ * (cuda/driver.clj:922-1019).  Offsets are applied by the caller.  Host
+ * memory should come from ct_host_alloc for a truly asynchronous copy. */
+int ct_memcpy_async(void* dst, const void* src, size_t bytes, int kind, void* stream);
+/* PStream memset: buffer[i] = (dtype)value for i in [0, n)
+ * (cuda/driver.clj:1020-1032; resources/memset.cu). */
+int ct_memset(void* stream, void* buffer, int dtype, double value, int64_t n);
+
+/* ------------------------------------------------- TensorMath (src/cortex/tensor/math.clj:11-104) */
+
+/* assign-constant! (tensor/math.clj:14-15; cpu/tensor_math.clj:137-153):
+ * dest[A(e)] = (dtype)value, e in [0, n). */
+int ct_assign_constant(void* stream, void* dest, const ct_dims* dest_dims, int dtype,
+                       double value, int64_t n);
+
+/* assign! (tensor/math.clj:16-26; cpu/tensor_math.clj:180-208):
+ * dest[Ad(e)] = (dest_dtype) src[As(e)], with JVM narrowing/widening rules. */
+int ct_assign(void* stream, void* dest, const ct_dims* dest_dims, int dest_dtype,
+              const void* src, const ct_dims* src_dims, int src_dtype, int64_t n);
+
+/* unary-accum! (tensor/math.clj:27-30; cpu/tensor_math.clj:226-240):
+ * dest = op(dest * alpha), in place. */
+int ct_unary_accum(void* stream, void* dest, const ct_dims* dest_dims, double alpha, int op,
+                   int dtype, int64_t n);
+
+/* unary-op! (tensor/math.clj:31-35; cpu/tensor_math.clj:243-262):
+ * dest = op(x * alpha). */
+int ct_unary_op(void* stream, void* dest, const ct_dims* dest_dims, const void* x,
+                const ct_dims* x_dims, double alpha, int op, int dtype, int64_t n);
+
+/* binary-accum-constant! (tensor/math.clj:36-42; cpu/tensor_math.clj:314-344):
+ * dest = dest*dest_alpha op scalar   (scalar op dest*dest_alpha when reverse_operands). */
+int ct_binary_accum_constant(void* stream, void* dest, const ct_dims* dest_dims,
+                             double dest_alpha, double scalar, int64_t n, int op,
+                             int reverse_operands, int dtype);
+
+/* binary-op-constant! (tensor/math.clj:44-51; cpu/tensor_math.clj:347-383):
+ * dest = x*x_alpha op scalar   (scalar op x*x_alpha when reverse_operands). */
+int ct_binary_op_constant(void* stream, void* dest, const ct_dims* dest_dims, const void* x,
+                          const ct_dims* x_dims, double x_alpha, double scalar, int64_t n,
+                          int op, int reverse_operands, int dtype);
+
+/* binary-accum! (tensor/math.clj:53-65; cpu/tensor_math.clj:386-420, 1439-1463):
+ * dest[Ad(e)] = dest[Ad(e)]*dest_alpha op y[Ay(e)]*y_alpha for e = 0..n-1.
+ * With dest_requires_cas != 0 several e may hit one dest address (dest is a
+ * broadcast target or indirectly indexed); the reference applies them serially
+ * in increasing e. */
+int ct_binary_accum(void* stream, void* dest, const ct_dims* dest_dims, double dest_alpha,
+                    const void* y, const ct_dims* y_dims, double y_alpha, int64_t n, int op,
+                    int reverse_operands, int dest_requires_cas, int dtype);
+
+/* binary-op! (tensor/math.clj:67-73; cpu/tensor_math.clj:424-462):
+ * dest = x*x_alpha op y*y_alpha. */
+int ct_binary_op(void* stream, void* dest, const ct_dims* dest_dims, const void* x,
+                 const ct_dims* x_dims, double x_alpha, const void* y, const ct_dims* y_dims,
+                 double y_alpha, int64_t n, int op, int dtype);
+
+/* ternary-op! (tensor/math.clj:75-82; cpu/tensor_math.clj:464-497):
+ * select: dest = (x*xa >= 0) ? z*za : y*ya. */
+int ct_ternary_op(void* stream, void* dest, const ct_dims* dest_dims, const void* x,
+                  const ct_dims* x_dims, double x_alpha, const void* y, const ct_dims* y_dims,
+                  double y_alpha, const void* z, const ct_dims* z_dims, double z_alpha,
+                  int64_t n, int op, int dtype);
+
+/* ternary-op-constant! (tensor/math.clj:84-92; cpu/tensor_math.clj:507-537).
+ * a and b are the tensor arguments in x,y,z order, `constant` the remaining
+ * one (already multiplied by its alpha, src/cortex/tensor.clj:802-803).
+ * arg_idx[k] for k = x,y,z is the position (0 = a, 1 = b, 2 = constant) that
+ * supplies that argument: cpu/tensor_math.clj:500-504 arg-order->indexes. */
+int ct_ternary_op_constant(void* stream, void* dest, const ct_dims* dest_dims, const void* a,
+                           const ct_dims* a_dims, double a_alpha, const void* b,
+                           const ct_dims* b_dims, double b_alpha, double constant, int64_t n,
+                           int op, const int8_t arg_idx[3], int dtype);
+
+/* ternary-op-constant-constant! (tensor/math.clj:94-102; cpu/tensor_math.clj:540-567).
+ * Positions: 0 = a, 1 = const_1, 2 = const_2. */
+int ct_ternary_op_constant_constant(void* stream, void* dest, const ct_dims* dest_dims,
+                                    const void* a, const ct_dims* a_dims, double a_alpha,
+                                    double const_1, double const_2, int64_t n, int op,
+                                    const int8_t arg_idx[3], int dtype);
+
+/* unary-reduce! (tensor/math.clj:104-108; cpu/tensor_math.clj:582-663):
+ * output [..., 1] <- reduce over the last axis of the input VIEW [..., k] of
+ * op(input * input_alpha). */
+int ct_unary_reduce(void* stream, void* output, const ct_dims* output_dims, double input_alpha,
+                    const void* input, const ct_dims* input_dims, int op, int dtype);
+
+/* ------------------------------------------------- optimizers */
+
+/* Adam step (src/cortex/optimize/adam.clj:68-102, 116-134; resources/adam.cu).
+ * m and v already point at the parameter buffer's offset inside the flat
+ * optimizer state.  dtype is CT_F32 or CT_F64. */
+int ct_adam_step(void* stream, int dtype, double alpha, double beta1, double beta2,
+                 double epsilon, double pow_beta1_t, double pow_beta2_t, double gradient_alpha,
+                 const void* gradient, void* parameters, void* m, void* v, int64_t n);
+
+/* Adadelta step (java/cortex/compute/optimize/AdadeltaOptimizer.java:29-64;
+ * src/cortex/optimize/adadelta.clj:32-67; resources/adadelta.cu).
+ * grad_sq_accum and dx_sq_accum already point at the parameter offset. */
+int ct_adadelta_step(void* stream, int dtype, double decay, double epsilon, void* grad_sq_accum,
+                     void* dx_sq_accum, double gradient_alpha, const void* gradient,
+                     void* parameters, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CORTEX_HIP_H */

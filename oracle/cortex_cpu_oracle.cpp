@@ -1,0 +1,816 @@
+// cortex_cpu_oracle.cpp -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+//
+// A CPU restatement of the cortex CPU tensor backend for the tensor-math hot
+// path, written from the reference's source text (the reference is Clojure on
+// the JVM and cannot be executed where this is built).  It exists to check the
+// HIP library and to serve as the timed CPU baseline.  Only the tests, the
+// smoke check and the benchmark's cpu_baseline leg may load it; the product
+// library never does.
+//
+// What follows which reference file (paths under /root/reference):
+//   address functions        src/cortex/compute/cpu/tensor_math.clj:33-134
+//                            src/cortex/tensor/dimensions.clj:178-211, 226-353
+//   casts                    src/cortex/compute/cpu/driver.clj:149-157 under
+//                            *unchecked-math* (cpu/tensor_math.clj:28): Java
+//                            primitive narrowing (JLS 5.1.3)
+//   assign-constant!         cpu/tensor_math.clj:137-153
+//   assign!                  cpu/tensor_math.clj:180-208
+//   unary-op!/unary-accum!   cpu/tensor_math.clj:211-262
+//   binary ops               cpu/tensor_math.clj:278-462
+//   ternary select           cpu/tensor_math.clj:464-580
+//   unary-reduce!            cpu/tensor_math.clj:582-663
+//   Adam                     src/cortex/optimize/adam.clj:68-102
+//   Adadelta                 java/cortex/compute/optimize/AdadeltaOptimizer.java:29-64
+//
+// Parity pinning: every function here is checked by tests/test_oracle_*.py
+// against the reference's stored vectors (src/cortex/verify/tensor.clj,
+// src/cortex/compute/verify/optimize.clj, examples/optimise/test/...) and
+// against closed forms / brute force.  CT_U8 has no reference counterpart
+// (the reference's :byte is signed); it is pinned by closed form only.
+//
+// Arithmetic model.  Clojure has no float arithmetic: float operands widen to
+// double, the operation runs in double, and the store rounds once.  Integer
+// operands widen to long; under *unchecked-math* long arithmetic wraps and the
+// narrowing casts truncate.  Each JVM operation rounds separately (no FMA), so
+// this file is compiled with -ffp-contract=off.
+
+#include <cmath>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <type_traits>
+
+#include "../include/cortex_hip.h"
+
+namespace {
+
+thread_local char g_err[256] = "";
+int fail(const char* msg) {
+  std::strncpy(g_err, msg, sizeof(g_err) - 1);
+  g_err[sizeof(g_err) - 1] = 0;
+  return CT_ERR_INVALID;
+}
+
+// ---------------------------------------------------------------- JVM casts
+
+inline int32_t j_d2i(double v) {  // JLS 5.1.3: NaN -> 0, saturating, toward zero
+  if (v != v) return 0;
+  if (v >= 2147483647.0) return INT32_MAX;
+  if (v <= -2147483648.0) return INT32_MIN;
+  return (int32_t)v;
+}
+inline int64_t j_d2l(double v) {
+  if (v != v) return 0;
+  if (v >= 9223372036854775808.0) return INT64_MAX;
+  if (v <= -9223372036854775808.0) return INT64_MIN;
+  return (int64_t)v;
+}
+
+// cast<T>(long) and cast<T>(double): datatype->cast-fn applied to the result of
+// an integer or floating computation.
+template <class T> inline T jcast(int64_t v) {
+  if constexpr (std::is_floating_point<T>::value) return (T)v;  // round to nearest even
+  else return (T)(uint64_t)v;                                   // truncate to the low bits
+}
+template <class T> inline T jcast(double v) {
+  if constexpr (std::is_same<T, double>::value) return v;
+  else if constexpr (std::is_same<T, float>::value) return (float)v;
+  else if constexpr (std::is_same<T, int64_t>::value) return j_d2l(v);
+  else return (T)(uint32_t)j_d2i(v);  // byte/short: through int, then truncate
+}
+// Element of type S converted to T (assign!).  float widens exactly to double,
+// every integer type widens exactly to long.
+template <class T, class S> inline T jconvert(S s) {
+  if constexpr (std::is_floating_point<S>::value) return jcast<T>((double)s);
+  else return jcast<T>((int64_t)s);
+}
+
+// Accumulator type of a tensor datatype: double for float/double, long otherwise.
+template <class T> struct acc_of {
+  using type = typename std::conditional<std::is_floating_point<T>::value, double, int64_t>::type;
+};
+
+inline int64_t wmul(int64_t a, int64_t b) { return (int64_t)((uint64_t)a * (uint64_t)b); }
+inline int64_t wadd(int64_t a, int64_t b) { return (int64_t)((uint64_t)a + (uint64_t)b); }
+inline int64_t wsub(int64_t a, int64_t b) { return (int64_t)((uint64_t)a - (uint64_t)b); }
+inline int64_t wneg(int64_t a) { return (int64_t)(0 - (uint64_t)a); }
+inline double wmul(double a, double b) { return a * b; }
+inline double wadd(double a, double b) { return a + b; }
+inline double wsub(double a, double b) { return a - b; }
+inline double wneg(double a) { return -a; }
+
+// java.lang.Math.round(double): nearest long, ties toward positive infinity.
+inline int64_t j_round(double v) {
+  if (v != v) return 0;
+  double r = std::floor(v);
+  if (v - r >= 0.5) r += 1.0;  // v - floor(v) is exact
+  return j_d2l(r);
+}
+// java.lang.Math.max/min(double, double): NaN propagates, +0 > -0.
+inline double j_max(double a, double b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  if (a == 0.0 && b == 0.0) return std::signbit(a) ? b : a;
+  return a > b ? a : b;
+}
+inline double j_min(double a, double b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  if (a == 0.0 && b == 0.0) return std::signbit(a) ? a : b;
+  return a < b ? a : b;
+}
+inline int64_t j_max(int64_t a, int64_t b) { return a > b ? a : b; }
+inline int64_t j_min(int64_t a, int64_t b) { return a < b ? a : b; }
+
+// ---------------------------------------------------------------- dimensions
+
+struct Dims {  // one operand, slowest first
+  int nd;
+  int64_t shape[CT_MAX_DIMS];
+  int64_t strides[CT_MAX_DIMS];
+  const int32_t* index[CT_MAX_DIMS];
+};
+
+bool load_dims(const ct_dims* in, Dims* out) {
+  if (!in || in->ndim < 1 || in->ndim > CT_MAX_DIMS) return false;
+  out->nd = in->ndim;
+  for (int i = 0; i < in->ndim; ++i) {
+    if (in->shape[i] < 1) return false;
+    out->shape[i] = in->shape[i];
+    out->strides[i] = in->strides[i];
+    out->index[i] = in->index[i];
+  }
+  return true;
+}
+
+int64_t ecount(const Dims& d) {  // dimensions.clj:131-134
+  int64_t n = 1;
+  for (int i = 0; i < d.nd; ++i) n *= d.shape[i];
+  return n;
+}
+bool direct(const Dims& d) {  // dimensions.clj:61-63, 194-196
+  for (int i = 0; i < d.nd; ++i)
+    if (d.index[i]) return false;
+  return true;
+}
+bool access_increasing(const Dims& d) {  // dimensions.clj:204-211
+  if (!direct(d)) return false;
+  for (int i = 0; i + 1 < d.nd; ++i)
+    if (d.strides[i] < d.strides[i + 1]) return false;
+  return true;
+}
+bool dense(const Dims& d) {  // dimensions.clj:178-191
+  if (!direct(d)) return false;
+  if (d.nd == 1) return d.strides[0] == 1;
+  // drop size-1 dims, stable-sort by stride descending, compare the largest
+  // stride with the product of the remaining shapes.
+  int64_t shp[CT_MAX_DIMS], str[CT_MAX_DIMS];
+  int k = 0;
+  for (int i = 0; i < d.nd; ++i)
+    if (d.shape[i] != 1) { shp[k] = d.shape[i]; str[k] = d.strides[i]; ++k; }
+  if (k == 0) return false;  // (first []) is nil; (= nil 1) is false
+  for (int i = 1; i < k; ++i)  // insertion sort, stable, descending stride
+    for (int j = i; j > 0 && str[j - 1] < str[j]; --j) {
+      std::swap(str[j - 1], str[j]);
+      std::swap(shp[j - 1], shp[j]);
+    }
+  int64_t prod = 1;
+  for (int i = 1; i < k; ++i) prod *= shp[i];
+  return str[0] == prod;
+}
+
+// max-extend-strides (dimensions.clj:280-300): left-pad strides with
+// stride*shape of the largest-stride dimension (first one on ties).
+void padded(const Dims& d, int max_nd, int64_t* shape, int64_t* strides, const int32_t** index) {
+  int mi = 0;
+  for (int i = 1; i < d.nd; ++i)
+    if (d.strides[i] > d.strides[mi]) mi = i;
+  int64_t pad = d.strides[mi] * d.shape[mi];
+  int off = max_nd - d.nd;
+  for (int i = 0; i < off; ++i) { shape[i] = 1; strides[i] = pad; index[i] = nullptr; }
+  for (int i = 0; i < d.nd; ++i) {
+    shape[off + i] = d.shape[i];
+    strides[off + i] = d.strides[i];
+    index[off + i] = d.index[i];
+  }
+}
+
+struct MaxShape { int nd; int64_t s[CT_MAX_DIMS]; };
+
+// dimension-seq->max-shape (dimensions.clj:326-353)
+MaxShape max_shape_of(const Dims* const* ops, int n_ops) {
+  MaxShape m;
+  m.nd = 0;
+  for (int k = 0; k < n_ops; ++k)
+    if (ops[k]->nd > m.nd) m.nd = ops[k]->nd;
+  for (int i = 0; i < m.nd; ++i) m.s[i] = 0;
+  for (int k = 0; k < n_ops; ++k) {
+    int off = m.nd - ops[k]->nd;
+    for (int i = 0; i < m.nd; ++i) {
+      int64_t v = i < off ? 1 : ops[k]->shape[i - off];
+      if (v > m.s[i]) m.s[i] = v;
+    }
+  }
+  return m;
+}
+
+// get-elem-dims->address (cpu/tensor_math.clj:82-134): the four address
+// objects of the CPU backend, selected exactly as the reference selects them.
+struct Addr {
+  enum Mode { IDENTITY, BCAST, REPEAT, GENERAL } mode;
+  int64_t ec, amt;
+  int nd;  // GENERAL: reversed (fastest first) data
+  int64_t rshape[CT_MAX_DIMS], rstrides[CT_MAX_DIMS], rmax[CT_MAX_DIMS];
+  const int32_t* rindex[CT_MAX_DIMS];
+
+  inline int64_t operator()(int64_t e) const {
+    switch (mode) {
+      case IDENTITY: return e;                  // SimpleElemIdxToAddr :50-53
+      case BCAST: return (e / amt) % ec;        // SimpleBcastAddr :56-60
+      case REPEAT: return e % ec;               // SimpleRepeatAddr :63-66
+      default: break;
+    }
+    // elem-idx->addr (dimensions.clj:226-252)
+    int64_t off = 0, arg = e;
+    for (int i = 0; i < nd; ++i) {
+      int64_t c = arg % rshape[i];
+      arg /= rmax[i];
+      off += rstrides[i] * (rindex[i] ? (int64_t)rindex[i][c] : c);
+    }
+    return off;
+  }
+};
+
+Addr make_addr(const Dims& d, const MaxShape& mx) {
+  Addr a;
+  std::memset(&a, 0, sizeof(a));
+  const bool dn = dense(d), inc = access_increasing(d), dir = direct(d);
+  const int64_t ec = ecount(d);
+  bool same_shape = d.nd == mx.nd;
+  for (int i = 0; same_shape && i < d.nd; ++i) same_shape = d.shape[i] == mx.s[i];
+  if (dir && same_shape && dn && inc) { a.mode = Addr::IDENTITY; return a; }
+  int64_t biggest = 0;
+  for (int i = 0; i < d.nd; ++i) biggest = d.shape[i] > biggest ? d.shape[i] : biggest;
+  if (dir && ec == biggest && dn && inc) {
+    // first position in the left-padded shape whose size equals ec
+    int off = mx.nd - d.nd, pos = -1;
+    for (int i = 0; i < mx.nd && pos < 0; ++i) {
+      int64_t v = i < off ? 1 : d.shape[i - off];
+      if (v == ec) pos = i;
+    }
+    int64_t amt = 1;
+    for (int i = pos + 1; i < mx.nd; ++i) amt *= mx.s[i];
+    a.mode = Addr::BCAST; a.ec = ec; a.amt = amt;
+    return a;
+  }
+  if (dir && dn && inc) {
+    int lead = 0;  // drop leading 1s, compare with the tail of max-shape
+    while (lead < d.nd && d.shape[lead] == 1) ++lead;
+    int m = d.nd - lead;
+    bool suffix = m <= mx.nd;
+    for (int i = 0; suffix && i < m; ++i) suffix = d.shape[lead + i] == mx.s[mx.nd - m + i];
+    if (suffix) { a.mode = Addr::REPEAT; a.ec = ec; return a; }
+  }
+  a.mode = Addr::GENERAL;
+  a.nd = mx.nd;
+  int64_t shp[CT_MAX_DIMS], str[CT_MAX_DIMS];
+  const int32_t* idx[CT_MAX_DIMS];
+  padded(d, mx.nd, shp, str, idx);
+  for (int i = 0; i < mx.nd; ++i) {
+    a.rshape[i] = shp[mx.nd - 1 - i];
+    a.rstrides[i] = str[mx.nd - 1 - i];
+    a.rindex[i] = idx[mx.nd - 1 - i];
+    a.rmax[i] = mx.s[mx.nd - 1 - i];
+  }
+  return a;
+}
+
+MaxShape own_shape(const Dims& d) {
+  MaxShape m;
+  m.nd = d.nd;
+  for (int i = 0; i < d.nd; ++i) m.s[i] = d.shape[i];
+  return m;
+}
+
+// ---------------------------------------------------------------- scalar ops
+
+// perform-unary-op-impl (cpu/tensor_math.clj:211-223); v = x * alpha in the
+// accumulator type.
+template <class T, class A> inline T unary_apply(int op, A v) {
+  switch (op) {
+    case CT_UOP_FLOOR: return jcast<T>(std::floor((double)v));
+    case CT_UOP_CEIL: return jcast<T>(std::ceil((double)v));
+    case CT_UOP_ROUND: return jcast<T>(j_round((double)v));
+    case CT_UOP_NEGATE: return jcast<T>(wneg(v));
+    case CT_UOP_TANH: return jcast<T>(std::tanh((double)v));
+    case CT_UOP_LOGISTIC: return jcast<T>(1.0 / (1.0 + std::exp((double)wneg(v))));
+    case CT_UOP_EXP: return jcast<T>(std::exp((double)v));
+    case CT_UOP_SQRT: return jcast<T>(std::sqrt((double)v));
+    default: return jcast<T>((double)v);  // :noop is (double x)
+  }
+}
+
+// (dtype-cast (/ a b)) on integer operands.  Clojure's (/ long long) yields a
+// Long when the division is exact and a Ratio otherwise.  The unchecked cast
+// of a Long truncates to the low bits; Ratio.longValue truncates toward zero;
+// Ratio.intValue (which the byte and short casts also go through) is
+// (int)doubleValue, i.e. it saturates at the int range.
+template <class T> inline T ratio_cast(int64_t n, int64_t d) {
+  if (n == INT64_MIN && d == -1) return jcast<T>(n);
+  const int64_t q = n / d;
+  if (n % d == 0 || std::is_same<T, int64_t>::value) return jcast<T>(q);
+  return jcast<T>((double)q);
+}
+
+inline int32_t unchecked_int(int64_t v) { return (int32_t)(uint32_t)(uint64_t)v; }
+inline int32_t unchecked_int(double v) { return j_d2i(v); }
+
+// perform-operation-impl (cpu/tensor_math.clj:278-304).  *div0 is raised when
+// an integer division by zero occurs (the reference throws ArithmeticException).
+template <class T, class A> inline T binary_apply(int op, A x, A y, bool* div0) {
+  switch (op) {
+    case CT_BOP_ADD: return jcast<T>(wadd(x, y));
+    case CT_BOP_SUB: return jcast<T>(wsub(x, y));
+    case CT_BOP_MUL: return jcast<T>(wmul(x, y));
+    case CT_BOP_DIV:
+      if constexpr (std::is_same<A, double>::value) {
+        return jcast<T>(x / y);
+      } else {  // boxed Ratio, then a truncating cast
+        if (y == 0) { *div0 = true; return (T)0; }
+        return ratio_cast<T>(x, y);
+      }
+    case CT_BOP_MAX: return jcast<T>(x > y ? x : y);
+    case CT_BOP_MIN: return jcast<T>(x > y ? y : x);
+    case CT_BOP_BIT_AND: return jcast<T>((int64_t)(unchecked_int(x) & unchecked_int(y)));
+    case CT_BOP_BIT_XOR: return jcast<T>((int64_t)(unchecked_int(x) ^ unchecked_int(y)));
+    case CT_BOP_EQ: return jcast<T>((int64_t)(x == y ? 1 : 0));
+    case CT_BOP_GT: return jcast<T>((int64_t)(x > y ? 1 : 0));
+    case CT_BOP_GE: return jcast<T>((int64_t)(x >= y ? 1 : 0));
+    case CT_BOP_LT: return jcast<T>((int64_t)(x < y ? 1 : 0));
+    default: return jcast<T>((int64_t)(x <= y ? 1 : 0));
+  }
+}
+
+#define DISPATCH_DTYPE(dt, ...)                                      \
+  switch (dt) {                                                      \
+    case CT_I8: { using T = int8_t; __VA_ARGS__; } break;            \
+    case CT_I16: { using T = int16_t; __VA_ARGS__; } break;          \
+    case CT_I32: { using T = int32_t; __VA_ARGS__; } break;          \
+    case CT_I64: { using T = int64_t; __VA_ARGS__; } break;          \
+    case CT_F32: { using T = float; __VA_ARGS__; } break;            \
+    case CT_F64: { using T = double; __VA_ARGS__; } break;           \
+    case CT_U8: { using T = uint8_t; __VA_ARGS__; } break;           \
+    default: return fail("unknown datatype");                        \
+  }
+
+// ---------------------------------------------------------------- op bodies
+
+template <class T>
+int assign_constant_t(T* d, const Dims& dd, double value, int64_t n) {
+  const Addr ad = make_addr(dd, own_shape(dd));
+  const T v = jcast<T>(value);
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < n; ++e) d[ad(e)] = v;
+  return 0;
+}
+
+template <class T, class S>
+int assign_t(T* d, const Dims& dd, const S* s, const Dims& sd, int64_t n) {
+  const Dims* ops[2] = {&dd, &sd};
+  const MaxShape mx = max_shape_of(ops, 2);
+  const Addr ad = make_addr(dd, mx), as = make_addr(sd, mx);
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < n; ++e) d[ad(e)] = jconvert<T, S>(s[as(e)]);
+  return 0;
+}
+
+template <class T>
+int unary_t(T* d, const Dims& dd, const T* x, const Dims* xd, double alpha, int op, int64_t n) {
+  using A = typename acc_of<T>::type;
+  const A al = (A)jcast<T>(alpha);
+  if (!xd) {  // unary-accum!: serial, in place
+    const Addr ad = make_addr(dd, own_shape(dd));
+    for (int64_t e = 0; e < n; ++e) {
+      const int64_t i = ad(e);
+      d[i] = unary_apply<T, A>(op, wmul((A)d[i], al));
+    }
+    return 0;
+  }
+  const Dims* ops[2] = {&dd, xd};
+  const MaxShape mx = max_shape_of(ops, 2);
+  const Addr ad = make_addr(dd, mx), ax = make_addr(*xd, mx);
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < n; ++e) d[ad(e)] = unary_apply<T, A>(op, wmul((A)x[ax(e)], al));
+  return 0;
+}
+
+// x == nullptr: accumulate into dest (serial).  y == nullptr: scalar operand.
+template <class T>
+int binary_t(T* d, const Dims& dd, const T* x, const Dims* xd, double x_alpha, const T* y,
+             const Dims* yd, double y_alpha, double scalar, int64_t n, int op, bool reverse) {
+  using A = typename acc_of<T>::type;
+  const A xa = (A)jcast<T>(x_alpha);
+  const A ya = (A)jcast<T>(y_alpha);
+  const A sc = (A)jcast<T>(scalar);
+  bool div0 = false;
+  const Dims* ops[3];
+  int n_ops = 0;
+  ops[n_ops++] = &dd;
+  if (xd) ops[n_ops++] = xd;
+  if (yd) ops[n_ops++] = yd;
+  // the accumulate-constant form takes its max-shape from dest alone
+  const MaxShape mx = (n_ops == 1) ? own_shape(dd) : max_shape_of(ops, n_ops);
+  const Addr ad = make_addr(dd, mx);
+  Addr ax = ad, ay = ad;
+  if (xd) ax = make_addr(*xd, mx);
+  if (yd) ay = make_addr(*yd, mx);
+  if (!x) {  // binary-accum! / binary-accum-constant!: c-for, increasing e
+    for (int64_t e = 0; e < n; ++e) {
+      const int64_t i = ad(e);
+      const A lhs = wmul((A)d[i], xa);
+      const A rhs = y ? wmul((A)y[ay(e)], ya) : sc;
+      d[i] = reverse ? binary_apply<T, A>(op, rhs, lhs, &div0) : binary_apply<T, A>(op, lhs, rhs, &div0);
+    }
+  } else {
+#pragma omp parallel for schedule(static) reduction(|| : div0)
+    for (int64_t e = 0; e < n; ++e) {
+      const A lhs = wmul((A)x[ax(e)], xa);
+      const A rhs = y ? wmul((A)y[ay(e)], ya) : sc;
+      d[ad(e)] = reverse ? binary_apply<T, A>(op, rhs, lhs, &div0) : binary_apply<T, A>(op, lhs, rhs, &div0);
+    }
+  }
+  return div0 ? fail("Divide by zero") : 0;
+}
+
+// select-impl (cpu/tensor_math.clj:464-466)
+template <class A> inline A select3(A x, A y, A z) { return (x >= (A)0) ? z : y; }
+
+// Three tensors: the comparison sees the unrounded products
+// (cpu/tensor_math.clj:469-497).  With constants every argument is cast to the
+// datatype BEFORE the comparison (cpu/tensor_math.clj:530-537, 560-567).
+template <class T>
+int ternary_t(T* d, const Dims& dd, const T* const* t, const Dims* const* td, const double* alpha,
+              int n_tensors, const double* constants, const int8_t* arg_idx, int64_t n) {
+  using A = typename acc_of<T>::type;
+  const Dims* ops[4];
+  ops[0] = &dd;
+  for (int k = 0; k < n_tensors; ++k) ops[k + 1] = td[k];
+  const MaxShape mx = max_shape_of(ops, n_tensors + 1);
+  const Addr ad = make_addr(dd, mx);
+  Addr at[3];
+  A al[3];
+  for (int k = 0; k < n_tensors; ++k) { at[k] = make_addr(*td[k], mx); al[k] = (A)jcast<T>(alpha[k]); }
+  if (n_tensors == 3) {
+#pragma omp parallel for schedule(static)
+    for (int64_t e = 0; e < n; ++e)
+      d[ad(e)] = jcast<T>(select3<A>(wmul(al[0], (A)t[0][at[0](e)]), wmul(al[1], (A)t[1][at[1](e)]),
+                                     wmul(al[2], (A)t[2][at[2](e)])));
+    return 0;
+  }
+  T cst[3] = {0, 0, 0};  // constants arrive as boxed doubles and are cast to T
+  for (int k = n_tensors; k < 3; ++k) cst[k] = jcast<T>(constants[k - n_tensors]);
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < n; ++e) {
+    T v[3];
+    for (int k = 0; k < 3; ++k)
+      v[k] = k < n_tensors ? jcast<T>(wmul(al[k], (A)t[k][at[k](e)])) : cst[k];
+    d[ad(e)] = jcast<T>(select3<A>((A)v[arg_idx[0]], (A)v[arg_idx[1]], (A)v[arg_idx[2]]));
+  }
+  return 0;
+}
+
+// do-unary-reduce-op (cpu/tensor_math.clj:588-629): sequential, accumulator in
+// the widened type, seeded with the first element.
+template <class T>
+int reduce_t(T* out, const Dims& od, double alpha, const T* in, const Dims& id, int op) {
+  using A = typename acc_of<T>::type;
+  const Addr ao = make_addr(od, own_shape(od)), ai = make_addr(id, own_shape(id));
+  const A al = (A)jcast<T>(alpha);
+  const int64_t par = ecount(od);
+  const int64_t iter = ecount(id) / par;
+  if (iter < 1) return fail("unary-reduce!: input smaller than output");
+#pragma omp parallel for schedule(static)
+  for (int64_t p = 0; p < par; ++p) {
+    const int64_t start = p * iter, stop = start + iter;
+    A acc = wmul(al, (A)in[ai(start)]);
+    if (op == CT_ROP_MAGNITUDE || op == CT_ROP_MAGNITUDE_SQUARED) acc = wmul(acc, acc);
+    for (int64_t i = start + 1; i < stop; ++i) {
+      const A v = wmul(al, (A)in[ai(i)]);
+      switch (op) {
+        case CT_ROP_MAX: acc = j_max(acc, v); break;
+        case CT_ROP_MIN: acc = j_min(acc, v); break;
+        case CT_ROP_SUM:
+        case CT_ROP_MEAN: acc = wadd(acc, v); break;
+        default: acc = wadd(acc, wmul(v, v)); break;
+      }
+    }
+    T r;
+    if (op == CT_ROP_MEAN) {
+      // (/ sum count): double division, or a Ratio truncated by the cast
+      if constexpr (std::is_same<A, double>::value) r = jcast<T>(acc / (double)iter);
+      else r = ratio_cast<T>(acc, iter);
+    } else if (op == CT_ROP_MAGNITUDE) {
+      r = jcast<T>(std::sqrt((double)acc));
+    } else {
+      r = jcast<T>(acc);
+    }
+    out[ao(p)] = r;
+  }
+  return 0;
+}
+
+// cpu-adam-step-impl! (adam.clj:68-102).  The scalars are cast to the datatype
+// first; the arithmetic then runs in double.
+template <class T>
+void adam_t(double alpha_, double beta1_, double beta2_, double eps_, double pb1_, double pb2_,
+            double ga_, const T* g, T* p, T* m, T* v, int64_t n) {
+  const double ga = (double)(T)ga_, alpha = (double)(T)alpha_, beta1 = (double)(T)beta1_,
+               beta2 = (double)(T)beta2_, eps = (double)(T)eps_, pb1 = (double)(T)pb1_,
+               pb2 = (double)(T)pb2_;
+  const double one = 1.0, omb1 = one - beta1, omb2 = one - beta2;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    const double gv = ga * (double)g[i];
+    const double pv = (double)p[i];
+    const double lm = beta1 * (double)m[i] + omb1 * gv;
+    const double lv = beta2 * (double)v[i] + (omb2 * gv) * gv;
+    const double dx = alpha * (lm / ((one - pb1) * (std::sqrt(lv / (one - pb2)) + eps)));
+    m[i] = (T)lm;
+    v[i] = (T)lv;
+    p[i] = (T)(pv - dx);
+  }
+}
+
+// AdadeltaOptimizer.microStep (:29-37); single-threaded like the reference.
+inline void adadelta_micro(double g, double decay, double eps, double ga_in, double dxa_in,
+                           double* ga_out, double* dxa_out, double* dx_out) {
+  const double ga = g * g * decay + ga_in * (1.0 - decay);
+  const double rms_g = std::sqrt(ga + eps);
+  const double rms_dx = std::sqrt(dxa_in + eps);
+  const double dx = (-1.0 * rms_dx * g) / rms_g;
+  *ga_out = ga;
+  *dxa_out = dx * dx * decay + dxa_in * (1.0 - decay);
+  *dx_out = dx;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ C entry points
+// Same argument lists as the library's entry points in include/cortex_hip.h
+// minus the stream; pointers are host pointers.
+
+#define LOAD(name, src)        \
+  Dims name;                   \
+  if (!load_dims(src, &name)) return fail("bad dimensions: " #src)
+
+extern "C" {
+
+const char* co_last_error(void) { return g_err; }
+
+int co_memset(void* buffer, int dtype, double value, int64_t n) {
+  DISPATCH_DTYPE(dtype, { T* b = (T*)buffer; const T v = jcast<T>(value); for (int64_t i = 0; i < n; ++i) b[i] = v; });
+  return 0;
+}
+
+int co_assign_constant(void* dest, const ct_dims* dest_dims, int dtype, double value, int64_t n) {
+  LOAD(dd, dest_dims);
+  DISPATCH_DTYPE(dtype, return assign_constant_t<T>((T*)dest, dd, value, n));
+  return 0;
+}
+
+int co_assign(void* dest, const ct_dims* dest_dims, int dest_dtype, const void* src,
+              const ct_dims* src_dims, int src_dtype, int64_t n) {
+  LOAD(dd, dest_dims);
+  LOAD(sd, src_dims);
+#define INNER(S) DISPATCH_DTYPE(dest_dtype, return (assign_t<T, S>((T*)dest, dd, (const S*)src, sd, n)))
+  switch (src_dtype) {
+    case CT_I8: INNER(int8_t); break;
+    case CT_I16: INNER(int16_t); break;
+    case CT_I32: INNER(int32_t); break;
+    case CT_I64: INNER(int64_t); break;
+    case CT_F32: INNER(float); break;
+    case CT_F64: INNER(double); break;
+    case CT_U8: INNER(uint8_t); break;
+    default: return fail("unknown source datatype");
+  }
+#undef INNER
+  return 0;
+}
+
+int co_unary_accum(void* dest, const ct_dims* dest_dims, double alpha, int op, int dtype, int64_t n) {
+  LOAD(dd, dest_dims);
+  if (op < 0 || op > CT_UOP_NOOP) return fail("unknown unary op");
+  DISPATCH_DTYPE(dtype, return unary_t<T>((T*)dest, dd, nullptr, nullptr, alpha, op, n));
+  return 0;
+}
+
+int co_unary_op(void* dest, const ct_dims* dest_dims, const void* x, const ct_dims* x_dims,
+                double alpha, int op, int dtype, int64_t n) {
+  LOAD(dd, dest_dims);
+  LOAD(xd, x_dims);
+  if (op < 0 || op > CT_UOP_NOOP) return fail("unknown unary op");
+  DISPATCH_DTYPE(dtype, return unary_t<T>((T*)dest, dd, (const T*)x, &xd, alpha, op, n));
+  return 0;
+}
+
+int co_binary_accum_constant(void* dest, const ct_dims* dest_dims, double dest_alpha, double scalar,
+                             int64_t n, int op, int reverse_operands, int dtype) {
+  LOAD(dd, dest_dims);
+  if (op < 0 || op > CT_BOP_LE) return fail("unknown binary op");
+  DISPATCH_DTYPE(dtype, return binary_t<T>((T*)dest, dd, nullptr, nullptr, dest_alpha, nullptr, nullptr,
+                                          0.0, scalar, n, op, reverse_operands != 0));
+  return 0;
+}
+
+int co_binary_op_constant(void* dest, const ct_dims* dest_dims, const void* x, const ct_dims* x_dims,
+                          double x_alpha, double scalar, int64_t n, int op, int reverse_operands,
+                          int dtype) {
+  LOAD(dd, dest_dims);
+  LOAD(xd, x_dims);
+  if (op < 0 || op > CT_BOP_LE) return fail("unknown binary op");
+  DISPATCH_DTYPE(dtype, return binary_t<T>((T*)dest, dd, (const T*)x, &xd, x_alpha, nullptr, nullptr, 0.0,
+                                          scalar, n, op, reverse_operands != 0));
+  return 0;
+}
+
+int co_binary_op(void* dest, const ct_dims* dest_dims, const void* x, const ct_dims* x_dims,
+                 double x_alpha, const void* y, const ct_dims* y_dims, double y_alpha, int64_t n,
+                 int op, int dtype);
+
+int co_binary_accum(void* dest, const ct_dims* dest_dims, double dest_alpha, const void* y,
+                    const ct_dims* y_dims, double y_alpha, int64_t n, int op, int reverse_operands,
+                    int dest_requires_cas, int dtype) {
+  if (!dest_requires_cas) {  // cpu/tensor_math.clj:1451-1463: re-enter binary-op!
+    return reverse_operands
+               ? co_binary_op(dest, dest_dims, y, y_dims, y_alpha, dest, dest_dims, dest_alpha, n, op, dtype)
+               : co_binary_op(dest, dest_dims, dest, dest_dims, dest_alpha, y, y_dims, y_alpha, n, op, dtype);
+  }
+  LOAD(dd, dest_dims);
+  LOAD(yd, y_dims);
+  if (op < 0 || op > CT_BOP_LE) return fail("unknown binary op");
+  DISPATCH_DTYPE(dtype, return binary_t<T>((T*)dest, dd, nullptr, nullptr, dest_alpha, (const T*)y, &yd,
+                                          y_alpha, 0.0, n, op, reverse_operands != 0));
+  return 0;
+}
+
+int co_binary_op(void* dest, const ct_dims* dest_dims, const void* x, const ct_dims* x_dims,
+                 double x_alpha, const void* y, const ct_dims* y_dims, double y_alpha, int64_t n,
+                 int op, int dtype) {
+  LOAD(dd, dest_dims);
+  LOAD(xd, x_dims);
+  LOAD(yd, y_dims);
+  if (op < 0 || op > CT_BOP_LE) return fail("unknown binary op");
+  DISPATCH_DTYPE(dtype, return binary_t<T>((T*)dest, dd, (const T*)x, &xd, x_alpha, (const T*)y, &yd,
+                                          y_alpha, 0.0, n, op, false));
+  return 0;
+}
+
+int co_ternary_op(void* dest, const ct_dims* dest_dims, const void* x, const ct_dims* x_dims,
+                  double x_alpha, const void* y, const ct_dims* y_dims, double y_alpha, const void* z,
+                  const ct_dims* z_dims, double z_alpha, int64_t n, int op, int dtype) {
+  LOAD(dd, dest_dims);
+  LOAD(xd, x_dims);
+  LOAD(yd, y_dims);
+  LOAD(zd, z_dims);
+  if (op != CT_TOP_SELECT) return fail("unknown ternary op");
+  const Dims* td[3] = {&xd, &yd, &zd};
+  const double al[3] = {x_alpha, y_alpha, z_alpha};
+  DISPATCH_DTYPE(dtype, {
+    const T* t[3] = {(const T*)x, (const T*)y, (const T*)z};
+    return ternary_t<T>((T*)dest, dd, t, td, al, 3, nullptr, nullptr, n);
+  });
+  return 0;
+}
+
+static bool valid_arg_idx(const int8_t* a) {
+  if (!a) return false;
+  int seen = 0;
+  for (int k = 0; k < 3; ++k) {
+    if (a[k] < 0 || a[k] > 2) return false;
+    seen |= 1 << a[k];
+  }
+  return seen == 7;
+}
+
+int co_ternary_op_constant(void* dest, const ct_dims* dest_dims, const void* a, const ct_dims* a_dims,
+                           double a_alpha, const void* b, const ct_dims* b_dims, double b_alpha,
+                           double constant, int64_t n, int op, const int8_t arg_idx[3], int dtype) {
+  LOAD(dd, dest_dims);
+  LOAD(ad, a_dims);
+  LOAD(bd, b_dims);
+  if (op != CT_TOP_SELECT) return fail("unknown ternary op");
+  if (!valid_arg_idx(arg_idx)) return fail("arg_idx must be a permutation of 0,1,2");
+  const Dims* td[2] = {&ad, &bd};
+  const double al[2] = {a_alpha, b_alpha};
+  const double cs[1] = {constant};
+  DISPATCH_DTYPE(dtype, {
+    const T* t[2] = {(const T*)a, (const T*)b};
+    return ternary_t<T>((T*)dest, dd, t, td, al, 2, cs, arg_idx, n);
+  });
+  return 0;
+}
+
+int co_ternary_op_constant_constant(void* dest, const ct_dims* dest_dims, const void* a,
+                                    const ct_dims* a_dims, double a_alpha, double const_1,
+                                    double const_2, int64_t n, int op, const int8_t arg_idx[3],
+                                    int dtype) {
+  LOAD(dd, dest_dims);
+  LOAD(ad, a_dims);
+  if (op != CT_TOP_SELECT) return fail("unknown ternary op");
+  if (!valid_arg_idx(arg_idx)) return fail("arg_idx must be a permutation of 0,1,2");
+  const Dims* td[1] = {&ad};
+  const double al[1] = {a_alpha};
+  const double cs[2] = {const_1, const_2};
+  DISPATCH_DTYPE(dtype, {
+    const T* t[1] = {(const T*)a};
+    return ternary_t<T>((T*)dest, dd, t, td, al, 1, cs, arg_idx, n);
+  });
+  return 0;
+}
+
+int co_unary_reduce(void* output, const ct_dims* output_dims, double input_alpha, const void* input,
+                    const ct_dims* input_dims, int op, int dtype) {
+  LOAD(od, output_dims);
+  LOAD(id, input_dims);
+  if (op < 0 || op > CT_ROP_MAGNITUDE_SQUARED) return fail("unknown reduction op");
+  DISPATCH_DTYPE(dtype, return reduce_t<T>((T*)output, od, input_alpha, (const T*)input, id, op));
+  return 0;
+}
+
+int co_adam_step(int dtype, double alpha, double beta1, double beta2, double epsilon,
+                 double pow_beta1_t, double pow_beta2_t, double gradient_alpha, const void* gradient,
+                 void* parameters, void* m, void* v, int64_t n) {
+  if (dtype == CT_F32)
+    adam_t<float>(alpha, beta1, beta2, epsilon, pow_beta1_t, pow_beta2_t, gradient_alpha,
+                  (const float*)gradient, (float*)parameters, (float*)m, (float*)v, n);
+  else if (dtype == CT_F64)
+    adam_t<double>(alpha, beta1, beta2, epsilon, pow_beta1_t, pow_beta2_t, gradient_alpha,
+                   (const double*)gradient, (double*)parameters, (double*)m, (double*)v, n);
+  else
+    return fail("adam: datatype must be float or double");
+  return 0;
+}
+
+// AdadeltaOptimizer.step_f / step_d (:39-64)
+int co_adadelta_step(int dtype, double decay, double epsilon, void* grad_sq_accum, void* dx_sq_accum,
+                     double gradient_alpha, const void* gradient, void* parameters, int64_t n) {
+  if (dtype == CT_F32) {
+    const float ga = (float)gradient_alpha, dc = (float)decay, ep = (float)epsilon;
+    const float* g = (const float*)gradient;
+    float *p = (float*)parameters, *gacc = (float*)grad_sq_accum, *dacc = (float*)dx_sq_accum;
+    for (int64_t i = 0; i < n; ++i) {
+      const double grad = (double)(float)(ga * g[i]);  // float product, then widened
+      double a, b, dx;
+      adadelta_micro(grad, (double)dc, (double)ep, (double)gacc[i], (double)dacc[i], &a, &b, &dx);
+      gacc[i] = (float)a;
+      dacc[i] = (float)b;
+      p[i] = (float)(p[i] + (float)dx);  // float += float
+    }
+  } else if (dtype == CT_F64) {
+    const double* g = (const double*)gradient;
+    double *p = (double*)parameters, *gacc = (double*)grad_sq_accum, *dacc = (double*)dx_sq_accum;
+    for (int64_t i = 0; i < n; ++i) {
+      double a, b, dx;
+      adadelta_micro(gradient_alpha * g[i], decay, epsilon, gacc[i], dacc[i], &a, &b, &dx);
+      gacc[i] = a;
+      dacc[i] = b;
+      p[i] += dx;
+    }
+  } else {
+    return fail("adadelta: datatype must be float or double");
+  }
+  return 0;
+}
+
+// Address of linear element e for an operand, given the other operands'
+// dimensions: exposes get-elem-dims->address so the tests can brute-force it.
+// all_dims[0..n_dims) are the operands that form the max-shape (pass only the
+// operand itself for the single-operand ops); which selects the operand.
+int co_elem_address(const ct_dims* const* all_dims, int n_dims, int which, int64_t e, int64_t* addr,
+                    int* mode) {
+  if (n_dims < 1 || n_dims > 4 || which < 0 || which >= n_dims) return fail("bad operand count");
+  Dims d[4];
+  const Dims* ops[4];
+  for (int k = 0; k < n_dims; ++k) {
+    if (!load_dims(all_dims[k], &d[k])) return fail("bad dimensions");
+    ops[k] = &d[k];
+  }
+  const MaxShape mx = max_shape_of(ops, n_dims);
+  const Addr a = make_addr(d[which], mx);
+  *addr = a(e);
+  if (mode) *mode = (int)a.mode;
+  return 0;
+}
+
+int co_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+}  // extern "C"
