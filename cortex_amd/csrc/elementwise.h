@@ -27,6 +27,22 @@ template <class T> __device__ __forceinline__ T const_from_bits(uint64_t bits) {
   __builtin_memcpy(&c, &bits, sizeof(T));
   return c;
 }
+// Streaming (non-temporal) load of any 1/2/4/8/16-byte object: the data is
+// used once, so it should not displace reusable lines from the caches.
+template <int BYTES> struct raw_bits;
+template <> struct raw_bits<1> { using type = uint8_t; };
+template <> struct raw_bits<2> { using type = uint16_t; };
+template <> struct raw_bits<4> { using type = uint32_t; };
+template <> struct raw_bits<8> { using type = uint32_t __attribute__((ext_vector_type(2))); };
+template <> struct raw_bits<16> { using type = uint32_t __attribute__((ext_vector_type(4))); };
+template <class V> __device__ __forceinline__ V nt_load(const V* p) {
+  using R = typename raw_bits<sizeof(V)>::type;
+  const R r = __builtin_nontemporal_load(reinterpret_cast<const R*>(p));
+  V v;
+  __builtin_memcpy(&v, &r, sizeof(V));
+  return v;
+}
+
 template <class T> inline uint64_t bits_of(T c) {
   uint64_t b = 0;
   std::memcpy(&b, &c, sizeof(T));
@@ -56,7 +72,7 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(const VecArgs& a, int k, int64_t
 #pragma unroll
     for (int i = 0; i < VEC; ++i) r.v[i] = c;
   } else if ((a.unit_mask >> k) & 1u) {
-    r = *reinterpret_cast<const Vec<T, VEC>*>(reinterpret_cast<const T*>(a.ptr[k]) + base + col);
+    r = nt_load(reinterpret_cast<const Vec<T, VEC>*>(reinterpret_cast<const T*>(a.ptr[k]) + base + col));
   } else {
     const T c = reinterpret_cast<const T*>(a.ptr[k])[base];
 #pragma unroll
@@ -153,32 +169,28 @@ template <class F> struct tile_edge {
 };
 constexpr size_t tile_slot_bytes(size_t elem, int ts) { return ((elem * ts * (ts + 1)) + 15) & ~size_t(15); }
 
-template <class T, int TS>
-__device__ __forceinline__ void tile_stage(const TileArgs& a, int k, T* lds, int64_t base, uint32_t a0,
-                                           uint32_t b0, int tx, int ty) {
-  // coalesced along B: lane tx walks B, rows of the tile walk A
+// Stages one TS x TS tile of an operand that is unit-stride along B into LDS.
+// Lane tx walks B (a 256-byte coalesced row segment per wave), the block's
+// ROWS waves-rows walk A.  All loads are issued before the LDS writes; the
+// pointer is advanced by a constant step instead of being recomputed.
+template <class T, int TS, bool FULL>
+__device__ __forceinline__ void tile_stage(T* lds, const T* p, int64_t step, uint32_t a_left, bool b_ok, int tx,
+                                           int ty) {
   constexpr int ROWS = kBlock / TS;
-  const T* p = reinterpret_cast<const T*>(a.ptr[k]) + base;
-  const uint32_t b = b0 + tx;
+  constexpr int IT = TS / ROWS;
+  T v[IT];
 #pragma unroll
-  for (int i = 0; i < TS / ROWS; ++i) {
-    const int row = ty + i * ROWS;
-    const uint32_t ai = a0 + row;
-    if (ai < a.sizeA && b < a.sizeB)
-      lds[row * (TS + 1) + tx] = p[(int64_t)ai * a.strideA[k] + (int64_t)b * a.strideB[k]];
+  for (int i = 0; i < IT; ++i) {
+    if (FULL || (b_ok && (uint32_t)(ty + i * ROWS) < a_left)) v[i] = nt_load(p + (int64_t)i * step);
+    else v[i] = T{};
   }
+#pragma unroll
+  for (int i = 0; i < IT; ++i) lds[(ty + i * ROWS) * (TS + 1) + tx] = v[i];
 }
 
-template <class T, int TS>
-__device__ __forceinline__ T tile_fetch(const TileArgs& a, int k, const T* lds, int64_t base, uint32_t ai,
-                                        uint32_t bi, int tx, int row) {
-  if ((a.const_mask >> k) & 1u) return const_from_bits<T>(a.cbits[k]);
-  if ((a.lds_mask >> k) & 1u) return lds[tx * (TS + 1) + row];
-  return reinterpret_cast<const T*>(a.ptr[k])[base + (int64_t)ai * a.strideA[k] + (int64_t)bi * a.strideB[k]];
-}
-
-template <class F>
-__global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileArgs a) {
+template <class F, bool FULL>
+__device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const int64_t* off, uint32_t a0, uint32_t b0,
+                                          typename F::In0* l0, typename F::In1* l1, typename F::In2* l2) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
   using In1 = typename F::In1;
@@ -186,6 +198,67 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
   constexpr int NIN = F::NIN;
   constexpr int TS = tile_edge<F>::value;
   constexpr int ROWS = kBlock / TS;
+  constexpr int IT = TS / ROWS;
+  const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
+  const uint32_t a_left = a.sizeA - a0, b_left = a.sizeB - b0;  // valid extent of this tile
+
+  // phase 1: operands that are unit-stride along B go through LDS
+  if constexpr (NIN >= 1)
+    if (l0) tile_stage<In0, TS, FULL>(l0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
+                                      (int64_t)ROWS * a.strideA[1], a_left, (uint32_t)tx < b_left, tx, ty);
+  if constexpr (NIN >= 2)
+    if (l1) tile_stage<In1, TS, FULL>(l1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
+                                      (int64_t)ROWS * a.strideA[2], a_left, (uint32_t)tx < b_left, tx, ty);
+  if constexpr (NIN >= 3)
+    if (l2) tile_stage<In2, TS, FULL>(l2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
+                                      (int64_t)ROWS * a.strideA[3], a_left, (uint32_t)tx < b_left, tx, ty);
+  __syncthreads();
+
+  // phase 2: lane tx walks A (the destination's unit-stride axis), rows walk B
+  const bool a_ok = (uint32_t)tx < a_left;
+  Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + off[0] + (int64_t)(a0 + tx) * a.strideA[0] + (int64_t)(b0 + ty) * a.strideB[0];
+  const int64_t dstep = (int64_t)ROWS * a.strideB[0];
+  const In0* q0 = nullptr;
+  const In1* q1 = nullptr;
+  const In2* q2 = nullptr;
+  int64_t s0 = 0, s1 = 0, s2 = 0;
+  In0 c0{};
+  In1 c1{};
+  In2 c2{};
+  if constexpr (NIN >= 1) {
+    if ((a.const_mask >> 1) & 1u) c0 = const_from_bits<In0>(a.cbits[1]);
+    else if (!l0) { q0 = reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + tx) * a.strideA[1] + (int64_t)(b0 + ty) * a.strideB[1]; s0 = (int64_t)ROWS * a.strideB[1]; }
+  }
+  if constexpr (NIN >= 2) {
+    if ((a.const_mask >> 2) & 1u) c1 = const_from_bits<In1>(a.cbits[2]);
+    else if (!l1) { q1 = reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + tx) * a.strideA[2] + (int64_t)(b0 + ty) * a.strideB[2]; s1 = (int64_t)ROWS * a.strideB[2]; }
+  }
+  if constexpr (NIN >= 3) {
+    if ((a.const_mask >> 3) & 1u) c2 = const_from_bits<In2>(a.cbits[3]);
+    else if (!l2) { q2 = reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + tx) * a.strideA[3] + (int64_t)(b0 + ty) * a.strideB[3]; s2 = (int64_t)ROWS * a.strideB[3]; }
+  }
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int row = ty + i * ROWS;
+    if (FULL || (a_ok && (uint32_t)row < b_left)) {
+      In0 p0 = c0;
+      In1 p1 = c1;
+      In2 p2 = c2;
+      if constexpr (NIN >= 1) { if (l0) p0 = l0[tx * (TS + 1) + row]; else if (q0) p0 = q0[(int64_t)i * s0]; }
+      if constexpr (NIN >= 2) { if (l1) p1 = l1[tx * (TS + 1) + row]; else if (q1) p1 = q1[(int64_t)i * s1]; }
+      if constexpr (NIN >= 3) { if (l2) p2 = l2[tx * (TS + 1) + row]; else if (q2) p2 = q2[(int64_t)i * s2]; }
+      dp[(int64_t)i * dstep] = f(p0, p1, p2);
+    }
+  }
+}
+
+template <class F>
+__global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileArgs a) {
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+  constexpr int TS = tile_edge<F>::value;
   extern __shared__ __align__(16) char smem[];
 
   // LDS slots are handed out in operand order to the operands that need one.
@@ -211,30 +284,8 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
     for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
   }
   const uint32_t a0 = ta * TS, b0 = tb * TS;
-  const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
-
-  if constexpr (NIN >= 1) if (l0) tile_stage<In0, TS>(a, 1, l0, off[1], a0, b0, tx, ty);
-  if constexpr (NIN >= 2) if (l1) tile_stage<In1, TS>(a, 2, l1, off[2], a0, b0, tx, ty);
-  if constexpr (NIN >= 3) if (l2) tile_stage<In2, TS>(a, 3, l2, off[3], a0, b0, tx, ty);
-  __syncthreads();
-
-  // coalesced along A: lane tx walks A, rows of the tile walk B
-  const uint32_t ai = a0 + tx;
-  Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + off[0];
-#pragma unroll
-  for (int i = 0; i < TS / ROWS; ++i) {
-    const int row = ty + i * ROWS;
-    const uint32_t bi = b0 + row;
-    if (ai < a.sizeA && bi < a.sizeB) {
-      In0 p0{};
-      In1 p1{};
-      In2 p2{};
-      if constexpr (NIN >= 1) p0 = tile_fetch<In0, TS>(a, 1, l0, off[1], ai, bi, tx, row);
-      if constexpr (NIN >= 2) p1 = tile_fetch<In1, TS>(a, 2, l1, off[2], ai, bi, tx, row);
-      if constexpr (NIN >= 3) p2 = tile_fetch<In2, TS>(a, 3, l2, off[3], ai, bi, tx, row);
-      dp[(int64_t)ai * a.strideA[0] + (int64_t)bi * a.strideB[0]] = f(p0, p1, p2);
-    }
-  }
+  if (a0 + TS <= a.sizeA && b0 + TS <= a.sizeB) tile_body<F, true>(f, a, off, a0, b0, l0, l1, l2);
+  else tile_body<F, false>(f, a, off, a0, b0, l0, l1, l2);
 }
 
 // ------------------------------------------------------------------ GENERAL

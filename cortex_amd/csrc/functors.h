@@ -120,10 +120,27 @@ template <class T, int OP> struct BinaryF {
   using In2 = T;
   using A = typename acc_of<T>::type;
   A xa, ya;
+  // Float tensors whose multipliers are +-1: x*xa and y*ya are exact in float,
+  // and a single float add, subtract, multiply or divide (correctly rounded)
+  // equals the double operation rounded once to float, so the widening can be
+  // skipped.  Comparisons and min/max see the same values either way.
+  int32_t narrow;
   __device__ __forceinline__ T operator()(T x, T y, T) const {
+    if constexpr (std::is_same<T, float>::value &&
+                  (OP == CT_BOP_ADD || OP == CT_BOP_SUB || OP == CT_BOP_MUL || OP == CT_BOP_DIV)) {
+      if (narrow) {
+        const float fx = xa < 0 ? -x : x, fy = ya < 0 ? -y : y;
+        if constexpr (OP == CT_BOP_ADD) return fx + fy;
+        else if constexpr (OP == CT_BOP_SUB) return fx - fy;
+        else if constexpr (OP == CT_BOP_MUL) return fx * fy;
+        else return fx / fy;
+      }
+    }
     return binary_value<T, OP, A>(w_mul((A)x, xa), w_mul((A)y, ya));
   }
 };
+
+template <class A> inline bool unit_magnitude(A v) { return v == (A)1 || v == (A)-1; }
 
 // ------------------------------------------------------------------ ternary select
 

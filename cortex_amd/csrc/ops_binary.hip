@@ -15,6 +15,7 @@ int binary_run(hipStream_t s, const BinaryCall& c) {
   // A scalar side has had its alpha folded in by the caller; its multiplier is 1.
   f.xa = c.x ? (A)jvm_cast<T>(c.x_alpha) : (A)1;
   f.ya = c.y ? (A)jvm_cast<T>(c.y_alpha) : (A)1;
+  f.narrow = unit_magnitude(f.xa) && unit_magnitude(f.ya);
   EwOperand ops[3] = {{c.dest, c.dest_dims, (int)sizeof(T), 0},
                       {c.x, c.x ? c.x_dims : nullptr, (int)sizeof(T), bits_of<T>(jvm_cast<T>(c.x_scalar))},
                       {c.y, c.y ? c.y_dims : nullptr, (int)sizeof(T), bits_of<T>(jvm_cast<T>(c.y_scalar))}};

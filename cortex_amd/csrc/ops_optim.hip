@@ -34,10 +34,10 @@ __global__ void __launch_bounds__(kBlock) adam_kernel(const AdamScalars s, const
   for (int u = 0; u < UNROLL; ++u) {
     const int64_t i = first + (int64_t)u * kBlock;
     if (i < n_vecs) {
-      gv[u] = reinterpret_cast<const V*>(g)[i];
-      pv[u] = reinterpret_cast<const V*>(p)[i];
-      mv[u] = reinterpret_cast<const V*>(m)[i];
-      vv[u] = reinterpret_cast<const V*>(v)[i];
+      gv[u] = nt_load(reinterpret_cast<const V*>(g) + i);
+      pv[u] = nt_load(reinterpret_cast<const V*>(p) + i);
+      mv[u] = nt_load(reinterpret_cast<const V*>(m) + i);
+      vv[u] = nt_load(reinterpret_cast<const V*>(v) + i);
     }
   }
 #pragma unroll
@@ -72,10 +72,10 @@ __global__ void __launch_bounds__(kBlock) adadelta_kernel(const AdadeltaScalars<
   for (int u = 0; u < UNROLL; ++u) {
     const int64_t i = first + (int64_t)u * kBlock;
     if (i < n_vecs) {
-      gv[u] = reinterpret_cast<const V*>(g)[i];
-      pv[u] = reinterpret_cast<const V*>(p)[i];
-      av[u] = reinterpret_cast<const V*>(gacc)[i];
-      dv[u] = reinterpret_cast<const V*>(dacc)[i];
+      gv[u] = nt_load(reinterpret_cast<const V*>(g) + i);
+      pv[u] = nt_load(reinterpret_cast<const V*>(p) + i);
+      av[u] = nt_load(reinterpret_cast<const V*>(gacc) + i);
+      dv[u] = nt_load(reinterpret_cast<const V*>(dacc) + i);
     }
   }
 #pragma unroll

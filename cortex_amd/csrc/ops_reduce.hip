@@ -131,7 +131,7 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
     const int64_t nv = a.k / VEC;
     int64_t i = lane;
     for (; i + TPR < nv; i += 2 * TPR) {
-      const V x0 = row[i], x1 = row[i + TPR];
+      const V x0 = nt_load(row + i), x1 = nt_load(row + i + TPR);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         acc0 = red_combine<A, RK>(acc0, red_value<T, A, RK>(x0.v[e], alpha));
@@ -139,7 +139,7 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
       }
     }
     if (i < nv) {
-      const V x0 = row[i];
+      const V x0 = nt_load(row + i);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) acc0 = red_combine<A, RK>(acc0, red_value<T, A, RK>(x0.v[e], alpha));
     }
@@ -204,19 +204,22 @@ __global__ void __launch_bounds__(kBlock) reduce_col_kernel(const ColArgs a, con
   int64_t r1 = r0 + a.rows_per_seg;
   if (r1 > a.k) r1 = a.k;
   if (live) {
-    const T* p = reinterpret_cast<const T*>(a.in) + base + col;
+    // each wave owns rows r0+wave, r0+wave+WAVES, ...; UN loads are in flight per lane
+    constexpr int UN = 8;
+    const int64_t step = (int64_t)WAVES * a.rstride;
+    const T* p = reinterpret_cast<const T*>(a.in) + base + col + (r0 + wave) * a.rstride;
     int64_t r = r0 + wave;
-    for (; r + WAVES < r1; r += 2 * WAVES) {
-      const V x0 = *reinterpret_cast<const V*>(p + r * a.rstride);
-      const V x1 = *reinterpret_cast<const V*>(p + (r + WAVES) * a.rstride);
+    for (; r + (UN - 1) * WAVES < r1; r += UN * WAVES, p += UN * step) {
+      V x[UN];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x0.v[e], alpha));
-        acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x1.v[e], alpha));
-      }
+      for (int j = 0; j < UN; ++j) x[j] = nt_load(reinterpret_cast<const V*>(p + j * step));
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x[j].v[e], alpha));
     }
-    if (r < r1) {
-      const V x0 = *reinterpret_cast<const V*>(p + r * a.rstride);
+    for (; r < r1; r += WAVES, p += step) {
+      const V x0 = nt_load(reinterpret_cast<const V*>(p));
 #pragma unroll
       for (int e = 0; e < VEC; ++e) acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x0.v[e], alpha));
     }

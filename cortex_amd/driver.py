@@ -1,0 +1,353 @@
+"""The ``:hip`` compute driver: a Python mirror of the reference's driver
+protocols for the tensor-math path, on top of the C ABI.
+
+It provides what ``cortex.compute.driver`` asks of a backend
+(``src/cortex/compute/driver.clj:46-221``) with the same names and argument
+meaning:
+
+* :class:`HipDriver`   -- ``PDriver``: ``get_devices``, ``allocate_host_buffer``
+* :class:`HipDevice`   -- ``PDevice``: ``memory_info``, ``create_stream``,
+  ``allocate_device_buffer``
+* :class:`HipStream`   -- ``PStream``: ``copy_host_to_device``,
+  ``copy_device_to_host``, ``copy_device_to_device``, ``memset``,
+  ``create_event``, ``sync_event``; and the twelve ``TensorMath`` methods of
+  ``src/cortex/tensor/math.clj:14-104`` (template:
+  ``src/cortex/compute/cuda/tensor_math.clj:289-631``)
+* :class:`DeviceBuffer` -- ``PBuffer``: ``sub_buffer``, ``alias``,
+  ``partially_alias`` (``src/cortex/compute/cuda/driver.clj:465-510``)
+* :class:`Event`       -- ``PEvent``: ``wait_for_event``
+
+Dimensions are the reference's ``{:shape :strides}`` maps as Python dicts
+``{"shape": [...], "strides": [...]}``; a shape entry may be an int32
+:class:`DeviceBuffer`-backed tensor (anything with ``.buffer``) for an
+indirectly addressed dimension.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence
+
+import numpy as np
+
+from . import capi
+
+DATATYPES = ("byte", "short", "int", "long", "float", "double", "ubyte")
+NUMPY_OF = {"byte": np.int8, "short": np.int16, "int": np.int32, "long": np.int64, "float": np.float32,
+            "double": np.float64, "ubyte": np.uint8}
+DATATYPE_OF_NUMPY = {np.dtype(v): k for k, v in NUMPY_OF.items()}
+
+
+def dtype_size(datatype: str) -> int:
+    return capi.DTYPE_SIZES[capi.DTYPE_CODES[datatype]]
+
+
+class DeviceBuffer:
+    """A typed range of device memory.  The owner frees it on ``release``;
+    sub-buffers share the owner's memory and own nothing
+    (``src/cortex/compute/cuda/driver.clj:502-506``)."""
+
+    def __init__(self, device: "HipDevice", ptr: int, ecount: int, datatype: str, owner: Optional["DeviceBuffer"] = None):
+        self.device = device
+        self.ptr = ptr
+        self._ecount = int(ecount)
+        self.datatype = datatype
+        self._owner = owner
+        self._released = False
+
+    def ecount(self) -> int:
+        return self._ecount
+
+    def get_datatype(self) -> str:
+        return self.datatype
+
+    @property
+    def nbytes(self) -> int:
+        return self._ecount * dtype_size(self.datatype)
+
+    def sub_buffer(self, offset: int, length: int) -> "DeviceBuffer":
+        """``drv/sub-buffer`` (``src/cortex/compute/driver.clj:206-214``)."""
+        offset, length = int(offset), int(length)
+        if offset < 0 or length < 0 or offset + length > self._ecount:
+            raise ValueError(f"Sub buffer out of range: offset {offset} length {length} of {self._ecount}")
+        return DeviceBuffer(self.device, self.ptr + offset * dtype_size(self.datatype), length, self.datatype,
+                            owner=self._owner or self)
+
+    def alias(self, other: "DeviceBuffer") -> bool:
+        """Same start address (``cuda/driver.clj:465-472``)."""
+        return self.ptr == other.ptr
+
+    def partially_alias(self, other: "DeviceBuffer") -> bool:
+        """Overlapping byte ranges that do not start at the same address
+        (``cuda/driver.clj:473-486``)."""
+        a0, a1 = self.ptr, self.ptr + self.nbytes
+        b0, b1 = other.ptr, other.ptr + other.nbytes
+        if a0 == b0:
+            return False
+        return a0 < b1 and b0 < a1
+
+    def release(self) -> None:
+        if self._owner is None and not self._released and self.ptr:
+            capi.call("ct_free", self.ptr)
+            self._released = True
+
+
+class HostBuffer:
+    """Pinned host memory exposed as a numpy array (``allocate-host-buffer``)."""
+
+    def __init__(self, ecount: int, datatype: str):
+        self.datatype = datatype
+        self._ecount = int(ecount)
+        p = C.c_void_p()
+        nbytes = max(1, self._ecount * dtype_size(datatype))
+        capi.call("ct_host_alloc", C.byref(p), nbytes)
+        self.ptr = p.value
+        raw = (C.c_char * nbytes).from_address(self.ptr)
+        self.array = np.frombuffer(raw, dtype=NUMPY_OF[datatype], count=self._ecount)
+        self._released = False
+
+    def ecount(self) -> int:
+        return self._ecount
+
+    def get_datatype(self) -> str:
+        return self.datatype
+
+    def release(self) -> None:
+        if not self._released:
+            self.array = None
+            capi.call("ct_host_free", self.ptr)
+            self._released = True
+
+
+class Event:
+    def __init__(self, handle: int):
+        self.handle = handle
+
+    def wait_for_event(self) -> None:
+        """``PEvent wait-for-event``: blocks the host."""
+        capi.call("ct_event_sync", self.handle)
+
+    def release(self) -> None:
+        if self.handle:
+            capi.call("ct_event_destroy", self.handle)
+            self.handle = None
+
+
+def _dims_struct(dims: dict) -> capi.CtDims:
+    shape, index = [], []
+    for entry in dims["shape"]:
+        if isinstance(entry, (int, np.integer)):
+            shape.append(int(entry))
+            index.append(None)
+        else:  # an index tensor: int32, dense (cpu/tensor_math.clj:68-80)
+            buf = entry.buffer
+            if buf.get_datatype() != "int":
+                raise TypeError("Index buffers must be integer tensors")
+            shape.append(int(buf.ecount()))
+            index.append(buf.ptr)
+    return capi.make_dims(shape, dims["strides"], index)
+
+
+def _arg_order_indexes(arg_order: Sequence[str]):
+    """``arg-order->indexes`` (``cpu/tensor_math.clj:500-504``)."""
+    pos = {name: i for i, name in enumerate(arg_order)}
+    return capi.arg_idx([pos["x"], pos["y"], pos["z"]])
+
+
+class HipStream:
+    """A HIP stream.  Calls are ordered on the stream and asynchronous to the
+    host; observe completion through ``create_event().wait_for_event()`` or
+    ``sync``."""
+
+    def __init__(self, device: "HipDevice", handle: Optional[int]):
+        self.device = device
+        self.handle = handle
+
+    def get_device(self) -> "HipDevice":
+        return self.device
+
+    def get_driver(self) -> "HipDriver":
+        return self.device.driver
+
+    # -- PStream ----------------------------------------------------------
+    def copy_host_to_device(self, host: HostBuffer, host_offset: int, dev: DeviceBuffer, dev_offset: int, n: int) -> None:
+        self._check_copy(host, host_offset, dev, dev_offset, n)
+        es = dtype_size(dev.datatype)
+        capi.call("ct_memcpy_async", dev.ptr + dev_offset * es, host.ptr + host_offset * es, n * es, capi.COPY_H2D,
+                  self.handle)
+
+    def copy_device_to_host(self, dev: DeviceBuffer, dev_offset: int, host: HostBuffer, host_offset: int, n: int) -> None:
+        self._check_copy(host, host_offset, dev, dev_offset, n)
+        es = dtype_size(dev.datatype)
+        capi.call("ct_memcpy_async", host.ptr + host_offset * es, dev.ptr + dev_offset * es, n * es, capi.COPY_D2H,
+                  self.handle)
+
+    def copy_device_to_device(self, src: DeviceBuffer, src_offset: int, dst: DeviceBuffer, dst_offset: int, n: int) -> None:
+        self._check_copy(src, src_offset, dst, dst_offset, n)
+        es = dtype_size(dst.datatype)
+        capi.call("ct_memcpy_async", dst.ptr + dst_offset * es, src.ptr + src_offset * es, n * es, capi.COPY_D2D,
+                  self.handle)
+
+    @staticmethod
+    def _check_copy(a, a_offset, b, b_offset, n) -> None:
+        # cuda/driver.clj:901-919: datatypes must match and both ranges must fit
+        if a.get_datatype() != b.get_datatype():
+            raise TypeError(f"Copy datatypes differ: {a.get_datatype()} vs {b.get_datatype()}")
+        if a_offset < 0 or b_offset < 0 or n < 0 or a_offset + n > a.ecount() or b_offset + n > b.ecount():
+            raise ValueError("Copy out of range")
+
+    def memset(self, dev: DeviceBuffer, offset: int, value, n: int) -> None:
+        if offset < 0 or n < 0 or offset + n > dev.ecount():
+            raise ValueError("memset out of range")
+        capi.call("ct_memset", self.handle, dev.ptr + offset * dtype_size(dev.datatype),
+                  capi.DTYPE_CODES[dev.datatype], float(value), n)
+
+    def create_event(self) -> Event:
+        h = C.c_void_p()
+        capi.call("ct_event_record", C.byref(h), self.handle)
+        return Event(h.value)
+
+    def sync_event(self, event: Event) -> None:
+        """Makes this stream wait for ``event`` (``PStream sync-event``)."""
+        capi.call("ct_stream_wait_event", self.handle, event.handle)
+
+    def sync(self) -> None:
+        """``drv/sync-stream`` (``compute/driver.clj:217-221``)."""
+        capi.call("ct_stream_sync", self.handle)
+
+    def release(self) -> None:
+        if self.handle:
+            capi.call("ct_stream_destroy", self.handle)
+            self.handle = None
+
+    # -- TensorMath (src/cortex/tensor/math.clj:14-104) ---------------------
+    def assign_constant(self, buffer, dimensions, value, n_elems) -> None:
+        capi.call("ct_assign_constant", self.handle, buffer.ptr, C.byref(_dims_struct(dimensions)),
+                  capi.DTYPE_CODES[buffer.datatype], float(value), int(n_elems))
+
+    def assign(self, dest, dest_dims, src, src_dims, n_elems) -> None:
+        capi.call("ct_assign", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), capi.DTYPE_CODES[dest.datatype],
+                  src.ptr, C.byref(_dims_struct(src_dims)), capi.DTYPE_CODES[src.datatype], int(n_elems))
+
+    def unary_accum(self, dest, dest_dims, alpha, op, n_elems) -> None:
+        capi.call("ct_unary_accum", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), float(alpha),
+                  capi.UNARY_OPS[op], capi.DTYPE_CODES[dest.datatype], int(n_elems))
+
+    def unary_op(self, dest, dest_dims, x, x_dims, alpha, op, n_elems) -> None:
+        capi.call("ct_unary_op", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), x.ptr,
+                  C.byref(_dims_struct(x_dims)), float(alpha), capi.UNARY_OPS[op], capi.DTYPE_CODES[dest.datatype],
+                  int(n_elems))
+
+    def binary_accum_constant(self, dest, dest_dims, dest_alpha, scalar, n_elems, operation, reverse_operands) -> None:
+        capi.call("ct_binary_accum_constant", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), float(dest_alpha),
+                  float(scalar), int(n_elems), capi.BINARY_OPS[operation], int(bool(reverse_operands)),
+                  capi.DTYPE_CODES[dest.datatype])
+
+    def binary_op_constant(self, dest, dest_dims, x, x_dims, x_alpha, scalar, n_elems, operation, reverse_operands) -> None:
+        capi.call("ct_binary_op_constant", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), x.ptr,
+                  C.byref(_dims_struct(x_dims)), float(x_alpha), float(scalar), int(n_elems),
+                  capi.BINARY_OPS[operation], int(bool(reverse_operands)), capi.DTYPE_CODES[dest.datatype])
+
+    def binary_accum(self, dest, dest_dims, dest_alpha, y, y_dims, y_alpha, n_elems, operation, reverse_operands,
+                     dest_requires_cas) -> None:
+        capi.call("ct_binary_accum", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), float(dest_alpha), y.ptr,
+                  C.byref(_dims_struct(y_dims)), float(y_alpha), int(n_elems), capi.BINARY_OPS[operation],
+                  int(bool(reverse_operands)), int(bool(dest_requires_cas)), capi.DTYPE_CODES[dest.datatype])
+
+    def binary_op(self, dest, dest_dims, x, x_dims, x_alpha, y, y_dims, y_alpha, n_elems, operation) -> None:
+        capi.call("ct_binary_op", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), x.ptr,
+                  C.byref(_dims_struct(x_dims)), float(x_alpha), y.ptr, C.byref(_dims_struct(y_dims)), float(y_alpha),
+                  int(n_elems), capi.BINARY_OPS[operation], capi.DTYPE_CODES[dest.datatype])
+
+    def ternary_op(self, dest, dest_dims, x, x_dims, x_alpha, y, y_dims, y_alpha, z, z_dims, z_alpha, n_elems,
+                   operation) -> None:
+        capi.call("ct_ternary_op", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), x.ptr,
+                  C.byref(_dims_struct(x_dims)), float(x_alpha), y.ptr, C.byref(_dims_struct(y_dims)), float(y_alpha),
+                  z.ptr, C.byref(_dims_struct(z_dims)), float(z_alpha), int(n_elems), capi.TERNARY_OPS[operation],
+                  capi.DTYPE_CODES[dest.datatype])
+
+    def ternary_op_constant(self, dest, dest_dims, a, a_dims, a_alpha, b, b_dims, b_alpha, constant, n_elems, operation,
+                            arg_order) -> None:
+        capi.call("ct_ternary_op_constant", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), a.ptr,
+                  C.byref(_dims_struct(a_dims)), float(a_alpha), b.ptr, C.byref(_dims_struct(b_dims)), float(b_alpha),
+                  float(constant), int(n_elems), capi.TERNARY_OPS[operation], _arg_order_indexes(arg_order),
+                  capi.DTYPE_CODES[dest.datatype])
+
+    def ternary_op_constant_constant(self, dest, dest_dims, a, a_dims, a_alpha, const_1, const_2, n_elems, operation,
+                                     arg_order) -> None:
+        capi.call("ct_ternary_op_constant_constant", self.handle, dest.ptr, C.byref(_dims_struct(dest_dims)), a.ptr,
+                  C.byref(_dims_struct(a_dims)), float(a_alpha), float(const_1), float(const_2), int(n_elems),
+                  capi.TERNARY_OPS[operation], _arg_order_indexes(arg_order), capi.DTYPE_CODES[dest.datatype])
+
+    def unary_reduce(self, output, output_dims, input_alpha, input, input_dims, op) -> None:
+        capi.call("ct_unary_reduce", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), float(input_alpha),
+                  input.ptr, C.byref(_dims_struct(input_dims)), capi.REDUCE_OPS[op], capi.DTYPE_CODES[output.datatype])
+
+    # -- optimizers ---------------------------------------------------------
+    def adam_step(self, alpha, beta1, beta2, epsilon, pow_beta1_t, pow_beta2_t, gradient_alpha, gradient, parameters,
+                  m, v, n) -> None:
+        capi.call("ct_adam_step", self.handle, capi.DTYPE_CODES[gradient.datatype], float(alpha), float(beta1),
+                  float(beta2), float(epsilon), float(pow_beta1_t), float(pow_beta2_t), float(gradient_alpha),
+                  gradient.ptr, parameters.ptr, m.ptr, v.ptr, int(n))
+
+    def adadelta_step(self, decay, epsilon, grad_accum, dx_accum, gradient_alpha, gradient, parameters, n) -> None:
+        capi.call("ct_adadelta_step", self.handle, capi.DTYPE_CODES[gradient.datatype], float(decay), float(epsilon),
+                  grad_accum.ptr, dx_accum.ptr, float(gradient_alpha), gradient.ptr, parameters.ptr, int(n))
+
+
+class HipDevice:
+    def __init__(self, driver: "HipDriver", index: int):
+        self.driver = driver
+        self.index = index
+
+    def get_driver(self) -> "HipDriver":
+        return self.driver
+
+    def make_current(self) -> None:
+        capi.call("ct_set_device", self.index)
+
+    def memory_info(self) -> dict:
+        self.make_current()
+        free, total = C.c_size_t(), C.c_size_t()
+        capi.call("ct_memory_info", C.byref(free), C.byref(total))
+        return {"free": free.value, "total": total.value}
+
+    def create_stream(self) -> HipStream:
+        self.make_current()
+        h = C.c_void_p()
+        capi.call("ct_stream_create", C.byref(h))
+        return HipStream(self, h.value)
+
+    def default_stream(self) -> HipStream:
+        return HipStream(self, None)
+
+    def allocate_device_buffer(self, elem_count: int, elem_type: str) -> DeviceBuffer:
+        if elem_type not in capi.DTYPE_CODES:
+            raise TypeError(f"Unknown datatype {elem_type!r}")
+        self.make_current()
+        p = C.c_void_p()
+        capi.call("ct_malloc", C.byref(p), max(1, int(elem_count) * dtype_size(elem_type)))
+        return DeviceBuffer(self, p.value, elem_count, elem_type)
+
+
+class HipDriver:
+    """``PDriver`` for the HIP backend."""
+
+    type = "hip"
+
+    def __init__(self):
+        n = C.c_int(0)
+        capi.call("ct_device_count", C.byref(n))
+        self._devices = [HipDevice(self, i) for i in range(n.value)]
+
+    def get_devices(self):
+        return list(self._devices)
+
+    def default_device(self) -> HipDevice:
+        if not self._devices:
+            raise RuntimeError("No HIP device is visible")
+        return self._devices[0]
+
+    def allocate_host_buffer(self, elem_count: int, elem_type: str, usage_type: str = "one-time") -> HostBuffer:
+        if usage_type not in ("one-time", "reusable"):
+            raise ValueError("Usage type is not in expected set")
+        return HostBuffer(elem_count, elem_type)

@@ -10,17 +10,15 @@ offset, as the reference's sub-buffers).
 from __future__ import annotations
 
 import ctypes as C
-import subprocess
 from pathlib import Path
 from typing import List, Optional, Sequence
 
 import numpy as np
 
 from cortex_amd import capi
+from oracle import binding as oracle_binding
 
 ROOT = Path(__file__).resolve().parent.parent
-ORACLE_DIR = ROOT / "oracle"
-ORACLE_LIB = ORACLE_DIR / "libcortex_cpu_oracle.so"
 
 NP_DTYPES = {capi.I8: np.int8, capi.I16: np.int16, capi.I32: np.int32, capi.I64: np.int64,
              capi.F32: np.float32, capi.F64: np.float64, capi.U8: np.uint8}
@@ -32,37 +30,11 @@ _P, _D, _I, _L = C.c_void_p, C.c_double, C.c_int, C.c_int64
 _DP = C.POINTER(capi.CtDims)
 
 
-def build_oracle() -> Path:
-    src = ORACLE_DIR / "cortex_cpu_oracle.cpp"
-    if not ORACLE_LIB.exists() or ORACLE_LIB.stat().st_mtime < src.stat().st_mtime:
-        subprocess.run(["make", "-C", str(ORACLE_DIR)], check=True, capture_output=True)
-    return ORACLE_LIB
-
-
-_oracle = None
-
-
 def oracle_lib() -> C.CDLL:
-    global _oracle
-    if _oracle is None:
-        lib = C.CDLL(str(build_oracle()))
-        for name, argtypes in capi.PROTOTYPES.items():
-            oname = "co_" + name[3:]
-            if not hasattr(lib, oname):
-                continue
-            fn = getattr(lib, oname)
-            fn.argtypes = argtypes[1:]  # the oracle takes no stream
-            fn.restype = C.c_int
-        lib.co_last_error.restype = C.c_char_p
-        lib.co_elem_address.argtypes = [C.POINTER(_DP), _I, _I, _L, C.POINTER(_L), C.POINTER(_I)]
-        lib.co_elem_address.restype = C.c_int
-        lib.co_num_threads.restype = C.c_int
-        _oracle = lib
-    return _oracle
+    return oracle_binding.lib()
 
 
-class OracleError(RuntimeError):
-    pass
+OracleError = oracle_binding.OracleError
 
 
 class Buf:
@@ -172,10 +144,7 @@ class Side:
             capi.call("ct_" + name, self.stream, *args)
             capi.call("ct_stream_sync", self.stream)
         else:
-            lib = oracle_lib()
-            rc = getattr(lib, "co_" + name)(*args)
-            if rc != 0:
-                raise OracleError(lib.co_last_error().decode())
+            oracle_binding.call(name, *args)
 
 
 def _pd(side: Side, v: View):
