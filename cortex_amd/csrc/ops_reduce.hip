@@ -33,7 +33,10 @@ using namespace cthip;
 
 namespace {
 
-enum RedKind { RK_MAX = 0, RK_MIN = 1, RK_SUM = 2, RK_SUMSQ = 3 };
+// The reduction is a template parameter (the values are the ct_reduce_op_t codes), so the
+// kernels carry no run-time branch on it.
+enum RedKind { RK_MAX = CT_ROP_MAX, RK_MIN = CT_ROP_MIN, RK_SUM = CT_ROP_SUM, RK_MEAN = CT_ROP_MEAN,
+               RK_MAG = CT_ROP_MAGNITUDE, RK_SUMSQ = CT_ROP_MAGNITUDE_SQUARED };
 
 __device__ __forceinline__ double jmax(double a, double b) {
   if (a != a) return a;
@@ -68,17 +71,19 @@ template <class A, int RK> __device__ __forceinline__ A red_combine(A a, A b) {
 }
 template <class T, class A, int RK> __device__ __forceinline__ A red_value(T x, A alpha) {
   const A v = w_mul(alpha, (A)x);
-  if constexpr (RK == RK_SUMSQ) return w_mul(v, v);
+  if constexpr (RK == RK_SUMSQ || RK == RK_MAG) return w_mul(v, v);
   else return v;
 }
 // Final cast, with mean and magnitude applied (cpu/tensor_math.clj:610-622).
-template <class T, class A> __device__ __forceinline__ T red_finish(A acc, int op, int64_t count) {
-  if (op == CT_ROP_MEAN) {
+template <class T, class A, int RK> __device__ __forceinline__ T red_finish(A acc, int64_t count) {
+  if constexpr (RK == RK_MEAN) {
     if constexpr (std::is_same<A, double>::value) return jvm_cast<T>(acc / (double)count);
     else return jvm_ratio_cast<T>(acc, count);
+  } else if constexpr (RK == RK_MAG) {
+    return jvm_cast<T>(sqrt((double)acc));
+  } else {
+    return jvm_cast<T>(acc);
   }
-  if (op == CT_ROP_MAGNITUDE) return jvm_cast<T>(sqrt((double)acc));
-  return jvm_cast<T>(acc);
 }
 
 template <class A> __device__ __forceinline__ A shfl_xor_any(A v, int mask) {
@@ -158,7 +163,7 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
     }
   }
   if (live && lane == 0)
-    reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc, a.op, a.k);
+    reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc, a.k);
 }
 
 struct ColArgs {
@@ -235,7 +240,7 @@ __global__ void __launch_bounds__(kBlock) reduce_col_kernel(const ColArgs a, con
 #pragma unroll
       for (int w = 0; w < WAVES - 1; ++w) acc[e] = red_combine<A, RK>(acc[e], lds[w][e * 64 + lane]);
       const int64_t p = pbase + (int64_t)(col + e) * a.u_pmul;
-      if (a.n_seg == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc[e], a.op, a.k);
+      if (a.n_seg == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc[e], a.k);
       else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc[e];
     }
   }
@@ -249,7 +254,7 @@ __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const ColArgs a) 
   const A* part = reinterpret_cast<const A*>(a.partials);
   A acc = part[p];
   for (uint32_t s = 1; s < a.n_seg; ++s) acc = red_combine<A, RK>(acc, part[(int64_t)s * a.n_out + p]);
-  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc, a.op, a.k);
+  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc, a.k);
 }
 
 struct AnyArgs {
@@ -274,7 +279,7 @@ __global__ void __launch_bounds__(kBlock) reduce_any_kernel(const AnyArgs a, con
   A acc = red_value<T, A, RK>(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start)], alpha);
   for (int64_t i = 1; i < a.k; ++i)
     acc = red_combine<A, RK>(acc, red_value<T, A, RK>(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start + i)], alpha));
-  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A>(acc, a.op, a.k);
+  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc, a.k);
 }
 
 // ------------------------------------------------------------------ host planning
@@ -444,9 +449,9 @@ int reduce_dispatch(hipStream_t st, void* out, const ct_dims* od, double alpha, 
   switch (op) {
     case CT_ROP_MAX: return reduce_typed<T, RK_MAX>(st, out, od, alpha, in, id, op);
     case CT_ROP_MIN: return reduce_typed<T, RK_MIN>(st, out, od, alpha, in, id, op);
-    case CT_ROP_SUM:
-    case CT_ROP_MEAN: return reduce_typed<T, RK_SUM>(st, out, od, alpha, in, id, op);
-    case CT_ROP_MAGNITUDE:
+    case CT_ROP_SUM: return reduce_typed<T, RK_SUM>(st, out, od, alpha, in, id, op);
+    case CT_ROP_MEAN: return reduce_typed<T, RK_MEAN>(st, out, od, alpha, in, id, op);
+    case CT_ROP_MAGNITUDE: return reduce_typed<T, RK_MAG>(st, out, od, alpha, in, id, op);
     case CT_ROP_MAGNITUDE_SQUARED: return reduce_typed<T, RK_SUMSQ>(st, out, od, alpha, in, id, op);
     default: return set_error(CT_ERR_INVALID, "unknown reduction operation %d", op);
   }

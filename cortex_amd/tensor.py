@@ -1,0 +1,490 @@
+"""Backend-neutral tensor API: a Python mirror of the front half of
+``src/cortex/tensor.clj`` (lines 1-884) for the tensor-math path.
+
+It does what the reference's tensor layer does before it reaches a backend:
+validation, alias detection, scalar folding, the ``:-`` to ``:+`` rewrite, the
+``x * const`` strength reduction, the choice between the plain / accumulate /
+constant variants, and the ``arg-order`` bookkeeping of ``ternary-op!``.  The
+backend is whatever *stream* is bound (:func:`tensor_context`); it must
+implement the ``TensorMath`` methods (``src/cortex/tensor/math.clj:14-104``)
+and the ``PStream`` copies.  :class:`cortex_amd.driver.HipStream` is the HIP
+backend; the tests bind a CPU-oracle stream to the very same functions.
+
+Names follow the reference with ``!`` dropped and ``-`` turned into ``_``.
+"""
+from __future__ import annotations
+
+import contextlib
+import contextvars
+import itertools
+import math
+from typing import Sequence
+
+import numpy as np
+
+from . import dimensions as dims
+
+_stream = contextvars.ContextVar("cortex_stream", default=None)
+_datatype = contextvars.ContextVar("cortex_datatype", default="double")
+
+UNARY_OPERATIONS = ["floor", "ceil", "round", "-", "tanh", "logistic", "exp", "sqrt", "noop"]  # tensor.clj:607-609
+BINARY_OPERATIONS = ["+", "-", "*", "/", "max", "min", "bit-and", "bit-xor", "eq", ">", ">=", "<", "<="]  # :764-765
+UNARY_REDUCTION_OPERATIONS = ["max", "min", "sum", "mean", "magnitude-squared", "magnitude"]  # :857-858
+
+NUMPY_OF = {"byte": np.int8, "short": np.int16, "int": np.int32, "long": np.int64, "float": np.float32,
+            "double": np.float64, "ubyte": np.uint8}
+
+
+class TensorError(ValueError):
+    """Stands in for the ``ex-info`` of ``when-not-error``."""
+
+
+@contextlib.contextmanager
+def tensor_context(stream, datatype: str = "double"):
+    """Binds ``*stream*`` and ``*datatype*`` (``tensor.clj:89-111``;
+    ``src/cortex/verify/tensor.clj:11-17``)."""
+    t1 = _stream.set(stream)
+    t2 = _datatype.set(datatype)
+    try:
+        yield stream
+    finally:
+        _stream.reset(t1)
+        _datatype.reset(t2)
+
+
+def check_stream():
+    s = _stream.get()
+    if s is None:
+        raise TensorError("Tensor stream is nil")
+    return s
+
+
+def current_datatype() -> str:
+    return _datatype.get()
+
+
+class Tensor:
+    """``(defrecord Tensor [device dimensions buffer])`` (``tensor.clj:174-195``)."""
+
+    def __init__(self, device, dimensions, buffer):
+        self.device = device
+        self.dimensions = dimensions
+        self.buffer = buffer
+
+    def get_datatype(self) -> str:
+        return self.buffer.get_datatype()
+
+    def ecount(self) -> int:
+        return dims.ecount(self.dimensions)
+
+    def shape(self):
+        return dims.shape(self.dimensions)
+
+    def _with(self, dimensions=None, buffer=None) -> "Tensor":
+        return Tensor(self.device, dimensions if dimensions is not None else self.dimensions,
+                      buffer if buffer is not None else self.buffer)
+
+
+def is_tensor(x) -> bool:
+    return isinstance(x, Tensor)
+
+
+def _is_number(x) -> bool:
+    return isinstance(x, (int, float, np.integer, np.floating)) and not isinstance(x, bool)
+
+
+def ecount(t) -> int:
+    return t.ecount()
+
+
+def shape(t):
+    return t.shape()
+
+
+def get_datatype(t) -> str:
+    return t.get_datatype()
+
+
+def dense(t: Tensor) -> bool:
+    return dims.dense(t.dimensions)
+
+
+def _dtype_cast(value, datatype: str):
+    """``drv/dtype-cast`` (``src/cortex/compute/driver.clj:17-43``) for scalars
+    folded on the host."""
+    if datatype in ("float", "double"):
+        return float(np.float32(value)) if datatype == "float" else float(value)
+    return int(value)
+
+
+# ---------------------------------------------------------------- construction
+
+def to_tensor(data, datatype: str = None) -> Tensor:
+    """``->tensor`` (``tensor.clj:415-435``): uploads nested data."""
+    datatype = datatype or current_datatype()
+    stream = check_stream()
+    arr = np.asarray(data)
+    flat = arr.astype(NUMPY_OF[datatype]).reshape(-1)
+    device = stream.get_device()
+    driver = device.get_driver()
+    host = driver.allocate_host_buffer(flat.size, datatype)
+    dev = device.allocate_device_buffer(flat.size, datatype)
+    host.array[...] = flat
+    stream.copy_host_to_device(host, 0, dev, 0, flat.size)
+    stream.sync()
+    host.release()
+    return Tensor(device, dims.dimensions(list(arr.shape)), dev)
+
+
+def new_tensor(shape_: Sequence[int], datatype: str = None, init_value=0) -> Tensor:
+    """``new-tensor`` (``tensor.clj:438-450``)."""
+    datatype = datatype or current_datatype()
+    stream = check_stream()
+    n = int(np.prod(shape_)) if len(shape_) else 1
+    device = stream.get_device()
+    dev = device.allocate_device_buffer(n, datatype)
+    if init_value is not None:
+        stream.memset(dev, 0, 0, n)
+    return Tensor(device, dims.dimensions(list(shape_)), dev)
+
+
+def as_dense(t: Tensor):
+    return t if dense(t) and dims.access_increasing(t.dimensions) else None
+
+
+def make_dense(t: Tensor) -> Tensor:
+    d = as_dense(t)
+    if d is not None:
+        return d
+    out = new_tensor(shape(t), datatype=t.get_datatype(), init_value=None)
+    assign(out, t)
+    return out
+
+
+def to_array_of_type(t: Tensor, datatype: str) -> np.ndarray:
+    """``copy-to-java-type`` (``tensor.clj:375-395``)."""
+    d = make_dense(t)
+    n = d.ecount()
+    stream = check_stream()
+    host = stream.get_driver().allocate_host_buffer(n, d.get_datatype())
+    stream.copy_device_to_host(d.buffer, 0, host, 0, n)
+    stream.create_event().wait_for_event()
+    out = np.array(host.array, dtype=NUMPY_OF[datatype])
+    host.release()
+    return out
+
+
+def to_double_array(t: Tensor) -> np.ndarray:
+    return to_array_of_type(t, "double")
+
+
+# ---------------------------------------------------------------- views
+
+def in_place_reshape(t: Tensor, shape_) -> Tensor:
+    return t._with(dimensions=dims.in_place_reshape(t.dimensions, list(shape_)))
+
+
+def as_vector(t: Tensor):
+    """``PVectorView as-vector`` (``tensor.clj:1647-1650``)."""
+    if dense(t):
+        return t._with(dimensions=dims.dimensions([t.ecount()]))
+    return None
+
+
+def to_vector(t: Tensor) -> Tensor:
+    d = make_dense(t)
+    return d._with(dimensions=dims.dimensions([d.ecount()]))
+
+
+def as_2d_matrix(t: Tensor) -> Tensor:
+    return in_place_reshape(t, dims.to_2d_shape(t.dimensions))
+
+
+def as_batch_matrix(t: Tensor) -> Tensor:
+    return in_place_reshape(t, dims.to_batch_shape(t.dimensions))
+
+
+def transpose(t: Tensor, reorder_vec) -> Tensor:
+    """``transpose`` (``tensor.clj:453-459``): a view; no data moves."""
+    return t._with(dimensions=dims.transpose(t.dimensions, list(reorder_vec)))
+
+
+def select(t: Tensor, *args) -> Tensor:
+    """``select`` (``tensor.clj:462-477``)."""
+    res = dims.select(t.dimensions, *args)
+    off = int(res["elem-offset"])
+    buf = t.buffer.sub_buffer(off, t.buffer.ecount() - off)
+    return t._with(dimensions=res["dimensions"], buffer=buf)
+
+
+def subvector(t: Tensor, offset: int, length: int = None) -> Tensor:
+    if offset < 0:
+        raise TensorError("Offset must be >= 0")
+    v = as_vector(t)
+    stop = offset + length if length is not None else v.ecount()
+    return select(v, list(range(offset, stop)))
+
+
+def submatrix(t: Tensor, row_start, row_length, col_start, col_length) -> Tensor:
+    """``submatrix`` (``tensor.clj:490-513``)."""
+    t2 = as_2d_matrix(t)
+    n_rows, n_cols = t2.shape()
+    d = t2.dimensions
+    rev_shape, rev_strides = list(reversed(d["shape"])), list(reversed(d["strides"]))
+    addr = dims.elem_idx_to_addr(rev_shape, rev_strides, rev_shape, row_start * n_cols + col_start)
+    buf = t2.buffer.sub_buffer(addr, t2.buffer.ecount() - addr)
+    return t2._with(dimensions={"shape": [row_length, col_length], "strides": list(d["strides"])}, buffer=buf)
+
+
+def rows(t: Tensor):
+    n_rows, n_cols = dims.to_2d_shape(t.dimensions)
+    return [select(t, r, list(range(n_cols))) for r in range(n_rows)]
+
+
+def columns(t: Tensor):
+    n_rows, n_cols = dims.to_2d_shape(t.dimensions)
+    return [select(t, list(range(n_rows)), c) for c in range(n_cols)]
+
+
+# ---------------------------------------------------------------- checks
+
+def _ensure_datatypes(datatype, *args) -> None:
+    if not all(a.get_datatype() == datatype for a in args):
+        raise TensorError(f"Not all arguments match required datatype {datatype}: {[a.get_datatype() for a in args]}")
+
+
+def _ensure_same_device(*args) -> None:
+    if not all(a.device is args[0].device for a in args[1:]):
+        raise TensorError("Tensor arguments are not all on same device")
+
+
+def _check_partial_alias(*args) -> None:
+    for a, b in itertools.combinations([t.buffer for t in args], 2):
+        if a.partially_alias(b):
+            raise TensorError("Partially overlapping arguments detected.")
+
+
+def _ensure_broadcast_rules(*args) -> None:
+    """``ensure-broadcast-rules`` (``tensor.clj:592-604``): every operand
+    dimension must divide the max dimension."""
+    info = dims.dimension_seq_to_max_shape(*[a.dimensions for a in args])
+    max_shape = info["max-shape"]
+    for d in info["dimensions"]:
+        for mx, s in zip(max_shape, dims.shape(d)):
+            if mx % s != 0:
+                raise TensorError("Shapes are not broadcast-compatible (dimension counts must be commensurate) "
+                                  f"{[dims.shape(x) for x in info['dimensions']]} vs {max_shape}")
+
+
+# ---------------------------------------------------------------- assign!
+
+def _memcpy_semantics(dest: Tensor, src: Tensor) -> bool:
+    return (dest.ecount() == src.ecount() and dense(dest) and dense(src)
+            and dims.access_increasing(dest.dimensions) and dims.access_increasing(src.dimensions)
+            and dest.get_datatype() == src.get_datatype())
+
+
+def assign(dest: Tensor, src) -> Tensor:
+    """``assign!`` / ``typed-assign!`` (``tensor.clj:535-589``)."""
+    stream = check_stream()
+    if _is_number(src):
+        if dense(dest):
+            stream.memset(dest.buffer, 0, src, dest.ecount())
+        else:
+            stream.assign_constant(dest.buffer, dest.dimensions, src, dest.ecount())
+        return dest
+    de, se = dest.ecount(), src.ecount()
+    if not de >= se:
+        raise TensorError("destination element count must be >= src element count")
+    if se != 0 and de % se != 0:
+        raise TensorError("Src element count must evenly divide dest ecount.")
+    _ensure_same_device(dest, src)
+    _check_partial_alias(dest, src)
+    if _memcpy_semantics(dest, src):
+        stream.copy_device_to_device(src.buffer, 0, dest.buffer, 0, se)
+    else:
+        stream.assign(dest.buffer, dest.dimensions, src.buffer, src.dimensions, max(se, de))
+    return dest
+
+
+# ---------------------------------------------------------------- unary-op!
+
+def _perform_unary_op(value: float, op: str) -> float:
+    """``perform-unary-op`` (``tensor.clj:612-624``)."""
+    if op == "ceil":
+        return math.ceil(value)
+    if op == "round":
+        return math.floor(value + 0.5)
+    if op == "floor":
+        return math.floor(value)
+    if op == "-":
+        return -value
+    if op == "tanh":
+        return math.tanh(value)
+    if op == "logistic":
+        return 1.0 / (1.0 + math.exp(-value))
+    if op == "exp":
+        return math.exp(value)
+    if op == "sqrt":
+        return math.sqrt(value)
+    if op == "noop":
+        return value
+    raise TensorError(f"Unknown unary operation {op}")
+
+
+def unary_op(dest: Tensor, alpha, x, op: str) -> Tensor:
+    """``unary-op!`` (``tensor.clj:627-651``): dest = op(alpha * x)."""
+    if op not in UNARY_OPERATIONS:
+        raise TensorError(f"Unknown unary operation {op}")
+    if _is_number(x):
+        dt = dest.get_datatype()
+        return assign(dest, _perform_unary_op(float(_dtype_cast(alpha, dt)) * float(_dtype_cast(x, dt)), op))
+    stream = check_stream()
+    if dest.buffer.alias(x.buffer):
+        stream.unary_accum(dest.buffer, dest.dimensions, alpha, op, dest.ecount())
+    else:
+        _ensure_datatypes(dest.get_datatype(), x)
+        _ensure_same_device(dest, x)
+        _ensure_broadcast_rules(dest, x)
+        _check_partial_alias(dest, x)
+        stream.unary_op(dest.buffer, dest.dimensions, x.buffer, x.dimensions, alpha, op, max(dest.ecount(), x.ecount()))
+    return dest
+
+
+# ---------------------------------------------------------------- binary-op!
+
+def _binary_op_constant(dest, alpha, x, beta, y, op, reverse_operands) -> Tensor:
+    """``binary-op-constant!`` (``tensor.clj:676-703``)."""
+    _ensure_broadcast_rules(dest, x)
+    _ensure_datatypes(dest.get_datatype(), x)
+    y = float(beta) * float(y)
+    stream = check_stream()
+    if op == "*":  # strength reduction
+        return unary_op(dest, float(alpha) * y, x, "noop")
+    if dest.buffer.alias(x.buffer):
+        stream.binary_accum_constant(dest.buffer, dest.dimensions, alpha, y, dest.ecount(), op, reverse_operands)
+    else:
+        _check_partial_alias(dest, x)
+        stream.binary_op_constant(dest.buffer, dest.dimensions, x.buffer, x.dimensions, alpha, y,
+                                  max(x.ecount(), dest.ecount()), op, reverse_operands)
+    return dest
+
+
+def _typed_binary_op(dest, alpha, x, beta, y, op) -> Tensor:
+    xn, yn = _is_number(x), _is_number(y)
+    if xn and yn:  # tensor.clj:662-673
+        a, b = float(alpha) * float(x), float(beta) * float(y)
+        table = {"+": lambda: a + b, "-": lambda: a - b, "*": lambda: a * b, "/": lambda: a / b,
+                 "max": lambda: max(a, b), "min": lambda: min(a, b)}
+        return assign(dest, table[op]())
+    if yn:
+        return _binary_op_constant(dest, alpha, x, beta, y, op, False)
+    if xn:
+        return _binary_op_constant(dest, beta, y, alpha, x, op, True)
+    # [:tensor :tensor] (tensor.clj:716-761)
+    stream = check_stream()
+    info = dims.dimension_seq_to_max_shape(dest.dimensions, x.dimensions, y.dimensions)
+    max_shape = info["max-shape"]
+    dest_dims, x_dims, y_dims = info["dimensions"]
+    x_alias = dest.buffer.alias(x.buffer)
+    arg_alias = x_alias or dest.buffer.alias(y.buffer)
+    # the comparison is against the raw shape vector, index tensors included
+    dest_is_max_shape = list(dest_dims["shape"]) == list(max_shape) and dims.direct(dest_dims)
+    if not dest_is_max_shape and not arg_alias:
+        raise TensorError("If destination is a broadcast target then it must be one of the operands")
+    if arg_alias:
+        if x_alias:
+            a, b, other, rev = alpha, beta, y, False
+        else:
+            a, b, other, rev = beta, alpha, x, True
+        _ensure_broadcast_rules(dest, other)
+        _ensure_datatypes(dest.get_datatype(), other)
+        stream.binary_accum(dest.buffer, dest.dimensions, a, other.buffer, other.dimensions, b,
+                            max(dest.ecount(), other.ecount()), op, rev, not dest_is_max_shape)
+    else:
+        _ensure_broadcast_rules(dest, x, y)
+        _ensure_datatypes(x.get_datatype(), y, dest)
+        stream.binary_op(dest.buffer, dest_dims, x.buffer, x_dims, alpha, y.buffer, y_dims, beta,
+                         max(dest.ecount(), x.ecount(), y.ecount()), op)
+    return dest
+
+
+def binary_op(dest: Tensor, alpha, x, beta, y, op: str) -> Tensor:
+    """``binary-op!`` (``tensor.clj:768-779``): dest = alpha*x op beta*y."""
+    if op not in BINARY_OPERATIONS:
+        raise TensorError(f"Unknown binary operation {op}")
+    if op == "-":
+        return _typed_binary_op(dest, alpha, x, -float(beta), y, "+")
+    return _typed_binary_op(dest, alpha, x, beta, y, op)
+
+
+# ---------------------------------------------------------------- ternary-op!
+
+def ternary_op(dest: Tensor, alpha, x, beta, y, gamma, z, op: str = "select") -> Tensor:
+    """``ternary-op!`` (``tensor.clj:808-854``).  select: ``(x >= 0) ? z : y``
+    (``cpu/tensor_math.clj:464-466``)."""
+    if op != "select":
+        raise TensorError(f"Unknown ternary operation {op}")
+    args = [(x, alpha, "x"), (y, beta, "y"), (z, gamma, "z")]
+    tensors = [(v, a, n) for v, a, n in args if is_tensor(v)]
+    consts = [(v, a, n) for v, a, n in args if not is_tensor(v)]
+    if not tensors:
+        value = float(gamma) * float(z) if float(alpha) * float(x) >= 0.0 else float(beta) * float(y)
+        return assign(dest, value)
+    max_ecount = max(t.ecount() for t, _, _ in tensors)
+    constants = [float(v) * float(a) for v, a, _ in consts]
+    arg_order = [n for _, _, n in tensors] + [n for _, _, n in consts]
+    tens_only = [t for t, _, _ in tensors]
+    _ensure_datatypes(dest.get_datatype(), *tens_only)
+    _ensure_same_device(dest, *tens_only)
+    for t in tens_only:
+        _ensure_broadcast_rules(dest, t)
+    stream = check_stream()
+    if len(tensors) == 3:
+        stream.ternary_op(dest.buffer, dest.dimensions, x.buffer, x.dimensions, alpha, y.buffer, y.dimensions, beta,
+                          z.buffer, z.dimensions, gamma, max_ecount, op)
+    elif len(tensors) == 2:
+        (a, am, _), (b, bm, _) = tensors
+        stream.ternary_op_constant(dest.buffer, dest.dimensions, a.buffer, a.dimensions, am, b.buffer, b.dimensions, bm,
+                                   constants[0], max_ecount, op, arg_order)
+    else:
+        (a, am, _), = tensors
+        stream.ternary_op_constant_constant(dest.buffer, dest.dimensions, a.buffer, a.dimensions, am, constants[0],
+                                            constants[1], max_ecount, op, arg_order)
+    return dest
+
+
+# ---------------------------------------------------------------- unary-reduce!
+
+def unary_reduce(output: Tensor, alpha, input: Tensor, op: str) -> Tensor:
+    """``unary-reduce!`` (``tensor.clj:861-884``): reduces the last axis of the
+    input view into an output whose last dimension is 1."""
+    if op not in UNARY_REDUCTION_OPERATIONS:
+        raise TensorError(f"Unknown reduction operation {op}")
+    out_shape, in_shape = output.shape(), input.shape()
+    if out_shape[:-1] != in_shape[:-1]:
+        raise TensorError(f"Output leading dimensions must match input leading dimensions {out_shape} {in_shape}")
+    if out_shape[-1] != 1:
+        raise TensorError(f"Last dimension of output must be 1 {out_shape}")
+    _ensure_same_device(output, input)
+    _ensure_datatypes(output.get_datatype(), input)
+    check_stream().unary_reduce(output.buffer, output.dimensions, alpha, input.buffer, input.dimensions, op)
+    return output
+
+
+# ---------------------------------------------------------------- composites
+
+def normalize(dest: Tensor, mag_vec: Tensor, radius_length, epsilon=1e-6) -> Tensor:
+    """``normalize!`` (``tensor.clj:1618-1626``)."""
+    unary_reduce(mag_vec, 1.0, dest, "magnitude")
+    binary_op(mag_vec, 1.0, mag_vec, 1.0, 1e-6, "+")
+    return binary_op(dest, 1.0, dest, 1.0 / float(radius_length), mag_vec, "/")
+
+
+def constrain_inside_hypersphere(dest: Tensor, mag_vec: Tensor, radius_length) -> Tensor:
+    """``constrain-inside-hypersphere!`` (``tensor.clj:1629-1644``)."""
+    unary_reduce(mag_vec, 1.0, dest, "magnitude")
+    binary_op(mag_vec, 1.0, mag_vec, 1.0, radius_length, "-")
+    ternary_op(mag_vec, 1.0, mag_vec, 0.0, 0.0, 1.0, mag_vec, "select")
+    binary_op(mag_vec, 1.0, mag_vec, 1.0, radius_length, "+")
+    return binary_op(dest, 1.0, dest, 1.0 / float(radius_length), mag_vec, "/")

@@ -1,0 +1,464 @@
+"""The reference's backend-neutral tests of the tensor-math path, restated.
+
+Every function takes ``(driver, datatype)`` like its original in
+``/root/reference/src/cortex/verify/tensor.clj`` (cited per function) and runs
+through the backend-neutral tensor API, so one body tests every backend: the
+CPU oracle (which pins the oracle to the reference's stored vectors) and the
+HIP driver.  Expected values are the reference's own.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+from cortex_amd import dimensions as ct_dims
+from cortex_amd import tensor as ct
+from cortex_amd.dimensions import ALL
+
+ALL_DTYPES = ["double", "float", "long", "int", "short", "byte"]   # def-all-dtype-test
+FLOAT_DTYPES = ["double", "float"]                                  # def-double-float-test
+
+
+def context(driver, datatype):
+    device = driver.default_device()
+    device.make_current()
+    return ct.tensor_context(device.create_stream(), datatype)
+
+
+def dtype_cast(value, datatype):
+    """``drv/dtype-cast`` as the tests use it on expected values."""
+    if datatype == "double":
+        return float(value)
+    if datatype == "float":
+        return float(np.float32(value))
+    return int(value)  # truncation toward zero
+
+
+def equals(expected, actual, eps=0.0):
+    e = np.asarray(expected, dtype=np.float64).reshape(-1)
+    a = np.asarray(actual, dtype=np.float64).reshape(-1)
+    assert e.shape == a.shape, (e.shape, a.shape)
+    assert np.all(np.abs(e - a) <= eps), (e, a)
+
+
+def partition(n, seq):
+    seq = list(seq)
+    return [seq[i:i + n] for i in range(0, len(seq) - n + 1, n)]
+
+
+# verify/tensor.clj:20-42
+def assign_constant(driver, datatype):
+    with context(driver, datatype):
+        tensor = ct.to_tensor(partition(3, range(9)))
+        assert ct.ecount(tensor) == 9
+        equals(range(9), ct.to_double_array(tensor))
+        ct.assign(tensor, 1)
+        equals([1] * 9, ct.to_double_array(tensor))
+        rows, columns = ct.rows(tensor), ct.columns(tensor)
+        for row in rows:
+            ct.assign(row, 2)
+        equals([2] * 9, ct.to_double_array(tensor))
+        c1, c2, c3 = columns
+        ct.assign(c1, 1)
+        ct.assign(c2, 2)
+        ct.assign(c3, 3)
+        equals([1, 2, 3] * 3, ct.to_double_array(tensor))
+
+
+# verify/tensor.clj:45-57
+def assign_marshal(driver, datatype):
+    with context(driver, datatype):
+        tensor = ct.to_tensor(partition(3, range(9)))
+        intermediate = ct.new_tensor([3, 3], datatype="int")
+        final = ct.new_tensor([3, 3], datatype="double")
+        ct.assign(intermediate, tensor)
+        ct.assign(final, intermediate)
+        equals(range(9), ct.to_double_array(final))
+
+
+# verify/tensor.clj:60-80
+def unary_op(driver, datatype):
+    with context(driver, datatype):
+        tens_a = ct.to_tensor(partition(3, range(9)))
+        tens_b = ct.to_tensor(partition(3, [1] * 9))
+        ct.unary_op(tens_b, 2.5, tens_a, "ceil")
+        equals([math.ceil(x * dtype_cast(2.5, datatype)) for x in range(9)], ct.to_double_array(tens_b))
+        ct.unary_op(tens_b, 1.0, tens_b, "-")
+        equals([-math.ceil(x * dtype_cast(2.5, datatype)) for x in range(9)], ct.to_double_array(tens_b))
+        src_data = [0, 1, 2, 3, 4]
+        tens_src = ct.to_tensor(src_data)
+        tens_b = ct.to_tensor(src_data)
+        ct.unary_op(tens_b, 1.0, tens_src, "exp")
+        # the float case tolerates the last float ulp: the reference compares
+        # against the JDK's Math.exp, ours against the platform's
+        eps = 4e-6 if datatype == "float" else 0.0
+        equals([dtype_cast(math.exp(x), datatype) for x in src_data], ct.to_double_array(tens_b), eps)
+        ct.unary_op(tens_b, 1.0, tens_src, "sqrt")
+        equals([dtype_cast(math.sqrt(x), datatype) for x in src_data], ct.to_double_array(tens_b))
+
+
+# verify/tensor.clj:83-94
+def channel_op(driver, datatype):
+    with context(driver, datatype):
+        tens_a = ct.to_tensor(np.arange(18).reshape(2, 3, 3))
+        tens_chan = ct.in_place_reshape(ct.to_tensor(range(3)), [3, 1])
+        tens_result = ct.new_tensor([2, 3, 3])
+        ct.binary_op(tens_result, 1.0, tens_a, 1.0, tens_chan, "*")
+        equals([0.0, 0.0, 0.0, 3.0, 4.0, 5.0, 12.0, 14.0, 16.0, 0.0, 0.0, 0.0, 12.0, 13.0, 14.0, 30.0, 32.0, 34.0],
+               ct.to_double_array(tens_result))
+
+
+# verify/tensor.clj:97-126
+def binary_constant_op(driver, datatype):
+    with context(driver, datatype):
+        tens_a = ct.to_tensor(partition(3, range(9)))
+        tens_b = ct.to_tensor(partition(3, [1] * 9))
+        if datatype != "byte":
+            ct.binary_op(tens_b, 2.0, tens_a, 3.0, 4.0, "*")
+            equals([24 * x for x in range(9)], ct.to_double_array(tens_b))
+        ct.binary_op(tens_b, 2.0, tens_a, 3.0, 4.0, "+")
+        equals([12 + 2 * x for x in range(9)], ct.to_double_array(tens_b))
+        ct.binary_op(tens_b, 3.0, 4.0, 2.0, tens_a, "-")  # reversed operands
+        equals([12 - 2 * x for x in range(9)], ct.to_double_array(tens_b))
+        ct.assign(tens_b, 1.0)
+        equals([1] * 9, ct.to_double_array(tens_b))
+        ct.binary_op(tens_b, 1.0, tens_b, 1.0, 1.0, "+")  # accumulation
+        equals([2] * 9, ct.to_double_array(tens_b))
+
+
+# verify/tensor.clj:129-249
+def binary_op(driver, datatype):
+    with context(driver, datatype):
+        tens_a = ct.to_tensor(partition(3, range(9)))
+        tens_b = ct.to_tensor(partition(3, [2] * 9))
+        tens_c = ct.to_tensor(partition(3, [10] * 9))
+        ct.binary_op(tens_c, 2.0, tens_a, 2.0, tens_b, "*")
+        equals([2 * 2 * 2 * x for x in range(9)], ct.to_double_array(tens_c))
+        ct.binary_op(tens_b, 1.0, tens_c, 2.0, tens_a, "-")
+        equals([0.0, 6.0, 12.0, 18.0, 24.0, 30.0, 36.0, 42.0, 48.0], ct.to_double_array(tens_b))
+        # destination is one of the operands
+        ct.binary_op(tens_c, 1.0, tens_c, 2.0, tens_a, "-")
+        equals([0.0, 6.0, 12.0, 18.0, 24.0, 30.0, 36.0, 42.0, 48.0], ct.to_double_array(tens_c))
+
+        tens_c_small = ct.subvector(tens_c, 0, length=3)
+        sub_fn = lambda nth: [row[nth] for row in partition(3, range(9))]
+        c_data = list(ct.to_double_array(tens_c))
+        ct.binary_op(tens_c_small, 1.0, tens_c_small, 2.0, tens_a, "-")
+        equals([c_data[i] - sum(2.0 * v for v in sub_fn(i)) for i in range(3)], ct.to_double_array(tens_c_small))
+        c_data = list(ct.to_double_array(tens_c_small))
+        ct.binary_op(tens_c_small, 2.0, tens_a, 1.0, tens_c_small, "+")
+        equals([c_data[i] + sum(2.0 * v for v in sub_fn(i)) for i in range(3)], ct.to_double_array(tens_c_small))
+
+        if datatype in ("float", "double"):
+            n_batches, n_channels, img_dim = 3, 5, 4
+            rng = np.random.default_rng(11)
+            big = rng.random((n_batches, n_channels, img_dim, img_dim))
+            sums = big.sum(axis=(0, 2, 3))
+            big_m = ct.to_tensor(big)
+            test_vec = ct.in_place_reshape(ct.new_tensor([n_channels]), [n_channels, 1, 1])
+            ct.binary_op(test_vec, 1.0, test_vec, 1.0, big_m, "+")  # broadcasting summation
+            equals(sums, ct.to_double_array(test_vec), 1e-4)
+
+        tens_a4 = ct.to_tensor([partition(3, range(9))] * 4)
+        result = ct.new_tensor(ct.shape(tens_a4))
+        ct.binary_op(result, 1.0, tens_a4, 1.0, 5, "eq")
+        equals([1 if int(v) == 5 else 0 for v in ct.to_double_array(tens_a4)], ct.to_double_array(result))
+
+        tens_z = ct.new_tensor([4, 3, 3])
+        bias = ct.in_place_reshape(ct.to_tensor([1, 2, 3, 4]), [4, 1, 1])
+        ct.binary_op(tens_z, 1.0, tens_z, 1.0, bias, "+")
+        equals(np.repeat([1, 2, 3, 4], 9), ct.to_double_array(tens_z))
+        # bias-gradient calculation
+        tens_g = ct.to_tensor([np.full((3, 3), v) for v in [1, 2, 3, 4]])
+        bias = ct.in_place_reshape(ct.new_tensor([4]), [4, 1, 1])
+        ct.binary_op(bias, 1.0, tens_g, 1.0, bias, "+")
+        equals([9, 18, 27, 36], ct.to_double_array(bias))
+
+        tens_1 = ct.to_tensor([1, 1, 0, 0])
+        tens_2 = ct.to_tensor([-1, 1, 2, -2])
+        result = ct.new_tensor(ct.shape(tens_2))
+        for op, want in ((">", [1, 0, 0, 1]), (">=", [1, 1, 0, 1]), ("<", [0, 0, 1, 0]), ("<=", [0, 1, 1, 0])):
+            ct.binary_op(result, 1.0, tens_1, 1.0, tens_2, op)
+            equals(want, ct.to_double_array(result))
+
+        tens_1 = ct.to_tensor([1, 1, 0, 0])
+        tens_2 = ct.to_tensor([1, 1, 1, 1])
+        result = ct.new_tensor(ct.shape(tens_2))
+        ct.binary_op(result, 1.0, tens_1, 1.0, tens_2, "bit-xor")
+        equals([0, 0, 1, 1], ct.to_double_array(result))
+
+
+# verify/tensor.clj:532-554 (the hot-path part: logistic, tanh, max 0)
+def activation_forward(driver, datatype):
+    with context(driver, datatype):
+        inp = ct.to_tensor(range(-4, 8))
+        output = ct.new_tensor([12])
+        ct.unary_op(output, 1.0, inp, "logistic")
+        equals([0.01798620996209156, 0.04742587317756678, 0.11920292202211755, 0.2689414213699951, 0.5,
+                0.7310585786300049, 0.8807970779778823, 0.9525741268224334, 0.9820137900379085, 0.9933071490757153,
+                0.9975273768433653, 0.9990889488055994], ct.to_double_array(output), 1e-4)
+        ct.unary_op(output, 1.0, inp, "tanh")
+        equals([-0.999329299739067, -0.9950547536867305, -0.9640275800758169, -0.7615941559557649, 0.0,
+                0.7615941559557649, 0.9640275800758169, 0.9950547536867305, 0.999329299739067, 0.9999092042625951,
+                0.9999877116507956, 0.9999983369439447], ct.to_double_array(output), 1e-4)
+        ct.binary_op(output, 1.0, inp, 0, 0, "max")
+        equals([0.0, 0.0, 0.0, 0.0, 0.0, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0], ct.to_double_array(output))
+
+
+# verify/tensor.clj:623-645
+def ternary_op_select(driver, datatype):
+    with context(driver, datatype):
+        dest = ct.to_tensor([0] * 10)
+        x_arg = ct.to_tensor(range(-5, 5))
+        y_arg = ct.to_tensor(range(10))
+        z_arg = ct.to_tensor([2] * 10)
+        ct.ternary_op(dest, 1, x_arg, 2.0, y_arg, 3.0, z_arg, "select")
+        equals([0, 2, 4, 6, 8, 6, 6, 6, 6, 6], ct.to_double_array(dest))
+        ct.ternary_op(dest, 1, x_arg, 1.0, -1, 3.0, z_arg, "select")
+        equals([-1, -1, -1, -1, -1, 6, 6, 6, 6, 6], ct.to_double_array(dest))
+        ct.ternary_op(dest, 1, x_arg, 3.0, z_arg, 1.0, -1, "select")
+        equals([6, 6, 6, 6, 6, -1, -1, -1, -1, -1], ct.to_double_array(dest))
+        ct.ternary_op(dest, 1, x_arg, 3.0, 2.0, 1.0, -1, "select")
+        equals([6, 6, 6, 6, 6, -1, -1, -1, -1, -1], ct.to_double_array(dest))
+        ct.ternary_op(dest, 1, x_arg, 1.0, -1, 3.0, 2.0, "select")
+        equals([-1, -1, -1, -1, -1, 6, 6, 6, 6, 6], ct.to_double_array(dest))
+
+
+# verify/tensor.clj:648-665
+def unary_reduce(driver, datatype):
+    with context(driver, datatype):
+        dest = ct.new_tensor([10, 1])
+        src_data = [0, 3, 5, 2, 1, 9, 5, 7, 7, 2]
+        src = ct.to_tensor([src_data] * 10)
+        ct.unary_reduce(dest, 2.0, src, "max")
+        equals([18] * 10, ct.to_double_array(dest))
+        ct.unary_reduce(dest, 1.0, src, "sum")
+        equals([sum(src_data)] * 10, ct.to_double_array(dest))
+        ct.unary_reduce(dest, 1.0, src, "mean")
+        equals([dtype_cast(sum(src_data) / len(src_data), datatype)] * 10, ct.to_double_array(dest))
+
+
+# verify/tensor.clj:668-684
+def transpose(driver, datatype):
+    with context(driver, datatype):
+        img_dim = 4
+        img_tensor = ct.to_tensor(np.tile([1, 2, 3], (img_dim, img_dim, 1)))
+        planar = ct.transpose(img_tensor, [2, 0, 1])
+        rgb = ct.transpose(planar, [1, 2, 0])
+        equals([1] * 16 + [2] * 16 + [3] * 16, ct.to_double_array(planar))
+        equals([1, 2, 3] * 16, ct.to_double_array(rgb))
+
+
+# verify/tensor.clj:687-717
+def mask(driver, datatype):
+    with context(driver, datatype):
+        rgba = 1 + (2 << 8) + (3 << 16) + (255 << 24)
+        rgba = rgba - (1 << 32) if rgba >= (1 << 31) else rgba  # the int the JVM holds
+        img_dim = 4
+        img_tensor = ct.to_tensor(np.full((img_dim, img_dim), rgba, dtype=np.int64))
+        mask_tensor = ct.in_place_reshape(ct.to_tensor([0xFF, 0xFF << 8, 0xFF << 16]), [3, 1, 1])
+        div_tensor = ct.in_place_reshape(ct.to_tensor([1, 1 << 8, 1 << 16]), [3, 1, 1])
+        result = ct.new_tensor([3, img_dim, img_dim])
+        ct.binary_op(result, 1.0, img_tensor, 1.0, mask_tensor, "bit-and")
+        ct.binary_op(result, 1.0, result, 1.0, div_tensor, "/")
+        equals([1] * 16 + [2] * 16 + [3] * 16, ct.to_double_array(result))
+
+
+# verify/tensor.clj:720-782
+def select(driver, datatype):
+    with context(driver, datatype):
+        mat = ct.to_tensor([partition(3, range(9))] * 2)
+        s = ct.select(mat, ALL, ALL, [1, 2])
+        equals([1, 2, 4, 5, 7, 8] * 2, ct.to_double_array(s))
+        assert ct.shape(s) == [2, 3, 2]
+        s = ct.select(mat, ALL, ALL, [2])
+        equals([2, 5, 8] * 2, ct.to_double_array(s))
+        assert ct.shape(s) == [2, 3, 1]
+        s = ct.select(mat, ALL, ALL, 2)
+        equals([2, 5, 8] * 2, ct.to_double_array(s))
+        assert ct.shape(s) == [2, 3] and not ct.dense(s)
+        s = ct.select(mat, ALL, [1, 2], ALL)
+        equals([3, 4, 5, 6, 7, 8] * 2, ct.to_double_array(s))
+        assert ct.shape(s) == [2, 2, 3] and not ct.dense(s)
+        s = ct.select(mat, ALL, [2], ALL)
+        equals([6, 7, 8] * 2, ct.to_double_array(s))
+        assert ct.shape(s) == [2, 1, 3] and not ct.dense(s)
+        s = ct.select(mat, ALL, 0, ALL)
+        equals([0, 1, 2] * 2, ct.to_double_array(s))
+        assert ct.shape(s) == [2, 3] and not ct.dense(s)
+        s = ct.select(mat, [1], [1], ALL)
+        equals([3, 4, 5], ct.to_double_array(s))
+        assert ct.shape(s) == [1, 1, 3] and ct.dense(s)
+        s = ct.select(mat, 1, 1, ALL)
+        equals([3, 4, 5], ct.to_double_array(s))
+        assert ct.shape(s) == [3] and ct.dense(s) and ct.as_vector(s) is not None
+        s = ct.select(mat, 1, ALL, 2)
+        equals([2, 5, 8], ct.to_double_array(s))
+        assert ct.shape(s) == [3] and not ct.dense(s)
+
+
+# verify/tensor.clj:785-805
+def select_transpose_interaction(driver, datatype):
+    with context(driver, datatype):
+        img_dim = 4
+        mat = ct.to_tensor(np.tile([1, 2, 3], (img_dim, img_dim, 1)))
+        planar = ct.transpose(mat, [2, 0, 1])
+        n_pixels = img_dim * img_dim
+        r, g, b = (ct.select(planar, i, ALL, ALL) for i in range(3))
+        equals([1] * n_pixels, ct.to_double_array(r))
+        equals([2] * n_pixels, ct.to_double_array(g))
+        equals([3] * n_pixels, ct.to_double_array(b))
+        bgr = ct.new_tensor([img_dim, img_dim, 3])
+        bgr_planes = ct.transpose(bgr, [2, 0, 1])
+        ct.assign(ct.select(bgr_planes, 0, ALL, ALL), b)
+        ct.assign(ct.select(bgr_planes, 1, ALL, ALL), g)
+        ct.assign(ct.select(bgr_planes, 2, ALL, ALL), r)
+        equals([3, 2, 1] * n_pixels, ct.to_double_array(bgr))
+
+
+# verify/tensor.clj:1147-1199
+def indexed_tensor(driver, datatype):
+    with context(driver, datatype):
+        mat = ct.to_tensor([partition(3, range(9))] * 2)
+        index_tens = ct.to_tensor([1, 2, 1, 2, 1, 2], datatype="int")
+        sel = ct.select(mat, ALL, ALL, index_tens)
+        assert not ct_dims.access_increasing(sel.dimensions)
+        assert ct.shape(sel) == [2, 3, 6]
+        equals([1, 2, 1, 2, 1, 2, 4, 5, 4, 5, 4, 5, 7, 8, 7, 8, 7, 8] * 2, ct.to_double_array(sel))
+        # center loss use case: gather, then scatter-add through duplicates
+        centers = ct.select(mat, 0, ct.to_tensor([0, 1, 0, 2, 1], datatype="int"), ALL)
+        batch_data = ct.new_tensor([5, 3])
+        ct.assign(batch_data, centers)
+        equals([0, 1, 2, 3, 4, 5, 0, 1, 2, 6, 7, 8, 3, 4, 5], ct.to_double_array(batch_data))
+        ct.binary_op(centers, 1.0, batch_data, 1.0, centers, "+")
+        equals([0, 3, 6, 9, 12, 15, 0, 3, 6, 12, 14, 16, 9, 12, 15], ct.to_double_array(centers))
+        # broadcasting, several index tensors in one tensor
+        mat2 = ct.to_tensor(partition(3, range(9)))
+        sel2 = ct.select(mat2, ct.to_tensor([0, 1, 1, 2], datatype="int"), ct.to_tensor([2, 1, 0], datatype="int"))
+        dest = ct.new_tensor([8, 6])
+        ct.assign(dest, sel2)
+        want = [[2, 1, 0], [2, 1, 0], [5, 4, 3], [5, 4, 3], [5, 4, 3], [5, 4, 3], [8, 7, 6], [8, 7, 6]] * 2
+        equals(np.array(want, dtype=np.float64), ct.to_double_array(dest))
+
+
+# verify/tensor.clj:1202-1228
+def magnitude_and_mag_squared(driver, datatype):
+    with context(driver, datatype):
+        num_elems = num_rows = 10
+        src = np.arange(num_rows * num_elems, dtype=np.float64).reshape(num_rows, num_elems)
+        src_tensor = ct.to_tensor(src)
+        dst = ct.new_tensor([num_rows, 1])
+        ct.unary_reduce(dst, 1.0, src_tensor, "magnitude-squared")
+        equals((src * src).sum(axis=1), ct.to_double_array(dst), 1e-4)
+        ct.unary_reduce(dst, 1.0, src_tensor, "magnitude")
+        equals(np.sqrt((src * src).sum(axis=1)), ct.to_double_array(dst), 1e-4)
+
+
+# verify/tensor.clj:1231-1248
+def constrain_inside_hypersphere(driver, datatype):
+    with context(driver, datatype):
+        num_elems = num_rows = 10
+        radius = 100
+        src = np.arange(num_rows * num_elems, dtype=np.float64).reshape(num_rows, num_elems)
+        src_tensor = ct.to_tensor(src)
+        mul_tensor = ct.new_tensor([num_rows, 1])
+        ct.constrain_inside_hypersphere(src_tensor, mul_tensor, radius)
+        got = ct.to_double_array(src_tensor).reshape(num_rows, num_elems)
+        mags = np.sqrt((got * got).sum(axis=1))
+        assert np.all(mags <= radius + 1e-4), mags
+        # rows shorter than the radius are untouched
+        short = np.sqrt((src * src).sum(axis=1)) <= radius
+        equals(src[short], got[short], 1e-4)
+
+
+# verify/tensor/operations.clj:37-230 (the sugar ops, all built on binary-op! / unary-op!)
+def operations_sugar(driver, datatype):
+    with context(driver, datatype):
+        x = ct.to_tensor([-1.5, 0.25, 2.0, 3.75])
+        out = ct.new_tensor([4])
+        ct.binary_op(out, 1.0, x, 1.0, 1.0, "max")
+        equals([1.0, 1.0, 2.0, 3.75], ct.to_double_array(out))
+        ct.binary_op(out, 1.0, x, 1.0, 1.0, "min")
+        equals([-1.5, 0.25, 1.0, 1.0], ct.to_double_array(out))
+        ct.unary_op(out, 1.0, x, "ceil")
+        equals([-1.0, 1.0, 2.0, 4.0], ct.to_double_array(out))
+        ct.unary_op(out, 1.0, x, "floor")
+        equals([-2.0, 0.0, 2.0, 3.0], ct.to_double_array(out))
+        ct.unary_op(out, 1.0, x, "round")
+        equals([-1.0, 0.0, 2.0, 4.0], ct.to_double_array(out))
+        # where: out = then*test + else*(test xor 1)
+        test = ct.to_tensor([1, 0, 1, 0])
+        then_, else_ = ct.to_tensor([1, 2, 3, 4]), ct.to_tensor([10, 20, 30, 40])
+        compl = ct.new_tensor([4])
+        ct.binary_op(compl, 1.0, test, 1.0, 1, "bit-xor")
+        ct.binary_op(then_, 1.0, then_, 1.0, test, "*")
+        ct.binary_op(else_, 1.0, else_, 1.0, compl, "*")
+        ct.binary_op(out, 1.0, then_, 1.0, else_, "+")
+        equals([1, 20, 3, 40], ct.to_double_array(out))
+
+
+# compute/verify/driver.clj:11-30
+def simple_stream(driver, datatype):
+    from cortex_amd.tensor import NUMPY_OF
+
+    device = driver.default_device()
+    device.make_current()
+    stream = device.create_stream()
+    buf_a = driver.allocate_host_buffer(10, datatype)
+    out_a = driver.allocate_host_buffer(10, datatype)
+    buf_b = device.allocate_device_buffer(10, datatype)
+    buf_a.array[...] = np.arange(10).astype(NUMPY_OF[datatype])
+    buf_a.array[0] = 100
+    stream.copy_host_to_device(buf_a, 0, buf_b, 0, 10)
+    stream.memset(buf_b, 5, 20.0, 5)
+    stream.copy_device_to_host(buf_b, 0, out_a, 0, 10)
+    stream.sync()
+    assert [float(v) for v in out_a.array] == [100.0, 1.0, 2.0, 3.0, 4.0, 20.0, 20.0, 20.0, 20.0, 20.0]
+
+
+# compute/verify/optimize.clj:11-61
+ADAM_ANSWERS = [
+    [0.999000000005, 1.9990000000025, 2.9990000000016668, 3.99900000000125],
+    [0.9980000262138343, 1.9980000130723587, 2.998000008707231, 3.998000006527546],
+    [0.9970000960651408, 1.9970000478972731, 2.9970000319014805, 3.9970000239148513],
+    [0.9960002269257634, 1.9960001131228113, 2.9960000753397424, 3.9960000564765217],
+    [0.995000436052392, 1.9950002173334274, 2.995000144735273, 3.995000108493863],
+    [0.9940007405541528, 1.9940003690339771, 2.994000245746984, 3.9940001842069432],
+    [0.9930011573564278, 1.9930005766318695, 2.9930003839675967, 3.993000287805732],
+    [0.9920017031661642, 1.9920008484199827, 2.992000564912314, 3.992000423421624],
+    [0.9910023944389119, 1.991001192560463, 2.9910007940080785, 3.9910005951194076],
+    [0.9900032473478027, 1.9900016170695067, 2.9900010765834972, 3.990000806889731],
+    [0.9890042777546556, 1.9890021298032192, 2.9890014178594777, 3.9890010626421075],
+    [0.9880055011833645, 1.9880027384446224, 2.9880018229406398, 3.988001366198499],
+    [0.9870069327956914, 1.987003450491873, 2.98700229680753, 3.9870017212875037],
+    [0.9860085873695607, 1.986004273247733, 2.9860028443096756, 3.9860021315391725],
+    [0.9850104792799151, 1.9850052138103236, 2.9850034701594894, 3.9850026004804673],
+    [0.9840126224821667, 1.984006279065173, 2.984004178927043, 3.984003131531364],
+    [0.9830150304982433, 1.9830074756785594, 2.9830049750356973, 3.9830037280016044],
+    [0.9820177164052082, 1.9820088100921336, 2.982005862758586, 3.9820043930880837],
+    [0.9810206928263993, 1.9810102885187928, 2.981006846215933, 3.9810051298728633],
+]
+
+
+def adam_trajectory(driver, datatype):
+    from cortex_amd import optimize as opt
+
+    with context(driver, datatype) as stream:
+        backend = opt.Backend(stream=stream, datatype=datatype, type=getattr(driver, "type", "hip"))
+        p1 = ct.to_tensor([1, 2, 3, 4])
+        p2 = ct.to_tensor([1, 2, 3, 4])
+        m = ct.new_tensor([8])
+        v = ct.new_tensor([8])
+        optimizer = opt.create_optimizer(backend, opt.adam())
+        state = {"m": m, "v": v}
+        for answer in ADAM_ANSWERS:
+            g1 = ct.to_tensor(2.0 * ct.to_double_array(p1))
+            g2 = ct.to_tensor(2.0 * ct.to_double_array(p2))
+            optimizer = optimizer.batch_update(state)
+            optimizer.compute_parameters(state, 1.0, 0, g1, p1)
+            optimizer.compute_parameters(state, 0.0, 4, g2, p2)
+            guess1, guess2 = ct.to_double_array(p1), ct.to_double_array(p2)
+            # about-there?: sum of absolute differences below 1e-6 (src/cortex/verify/utils.clj:20-27)
+            assert np.abs(guess1 - np.array(answer)).sum() < 1e-6, (guess1, answer)
+            assert np.abs(guess2 - np.array([1.0, 2.0, 3.0, 4.0])).sum() < 1e-6, guess2

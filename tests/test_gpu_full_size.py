@@ -1,0 +1,221 @@
+"""The BASELINE configurations at their full sizes on the GPU: compared with the
+CPU oracle where it finishes in seconds, and through size-independent
+properties (closed forms, a checksum of checksums, selection consistency).
+Inputs follow BASELINE.md: numpy default_rng(seed), generated in float64 and
+cast.  Needs a GPU.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from cortex_amd import capi
+from oracle import binding as ob
+
+pytestmark = pytest.mark.gpu
+
+
+class Dev:
+    """A device array holding a copy of a host array."""
+
+    def __init__(self, host: np.ndarray):
+        self.host = np.ascontiguousarray(host).reshape(-1)
+        p = C.c_void_p()
+        capi.call("ct_malloc", C.byref(p), max(1, self.host.nbytes))
+        self.ptr = p.value
+        capi.call("ct_memcpy_async", self.ptr, self.host.ctypes.data, self.host.nbytes, capi.COPY_H2D, None)
+        capi.call("ct_stream_sync", None)
+
+    def download(self) -> np.ndarray:
+        out = np.empty_like(self.host)
+        capi.call("ct_stream_sync", None)
+        capi.call("ct_memcpy_async", out.ctypes.data, self.ptr, out.nbytes, capi.COPY_D2H, None)
+        capi.call("ct_stream_sync", None)
+        return out
+
+    def free(self):
+        capi.call("ct_free", self.ptr)
+
+
+@pytest.fixture(autouse=True)
+def device():
+    capi.call("ct_set_device", 0)
+    capi.call("ct_set_debug_sync", 1)
+    yield
+
+
+def dims(shape, strides=None):
+    if strides is None:
+        strides, m = [], 1
+        for s in reversed(shape):
+            strides.insert(0, m)
+            m *= s
+    return capi.make_dims(shape, strides)
+
+
+def bits_equal(a, b) -> bool:
+    return bool(np.array_equal(a.view(f"u{a.itemsize}"), b.view(f"u{b.itemsize}")))
+
+
+def test_config0_bias_add():
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    b = rng.uniform(-1, 1, 1024).astype(np.float32)
+    dx, db, dd = Dev(x), Dev(b), Dev(np.zeros_like(x))
+    capi.call("ct_binary_op", None, dd.ptr, C.byref(dims([1024, 1024])), dx.ptr, C.byref(dims([1024, 1024])), 1.0, db.ptr,
+              C.byref(dims([1024])), 1.0, 1024 * 1024, capi.BINARY_OPS["+"], capi.F32)
+    got = dd.download().reshape(1024, 1024)
+    assert capi.last_kernel() == "vec"
+    assert bits_equal(got, x + b[None, :])  # one float add per element is the closed form
+    want = np.zeros(1024 * 1024, np.float32)
+    ob.call("binary_op", want.ctypes.data, C.byref(dims([1024, 1024])), x.ctypes.data, C.byref(dims([1024, 1024])), 1.0,
+            b.ctypes.data, C.byref(dims([1024])), 1.0, 1024 * 1024, capi.BINARY_OPS["+"], capi.F32)
+    assert bits_equal(got.reshape(-1), want)
+    for t in (dx, db, dd):
+        t.free()
+
+
+def test_config1_transposed_views_8192():
+    n = 8192
+    hosts = [np.random.default_rng(seed).standard_normal(n * n).astype(np.float32) for seed in (1, 2, 3)]
+    devs = [Dev(h) for h in hosts]
+    dest = Dev(np.zeros(n * n, np.float32))
+    cont, view = dims([n, n]), dims([n, n], [1, n])
+    want = np.zeros(n * n, np.float32)
+    for op in ("exp", "tanh"):
+        capi.call("ct_unary_op", None, dest.ptr, C.byref(cont), devs[0].ptr, C.byref(view), 1.0, capi.UNARY_OPS[op],
+                  capi.F32, n * n)
+        assert capi.last_kernel() == "tile"
+        got = dest.download()
+        ob.call("unary_op", want.ctypes.data, C.byref(cont), hosts[0].ctypes.data, C.byref(view), 1.0, capi.UNARY_OPS[op],
+                capi.F32, n * n)
+        rel = np.abs(got.astype(np.float64) - want) / np.abs(want)
+        assert np.nanmax(rel) <= 2e-6, (op, np.nanmax(rel))
+        # indexing is exact: element (i, j) of the result comes from element (j, i) of the input
+        fn = np.exp if op == "exp" else np.tanh
+        sample = fn(hosts[0].reshape(n, n)[::97, ::89].T.astype(np.float64))
+        assert np.max(np.abs(got.reshape(n, n)[::89, ::97] - sample) / np.abs(sample)) <= 2e-6
+    capi.call("ct_ternary_op", None, dest.ptr, C.byref(cont), devs[0].ptr, C.byref(view), 1.0, devs[1].ptr, C.byref(view),
+              1.0, devs[2].ptr, C.byref(view), 1.0, n * n, 0, capi.F32)
+    assert capi.last_kernel() == "tile"
+    got = dest.download()
+    ob.call("ternary_op", want.ctypes.data, C.byref(cont), hosts[0].ctypes.data, C.byref(view), 1.0,
+            hosts[1].ctypes.data, C.byref(view), 1.0, hosts[2].ctypes.data, C.byref(view), 1.0, n * n, 0, capi.F32)
+    assert bits_equal(got, want)
+    # closed form: (x >= 0) ? z : y on the transposed data
+    xt, yt, zt = (h.reshape(n, n).T for h in hosts)
+    assert bits_equal(got.reshape(n, n), np.where(xt >= 0, zt, yt))
+    for t in devs + [dest]:
+        t.free()
+
+
+@pytest.mark.parametrize("code,shape,seed", [(capi.F32, (16384, 4096), 4), (capi.F64, (4096, 4096), 5)])
+def test_config2_reductions(code, shape, seed):
+    r, c = shape
+    dt = np.float32 if code == capi.F32 else np.float64
+    x = np.random.default_rng(seed).standard_normal(r * c).astype(dt)
+    dx = Dev(x)
+    rows_out, cols_out = Dev(np.zeros(r, dt)), Dev(np.zeros(c, dt))
+    tol = 2e-6 if code == capi.F32 else 1e-12
+    x64 = x.reshape(r, c).astype(np.float64)
+    for op in ("sum", "max", "magnitude-squared"):
+        capi.call("ct_unary_reduce", None, rows_out.ptr, C.byref(dims([r, 1])), 1.0, dx.ptr, C.byref(dims([r, c])),
+                  capi.REDUCE_OPS[op], code)
+        k_rows = capi.last_kernel()
+        capi.call("ct_unary_reduce", None, cols_out.ptr, C.byref(dims([c, 1])), 1.0, dx.ptr, C.byref(dims([c, r], [1, c])),
+                  capi.REDUCE_OPS[op], code)
+        k_cols = capi.last_kernel()
+        assert k_rows.startswith("reduce_row") and k_cols.startswith("reduce_col"), (k_rows, k_cols)
+        got_r, got_c = rows_out.download().astype(np.float64), cols_out.download().astype(np.float64)
+        want_r, want_c = np.zeros(r, dt), np.zeros(c, dt)
+        ob.call("unary_reduce", want_r.ctypes.data, C.byref(dims([r, 1])), 1.0, x.ctypes.data, C.byref(dims([r, c])),
+                capi.REDUCE_OPS[op], code)
+        ob.call("unary_reduce", want_c.ctypes.data, C.byref(dims([c, 1])), 1.0, x.ctypes.data,
+                C.byref(dims([c, r], [1, c])), capi.REDUCE_OPS[op], code)
+        if op == "max":
+            assert np.array_equal(got_r, want_r) and np.array_equal(got_c, want_c)
+            assert got_r.max() == got_c.max() == x64.max()
+            continue
+        mag = np.abs(x64) if op == "sum" else x64 * x64
+        assert np.all(np.abs(got_r - want_r) <= tol * mag.sum(axis=1)), op
+        assert np.all(np.abs(got_c - want_c) <= tol * mag.sum(axis=0)), op
+        # checksum of checksums: both directions add up to the same total
+        total = mag.sum() if op != "sum" else np.abs(x64).sum()
+        assert abs(got_r.sum() - got_c.sum()) <= 4 * tol * total
+    for t in (dx, rows_out, cols_out):
+        t.free()
+
+
+def test_config3_adam_and_adadelta_2_28():
+    n = 1 << 28
+    rng = np.random.default_rng(6)
+    p = rng.uniform(-0.05, 0.05, n).astype(np.float32)
+    g = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    m = np.zeros(n, np.float32)
+    v = np.full(n, 1e-6, np.float32)
+    dp, dg, dm, dv = Dev(p), Dev(g), Dev(m), Dev(v)
+    pb1 = pb2 = 1.0
+    for _ in range(10):
+        pb1, pb2 = pb1 * 0.9, pb2 * 0.999
+    capi.call("ct_adam_step", None, capi.F32, 1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 1.0, dg.ptr, dp.ptr, dm.ptr, dv.ptr, n)
+    assert capi.last_kernel() == "adam_vec"
+    ob.call("adam_step", capi.F32, 1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 1.0, g.ctypes.data, p.ctypes.data, m.ctypes.data,
+            v.ctypes.data, n)  # the oracle updates p, m, v in place
+    for name, dev, want in (("params", dp, p), ("m", dm, m), ("v", dv, v)):
+        assert bits_equal(dev.download(), want), name
+    # Adadelta on the same parameters and gradients, accumulators 0
+    capi.call("ct_memset", None, dm.ptr, capi.F32, 0.0, n)
+    capi.call("ct_memset", None, dv.ptr, capi.F32, 0.0, n)
+    m[...] = 0
+    v[...] = 0
+    capi.call("ct_adadelta_step", None, capi.F32, 0.05, 1e-6, dm.ptr, dv.ptr, 1.0, dg.ptr, dp.ptr, n)
+    # the Java step is single-threaded; the oracle restates it that way, so check a bounded prefix and suffix
+    k = 1 << 22
+    got_p, got_m, got_v = dp.download(), dm.download(), dv.download()
+    for lo in (0, n // 2 - 12345, n - k):
+        sl = slice(lo, lo + k)
+        pp, mm, vv, gg = p[sl].copy(), m[sl].copy(), v[sl].copy(), g[sl].copy()
+        ob.call("adadelta_step", capi.F32, 0.05, 1e-6, mm.ctypes.data, vv.ctypes.data, 1.0, gg.ctypes.data,
+                pp.ctypes.data, k)
+        assert bits_equal(got_p[sl], pp) and bits_equal(got_m[sl], mm) and bits_equal(got_v[sl], vv), lo
+    for t in (dp, dg, dm, dv):
+        t.free()
+
+
+def test_config4_image_normalise_and_int_to_double():
+    shp = [256, 3, 224, 224]
+    n = int(np.prod(shp))
+    u8 = np.random.default_rng(7).integers(0, 256, n, dtype=np.uint8)
+    du8, df, df2 = Dev(u8), Dev(np.zeros(n, np.float32)), Dev(np.zeros(n, np.float32))
+    capi.call("ct_assign", None, df.ptr, C.byref(dims(shp)), capi.F32, du8.ptr, C.byref(dims(shp)), capi.U8, n)
+    assert capi.last_kernel() == "vec"
+    f = df.download()
+    assert bits_equal(f, u8.astype(np.float32))  # uint8 -> float32 is exact
+    mean = (np.array([0.485, 0.456, 0.406]) * 255).astype(np.float32)
+    std = (np.array([0.229, 0.224, 0.225]) * 255).astype(np.float32)
+    dmean, dstd = Dev(mean), Dev(std)
+    f4 = f.reshape(shp)
+    # :- arrives as :+ with y_alpha -1 (src/cortex/tensor.clj:774-777)
+    capi.call("ct_binary_op", None, df2.ptr, C.byref(dims(shp)), df.ptr, C.byref(dims(shp)), 1.0, dmean.ptr,
+              C.byref(dims([3, 1, 1])), -1.0, n, capi.BINARY_OPS["+"], capi.F32)
+    assert capi.last_kernel() == "vec"
+    sub = df2.download()
+    assert bits_equal(sub.reshape(shp), f4 - mean[None, :, None, None])
+    capi.call("ct_binary_op", None, df.ptr, C.byref(dims(shp)), df2.ptr, C.byref(dims(shp)), 1.0, dstd.ptr,
+              C.byref(dims([3, 1, 1])), 1.0, n, capi.BINARY_OPS["/"], capi.F32)
+    div = df.download()
+    assert bits_equal(div.reshape(shp), sub.reshape(shp) / std[None, :, None, None])
+    want = np.zeros(n, np.float32)
+    ob.call("binary_op", want.ctypes.data, C.byref(dims(shp)), sub.ctypes.data, C.byref(dims(shp)), 1.0, std.ctypes.data,
+            C.byref(dims([3, 1, 1])), 1.0, n, capi.BINARY_OPS["/"], capi.F32)
+    assert bits_equal(div, want)
+    for t in (du8, df, df2, dmean, dstd):
+        t.free()
+
+    n = 1 << 26
+    i32 = np.random.default_rng(8).integers(-2 ** 31, 2 ** 31, n, dtype=np.int64).astype(np.int32)
+    di, dd = Dev(i32), Dev(np.zeros(n, np.float64))
+    capi.call("ct_assign", None, dd.ptr, C.byref(dims([n])), capi.F64, di.ptr, C.byref(dims([n])), capi.I32, n)
+    assert bits_equal(dd.download(), i32.astype(np.float64))
+    di.free()
+    dd.free()

@@ -1,0 +1,491 @@
+"""Parity of the HIP library with the CPU oracle, call by call through the C
+ABI, on identical seeded inputs.  Bar: bit-exact for integer work, for
+assign / convert / select / indexing and for the non-transcendental float ops;
+<= 2e-6 relative for exp / tanh / logistic and for reductions.  Needs a GPU.
+"""
+import numpy as np
+import pytest
+
+import harness as H
+from cortex_amd import capi
+from harness import View
+
+pytestmark = pytest.mark.gpu
+
+NP = H.NP_DTYPES
+FLOATS = (capi.F32, capi.F64)
+TRANSCENDENTAL = ("exp", "tanh", "logistic")
+REL_TOL = 2e-6          # float32 transcendentals and reductions
+REL_TOL_F64 = 1e-12
+
+
+@pytest.fixture()
+def P(pair_factory):
+    with pair_factory() as pair:
+        yield pair
+
+
+def values(rng, code, n, lo=-100, hi=100, nonzero=False):
+    if code in FLOATS:
+        v = rng.standard_normal(n) * 3.0
+        if nonzero:
+            v = np.where(np.abs(v) < 0.1, 0.5, v)
+        return v.astype(NP[code])
+    info = np.iinfo(NP[code])
+    lo, hi = max(lo, info.min), min(hi, info.max)
+    v = rng.integers(lo, hi + 1, n)
+    if nonzero:
+        v = np.where(v == 0, 3, v)
+    return v.astype(NP[code])
+
+
+def compare(buf, what, tol=None):
+    got, want = buf.download(), buf.host
+    if tol is None:
+        H.assert_bit_exact(got, want, what)
+        return
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    ok = (np.abs(g - w) <= tol * np.abs(w)) | (np.isnan(g) & np.isnan(w)) | (g == w)
+    assert np.all(ok), f"{what}: max rel err {np.nanmax(np.abs(g - w) / np.abs(w))}"
+
+
+# ------------------------------------------------------------------ access patterns
+# Each pattern builds (dest view, input views) over fresh buffers; `kernel` is the
+# family the planner must choose for it.
+
+def pat_flat(P, rng, code, n_in):
+    n = 1003
+    return View(P.buf(np.zeros(n, NP[code])), [n]), [View(P.buf(values(rng, code, n)), [n]) for _ in range(n_in)], "vec"
+
+
+def pat_flat_misaligned(P, rng, code, n_in):
+    n = 517
+    d = View(P.buf(np.zeros(n + 8, NP[code])), [n], offset=1)
+    return d, [View(P.buf(values(rng, code, n + 8)), [n], offset=3) for _ in range(n_in)], "vec1"
+
+
+def pat_row_bcast(P, rng, code, n_in):
+    r, c = 37, 64
+    ins = [View(P.buf(values(rng, code, r * c)), [r, c])] + [View(P.buf(values(rng, code, c)), [c]) for _ in range(n_in - 1)]
+    return View(P.buf(np.zeros(r * c, NP[code])), [r, c]), ins, "vec"
+
+
+def pat_row_bcast_odd(P, rng, code, n_in):
+    r, c = 33, 51
+    ins = [View(P.buf(values(rng, code, r * c)), [r, c])] + [View(P.buf(values(rng, code, c)), [c]) for _ in range(n_in - 1)]
+    return View(P.buf(np.zeros(r * c, NP[code])), [r, c]), ins, "vec1"
+
+
+def pat_col_bcast(P, rng, code, n_in):
+    r, c = 37, 64
+    ins = [View(P.buf(values(rng, code, r * c)), [r, c])] + [View(P.buf(values(rng, code, r)), [r, 1]) for _ in range(n_in - 1)]
+    return View(P.buf(np.zeros(r * c, NP[code])), [r, c]), ins, "vec"
+
+
+def pat_channel(P, rng, code, n_in):
+    shp = [4, 3, 8, 8]
+    n = int(np.prod(shp))
+    ins = [View(P.buf(values(rng, code, n)), shp)] + [View(P.buf(values(rng, code, 3)), [3, 1, 1]) for _ in range(n_in - 1)]
+    return View(P.buf(np.zeros(n, NP[code])), shp), ins, "vec"
+
+
+def pat_pitched(P, rng, code, n_in):
+    d = View(P.buf(np.zeros(5 * 16 + 8, NP[code])), [5, 7], [16, 1], offset=3)
+    return d, [View(P.buf(values(rng, code, 5 * 12 + 4)), [5, 7], [12, 1], offset=2) for _ in range(n_in)], "vec1"
+
+
+def pat_transposed(P, rng, code, n_in):
+    a, b = 70, 130
+    ins = [View(P.buf(values(rng, code, a * b)), [b, a]).transpose([1, 0]) for _ in range(n_in)]
+    return View(P.buf(np.zeros(a * b, NP[code])), [a, b]), ins, "tile"
+
+
+def pat_transposed_mixed(P, rng, code, n_in):
+    # first input transposed, the others contiguous / row vector
+    a, b = 96, 80
+    ins = [View(P.buf(values(rng, code, a * b)), [b, a]).transpose([1, 0])]
+    if n_in >= 2:
+        ins.append(View(P.buf(values(rng, code, a * b)), [a, b]))
+    if n_in >= 3:
+        ins.append(View(P.buf(values(rng, code, b)), [b]))
+    return View(P.buf(np.zeros(a * b, NP[code])), [a, b]), ins, "tile"
+
+
+def pat_permuted_3d(P, rng, code, n_in):
+    # planar <- interleaved: dest [3,20,24] contiguous, inputs [20,24,3] viewed through transpose [2 0 1]
+    ins = [View(P.buf(values(rng, code, 20 * 24 * 3)), [20, 24, 3]).transpose([2, 0, 1]) for _ in range(n_in)]
+    return View(P.buf(np.zeros(3 * 20 * 24, NP[code])), [3, 20, 24]), ins, None
+
+
+def pat_dest_transposed(P, rng, code, n_in):
+    a, b = 40, 72
+    d = View(P.buf(np.zeros(a * b, NP[code])), [b, a]).transpose([1, 0])
+    return d, [View(P.buf(values(rng, code, a * b)), [a, b]) for _ in range(n_in)], "tile"
+
+
+def pat_strided_vector(P, rng, code, n_in):
+    d = View(P.buf(np.zeros(50, NP[code])), [9], [5], offset=2)
+    return d, [View(P.buf(values(rng, code, 40)), [9], [4], offset=1) for _ in range(n_in)], "general"
+
+
+def pat_commensurate(P, rng, code, n_in):
+    # [8,6] <- [4,3]: dimensions divide but are neither 1 nor full
+    ins = [View(P.buf(values(rng, code, 12)), [4, 3]) for _ in range(n_in)]
+    return View(P.buf(np.zeros(48, NP[code])), [8, 6]), ins, "general"
+
+
+def pat_gather(P, rng, code, n_in):
+    idx = P.buf(np.array([1, 2, 1, 0, 2, 1], np.int32))
+    ins = [View(P.buf(values(rng, code, 2 * 3 * 3)), [2, 3, 6], [9, 3, 1], index=[None, None, idx]) for _ in range(n_in)]
+    return View(P.buf(np.zeros(36, NP[code])), [2, 3, 6]), ins, "general"
+
+
+def pat_single(P, rng, code, n_in):
+    return View(P.buf(np.zeros(1, NP[code])), [1]), [View(P.buf(values(rng, code, 1)), [1]) for _ in range(n_in)], None
+
+
+PATTERNS = [pat_flat, pat_flat_misaligned, pat_row_bcast, pat_row_bcast_odd, pat_col_bcast, pat_channel, pat_pitched,
+            pat_transposed, pat_transposed_mixed, pat_permuted_3d, pat_dest_transposed, pat_strided_vector,
+            pat_commensurate, pat_gather, pat_single]
+
+
+@pytest.mark.parametrize("pattern", PATTERNS, ids=lambda f: f.__name__[4:])
+@pytest.mark.parametrize("code", H.ALL_DTYPES)
+def test_binary_op_patterns(P, pattern, code):
+    rng = np.random.default_rng(1)
+    dest, (x, y), kernel = pattern(P, rng, code, 2)
+    for op, xa, ya in (("+", 1.0, 1.0), ("+", 1.0, -1.0), ("*", 2.0, 0.5 if code in FLOATS else 3.0), ("max", 1.0, 1.0)):
+        k = P.run(H.binary_op, dest, x, xa, y, ya, op)
+        compare(dest.buf, f"{pattern.__name__} {op} ({k})")
+        if kernel:
+            assert k == kernel, (pattern.__name__, k)
+
+
+@pytest.mark.parametrize("pattern", PATTERNS, ids=lambda f: f.__name__[4:])
+@pytest.mark.parametrize("code", [capi.F32, capi.I16, capi.F64])
+def test_ternary_and_unary_patterns(P, pattern, code):
+    rng = np.random.default_rng(2)
+    dest, (x, y, z), kernel = pattern(P, rng, code, 3)
+    k = P.run(H.ternary_op, dest, x, 1.0, y, 1.0, z, 1.0)
+    compare(dest.buf, f"select {pattern.__name__} ({k})")
+    if kernel:
+        assert k == kernel
+    k = P.run(H.ternary_op, dest, x, -1.0, y, 2.0, z, 3.0)
+    compare(dest.buf, f"select alphas {pattern.__name__} ({k})")
+    k = P.run(H.unary_op, dest, x, 1.0, "noop")
+    compare(dest.buf, f"noop {pattern.__name__} ({k})")
+    k = P.run(H.unary_op, dest, y, 1.0, "exp")
+    compare(dest.buf, f"exp {pattern.__name__} ({k})", tol=REL_TOL if code == capi.F32 else (REL_TOL_F64 if code == capi.F64 else None))
+
+
+@pytest.mark.parametrize("pattern", [pat_flat, pat_transposed, pat_pitched, pat_gather, pat_commensurate, pat_channel],
+                         ids=lambda f: f.__name__[4:])
+@pytest.mark.parametrize("src", H.ALL_DTYPES)
+@pytest.mark.parametrize("dst", H.ALL_DTYPES)
+def test_assign_all_dtype_pairs(P, pattern, src, dst):
+    rng = np.random.default_rng(3)
+    dest, (x,), _ = pattern(P, rng, src, 1)
+    # swap the destination buffer for one of the destination datatype
+    dbuf = P.buf(np.zeros(dest.buf.init.size, NP[dst]))
+    dest = View(dbuf, dest.shape, dest.strides, dest.offset)
+    # spread the source values over the whole range of its type, specials included
+    raw = x.buf.init.copy()
+    if src in FLOATS:
+        raw = (raw.astype(np.float64) * 1e4).astype(NP[src])
+        raw[:8] = np.array([np.nan, np.inf, -np.inf, 3e9, -3e9, 1e19, -1e19, 300.7][:min(8, raw.size)], NP[src])[:raw.size]
+    else:
+        info = np.iinfo(NP[src])
+        raw = rng.integers(info.min, info.max, raw.size, endpoint=True).astype(NP[src])
+    x.buf.init[...] = raw
+    x.buf.reset()
+    k = P.run(H.assign, dest, x)
+    compare(dbuf, f"assign {src}->{dst} {pattern.__name__} ({k})")
+
+
+@pytest.mark.parametrize("code", H.ALL_DTYPES)
+@pytest.mark.parametrize("op", list(capi.UNARY_OPS))
+def test_unary_ops_all_dtypes(P, code, op):
+    rng = np.random.default_rng(4)
+    n = 777
+    x = values(rng, code, n, lo=-60, hi=60)
+    if code in FLOATS:
+        x[:12] = np.array([0.0, -0.0, 0.5, 1.5, 2.5, -0.5, -1.5, 0.49999997, np.nan, np.inf, -np.inf, 88.0], NP[code])
+    xb, db = P.buf(x), P.buf(np.zeros(n, NP[code]))
+    tol = None
+    if op in TRANSCENDENTAL:
+        # integer tensors evaluate these in double too; a long result above 2^53 shows the
+        # last-ulp difference between the device's and the host's exp
+        tol = REL_TOL if code == capi.F32 else REL_TOL_F64
+    for alpha in (1.0, -1.0, 0.37 if code in FLOATS else 2.0):
+        k = P.run(H.unary_op, View(db, [n]), View(xb, [n]), alpha, op)
+        compare(db, f"{op} alpha {alpha} ({k})", tol=tol)
+    # in place (unary-accum!)
+    k = P.run(H.unary_accum, View(xb, [n]), 1.0, op)
+    compare(xb, f"accum {op} ({k})", tol=tol)
+
+
+@pytest.mark.parametrize("code", H.ALL_DTYPES)
+@pytest.mark.parametrize("op", list(capi.BINARY_OPS))
+def test_binary_ops_all_dtypes(P, code, op):
+    rng = np.random.default_rng(5)
+    n = 640
+    # every form below divides by x or by y somewhere, so both stay away from zero for :/
+    x = values(rng, code, n, nonzero=(op == "/"))
+    y = values(rng, code, n, nonzero=(op == "/"))
+    if code in FLOATS:
+        sp = np.array([0.0, -0.0, np.nan, np.inf, -np.inf, 1.0, -1.0, 1e30], NP[code])
+        x[:8], y[:8] = sp, sp[::-1]
+        x[8:16], y[8:16] = sp, sp
+    xb, yb, db = P.buf(x), P.buf(y), P.buf(np.zeros(n, NP[code]))
+    V = lambda b: View(b, [n])
+    for xa, ya in ((1.0, 1.0), (1.0, -1.0), (2.0, 3.0)):
+        k = P.run(H.binary_op, V(db), V(xb), xa, V(yb), ya, op)
+        compare(db, f"binary {op} {xa},{ya} ({k})")
+    scalar = 3.0
+    for rev in (False, True):
+        k = P.run(H.binary_op_constant, V(db), V(xb), 2.0, scalar, op, reverse=rev)
+        compare(db, f"binary-constant {op} rev={rev} ({k})")
+    # accumulate forms (dest is an operand)
+    acc = P.buf(y)
+    for rev in (False, True):
+        k = P.run(H.binary_accum, V(acc), 1.0, V(xb), 1.0, op, reverse=rev, requires_cas=False)
+        compare(acc, f"binary-accum {op} rev={rev} ({k})")
+        acc.reset()
+        k = P.run(H.binary_accum_constant, V(acc), 1.0, scalar, op, reverse=rev)
+        compare(acc, f"binary-accum-constant {op} rev={rev} ({k})")
+        acc.reset()
+
+
+@pytest.mark.parametrize("code", H.ALL_DTYPES)
+def test_ternary_constant_variants(P, code):
+    rng = np.random.default_rng(6)
+    n = 300
+    a, b = P.buf(values(rng, code, n, -5, 5)), P.buf(values(rng, code, n, -5, 5))
+    d = P.buf(np.zeros(n, NP[code]))
+    V = lambda t: View(t, [n])
+    import itertools
+    for arg_idx in itertools.permutations([0, 1, 2]):
+        k = P.run(H.ternary_op_constant, V(d), V(a), 1.0, V(b), 2.0, -1.5, list(arg_idx))
+        compare(d, f"ternary-constant {arg_idx} ({k})")
+        k = P.run(H.ternary_op_constant_constant, V(d), V(a), -1.0, 2.5, -3.0, list(arg_idx))
+        compare(d, f"ternary-constant-constant {arg_idx} ({k})")
+
+
+def test_select_compares_unrounded_products_and_casts_constants_first(P):
+    x = np.array([1.0, -1.0, 0.0, -0.0, np.nan, 1e-30, -1e-30], np.float32)
+    xb, yb, zb = P.buf(x), P.buf(np.full(7, 10.0, np.float32)), P.buf(np.full(7, 20.0, np.float32))
+    d = P.buf(np.zeros(7, np.float32))
+    V = lambda t: View(t, [7])
+    P.run(H.ternary_op, V(d), V(xb), 1e-30, V(yb), 1.0, V(zb), 1.0)
+    compare(d, "three tensors")
+    assert d.host.tolist() == [20.0, 10.0, 20.0, 20.0, 10.0, 20.0, 10.0]
+    P.run(H.ternary_op_constant, V(d), V(xb), 1e-30, V(yb), 1.0, 20.0, [0, 1, 2])
+    compare(d, "two tensors and a constant")
+    assert d.host.tolist() == [20.0, 10.0, 20.0, 20.0, 10.0, 20.0, 20.0]
+
+
+@pytest.mark.parametrize("code", H.ALL_DTYPES)
+def test_assign_constant_and_memset(P, code):
+    n = 1000
+    d = P.buf(np.zeros(n + 5, NP[code]))
+    for value in (0.0, 7.0, -3.9, 300.7):
+        P.run(H.memset, View(d, [n], offset=5), value, n)
+        compare(d, f"memset {value}")
+    s = P.buf(np.zeros(64, NP[code]))
+    # a column of a [8,8] matrix (non dense): assign-constant!
+    k = P.run(H.assign_constant, View(s, [8], [8], offset=3), 5.0)
+    compare(s, f"assign-constant column ({k})")
+    k = P.run(H.assign_constant, View(s, [4, 3], [8, 1], offset=9), -2.0)
+    compare(s, f"assign-constant submatrix ({k})")
+
+
+# ------------------------------------------------------------------ accumulate into a broadcast / indexed destination
+
+@pytest.mark.parametrize("code", [capi.F32, capi.F64, capi.I32, capi.I64, capi.I8])
+def test_binary_accum_broadcast_destination_is_serial_exact(P, code):
+    rng = np.random.default_rng(7)
+    for dshape, yshape in (([5, 1, 1], [3, 5, 4, 4]), ([7], [6, 7]), ([6, 1], [6, 9]), ([1], [50])):
+        ny = int(np.prod(yshape))
+        y = P.buf(values(rng, code, ny, -9, 9, nonzero=True))
+        d = P.buf(values(rng, code, int(np.prod(dshape)), -9, 9))
+        for op, da, ya, rev in (("+", 1.0, 1.0, False), ("+", 1.0, 2.0, True), ("-", 1.0, 1.0, True), ("max", 1.0, 1.0, False),
+                                ("*", 1.0, 1.0, False) if code in FLOATS else ("bit-xor", 1.0, 1.0, False)):
+            k = P.run(H.binary_accum, View(d, dshape), da, View(y, yshape), ya, op, reverse=rev, requires_cas=True)
+            compare(d, f"accum {op} {dshape}<-{yshape} ({k})")
+            assert k == "accum_owner", k
+            d.reset()
+
+
+def test_binary_accum_large_sum_uses_double_accumulation(P):
+    # bias gradient: dest [C,1,1] += y [N,C,H,W]; the reference tolerates 1e-4 here
+    rng = np.random.default_rng(8)
+    n, c, hw = 16, 6, 32 * 32
+    y = P.buf(rng.random(n * c * hw).astype(np.float32))
+    d = P.buf(np.zeros(c, np.float32))
+    k = P.run(H.binary_accum, View(d, [c, 1, 1]), 1.0, View(y, [n, c, 32, 32]), 1.0, "+", requires_cas=True)
+    assert k == "accum_sum"
+    exact = y.init.astype(np.float64).reshape(n, c, hw).sum(axis=(0, 2))
+    got = d.download().astype(np.float64)
+    assert np.all(np.abs(got - exact) <= 1e-6 * exact)              # ours: one rounding
+    assert np.all(np.abs(d.host - exact) <= 1e-4 * exact)           # the serial float sum drifts
+
+
+@pytest.mark.parametrize("code", [capi.F32, capi.I32, capi.F64, capi.I16])
+def test_scatter_add_through_duplicate_indexes(P, code):
+    # center-loss use case (src/cortex/verify/tensor.clj:1162-1174)
+    mat = P.buf(np.tile(np.arange(9), 2).astype(NP[code]))
+    idx = P.buf(np.array([0, 1, 0, 2, 1], np.int32))
+    centers = View(mat, [5, 3], [3, 1], index=[idx, None])
+    batch = P.buf(np.zeros(15, NP[code]))
+    P.run(H.assign, View(batch, [5, 3]), centers)
+    compare(batch, "gather")
+    assert batch.host.tolist() == [0, 1, 2, 3, 4, 5, 0, 1, 2, 6, 7, 8, 3, 4, 5]
+    k = P.run(H.binary_accum, centers, 1.0, View(batch, [5, 3]), 1.0, "+", reverse=True, requires_cas=True)
+    compare(mat, f"scatter-add ({k})")
+    assert k == "serial"
+    assert mat.host[:9].tolist() == [0, 3, 6, 9, 12, 15, 12, 14, 16]
+
+
+# ------------------------------------------------------------------ reductions
+
+def reduce_scale(x64, axis, op, alpha):
+    v = np.abs(x64 * alpha)
+    if op in ("magnitude-squared",):
+        return (v * v).sum(axis=axis)
+    return v.sum(axis=axis) if op in ("sum", "mean", "magnitude") else v.max(axis=axis)
+
+
+@pytest.mark.parametrize("code", H.ALL_DTYPES)
+@pytest.mark.parametrize("shape", [(5, 10), (33, 64), (17, 257), (9, 2048), (300, 16), (2, 3, 40)], ids=str)
+def test_reduce_last_axis_and_transposed(P, code, shape):
+    rng = np.random.default_rng(9)
+    n = int(np.prod(shape))
+    x = values(rng, code, n, -11, 11)
+    xb = P.buf(x)
+    lead = int(np.prod(shape[:-1]))
+    for alpha in (1.0, 2.0):
+        for op in capi.REDUCE_OPS:
+            out = P.buf(np.zeros(lead, NP[code]))
+            k = P.run(H.unary_reduce, View(out, list(shape[:-1]) + [1]), alpha, View(xb, list(shape)), op)
+            check_reduce(out, x.reshape(lead, shape[-1]).astype(np.float64), 1, op, alpha, code, f"rows {shape} ({k})")
+            if len(shape) == 2:  # the other axis, through a transposed view
+                out2 = P.buf(np.zeros(shape[1], NP[code]))
+                k = P.run(H.unary_reduce, View(out2, [shape[1], 1]), alpha, View(xb, list(shape)).transpose([1, 0]), op)
+                check_reduce(out2, x.reshape(shape).astype(np.float64), 0, op, alpha, code, f"cols {shape} ({k})")
+
+
+def check_reduce(out, x64, axis, op, alpha, code, what):
+    if code not in FLOATS:
+        compare(out, what)            # integer reductions are exact in any order
+        return
+    got, want = out.download().astype(np.float64), out.host.astype(np.float64)
+    if op in ("max", "min"):
+        H.assert_bit_exact(out.download(), out.host, what)
+        return
+    # relative to the sum of magnitudes: a sum of N(0,1) values can land anywhere near zero
+    scale = reduce_scale(x64, axis, op, alpha)
+    if op == "mean":
+        scale = scale / x64.shape[axis]
+    if op == "magnitude":
+        scale = np.sqrt(reduce_scale(x64, axis, "magnitude-squared", alpha))
+    tol = REL_TOL if code == capi.F32 else REL_TOL_F64
+    assert np.all(np.abs(got - want) <= tol * scale + 0.0), (what, np.max(np.abs(got - want) / scale))
+
+
+def test_reduce_kernel_selection(P):
+    rng = np.random.default_rng(10)
+    x = P.buf(rng.standard_normal(64 * 4096).astype(np.float32))
+    out = P.buf(np.zeros(4096, np.float32))
+    assert P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 4096]), "sum") == "reduce_row256_vec"
+    assert P.run(H.unary_reduce, View(out, [1024, 1]), 1.0, View(x, [1024, 256]), "sum") == "reduce_row64_vec"
+    assert P.run(H.unary_reduce, View(out, [4096, 1]), 1.0, View(x, [4096, 64]), "sum") == "reduce_row16"
+    assert P.run(H.unary_reduce, View(out, [4096, 1]), 1.0, View(x, [64, 4096]).transpose([1, 0]), "sum") == "reduce_col_vec"
+    idx = P.buf(np.arange(63, -1, -1).astype(np.int32))
+    k = P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 64], [4096, 1], index=[idx, None]), "max")
+    assert k == "reduce_any"
+    compare(out, "indexed reduce")
+
+
+def test_reduce_nan_propagates_and_signed_zero(P):
+    x = np.zeros((4, 512), np.float32)
+    x[0, 100] = np.nan
+    x[1, :] = -0.0
+    x[2, ::2] = -0.0
+    x[3, :] = -1.0
+    xb, out = P.buf(x), P.buf(np.zeros(4, np.float32))
+    for op in ("max", "min"):
+        P.run(H.unary_reduce, View(out, [4, 1]), 1.0, View(xb, [4, 512]), op)
+        H.assert_bit_exact(out.download(), out.host, op)
+        out2 = P.buf(np.zeros(512, np.float32))
+        P.run(H.unary_reduce, View(out2, [512, 1]), 1.0, View(xb, [4, 512]).transpose([1, 0]), op)
+        H.assert_bit_exact(out2.download(), out2.host, op + " columns")
+
+
+# ------------------------------------------------------------------ optimizers
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("n,offsets", [(1, (0, 0)), (4099, (0, 0)), (1000, (4, 4)), (1001, (1, 3)), (65536 + 7, (2, 2))])
+def test_adam_and_adadelta_bit_exact(P, code, n, offsets):
+    rng = np.random.default_rng(12)
+    dt = NP[code]
+    p = P.buf(rng.uniform(-0.05, 0.05, n).astype(dt))
+    g = P.buf((rng.standard_normal(n) * 1e-3).astype(dt))
+    # m and v live at an element offset inside a larger flat state buffer
+    m = P.buf((rng.standard_normal(n + 8) * 1e-4).astype(dt))
+    v = P.buf((rng.random(n + 8) * 1e-6).astype(dt))
+    Vm, Vv = View(m, [n], offset=offsets[0]), View(v, [n], offset=offsets[1])
+    pb1 = pb2 = 1.0
+    for step in range(3):
+        pb1, pb2 = pb1 * 0.9, pb2 * 0.999
+        k = P.run(H.adam_step, 1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 0.5, View(g, [n]), View(p, [n]), Vm, Vv, n)
+        for name, b in (("params", p), ("m", m), ("v", v)):
+            compare(b, f"adam {name} step {step} ({k})")
+    for step in range(3):
+        k = P.run(H.adadelta_step, 0.05, 1e-6, Vm, Vv, 0.7, View(g, [n]), View(p, [n]), n)
+        for name, b in (("params", p), ("grad-accum", m), ("dx-accum", v)):
+            compare(b, f"adadelta {name} step {step} ({k})")
+
+
+# ------------------------------------------------------------------ errors
+
+def test_invalid_arguments_are_reported(P):
+    import ctypes as C
+    d = P.buf(np.zeros(4, np.float32))
+    dims = capi.make_dims([4], [1])
+    with pytest.raises(capi.CortexHipError, match="unknown datatype"):
+        capi.call("ct_assign_constant", None, d.dev, C.byref(dims), 42, 1.0, 4)
+    with pytest.raises(capi.CortexHipError, match="unknown unary"):
+        capi.call("ct_unary_op", None, d.dev, C.byref(dims), d.dev, C.byref(dims), 1.0, 99, capi.F32, 4)
+    with pytest.raises(capi.CortexHipError, match="unknown binary"):
+        capi.call("ct_binary_op", None, d.dev, C.byref(dims), d.dev, C.byref(dims), 1.0, d.dev, C.byref(dims), 1.0, 4, 77, capi.F32)
+    with pytest.raises(capi.CortexHipError, match="null"):
+        capi.call("ct_binary_op", None, d.dev, C.byref(dims), None, C.byref(dims), 1.0, d.dev, C.byref(dims), 1.0, 4, 0, capi.F32)
+    bad = capi.CtDims()
+    bad.ndim = 9
+    with pytest.raises(capi.CortexHipError, match="rank"):
+        capi.call("ct_assign_constant", None, d.dev, C.byref(bad), capi.F32, 1.0, 4)
+    with pytest.raises(capi.CortexHipError, match="float or double"):
+        capi.call("ct_adam_step", None, capi.I32, 1e-3, 0.9, 0.999, 1e-8, 0.9, 0.999, 1.0, d.dev, d.dev, d.dev, d.dev, 4)
+    with pytest.raises(capi.CortexHipError, match="permutation"):
+        capi.call("ct_ternary_op_constant_constant", None, d.dev, C.byref(dims), d.dev, C.byref(dims), 1.0, 1.0, 2.0, 4, 0,
+                  capi.arg_idx([0, 0, 1]), capi.F32)
+    # empty work is a no-op
+    capi.call("ct_assign_constant", None, d.dev, C.byref(dims), capi.F32, 1.0, 0)
+
+
+def test_streams_and_events(P):
+    import ctypes as C
+    s = C.c_void_p()
+    capi.call("ct_stream_create", C.byref(s))
+    d = P.buf(np.zeros(1 << 20, np.float32))
+    capi.call("ct_memset", s, d.dev, capi.F32, 2.5, 1 << 20)
+    e = C.c_void_p()
+    capi.call("ct_event_record", C.byref(e), s)
+    capi.call("ct_stream_wait_event", None, e)
+    capi.call("ct_event_sync", e)
+    assert np.all(d.download() == 2.5)
+    capi.call("ct_event_destroy", e)
+    capi.call("ct_stream_destroy", s)
+    free, total = C.c_size_t(), C.c_size_t()
+    capi.call("ct_memory_info", C.byref(free), C.byref(total))
+    assert 0 < free.value <= total.value

@@ -1,0 +1,450 @@
+"""Pins the CPU oracle where the reference holds no stored vector: closed forms
+(IEEE-754, Java primitive conversion rules), brute force on tiny shapes, and
+hand-computed optimizer steps the reference keeps in its examples.  CPU only.
+"""
+import itertools
+import math
+
+import numpy as np
+import pytest
+
+import harness as H
+from cortex_amd import capi
+from harness import ORACLE, Buf, View
+
+NP = H.NP_DTYPES
+
+
+def hbuf(a):
+    return Buf(np.asarray(a), gpu=False)
+
+
+# ------------------------------------------------------------------ Java conversion rules (JLS 5.1.3), restated independently
+
+INT_BITS = {capi.I8: 8, capi.I16: 16, capi.I32: 32, capi.I64: 64, capi.U8: 8}
+
+
+def java_narrow_int(v: int, code: int) -> int:
+    bits = INT_BITS[code]
+    v &= (1 << bits) - 1
+    if code != capi.U8 and v >= 1 << (bits - 1):
+        v -= 1 << bits
+    return v
+
+
+def java_fp_to_int(v: float, code: int) -> int:
+    if math.isnan(v):
+        wide = 0
+    elif code == capi.I64:
+        wide = max(-(1 << 63), min((1 << 63) - 1, int(v))) if math.isfinite(v) else ((1 << 63) - 1 if v > 0 else -(1 << 63))
+        return wide
+    else:  # through int (saturating), then truncated
+        wide = max(-(1 << 31), min((1 << 31) - 1, int(v))) if math.isfinite(v) else ((1 << 31) - 1 if v > 0 else -(1 << 31))
+    return java_narrow_int(wide, code)
+
+
+def java_convert(value, src_code: int, dst_code: int):
+    if dst_code in (capi.F32, capi.F64):
+        return NP[dst_code](value)  # numpy rounds to nearest even from ints and from double
+    if src_code in (capi.F32, capi.F64):
+        return java_fp_to_int(float(value), dst_code)
+    return java_narrow_int(int(value), dst_code)
+
+
+EDGE_VALUES = {
+    capi.F64: [0.0, -0.0, 1.5, -1.5, 300.7, -300.7, 127.9, 128.0, -129.2, 65535.6, 2147483647.0, 2147483648.0,
+               -2147483649.0, 4294967296.0 + 44.9, 1e19, -1e19, 9.3e18, float("inf"), float("-inf"), float("nan"),
+               2.0 ** 53 + 2, 16777217.0],
+    capi.I64: [0, 1, -1, 127, 128, -129, 255, 256, 32767, 32768, 65536 + 5, 2 ** 31 - 1, 2 ** 31, -2 ** 31 - 1,
+               2 ** 53 + 1, 2 ** 63 - 1, -2 ** 63, 16777217, 2 ** 24 + 3],
+}
+EDGE_VALUES[capi.F32] = [np.float32(v) for v in EDGE_VALUES[capi.F64][:-2]] + [np.float32(16777216.0)]
+EDGE_VALUES[capi.I32] = [v for v in EDGE_VALUES[capi.I64] if -2 ** 31 <= v < 2 ** 31]
+EDGE_VALUES[capi.I16] = [v for v in EDGE_VALUES[capi.I64] if -2 ** 15 <= v < 2 ** 15]
+EDGE_VALUES[capi.I8] = [v for v in EDGE_VALUES[capi.I64] if -2 ** 7 <= v < 2 ** 7]
+EDGE_VALUES[capi.U8] = [0, 1, 127, 128, 200, 255]
+
+
+@pytest.mark.parametrize("src", H.ALL_DTYPES)
+@pytest.mark.parametrize("dst", H.ALL_DTYPES)
+def test_assign_conversion_edge_values(src, dst):
+    vals = np.array(EDGE_VALUES[src], dtype=NP[src])
+    s, d = hbuf(vals), hbuf(np.zeros(vals.size, NP[dst]))
+    H.assign(ORACLE, View(d, [vals.size]), View(s, [vals.size]))
+    with np.errstate(all="ignore"):
+        want = np.array([java_convert(v, src, dst) for v in vals], dtype=NP[dst])
+    H.assert_bit_exact(d.host, want, f"assign {src}->{dst}")
+
+
+def test_assign_exhaustive_int16_and_bytes():
+    all16 = np.arange(-32768, 32768, dtype=np.int16)
+    s = hbuf(all16)
+    for dst in (capi.I8, capi.U8, capi.I32, capi.F32):
+        d = hbuf(np.zeros(all16.size, NP[dst]))
+        H.assign(ORACLE, View(d, [all16.size]), View(s, [all16.size]))
+        want = all16.astype(np.int64)
+        want = (want & 0xFF).astype(np.uint8).view(np.int8 if dst == capi.I8 else np.uint8) if dst in (capi.I8, capi.U8) \
+            else want.astype(NP[dst])
+        H.assert_bit_exact(d.host, want.astype(NP[dst]), f"int16->{dst}")
+    u8 = np.arange(256, dtype=np.uint8)
+    d = hbuf(np.zeros(256, np.float32))
+    H.assign(ORACLE, View(d, [256]), View(hbuf(u8), [256]))
+    H.assert_bit_exact(d.host, u8.astype(np.float32), "u8->f32 is exact")
+    # the reference's own marshal example in the narrowing direction: 300.7 -> (byte)(int)300.7 = 44
+    d = hbuf(np.zeros(1, np.int8))
+    H.assign(ORACLE, View(d, [1]), View(hbuf(np.array([300.7], np.float32)), [1]))
+    assert int(d.host[0]) == 44
+
+
+# ------------------------------------------------------------------ address functions: every fast path against the general formula
+
+def general_address(shape, strides, max_shape, e):
+    """elem-idx->addr (dimensions.clj:226-252) written out: dims reversed, index
+    = running quotient mod the operand's dim, quotient by the max dim."""
+    rank = len(max_shape)
+    pad = rank - len(shape)
+    mi = max(range(len(shape)), key=lambda i: (strides[i], -i))
+    shp = [1] * pad + list(shape)
+    st = [strides[mi] * shape[mi]] * pad + list(strides)
+    off, arg = 0, e
+    for i in reversed(range(rank)):
+        off += st[i] * (arg % shp[i])
+        arg //= max_shape[i]
+    return off
+
+
+def oracle_address(all_dims, which, e):
+    import ctypes as C
+    from oracle import binding as ob
+
+    structs = [capi.make_dims(s, st) for s, st in all_dims]
+    arr = (C.POINTER(capi.CtDims) * len(structs))(*[C.pointer(s) for s in structs])
+    addr, mode = C.c_int64(), C.c_int()
+    rc = ob.lib().co_elem_address(arr, len(structs), which, e, C.byref(addr), C.byref(mode))
+    assert rc == 0
+    return addr.value, mode.value
+
+
+def test_fast_address_paths_equal_the_general_formula():
+    """All shapes of rank <= 3 with dims in {1,2,3,4} as the max-shape, every
+    operand shape whose dims divide it (dense row-major and transposed)."""
+    seen_modes = set()
+    for rank in (1, 2, 3):
+        for max_shape in itertools.product([1, 2, 3, 4], repeat=rank):
+            full = (list(max_shape), H.row_major(max_shape))
+            n = int(np.prod(max_shape))
+            for op_rank in range(1, rank + 1):
+                tail = max_shape[rank - op_rank:]
+                for shp in itertools.product(*[[d for d in (1, 2, 3, 4) if m % d == 0] for m in tail]):
+                    for perm in itertools.permutations(range(op_rank)):
+                        base = H.row_major([shp[i] for i in perm])
+                        strides = [0] * op_rank
+                        for pos, i in enumerate(perm):
+                            strides[i] = base[pos]
+                        for e in range(n):
+                            got, mode = oracle_address([full, (list(shp), strides)], 1, e)
+                            seen_modes.add(mode)
+                            assert got == general_address(list(shp), strides, list(max_shape), e), \
+                                (max_shape, shp, strides, e, mode)
+    assert seen_modes == {0, 1, 2, 3}  # identity, broadcast, repeat and general were all exercised
+
+
+# ------------------------------------------------------------------ arithmetic closed forms
+
+def f32_special():
+    vals = [0.0, -0.0, 1.0, -1.0, 0.1, -0.1, 3.4e38, -3.4e38, 1e-45, -1e-45, 1.17549435e-38, 16777216.0, 16777217.0,
+            float("inf"), float("-inf"), float("nan"), 0.5, 1.5, 2.5, -0.5, -1.5, 0.49999997, 123456.789, -7.25]
+    return np.array(vals, dtype=np.float32)
+
+
+def pairs(v):
+    a, b = np.meshgrid(v, v)
+    return a.reshape(-1).copy(), b.reshape(-1).copy()
+
+
+@pytest.mark.parametrize("op", ["+", "*", "/", "max", "min", "eq", ">", ">=", "<", "<=", "bit-and", "bit-xor"])
+def test_binary_float_closed_form(op):
+    """One operation in double, one rounding to float."""
+    x, y = pairs(f32_special())
+    n = x.size
+    bx, by, bd = hbuf(x), hbuf(y), hbuf(np.zeros(n, np.float32))
+    H.binary_op(ORACLE, View(bd, [n]), View(bx, [n]), 1.0, View(by, [n]), 1.0, op)
+    xd, yd = x.astype(np.float64), y.astype(np.float64)
+    with np.errstate(all="ignore"):
+        if op == "+":
+            want = (xd + yd).astype(np.float32)
+        elif op == "*":
+            want = (xd * yd).astype(np.float32)
+        elif op == "/":
+            want = (xd / yd).astype(np.float32)
+        elif op == "max":   # (if (> x y) x y): NaN in either place yields y
+            want = np.where(xd > yd, x, y)
+        elif op == "min":   # (if (> x y) y x)
+            want = np.where(xd > yd, y, x)
+        elif op in ("bit-and", "bit-xor"):
+            to_int = lambda a: np.array([java_fp_to_int(float(t), capi.I32) for t in a], dtype=np.int64)
+            r = to_int(xd) & to_int(yd) if op == "bit-and" else to_int(xd) ^ to_int(yd)
+            want = r.astype(np.float32)
+        else:
+            fn = {"eq": np.equal, ">": np.greater, ">=": np.greater_equal, "<": np.less, "<=": np.less_equal}[op]
+            want = fn(xd, yd).astype(np.float32)
+    H.assert_bit_exact(bd.host, want.astype(np.float32), op)
+
+
+def test_binary_alpha_is_applied_in_double_before_the_op():
+    x = np.array([0.1, 1e30, 3.0, -7.5], np.float32)
+    y = np.array([0.2, 1e30, 1e-3, 2.25], np.float32)
+    bd = hbuf(np.zeros(4, np.float32))
+    H.binary_op(ORACLE, View(bd, [4]), View(hbuf(x), [4]), 2.5, View(hbuf(y), [4]), -0.3, "+")
+    a, b = np.float64(np.float32(2.5)), np.float64(np.float32(-0.3))
+    want = (x.astype(np.float64) * a + y.astype(np.float64) * b).astype(np.float32)
+    H.assert_bit_exact(bd.host, want, "alpha in double")
+
+
+@pytest.mark.parametrize("code", [capi.I8, capi.I16, capi.I32, capi.I64, capi.U8])
+def test_binary_integer_wraps_and_truncates(code):
+    info = np.iinfo(NP[code])
+    v = np.array([info.min, info.min + 1, -3 if info.min < 0 else 3, 0, 1, 2, 7, info.max - 1, info.max], dtype=NP[code])
+    x, y = pairs(v)
+    n = x.size
+    for op in ("+", "*", "/", "max", "min", "bit-and", "eq", "<"):
+        yy = np.where(y == 0, 1, y).astype(NP[code]) if op == "/" else y
+        bd = hbuf(np.zeros(n, NP[code]))
+        H.binary_op(ORACLE, View(bd, [n]), View(hbuf(x), [n]), 1.0, View(hbuf(yy), [n]), 1.0, op)
+        want = []
+        for a, b in zip(x.tolist(), yy.tolist()):
+            if op == "+":
+                r = a + b
+            elif op == "*":
+                r = a * b
+            elif op == "/":
+                q = abs(a) // abs(b) * (1 if (a >= 0) == (b >= 0) else -1)  # toward zero
+                exact = q * b == a
+                if exact or code == capi.I64:
+                    r = q
+                else:                      # Ratio.intValue saturates at the int range
+                    r = max(-2 ** 31, min(2 ** 31 - 1, q))
+            elif op == "max":
+                r = a if a > b else b
+            elif op == "min":
+                r = b if a > b else a
+            elif op == "bit-and":
+                r = java_narrow_int(a, capi.I32) & java_narrow_int(b, capi.I32)
+            elif op == "eq":
+                r = int(a == b)
+            else:
+                r = int(a < b)
+            want.append(java_narrow_int(r, code))
+        H.assert_bit_exact(bd.host, np.array(want, dtype=NP[code]), f"{op} {code}")
+
+
+def test_integer_division_by_zero_is_an_error():
+    bd = hbuf(np.zeros(2, np.int32))
+    with pytest.raises(H.OracleError, match="Divide by zero"):
+        H.binary_op(ORACLE, View(bd, [2]), View(hbuf(np.array([1, 2], np.int32)), [2]), 1.0,
+                    View(hbuf(np.array([1, 0], np.int32)), [2]), 1.0, "/")
+
+
+def java_round(v: float) -> int:
+    if math.isnan(v):
+        return 0
+    if math.isinf(v):
+        return (1 << 63) - 1 if v > 0 else -(1 << 63)
+    r = math.floor(v)
+    if v - r >= 0.5:
+        r += 1
+    return max(-(1 << 63), min((1 << 63) - 1, int(r)))
+
+
+@pytest.mark.parametrize("op", H.capi.UNARY_OPS.keys())
+def test_unary_float_closed_form(op):
+    x = f32_special()
+    n = x.size
+    for alpha in (1.0, -2.5):
+        bd = hbuf(np.zeros(n, np.float32))
+        H.unary_op(ORACLE, View(bd, [n]), View(hbuf(x), [n]), alpha, op)
+        v = x.astype(np.float64) * np.float64(np.float32(alpha))
+        with np.errstate(all="ignore"):
+            if op == "round":
+                want = np.array([java_round(float(t)) for t in v], dtype=np.float64).astype(np.float32)
+            else:
+                fn = {"floor": np.floor, "ceil": np.ceil, "-": np.negative, "tanh": np.tanh, "exp": np.exp,
+                      "sqrt": np.sqrt, "noop": lambda t: t, "logistic": lambda t: 1.0 / (1.0 + np.exp(-t))}[op]
+                want = fn(v).astype(np.float32)
+        if op in ("tanh", "exp", "logistic"):
+            # libm's double results are below one double ulp from correctly rounded, so after the
+            # rounding to float they can differ from numpy's by at most one float ulp, and rarely
+            assert H.ulp_diff_f32(bd.host, want).max() <= 1
+        else:
+            H.assert_bit_exact(bd.host, want, f"{op} alpha={alpha}")
+
+
+def test_unary_integer_routes():
+    # floor/ceil/noop go through double and saturate; round and negate stay in long and wrap
+    x = np.array([2 ** 30, -2 ** 30, 7, -7], np.int32)
+    for op, want in (("noop", [2 ** 31 - 1, -2 ** 31, 28, -28]),      # (int)(double)(x*4)
+                     ("round", [0, 0, 28, -28]),                      # (int)(long)2^32 wraps
+                     ("-", [0, 0, -28, 28]),
+                     ("sqrt", [65536, 0, 5, 0]),                      # sqrt(2^32); NaN -> 0
+                     ("logistic", [1, 0, 0, 0])):                     # 1/(1+exp(-28)) < 1 truncates to 0
+        bd = hbuf(np.zeros(4, np.int32))
+        H.unary_op(ORACLE, View(bd, [4]), View(hbuf(x), [4]), 4.0, op)
+        assert bd.host.tolist() == want, (op, bd.host.tolist())
+    # alpha is cast to the tensor datatype first: (int 2.5) = 2
+    bd = hbuf(np.zeros(2, np.int32))
+    H.unary_op(ORACLE, View(bd, [2]), View(hbuf(np.array([3, -3], np.int32)), [2]), 2.5, "noop")
+    assert bd.host.tolist() == [6, -6]
+
+
+def test_select_semantics():
+    x = np.array([1.0, -1.0, 0.0, -0.0, float("nan"), 1e-30, -1e-30], np.float32)
+    y = np.full(7, 10.0, np.float32)
+    z = np.full(7, 20.0, np.float32)
+    bd = hbuf(np.zeros(7, np.float32))
+    H.ternary_op(ORACLE, View(bd, [7]), View(hbuf(x), [7]), 1.0, View(hbuf(y), [7]), 1.0, View(hbuf(z), [7]), 1.0)
+    # (>= x 0) ? z : y; -0.0 >= 0 is true, NaN >= 0 is false
+    assert bd.host.tolist() == [20.0, 10.0, 20.0, 20.0, 10.0, 20.0, 10.0]
+    # with a constant every argument is cast to float BEFORE the comparison:
+    # -1e-30 * 1e-30 underflows to -0.0f, and -0.0 >= 0 holds
+    H.ternary_op_constant(ORACLE, View(bd, [7]), View(hbuf(x), [7]), 1e-30, View(hbuf(y), [7]), 1.0, 20.0, [0, 1, 2])
+    assert bd.host.tolist() == [20.0, 10.0, 20.0, 20.0, 10.0, 20.0, 20.0]
+    # three tensors compare the unrounded double product
+    H.ternary_op(ORACLE, View(bd, [7]), View(hbuf(x), [7]), 1e-30, View(hbuf(y), [7]), 1.0, View(hbuf(z), [7]), 1.0)
+    assert bd.host.tolist() == [20.0, 10.0, 20.0, 20.0, 10.0, 20.0, 10.0]
+
+
+# ------------------------------------------------------------------ reductions
+
+@pytest.mark.parametrize("code", [capi.F32, capi.F64])
+def test_reduce_is_sequential_double(code):
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((7, 1000)) * 1e3).astype(NP[code])
+    for alpha in (1.0, 0.37):
+        a = np.float64(NP[code](alpha))
+        for op in capi.REDUCE_OPS:
+            out = hbuf(np.zeros(7, NP[code]))
+            H.unary_reduce(ORACLE, View(out, [7, 1]), alpha, View(hbuf(x), [7, 1000]), op)
+            want = []
+            for row in x.astype(np.float64):
+                v = row * a
+                if op in ("sum", "mean"):
+                    acc = float(np.cumsum(v)[-1])  # numpy cumsum is the same left-to-right sum
+                    want.append(acc / 1000 if op == "mean" else acc)
+                elif op in ("magnitude", "magnitude-squared"):
+                    acc = float(np.cumsum(v * v)[-1])
+                    want.append(math.sqrt(acc) if op == "magnitude" else acc)
+                else:
+                    want.append(float(v.max() if op == "max" else v.min()))
+            H.assert_bit_exact(out.host, np.array(want, dtype=np.float64).astype(NP[code]), f"{op} {alpha}")
+
+
+def test_reduce_nan_and_signed_zero():
+    x = np.array([[1.0, float("nan"), 3.0], [-0.0, 0.0, -0.0], [0.0, -0.0, -0.0]], np.float32)
+    out = hbuf(np.zeros(3, np.float32))
+    H.unary_reduce(ORACLE, View(out, [3, 1]), 1.0, View(hbuf(x), [3, 3]), "max")
+    assert math.isnan(out.host[0]) and not np.signbit(out.host[1]) and not np.signbit(out.host[2])
+    H.unary_reduce(ORACLE, View(out, [3, 1]), 1.0, View(hbuf(x), [3, 3]), "min")
+    assert math.isnan(out.host[0]) and np.signbit(out.host[1]) and np.signbit(out.host[2])
+
+
+def test_reduce_integer_mean_truncates_toward_zero():
+    x = np.array([[1, 2, 4], [-1, -2, -4], [100, 27, 0]], np.int32)
+    out = hbuf(np.zeros(3, np.int32))
+    H.unary_reduce(ORACLE, View(out, [3, 1]), 1.0, View(hbuf(x), [3, 3]), "mean")
+    assert out.host.tolist() == [2, -2, 42]
+    H.unary_reduce(ORACLE, View(out, [3, 1]), 1.0, View(hbuf(x), [3, 3]), "magnitude")
+    assert out.host.tolist() == [4, 4, 103]
+
+
+def test_reduce_through_a_transposed_view():
+    x = np.arange(12, dtype=np.float64).reshape(3, 4)
+    out = hbuf(np.zeros(4))
+    H.unary_reduce(ORACLE, View(out, [4, 1]), 1.0, View(hbuf(x), [3, 4]).transpose([1, 0]), "sum")
+    assert out.host.tolist() == x.sum(axis=0).tolist()
+
+
+# ------------------------------------------------------------------ accumulate: serial order
+
+def test_binary_accum_applies_updates_in_increasing_order():
+    # dest [3] <- y [4,3], op :*, dest_alpha 2: d = ((d*2*y0)*2*y1)...; the order matters once rounding bites
+    y = (np.arange(12, dtype=np.float32) + 1.1).reshape(4, 3)
+    d0 = np.array([1.0, 2.0, 3.0], np.float32)
+    dest = hbuf(d0)
+    H.binary_accum(ORACLE, View(dest, [3]), 2.0, View(hbuf(y), [4, 3]), 1.0, "*", requires_cas=True)
+    want = d0.copy()
+    for r in range(4):
+        want = (want.astype(np.float64) * 2.0 * y[r].astype(np.float64)).astype(np.float32)
+    H.assert_bit_exact(dest.host, want, "serial accumulate")
+    # reversed operands: dest = y - dest
+    dest = hbuf(d0)
+    H.binary_accum(ORACLE, View(dest, [3]), 1.0, View(hbuf(y), [4, 3]), 1.0, "-", reverse=True, requires_cas=True)
+    want = d0.copy()
+    for r in range(4):
+        want = (y[r].astype(np.float64) - want.astype(np.float64)).astype(np.float32)
+    H.assert_bit_exact(dest.host, want, "reversed accumulate")
+
+
+# ------------------------------------------------------------------ optimizers
+
+def test_adam_hand_computed_step():
+    """examples/optimise/test/cortex/optimise/optimisers_test.clj:71-87: step size 5, decays
+    0.75 / 0.3, conditioning 0.2, third step."""
+    p, g = hbuf(np.array([1.0, 2.0, -5.0])), hbuf(np.array([5.0, 3.0, 7.0]))
+    m, v = hbuf(np.array([5.0, 2.0, -3.0])), hbuf(np.array([-1.0, -3.0, -8.0]))
+    V = lambda b: View(b, [3])
+    H.adam_step(ORACLE, 5, 0.75, 0.3, 0.2, 0.75 ** 3, 0.3 ** 3, 1.0, V(g), V(p), V(m), V(v), 3)
+    assert np.allclose(p.host, [-8.81811015, -5.613809809, -4.270259223], atol=1e-8, rtol=0)
+    assert np.allclose(m.host, [5.0, 2.25, -0.5], atol=1e-12, rtol=0)
+    assert np.allclose(v.host, [17.2, 5.4, 31.9], atol=1e-12, rtol=0)
+
+
+def test_adam_float_runs_in_double_and_rounds_once():
+    rng = np.random.default_rng(5)
+    n = 257
+    p0 = rng.uniform(-0.05, 0.05, n).astype(np.float32)
+    g0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    m0 = (rng.standard_normal(n) * 1e-4).astype(np.float32)
+    v0 = (rng.random(n) * 1e-6).astype(np.float32)
+    p, g, m, v = hbuf(p0), hbuf(g0), hbuf(m0), hbuf(v0)
+    V = lambda b: View(b, [n])
+    pb1, pb2 = 0.9 ** 7, 0.999 ** 7
+    H.adam_step(ORACLE, 1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 0.5, V(g), V(p), V(m), V(v), n)
+    f = lambda t: np.float64(np.float32(t))
+    gv = f(0.5) * g0.astype(np.float64)
+    lm = f(0.9) * m0.astype(np.float64) + (1.0 - f(0.9)) * gv
+    lv = f(0.999) * v0.astype(np.float64) + ((1.0 - f(0.999)) * gv) * gv
+    dx = f(1e-3) * (lm / ((1.0 - f(pb1)) * (np.sqrt(lv / (1.0 - f(pb2))) + f(1e-8))))
+    H.assert_bit_exact(m.host, lm.astype(np.float32), "m")
+    H.assert_bit_exact(v.host, lv.astype(np.float32), "v")
+    H.assert_bit_exact(p.host, (p0.astype(np.float64) - dx).astype(np.float32), "params")
+
+
+def test_adadelta_hand_computed_step():
+    """examples/optimise/test/cortex/optimise/optimisers_test.clj:57-69 (decay 0.5 is where the
+    example's and the core's conventions coincide), conditioning 1."""
+    p, g = hbuf(np.array([1.0, 2.0, 3.0])), hbuf(np.array([2.0, 4.0, 8.0]))
+    ga, da = hbuf(np.array([6.0, 3.0, 9.0])), hbuf(np.array([7.0, 8.0, 7.0]))
+    V = lambda b: View(b, [3])
+    H.adadelta_step(ORACLE, 0.5, 1.0, V(ga), V(da), 1.0, V(g), V(p), 3)
+    assert np.allclose(p.host, [-1.309401077, -1.703280399, -0.6950417228], atol=1e-8, rtol=0)
+    assert np.allclose(ga.host, [5.0, 9.5, 36.5], atol=1e-12, rtol=0)
+    assert np.allclose(da.host, [6.166666667, 10.85714286, 10.32666667], atol=1e-7, rtol=0)
+
+
+def test_adadelta_float_follows_the_java_step():
+    rng = np.random.default_rng(9)
+    n = 130
+    p0 = rng.uniform(-1, 1, n).astype(np.float32)
+    g0 = rng.standard_normal(n).astype(np.float32)
+    a0, d0 = rng.random(n).astype(np.float32), rng.random(n).astype(np.float32)
+    p, g, ga, da = hbuf(p0), hbuf(g0), hbuf(a0), hbuf(d0)
+    V = lambda b: View(b, [n])
+    H.adadelta_step(ORACLE, 0.05, 1e-6, V(ga), V(da), 0.7, V(g), V(p), n)
+    dec, eps = np.float64(np.float32(0.05)), np.float64(np.float32(1e-6))
+    grad = (np.float32(0.7) * g0).astype(np.float64)            # float product, then widened
+    acc = grad * grad * dec + a0.astype(np.float64) * (1.0 - dec)
+    dx = (-1.0 * np.sqrt(d0.astype(np.float64) + eps) * grad) / np.sqrt(acc + eps)
+    dacc = dx * dx * dec + d0.astype(np.float64) * (1.0 - dec)
+    H.assert_bit_exact(ga.host, acc.astype(np.float32), "grad accum")
+    H.assert_bit_exact(da.host, dacc.astype(np.float32), "dx accum")
+    H.assert_bit_exact(p.host, p0 + dx.astype(np.float32), "params (float +=)")

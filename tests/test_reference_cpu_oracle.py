@@ -1,0 +1,37 @@
+"""Pins the CPU oracle to the reference's own stored vectors: the reference's
+backend-neutral test bodies (tests/reference_suite.py) run on the oracle
+driver.  CPU only."""
+import pytest
+
+import reference_suite as rs
+from oracle_backend import OracleDriver
+
+ALL_DTYPE_TESTS = ["assign_constant", "assign_marshal", "binary_constant_op", "binary_op", "unary_op", "channel_op",
+                   "ternary_op_select", "unary_reduce", "transpose", "select", "select_transpose_interaction",
+                   "indexed_tensor", "simple_stream"]
+FLOAT_TESTS = ["activation_forward", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
+               "adam_trajectory"]
+
+
+@pytest.fixture(scope="module")
+def driver():
+    return OracleDriver()
+
+
+@pytest.mark.parametrize("datatype", rs.ALL_DTYPES)
+@pytest.mark.parametrize("name", ALL_DTYPE_TESTS)
+def test_all_dtypes(driver, name, datatype):
+    getattr(rs, name)(driver, datatype)
+
+
+@pytest.mark.parametrize("datatype", rs.FLOAT_DTYPES)
+@pytest.mark.parametrize("name", FLOAT_TESTS)
+def test_float_double(driver, name, datatype):
+    getattr(rs, name)(driver, datatype)
+
+
+@pytest.mark.parametrize("datatype", ["int", "long"])
+def test_mask(driver, datatype):
+    # the reference runs the body with :int under both names
+    # (test/clj/cortex/compute/cpu/tensor_test.clj:91-92)
+    rs.mask(driver, "int")
