@@ -101,7 +101,11 @@ def gbs(nbytes: float, ms: float) -> float:
 
 
 def run_extras(drv, device, stream, timer, capi) -> dict:
-    """BASELINE configs 0, 2, 3, 4 (additional information, not the headline)."""
+    """BASELINE configs 0, 2, 3, 4 (additional information, not the headline).
+
+    Buffers are not released between configs: on this board a large buffer
+    allocated after frees can land less favourably and cost several percent of
+    bandwidth, which would make the figures depend on the order of the configs."""
     out = {}
     rng = np.random.default_rng(0)
 
@@ -116,8 +120,6 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
     ms = time_launches(timer, stream, lambda: stream.binary_op(d, dims([1024, 1024]), x, dims([1024, 1024]), 1.0, b,
                                                                dims([1024]), 1.0, 1024 * 1024, "+"), 200)
     out["config0 binary-op! :+ [1024,1024]+[1024]"] = entry(8392704, ms)
-    for t in (x, b, d):
-        t.release()
     # the same op at a size that exercises HBM
     n = 16384
     x = upload(drv, device, stream, rng.standard_normal(n * n, dtype=np.float32))
@@ -126,8 +128,6 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
     ms = time_launches(timer, stream, lambda: stream.binary_op(d, dims([n, n]), x, dims([n, n]), 1.0, b, dims([n]), 1.0,
                                                                n * n, "+"), 20)
     out["config0 scaled binary-op! :+ [16384,16384]+[16384]"] = entry(8 * n * n + 4 * n, ms)
-    for t in (x, b, d):
-        t.release()
 
     # configs[2]: unary-reduce!
     r, c = 16384, 4096
@@ -139,8 +139,6 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
         out[f"config2 unary-reduce! :{op} last axis f32 [16384,4096]"] = entry(4 * r * c + 4 * r, ms)
         ms = time_launches(timer, stream, lambda: stream.unary_reduce(o_cols, dims([c, 1]), 1.0, x, dims([c, r], [1, c]), op), 20)
         out[f"config2 unary-reduce! :{op} axis 0 (transposed view) f32"] = entry(4 * r * c + 4 * c, ms)
-    for t in (x, o_rows, o_cols):
-        t.release()
     r = c = 4096
     x = upload(drv, device, stream, np.random.default_rng(5).standard_normal(r * c))
     o = device.allocate_device_buffer(r, "double")
@@ -149,8 +147,6 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
         out[f"config2 unary-reduce! :{op} last axis f64 [4096,4096]"] = entry(8 * r * c + 8 * r, ms)
         ms = time_launches(timer, stream, lambda: stream.unary_reduce(o, dims([c, 1]), 1.0, x, dims([c, r], [1, c]), op), 20)
         out[f"config2 unary-reduce! :{op} axis 0 (transposed view) f64"] = entry(8 * r * c + 8 * r, ms)
-    for t in (x, o):
-        t.release()
 
     # configs[3]: Adam and Adadelta over 2^28 float parameters
     n = 1 << 28
@@ -171,8 +167,6 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
     stream.memset(v, 0, 0.0, n)
     ms = time_launches(timer, stream, lambda: stream.adadelta_step(0.05, 1e-6, m, v, 1.0, g, p, n), 10)
     out["config3 Adadelta step 2^28 f32"] = entry(28 * n, ms)
-    for t in (p, g, m, v):
-        t.release()
 
     # configs[4]: mixed-dtype image normalise
     shp = [256, 3, 224, 224]
@@ -190,15 +184,11 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
     ms = time_launches(timer, stream, lambda: stream.binary_op(f2, dims(shp), f, dims(shp), 1.0, std, dims([3, 1, 1]),
                                                                1.0, n, "/"), 20)
     out["config4 binary-op! :/ per-channel std"] = entry(8 * n + 12, ms)
-    for t in (u8, f, f2, mean, std):
-        t.release()
     n = 1 << 26
     i32 = upload(drv, device, stream, np.random.default_rng(8).integers(-2 ** 31, 2 ** 31, n, dtype=np.int64).astype(np.int32))
     f64 = device.allocate_device_buffer(n, "double")
     ms = time_launches(timer, stream, lambda: stream.assign(f64, dims([n]), i32, dims([n]), n), 20)
     out["config4 assign! i32->f64 [64M]"] = entry(12 * n, ms)
-    for t in (i32, f64):
-        t.release()
     return out
 
 
@@ -336,9 +326,6 @@ def main() -> int:
             "ternary-op! :select (3 transposed)": {"us": round(sel_avg * 1e3, 2), "GB/s": round(achieved, 1)},
         },
     }
-    for t in xs + [dest]:
-        t.release()
-
     if not args.no_extras:
         log("timing the other BASELINE configs ...")
         result["others"] = run_extras(drv, device, stream, timer, capi)

@@ -8,16 +8,30 @@ namespace cthip {
 namespace {
 constexpr int64_t kLim31 = int64_t(1) << 31;
 
+// A call whose operands together exceed what the caches can hold streams
+// through them: its accesses are marked non-temporal.
+bool is_streaming(const Plan& plan, const EwOperand* ops) {
+  int64_t bytes = 0;
+  for (int k = 0; k < plan.n_ops; ++k)
+    if (ops[k].ptr) bytes += plan.n * ops[k].elem_size;
+  return bytes >= (int64_t(64) << 20);
+}
+
 void common_vec(const Plan& plan, const EwOperand* ops, VecArgs* a) {
   const Canon& c = plan.canon;
   std::memset(a, 0, sizeof(*a));
   a->n_outer = c.nd - 1;
+  a->streaming = is_streaming(plan, ops) ? 1u : 0u;
   for (int d = 0; d + 1 < c.nd; ++d) a->outer_fd[d] = FastDiv((uint32_t)c.size[d + 1]);
   for (int k = 0; k < plan.n_ops; ++k) {
     a->ptr[k] = (char*)ops[k].ptr;
     a->cbits[k] = ops[k].cbits;
     if (!ops[k].ptr) a->const_mask |= 1u << k;
     else if (c.stride[k][0] == 1) a->unit_mask |= 1u << k;
+    bool once = ops[k].ptr != nullptr;
+    for (int d = 0; d < c.nd; ++d)
+      if (c.stride[k][d] == 0 && c.size[d] > 1) once = false;
+    if (once) a->nt_mask |= 1u << k;
     for (int d = 0; d + 1 < c.nd; ++d) a->outer_stride[k][d] = c.stride[k][d + 1];
   }
 }
@@ -89,6 +103,7 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int ts, TileArgs* a, si
     ++no;
   }
   a->n_outer = no;
+  a->streaming = is_streaming(plan, ops) ? 1u : 0u;
   CT_REQUIRE(blocks < kLim31, "internal: tile grid too large");
   *grid = (uint32_t)blocks;
   size_t lds = 0;
@@ -100,7 +115,7 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int ts, TileArgs* a, si
     if (!ops[k].ptr) a->const_mask |= 1u << k;
     if (plan.via_lds[k]) {
       a->lds_mask |= 1u << k;
-      lds += tile_slot_bytes((size_t)ops[k].elem_size, ts);
+      lds = std::max(lds, tile_slot_bytes((size_t)ops[k].elem_size, ts));  // one tile, used in turn
     }
   }
   *lds_bytes = lds;

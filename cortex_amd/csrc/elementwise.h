@@ -43,6 +43,13 @@ template <class V> __device__ __forceinline__ V nt_load(const V* p) {
   return v;
 }
 
+template <class V> __device__ __forceinline__ void nt_store(const V& v, V* p) {
+  using R = typename raw_bits<sizeof(V)>::type;
+  R r;
+  __builtin_memcpy(&r, &v, sizeof(V));
+  __builtin_nontemporal_store(r, reinterpret_cast<R*>(p));
+}
+
 template <class T> inline uint64_t bits_of(T c) {
   uint64_t b = 0;
   std::memcpy(&b, &c, sizeof(T));
@@ -61,10 +68,12 @@ struct VecArgs {
   int64_t outer_stride[kMaxOps][CT_MAX_DIMS - 1];
   uint32_t unit_mask;   // bit k: operand k is unit-stride along the inner axis
   uint32_t const_mask;  // bit k: operand k is a scalar constant
+  uint32_t streaming;   // the call moves more data than the caches hold: non-temporal loads
+  uint32_t nt_mask;     // bit k: operand k is read exactly once (no broadcast axis), so its loads may bypass the caches
   uint64_t cbits[kMaxOps];
 };
 
-template <class T, int VEC>
+template <class T, int VEC, bool STREAM>
 __device__ __forceinline__ Vec<T, VEC> vec_load(const VecArgs& a, int k, int64_t base, int64_t col) {
   Vec<T, VEC> r;
   if ((a.const_mask >> k) & 1u) {
@@ -72,7 +81,10 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(const VecArgs& a, int k, int64_t
 #pragma unroll
     for (int i = 0; i < VEC; ++i) r.v[i] = c;
   } else if ((a.unit_mask >> k) & 1u) {
-    r = nt_load(reinterpret_cast<const Vec<T, VEC>*>(reinterpret_cast<const T*>(a.ptr[k]) + base + col));
+    const Vec<T, VEC>* p = reinterpret_cast<const Vec<T, VEC>*>(reinterpret_cast<const T*>(a.ptr[k]) + base + col);
+    // a broadcast operand (a bias row, say) is re-read by every outer index and must stay cached
+    if (STREAM && ((a.nt_mask >> k) & 1u)) r = nt_load(p);
+    else r = *p;
   } else {
     const T c = reinterpret_cast<const T*>(a.ptr[k])[base];
 #pragma unroll
@@ -81,7 +93,13 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(const VecArgs& a, int k, int64_t
   return r;
 }
 
-template <class F, int VEC, int UNROLL>
+// One 16-byte vector per lane.  On this part one vector per lane with many
+// resident blocks sustains more bandwidth than several vectors per lane, and
+// non-temporal loads and stores add about 8 % on streams larger than the caches.
+// STREAM is a template parameter: a run-time choice between a plain and a
+// non-temporal access to the same address is folded into one plain access by
+// the compiler, which loses the hint.
+template <class F, int VEC, bool STREAM>
 __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs a) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
@@ -89,55 +107,43 @@ __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs
   using In2 = typename F::In2;
   constexpr int NIN = F::NIN;
 
-  const uint64_t first = (uint64_t)blockIdx.x * (uint64_t)(kBlock * UNROLL) + threadIdx.x;
-  Vec<In0, VEC> x0[UNROLL];
-  Vec<In1, VEC> x1[UNROLL];
-  Vec<In2, VEC> x2[UNROLL];
-  int64_t dst[UNROLL];
-  bool live[UNROLL];
-
+  const uint64_t v = (uint64_t)blockIdx.x * (uint64_t)kBlock + threadIdx.x;
+  if (v >= a.total_vecs) return;
+  int64_t off[kMaxOps] = {0, 0, 0, 0};
+  int64_t col;
+  if (a.n_outer == 0) {
+    col = (int64_t)v * VEC;
+  } else {
+    uint32_t row, cv;
+    a.inner_fd.divmod((uint32_t)v, row, cv);
+    col = (int64_t)cv * VEC;
+    for (int d = 0; d < a.n_outer; ++d) {
+      uint32_t q, r;
+      a.outer_fd[d].divmod(row, q, r);
+      row = q;
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    const uint64_t v = first + (uint64_t)u * kBlock;
-    live[u] = v < a.total_vecs;
-    if (!live[u]) continue;
-    int64_t off[kMaxOps] = {0, 0, 0, 0};
-    int64_t col;
-    if (a.n_outer == 0) {
-      col = (int64_t)v * VEC;
-    } else {
-      uint32_t row, cv;
-      a.inner_fd.divmod((uint32_t)v, row, cv);
-      col = (int64_t)cv * VEC;
-      for (int d = 0; d < a.n_outer; ++d) {
-        uint32_t q, r;
-        a.outer_fd[d].divmod(row, q, r);
-        row = q;
-#pragma unroll
-        for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
-      }
+      for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
     }
-    dst[u] = off[0] + col;
-    if constexpr (NIN >= 1) x0[u] = vec_load<In0, VEC>(a, 1, off[1], col);
-    if constexpr (NIN >= 2) x1[u] = vec_load<In1, VEC>(a, 2, off[2], col);
-    if constexpr (NIN >= 3) x2[u] = vec_load<In2, VEC>(a, 3, off[3], col);
   }
+  Vec<In0, VEC> x0;
+  Vec<In1, VEC> x1;
+  Vec<In2, VEC> x2;
+  if constexpr (NIN >= 1) x0 = vec_load<In0, VEC, STREAM>(a, 1, off[1], col);
+  if constexpr (NIN >= 2) x1 = vec_load<In1, VEC, STREAM>(a, 2, off[2], col);
+  if constexpr (NIN >= 3) x2 = vec_load<In2, VEC, STREAM>(a, 3, off[3], col);
+  Vec<Out, VEC> r;
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    if (!live[u]) continue;
-    Vec<Out, VEC> r;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      In0 p0{};
-      In1 p1{};
-      In2 p2{};
-      if constexpr (NIN >= 1) p0 = x0[u].v[i];
-      if constexpr (NIN >= 2) p1 = x1[u].v[i];
-      if constexpr (NIN >= 3) p2 = x2[u].v[i];
-      r.v[i] = f(p0, p1, p2);
-    }
-    *reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(a.ptr[0]) + dst[u]) = r;
+  for (int i = 0; i < VEC; ++i) {
+    In0 p0{};
+    In1 p1{};
+    In2 p2{};
+    if constexpr (NIN >= 1) p0 = x0.v[i];
+    if constexpr (NIN >= 2) p1 = x1.v[i];
+    if constexpr (NIN >= 3) p2 = x2.v[i];
+    r.v[i] = f(p0, p1, p2);
   }
+  Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(a.ptr[0]) + off[0] + col);
+  *dp = r;  // plain stores: non-temporal ones measured no faster here and slower for narrow inputs
 }
 
 // ------------------------------------------------------------------ TILE
@@ -152,6 +158,7 @@ struct TileArgs {
   int64_t outer_stride[kMaxOps][CT_MAX_DIMS - 2];
   uint32_t lds_mask;    // bit k: operand k is unit-stride along B and goes through LDS
   uint32_t const_mask;
+  uint32_t streaming;   // non-temporal loads and stores (see VecArgs)
   uint64_t cbits[kMaxOps];
 };
 
@@ -169,28 +176,43 @@ template <class F> struct tile_edge {
 };
 constexpr size_t tile_slot_bytes(size_t elem, int ts) { return ((elem * ts * (ts + 1)) + 15) & ~size_t(15); }
 
-// Stages one TS x TS tile of an operand that is unit-stride along B into LDS.
-// Lane tx walks B (a 256-byte coalesced row segment per wave), the block's
-// ROWS waves-rows walk A.  All loads are issued before the LDS writes; the
-// pointer is advanced by a constant step instead of being recomputed.
-template <class T, int TS, bool FULL>
-__device__ __forceinline__ void tile_stage(T* lds, const T* p, int64_t step, uint32_t a_left, bool b_ok, int tx,
-                                           int ty) {
+// Reads this lane's share of a TS x TS tile of an operand that is unit-stride
+// along B: lane tx walks B (a 256-byte coalesced row segment per wave), the
+// block's ROWS wave-rows walk A.  The pointer advances by a constant step.
+template <class T, int TS, bool FULL, bool STREAM>
+__device__ __forceinline__ void tile_read(T* v, const T* p, int64_t step, uint32_t a_left, bool b_ok, int ty) {
   constexpr int ROWS = kBlock / TS;
   constexpr int IT = TS / ROWS;
-  T v[IT];
 #pragma unroll
   for (int i = 0; i < IT; ++i) {
-    if (FULL || (b_ok && (uint32_t)(ty + i * ROWS) < a_left)) v[i] = nt_load(p + (int64_t)i * step);
-    else v[i] = T{};
+    if (FULL || (b_ok && (uint32_t)(ty + i * ROWS) < a_left)) {
+      if constexpr (STREAM) v[i] = nt_load(p + (int64_t)i * step);
+      else v[i] = p[(int64_t)i * step];
+    } else {
+      v[i] = T{};
+    }
   }
-#pragma unroll
-  for (int i = 0; i < IT; ++i) lds[(ty + i * ROWS) * (TS + 1) + tx] = v[i];
 }
 
-template <class F, bool FULL>
+// Transposes the lane values through the block's single LDS tile (padded to
+// TS + 1 columns: conflict-free both ways): v[i] holds element (a = ty + i*ROWS,
+// b = tx) on entry and element (a = tx, b = ty + i*ROWS) on exit.
+template <class T, int TS>
+__device__ __forceinline__ void tile_transpose(T* v, char* smem, int tx, int ty, bool need_sync_before) {
+  constexpr int ROWS = kBlock / TS;
+  constexpr int IT = TS / ROWS;
+  T* lds = reinterpret_cast<T*>(smem);
+  if (need_sync_before) __syncthreads();
+#pragma unroll
+  for (int i = 0; i < IT; ++i) lds[(ty + i * ROWS) * (TS + 1) + tx] = v[i];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < IT; ++i) v[i] = lds[tx * (TS + 1) + ty + i * ROWS];
+}
+
+template <class F, bool FULL, bool STREAM>
 __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const int64_t* off, uint32_t a0, uint32_t b0,
-                                          typename F::In0* l0, typename F::In1* l1, typename F::In2* l2) {
+                                          char* smem) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
   using In1 = typename F::In1;
@@ -201,18 +223,27 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   constexpr int IT = TS / ROWS;
   const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
   const uint32_t a_left = a.sizeA - a0, b_left = a.sizeB - b0;  // valid extent of this tile
+  const bool t0 = NIN >= 1 && ((a.lds_mask >> 1) & 1u), t1 = NIN >= 2 && ((a.lds_mask >> 2) & 1u),
+             t2 = NIN >= 3 && ((a.lds_mask >> 3) & 1u);
 
-  // phase 1: operands that are unit-stride along B go through LDS
+  // phase 1: every load of every transposed operand is issued before the first LDS round
+  In0 v0[IT];
+  In1 v1[IT];
+  In2 v2[IT];
+  const bool b_ok = (uint32_t)tx < b_left;
   if constexpr (NIN >= 1)
-    if (l0) tile_stage<In0, TS, FULL>(l0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
-                                      (int64_t)ROWS * a.strideA[1], a_left, (uint32_t)tx < b_left, tx, ty);
+    if (t0) tile_read<In0, TS, FULL, STREAM>(v0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
+                                     (int64_t)ROWS * a.strideA[1], a_left, b_ok, ty);
   if constexpr (NIN >= 2)
-    if (l1) tile_stage<In1, TS, FULL>(l1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
-                                      (int64_t)ROWS * a.strideA[2], a_left, (uint32_t)tx < b_left, tx, ty);
+    if (t1) tile_read<In1, TS, FULL, STREAM>(v1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
+                                     (int64_t)ROWS * a.strideA[2], a_left, b_ok, ty);
   if constexpr (NIN >= 3)
-    if (l2) tile_stage<In2, TS, FULL>(l2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
-                                      (int64_t)ROWS * a.strideA[3], a_left, (uint32_t)tx < b_left, tx, ty);
-  __syncthreads();
+    if (t2) tile_read<In2, TS, FULL, STREAM>(v2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
+                                     (int64_t)ROWS * a.strideA[3], a_left, b_ok, ty);
+  bool used = false;
+  if constexpr (NIN >= 1) if (t0) { tile_transpose<In0, TS>(v0, smem, tx, ty, used); used = true; }
+  if constexpr (NIN >= 2) if (t1) { tile_transpose<In1, TS>(v1, smem, tx, ty, used); used = true; }
+  if constexpr (NIN >= 3) if (t2) { tile_transpose<In2, TS>(v2, smem, tx, ty, used); used = true; }
 
   // phase 2: lane tx walks A (the destination's unit-stride axis), rows walk B
   const bool a_ok = (uint32_t)tx < a_left;
@@ -227,15 +258,15 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   In2 c2{};
   if constexpr (NIN >= 1) {
     if ((a.const_mask >> 1) & 1u) c0 = const_from_bits<In0>(a.cbits[1]);
-    else if (!l0) { q0 = reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + tx) * a.strideA[1] + (int64_t)(b0 + ty) * a.strideB[1]; s0 = (int64_t)ROWS * a.strideB[1]; }
+    else if (!t0) { q0 = reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + tx) * a.strideA[1] + (int64_t)(b0 + ty) * a.strideB[1]; s0 = (int64_t)ROWS * a.strideB[1]; }
   }
   if constexpr (NIN >= 2) {
     if ((a.const_mask >> 2) & 1u) c1 = const_from_bits<In1>(a.cbits[2]);
-    else if (!l1) { q1 = reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + tx) * a.strideA[2] + (int64_t)(b0 + ty) * a.strideB[2]; s1 = (int64_t)ROWS * a.strideB[2]; }
+    else if (!t1) { q1 = reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + tx) * a.strideA[2] + (int64_t)(b0 + ty) * a.strideB[2]; s1 = (int64_t)ROWS * a.strideB[2]; }
   }
   if constexpr (NIN >= 3) {
     if ((a.const_mask >> 3) & 1u) c2 = const_from_bits<In2>(a.cbits[3]);
-    else if (!l2) { q2 = reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + tx) * a.strideA[3] + (int64_t)(b0 + ty) * a.strideB[3]; s2 = (int64_t)ROWS * a.strideB[3]; }
+    else if (!t2) { q2 = reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + tx) * a.strideA[3] + (int64_t)(b0 + ty) * a.strideB[3]; s2 = (int64_t)ROWS * a.strideB[3]; }
   }
 #pragma unroll
   for (int i = 0; i < IT; ++i) {
@@ -244,33 +275,23 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
       In0 p0 = c0;
       In1 p1 = c1;
       In2 p2 = c2;
-      if constexpr (NIN >= 1) { if (l0) p0 = l0[tx * (TS + 1) + row]; else if (q0) p0 = q0[(int64_t)i * s0]; }
-      if constexpr (NIN >= 2) { if (l1) p1 = l1[tx * (TS + 1) + row]; else if (q1) p1 = q1[(int64_t)i * s1]; }
-      if constexpr (NIN >= 3) { if (l2) p2 = l2[tx * (TS + 1) + row]; else if (q2) p2 = q2[(int64_t)i * s2]; }
+      if constexpr (NIN >= 1) { if (t0) p0 = v0[i]; else if (q0) p0 = q0[(int64_t)i * s0]; }
+      if constexpr (NIN >= 2) { if (t1) p1 = v1[i]; else if (q1) p1 = q1[(int64_t)i * s1]; }
+      if constexpr (NIN >= 3) { if (t2) p2 = v2[i]; else if (q2) p2 = q2[(int64_t)i * s2]; }
+      // plain stores: element-wide non-temporal stores measured slower here
       dp[(int64_t)i * dstep] = f(p0, p1, p2);
     }
   }
 }
 
-template <class F>
+// One block per TS x TS tile.  All transposed operands share one LDS tile,
+// used in turn, so the LDS footprint (and with it the number of resident
+// blocks) does not grow with the operand count.
+template <class F, bool STREAM>
 __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileArgs a) {
-  using In0 = typename F::In0;
-  using In1 = typename F::In1;
-  using In2 = typename F::In2;
   constexpr int NIN = F::NIN;
   constexpr int TS = tile_edge<F>::value;
   extern __shared__ __align__(16) char smem[];
-
-  // LDS slots are handed out in operand order to the operands that need one.
-  In0* l0 = nullptr;
-  In1* l1 = nullptr;
-  In2* l2 = nullptr;
-  {
-    char* p = smem;
-    if (NIN >= 1 && ((a.lds_mask >> 1) & 1u)) { l0 = reinterpret_cast<In0*>(p); p += tile_slot_bytes(sizeof(In0), TS); }
-    if (NIN >= 2 && ((a.lds_mask >> 2) & 1u)) { l1 = reinterpret_cast<In1*>(p); p += tile_slot_bytes(sizeof(In1), TS); }
-    if (NIN >= 3 && ((a.lds_mask >> 3) & 1u)) { l2 = reinterpret_cast<In2*>(p); }
-  }
 
   uint32_t bid, tb, ta, q0;
   a.tilesB_fd.divmod(blockIdx.x, q0, tb);
@@ -284,8 +305,8 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
     for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
   }
   const uint32_t a0 = ta * TS, b0 = tb * TS;
-  if (a0 + TS <= a.sizeA && b0 + TS <= a.sizeB) tile_body<F, true>(f, a, off, a0, b0, l0, l1, l2);
-  else tile_body<F, false>(f, a, off, a0, b0, l0, l1, l2);
+  if (a0 + TS <= a.sizeA && b0 + TS <= a.sizeB) tile_body<F, true, STREAM>(f, a, off, a0, b0, smem);
+  else tile_body<F, false, STREAM>(f, a, off, a0, b0, smem);
 }
 
 // ------------------------------------------------------------------ GENERAL
@@ -423,12 +444,9 @@ int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use
 template <class F, int VEC>
 inline void launch_vec(hipStream_t s, const F& f, const VecArgs& a) {
   if (a.total_vecs == 0) return;
-  if (a.total_vecs >= (uint64_t)kBlock * 4 * 512) {
-    const uint64_t per = (uint64_t)kBlock * 4;
-    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 4>), dim3((uint32_t)((a.total_vecs + per - 1) / per)), dim3(kBlock), 0, s, f, a);
-  } else {
-    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 1>), dim3((uint32_t)((a.total_vecs + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, f, a);
-  }
+  const dim3 grid((uint32_t)((a.total_vecs + kBlock - 1) / kBlock));
+  if (a.streaming) hipLaunchKernelGGL((ew_vec_kernel<F, VEC, true>), grid, dim3(kBlock), 0, s, f, a);
+  else hipLaunchKernelGGL((ew_vec_kernel<F, VEC, false>), grid, dim3(kBlock), 0, s, f, a);
 }
 
 // ops[0] is the destination; ops[1..NIN] the inputs in functor order.
@@ -464,7 +482,8 @@ int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t 
     uint32_t grid = 0;
     if (int rc = prepare_tile(plan, ops, tile_edge<F>::value, &ta, &lds, &grid)) return rc;
     note_kernel("tile");
-    hipLaunchKernelGGL((ew_tile_kernel<F>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+    if (ta.streaming) hipLaunchKernelGGL((ew_tile_kernel<F, true>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+    else hipLaunchKernelGGL((ew_tile_kernel<F, false>), dim3(grid), dim3(kBlock), lds, s, f, ta);
     return after_launch(s);
   }
   GenArgs ga;

@@ -53,43 +53,92 @@ __device__ __forceinline__ double jmin(double a, double b) {
 __device__ __forceinline__ int64_t jmax(int64_t a, int64_t b) { return a > b ? a : b; }
 __device__ __forceinline__ int64_t jmin(int64_t a, int64_t b) { return a < b ? a : b; }
 
-template <class A, int RK> __device__ __forceinline__ A red_identity() {
-  if constexpr (RK == RK_MAX) {
-    if constexpr (std::is_same<A, double>::value) return -__builtin_huge_val();
-    else return INT64_MIN;
-  } else if constexpr (RK == RK_MIN) {
-    if constexpr (std::is_same<A, double>::value) return __builtin_huge_val();
-    else return INT64_MAX;
-  } else {
-    return (A)0;
+// Reduction policy with the reference's accumulator: a double for float and
+// double tensors, a long for integer tensors (cpu/tensor_math.clj:588-629).
+template <class T, int RK> struct RedWide {
+  using Elem = T;
+  using Acc = typename acc_of<T>::type;
+  using Alpha = Acc;
+  static __device__ __forceinline__ Acc identity() {
+    if constexpr (RK == RK_MAX) {
+      if constexpr (std::is_same<Acc, double>::value) return -__builtin_huge_val();
+      else return INT64_MIN;
+    } else if constexpr (RK == RK_MIN) {
+      if constexpr (std::is_same<Acc, double>::value) return __builtin_huge_val();
+      else return INT64_MAX;
+    } else {
+      return (Acc)0;
+    }
   }
-}
-template <class A, int RK> __device__ __forceinline__ A red_combine(A a, A b) {
-  if constexpr (RK == RK_MAX) return jmax(a, b);
-  else if constexpr (RK == RK_MIN) return jmin(a, b);
-  else return w_add(a, b);
-}
-template <class T, class A, int RK> __device__ __forceinline__ A red_value(T x, A alpha) {
-  const A v = w_mul(alpha, (A)x);
-  if constexpr (RK == RK_SUMSQ || RK == RK_MAG) return w_mul(v, v);
-  else return v;
-}
-// Final cast, with mean and magnitude applied (cpu/tensor_math.clj:610-622).
-template <class T, class A, int RK> __device__ __forceinline__ T red_finish(A acc, int64_t count) {
-  if constexpr (RK == RK_MEAN) {
-    if constexpr (std::is_same<A, double>::value) return jvm_cast<T>(acc / (double)count);
-    else return jvm_ratio_cast<T>(acc, count);
-  } else if constexpr (RK == RK_MAG) {
-    return jvm_cast<T>(sqrt((double)acc));
-  } else {
-    return jvm_cast<T>(acc);
+  static __device__ __forceinline__ Acc value(T x, Alpha alpha) {
+    const Acc v = w_mul(alpha, (Acc)x);
+    if constexpr (RK == RK_SUMSQ || RK == RK_MAG) return w_mul(v, v);
+    else return v;
   }
-}
+  static __device__ __forceinline__ Acc combine(Acc a, Acc b) {
+    if constexpr (RK == RK_MAX) return jmax(a, b);
+    else if constexpr (RK == RK_MIN) return jmin(a, b);
+    else return w_add(a, b);
+  }
+  // Final cast, with mean and magnitude applied (cpu/tensor_math.clj:610-622).
+  static __device__ __forceinline__ T finish(Acc acc, int64_t count) {
+    if constexpr (RK == RK_MEAN) {
+      if constexpr (std::is_same<Acc, double>::value) return jvm_cast<T>(acc / (double)count);
+      else return jvm_ratio_cast<T>(acc, count);
+    } else if constexpr (RK == RK_MAG) {
+      return jvm_cast<T>(sqrt((double)acc));
+    } else {
+      return jvm_cast<T>(acc);
+    }
+  }
+  static __device__ __forceinline__ Acc shfl(Acc v, int mask) {
+    if constexpr (std::is_same<Acc, double>::value) return __shfl_xor(v, mask, 64);
+    else return (Acc)__shfl_xor((long long)v, mask, 64);
+  }
+};
 
-template <class A> __device__ __forceinline__ A shfl_xor_any(A v, int mask) {
-  if constexpr (std::is_same<A, double>::value) return __shfl_xor(v, mask, 64);
-  else return (A)__shfl_xor((long long)v, mask, 64);
-}
+// max / min of float or double tensors with alpha == 1, without widening.
+// The IEEE bit pattern is mapped to a signed integer key whose order is the
+// numeric order with -0 below +0 (flip the magnitude bits of negative values).
+// Positive NaNs map above +infinity and negative NaNs below -infinity, so
+// keeping the largest and the smallest key seen tells whether any NaN took
+// part; Math.max / Math.min then return NaN (cpu/tensor_math.clj:591-602).
+template <class T, int RK> struct RedKeyed {
+  using Elem = T;
+  using K = typename std::conditional<sizeof(T) == 4, int32_t, int64_t>::type;
+  struct Acc { K hi, lo; };
+  using Alpha = typename acc_of<T>::type;  // unused: alpha is 1
+  static constexpr K kMag = sizeof(T) == 4 ? (K)0x7fffffff : (K)0x7fffffffffffffffLL;
+  static constexpr K kPosInf = sizeof(T) == 4 ? (K)0x7f800000 : (K)0x7ff0000000000000LL;
+  static constexpr K kNegInf = sizeof(T) == 4 ? (K)(int32_t)0x807fffff : (K)0x800fffffffffffffLL;
+  static __device__ __forceinline__ K key_of(T x) {
+    K b;
+    __builtin_memcpy(&b, &x, sizeof(T));
+    return b ^ ((b >> (sizeof(T) * 8 - 1)) & kMag);
+  }
+  static __device__ __forceinline__ Acc identity() {
+    return Acc{sizeof(T) == 4 ? (K)INT32_MIN : (K)INT64_MIN, sizeof(T) == 4 ? (K)INT32_MAX : (K)INT64_MAX};
+  }
+  static __device__ __forceinline__ Acc value(T x, Alpha) {
+    const K k = key_of(x);
+    return Acc{k, k};
+  }
+  static __device__ __forceinline__ Acc combine(Acc a, Acc b) {
+    return Acc{a.hi > b.hi ? a.hi : b.hi, a.lo < b.lo ? a.lo : b.lo};
+  }
+  static __device__ __forceinline__ T finish(Acc acc, int64_t) {
+    if (acc.hi > kPosInf || acc.lo < kNegInf) return (T)__builtin_nanf("");
+    const K k = RK == RK_MAX ? acc.hi : acc.lo;
+    const K b = k ^ ((k >> (sizeof(T) * 8 - 1)) & kMag);
+    T r;
+    __builtin_memcpy(&r, &b, sizeof(T));
+    return r;
+  }
+  static __device__ __forceinline__ Acc shfl(Acc v, int mask) {
+    if constexpr (sizeof(T) == 4) return Acc{__shfl_xor(v.hi, mask, 64), __shfl_xor(v.lo, mask, 64)};
+    else return Acc{(K)__shfl_xor((long long)v.hi, mask, 64), (K)__shfl_xor((long long)v.lo, mask, 64)};
+  }
+};
 
 struct OutAddr {
   int32_t identity;  // output address == logical index
@@ -113,16 +162,17 @@ struct RowArgs {
 };
 
 // TPR lanes per output; kBlock / TPR outputs per block.
-template <class T, int RK, int VEC, int TPR>
-__global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, const typename acc_of<T>::type alpha) {
-  using A = typename acc_of<T>::type;
+template <class P, int VEC, int TPR>
+__global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, const typename P::Alpha alpha) {
+  using T = typename P::Elem;
+  using A = typename P::Acc;
   using V = Vec<T, VEC>;
   constexpr int RPB = kBlock / TPR;
   __shared__ A lds[kBlock / 64];
   const int lane = threadIdx.x % TPR;
   const int64_t p = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
   const bool live = p < a.n_out;
-  A acc0 = red_identity<A, RK>(), acc1 = red_identity<A, RK>();
+  A acc0 = P::identity(), acc1 = P::identity();
   if (live) {
     int64_t base = 0;
     uint32_t rem = (uint32_t)p;
@@ -139,31 +189,31 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
       const V x0 = nt_load(row + i), x1 = nt_load(row + i + TPR);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        acc0 = red_combine<A, RK>(acc0, red_value<T, A, RK>(x0.v[e], alpha));
-        acc1 = red_combine<A, RK>(acc1, red_value<T, A, RK>(x1.v[e], alpha));
+        acc0 = P::combine(acc0, P::value(x0.v[e], alpha));
+        acc1 = P::combine(acc1, P::value(x1.v[e], alpha));
       }
     }
     if (i < nv) {
       const V x0 = nt_load(row + i);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) acc0 = red_combine<A, RK>(acc0, red_value<T, A, RK>(x0.v[e], alpha));
+      for (int e = 0; e < VEC; ++e) acc0 = P::combine(acc0, P::value(x0.v[e], alpha));
     }
   }
-  A acc = red_combine<A, RK>(acc0, acc1);
+  A acc = P::combine(acc0, acc1);
   constexpr int W = TPR < 64 ? TPR : 64;
 #pragma unroll
-  for (int m = W / 2; m >= 1; m >>= 1) acc = red_combine<A, RK>(acc, shfl_xor_any<A>(acc, m));
+  for (int m = W / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
   if constexpr (TPR > 64) {
     if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = acc;
     __syncthreads();
     if (threadIdx.x == 0) {
       acc = lds[0];
 #pragma unroll
-      for (int w = 1; w < kBlock / 64; ++w) acc = red_combine<A, RK>(acc, lds[w]);
+      for (int w = 1; w < kBlock / 64; ++w) acc = P::combine(acc, lds[w]);
     }
   }
   if (live && lane == 0)
-    reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc, a.k);
+    reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
 }
 
 struct ColArgs {
@@ -182,11 +232,17 @@ struct ColArgs {
   int32_t op;
 };
 
-template <class T, int RK, int VEC>
-__global__ void __launch_bounds__(kBlock) reduce_col_kernel(const ColArgs a, const typename acc_of<T>::type alpha) {
-  using A = typename acc_of<T>::type;
+// 16 waves per block: each wave-load is one 1 KiB row segment, 16 consecutive
+// rows are in flight per block, 8 loads per lane.  Measured best among 1-16
+// waves and 32-512 rows per block for a [16384, 4096] float input.
+constexpr int kColBlock = 1024;
+
+template <class P, int VEC>
+__global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, const typename P::Alpha alpha) {
+  using T = typename P::Elem;
+  using A = typename P::Acc;
   using V = Vec<T, VEC>;
-  constexpr int WAVES = kBlock / 64;
+  constexpr int WAVES = kColBlock / 64;
   __shared__ A lds[WAVES - 1][64 * VEC];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   uint32_t q0, strip, seg, rest;
@@ -204,7 +260,7 @@ __global__ void __launch_bounds__(kBlock) reduce_col_kernel(const ColArgs a, con
   const bool live = col < a.u;
   A acc[VEC];
 #pragma unroll
-  for (int e = 0; e < VEC; ++e) acc[e] = red_identity<A, RK>();
+  for (int e = 0; e < VEC; ++e) acc[e] = P::identity();
   const int64_t r0 = (int64_t)seg * a.rows_per_seg;
   int64_t r1 = r0 + a.rows_per_seg;
   if (r1 > a.k) r1 = a.k;
@@ -221,12 +277,12 @@ __global__ void __launch_bounds__(kBlock) reduce_col_kernel(const ColArgs a, con
 #pragma unroll
       for (int j = 0; j < UN; ++j)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x[j].v[e], alpha));
+        for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
     }
     for (; r < r1; r += WAVES, p += step) {
       const V x0 = nt_load(reinterpret_cast<const V*>(p));
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) acc[e] = red_combine<A, RK>(acc[e], red_value<T, A, RK>(x0.v[e], alpha));
+      for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x0.v[e], alpha));
     }
   }
   if (wave > 0) {
@@ -238,23 +294,24 @@ __global__ void __launch_bounds__(kBlock) reduce_col_kernel(const ColArgs a, con
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
 #pragma unroll
-      for (int w = 0; w < WAVES - 1; ++w) acc[e] = red_combine<A, RK>(acc[e], lds[w][e * 64 + lane]);
+      for (int w = 0; w < WAVES - 1; ++w) acc[e] = P::combine(acc[e], lds[w][e * 64 + lane]);
       const int64_t p = pbase + (int64_t)(col + e) * a.u_pmul;
-      if (a.n_seg == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc[e], a.k);
+      if (a.n_seg == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc[e], a.k);
       else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc[e];
     }
   }
 }
 
-template <class T, int RK>
+template <class P>
 __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const ColArgs a) {
-  using A = typename acc_of<T>::type;
+  using T = typename P::Elem;
+  using A = typename P::Acc;
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= a.n_out) return;
   const A* part = reinterpret_cast<const A*>(a.partials);
   A acc = part[p];
-  for (uint32_t s = 1; s < a.n_seg; ++s) acc = red_combine<A, RK>(acc, part[(int64_t)s * a.n_out + p]);
-  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc, a.k);
+  for (uint32_t s = 1; s < a.n_seg; ++s) acc = P::combine(acc, part[(int64_t)s * a.n_out + p]);
+  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
 }
 
 struct AnyArgs {
@@ -269,17 +326,18 @@ struct AnyArgs {
 };
 
 // One lane per output, in the reference's own order (sequential accumulation).
-template <class T, int RK>
-__global__ void __launch_bounds__(kBlock) reduce_any_kernel(const AnyArgs a, const typename acc_of<T>::type alpha) {
-  using A = typename acc_of<T>::type;
+template <class P>
+__global__ void __launch_bounds__(kBlock) reduce_any_kernel(const AnyArgs a, const typename P::Alpha alpha) {
+  using T = typename P::Elem;
+  using A = typename P::Acc;
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= a.n_out) return;
   const T* in = reinterpret_cast<const T*>(a.in);
   const int64_t start = p * a.k;
-  A acc = red_value<T, A, RK>(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start)], alpha);
+  A acc = P::value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start)], alpha);
   for (int64_t i = 1; i < a.k; ++i)
-    acc = red_combine<A, RK>(acc, red_value<T, A, RK>(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start + i)], alpha));
-  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = red_finish<T, A, RK>(acc, a.k);
+    acc = P::combine(acc, P::value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start + i)], alpha));
+  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
 }
 
 // ------------------------------------------------------------------ host planning
@@ -324,11 +382,12 @@ RedShape analyse(const ct_dims& in, int64_t k) {
 
 template <class T> bool aligned_for(const void* p, int vec) { return ((uintptr_t)p % (uintptr_t)(vec * sizeof(T))) == 0; }
 
-template <class T, int RK>
-int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha_d, const void* in, const ct_dims* id,
-                 int op) {
-  using A = typename acc_of<T>::type;
-  const A alpha = (A)jvm_cast<T>(alpha_d);
+template <class P>
+int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, const void* in, const ct_dims* id,
+               int op) {
+  using T = typename P::Elem;
+  using A = typename P::Acc;
+  const typename P::Alpha alpha = (typename P::Alpha)jvm_cast<T>(alpha_d);
   const int64_t n_out = dims_ecount(*od), total = dims_ecount(*id);
   const int64_t k = total / n_out;
   CT_REQUIRE(k >= 1, "unary-reduce!: input (%lld elements) is smaller than output (%lld)", (long long)total,
@@ -359,7 +418,7 @@ int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha_d, c
     }
     const int64_t row_bytes = k * (int64_t)sizeof(T);
 #define CT_ROW(VEC, TPR)                                                                                        \
-  hipLaunchKernelGGL((reduce_row_kernel<T, RK, VEC, TPR>), dim3((uint32_t)((n_out + (kBlock / TPR) - 1) / (kBlock / TPR))), \
+  hipLaunchKernelGGL((reduce_row_kernel<P, VEC, TPR>), dim3((uint32_t)((n_out + (kBlock / TPR) - 1) / (kBlock / TPR))), \
                      dim3(kBlock), 0, st, a, alpha)
     if (row_bytes >= 4096) {
       note_kernel(vec_ok ? "reduce_row256_vec" : "reduce_row256");
@@ -403,14 +462,13 @@ int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha_d, c
     const int vec = vec_ok ? VMAX : 1;
     a.n_strips = (a.u + 64 * vec - 1) / (64 * vec);
     const int64_t base_blocks = (int64_t)a.n_strips * rest_count;
-    // enough blocks to fill 256 CUs several times over, at least 16 rows per segment,
-    // partials capped at 16 MiB
-    int64_t seg = (4096 + base_blocks - 1) / base_blocks;
-    seg = std::min<int64_t>(seg, std::max<int64_t>(1, k / 16));
-    seg = std::min<int64_t>(seg, std::max<int64_t>(1, (int64_t(16) << 20) / (n_out * (int64_t)sizeof(A))));
-    seg = std::max<int64_t>(seg, 1);
-    int64_t rows = (k + seg - 1) / seg;
-    seg = (k + rows - 1) / rows;
+    // 256 rows per block when that still leaves >= 1024 blocks, fewer rows otherwise
+    // (never below one row per wave); partials capped at 16 MiB
+    int64_t rows = 256;
+    while (rows > 16 && base_blocks * ((k + rows - 1) / rows) < 1024) rows /= 2;
+    const int64_t seg_cap = std::max<int64_t>(1, (int64_t(16) << 20) / (n_out * (int64_t)sizeof(A)));
+    if ((k + rows - 1) / rows > seg_cap) rows = (k + seg_cap - 1) / seg_cap;
+    int64_t seg = (k + rows - 1) / rows;
     a.n_seg = (uint32_t)seg;
     a.rows_per_seg = (uint32_t)rows;
     a.strips_fd = FastDiv(a.n_strips);
@@ -421,10 +479,10 @@ int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha_d, c
         if (int rc = stream_scratch(st, (size_t)(seg * n_out) * sizeof(A), &a.partials)) return rc;
       }
       note_kernel(vec_ok ? "reduce_col_vec" : "reduce_col");
-      if (vec_ok) hipLaunchKernelGGL((reduce_col_kernel<T, RK, VMAX>), dim3((uint32_t)grid), dim3(kBlock), 0, st, a, alpha);
-      else hipLaunchKernelGGL((reduce_col_kernel<T, RK, 1>), dim3((uint32_t)grid), dim3(kBlock), 0, st, a, alpha);
+      if (vec_ok) hipLaunchKernelGGL((reduce_col_kernel<P, VMAX>), dim3((uint32_t)grid), dim3(kColBlock), 0, st, a, alpha);
+      else hipLaunchKernelGGL((reduce_col_kernel<P, 1>), dim3((uint32_t)grid), dim3(kColBlock), 0, st, a, alpha);
       if (seg > 1)
-        hipLaunchKernelGGL((reduce_finish_kernel<T, RK>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock),
+        hipLaunchKernelGGL((reduce_finish_kernel<P>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock),
                            0, st, a);
       return after_launch(st);
     }
@@ -438,9 +496,17 @@ int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha_d, c
   a.in_nd = in_rank;
   CT_REQUIRE((n_out + kBlock - 1) / kBlock < (int64_t(1) << 31), "unary-reduce!: too many outputs");
   note_kernel("reduce_any");
-  hipLaunchKernelGGL((reduce_any_kernel<T, RK>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
+  hipLaunchKernelGGL((reduce_any_kernel<P>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock), 0, st,
                      a, alpha);
   return after_launch(st);
+}
+
+template <class T, int RK>
+int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha, const void* in, const ct_dims* id, int op) {
+  if constexpr (std::is_floating_point<T>::value && (RK == RK_MAX || RK == RK_MIN)) {
+    if (jvm_cast<T>(alpha) == (T)1) return reduce_run<RedKeyed<T, RK>>(st, out, od, alpha, in, id, op);
+  }
+  return reduce_run<RedWide<T, RK>>(st, out, od, alpha, in, id, op);
 }
 
 template <class T>
