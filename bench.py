@@ -288,6 +288,8 @@ def main() -> int:
     # per-op times of the other two kernels of the step
     ms_exp = time_launches(timer, stream, lambda: stream.unary_op(dest, cont, xs[0], view, 1.0, "exp", nn), 20)
     ms_tanh = time_launches(timer, stream, lambda: stream.unary_op(dest, cont, xs[0], view, 1.0, "tanh", nn), 20)
+    # a plain contiguous copy of the same size: the reference point for the hardware counters
+    ms_copy = time_launches(timer, stream, lambda: stream.unary_op(dest, cont, xs[0], cont, 1.0, "noop", nn), 20)
 
     result = {
         "metric": "achieved HBM GB/s (% of MI355X peak) for binary-op!, unary-reduce!, Adam step",
@@ -323,6 +325,7 @@ def main() -> int:
         "kernels": {
             "unary-op! :exp (transposed)": {"us": round(ms_exp * 1e3, 2), "GB/s": round(gbs(8 * nn, ms_exp), 1)},
             "unary-op! :tanh (transposed)": {"us": round(ms_tanh * 1e3, 2), "GB/s": round(gbs(8 * nn, ms_tanh), 1)},
+            "unary-op! :noop (contiguous copy, calibration)": {"us": round(ms_copy * 1e3, 2), "GB/s": round(gbs(8 * nn, ms_copy), 1)},
             "ternary-op! :select (3 transposed)": {"us": round(sel_avg * 1e3, 2), "GB/s": round(achieved, 1)},
         },
     }

@@ -294,6 +294,9 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
   extern __shared__ __align__(16) char smem[];
 
   uint32_t bid, tb, ta, q0;
+  // tiles along B vary fastest: consecutive blocks read neighbouring 256-byte
+  // segments of the same source rows (measured 71 % of peak against 58 % with
+  // tiles along A fastest on a transposed [8192,8192] float input)
   a.tilesB_fd.divmod(blockIdx.x, q0, tb);
   a.tilesA_fd.divmod(q0, bid, ta);
   int64_t off[kMaxOps] = {0, 0, 0, 0};
