@@ -21,9 +21,11 @@ const char** last_kernel_slot();
 int set_error(int code, const char* fmt, ...);
 bool debug_sync();
 
-// Scratch memory owned by the library, one growing block per (device, stream).
-// Kernels of one stream run in order, so consecutive calls may reuse it.
-int stream_scratch(hipStream_t s, size_t bytes, void** out);
+// Scratch memory owned by the library, one growing block per (device, stream,
+// slot).  Kernels of one stream run in order, so consecutive calls may reuse a
+// slot; a call that needs two live temporaries uses two slots.
+enum ScratchSlot { kScratchReduce = 0, kScratchAccumA = 1, kScratchAccumB = 2, kScratchSlots = 3 };
+int stream_scratch(hipStream_t s, size_t bytes, void** out, int slot = kScratchReduce);
 void release_stream_scratch(hipStream_t s);
 
 inline void note_kernel(const char* name) { *last_kernel_slot() = name; }

@@ -24,18 +24,23 @@ namespace {
 struct ScratchKey {
   int device;
   hipStream_t stream;
-  bool operator<(const ScratchKey& o) const { return device != o.device ? device < o.device : stream < o.stream; }
+  int slot;
+  bool operator<(const ScratchKey& o) const {
+    if (device != o.device) return device < o.device;
+    if (stream != o.stream) return stream < o.stream;
+    return slot < o.slot;
+  }
 };
 struct ScratchBlock { void* ptr; size_t bytes; };
 std::mutex g_scratch_mutex;
 std::map<ScratchKey, ScratchBlock> g_scratch;
 }  // namespace
 
-int stream_scratch(hipStream_t s, size_t bytes, void** out) {
+int stream_scratch(hipStream_t s, size_t bytes, void** out, int slot) {
   int dev = 0;
   CT_HIP(hipGetDevice(&dev));
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  ScratchBlock& b = g_scratch[ScratchKey{dev, s}];
+  ScratchBlock& b = g_scratch[ScratchKey{dev, s, slot}];
   if (b.bytes < bytes) {
     if (b.ptr) {
       // earlier kernels of this stream may still be reading the old block
@@ -56,10 +61,12 @@ void release_stream_scratch(hipStream_t s) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return;
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  auto it = g_scratch.find(ScratchKey{dev, s});
-  if (it == g_scratch.end()) return;
-  if (it->second.ptr) (void)hipFree(it->second.ptr);
-  g_scratch.erase(it);
+  for (int slot = 0; slot < kScratchSlots; ++slot) {
+    auto it = g_scratch.find(ScratchKey{dev, s, slot});
+    if (it == g_scratch.end()) continue;
+    if (it->second.ptr) (void)hipFree(it->second.ptr);
+    g_scratch.erase(it);
+  }
 }
 
 int set_error(int code, const char* fmt, ...) {

@@ -7,14 +7,21 @@
 // integer tensors), seeded with the first element, and is rounded once at the
 // store.  max and min are java.lang.Math.max/min: NaN propagates and +0 > -0.
 //
-// Three kernels:
-//   reduce_row_kernel   the reduced axis is unit-stride in memory: a group of
-//                       16, 64 or 256 lanes owns one output, reads its row with
-//                       128-bit loads, accumulates in double and combines with
-//                       wavefront shuffles (and LDS across the 4 waves)
+// Kernels:
+//   reduce_row_small_kernel  unit-stride rows of at most 256 vectors: a group
+//                       of 4, 16 or 64 lanes inside one wave takes up to four
+//                       consecutive rows, issues every load up front and
+//                       combines with shuffles only
+//   reduce_row_kernel   longer unit-stride rows: a group of 64 or 256 lanes
+//                       owns one output, reads its row with 128-bit loads,
+//                       accumulates in double and combines with wavefront
+//                       shuffles (and LDS across the 4 waves); when there are
+//                       too few rows to fill the chip each row is cut into
+//                       chunks whose partial results reduce_finish_kernel
+//                       combines
 //   reduce_col_kernel   the reduced axis is strided and another axis is
 //                       unit-stride (a transposed view): lanes own columns,
-//                       the 4 waves of a block stride down the rows so every
+//                       the 16 waves of a block stride down the rows so every
 //                       load stays coalesced; rows are split over blocks into
 //                       segments whose partial results go to scratch memory and
 //                       are combined by reduce_finish_kernel (deterministic, no
@@ -67,7 +74,10 @@ template <class T, int RK> struct RedWide {
       if constexpr (std::is_same<Acc, double>::value) return __builtin_huge_val();
       else return INT64_MAX;
     } else {
-      return (Acc)0;
+      // -0.0 is the additive identity that keeps a sum of negative zeros negative,
+      // as the reference's first-element seed does
+      if constexpr (std::is_same<Acc, double>::value) return -0.0;
+      else return (Acc)0;
     }
   }
   static __device__ __forceinline__ Acc value(T x, Alpha alpha) {
@@ -150,10 +160,24 @@ __device__ __forceinline__ int64_t out_address(const OutAddr& o, int64_t p) {
   return o.identity ? p : ref_address(o.op, o.nd, o.rmax, p);
 }
 
+// Partial accumulators of a reduction split over several blocks:
+// partials[seg * n_out + p], combined in increasing seg by reduce_finish_kernel.
+struct FinishArgs {
+  const void* partials;
+  void* out;
+  int64_t k, n_out;
+  uint32_t n_seg;
+  OutAddr oa;
+};
+
 struct RowArgs {
   const void* in;
   void* out;
+  void* partials;       // [n_split][n_out] accumulators when n_split > 1
   int64_t k, n_out;
+  int64_t chunk;        // elements of a row one lane group covers (k when n_split == 1)
+  FastDiv split_fd;     // n_split
+  uint32_t n_split;
   int32_t n_outer;
   FastDiv osize[CT_MAX_DIMS];   // kept axes, fastest first
   int64_t ostride[CT_MAX_DIMS];
@@ -161,7 +185,9 @@ struct RowArgs {
   int32_t op;
 };
 
-// TPR lanes per output; kBlock / TPR outputs per block.
+// TPR lanes per output; kBlock / TPR outputs per block.  A long row may be cut
+// into n_split chunks, each taken by its own lane group, when there are too
+// few rows to fill the chip (the norm of a whole parameter vector).
 template <class P, int VEC, int TPR>
 __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, const typename P::Alpha alpha) {
   using T = typename P::Elem;
@@ -170,12 +196,16 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
   constexpr int RPB = kBlock / TPR;
   __shared__ A lds[kBlock / 64];
   const int lane = threadIdx.x % TPR;
-  const int64_t p = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
-  const bool live = p < a.n_out;
+  const int64_t vp = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+  const bool live = vp < a.n_out * (int64_t)a.n_split;
+  uint32_t p = (uint32_t)vp, seg = 0;
+  if (a.n_split > 1) a.split_fd.divmod((uint32_t)vp, p, seg);
   A acc0 = P::identity(), acc1 = P::identity();
   if (live) {
-    int64_t base = 0;
-    uint32_t rem = (uint32_t)p;
+    int64_t base = (int64_t)seg * a.chunk;
+    int64_t len = a.k - base;
+    if (len > a.chunk) len = a.chunk;
+    uint32_t rem = p;
     for (int d = 0; d < a.n_outer; ++d) {
       uint32_t q, r;
       a.osize[d].divmod(rem, q, r);
@@ -183,7 +213,7 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
       base += (int64_t)r * a.ostride[d];
     }
     const V* row = reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.in) + base);
-    const int64_t nv = a.k / VEC;
+    const int64_t nv = len / VEC;
     int64_t i = lane;
     for (; i + TPR < nv; i += 2 * TPR) {
       const V x0 = nt_load(row + i), x1 = nt_load(row + i + TPR);
@@ -212,8 +242,62 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
       for (int w = 1; w < kBlock / 64; ++w) acc = P::combine(acc, lds[w]);
     }
   }
-  if (live && lane == 0)
-    reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+  if (live && lane == 0) {
+    if (a.n_split == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+    else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc;
+  }
+}
+
+// Rows of at most L * TPR vectors (L <= 4, TPR <= 64): a group of TPR lanes
+// inside one wave takes U = 4 / L rows, issues all of its loads before the
+// first use, and combines with shuffles only (no LDS, no barrier).  For each
+// of the U passes the groups of a block take consecutive rows, so one load
+// instruction of a wave covers consecutive rows.
+template <class P, int VEC, int TPR, int L>
+__global__ void __launch_bounds__(kBlock) reduce_row_small_kernel(const RowArgs a, const typename P::Alpha alpha) {
+  using T = typename P::Elem;
+  using A = typename P::Acc;
+  using V = Vec<T, VEC>;
+  constexpr int U = 4 / L;
+  constexpr int GPB = kBlock / TPR;
+  const int lane = threadIdx.x % TPR;
+  const int64_t p0 = (int64_t)blockIdx.x * (GPB * U) + threadIdx.x / TPR;
+  const int nv = (int)(a.k / VEC);
+  V x[U][L];
+#pragma unroll
+  for (int r = 0; r < U; ++r) {
+    const int64_t p = p0 + r * GPB;
+    if (p < a.n_out) {
+      int64_t base = 0;
+      uint32_t rem = (uint32_t)p;
+      for (int d = 0; d < a.n_outer; ++d) {
+        uint32_t q, m;
+        a.osize[d].divmod(rem, q, m);
+        rem = q;
+        base += (int64_t)m * a.ostride[d];
+      }
+      const V* row = reinterpret_cast<const V*>(reinterpret_cast<const T*>(a.in) + base);
+#pragma unroll
+      for (int j = 0; j < L; ++j)
+        if (lane + j * TPR < nv) x[r][j] = nt_load(row + lane + j * TPR);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < U; ++r) {
+    const int64_t p = p0 + r * GPB;
+    A acc = P::identity();
+    if (p < a.n_out) {
+#pragma unroll
+      for (int j = 0; j < L; ++j)
+        if (lane + j * TPR < nv) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc = P::combine(acc, P::value(x[r][j].v[e], alpha));
+        }
+    }
+#pragma unroll
+    for (int m = TPR / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
+    if (p < a.n_out && lane == 0) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+  }
 }
 
 struct ColArgs {
@@ -236,6 +320,7 @@ struct ColArgs {
 // rows are in flight per block, 8 loads per lane.  Measured best among 1-16
 // waves and 32-512 rows per block for a [16384, 4096] float input.
 constexpr int kColBlock = 1024;
+constexpr int64_t kRowSplitBytes = 16384;  // smallest chunk a split row is cut into
 
 template <class P, int VEC>
 __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, const typename P::Alpha alpha) {
@@ -302,16 +387,31 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
   }
 }
 
-template <class P>
-__global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const ColArgs a) {
+// LPO lanes share one output's partials (64 when there are many segments).
+template <class P, int LPO>
+__global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs a) {
   using T = typename P::Elem;
   using A = typename P::Acc;
-  const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (p >= a.n_out) return;
+  const int lane = threadIdx.x % LPO;
+  const int64_t p = (int64_t)blockIdx.x * (kBlock / LPO) + threadIdx.x / LPO;
+  const bool live = p < a.n_out;
   const A* part = reinterpret_cast<const A*>(a.partials);
-  A acc = part[p];
-  for (uint32_t s = 1; s < a.n_seg; ++s) acc = P::combine(acc, part[(int64_t)s * a.n_out + p]);
-  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+  A acc = P::identity();
+  if (live)
+    for (uint32_t s = lane; s < a.n_seg; s += LPO) acc = P::combine(acc, part[(int64_t)s * a.n_out + p]);
+#pragma unroll
+  for (int m = LPO / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
+  if (live && lane == 0) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+}
+
+template <class P>
+void launch_finish(hipStream_t st, const FinishArgs& f) {
+  if (f.n_seg >= 32)
+    hipLaunchKernelGGL((reduce_finish_kernel<P, 64>), dim3((uint32_t)((f.n_out + kBlock / 64 - 1) / (kBlock / 64))),
+                       dim3(kBlock), 0, st, f);
+  else
+    hipLaunchKernelGGL((reduce_finish_kernel<P, 1>), dim3((uint32_t)((f.n_out + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       st, f);
 }
 
 struct AnyArgs {
@@ -416,21 +516,59 @@ int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, con
       a.ostride[d] = rs.kstride[src];
       if (rs.kstride[src] % VMAX != 0) vec_ok = false;
     }
-    const int64_t row_bytes = k * (int64_t)sizeof(T);
+    // too few rows for the chip and long ones: cut each row into chunks of at
+    // least 16 KiB until about 4096 lane groups exist
+    int64_t split = 1, chunk = k;
+    if (n_out < 2048 && k * (int64_t)sizeof(T) >= 2 * kRowSplitBytes) {
+      const int64_t quantum = kRowSplitBytes / (int64_t)sizeof(T);
+      const int64_t want = (4096 + n_out - 1) / n_out;
+      chunk = std::max<int64_t>(quantum, ((k + want - 1) / want + quantum - 1) / quantum * quantum);
+      split = (k + chunk - 1) / chunk;
+      if (split <= 1) { split = 1; chunk = k; }
+    }
+    a.chunk = chunk;
+    a.n_split = (uint32_t)split;
+    a.split_fd = FastDiv((uint32_t)split);
+    if (split > 1) {
+      if (int rc = stream_scratch(st, (size_t)(split * n_out) * sizeof(A), &a.partials)) return rc;
+    }
+    const int64_t n_groups = n_out * split;
+    const int64_t row_bytes = chunk * (int64_t)sizeof(T);
 #define CT_ROW(VEC, TPR)                                                                                        \
-  hipLaunchKernelGGL((reduce_row_kernel<P, VEC, TPR>), dim3((uint32_t)((n_out + (kBlock / TPR) - 1) / (kBlock / TPR))), \
+  hipLaunchKernelGGL((reduce_row_kernel<P, VEC, TPR>), dim3((uint32_t)((n_groups + (kBlock / TPR) - 1) / (kBlock / TPR))), \
                      dim3(kBlock), 0, st, a, alpha)
-    if (row_bytes >= 4096) {
+#define CT_ROW_SMALL(VEC, TPR, L)                                                                                   \
+  hipLaunchKernelGGL((reduce_row_small_kernel<P, VEC, TPR, L>),                                                     \
+                     dim3((uint32_t)((n_out + (kBlock / TPR) * (4 / L) - 1) / ((kBlock / TPR) * (4 / L)))),          \
+                     dim3(kBlock), 0, st, a, alpha)
+#define CT_ROW_SMALL_SHAPES(VEC)                  \
+  if (nv <= 1) CT_ROW_SMALL(VEC, 1, 1);           \
+  else if (nv <= 2) CT_ROW_SMALL(VEC, 2, 1);      \
+  else if (nv <= 4) CT_ROW_SMALL(VEC, 4, 1);      \
+  else if (nv <= 8) CT_ROW_SMALL(VEC, 8, 1);      \
+  else if (nv <= 16) CT_ROW_SMALL(VEC, 16, 1);    \
+  else if (nv <= 32) CT_ROW_SMALL(VEC, 16, 2);    \
+  else if (nv <= 64) CT_ROW_SMALL(VEC, 16, 4);    \
+  else if (nv <= 128) CT_ROW_SMALL(VEC, 64, 2);   \
+  else CT_ROW_SMALL(VEC, 64, 4)
+    const int64_t nv = vec_ok ? k / VMAX : k;
+    if (split == 1 && nv <= 256) {
+      note_kernel(vec_ok ? "reduce_row_small_vec" : "reduce_row_small");
+      if (vec_ok) { CT_ROW_SMALL_SHAPES(VMAX); } else { CT_ROW_SMALL_SHAPES(1); }
+    } else if (row_bytes >= 4096) {
       note_kernel(vec_ok ? "reduce_row256_vec" : "reduce_row256");
       if (vec_ok) CT_ROW(VMAX, 256); else CT_ROW(1, 256);
-    } else if (row_bytes >= 512) {
-      note_kernel(vec_ok ? "reduce_row64_vec" : "reduce_row64");
-      if (vec_ok) CT_ROW(VMAX, 64); else CT_ROW(1, 64);
     } else {
-      note_kernel("reduce_row16");
-      CT_ROW(1, 16);
+      note_kernel("reduce_row64");
+      CT_ROW(1, 64);
     }
+#undef CT_ROW_SMALL_SHAPES
+#undef CT_ROW_SMALL
 #undef CT_ROW
+    if (split > 1) {
+      const FinishArgs f{a.partials, out, k, n_out, (uint32_t)split, oa};
+      launch_finish<P>(st, f);
+    }
     return after_launch(st);
   }
 
@@ -481,9 +619,10 @@ int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, con
       note_kernel(vec_ok ? "reduce_col_vec" : "reduce_col");
       if (vec_ok) hipLaunchKernelGGL((reduce_col_kernel<P, VMAX>), dim3((uint32_t)grid), dim3(kColBlock), 0, st, a, alpha);
       else hipLaunchKernelGGL((reduce_col_kernel<P, 1>), dim3((uint32_t)grid), dim3(kColBlock), 0, st, a, alpha);
-      if (seg > 1)
-        hipLaunchKernelGGL((reduce_finish_kernel<P>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock),
-                           0, st, a);
+      if (seg > 1) {
+        const FinishArgs f{a.partials, out, k, n_out, (uint32_t)seg, oa};
+        launch_finish<P>(st, f);
+      }
       return after_launch(st);
     }
   }

@@ -323,11 +323,46 @@ def test_binary_accum_large_sum_uses_double_accumulation(P):
     y = P.buf(rng.random(n * c * hw).astype(np.float32))
     d = P.buf(np.zeros(c, np.float32))
     k = P.run(H.binary_accum, View(d, [c, 1, 1]), 1.0, View(y, [n, c, 32, 32]), 1.0, "+", requires_cas=True)
-    assert k == "accum_sum"
+    assert k == "accum_staged_sum"
     exact = y.init.astype(np.float64).reshape(n, c, hw).sum(axis=(0, 2))
     got = d.download().astype(np.float64)
-    assert np.all(np.abs(got - exact) <= 1e-6 * exact)              # ours: one rounding
+    assert np.all(np.abs(got - exact) <= 1e-6 * exact)              # ours: sums formed in double
     assert np.all(np.abs(d.host - exact) <= 1e-4 * exact)           # the serial float sum drifts
+
+
+# (dest shape, dest strides, y shape, y strides): every layout takes the staged-sum route
+STAGED_LAYOUTS = [
+    ([96], None, [400, 96], None),                       # sum the rows into a vector
+    ([300, 1], None, [300, 130], None),                  # sum each row
+    ([6, 1, 1], None, [8, 6, 24, 24], None),             # per-channel bias gradient: two passes
+    ([1], None, [40000], None),                          # everything into one element
+    ([50], [3], [700, 50], [64, 1]),                     # strided destination, padded rows
+    ([33, 1], None, [33, 900], [1, 33]),                 # y is a transposed view
+    ([4, 1, 5], None, [4, 1000, 5], None),               # reduced axis in the middle
+]
+
+
+@pytest.mark.parametrize("code", [capi.F32, capi.F64, capi.I32, capi.I64, capi.I16, capi.I8, capi.U8])
+def test_binary_accum_staged_sum(P, code):
+    rng = np.random.default_rng(81)
+    for dshape, dstrides, yshape, ystrides in STAGED_LAYOUTS:
+        y_elems = 1 + sum((s - 1) * st for s, st in zip(yshape, ystrides)) if ystrides else int(np.prod(yshape))
+        d_elems = 1 + sum((s - 1) * st for s, st in zip(dshape, dstrides)) if dstrides else int(np.prod(dshape))
+        if code in FLOATS:
+            yv, dv = (rng.random(y_elems) + 0.5).astype(NP[code]), rng.random(d_elems).astype(NP[code])
+        else:
+            yv, dv = values(rng, code, y_elems, -100, 100), values(rng, code, d_elems, -100, 100)
+        y, d = P.buf(yv), P.buf(dv)
+        for ya, rev in ((1.0, False), (3.0, True)):
+            k = P.run(H.binary_accum, View(d, dshape, dstrides), 1.0, View(y, yshape, ystrides), ya, "+", reverse=rev,
+                      requires_cas=True)
+            assert k == "accum_staged_sum", (k, dshape, yshape)
+            what = f"staged accum {dshape}<-{yshape} ya={ya}"
+            if code in FLOATS:
+                compare(d, what, tol=1e-4 if code == capi.F32 else 1e-12)
+            else:
+                compare(d, what)                              # integer sums wrap identically
+            d.reset()
 
 
 @pytest.mark.parametrize("code", [capi.F32, capi.I32, capi.F64, capi.I16])
@@ -356,7 +391,9 @@ def reduce_scale(x64, axis, op, alpha):
 
 
 @pytest.mark.parametrize("code", H.ALL_DTYPES)
-@pytest.mark.parametrize("shape", [(5, 10), (33, 64), (17, 257), (9, 2048), (300, 16), (2, 3, 40)], ids=str)
+@pytest.mark.parametrize("shape", [(5, 10), (33, 64), (17, 257), (9, 2048), (300, 16), (2, 3, 40), (3, 40000), (1, 100003),
+                                   (40, 4), (1000, 8), (21, 32), (19, 100), (13, 200), (11, 500), (7, 1000)],
+                         ids=str)
 def test_reduce_last_axis_and_transposed(P, code, shape):
     rng = np.random.default_rng(9)
     n = int(np.prod(shape))
@@ -397,8 +434,9 @@ def test_reduce_kernel_selection(P):
     x = P.buf(rng.standard_normal(64 * 4096).astype(np.float32))
     out = P.buf(np.zeros(4096, np.float32))
     assert P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 4096]), "sum") == "reduce_row256_vec"
-    assert P.run(H.unary_reduce, View(out, [1024, 1]), 1.0, View(x, [1024, 256]), "sum") == "reduce_row64_vec"
-    assert P.run(H.unary_reduce, View(out, [4096, 1]), 1.0, View(x, [4096, 64]), "sum") == "reduce_row16"
+    assert P.run(H.unary_reduce, View(out, [1024, 1]), 1.0, View(x, [1024, 256]), "sum") == "reduce_row_small_vec"
+    assert P.run(H.unary_reduce, View(out, [4096, 1]), 1.0, View(x, [4096, 63]), "sum") == "reduce_row_small"
+    compare(out, "unaligned short rows", tol=2e-6)
     assert P.run(H.unary_reduce, View(out, [4096, 1]), 1.0, View(x, [64, 4096]).transpose([1, 0]), "sum") == "reduce_col_vec"
     idx = P.buf(np.arange(63, -1, -1).astype(np.int32))
     k = P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 64], [4096, 1], index=[idx, None]), "max")
