@@ -364,10 +364,17 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
     }
-    for (; r < r1; r += WAVES, p += step) {
-      const V x0 = nt_load(reinterpret_cast<const V*>(p));
+    if (r < r1) {  // the last, partial batch: same depth, rows past the end skipped
+      V x[UN];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x0.v[e], alpha));
+      for (int j = 0; j < UN; ++j)
+        if (r + j * WAVES < r1) x[j] = nt_load(reinterpret_cast<const V*>(p + j * step));
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        if (r + j * WAVES < r1) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
+        }
     }
   }
   if (wave > 0) {
@@ -398,6 +405,7 @@ __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs 
   const A* part = reinterpret_cast<const A*>(a.partials);
   A acc = P::identity();
   if (live)
+#pragma unroll 8
     for (uint32_t s = lane; s < a.n_seg; s += LPO) acc = P::combine(acc, part[(int64_t)s * a.n_out + p]);
 #pragma unroll
   for (int m = LPO / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
@@ -406,7 +414,7 @@ __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs 
 
 template <class P>
 void launch_finish(hipStream_t st, const FinishArgs& f) {
-  if (f.n_seg >= 32)
+  if (f.n_seg >= 64 || (f.n_seg >= 8 && f.n_out <= 256))
     hipLaunchKernelGGL((reduce_finish_kernel<P, 64>), dim3((uint32_t)((f.n_out + kBlock / 64 - 1) / (kBlock / 64))),
                        dim3(kBlock), 0, st, f);
   else
@@ -600,10 +608,12 @@ int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, con
     const int vec = vec_ok ? VMAX : 1;
     a.n_strips = (a.u + 64 * vec - 1) / (64 * vec);
     const int64_t base_blocks = (int64_t)a.n_strips * rest_count;
-    // 256 rows per block when that still leaves >= 1024 blocks, fewer rows otherwise
-    // (never below one row per wave); partials capped at 16 MiB
-    int64_t rows = 256;
-    while (rows > 16 && base_blocks * ((k + rows - 1) / rows) < 1024) rows /= 2;
+    // Rows are cut into segments until about two blocks per compute unit exist
+    // (one round of resident blocks measured better than several shorter ones);
+    // a segment is a whole number of load batches; partials capped at 16 MiB.
+    constexpr int64_t kRowQuantum = 128;  // 16 waves x 8 loads in flight
+    const int64_t want_seg = std::max<int64_t>(1, std::min<int64_t>(512 / base_blocks, k / kRowQuantum));
+    int64_t rows = ((k + want_seg - 1) / want_seg + kRowQuantum - 1) / kRowQuantum * kRowQuantum;
     const int64_t seg_cap = std::max<int64_t>(1, (int64_t(16) << 20) / (n_out * (int64_t)sizeof(A)));
     if ((k + rows - 1) / rows > seg_cap) rows = (k + seg_cap - 1) / seg_cap;
     int64_t seg = (k + rows - 1) / rows;
