@@ -169,20 +169,25 @@ template <class F> struct elem_sizes {
   static constexpr size_t max_in = m012;
   static constexpr size_t max_all = m012 > sizeof(typename F::Out) ? m012 : sizeof(typename F::Out);
 };
-// Tile edge: 64 elements for input types up to 4 bytes, 32 for 8-byte types,
-// so one tile row is at most a 256-byte contiguous segment.
-template <class F> struct tile_edge {
-  static constexpr int value = elem_sizes<F>::max_in > 4 ? 32 : 64;
+// Tile shape: kTileA elements along A (the destination's unit-stride axis) by
+// tile_b<F> elements along B (the axis the transposed inputs are unit-stride
+// along).  The read side matters most: 512-byte source segments measured
+// 83 % of peak on a transposing float copy against 76 % for 256-byte ones, while
+// shrinking the written segments from 256 to 128 bytes cost about 1 %.
+constexpr int kTileA = 32;
+template <class F> struct tile_b {
+  static constexpr int value = elem_sizes<F>::max_in > 4 ? 64 : 128;
 };
-constexpr size_t tile_slot_bytes(size_t elem, int ts) { return ((elem * ts * (ts + 1)) + 15) & ~size_t(15); }
+constexpr size_t tile_slot_bytes(size_t elem, int tb) { return ((elem * kTileA * (tb + 1)) + 15) & ~size_t(15); }
 
-// Reads this lane's share of a TS x TS tile of an operand that is unit-stride
-// along B: lane tx walks B (a 256-byte coalesced row segment per wave), the
-// block's ROWS wave-rows walk A.  The pointer advances by a constant step.
-template <class T, int TS, bool FULL, bool STREAM>
+// Reads this lane's share of a kTileA x TB tile of an operand that is
+// unit-stride along B: lane tx walks B (TB consecutive elements per source
+// row), the block's ROWS lane rows walk A.  The pointer advances by a constant
+// step.
+template <class T, int TB, bool FULL, bool STREAM>
 __device__ __forceinline__ void tile_read(T* v, const T* p, int64_t step, uint32_t a_left, bool b_ok, int ty) {
-  constexpr int ROWS = kBlock / TS;
-  constexpr int IT = TS / ROWS;
+  constexpr int ROWS = kBlock / TB;
+  constexpr int IT = kTileA / ROWS;
 #pragma unroll
   for (int i = 0; i < IT; ++i) {
     if (FULL || (b_ok && (uint32_t)(ty + i * ROWS) < a_left)) {
@@ -194,20 +199,24 @@ __device__ __forceinline__ void tile_read(T* v, const T* p, int64_t step, uint32
   }
 }
 
-// Transposes the lane values through the block's single LDS tile (padded to
-// TS + 1 columns: conflict-free both ways): v[i] holds element (a = ty + i*ROWS,
-// b = tx) on entry and element (a = tx, b = ty + i*ROWS) on exit.
-template <class T, int TS>
-__device__ __forceinline__ void tile_transpose(T* v, char* smem, int tx, int ty, bool need_sync_before) {
-  constexpr int ROWS = kBlock / TS;
-  constexpr int IT = TS / ROWS;
+// Transposes the lane values through the block's single LDS tile (rows padded
+// to TB + 1 elements: conflict-free both ways).  On entry v[i] holds element
+// (a = ty + i*ROWS_R, b = tx) with tx = t % TB; on exit element
+// (a = wx, b = wy + i*ROWS_W) with wx = t % kTileA.
+template <class T, int TB>
+__device__ __forceinline__ void tile_transpose(T* v, char* smem, bool need_sync_before) {
+  constexpr int ROWS_R = kBlock / TB, ROWS_W = kBlock / kTileA;
+  constexpr int IT = kTileA / ROWS_R;
+  static_assert(IT == TB / ROWS_W, "both phases move the same number of elements per lane");
+  const int tx = threadIdx.x % TB, ty = threadIdx.x / TB;
+  const int wx = threadIdx.x % kTileA, wy = threadIdx.x / kTileA;
   T* lds = reinterpret_cast<T*>(smem);
   if (need_sync_before) __syncthreads();
 #pragma unroll
-  for (int i = 0; i < IT; ++i) lds[(ty + i * ROWS) * (TS + 1) + tx] = v[i];
+  for (int i = 0; i < IT; ++i) lds[(ty + i * ROWS_R) * (TB + 1) + tx] = v[i];
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < IT; ++i) v[i] = lds[tx * (TS + 1) + ty + i * ROWS];
+  for (int i = 0; i < IT; ++i) v[i] = lds[wx * (TB + 1) + wy + i * ROWS_W];
 }
 
 template <class F, bool FULL, bool STREAM>
@@ -218,10 +227,11 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   using In1 = typename F::In1;
   using In2 = typename F::In2;
   constexpr int NIN = F::NIN;
-  constexpr int TS = tile_edge<F>::value;
-  constexpr int ROWS = kBlock / TS;
-  constexpr int IT = TS / ROWS;
-  const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
+  constexpr int TB = tile_b<F>::value;
+  constexpr int ROWS_R = kBlock / TB, ROWS_W = kBlock / kTileA;
+  constexpr int IT = kTileA / ROWS_R;
+  const int tx = threadIdx.x % TB, ty = threadIdx.x / TB;
+  const int wx = threadIdx.x % kTileA, wy = threadIdx.x / kTileA;
   const uint32_t a_left = a.sizeA - a0, b_left = a.sizeB - b0;  // valid extent of this tile
   const bool t0 = NIN >= 1 && ((a.lds_mask >> 1) & 1u), t1 = NIN >= 2 && ((a.lds_mask >> 2) & 1u),
              t2 = NIN >= 3 && ((a.lds_mask >> 3) & 1u);
@@ -232,23 +242,23 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   In2 v2[IT];
   const bool b_ok = (uint32_t)tx < b_left;
   if constexpr (NIN >= 1)
-    if (t0) tile_read<In0, TS, FULL, STREAM>(v0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
-                                     (int64_t)ROWS * a.strideA[1], a_left, b_ok, ty);
+    if (t0) tile_read<In0, TB, FULL, STREAM>(v0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
+                                     (int64_t)ROWS_R * a.strideA[1], a_left, b_ok, ty);
   if constexpr (NIN >= 2)
-    if (t1) tile_read<In1, TS, FULL, STREAM>(v1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
-                                     (int64_t)ROWS * a.strideA[2], a_left, b_ok, ty);
+    if (t1) tile_read<In1, TB, FULL, STREAM>(v1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
+                                     (int64_t)ROWS_R * a.strideA[2], a_left, b_ok, ty);
   if constexpr (NIN >= 3)
-    if (t2) tile_read<In2, TS, FULL, STREAM>(v2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
-                                     (int64_t)ROWS * a.strideA[3], a_left, b_ok, ty);
+    if (t2) tile_read<In2, TB, FULL, STREAM>(v2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
+                                     (int64_t)ROWS_R * a.strideA[3], a_left, b_ok, ty);
   bool used = false;
-  if constexpr (NIN >= 1) if (t0) { tile_transpose<In0, TS>(v0, smem, tx, ty, used); used = true; }
-  if constexpr (NIN >= 2) if (t1) { tile_transpose<In1, TS>(v1, smem, tx, ty, used); used = true; }
-  if constexpr (NIN >= 3) if (t2) { tile_transpose<In2, TS>(v2, smem, tx, ty, used); used = true; }
+  if constexpr (NIN >= 1) if (t0) { tile_transpose<In0, TB>(v0, smem, used); used = true; }
+  if constexpr (NIN >= 2) if (t1) { tile_transpose<In1, TB>(v1, smem, used); used = true; }
+  if constexpr (NIN >= 3) if (t2) { tile_transpose<In2, TB>(v2, smem, used); used = true; }
 
-  // phase 2: lane tx walks A (the destination's unit-stride axis), rows walk B
-  const bool a_ok = (uint32_t)tx < a_left;
-  Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + off[0] + (int64_t)(a0 + tx) * a.strideA[0] + (int64_t)(b0 + ty) * a.strideB[0];
-  const int64_t dstep = (int64_t)ROWS * a.strideB[0];
+  // phase 2: lane wx walks A (the destination's unit-stride axis), lane rows walk B
+  const bool a_ok = (uint32_t)wx < a_left;
+  Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + off[0] + (int64_t)(a0 + wx) * a.strideA[0] + (int64_t)(b0 + wy) * a.strideB[0];
+  const int64_t dstep = (int64_t)ROWS_W * a.strideB[0];
   const In0* q0 = nullptr;
   const In1* q1 = nullptr;
   const In2* q2 = nullptr;
@@ -258,19 +268,19 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   In2 c2{};
   if constexpr (NIN >= 1) {
     if ((a.const_mask >> 1) & 1u) c0 = const_from_bits<In0>(a.cbits[1]);
-    else if (!t0) { q0 = reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + tx) * a.strideA[1] + (int64_t)(b0 + ty) * a.strideB[1]; s0 = (int64_t)ROWS * a.strideB[1]; }
+    else if (!t0) { q0 = reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + wx) * a.strideA[1] + (int64_t)(b0 + wy) * a.strideB[1]; s0 = (int64_t)ROWS_W * a.strideB[1]; }
   }
   if constexpr (NIN >= 2) {
     if ((a.const_mask >> 2) & 1u) c1 = const_from_bits<In1>(a.cbits[2]);
-    else if (!t1) { q1 = reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + tx) * a.strideA[2] + (int64_t)(b0 + ty) * a.strideB[2]; s1 = (int64_t)ROWS * a.strideB[2]; }
+    else if (!t1) { q1 = reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + wx) * a.strideA[2] + (int64_t)(b0 + wy) * a.strideB[2]; s1 = (int64_t)ROWS_W * a.strideB[2]; }
   }
   if constexpr (NIN >= 3) {
     if ((a.const_mask >> 3) & 1u) c2 = const_from_bits<In2>(a.cbits[3]);
-    else if (!t2) { q2 = reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + tx) * a.strideA[3] + (int64_t)(b0 + ty) * a.strideB[3]; s2 = (int64_t)ROWS * a.strideB[3]; }
+    else if (!t2) { q2 = reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + wx) * a.strideA[3] + (int64_t)(b0 + wy) * a.strideB[3]; s2 = (int64_t)ROWS_W * a.strideB[3]; }
   }
 #pragma unroll
   for (int i = 0; i < IT; ++i) {
-    const int row = ty + i * ROWS;
+    const int row = wy + i * ROWS_W;
     if (FULL || (a_ok && (uint32_t)row < b_left)) {
       In0 p0 = c0;
       In1 p1 = c1;
@@ -284,19 +294,19 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   }
 }
 
-// One block per TS x TS tile.  All transposed operands share one LDS tile,
+// One block per kTileA x TB tile.  All transposed operands share one LDS tile,
 // used in turn, so the LDS footprint (and with it the number of resident
 // blocks) does not grow with the operand count.
 template <class F, bool STREAM>
 __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileArgs a) {
   constexpr int NIN = F::NIN;
-  constexpr int TS = tile_edge<F>::value;
+  constexpr int TB = tile_b<F>::value;
   extern __shared__ __align__(16) char smem[];
 
   uint32_t bid, tb, ta, q0;
-  // tiles along B vary fastest: consecutive blocks read neighbouring 256-byte
-  // segments of the same source rows (measured 71 % of peak against 58 % with
-  // tiles along A fastest on a transposed [8192,8192] float input)
+  // tiles along B vary fastest: consecutive blocks read neighbouring segments
+  // of the same source rows (measured 71 % of peak against 58 % with tiles
+  // along A fastest on a transposed [8192,8192] float input)
   a.tilesB_fd.divmod(blockIdx.x, q0, tb);
   a.tilesA_fd.divmod(q0, bid, ta);
   int64_t off[kMaxOps] = {0, 0, 0, 0};
@@ -307,8 +317,8 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
 #pragma unroll
     for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
   }
-  const uint32_t a0 = ta * TS, b0 = tb * TS;
-  if (a0 + TS <= a.sizeA && b0 + TS <= a.sizeB) tile_body<F, true, STREAM>(f, a, off, a0, b0, smem);
+  const uint32_t a0 = ta * kTileA, b0 = tb * TB;
+  if (a0 + kTileA <= a.sizeA && b0 + TB <= a.sizeB) tile_body<F, true, STREAM>(f, a, off, a0, b0, smem);
   else tile_body<F, false, STREAM>(f, a, off, a0, b0, smem);
 }
 
@@ -440,7 +450,7 @@ struct EwOperand {
 
 int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_args, int* main_vec,
                 VecArgs* tail_args, bool* has_tail);
-int prepare_tile(const Plan& plan, const EwOperand* ops, int ts, TileArgs* args, size_t* lds_bytes,
+int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_b_edge, TileArgs* args, size_t* lds_bytes,
                  uint32_t* grid);
 int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use64, uint32_t* grid);
 
@@ -483,7 +493,7 @@ int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t 
     TileArgs ta;
     size_t lds = 0;
     uint32_t grid = 0;
-    if (int rc = prepare_tile(plan, ops, tile_edge<F>::value, &ta, &lds, &grid)) return rc;
+    if (int rc = prepare_tile(plan, ops, tile_b<F>::value, &ta, &lds, &grid)) return rc;
     note_kernel("tile");
     if (ta.streaming) hipLaunchKernelGGL((ew_tile_kernel<F, true>), dim3(grid), dim3(kBlock), lds, s, f, ta);
     else hipLaunchKernelGGL((ew_tile_kernel<F, false>), dim3(grid), dim3(kBlock), lds, s, f, ta);
