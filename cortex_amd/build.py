@@ -28,6 +28,7 @@ SOURCES = [
     "ops_accum.hip",
     "ops_reduce.hip",
     "ops_optim.hip",
+    "ops_nn.hip",
 ]
 
 # -ffp-contract=off: the reference's CPU backend rounds after every JVM

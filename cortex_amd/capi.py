@@ -29,6 +29,7 @@ UNARY_OPS = {"floor": 0, "ceil": 1, "round": 2, "-": 3, "tanh": 4, "logistic": 5
 BINARY_OPS = {"+": 0, "-": 1, "*": 2, "/": 3, "min": 4, "max": 5, "bit-and": 6, "bit-xor": 7, "eq": 8,
               ">": 9, ">=": 10, "<": 11, "<=": 12}
 TERNARY_OPS = {"select": 0}
+ACTIVATION_OPS = {"logistic": 0, "tanh": 1, "relu": 2}
 REDUCE_OPS = {"max": 0, "min": 1, "sum": 2, "mean": 3, "magnitude": 4, "magnitude-squared": 5}
 
 COPY_H2D, COPY_D2H, COPY_D2D = 0, 1, 2
@@ -107,6 +108,9 @@ PROTOTYPES = {
     "ct_ternary_op_constant": [_P, _P, _DP, _P, _DP, _D, _P, _DP, _D, _D, _L, _I, C.POINTER(C.c_int8), _I],
     "ct_ternary_op_constant_constant": [_P, _P, _DP, _P, _DP, _D, _D, _D, _L, _I, C.POINTER(C.c_int8), _I],
     "ct_unary_reduce": [_P, _P, _DP, _D, _P, _DP, _I, _I],
+    "ct_activation_gradient": [_P, _P, _DP, _P, _DP, _P, _DP, _I, _L, _I],
+    "ct_softmax_eltwise": [_P, _P, _DP, _P, _DP, _I],
+    "ct_softmax_spatial": [_P, _P, _DP, _P, _DP, _I],
     "ct_adam_step": [_P, _I, _D, _D, _D, _D, _D, _D, _D, _P, _P, _P, _P, _L],
     "ct_adadelta_step": [_P, _I, _D, _D, _P, _P, _D, _P, _P, _L],
 }

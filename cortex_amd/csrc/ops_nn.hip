@@ -1,0 +1,283 @@
+// ops_nn.hip -- activation-gradient!, softmax-eltwise!, softmax-spatial!
+// (src/cortex/tensor/math.clj:176-189;
+//  src/cortex/compute/cpu/tensor_math.clj:1037-1103, 1318-1362).
+//
+// activation-gradient! is one more elementwise functor over the shared
+// launcher, so it accepts every access pattern the other elementwise ops do.
+//
+// softmax works on rows of k elements laid out as [outer, rows, k] with
+// arbitrary (direct) strides per operand; the spatial form is the same thing
+// with the channel axis taken as k.  Per row, as the CPU backend does it:
+//   m   = max(x)                       (java.lang.Math.max: NaN propagates)
+//   e_i = T(exp(double(x_i) - double(m)))
+//   s   = T(sum of double(e_i))
+//   y_i = e_i / s                      (a division in T)
+// Two kernels cover the layouts:
+//   softmax_wave_kernel  a group of 16 or 64 lanes owns a row and walks k
+//                        (coalesced when k is the unit-stride axis); rows of up
+//                        to 16 elements per lane stay in registers, longer
+//                        rows are re-read from cache
+//   softmax_lane_kernel  one lane owns a row and walks k sequentially, the
+//                        lanes of a wave take neighbouring rows (coalesced when
+//                        the row axis is unit-stride: the spatial form, where
+//                        k is the channel axis).  Its sum runs in the
+//                        reference's own order.
+// The reference's maximum loop reads elements 1..k-1 of the input through the
+// output's address object (cpu/tensor_math.clj:1067-1072); that only matters
+// when the two layouts differ, and then only through rounding, because the
+// result of a softmax does not depend on the value subtracted.  The kernels
+// take the true row maximum.
+#include <algorithm>
+
+#include "elementwise.h"
+#include "functors.h"
+
+using namespace cthip;
+
+namespace {
+
+// act-backward-impl (cpu/tensor_math.clj:1318-1362): operands widen to double,
+// the products run left to right, the store rounds once.
+template <class T, int OP> struct ActGradF {
+  static constexpr int NIN = 2;
+  using Out = T;
+  using In0 = T;  // output
+  using In1 = T;  // output gradient
+  using In2 = T;
+  __device__ __forceinline__ T operator()(T out, T grad, T) const {
+    const double o = (double)out, g = (double)grad;
+    if constexpr (OP == CT_ACT_LOGISTIC) return (T)((o * (1.0 - o)) * g);
+    else if constexpr (OP == CT_ACT_TANH) return (T)((1.0 - o * o) * g);
+    else return (T)((o > 0.0 ? 1.0 : 0.0) * g);
+  }
+};
+
+template <class T, int OP>
+int act_grad_run(hipStream_t s, void* ig, const ct_dims* igd, const void* og, const ct_dims* ogd, const void* out,
+                 const ct_dims* od, int64_t n) {
+  ActGradF<T, OP> f;
+  EwOperand ops[3] = {{ig, igd, (int)sizeof(T), 0}, {out, od, (int)sizeof(T), 0}, {og, ogd, (int)sizeof(T), 0}};
+  return launch_elementwise(s, f, ops, n);
+}
+
+template <class T>
+int act_grad_typed(hipStream_t s, void* ig, const ct_dims* igd, const void* og, const ct_dims* ogd, const void* out,
+                   const ct_dims* od, int op, int64_t n) {
+  switch (op) {
+    case CT_ACT_LOGISTIC: return act_grad_run<T, CT_ACT_LOGISTIC>(s, ig, igd, og, ogd, out, od, n);
+    case CT_ACT_TANH: return act_grad_run<T, CT_ACT_TANH>(s, ig, igd, og, ogd, out, od, n);
+    case CT_ACT_RELU: return act_grad_run<T, CT_ACT_RELU>(s, ig, igd, og, ogd, out, od, n);
+    default: return set_error(CT_ERR_INVALID, "Only :logistic :tanh and :relu are supported (got %d)", op);
+  }
+}
+
+// ------------------------------------------------------------------ softmax
+
+// java.lang.Math.max on the tensor's own type.
+template <class T> __device__ __forceinline__ T jvm_max(T a, T b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  if (a == (T)0 && b == (T)0) return __builtin_signbit(a) ? b : a;
+  return a > b ? a : b;
+}
+
+// T(exp(double(x) - double(m))).  For float the exact double difference is split
+// into a float head and tail: exp(h + t) = exp(h) * (1 + t) to well below half an
+// ulp, and expf is accurate to about an ulp; a plain float subtraction would
+// lose up to |x - m| * 2^-24 relative (3e-6 at a difference of 50).
+template <class T> __device__ __forceinline__ T shifted_exp(T x, T m) {
+  const double d = (double)x - (double)m;
+  if constexpr (std::is_same<T, float>::value) {
+    const float h = (float)d;
+    const float t = (float)(d - (double)h);
+    const float e = expf(h);
+    return e + e * t;
+  } else {
+    return exp(d);
+  }
+}
+
+struct SoftmaxArgs {
+  const void* in;
+  void* out;
+  int64_t n_rows;        // outer * rows
+  uint32_t k;
+  FastDiv rows_fd;       // rows per outer index
+  int64_t in_outer, in_row, in_k;
+  int64_t out_outer, out_row, out_k;
+};
+
+__device__ __forceinline__ void softmax_row_base(const SoftmaxArgs& a, int64_t r, int64_t* ib, int64_t* ob) {
+  uint32_t o, p;
+  a.rows_fd.divmod((uint32_t)r, o, p);
+  *ib = (int64_t)o * a.in_outer + (int64_t)p * a.in_row;
+  *ob = (int64_t)o * a.out_outer + (int64_t)p * a.out_row;
+}
+
+// TPR lanes per row.  ITER > 0: the row (k <= TPR * ITER) is held in registers.
+// ITER == 0: any k, the row is read three times.
+template <class T, int TPR, int ITER>
+__global__ void __launch_bounds__(kBlock) softmax_wave_kernel(const SoftmaxArgs a) {
+  const int lane = threadIdx.x % TPR;
+  const int64_t r = (int64_t)blockIdx.x * (kBlock / TPR) + threadIdx.x / TPR;
+  const bool live = r < a.n_rows;
+  int64_t ib = 0, ob = 0;
+  if (live) softmax_row_base(a, r, &ib, &ob);
+  const T* in = reinterpret_cast<const T*>(a.in) + ib;
+  T* out = reinterpret_cast<T*>(a.out) + ob;
+  constexpr int NX = ITER > 0 ? ITER : 1;
+  T x[NX];
+  // identity of Math.max that lets NaN through
+  T m = -__builtin_huge_valf();
+  if constexpr (ITER > 0) {
+#pragma unroll
+    for (int j = 0; j < ITER; ++j) {
+      const uint32_t i = lane + j * TPR;
+      if (live && i < a.k) { x[j] = in[(int64_t)i * a.in_k]; m = jvm_max(m, x[j]); }
+    }
+  } else {
+    if (live)
+      for (uint32_t i = lane; i < a.k; i += TPR) m = jvm_max(m, in[(int64_t)i * a.in_k]);
+  }
+#pragma unroll
+  for (int s = TPR / 2; s >= 1; s >>= 1) m = jvm_max(m, (T)__shfl_xor(m, s, 64));
+  double sum = 0.0;
+  if constexpr (ITER > 0) {
+#pragma unroll
+    for (int j = 0; j < ITER; ++j) {
+      const uint32_t i = lane + j * TPR;
+      if (live && i < a.k) { x[j] = shifted_exp(x[j], m); sum += (double)x[j]; }
+    }
+  } else {
+    if (live)
+      for (uint32_t i = lane; i < a.k; i += TPR) sum += (double)shifted_exp(in[(int64_t)i * a.in_k], m);
+  }
+#pragma unroll
+  for (int s = TPR / 2; s >= 1; s >>= 1) sum += __shfl_xor(sum, s, 64);
+  const T denom = (T)sum;
+  if constexpr (ITER > 0) {
+#pragma unroll
+    for (int j = 0; j < ITER; ++j) {
+      const uint32_t i = lane + j * TPR;
+      if (live && i < a.k) out[(int64_t)i * a.out_k] = x[j] / denom;
+    }
+  } else {
+    if (live)
+      for (uint32_t i = lane; i < a.k; i += TPR)
+        out[(int64_t)i * a.out_k] = shifted_exp(in[(int64_t)i * a.in_k], m) / denom;
+  }
+}
+
+// One lane per row; in place is fine (each pass reads x_i before y_i is written).
+template <class T>
+__global__ void __launch_bounds__(kBlock) softmax_lane_kernel(const SoftmaxArgs a) {
+  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= a.n_rows) return;
+  int64_t ib, ob;
+  softmax_row_base(a, r, &ib, &ob);
+  const T* in = reinterpret_cast<const T*>(a.in) + ib;
+  T* out = reinterpret_cast<T*>(a.out) + ob;
+  T m = in[0];
+  for (uint32_t i = 1; i < a.k; ++i) m = jvm_max(m, in[(int64_t)i * a.in_k]);
+  double sum = (double)shifted_exp(in[0], m);
+  for (uint32_t i = 1; i < a.k; ++i) sum += (double)shifted_exp(in[(int64_t)i * a.in_k], m);
+  const T denom = (T)sum;
+  for (uint32_t i = 0; i < a.k; ++i) out[(int64_t)i * a.out_k] = shifted_exp(in[(int64_t)i * a.in_k], m) / denom;
+}
+
+struct RowLayout { int64_t outer, rows, k, s_outer, s_row, s_k; };
+
+// [rows, k] or [outer, rows, k]; spatial swaps the last two axes (dimensions.clj:473-484 with [0 2 1]).
+int row_layout(const ct_dims* d, bool spatial, const char* what, RowLayout* l) {
+  if (int rc = check_dims(d, what)) return rc;
+  CT_REQUIRE(dims_direct(*d), "softmax!: %s must have direct dimensions", what);
+  CT_REQUIRE(d->ndim == 2 || d->ndim == 3, "softmax implementation only supports shapes of 2 or 3 dimensions");
+  CT_REQUIRE(!spatial || d->ndim == 3, "softmax-spatial! needs [batch channels elements]");
+  if (d->ndim == 2) {
+    *l = RowLayout{1, d->shape[0], d->shape[1], 0, d->strides[0], d->strides[1]};
+  } else if (!spatial) {
+    *l = RowLayout{d->shape[0], d->shape[1], d->shape[2], d->strides[0], d->strides[1], d->strides[2]};
+  } else {
+    *l = RowLayout{d->shape[0], d->shape[2], d->shape[1], d->strides[0], d->strides[2], d->strides[1]};
+  }
+  return CT_OK;
+}
+
+template <class T>
+int softmax_run(hipStream_t s, void* out, const RowLayout& ol, const void* in, const RowLayout& il) {
+  SoftmaxArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.in = in; a.out = out;
+  a.n_rows = il.outer * il.rows;
+  a.k = (uint32_t)il.k;
+  a.rows_fd = FastDiv((uint32_t)il.rows);
+  a.in_outer = il.s_outer; a.in_row = il.s_row; a.in_k = il.s_k;
+  a.out_outer = ol.s_outer; a.out_row = ol.s_row; a.out_k = ol.s_k;
+  if (a.n_rows == 0) return CT_OK;
+  // lanes along the row axis when that is the unit-stride one (spatial form) or the rows are tiny
+  const bool row_major = il.s_k == 1 || il.k == 1;
+  if (il.k < 8 || (!row_major && il.s_row == 1)) {
+    note_kernel("softmax_lane");
+    hipLaunchKernelGGL((softmax_lane_kernel<T>), dim3((uint32_t)((a.n_rows + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, a);
+    return after_launch(s);
+  }
+#define CT_SM(TPR, ITER)                                                                                         \
+  hipLaunchKernelGGL((softmax_wave_kernel<T, TPR, ITER>),                                                       \
+                     dim3((uint32_t)((a.n_rows + (kBlock / TPR) - 1) / (kBlock / TPR))), dim3(kBlock), 0, s, a)
+  note_kernel(il.k <= 1024 ? "softmax_wave" : "softmax_wave_loop");
+  if (il.k <= 16) CT_SM(16, 1);
+  else if (il.k <= 32) CT_SM(16, 2);
+  else if (il.k <= 64) CT_SM(16, 4);
+  else if (il.k <= 128) CT_SM(64, 2);
+  else if (il.k <= 256) CT_SM(64, 4);
+  else if (il.k <= 512) CT_SM(64, 8);
+  else if (il.k <= 1024) CT_SM(64, 16);
+  else CT_SM(64, 0);
+#undef CT_SM
+  return after_launch(s);
+}
+
+int softmax_entry(void* stream, void* output, const ct_dims* od, const void* input, const ct_dims* id, int dtype,
+                  bool spatial) {
+  CT_REQUIRE(output && input, "softmax!: null buffer");
+  RowLayout ol, il;
+  if (int rc = row_layout(od, spatial, "output", &ol)) return rc;
+  if (int rc = row_layout(id, spatial, "input", &il)) return rc;
+  CT_REQUIRE(ol.outer == il.outer && ol.rows == il.rows && ol.k == il.k, "Input, output shapes do not match");
+  CT_REQUIRE(il.outer * il.rows < (int64_t(1) << 31) && il.k < (int64_t(1) << 31), "softmax!: too many rows");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == CT_F32) return softmax_run<float>(s, output, ol, input, il);
+  if (dtype == CT_F64) return softmax_run<double>(s, output, ol, input, il);
+  return set_error(CT_ERR_INVALID, "softmax! is only defined for float and double tensors");
+}
+
+}  // namespace
+
+extern "C" {
+
+int ct_activation_gradient(void* stream, void* input_gradient, const ct_dims* input_gradient_dims,
+                           const void* output_gradient, const ct_dims* output_gradient_dims, const void* output,
+                           const ct_dims* output_dims, int op, int64_t n, int dtype) {
+  CT_REQUIRE(input_gradient && output_gradient && output, "ct_activation_gradient: null buffer");
+  CT_REQUIRE(n >= 0, "ct_activation_gradient: negative count");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == CT_F32)
+    return act_grad_typed<float>(s, input_gradient, input_gradient_dims, output_gradient, output_gradient_dims, output,
+                                 output_dims, op, n);
+  if (dtype == CT_F64)
+    return act_grad_typed<double>(s, input_gradient, input_gradient_dims, output_gradient, output_gradient_dims,
+                                  output, output_dims, op, n);
+  return set_error(CT_ERR_INVALID, "activation-gradient! is only defined for float and double tensors");
+}
+
+int ct_softmax_eltwise(void* stream, void* output, const ct_dims* output_dims, const void* input,
+                       const ct_dims* input_dims, int dtype) {
+  return softmax_entry(stream, output, output_dims, input, input_dims, dtype, false);
+}
+
+int ct_softmax_spatial(void* stream, void* output, const ct_dims* output_dims, const void* input,
+                       const ct_dims* input_dims, int dtype) {
+  return softmax_entry(stream, output, output_dims, input, input_dims, dtype, true);
+}
+
+}  // extern "C"

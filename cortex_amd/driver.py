@@ -282,6 +282,22 @@ class HipStream:
         capi.call("ct_unary_reduce", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), float(input_alpha),
                   input.ptr, C.byref(_dims_struct(input_dims)), capi.REDUCE_OPS[op], capi.DTYPE_CODES[output.datatype])
 
+    # -- neural-network tensor ops (tensor/math.clj:176-189) ------------------
+    def activation_gradient(self, input_gradient, input_grad_dims, output_gradient, output_grad_dims, output,
+                            output_dims, op, element_count) -> None:
+        capi.call("ct_activation_gradient", self.handle, input_gradient.ptr, C.byref(_dims_struct(input_grad_dims)),
+                  output_gradient.ptr, C.byref(_dims_struct(output_grad_dims)), output.ptr,
+                  C.byref(_dims_struct(output_dims)), capi.ACTIVATION_OPS[op], int(element_count),
+                  capi.DTYPE_CODES[input_gradient.datatype])
+
+    def softmax_eltwise(self, output, output_dims, input, input_dims) -> None:
+        capi.call("ct_softmax_eltwise", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), input.ptr,
+                  C.byref(_dims_struct(input_dims)), capi.DTYPE_CODES[output.datatype])
+
+    def softmax_spatial(self, output, output_dims, input, input_dims) -> None:
+        capi.call("ct_softmax_spatial", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), input.ptr,
+                  C.byref(_dims_struct(input_dims)), capi.DTYPE_CODES[output.datatype])
+
     # -- optimizers ---------------------------------------------------------
     def adam_step(self, alpha, beta1, beta2, epsilon, pow_beta1_t, pow_beta2_t, gradient_alpha, gradient, parameters,
                   m, v, n) -> None:

@@ -472,6 +472,47 @@ def unary_reduce(output: Tensor, alpha, input: Tensor, op: str) -> Tensor:
     return output
 
 
+# ---------------------------------------------------------------- activation-gradient!, softmax!
+
+def _external_library_check(method_name: str, *tensors) -> None:
+    """``external-library-check!`` (``tensor.clj:895-917``)."""
+    _ensure_datatypes(tensors[0].get_datatype(), *tensors[1:])
+    _ensure_same_device(*tensors)
+    if tensors[0].get_datatype() not in ("float", "double"):
+        raise TensorError(f"{method_name} is only defined for float and double tensors")
+    if not all(dims.access_increasing(t.dimensions) for t in tensors):
+        raise TensorError("External libraries (blas (gemm gemv) and cudnn require dimensions access to be increasing")
+
+
+def activation_gradient(input_gradient: Tensor, output_gradient: Tensor, output: Tensor, op: str) -> Tensor:
+    """``activation-gradient!`` (``tensor.clj:1256-1284``)."""
+    _external_library_check("activation-gradient!", input_gradient, output, output_gradient)
+    if op not in ("logistic", "tanh", "relu"):
+        raise TensorError("Only :logistic :tanh and :relu are supported")
+    n = ecount(output)
+    if n != ecount(input_gradient) or n != ecount(output_gradient):
+        raise TensorError("All element ecounts must match")
+    check_stream().activation_gradient(input_gradient.buffer, input_gradient.dimensions, output_gradient.buffer,
+                                       output_gradient.dimensions, output.buffer, output.dimensions, op, n)
+    return input_gradient
+
+
+def softmax(output: Tensor, input: Tensor) -> Tensor:
+    """``softmax!`` (``tensor.clj:1286-1312``): three dimensions mean
+    [batch channels elements] and a softmax across the channels; anything else
+    is squashed to [batch, n] and normalised along n."""
+    _external_library_check("softmax!", output, input)
+    if output.shape() != input.shape():
+        raise TensorError(f"Input, output shapes do not match {input.shape()} {output.shape()}")
+    stream = check_stream()
+    if len(input.shape()) == 3:
+        stream.softmax_spatial(output.buffer, output.dimensions, input.buffer, input.dimensions)
+    else:
+        i, o = as_batch_matrix(input), as_batch_matrix(output)
+        stream.softmax_eltwise(o.buffer, o.dimensions, i.buffer, i.dimensions)
+    return output
+
+
 # ---------------------------------------------------------------- composites
 
 def normalize(dest: Tensor, mag_vec: Tensor, radius_length, epsilon=1e-6) -> Tensor:

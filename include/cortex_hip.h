@@ -80,6 +80,12 @@ typedef enum ct_reduce_op_t {
   CT_ROP_MAGNITUDE_SQUARED = 5
 } ct_reduce_op_t;
 
+/* activation-gradient! operations (src/cortex/tensor.clj:1256-1284; the CUDA
+ * backend maps the same three keywords in cuda/tensor_math.clj:179-185). */
+typedef enum ct_activation_op_t {
+  CT_ACT_LOGISTIC = 0, CT_ACT_TANH = 1, CT_ACT_RELU = 2
+} ct_activation_op_t;
+
 typedef enum ct_status {
   CT_OK = 0,
   CT_ERR_INVALID = 1,     /* bad argument: rank, dtype, op code, null pointer, shape rule */
@@ -232,6 +238,31 @@ int ct_ternary_op_constant_constant(void* stream, void* dest, const ct_dims* des
  * op(input * input_alpha). */
 int ct_unary_reduce(void* stream, void* output, const ct_dims* output_dims, double input_alpha,
                     const void* input, const ct_dims* input_dims, int op, int dtype);
+
+/* ------------------------------------------------- neural-network tensor ops */
+
+/* activation-gradient! (tensor/math.clj:176-181; cpu/tensor_math.clj:1318-1362):
+ *   logistic  input_gradient = output * (1 - output) * output_gradient
+ *   tanh      input_gradient = (1 - output * output) * output_gradient
+ *   relu      input_gradient = (output > 0 ? 1 : 0) * output_gradient
+ * each evaluated in double and rounded once.  dtype is CT_F32 or CT_F64. */
+int ct_activation_gradient(void* stream, void* input_gradient, const ct_dims* input_gradient_dims,
+                           const void* output_gradient, const ct_dims* output_gradient_dims,
+                           const void* output, const ct_dims* output_dims, int op, int64_t n,
+                           int dtype);
+
+/* softmax-eltwise! (tensor/math.clj:183-185; cpu/tensor_math.clj:1037-1094):
+ * dimensions are [rows, k] or [outer, rows, k]; every row becomes
+ * exp(x - max(x)) / sum(exp(x - max(x))).  Direct dimensions only; dtype is
+ * CT_F32 or CT_F64. */
+int ct_softmax_eltwise(void* stream, void* output, const ct_dims* output_dims, const void* input,
+                       const ct_dims* input_dims, int dtype);
+
+/* softmax-spatial! (tensor/math.clj:187-189; cpu/tensor_math.clj:1097-1103):
+ * dimensions are [batch, channels, elements]; the softmax runs across the
+ * channels of every (batch, element) position. */
+int ct_softmax_spatial(void* stream, void* output, const ct_dims* output_dims, const void* input,
+                       const ct_dims* input_dims, int dtype);
 
 /* ------------------------------------------------- optimizers */
 

@@ -19,6 +19,8 @@
 //   binary ops               cpu/tensor_math.clj:278-462
 //   ternary select           cpu/tensor_math.clj:464-580
 //   unary-reduce!            cpu/tensor_math.clj:582-663
+//   activation-gradient!     cpu/tensor_math.clj:1318-1362
+//   softmax (both forms)     cpu/tensor_math.clj:1037-1103
 //   Adam                     src/cortex/optimize/adam.clj:68-102
 //   Adadelta                 java/cortex/compute/optimize/AdadeltaOptimizer.java:29-64
 //
@@ -522,6 +524,69 @@ int reduce_t(T* out, const Dims& od, double alpha, const T* in, const Dims& id, 
   return 0;
 }
 
+// act-backward-impl (cpu/tensor_math.clj:1318-1362).  Float operands widen to
+// double, the products run left to right in double, the store rounds once.
+template <class T>
+int activation_gradient_t(T* ig, const Dims& igd, const T* og, const Dims& ogd, const T* out, const Dims& od,
+                          int op, int64_t n) {
+  const Dims* ops[3] = {&igd, &ogd, &od};
+  const MaxShape mx = max_shape_of(ops, 3);
+  const Addr ia = make_addr(igd, mx), ga = make_addr(ogd, mx), oa = make_addr(od, mx);
+#pragma omp parallel for schedule(static)
+  for (int64_t e = 0; e < n; ++e) {
+    const double o = (double)out[oa(e)], g = (double)og[ga(e)];
+    double r;
+    switch (op) {
+      case CT_ACT_LOGISTIC: r = (o * (1.0 - o)) * g; break;
+      case CT_ACT_TANH: r = (1.0 - o * o) * g; break;
+      default: r = (o > 0.0 ? 1.0 : 0.0) * g; break;  // relu
+    }
+    ig[ia(e)] = (T)r;
+  }
+  return 0;
+}
+
+// softmax-impl (cpu/tensor_math.clj:1037-1088).  The loop that finds the row
+// maximum reads element 0 through the input's address object and elements
+// 1..k-1 of the INPUT buffer through the OUTPUT's address object (:1067-1072);
+// that is restated as written.  The exponentials are stored rounded to T, their
+// stored values are summed sequentially in double, the sum is rounded to T and
+// every element is divided by it in T (ArrayView.diveq).
+template <class T>
+int softmax_t(T* out, const Dims& od, const T* in, const Dims& id) {
+  const Dims* ops[2] = {&od, &id};
+  const MaxShape mx = max_shape_of(ops, 2);
+  if (mx.nd != 2 && mx.nd != 3) return fail("softmax implementation only supports shapes of 2 or 3 dimensions");
+  const Addr oa = make_addr(od, mx), ia = make_addr(id, mx);
+  const int64_t outer = mx.nd == 2 ? 1 : mx.s[0], par = mx.nd == 2 ? mx.s[0] : mx.s[1],
+                k = mx.nd == 2 ? mx.s[1] : mx.s[2];
+  for (int64_t o = 0; o < outer; ++o) {
+#pragma omp parallel for schedule(static)
+    for (int64_t p = 0; p < par; ++p) {
+      const int64_t off = o * par * k + p * k;
+      double mv = (double)in[ia(off)];
+      for (int64_t i = 1; i < k; ++i) mv = j_max(mv, (double)in[oa(off + i)]);
+      const T max_val = (T)mv;
+      for (int64_t i = 0; i < k; ++i) out[oa(off + i)] = (T)std::exp((double)in[ia(off + i)] - (double)max_val);
+      double sum = (double)out[oa(off)];
+      for (int64_t i = 1; i < k; ++i) sum += (double)out[oa(off + i)];
+      const T sum_val = (T)sum;
+      for (int64_t i = 0; i < k; ++i) out[oa(off + i)] = out[oa(off + i)] / sum_val;
+    }
+  }
+  return 0;
+}
+
+// dimensions/transpose with [0 2 1] (dimensions.clj:473-484)
+inline bool transpose_021(const Dims& d, Dims* t) {
+  if (d.nd != 3) return false;
+  *t = d;
+  std::swap(t->shape[1], t->shape[2]);
+  std::swap(t->strides[1], t->strides[2]);
+  std::swap(t->index[1], t->index[2]);
+  return true;
+}
+
 // cpu-adam-step-impl! (adam.clj:68-102).  The scalars are cast to the datatype
 // first; the arithmetic then runs in double.
 template <class T>
@@ -738,6 +803,42 @@ int co_unary_reduce(void* output, const ct_dims* output_dims, double input_alpha
   if (op < 0 || op > CT_ROP_MAGNITUDE_SQUARED) return fail("unknown reduction op");
   DISPATCH_DTYPE(dtype, return reduce_t<T>((T*)output, od, input_alpha, (const T*)input, id, op));
   return 0;
+}
+
+int co_activation_gradient(void* input_gradient, const ct_dims* input_gradient_dims, const void* output_gradient,
+                           const ct_dims* output_gradient_dims, const void* output, const ct_dims* output_dims,
+                           int op, int64_t n, int dtype) {
+  LOAD(igd, input_gradient_dims);
+  LOAD(ogd, output_gradient_dims);
+  LOAD(od, output_dims);
+  if (op < CT_ACT_LOGISTIC || op > CT_ACT_RELU) return fail("Only :logistic :tanh and :relu are supported");
+  if (dtype == CT_F32)
+    return activation_gradient_t<float>((float*)input_gradient, igd, (const float*)output_gradient, ogd,
+                                        (const float*)output, od, op, n);
+  if (dtype == CT_F64)
+    return activation_gradient_t<double>((double*)input_gradient, igd, (const double*)output_gradient, ogd,
+                                         (const double*)output, od, op, n);
+  return fail("activation-gradient! is only defined for float and double tensors");
+}
+
+int co_softmax_eltwise(void* output, const ct_dims* output_dims, const void* input, const ct_dims* input_dims,
+                       int dtype) {
+  LOAD(od, output_dims);
+  LOAD(id, input_dims);
+  if (dtype == CT_F32) return softmax_t<float>((float*)output, od, (const float*)input, id);
+  if (dtype == CT_F64) return softmax_t<double>((double*)output, od, (const double*)input, id);
+  return fail("softmax! is only defined for float and double tensors");
+}
+
+int co_softmax_spatial(void* output, const ct_dims* output_dims, const void* input, const ct_dims* input_dims,
+                       int dtype) {
+  LOAD(od, output_dims);
+  LOAD(id, input_dims);
+  Dims odt, idt;
+  if (!transpose_021(od, &odt) || !transpose_021(id, &idt)) return fail("softmax-spatial! needs [batch channels elements]");
+  if (dtype == CT_F32) return softmax_t<float>((float*)output, odt, (const float*)input, idt);
+  if (dtype == CT_F64) return softmax_t<double>((double*)output, odt, (const double*)input, idt);
+  return fail("softmax! is only defined for float and double tensors");
 }
 
 int co_adam_step(int dtype, double alpha, double beta1, double beta2, double epsilon,

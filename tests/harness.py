@@ -218,6 +218,15 @@ def unary_reduce(side, out: View, alpha, inp: View, op):
     side.call("unary_reduce", *_pd(side, out), float(alpha), *_pd(side, inp), capi.REDUCE_OPS[op], out.buf.dtype)
 
 
+def activation_gradient(side, ig: View, og: View, out: View, op, n):
+    side.call("activation_gradient", *_pd(side, ig), *_pd(side, og), *_pd(side, out), capi.ACTIVATION_OPS[op], n,
+              ig.buf.dtype)
+
+
+def softmax(side, out: View, inp: View, spatial=False):
+    side.call("softmax_spatial" if spatial else "softmax_eltwise", *_pd(side, out), *_pd(side, inp), out.buf.dtype)
+
+
 def adam_step(side, alpha, beta1, beta2, eps, pb1, pb2, ga, grad: View, params: View, m: View, v: View, n):
     args = (grad.buf.dtype, float(alpha), float(beta1), float(beta2), float(eps), float(pb1), float(pb2), float(ga),
             side.ptr(grad), side.ptr(params), side.ptr(m), side.ptr(v), n)

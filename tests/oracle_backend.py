@@ -151,6 +151,18 @@ class OracleStream:
         ob.call("unary_reduce", out.ptr, C.byref(_dims(od)), float(alpha), inp.ptr, C.byref(_dims(idims)),
                 capi.REDUCE_OPS[op], capi.DTYPE_CODES[out.datatype])
 
+    def activation_gradient(self, ig, igd, og, ogd, out, od, op, n):
+        ob.call("activation_gradient", ig.ptr, C.byref(_dims(igd)), og.ptr, C.byref(_dims(ogd)), out.ptr,
+                C.byref(_dims(od)), capi.ACTIVATION_OPS[op], int(n), capi.DTYPE_CODES[ig.datatype])
+
+    def softmax_eltwise(self, out, od, inp, idims):
+        ob.call("softmax_eltwise", out.ptr, C.byref(_dims(od)), inp.ptr, C.byref(_dims(idims)),
+                capi.DTYPE_CODES[out.datatype])
+
+    def softmax_spatial(self, out, od, inp, idims):
+        ob.call("softmax_spatial", out.ptr, C.byref(_dims(od)), inp.ptr, C.byref(_dims(idims)),
+                capi.DTYPE_CODES[out.datatype])
+
     def adam_step(self, alpha, beta1, beta2, eps, pb1, pb2, ga, gradient, parameters, m, v, n):
         ob.call("adam_step", capi.DTYPE_CODES[gradient.datatype], float(alpha), float(beta1), float(beta2), float(eps),
                 float(pb1), float(pb2), float(ga), gradient.ptr, parameters.ptr, m.ptr, v.ptr, int(n))

@@ -206,6 +206,46 @@ def activation_forward(driver, datatype):
         equals([0.0, 0.0, 0.0, 0.0, 0.0, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0], ct.to_double_array(output))
 
 
+# verify/tensor.clj:557-574
+def activation_gradient(driver, datatype):
+    with context(driver, datatype):
+        output = ct.to_tensor(range(12))
+        output_gradient = ct.to_tensor(range(-4, 8))
+        input_gradient = ct.new_tensor([12])
+        ct.activation_gradient(input_gradient, output_gradient, output, "logistic")
+        equals([-0.0, -0.0, 4.0, 6.0, -0.0, -20.0, -60.0, -126.0, -224.0, -360.0, -540.0, -770.0],
+               ct.to_double_array(input_gradient))
+        ct.activation_gradient(input_gradient, output_gradient, output, "tanh")
+        equals([-4.0, -0.0, 6.0, 8.0, -0.0, -24.0, -70.0, -144.0, -252.0, -400.0, -594.0, -840.0],
+               ct.to_double_array(input_gradient))
+        ct.activation_gradient(input_gradient, output_gradient, output, "relu")
+        equals([0.0, -3.0, -2.0, -1.0, 0.0, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0], ct.to_double_array(input_gradient))
+
+
+SOFTMAX_1234 = [0.03205860328008499, 0.08714431874203256, 0.2368828180899101, 0.6439142598879722]
+
+
+# verify/tensor.clj:577-620
+def softmax(driver, datatype):
+    with context(driver, datatype):
+        inp = ct.to_tensor([[1, 2, 3, 4]] * 10)
+        output = ct.new_tensor([10, 4])
+        ct.softmax(output, inp)
+        equals(SOFTMAX_1234 * 10, ct.to_double_array(output), 1e-4)
+        img_dim = 4
+        inp = ct.to_tensor([[[v] * (img_dim * img_dim) for v in (1, 2, 3, 4)]])
+        output = ct.new_tensor([1, 4, img_dim * img_dim])
+        ct.softmax(output, inp)
+        equals([v for v in SOFTMAX_1234 for _ in range(img_dim * img_dim)], ct.to_double_array(output), 1e-4)
+        # some loss terms use softmax with strides that aren't contiguous
+        pred_matrix = ct.to_tensor([list(range(10))] * 5)
+        sel_pred_matr = ct.select(pred_matrix, "all", range(2, 10))
+        test_tensor = ct.to_tensor(range(2, 10))
+        answer = ct.softmax(test_tensor, test_tensor)
+        ct.softmax(sel_pred_matr, sel_pred_matr)
+        equals(([0, 1] + list(ct.to_double_array(answer))) * 5, ct.to_double_array(pred_matrix))
+
+
 # verify/tensor.clj:623-645
 def ternary_op_select(driver, datatype):
     with context(driver, datatype):

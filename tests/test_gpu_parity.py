@@ -527,3 +527,86 @@ def test_streams_and_events(P):
     free, total = C.c_size_t(), C.c_size_t()
     capi.call("ct_memory_info", C.byref(free), C.byref(total))
     assert 0 < free.value <= total.value
+
+
+# ------------------------------------------------------------------ activation-gradient!, softmax
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("op", ["logistic", "tanh", "relu"])
+def test_activation_gradient_bit_exact(P, code, op):
+    rng = np.random.default_rng(30)
+    n = 4099
+    o = values(rng, code, n)
+    o[:4] = [0.0, -0.0, np.nan, 1.0]
+    out, grad = P.buf(o), P.buf(values(rng, code, n))
+    ig = P.buf(np.zeros(n, NP[code]))
+    k = P.run(H.activation_gradient, View(ig, [n]), View(grad, [n]), View(out, [n]), op, n)
+    compare(ig, f"activation-gradient {op} ({k})")
+    # in place over the gradient, and with a transposed output view
+    P.run(H.activation_gradient, View(grad, [n]), View(grad, [n]), View(out, [n]), op, n)
+    compare(grad, f"activation-gradient {op} in place")
+    m = 96
+    o2, g2, i2 = P.buf(values(rng, code, m * m)), P.buf(values(rng, code, m * m)), P.buf(np.zeros(m * m, NP[code]))
+    k = P.run(H.activation_gradient, View(i2, [m, m]), View(g2, [m, m]), View(o2, [m, m]).transpose([1, 0]), op, m * m)
+    compare(i2, f"activation-gradient {op} transposed ({k})")
+
+
+SOFTMAX_SHAPES = [(5, 1), (9, 3), (300, 10), (64, 16), (33, 40), (17, 100), (12, 200), (9, 500), (5, 1000), (3, 3000)]
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=str)
+def test_softmax_rows(P, code, shape):
+    rng = np.random.default_rng(31)
+    rows, k = shape
+    x = P.buf((rng.standard_normal(rows * k) * 4).astype(NP[code]))
+    out = P.buf(np.zeros(rows * k, NP[code]))
+    tol = 2e-6 if code == capi.F32 else 1e-12
+    kern = P.run(H.softmax, View(out, [rows, k]), View(x, [rows, k]))
+    compare(out, f"softmax {shape} ({kern})", tol=tol)
+    assert kern == ("softmax_lane" if k < 8 else "softmax_wave" if k <= 1024 else "softmax_wave_loop")
+    P.run(H.softmax, View(x, [rows, k]), View(x, [rows, k]))     # in place
+    compare(x, f"softmax {shape} in place", tol=tol)
+
+
+@pytest.mark.parametrize("code", FLOATS)
+def test_softmax_layouts(P, code):
+    rng = np.random.default_rng(32)
+    tol = 2e-6 if code == capi.F32 else 1e-12
+    # spatial: [batch, channels, elements], softmax across channels
+    b, c, e = 3, 21, 130
+    x = P.buf((rng.standard_normal(b * c * e) * 3).astype(NP[code]))
+    out = P.buf(np.zeros(b * c * e, NP[code]))
+    kern = P.run(H.softmax, View(out, [b, c, e]), View(x, [b, c, e]), True)
+    compare(out, f"softmax-spatial ({kern})", tol=tol)
+    assert kern == "softmax_lane"
+    got = out.download().reshape(b, c, e).astype(np.float64)
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
+    # eltwise on three dimensions
+    kern = P.run(H.softmax, View(out, [b, c, e]), View(x, [b, c, e]))
+    compare(out, f"softmax 3-d eltwise ({kern})", tol=tol)
+    # pitched rows in place: select :all (range 2 10) of a [5, 10] matrix (verify/tensor.clj:611-620)
+    m = P.buf(np.tile(np.arange(10), 5).astype(NP[code]))
+    sel = View(m, [5, 8], [10, 1], offset=2)
+    P.run(H.softmax, sel, sel)
+    compare(m, "softmax pitched in place", tol=tol)
+    # NaN poisons its row only; infinities of one sign
+    y = (rng.standard_normal(4 * 50)).astype(NP[code])
+    y[7] = np.nan
+    y[60] = np.inf
+    yb, ob = P.buf(y), P.buf(np.zeros(200, NP[code]))
+    P.run(H.softmax, View(ob, [4, 50]), View(yb, [4, 50]))
+    compare(ob, "softmax with NaN and inf rows", tol=tol)
+
+
+def test_softmax_and_activation_gradient_errors(P):
+    x = P.buf(np.zeros(16, np.float32))
+    xi = P.buf(np.zeros(16, np.int32))
+    with pytest.raises(capi.CortexHipError, match="float and double"):
+        H.softmax(P.hip, View(xi, [4, 4]), View(xi, [4, 4]))
+    with pytest.raises(capi.CortexHipError, match="2 or 3 dimensions"):
+        H.softmax(P.hip, View(x, [16]), View(x, [16]))
+    with pytest.raises(capi.CortexHipError, match="do not match"):
+        H.softmax(P.hip, View(x, [4, 4]), View(x, [2, 8]))
+    with pytest.raises(capi.CortexHipError, match="float and double"):
+        H.activation_gradient(P.hip, View(xi, [16]), View(xi, [16]), View(xi, [16]), "relu", 16)

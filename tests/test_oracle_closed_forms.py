@@ -448,3 +448,73 @@ def test_adadelta_float_follows_the_java_step():
     H.assert_bit_exact(ga.host, acc.astype(np.float32), "grad accum")
     H.assert_bit_exact(da.host, dacc.astype(np.float32), "dx accum")
     H.assert_bit_exact(p.host, p0 + dx.astype(np.float32), "params (float +=)")
+
+
+# ------------------------------------------------------------------ activation-gradient!, softmax
+
+@pytest.mark.parametrize("code", [capi.F32, capi.F64])
+def test_activation_gradient_closed_form(code):
+    rng = np.random.default_rng(21)
+    n = 257
+    out = rng.standard_normal(n).astype(NP[code])
+    grad = rng.standard_normal(n).astype(NP[code])
+    out[:4] = [0.0, -0.0, np.nan, 1.0]
+    o64, g64 = out.astype(np.float64), grad.astype(np.float64)
+    want = {"logistic": (o64 * (1.0 - o64)) * g64, "tanh": (1.0 - o64 * o64) * g64,
+            "relu": np.where(o64 > 0.0, 1.0, 0.0) * g64}
+    for op, w in want.items():
+        ob, gb, ib = hbuf(out), hbuf(grad), hbuf(np.zeros(n, NP[code]))
+        H.activation_gradient(ORACLE, View(ib, [n]), View(gb, [n]), View(ob, [n]), op, n)
+        H.assert_bit_exact(ib.host, w.astype(NP[code]), op)   # one rounding of the double result
+
+
+def test_activation_gradient_broadcasts_like_the_other_elementwise_ops():
+    out, grad = hbuf(np.array([2.0, -1.0, 0.5], np.float32)), hbuf(np.arange(6, dtype=np.float32))
+    ib = hbuf(np.zeros(6, np.float32))
+    H.activation_gradient(ORACLE, View(ib, [2, 3]), View(grad, [2, 3]), View(out, [3]), "relu", 6)
+    assert ib.host.tolist() == [0.0, 0.0, 2.0, 3.0, 0.0, 5.0]
+
+
+@pytest.mark.parametrize("code", [capi.F32, capi.F64])
+def test_softmax_closed_form_and_invariants(code):
+    rng = np.random.default_rng(22)
+    rows, k = 7, 13
+    x = (rng.standard_normal((rows, k)) * 5).astype(NP[code])
+    xb, ob = hbuf(x.ravel()), hbuf(np.zeros(rows * k, NP[code]))
+    H.softmax(ORACLE, View(ob, [rows, k]), View(xb, [rows, k]))
+    got = ob.host.reshape(rows, k).astype(np.float64)
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    want = e / e.sum(axis=1, keepdims=True)
+    tol = 1e-6 if code == capi.F32 else 1e-14
+    assert np.allclose(got, want, rtol=tol, atol=0)
+    assert np.allclose(got.sum(axis=1), 1.0, atol=k * tol)
+    # a shifted input gives the same distribution; the largest entry of a row is exp(0)/sum
+    sb, o2 = hbuf((x + NP[code](3.0)).ravel()), hbuf(np.zeros(rows * k, NP[code]))
+    H.softmax(ORACLE, View(o2, [rows, k]), View(sb, [rows, k]))
+    assert np.allclose(o2.host.astype(np.float64), ob.host.astype(np.float64), rtol=20 * tol)
+    assert np.allclose(got.max(axis=1), 1.0 / e.sum(axis=1), rtol=tol)
+
+
+def test_softmax_spatial_runs_across_channels_and_three_dims_batch():
+    rng = np.random.default_rng(23)
+    b, c, e = 2, 5, 6
+    x = rng.standard_normal((b, c, e))
+    xb, ob = hbuf(x.ravel()), hbuf(np.zeros(b * c * e))
+    H.softmax(ORACLE, View(ob, [b, c, e]), View(xb, [b, c, e]), spatial=True)
+    ex = np.exp(x - x.max(axis=1, keepdims=True))
+    assert np.allclose(ob.host.reshape(b, c, e), ex / ex.sum(axis=1, keepdims=True), rtol=1e-14)
+    # the eltwise form on three dimensions normalises the last axis of every [outer, row]
+    H.softmax(ORACLE, View(ob, [b, c, e]), View(xb, [b, c, e]))
+    ex = np.exp(x - x.max(axis=2, keepdims=True))
+    assert np.allclose(ob.host.reshape(b, c, e), ex / ex.sum(axis=2, keepdims=True), rtol=1e-14)
+
+
+def test_softmax_stores_float_exponentials_before_summing():
+    # every stage rounds to the tensor type: e_i = float(exp(x_i - max)), s = float(sum of e_i), y_i = e_i / s in float
+    x = np.array([0.1, 0.2, 0.3, 0.7, -1.5], np.float32)
+    xb, ob = hbuf(x), hbuf(np.zeros(5, np.float32))
+    H.softmax(ORACLE, View(ob, [1, 5]), View(xb, [1, 5]))
+    e = np.exp(x.astype(np.float64) - np.float64(x.max())).astype(np.float32)
+    s = np.float32(np.cumsum(e.astype(np.float64))[-1])
+    H.assert_bit_exact(ob.host, e / s, "softmax staging")
