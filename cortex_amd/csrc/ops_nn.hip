@@ -12,16 +12,18 @@
 //   e_i = T(exp(double(x_i) - double(m)))
 //   s   = T(sum of double(e_i))
 //   y_i = e_i / s                      (a division in T)
-// Two kernels cover the layouts:
-//   softmax_wave_kernel  a group of 16 or 64 lanes owns a row and walks k
-//                        (coalesced when k is the unit-stride axis); rows of up
-//                        to 16 elements per lane stay in registers, longer
-//                        rows are re-read from cache
-//   softmax_lane_kernel  one lane owns a row and walks k sequentially, the
-//                        lanes of a wave take neighbouring rows (coalesced when
-//                        the row axis is unit-stride: the spatial form, where
-//                        k is the channel axis).  Its sum runs in the
-//                        reference's own order.
+// Three kernels cover the layouts:
+//   softmax_wave_kernel   a group of 4, 16 or 64 lanes owns a row of up to 1024
+//                         vectors, kept in registers (128-bit accesses when the
+//                         rows are unit-stride and aligned)
+//   softmax_block_kernel  longer rows: one block per row, exponentials parked
+//                         in the output and scaled in a third pass
+//   softmax_lane_kernel   one lane owns a row and walks k sequentially, the
+//                         lanes of a wave take neighbouring rows (coalesced when
+//                         the row axis is unit-stride: the spatial form, where
+//                         k is the channel axis); rows of up to 32 elements stay
+//                         in registers.  Its sum runs in the reference's order.
+// y_i is formed as e_i * (1 / s): at most one ulp from the reference's e_i / s.
 // The reference's maximum loop reads elements 1..k-1 of the input through the
 // output's address object (cpu/tensor_math.clj:1067-1072); that only matters
 // when the two layouts differ, and then only through rounding, because the
@@ -81,19 +83,21 @@ template <class T> __device__ __forceinline__ T jvm_max(T a, T b) {
   return a > b ? a : b;
 }
 
-// T(exp(double(x) - double(m))).  For float the exact double difference is split
-// into a float head and tail: exp(h + t) = exp(h) * (1 + t) to well below half an
-// ulp, and expf is accurate to about an ulp; a plain float subtraction would
-// lose up to |x - m| * 2^-24 relative (3e-6 at a difference of 50).
+// T(exp(double(x) - double(m))).  For float, x - m is formed exactly as a float
+// head h and tail t (an error-free sum), exp(h + t) = exp(h) * (1 + t) to well
+// below half an ulp, and expf is accurate to about an ulp; a plain float
+// subtraction alone would lose up to |x - m| * 2^-24 relative (3e-6 at a
+// difference of 50).  Infinite operands make the tail meaningless: it is dropped.
 template <class T> __device__ __forceinline__ T shifted_exp(T x, T m) {
-  const double d = (double)x - (double)m;
   if constexpr (std::is_same<T, float>::value) {
-    const float h = (float)d;
-    const float t = (float)(d - (double)h);
+    const float h = x - m;
+    const float bb = h - x;
+    float t = (x - (h - bb)) + (-m - bb);
+    if (!(fabsf(t) < __builtin_huge_valf())) t = 0.0f;
     const float e = expf(h);
-    return e + e * t;
+    return fmaf(e, t, e);
   } else {
-    return exp(d);
+    return exp(x - m);
   }
 }
 
@@ -114,10 +118,13 @@ __device__ __forceinline__ void softmax_row_base(const SoftmaxArgs& a, int64_t r
   *ob = (int64_t)o * a.out_outer + (int64_t)p * a.out_row;
 }
 
-// TPR lanes per row.  ITER > 0: the row (k <= TPR * ITER) is held in registers.
-// ITER == 0: any k, the row is read three times.
-template <class T, int TPR, int ITER>
+// TPR lanes (inside one wave) own a row of at most TPR * ITER vectors and keep
+// it in registers: one read, one write.  VEC > 1 needs unit-stride, aligned rows.
+// The division by the row sum is a multiplication by its reciprocal (at most
+// one ulp from the quotient).
+template <class T, int VEC, int TPR, int ITER>
 __global__ void __launch_bounds__(kBlock) softmax_wave_kernel(const SoftmaxArgs a) {
+  using V = Vec<T, VEC>;
   const int lane = threadIdx.x % TPR;
   const int64_t r = (int64_t)blockIdx.x * (kBlock / TPR) + threadIdx.x / TPR;
   const bool live = r < a.n_rows;
@@ -125,51 +132,86 @@ __global__ void __launch_bounds__(kBlock) softmax_wave_kernel(const SoftmaxArgs 
   if (live) softmax_row_base(a, r, &ib, &ob);
   const T* in = reinterpret_cast<const T*>(a.in) + ib;
   T* out = reinterpret_cast<T*>(a.out) + ob;
-  constexpr int NX = ITER > 0 ? ITER : 1;
-  T x[NX];
-  // identity of Math.max that lets NaN through
-  T m = -__builtin_huge_valf();
-  if constexpr (ITER > 0) {
+  const uint32_t nv = a.k / VEC;
+  V x[ITER];
+  T m = -__builtin_huge_valf();  // identity of Math.max that lets NaN through
 #pragma unroll
-    for (int j = 0; j < ITER; ++j) {
-      const uint32_t i = lane + j * TPR;
-      if (live && i < a.k) { x[j] = in[(int64_t)i * a.in_k]; m = jvm_max(m, x[j]); }
+  for (int j = 0; j < ITER; ++j) {
+    const uint32_t i = lane + j * TPR;
+    if (live && i < nv) {
+      if constexpr (VEC > 1) x[j] = *reinterpret_cast<const V*>(in + (int64_t)i * VEC);
+      else x[j].v[0] = in[(int64_t)i * a.in_k];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) m = jvm_max(m, x[j].v[e]);
     }
-  } else {
-    if (live)
-      for (uint32_t i = lane; i < a.k; i += TPR) m = jvm_max(m, in[(int64_t)i * a.in_k]);
   }
 #pragma unroll
   for (int s = TPR / 2; s >= 1; s >>= 1) m = jvm_max(m, (T)__shfl_xor(m, s, 64));
   double sum = 0.0;
-  if constexpr (ITER > 0) {
 #pragma unroll
-    for (int j = 0; j < ITER; ++j) {
-      const uint32_t i = lane + j * TPR;
-      if (live && i < a.k) { x[j] = shifted_exp(x[j], m); sum += (double)x[j]; }
+  for (int j = 0; j < ITER; ++j) {
+    const uint32_t i = lane + j * TPR;
+    if (live && i < nv) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) { x[j].v[e] = shifted_exp(x[j].v[e], m); sum += (double)x[j].v[e]; }
     }
-  } else {
-    if (live)
-      for (uint32_t i = lane; i < a.k; i += TPR) sum += (double)shifted_exp(in[(int64_t)i * a.in_k], m);
   }
 #pragma unroll
   for (int s = TPR / 2; s >= 1; s >>= 1) sum += __shfl_xor(sum, s, 64);
-  const T denom = (T)sum;
-  if constexpr (ITER > 0) {
+  const T inv = (T)1 / (T)sum;
 #pragma unroll
-    for (int j = 0; j < ITER; ++j) {
-      const uint32_t i = lane + j * TPR;
-      if (live && i < a.k) out[(int64_t)i * a.out_k] = x[j] / denom;
+  for (int j = 0; j < ITER; ++j) {
+    const uint32_t i = lane + j * TPR;
+    if (live && i < nv) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) x[j].v[e] *= inv;
+      if constexpr (VEC > 1) *reinterpret_cast<V*>(out + (int64_t)i * VEC) = x[j];
+      else out[(int64_t)i * a.out_k] = x[j].v[0];
     }
-  } else {
-    if (live)
-      for (uint32_t i = lane; i < a.k; i += TPR)
-        out[(int64_t)i * a.out_k] = shifted_exp(in[(int64_t)i * a.in_k], m) / denom;
   }
 }
 
-// One lane per row; in place is fine (each pass reads x_i before y_i is written).
+// One block per row of any length: the exponentials are parked in the output
+// (rounded to T, as the CPU backend stores them) and scaled in a third pass.
 template <class T>
+__global__ void __launch_bounds__(kBlock) softmax_block_kernel(const SoftmaxArgs a) {
+  __shared__ double lds[kBlock / 64];
+  int64_t ib, ob;
+  softmax_row_base(a, blockIdx.x, &ib, &ob);
+  const T* in = reinterpret_cast<const T*>(a.in) + ib;
+  T* out = reinterpret_cast<T*>(a.out) + ob;
+  const int wave = threadIdx.x >> 6;
+  T m = -__builtin_huge_valf();
+  for (uint32_t i = threadIdx.x; i < a.k; i += kBlock) m = jvm_max(m, in[(int64_t)i * a.in_k]);
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) m = jvm_max(m, (T)__shfl_xor(m, s, 64));
+  if ((threadIdx.x & 63) == 0) lds[wave] = (double)m;
+  __syncthreads();
+  m = (T)lds[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / 64; ++w) m = jvm_max(m, (T)lds[w]);
+  __syncthreads();
+  double sum = 0.0;
+  for (uint32_t i = threadIdx.x; i < a.k; i += kBlock) {
+    const T e = shifted_exp(in[(int64_t)i * a.in_k], m);
+    out[(int64_t)i * a.out_k] = e;
+    sum += (double)e;
+  }
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) sum += __shfl_xor(sum, s, 64);
+  if ((threadIdx.x & 63) == 0) lds[wave] = sum;
+  __syncthreads();
+  sum = lds[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / 64; ++w) sum += lds[w];
+  const T inv = (T)1 / (T)sum;
+  for (uint32_t i = threadIdx.x; i < a.k; i += kBlock) out[(int64_t)i * a.out_k] *= inv;  // each lane re-reads its own stores
+}
+
+// One lane per row, the lanes of a wave on neighbouring rows.  CMAX > 0: the row
+// (k <= CMAX) stays in registers.  CMAX == 0: any k, exponentials parked in the
+// output.  The sum runs in the reference's own order.
+template <class T, int CMAX>
 __global__ void __launch_bounds__(kBlock) softmax_lane_kernel(const SoftmaxArgs a) {
   const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (r >= a.n_rows) return;
@@ -177,12 +219,32 @@ __global__ void __launch_bounds__(kBlock) softmax_lane_kernel(const SoftmaxArgs 
   softmax_row_base(a, r, &ib, &ob);
   const T* in = reinterpret_cast<const T*>(a.in) + ib;
   T* out = reinterpret_cast<T*>(a.out) + ob;
-  T m = in[0];
-  for (uint32_t i = 1; i < a.k; ++i) m = jvm_max(m, in[(int64_t)i * a.in_k]);
-  double sum = (double)shifted_exp(in[0], m);
-  for (uint32_t i = 1; i < a.k; ++i) sum += (double)shifted_exp(in[(int64_t)i * a.in_k], m);
-  const T denom = (T)sum;
-  for (uint32_t i = 0; i < a.k; ++i) out[(int64_t)i * a.out_k] = shifted_exp(in[(int64_t)i * a.in_k], m) / denom;
+  if constexpr (CMAX > 0) {
+    T x[CMAX];
+    T m = -__builtin_huge_valf();
+#pragma unroll
+    for (int i = 0; i < CMAX; ++i)
+      if ((uint32_t)i < a.k) { x[i] = in[(int64_t)i * a.in_k]; m = jvm_max(m, x[i]); }
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < CMAX; ++i)
+      if ((uint32_t)i < a.k) { x[i] = shifted_exp(x[i], m); sum += (double)x[i]; }
+    const T inv = (T)1 / (T)sum;
+#pragma unroll
+    for (int i = 0; i < CMAX; ++i)
+      if ((uint32_t)i < a.k) out[(int64_t)i * a.out_k] = x[i] * inv;
+  } else {
+    T m = in[0];
+    for (uint32_t i = 1; i < a.k; ++i) m = jvm_max(m, in[(int64_t)i * a.in_k]);
+    double sum = 0.0;
+    for (uint32_t i = 0; i < a.k; ++i) {
+      const T e = shifted_exp(in[(int64_t)i * a.in_k], m);
+      out[(int64_t)i * a.out_k] = e;
+      sum += (double)e;
+    }
+    const T inv = (T)1 / (T)sum;
+    for (uint32_t i = 0; i < a.k; ++i) out[(int64_t)i * a.out_k] *= inv;
+  }
 }
 
 struct RowLayout { int64_t outer, rows, k, s_outer, s_row, s_k; };
@@ -217,22 +279,40 @@ int softmax_run(hipStream_t s, void* out, const RowLayout& ol, const void* in, c
   // lanes along the row axis when that is the unit-stride one (spatial form) or the rows are tiny
   const bool row_major = il.s_k == 1 || il.k == 1;
   if (il.k < 8 || (!row_major && il.s_row == 1)) {
-    note_kernel("softmax_lane");
-    hipLaunchKernelGGL((softmax_lane_kernel<T>), dim3((uint32_t)((a.n_rows + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, a);
+    const dim3 grid((uint32_t)((a.n_rows + kBlock - 1) / kBlock));
+    note_kernel(il.k <= 32 ? "softmax_lane" : "softmax_lane_loop");
+    if (il.k <= 8) hipLaunchKernelGGL((softmax_lane_kernel<T, 8>), grid, dim3(kBlock), 0, s, a);
+    else if (il.k <= 32) hipLaunchKernelGGL((softmax_lane_kernel<T, 32>), grid, dim3(kBlock), 0, s, a);
+    else hipLaunchKernelGGL((softmax_lane_kernel<T, 0>), grid, dim3(kBlock), 0, s, a);
     return after_launch(s);
   }
-#define CT_SM(TPR, ITER)                                                                                         \
-  hipLaunchKernelGGL((softmax_wave_kernel<T, TPR, ITER>),                                                       \
+  constexpr int VMAX = 16 / (int)sizeof(T);
+  auto aligned = [](const void* p, const RowLayout& l) {
+    return l.s_k == 1 && l.k % VMAX == 0 && l.s_row % VMAX == 0 && l.s_outer % VMAX == 0 &&
+           (uintptr_t)p % 16 == 0;
+  };
+  const bool vec_ok = aligned(in, il) && aligned(out, ol);
+  const int64_t nv = vec_ok ? il.k / VMAX : il.k;
+#define CT_SM(VEC, TPR, ITER)                                                                                    \
+  hipLaunchKernelGGL((softmax_wave_kernel<T, VEC, TPR, ITER>),                                                  \
                      dim3((uint32_t)((a.n_rows + (kBlock / TPR) - 1) / (kBlock / TPR))), dim3(kBlock), 0, s, a)
-  note_kernel(il.k <= 1024 ? "softmax_wave" : "softmax_wave_loop");
-  if (il.k <= 16) CT_SM(16, 1);
-  else if (il.k <= 32) CT_SM(16, 2);
-  else if (il.k <= 64) CT_SM(16, 4);
-  else if (il.k <= 128) CT_SM(64, 2);
-  else if (il.k <= 256) CT_SM(64, 4);
-  else if (il.k <= 512) CT_SM(64, 8);
-  else if (il.k <= 1024) CT_SM(64, 16);
-  else CT_SM(64, 0);
+#define CT_SM_SHAPES(VEC)                     \
+  if (nv <= 4) CT_SM(VEC, 4, 1);              \
+  else if (nv <= 16) CT_SM(VEC, 16, 1);       \
+  else if (nv <= 32) CT_SM(VEC, 16, 2);       \
+  else if (nv <= 64) CT_SM(VEC, 16, 4);       \
+  else if (nv <= 128) CT_SM(VEC, 64, 2);      \
+  else if (nv <= 256) CT_SM(VEC, 64, 4);      \
+  else if (nv <= 512) CT_SM(VEC, 64, 8);      \
+  else CT_SM(VEC, 64, 16)
+  if (nv <= 1024) {
+    note_kernel(vec_ok ? "softmax_wave_vec" : "softmax_wave");
+    if (vec_ok) { CT_SM_SHAPES(VMAX); } else { CT_SM_SHAPES(1); }
+  } else {
+    note_kernel("softmax_block");
+    hipLaunchKernelGGL((softmax_block_kernel<T>), dim3((uint32_t)a.n_rows), dim3(kBlock), 0, s, a);
+  }
+#undef CT_SM_SHAPES
 #undef CT_SM
   return after_launch(s);
 }

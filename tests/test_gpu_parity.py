@@ -551,7 +551,8 @@ def test_activation_gradient_bit_exact(P, code, op):
     compare(i2, f"activation-gradient {op} transposed ({k})")
 
 
-SOFTMAX_SHAPES = [(5, 1), (9, 3), (300, 10), (64, 16), (33, 40), (17, 100), (12, 200), (9, 500), (5, 1000), (3, 3000)]
+SOFTMAX_SHAPES = [(5, 1), (9, 3), (300, 10), (64, 16), (33, 40), (17, 100), (12, 200), (9, 500), (5, 1000), (3, 3000),
+                  (2, 5001), (2, 70000)]
 
 
 @pytest.mark.parametrize("code", FLOATS)
@@ -564,7 +565,7 @@ def test_softmax_rows(P, code, shape):
     tol = 2e-6 if code == capi.F32 else 1e-12
     kern = P.run(H.softmax, View(out, [rows, k]), View(x, [rows, k]))
     compare(out, f"softmax {shape} ({kern})", tol=tol)
-    assert kern == ("softmax_lane" if k < 8 else "softmax_wave" if k <= 1024 else "softmax_wave_loop")
+    assert kern == "softmax_lane" if k < 8 else kern in ("softmax_wave", "softmax_wave_vec", "softmax_block")
     P.run(H.softmax, View(x, [rows, k]), View(x, [rows, k]))     # in place
     compare(x, f"softmax {shape} in place", tol=tol)
 
@@ -580,6 +581,11 @@ def test_softmax_layouts(P, code):
     kern = P.run(H.softmax, View(out, [b, c, e]), View(x, [b, c, e]), True)
     compare(out, f"softmax-spatial ({kern})", tol=tol)
     assert kern == "softmax_lane"
+    c2 = 70                                       # more channels than the register-resident form holds
+    x2, out2 = P.buf((rng.standard_normal(2 * c2 * 90) * 3).astype(NP[code])), P.buf(np.zeros(2 * c2 * 90, NP[code]))
+    kern2 = P.run(H.softmax, View(out2, [2, c2, 90]), View(x2, [2, c2, 90]), True)
+    compare(out2, f"softmax-spatial wide ({kern2})", tol=tol)
+    assert kern2 == "softmax_lane_loop"
     got = out.download().reshape(b, c, e).astype(np.float64)
     assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
     # eltwise on three dimensions
