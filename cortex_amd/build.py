@@ -29,6 +29,7 @@ SOURCES = [
     "ops_reduce.hip",
     "ops_optim.hip",
     "ops_nn.hip",
+    "ops_batchnorm.hip",
 ]
 
 # -ffp-contract=off: the reference's CPU backend rounds after every JVM

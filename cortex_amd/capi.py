@@ -111,6 +111,12 @@ PROTOTYPES = {
     "ct_activation_gradient": [_P, _P, _DP, _P, _DP, _P, _DP, _I, _L, _I],
     "ct_softmax_eltwise": [_P, _P, _DP, _P, _DP, _I],
     "ct_softmax_spatial": [_P, _P, _DP, _P, _DP, _I],
+    "ct_batch_normalize_eltwise": [_P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _I],
+    "ct_batch_normalize_spatial": [_P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _L, _I],
+    "ct_batch_normalize_update_and_apply_eltwise": [_P, _P, _P, _P, _P, _P, _P, _D, _P, _P, _D, _L, _L, _I],
+    "ct_batch_normalize_update_and_apply_spatial": [_P, _P, _P, _P, _P, _P, _P, _D, _P, _P, _D, _L, _L, _L, _I],
+    "ct_batch_normalize_gradients_eltwise": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _I],
+    "ct_batch_normalize_gradients_spatial": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _L, _I],
     "ct_adam_step": [_P, _I, _D, _D, _D, _D, _D, _D, _D, _P, _P, _P, _P, _L],
     "ct_adadelta_step": [_P, _I, _D, _D, _P, _P, _D, _P, _P, _L],
 }

@@ -1,0 +1,787 @@
+// ops_batchnorm.hip -- the six batch-normalization methods of the TensorMath
+// protocol (src/cortex/tensor/math.clj:124-174) after the CPU backend
+// (src/cortex/compute/cpu/tensor_math.clj:731-1033, 1558-1638).
+//
+// All buffers are packed: values [batch, channels, elements], one statistic per
+// channel; the eltwise forms are the spatial forms with one element per channel
+// (BNEltwiseOffsetter and BNSpatialOffsetter, :737-753, give the same offsets).
+//
+// The CPU backend walks each channel several times (five sums in the gradient).
+// Here every method is
+//   statistics pass   all sums of a channel in one read of the operands, in
+//                     double, as per-block partial sums in scratch memory
+//   finishing pass    one wave per channel adds the partials in a fixed order
+//                     and derives the channel's constants
+//   apply pass        one flat, 128-bit vectorised elementwise pass
+// so the operands are read twice and the result written once.  Per-element
+// arithmetic follows the CPU backend operation by operation (double, one
+// rounding at the store); only the order of the additions inside a sum differs
+// (a tree instead of left to right), which moves a double sum by a few units in
+// its last place.
+//
+// Variance: the CPU backend takes the mean first and then sums (mean - x)^2 in
+// a second walk.  The statistics pass here accumulates d = x - K and d^2 for a
+// pivot K (the channel's first value) and forms
+//   sum (m - x)^2 = sum d^2 - 2 (m - K) sum d + n (m - K)^2
+// with m the mean already rounded to the tensor type, as the reference uses it.
+// With K inside the data's range the cancellation costs a few bits of a double.
+#include <algorithm>
+
+#include "elementwise.h"
+
+using namespace cthip;
+
+namespace {
+
+enum { kBnNormalize = 0, kBnGradient = 1 };
+constexpr int kParamStride = 8;  // doubles per channel in the parameter table
+// parameter table, normalize: mean, inv_std (rounded to T), scale, shift
+// parameter table, gradient:  mean, inv_std (double), scale, d_var, 2 * d_var_d_out, d_mean_d_out / n, 1 / n
+constexpr int kUnroll = 4;
+
+template <int MODE> struct bn_nacc { static constexpr int value = MODE == kBnGradient ? 5 : 2; };
+template <int MODE> struct bn_nparam { static constexpr int value = MODE == kBnGradient ? 7 : 4; };
+
+struct BnArgs {
+  const void* x;    // input
+  const void* og;   // output gradient (gradient mode)
+  void* out;        // output, or input gradient
+  double* params;   // [channels][kParamStride]
+  double* partials;
+  int64_t B, C, E, W;        // W = C * E, the length of one batch row
+  int64_t N;                 // B * C * E
+  uint32_t S;                // row segments of the statistics pass
+  uint32_t rows_per_seg;
+  uint32_t nv;               // vectors per (batch, channel) row, row-style statistics
+  uint32_t part_E;           // partial sums kept per channel and segment (1 row-style, E column-style)
+  FastDiv nv_fd, s_fd, e_fd, c_fd;
+  // apply pass
+  int64_t first, count;      // element range of this launch
+  uint32_t table_slots;      // channels held in the LDS table
+  uint32_t table_full;       // the table holds every channel (indexed by channel) instead of a window of rows
+  uint32_t apply_rows_per_seg;  // column-style apply: batch rows per block
+};
+
+struct BnFinish {
+  // normalize (update) mode
+  void* batch_means; void* batch_variances; void* running_means; void* running_variances;
+  const void* scale; const void* bias;
+  double average_factor, epsilon;
+  // gradient mode
+  void* scale_gradient; void* bias_gradient;
+};
+
+// ---------------------------------------------------------------- per-element sums
+
+// Update: d = x - pivot; sums d and d*d.
+template <class T> __device__ __forceinline__ void bn_accumulate_update(double* acc, T x, double pivot) {
+  const double d = (double)x - pivot;
+  acc[0] += d;
+  acc[1] += d * d;
+}
+
+// The scaled output gradient as the CPU backend parks it in the input-gradient
+// buffer (:956-960): scale * og evaluated in double and rounded to T.  For float
+// that is the float product (the double product of two floats is exact).
+template <class T> __device__ __forceinline__ double bn_d_x_hat(T scale, T og) {
+  return (double)(T)(scale * og);
+}
+
+// Gradient: the five sums of batch-normalize-gradients-impl (cpu/tensor_math.clj:928-983)
+// with their per-channel factors taken out of the sums:
+//   acc0 = sum og                 bias gradient
+//   acc1 = sum og * (x - mean)    scale gradient   = inv_std * acc1
+//   acc2 = sum d_x_hat * (x-mean) d_var_d_out      = d_var * acc2
+//   acc3 = sum d_x_hat            first term of d_mean_d_out = -inv_std * acc3
+//   acc4 = sum (x - mean)         second term      = -2 * acc4
+template <class T>
+__device__ __forceinline__ void bn_accumulate_gradient(double* acc, T x, T g, double mean, T scale) {
+  const double og = (double)g;
+  const double xm = (double)x - mean;
+  const double d_x_hat = bn_d_x_hat<T>(scale, g);
+  acc[0] += og;
+  acc[1] += og * xm;
+  acc[2] += d_x_hat * xm;
+  acc[3] += d_x_hat;
+  acc[4] += xm;
+}
+
+// A vector of N elements that is only element-aligned: rows of a length that is
+// not a multiple of the vector width start off the 16-byte grid.  The hardware
+// takes multi-dword global loads at any dword address.
+template <class T, int N> struct __attribute__((packed, aligned(sizeof(T)))) UVec { T v[N]; };
+
+// Loads VEC elements from p.  ALIGNED: p is VEC-element aligned and all VEC exist.
+// Otherwise `valid` elements exist (the row's tail vector is partial).
+template <class T, int VEC, bool ALIGNED, bool NT>
+__device__ __forceinline__ Vec<T, VEC> bn_load(const T* p, int valid) {
+  Vec<T, VEC> r;
+  if constexpr (ALIGNED) {
+    if constexpr (NT) r = nt_load(reinterpret_cast<const Vec<T, VEC>*>(p));
+    else r = *reinterpret_cast<const Vec<T, VEC>*>(p);
+  } else {
+    if (valid >= VEC) {
+      const UVec<T, VEC> u = *reinterpret_cast<const UVec<T, VEC>*>(p);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) r.v[e] = u.v[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) r.v[e] = e < valid ? p[e] : (T)0;
+    }
+  }
+  return r;
+}
+
+template <int NACC>
+__device__ __forceinline__ void bn_block_reduce_store(double* acc, double* dst, double* lds) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < NACC; ++k) {
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) acc[k] += __shfl_xor(acc[k], s, 64);
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < NACC; ++k) lds[wave * NACC + k] = acc[k];
+  }
+  __syncthreads();
+  if (threadIdx.x < NACC) {
+    double r = lds[threadIdx.x];
+#pragma unroll
+    for (int w = 1; w < kBlock / 64; ++w) r += lds[w * NACC + threadIdx.x];
+    dst[threadIdx.x] = r;
+  }
+}
+
+// ---------------------------------------------------------------- statistics, row style
+// One block per (channel, segment of the batch).  The (batch, channel) rows of
+// the segment are walked as one list of vectors, 256 lanes wide, kUnroll loads
+// in flight per lane.
+template <class T, int VEC, int MODE, bool ALIGNED, bool NT>
+__global__ void __launch_bounds__(kBlock) bn_stats_row_kernel(const BnArgs a) {
+  using V = Vec<T, VEC>;
+  constexpr int NACC = bn_nacc<MODE>::value;
+  __shared__ double lds[(kBlock / 64) * NACC];
+  uint32_t c, s;
+  a.s_fd.divmod(blockIdx.x, c, s);
+  const int64_t b0 = (int64_t)s * a.rows_per_seg;
+  const int64_t nb = b0 < a.B ? (a.B - b0 < (int64_t)a.rows_per_seg ? a.B - b0 : (int64_t)a.rows_per_seg) : 0;
+  const uint32_t items = (uint32_t)nb * a.nv;
+  const int64_t base = (b0 * a.C + c) * a.E;
+  const T* x = reinterpret_cast<const T*>(a.x) + base;
+  const T* og = reinterpret_cast<const T*>(a.og) + base;
+  const double* pm = a.params + (int64_t)c * kParamStride;
+  double p0;
+  T scale = (T)0;
+  if constexpr (MODE == kBnGradient) { p0 = pm[0]; scale = (T)pm[2]; }
+  else p0 = (double)reinterpret_cast<const T*>(a.x)[(int64_t)c * a.E];  // pivot: the channel's first value
+  double acc[NACC];
+#pragma unroll
+  for (int k = 0; k < NACC; ++k) acc[k] = 0.0;
+  for (uint32_t i0 = threadIdx.x; i0 < items; i0 += kBlock * kUnroll) {
+    V xv[kUnroll], gv[kUnroll];
+    int valid[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const uint32_t i = i0 + u * kBlock;
+      valid[u] = 0;
+      if (i < items) {
+        uint32_t rr, vv;
+        a.nv_fd.divmod(i, rr, vv);
+        const int64_t off = (int64_t)rr * a.W + (int64_t)vv * VEC;
+        const int64_t left = a.E - (int64_t)vv * VEC;  // elements of the row from this vector on
+        valid[u] = ALIGNED || left >= VEC ? VEC : (int)left;
+        xv[u] = bn_load<T, VEC, ALIGNED, NT>(x + off, valid[u]);
+        if constexpr (MODE == kBnGradient) gv[u] = bn_load<T, VEC, ALIGNED, NT>(og + off, valid[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        if (e < valid[u]) {
+          if constexpr (MODE == kBnGradient) bn_accumulate_gradient<T>(acc, xv[u].v[e], gv[u].v[e], p0, scale);
+          else bn_accumulate_update<T>(acc, xv[u].v[e], p0);
+        }
+      }
+    }
+  }
+  bn_block_reduce_store<NACC>(acc, a.partials + ((int64_t)s * a.C + c) * NACC, lds);
+}
+
+// ---------------------------------------------------------------- statistics, column style
+// For few elements per channel (the eltwise form has one): the tensor is the
+// matrix [batch, channels * elements]; a lane owns VEC neighbouring columns, the
+// four waves of a block take every fourth row of the block's batch segment.
+// Partial sums are kept per column.
+template <class T, int VEC, int MODE>
+__global__ void __launch_bounds__(kBlock) bn_stats_col_kernel(const BnArgs a) {
+  using V = Vec<T, VEC>;
+  constexpr int NACC = bn_nacc<MODE>::value;
+  constexpr int WAVES = kBlock / 64;
+  __shared__ double lds[(WAVES - 1) * 64 * VEC * NACC];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t j0 = ((int64_t)blockIdx.x * 64 + lane) * VEC;
+  const bool live = j0 < a.W;
+  const uint32_t s = blockIdx.y;
+  const int64_t b0 = (int64_t)s * a.rows_per_seg;
+  const int64_t nb = b0 < a.B ? (a.B - b0 < (int64_t)a.rows_per_seg ? a.B - b0 : (int64_t)a.rows_per_seg) : 0;
+  double p0[VEC];
+  T scale[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    p0[e] = 0.0;
+    scale[e] = (T)0;
+    if (live) {
+      const uint32_t ch = a.e_fd.div((uint32_t)(j0 + e));
+      if constexpr (MODE == kBnGradient) {
+        const double* pm = a.params + (int64_t)ch * kParamStride;
+        p0[e] = pm[0]; scale[e] = (T)pm[2];
+      } else {
+        p0[e] = (double)reinterpret_cast<const T*>(a.x)[(int64_t)ch * a.E];
+      }
+    }
+  }
+  double acc[VEC][NACC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e)
+#pragma unroll
+    for (int k = 0; k < NACC; ++k) acc[e][k] = 0.0;
+  const T* x = reinterpret_cast<const T*>(a.x) + b0 * a.W + j0;
+  const T* og = reinterpret_cast<const T*>(a.og) + b0 * a.W + j0;
+  if (live) {
+    for (int64_t r0 = wave; r0 < nb; r0 += WAVES * kUnroll) {
+      V xv[kUnroll], gv[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t r = r0 + u * WAVES;
+        if (r < nb) {
+          xv[u] = *reinterpret_cast<const V*>(x + r * a.W);
+          if constexpr (MODE == kBnGradient) gv[u] = *reinterpret_cast<const V*>(og + r * a.W);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        if (r0 + u * WAVES < nb) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            if constexpr (MODE == kBnGradient)
+              bn_accumulate_gradient<T>(acc[e], xv[u].v[e], gv[u].v[e], p0[e], scale[e]);
+            else bn_accumulate_update<T>(acc[e], xv[u].v[e], p0[e]);
+          }
+        }
+      }
+    }
+  }
+  if (wave > 0) {
+    double* mine = lds + ((wave - 1) * 64 + lane) * (VEC * NACC);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+#pragma unroll
+      for (int k = 0; k < NACC; ++k) mine[e * NACC + k] = acc[e][k];
+  }
+  __syncthreads();
+  if (wave == 0 && live) {
+#pragma unroll
+    for (int w = 0; w < WAVES - 1; ++w) {
+      const double* theirs = lds + (w * 64 + lane) * (VEC * NACC);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+#pragma unroll
+        for (int k = 0; k < NACC; ++k) acc[e][k] += theirs[e * NACC + k];
+    }
+    double* dst = a.partials + ((int64_t)s * a.W + j0) * NACC;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+#pragma unroll
+      for (int k = 0; k < NACC; ++k) dst[e * NACC + k] = acc[e][k];
+  }
+}
+
+// ---------------------------------------------------------------- per-channel constants
+
+// Normalization with given statistics (batch-normalize-impl, :766-777).
+template <class T>
+__device__ __forceinline__ void bn_store_normalize_params(double* pm, T mean, T variance, T scale, T shift, double epsilon) {
+  const T eps = (T)epsilon;
+  pm[0] = (double)mean;
+  pm[1] = (double)(T)sqrt(1.0 / ((double)variance + (double)eps));
+  pm[2] = (double)scale;
+  pm[3] = (double)shift;
+}
+
+template <class T>
+__global__ void __launch_bounds__(kBlock) bn_prepare_normalize_kernel(double* params, const T* means, const T* variances,
+                                                                      const T* scale, const T* bias, double epsilon,
+                                                                      int64_t C) {
+  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c < C) bn_store_normalize_params<T>(params + c * kParamStride, means[c], variances[c], scale[c], bias[c], epsilon);
+}
+
+// Gradient constants known before the sums (batch-normalize-gradients-impl, :922-931).
+template <class T>
+__global__ void __launch_bounds__(kBlock) bn_prepare_gradient_kernel(double* params, const T* means, const T* variances,
+                                                                     const T* scale, double epsilon, int64_t C) {
+  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (c >= C) return;
+  const T eps = (T)epsilon;
+  const T pow_factor = (T)(-3.0 / 2.0);
+  const double variance = (double)eps + (double)variances[c];
+  double* pm = params + c * kParamStride;
+  pm[0] = (double)means[c];
+  pm[1] = 1.0 / sqrt(variance);
+  pm[2] = (double)scale[c];
+  pm[3] = (double)(T)(-0.5 * pow(variance, (double)pow_factor));
+}
+
+// One wave per channel adds the channel's partial sums (segments, and columns in
+// the column style) in a fixed order, then lane 0 finishes the channel.
+template <class T, int MODE>
+__global__ void __launch_bounds__(kBlock) bn_finish_kernel(const BnArgs a, const BnFinish f) {
+  constexpr int NACC = bn_nacc<MODE>::value;
+  const int lane = threadIdx.x & 63;
+  const int64_t c = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (c >= a.C) return;
+  double acc[NACC];
+#pragma unroll
+  for (int k = 0; k < NACC; ++k) acc[k] = 0.0;
+  const uint32_t pe = a.part_E;
+  const uint32_t n_part = a.S * pe;
+  const int64_t seg_stride = a.C * (int64_t)pe;
+  for (uint32_t i = lane; i < n_part; i += 64) {
+    const uint32_t s = i / pe, e = i - s * pe;
+    const double* p = a.partials + ((int64_t)s * seg_stride + c * pe + e) * NACC;
+#pragma unroll
+    for (int k = 0; k < NACC; ++k) acc[k] += p[k];
+  }
+#pragma unroll
+  for (int k = 0; k < NACC; ++k) {
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) acc[k] += __shfl_xor(acc[k], s, 64);
+  }
+  if (lane != 0) return;
+  double* pm = a.params + c * kParamStride;
+  const int64_t count = a.B * a.E;
+  if constexpr (MODE == kBnGradient) {
+    // :932-983, with the factors put back
+    const double inv_std = pm[1], d_var = pm[3];
+    reinterpret_cast<T*>(f.bias_gradient)[c] = (T)acc[0];
+    reinterpret_cast<T*>(f.scale_gradient)[c] = (T)(inv_std * acc[1]);
+    const T d_var_d_out = (T)(d_var * acc[2]);
+    const T d_mean_d_out = (T)((-inv_std) * acc[3] + (double)d_var_d_out * ((-2.0 * acc[4]) / (double)count));
+    const double one_over_count = 1.0 / (double)count;
+    pm[4] = (double)d_var_d_out * 2.0;
+    pm[5] = (double)d_mean_d_out * one_over_count;
+    pm[6] = one_over_count;
+  } else {
+    // batch-normalize-update-impl, :831-870
+    const T ave_factor = (T)f.average_factor;
+    const double ave_lerp = (double)(T)1.0 - (double)ave_factor;
+    const double count_val = fmax(1.0, (double)count);
+    const double running_count_val = fmax(1.0, count_val - 1.0);
+    const double pivot = (double)reinterpret_cast<const T*>(a.x)[c * a.E];
+    const T new_mean = (T)(pivot + acc[0] / count_val);
+    const double delta = (double)new_mean - pivot;
+    double new_var = (acc[1] - 2.0 * delta * acc[0]) + (double)count * delta * delta;
+    new_var = new_var < 0.0 ? 0.0 : new_var;
+    T* running_means = reinterpret_cast<T*>(f.running_means);
+    T* running_variances = reinterpret_cast<T*>(f.running_variances);
+    const T mean = running_means[c], variance = running_variances[c];
+    const T batch_variance = (T)(new_var / count_val);
+    reinterpret_cast<T*>(f.batch_means)[c] = new_mean;
+    reinterpret_cast<T*>(f.batch_variances)[c] = batch_variance;
+    running_means[c] = (T)((double)mean * ave_lerp + (double)new_mean * (double)ave_factor);
+    running_variances[c] =
+        (T)((double)variance * ave_lerp + (double)(T)(new_var / running_count_val) * (double)ave_factor);
+    bn_store_normalize_params<T>(pm, new_mean, batch_variance, reinterpret_cast<const T*>(f.scale)[c],
+                                 reinterpret_cast<const T*>(f.bias)[c], f.epsilon);
+  }
+}
+
+// ---------------------------------------------------------------- apply pass
+
+// One output element from its channel's constants p (layout: see kParamStride).
+template <class T, int MODE>
+__device__ __forceinline__ T bn_apply_one(const double* p, T x, T g) {
+  const double xm = (double)x - p[0];
+  if constexpr (MODE == kBnGradient) {
+    // cpu/tensor_math.clj:986-1001
+    const double d_x_hat = bn_d_x_hat<T>((T)p[2], g);
+    const double part1 = d_x_hat * p[1];
+    const double part2 = (p[4] * xm) * p[6];
+    return (T)((part1 + part2) + p[5]);
+  } else {
+    // cpu/tensor_math.clj:778-784
+    return (T)((xm * p[1]) * p[2] + p[3]);
+  }
+}
+
+// Column style, for few elements per channel: a lane keeps the constants of its
+// VEC neighbouring columns of [batch, channels * elements] in registers and walks
+// the rows of the block's batch segment.
+template <class T, int VEC, int MODE>
+__global__ void __launch_bounds__(kBlock) bn_apply_col_kernel(const BnArgs a) {
+  using V = Vec<T, VEC>;
+  constexpr int NP = bn_nparam<MODE>::value;
+  const int64_t j0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
+  if (j0 >= a.W) return;
+  double p[VEC][NP];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    const uint32_t ch = a.e_fd.div((uint32_t)(j0 + e));
+    const double* pm = a.params + (int64_t)ch * kParamStride;
+#pragma unroll
+    for (int k = 0; k < NP; ++k) p[e][k] = pm[k];
+  }
+  const int64_t b0 = (int64_t)blockIdx.y * a.apply_rows_per_seg;
+  const int64_t nb = a.B - b0 < (int64_t)a.apply_rows_per_seg ? a.B - b0 : (int64_t)a.apply_rows_per_seg;
+  const T* x = reinterpret_cast<const T*>(a.x) + b0 * a.W + j0;
+  const T* og = reinterpret_cast<const T*>(a.og) + b0 * a.W + j0;
+  T* out = reinterpret_cast<T*>(a.out) + b0 * a.W + j0;
+  for (int64_t r0 = 0; r0 < nb; r0 += kUnroll) {
+    V xv[kUnroll], gv[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      if (r0 + u < nb) {
+        xv[u] = nt_load(reinterpret_cast<const V*>(x + (r0 + u) * a.W));
+        if constexpr (MODE == kBnGradient) gv[u] = nt_load(reinterpret_cast<const V*>(og + (r0 + u) * a.W));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      if (r0 + u < nb) {
+        V r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.v[e] = bn_apply_one<T, MODE>(p[e], xv[u].v[e], MODE == kBnGradient ? gv[u].v[e] : (T)0);
+        *reinterpret_cast<V*>(out + (r0 + u) * a.W) = r;
+      }
+    }
+  }
+}
+
+// Flat over [first, first + count).  The constants of the channels a block can
+// meet sit in an LDS table: either every channel, or the window of
+// (batch, channel) rows the block's element range touches.
+template <class T, int VEC, int MODE, int UNROLL>
+__global__ void __launch_bounds__(kBlock) bn_apply_kernel(const BnArgs a) {
+  using V = Vec<T, VEC>;
+  constexpr int NP = bn_nparam<MODE>::value;
+  extern __shared__ __align__(16) double table[];
+  constexpr int64_t kSpan = (int64_t)kBlock * VEC * UNROLL;
+  const int64_t blk_first = a.first + (int64_t)blockIdx.x * kSpan;
+  const int64_t row_first = blk_first / a.E;                       // block-uniform
+  const uint32_t ch_first = (uint32_t)(row_first % a.C);           // channel of that (batch, channel) row
+  const uint32_t ch_base = a.table_full ? 0u : ch_first;           // channel held in table slot 0
+  const int64_t end = a.first + a.count;
+  const uint32_t rel0 = (uint32_t)(blk_first - row_first * a.E);  // < E
+  const T* x = reinterpret_cast<const T*>(a.x);
+  const T* og = reinterpret_cast<const T*>(a.og);
+  T* out = reinterpret_cast<T*>(a.out);
+  // the operands' loads are in flight while the table is filled
+  V xv[UNROLL], gv[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t j = blk_first + ((int64_t)u * kBlock + threadIdx.x) * VEC;
+    if (j < end) {
+      xv[u] = nt_load(reinterpret_cast<const V*>(x + j));
+      if constexpr (MODE == kBnGradient) gv[u] = nt_load(reinterpret_cast<const V*>(og + j));
+    }
+  }
+  for (uint32_t i = threadIdx.x; i < a.table_slots * NP; i += kBlock) {
+    const uint32_t slot = i / NP, k = i - slot * NP;
+    uint32_t q, ch;
+    a.c_fd.divmod(ch_base + slot, q, ch);
+    table[i] = a.params[(int64_t)ch * kParamStride + k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const uint32_t jr = (u * kBlock + threadIdx.x) * VEC;
+    const int64_t j = blk_first + jr;
+    if (j < end) {
+      V r;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        uint32_t slot = a.e_fd.div(rel0 + jr + e);  // (batch, channel) rows past row_first
+        if (a.table_full) {
+          uint32_t q;
+          a.c_fd.divmod(ch_first + slot, q, slot);
+        }
+        r.v[e] = bn_apply_one<T, MODE>(table + slot * NP, xv[u].v[e], MODE == kBnGradient ? gv[u].v[e] : (T)0);
+      }
+      *reinterpret_cast<V*>(out + j) = r;
+    }
+  }
+}
+
+// ---------------------------------------------------------------- host side
+
+struct BnPlan {
+  BnArgs a;
+  bool col_style;   // few elements per channel: lanes own columns of [batch, channels * elements]
+  bool vec_stats;
+  bool nt_stats;    // the operands exceed the caches: the statistics pass reads them with non-temporal loads
+  dim3 stats_grid;
+  size_t scratch_bytes;
+};
+
+constexpr int64_t kRowStyleMinBytes = 128;           // (batch, channel) rows at least this long are walked row style
+constexpr size_t kMaxPartialBytes = size_t(32) << 20;
+constexpr size_t kStreamingBytes = size_t(64) << 20;
+
+template <class T, int MODE>
+int bn_plan(hipStream_t s, int64_t B, int64_t C, int64_t E, const void* x, const void* og, void* out, bool need_stats,
+            BnPlan* plan) {
+  constexpr int NACC = bn_nacc<MODE>::value;
+  constexpr int VMAX = 16 / (int)sizeof(T);
+  CT_REQUIRE(B >= 1 && C >= 1 && E >= 1, "batch-normalize: batch, channel and element counts must be positive");
+  CT_REQUIRE(B < (int64_t(1) << 31) && C < (int64_t(1) << 30) && E < (int64_t(1) << 30),
+             "batch-normalize: a count exceeds the supported range");
+  CT_REQUIRE((double)B * (double)C * (double)E < 5.0e11, "batch-normalize: tensor too large");
+  BnArgs& a = plan->a;
+  std::memset(&a, 0, sizeof(a));
+  a.x = x; a.og = og; a.out = out;
+  a.B = B; a.C = C; a.E = E; a.W = C * E; a.N = B * C * E;
+  a.e_fd = FastDiv((uint32_t)E);
+  a.c_fd = FastDiv((uint32_t)C);
+  size_t partial_bytes = 0;
+  plan->col_style = E * (int64_t)sizeof(T) < kRowStyleMinBytes;
+  plan->vec_stats = false;
+  plan->nt_stats = (double)a.N * sizeof(T) * (og ? 2 : 1) >= (double)kStreamingBytes;
+  if (plan->col_style) CT_REQUIRE(a.W < (int64_t(1) << 31), "batch-normalize: channels * elements exceeds the supported range");
+  if (need_stats) {
+    const bool aligned = (uintptr_t)x % 16 == 0 && (og == nullptr || (uintptr_t)og % 16 == 0);
+    if (plan->col_style) {
+      plan->vec_stats = aligned && a.W % VMAX == 0;
+      const int vec = plan->vec_stats ? VMAX : 1;
+      const int64_t gx = (a.W + 64 * vec - 1) / (64 * vec);
+      int64_t S = std::max<int64_t>(1, std::min<int64_t>((B + 15) / 16, (1024 + gx - 1) / gx));
+      S = std::min<int64_t>(S, 65535);
+      while (S > 1 && (size_t)S * a.W * NACC * sizeof(double) > kMaxPartialBytes) S = (S + 1) / 2;
+      a.S = (uint32_t)S;
+      a.rows_per_seg = (uint32_t)((B + S - 1) / S);
+      a.part_E = (uint32_t)E;
+      plan->stats_grid = dim3((uint32_t)gx, (uint32_t)S);
+      partial_bytes = (size_t)S * a.W * NACC * sizeof(double);
+    } else {
+      // every row is walked in vectors; rows off the 16-byte grid take element-aligned loads and a partial last vector
+      plan->vec_stats = aligned && E % VMAX == 0;
+      a.nv = (uint32_t)((E + VMAX - 1) / VMAX);
+      a.nv_fd = FastDiv(a.nv);
+      int64_t S = std::max<int64_t>(1, std::min<int64_t>(B, (2048 + C - 1) / C));
+      // a block's list of vectors is indexed with 31 bits
+      while ((B + S - 1) / S * (int64_t)a.nv >= (int64_t(1) << 31)) S *= 2;
+      S = std::min(S, B);
+      a.S = (uint32_t)S;
+      a.rows_per_seg = (uint32_t)((B + S - 1) / S);
+      CT_REQUIRE((int64_t)a.rows_per_seg * a.nv < (int64_t(1) << 31) && C * S < (int64_t(1) << 31),
+                 "batch-normalize: tensor shape exceeds the supported range");
+      a.s_fd = FastDiv(a.S);
+      a.part_E = 1;
+      plan->stats_grid = dim3((uint32_t)(C * S));
+      partial_bytes = (size_t)S * C * NACC * sizeof(double);
+    }
+  }
+  const size_t param_bytes = (size_t)C * kParamStride * sizeof(double);
+  plan->scratch_bytes = param_bytes + partial_bytes;
+  void* scratch = nullptr;
+  if (int rc = stream_scratch(s, plan->scratch_bytes, &scratch)) return rc;
+  a.params = reinterpret_cast<double*>(scratch);
+  a.partials = reinterpret_cast<double*>(reinterpret_cast<char*>(scratch) + param_bytes);
+  return CT_OK;
+}
+
+template <class T, int MODE>
+void bn_launch_stats(hipStream_t s, const BnPlan& plan) {
+  constexpr int VMAX = 16 / (int)sizeof(T);
+  if (plan.col_style) {
+    if (plan.vec_stats) hipLaunchKernelGGL((bn_stats_col_kernel<T, VMAX, MODE>), plan.stats_grid, dim3(kBlock), 0, s, plan.a);
+    else hipLaunchKernelGGL((bn_stats_col_kernel<T, 1, MODE>), plan.stats_grid, dim3(kBlock), 0, s, plan.a);
+  } else {
+    if (plan.vec_stats && plan.nt_stats) hipLaunchKernelGGL((bn_stats_row_kernel<T, VMAX, MODE, true, true>), plan.stats_grid, dim3(kBlock), 0, s, plan.a);
+    else if (plan.vec_stats) hipLaunchKernelGGL((bn_stats_row_kernel<T, VMAX, MODE, true, false>), plan.stats_grid, dim3(kBlock), 0, s, plan.a);
+    else hipLaunchKernelGGL((bn_stats_row_kernel<T, VMAX, MODE, false, false>), plan.stats_grid, dim3(kBlock), 0, s, plan.a);
+  }
+}
+
+constexpr size_t kMaxTableBytes = size_t(60) << 10;
+
+template <class T, int VEC, int MODE, int UNROLL>
+bool bn_try_apply_range(hipStream_t s, BnArgs a, int64_t first, int64_t count) {
+  constexpr int NP = bn_nparam<MODE>::value;
+  constexpr int64_t kSpan = (int64_t)kBlock * VEC * UNROLL;
+  a.first = first;
+  a.count = count;
+  const int64_t window = (kSpan + a.E - 1) / a.E + 1;  // (batch, channel) rows a block's range can touch
+  a.table_full = window >= a.C ? 1u : 0u;
+  a.table_slots = (uint32_t)(a.table_full ? a.C : window);
+  const size_t lds = (size_t)a.table_slots * NP * sizeof(double);
+  if (lds > kMaxTableBytes) return false;
+  const dim3 grid((uint32_t)((count + kSpan - 1) / kSpan));
+  hipLaunchKernelGGL((bn_apply_kernel<T, VEC, MODE, UNROLL>), grid, dim3(kBlock), lds, s, a);
+  return true;
+}
+
+// Few elements per channel make the table of a wide block large: narrow the block then.
+template <class T, int VEC, int MODE>
+void bn_launch_apply_range(hipStream_t s, const BnArgs& a, int64_t first, int64_t count) {
+  if (count <= 0) return;
+  if (!bn_try_apply_range<T, VEC, MODE, kUnroll>(s, a, first, count)) bn_try_apply_range<T, VEC, MODE, 1>(s, a, first, count);
+}
+
+template <class T, int VEC, int MODE>
+void bn_launch_apply_col(hipStream_t s, BnArgs a) {
+  const int64_t gx = (a.W + (int64_t)kBlock * VEC - 1) / ((int64_t)kBlock * VEC);
+  int64_t segs = std::max<int64_t>(1, std::min<int64_t>((a.B + 3) / 4, (2048 + gx - 1) / gx));
+  segs = std::min<int64_t>(segs, 65535);
+  a.apply_rows_per_seg = (uint32_t)((a.B + segs - 1) / segs);
+  segs = (a.B + a.apply_rows_per_seg - 1) / a.apply_rows_per_seg;
+  hipLaunchKernelGGL((bn_apply_col_kernel<T, VEC, MODE>), dim3((uint32_t)gx, (uint32_t)segs), dim3(kBlock), 0, s, a);
+}
+
+template <class T, int MODE>
+void bn_launch_apply(hipStream_t s, const BnPlan& plan) {
+  constexpr int VMAX = 16 / (int)sizeof(T);
+  const BnArgs& a = plan.a;
+  const bool aligned = (uintptr_t)a.x % 16 == 0 && (uintptr_t)a.out % 16 == 0 &&
+                       (a.og == nullptr || (uintptr_t)a.og % 16 == 0);
+  if (plan.col_style) {
+    if (aligned && a.W % VMAX == 0) bn_launch_apply_col<T, VMAX, MODE>(s, a);
+    else bn_launch_apply_col<T, 1, MODE>(s, a);
+  } else if (aligned && VMAX > 1) {
+    const int64_t body = a.N / VMAX * VMAX;
+    bn_launch_apply_range<T, VMAX, MODE>(s, a, 0, body);
+    bn_launch_apply_range<T, 1, MODE>(s, a, body, a.N - body);
+  } else {
+    bn_launch_apply_range<T, 1, MODE>(s, a, 0, a.N);
+  }
+}
+
+inline dim3 channel_grid(int64_t C, int per_block) { return dim3((uint32_t)((C + per_block - 1) / per_block)); }
+
+template <class T>
+int bn_normalize(hipStream_t s, void* output, const void* input, const void* means, const void* variances,
+                 const void* scale, const void* bias, double epsilon, int64_t B, int64_t C, int64_t E) {
+  BnPlan plan;
+  if (int rc = bn_plan<T, kBnNormalize>(s, B, C, E, input, nullptr, output, false, &plan)) return rc;
+  note_kernel("bn_apply");
+  hipLaunchKernelGGL((bn_prepare_normalize_kernel<T>), channel_grid(C, kBlock), dim3(kBlock), 0, s, plan.a.params,
+                     (const T*)means, (const T*)variances, (const T*)scale, (const T*)bias, epsilon, C);
+  bn_launch_apply<T, kBnNormalize>(s, plan);
+  return after_launch(s);
+}
+
+template <class T>
+int bn_update_and_apply(hipStream_t s, void* output, const void* input, void* batch_means, void* batch_variances,
+                        void* running_means, void* running_variances, double average_factor, const void* scale,
+                        const void* bias, double epsilon, int64_t B, int64_t C, int64_t E) {
+  BnPlan plan;
+  if (int rc = bn_plan<T, kBnNormalize>(s, B, C, E, input, nullptr, output, true, &plan)) return rc;
+  note_kernel(plan.col_style ? "bn_update_col" : "bn_update_row");
+  bn_launch_stats<T, kBnNormalize>(s, plan);
+  BnFinish f;
+  std::memset(&f, 0, sizeof(f));
+  f.batch_means = batch_means; f.batch_variances = batch_variances;
+  f.running_means = running_means; f.running_variances = running_variances;
+  f.scale = scale; f.bias = bias;
+  f.average_factor = average_factor; f.epsilon = epsilon;
+  hipLaunchKernelGGL((bn_finish_kernel<T, kBnNormalize>), channel_grid(C, kBlock / 64), dim3(kBlock), 0, s, plan.a, f);
+  bn_launch_apply<T, kBnNormalize>(s, plan);
+  return after_launch(s);
+}
+
+template <class T>
+int bn_gradients(hipStream_t s, void* input_gradient, void* scale_gradient, void* bias_gradient,
+                 const void* output_gradient, const void* input, const void* batch_means, const void* batch_variances,
+                 const void* scale, double epsilon, int64_t B, int64_t C, int64_t E) {
+  BnPlan plan;
+  if (int rc = bn_plan<T, kBnGradient>(s, B, C, E, input, output_gradient, input_gradient, true, &plan)) return rc;
+  note_kernel(plan.col_style ? "bn_gradients_col" : "bn_gradients_row");
+  hipLaunchKernelGGL((bn_prepare_gradient_kernel<T>), channel_grid(C, kBlock), dim3(kBlock), 0, s, plan.a.params,
+                     (const T*)batch_means, (const T*)batch_variances, (const T*)scale, epsilon, C);
+  bn_launch_stats<T, kBnGradient>(s, plan);
+  BnFinish f;
+  std::memset(&f, 0, sizeof(f));
+  f.scale_gradient = scale_gradient; f.bias_gradient = bias_gradient;
+  hipLaunchKernelGGL((bn_finish_kernel<T, kBnGradient>), channel_grid(C, kBlock / 64), dim3(kBlock), 0, s, plan.a, f);
+  bn_launch_apply<T, kBnGradient>(s, plan);
+  return after_launch(s);
+}
+
+#define CT_BN_FLOAT(dtype, ...)                                                                               \
+  do {                                                                                                        \
+    if ((dtype) == CT_F32) { using T = float; return __VA_ARGS__; }                                           \
+    if ((dtype) == CT_F64) { using T = double; return __VA_ARGS__; }                                          \
+    return set_error(CT_ERR_INVALID, "batch-normalization is only defined for float and double tensors");     \
+  } while (0)
+
+}  // namespace
+
+extern "C" {
+
+int ct_batch_normalize_spatial(void* stream, void* output, const void* input, const void* means,
+                               const void* variances, const void* scale, const void* bias, double epsilon,
+                               int64_t batch_count, int64_t channel_count, int64_t element_count, int dtype) {
+  CT_REQUIRE(output && input && means && variances && scale && bias, "batch-normalize!: null buffer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CT_BN_FLOAT(dtype, bn_normalize<T>(s, output, input, means, variances, scale, bias, epsilon, batch_count,
+                                     channel_count, element_count));
+}
+
+int ct_batch_normalize_eltwise(void* stream, void* output, const void* input, const void* means,
+                               const void* variances, const void* scale, const void* bias, double epsilon,
+                               int64_t batch_count, int64_t element_count, int dtype) {
+  return ct_batch_normalize_spatial(stream, output, input, means, variances, scale, bias, epsilon, batch_count,
+                                    element_count, 1, dtype);
+}
+
+int ct_batch_normalize_update_and_apply_spatial(void* stream, void* output, const void* input, void* batch_means,
+                                                void* batch_variances, void* running_means,
+                                                void* running_variances, double average_factor, const void* scale,
+                                                const void* bias, double epsilon, int64_t batch_count,
+                                                int64_t channel_count, int64_t element_count, int dtype) {
+  CT_REQUIRE(output && input && batch_means && batch_variances && running_means && running_variances && scale && bias,
+             "batch-normalize-update-and-apply!: null buffer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CT_BN_FLOAT(dtype, bn_update_and_apply<T>(s, output, input, batch_means, batch_variances, running_means,
+                                            running_variances, average_factor, scale, bias, epsilon, batch_count,
+                                            channel_count, element_count));
+}
+
+int ct_batch_normalize_update_and_apply_eltwise(void* stream, void* output, const void* input, void* batch_means,
+                                                void* batch_variances, void* running_means,
+                                                void* running_variances, double average_factor, const void* scale,
+                                                const void* bias, double epsilon, int64_t batch_count,
+                                                int64_t element_count, int dtype) {
+  return ct_batch_normalize_update_and_apply_spatial(stream, output, input, batch_means, batch_variances,
+                                                     running_means, running_variances, average_factor, scale, bias,
+                                                     epsilon, batch_count, element_count, 1, dtype);
+}
+
+int ct_batch_normalize_gradients_spatial(void* stream, void* input_gradient, void* scale_gradient,
+                                         void* bias_gradient, const void* output_gradient, const void* output,
+                                         const void* input, const void* batch_means, const void* batch_variances,
+                                         const void* scale, const void* bias, double epsilon, int64_t batch_count,
+                                         int64_t channel_count, int64_t element_count, int dtype) {
+  (void)output;
+  (void)bias;
+  CT_REQUIRE(input_gradient && scale_gradient && bias_gradient && output_gradient && input && batch_means &&
+                 batch_variances && scale,
+             "batch-normalize-gradients!: null buffer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CT_BN_FLOAT(dtype, bn_gradients<T>(s, input_gradient, scale_gradient, bias_gradient, output_gradient, input,
+                                     batch_means, batch_variances, scale, epsilon, batch_count, channel_count,
+                                     element_count));
+}
+
+int ct_batch_normalize_gradients_eltwise(void* stream, void* input_gradient, void* scale_gradient,
+                                         void* bias_gradient, const void* output_gradient, const void* output,
+                                         const void* input, const void* batch_means, const void* batch_variances,
+                                         const void* scale, const void* bias, double epsilon, int64_t batch_count,
+                                         int64_t element_count, int dtype) {
+  return ct_batch_normalize_gradients_spatial(stream, input_gradient, scale_gradient, bias_gradient, output_gradient,
+                                              output, input, batch_means, batch_variances, scale, bias, epsilon,
+                                              batch_count, element_count, 1, dtype);
+}
+
+}  // extern "C"

@@ -298,6 +298,50 @@ class HipStream:
         capi.call("ct_softmax_spatial", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), input.ptr,
                   C.byref(_dims_struct(input_dims)), capi.DTYPE_CODES[output.datatype])
 
+    # -- batch normalization (tensor/math.clj:124-174); every buffer is packed --
+    def batch_normalize_eltwise(self, output, input, means, variances, scale, bias, epsilon, batch_count,
+                                element_count) -> None:
+        capi.call("ct_batch_normalize_eltwise", self.handle, output.ptr, input.ptr, means.ptr, variances.ptr,
+                  scale.ptr, bias.ptr, float(epsilon), int(batch_count), int(element_count),
+                  capi.DTYPE_CODES[output.datatype])
+
+    def batch_normalize_spatial(self, output, input, means, variances, scale, bias, epsilon, batch_count,
+                                channel_count, element_count) -> None:
+        capi.call("ct_batch_normalize_spatial", self.handle, output.ptr, input.ptr, means.ptr, variances.ptr,
+                  scale.ptr, bias.ptr, float(epsilon), int(batch_count), int(channel_count), int(element_count),
+                  capi.DTYPE_CODES[output.datatype])
+
+    def batch_normalize_update_and_apply_eltwise(self, output, input, batch_means, batch_variances, running_means,
+                                                 running_variances, average_factor, scale, bias, epsilon,
+                                                 batch_count, element_count) -> None:
+        capi.call("ct_batch_normalize_update_and_apply_eltwise", self.handle, output.ptr, input.ptr, batch_means.ptr,
+                  batch_variances.ptr, running_means.ptr, running_variances.ptr, float(average_factor), scale.ptr,
+                  bias.ptr, float(epsilon), int(batch_count), int(element_count), capi.DTYPE_CODES[output.datatype])
+
+    def batch_normalize_update_and_apply_spatial(self, output, input, batch_means, batch_variances, running_means,
+                                                 running_variances, average_factor, scale, bias, epsilon,
+                                                 batch_count, channel_count, element_count) -> None:
+        capi.call("ct_batch_normalize_update_and_apply_spatial", self.handle, output.ptr, input.ptr, batch_means.ptr,
+                  batch_variances.ptr, running_means.ptr, running_variances.ptr, float(average_factor), scale.ptr,
+                  bias.ptr, float(epsilon), int(batch_count), int(channel_count), int(element_count),
+                  capi.DTYPE_CODES[output.datatype])
+
+    def batch_normalize_gradients_eltwise(self, input_gradient, scale_gradient, bias_gradient, output_gradient,
+                                          output, input, batch_means, batch_variances, scale, bias, epsilon,
+                                          batch_count, element_count) -> None:
+        capi.call("ct_batch_normalize_gradients_eltwise", self.handle, input_gradient.ptr, scale_gradient.ptr,
+                  bias_gradient.ptr, output_gradient.ptr, output.ptr, input.ptr, batch_means.ptr, batch_variances.ptr,
+                  scale.ptr, bias.ptr, float(epsilon), int(batch_count), int(element_count),
+                  capi.DTYPE_CODES[input_gradient.datatype])
+
+    def batch_normalize_gradients_spatial(self, input_gradient, scale_gradient, bias_gradient, output_gradient,
+                                          output, input, batch_means, batch_variances, scale, bias, epsilon,
+                                          batch_count, channel_count, element_count) -> None:
+        capi.call("ct_batch_normalize_gradients_spatial", self.handle, input_gradient.ptr, scale_gradient.ptr,
+                  bias_gradient.ptr, output_gradient.ptr, output.ptr, input.ptr, batch_means.ptr, batch_variances.ptr,
+                  scale.ptr, bias.ptr, float(epsilon), int(batch_count), int(channel_count), int(element_count),
+                  capi.DTYPE_CODES[input_gradient.datatype])
+
     # -- optimizers ---------------------------------------------------------
     def adam_step(self, alpha, beta1, beta2, epsilon, pow_beta1_t, pow_beta2_t, gradient_alpha, gradient, parameters,
                   m, v, n) -> None:

@@ -513,6 +513,112 @@ def softmax(output: Tensor, input: Tensor) -> Tensor:
     return output
 
 
+# ---------------------------------------------------------------- batch normalization
+
+def _num_columns(t: Tensor) -> int:
+    return int(t.shape()[-1])
+
+
+def as_row_vector(t: Tensor) -> Tensor:
+    """``as-row-vector`` (``tensor.clj:307-314``)."""
+    if not (_num_columns(t) == 1 or dense(t)):
+        raise TensorError("Row vectors must either be dense or have num-columns = 1")
+    return t._with(dimensions=dims.dimensions([t.ecount()]))
+
+
+def _batch_normalize_setup(io_args, mvbs_args, epsilon):
+    """``batch-normalize-setup`` (``tensor.clj:1040-1099``).  Returns
+    (kind, row-vector statistics tensors, input shape).  The backends take
+    packed buffers (``tensor/math.clj:124-137``); the reference does not check
+    that, this mirror does."""
+    all_args = list(io_args) + list(mvbs_args)
+    inp = io_args[0]
+    input_shape = list(inp.shape())
+    if len(input_shape) == 1:
+        input_shape = [1, input_shape[0]]
+    _external_library_check("batch-normalize", *all_args)
+    if not float(epsilon) > 1e-5:
+        raise TensorError("Epsilon cannot be smaller than 1e-5 (cudnn limitation")
+    for t in mvbs_args:
+        if not (dense(t) or _num_columns(t) == 1):
+            raise TensorError("Argument is not vector-indexable")
+    vectors = [as_row_vector(t) for t in mvbs_args]
+    if len(input_shape) < 2:
+        raise TensorError("Input shape needs at least 2 dimensions")
+    if len({tuple(t.shape()) for t in io_args}) != 1:
+        raise TensorError("Tensor input and output shapes do not match")
+    if len({tuple(t.shape()) for t in vectors}) != 1:
+        raise TensorError("means, variances, scale, bias must have same shape")
+    if not all(dense(t) for t in all_args):
+        raise TensorError("batch-normalize: all tensors must be packed")
+    n_stats = vectors[0].shape()[0]
+    if len(input_shape) == 2:
+        if input_shape[1] != n_stats:
+            raise TensorError("Means, variances, scale, bias must match input element count.")
+        return "eltwise", vectors, input_shape
+    if input_shape[-2] != n_stats:
+        raise TensorError("means, variances, scale bias size must match input channel count")
+    return "spatial", vectors, input_shape
+
+
+def _bn_counts(input_shape):
+    batch_count = int(np.prod(input_shape[:-2], dtype=np.int64))
+    return batch_count, int(input_shape[-2]), int(input_shape[-1])
+
+
+def batch_normalize(output: Tensor, input: Tensor, means: Tensor, variances: Tensor, scale: Tensor, bias: Tensor,
+                    epsilon) -> Tensor:
+    """``batch-normalize!`` (``tensor.clj:1102-1147``):
+    output = (input - mean) / sqrt(variance + epsilon) * scale + bias, per
+    trailing element for two dimensions, per channel (second to last dimension)
+    for more."""
+    kind, (means, variances, scale, bias), input_shape = _batch_normalize_setup(
+        [output, input], [means, variances, scale, bias], epsilon)
+    stream = check_stream()
+    if kind == "eltwise":
+        stream.batch_normalize_eltwise(output.buffer, input.buffer, means.buffer, variances.buffer, scale.buffer,
+                                       bias.buffer, epsilon, input_shape[0], input_shape[1])
+    else:
+        stream.batch_normalize_spatial(output.buffer, input.buffer, means.buffer, variances.buffer, scale.buffer,
+                                       bias.buffer, epsilon, *_bn_counts(input_shape))
+    return output
+
+
+def batch_normalize_update_and_apply(output: Tensor, input: Tensor, batch_means: Tensor, batch_variances: Tensor,
+                                     running_means: Tensor, running_variances: Tensor, ave_factor, scale: Tensor,
+                                     bias: Tensor, epsilon):
+    """``batch-normalize-update-and-apply!`` (``tensor.clj:1149-1202``)."""
+    kind, vecs, input_shape = _batch_normalize_setup(
+        [output, input], [batch_means, batch_variances, running_means, running_variances, scale, bias], epsilon)
+    batch_means, batch_variances, running_means, running_variances, scale, bias = vecs
+    stream = check_stream()
+    bufs = (output.buffer, input.buffer, batch_means.buffer, batch_variances.buffer, running_means.buffer,
+            running_variances.buffer, ave_factor, scale.buffer, bias.buffer, epsilon)
+    if kind == "eltwise":
+        stream.batch_normalize_update_and_apply_eltwise(*bufs, input_shape[0], input_shape[1])
+    else:
+        stream.batch_normalize_update_and_apply_spatial(*bufs, *_bn_counts(input_shape))
+    return [output, batch_means, batch_variances, running_means, running_variances]
+
+
+def batch_normalize_gradients(input_gradient: Tensor, scale_gradient: Tensor, bias_gradient: Tensor,
+                              output_gradient: Tensor, output: Tensor, input: Tensor, batch_means: Tensor,
+                              batch_variances: Tensor, scale: Tensor, bias: Tensor, epsilon):
+    """``batch-normalize-gradients!`` (``tensor.clj:1205-1253``)."""
+    kind, vecs, input_shape = _batch_normalize_setup(
+        [output, input, output_gradient, input_gradient],
+        [batch_means, batch_variances, scale, bias, scale_gradient, bias_gradient], epsilon)
+    batch_means, batch_variances, scale, bias, scale_gradient, bias_gradient = vecs
+    stream = check_stream()
+    bufs = (input_gradient.buffer, scale_gradient.buffer, bias_gradient.buffer, output_gradient.buffer, output.buffer,
+            input.buffer, batch_means.buffer, batch_variances.buffer, scale.buffer, bias.buffer, epsilon)
+    if kind == "eltwise":
+        stream.batch_normalize_gradients_eltwise(*bufs, input_shape[0], input_shape[1])
+    else:
+        stream.batch_normalize_gradients_spatial(*bufs, *_bn_counts(input_shape))
+    return [input_gradient, scale_gradient, bias_gradient]
+
+
 # ---------------------------------------------------------------- composites
 
 def normalize(dest: Tensor, mag_vec: Tensor, radius_length, epsilon=1e-6) -> Tensor:

@@ -264,6 +264,63 @@ int ct_softmax_eltwise(void* stream, void* output, const ct_dims* output_dims, c
 int ct_softmax_spatial(void* stream, void* output, const ct_dims* output_dims, const void* input,
                        const ct_dims* input_dims, int dtype);
 
+/* Batch normalization.  Every buffer is packed: input and output hold
+ * batch_count x channel_count x element_count values (the eltwise forms have
+ * one element per channel: [batch_count, element_count] with a statistic per
+ * element), the statistics / scale / bias vectors hold channel_count values.
+ * dtype is CT_F32 or CT_F64.  The stream's scratch memory holds the partial
+ * sums between the passes. */
+
+/* batch-normalize-eltwise! / -spatial! (tensor/math.clj:124-137;
+ * cpu/tensor_math.clj:756-802):
+ *   output = (input - mean) * T(sqrt(1 / (variance + epsilon))) * scale + bias. */
+int ct_batch_normalize_eltwise(void* stream, void* output, const void* input, const void* means,
+                               const void* variances, const void* scale, const void* bias,
+                               double epsilon, int64_t batch_count, int64_t element_count, int dtype);
+int ct_batch_normalize_spatial(void* stream, void* output, const void* input, const void* means,
+                               const void* variances, const void* scale, const void* bias,
+                               double epsilon, int64_t batch_count, int64_t channel_count,
+                               int64_t element_count, int dtype);
+
+/* batch-normalize-update-and-apply-eltwise! / -spatial! (tensor/math.clj:138-156;
+ * cpu/tensor_math.clj:820-900, 1574-1608): batch_means = mean over the batch,
+ * batch_variances = population variance (divisor N),
+ * running = running * (1 - average_factor) + batch * average_factor, where the
+ * running variance takes the sample variance (divisor N - 1); then the
+ * normalization above with the batch statistics. */
+int ct_batch_normalize_update_and_apply_eltwise(void* stream, void* output, const void* input,
+                                                void* batch_means, void* batch_variances,
+                                                void* running_means, void* running_variances,
+                                                double average_factor, const void* scale,
+                                                const void* bias, double epsilon,
+                                                int64_t batch_count, int64_t element_count, int dtype);
+int ct_batch_normalize_update_and_apply_spatial(void* stream, void* output, const void* input,
+                                                void* batch_means, void* batch_variances,
+                                                void* running_means, void* running_variances,
+                                                double average_factor, const void* scale,
+                                                const void* bias, double epsilon,
+                                                int64_t batch_count, int64_t channel_count,
+                                                int64_t element_count, int dtype);
+
+/* batch-normalize-gradients-eltwise! / -spatial! (tensor/math.clj:157-174;
+ * cpu/tensor_math.clj:903-1033): input_gradient, scale_gradient and
+ * bias_gradient are written; `output` and `bias` are accepted for signature
+ * parity and not read (the CPU backend does not read them either).
+ * input_gradient may alias output_gradient. */
+int ct_batch_normalize_gradients_eltwise(void* stream, void* input_gradient, void* scale_gradient,
+                                         void* bias_gradient, const void* output_gradient,
+                                         const void* output, const void* input,
+                                         const void* batch_means, const void* batch_variances,
+                                         const void* scale, const void* bias, double epsilon,
+                                         int64_t batch_count, int64_t element_count, int dtype);
+int ct_batch_normalize_gradients_spatial(void* stream, void* input_gradient, void* scale_gradient,
+                                         void* bias_gradient, const void* output_gradient,
+                                         const void* output, const void* input,
+                                         const void* batch_means, const void* batch_variances,
+                                         const void* scale, const void* bias, double epsilon,
+                                         int64_t batch_count, int64_t channel_count,
+                                         int64_t element_count, int dtype);
+
 /* ------------------------------------------------- optimizers */
 
 /* Adam step (src/cortex/optimize/adam.clj:68-102, 116-134; resources/adam.cu).

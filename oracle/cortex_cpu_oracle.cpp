@@ -21,6 +21,7 @@
 //   unary-reduce!            cpu/tensor_math.clj:582-663
 //   activation-gradient!     cpu/tensor_math.clj:1318-1362
 //   softmax (both forms)     cpu/tensor_math.clj:1037-1103
+//   batch-normalize (6 forms) cpu/tensor_math.clj:731-1033, 1558-1638
 //   Adam                     src/cortex/optimize/adam.clj:68-102
 //   Adadelta                 java/cortex/compute/optimize/AdadeltaOptimizer.java:29-64
 //
@@ -36,6 +37,7 @@
 // narrowing casts truncate.  Each JVM operation rounds separately (no FMA), so
 // this file is compiled with -ffp-contract=off.
 
+#include <algorithm>
 #include <cmath>
 #ifdef _OPENMP
 #include <omp.h>
@@ -587,6 +589,122 @@ inline bool transpose_021(const Dims& d, Dims* t) {
   return true;
 }
 
+// ---------------------------------------------------------------- batch normalization
+// BNEltwiseOffsetter / BNSpatialOffsetter (cpu/tensor_math.clj:737-753): the
+// "parallel" index selects the statistic (an element, or a channel), the other
+// index walks the values that share it.  The eltwise form is the spatial form
+// with one element per channel.
+struct BnOffsetter {
+  int64_t batch, channels, elements;
+  int64_t parallel_count() const { return channels; }
+  int64_t idx_count() const { return batch * elements; }
+  int64_t operator()(int64_t c, int64_t i) const {
+    return (i % elements) + c * elements + (i / elements) * (channels * elements);
+  }
+};
+
+// sum-double-var (cpu/tensor_math.clj:805-817): a sequential double sum seeded
+// with the first term.
+template <class F> inline double sum_double_var(int64_t n, F term) {
+  if (n == 0) return 0.0;
+  double s = term((int64_t)0);
+  for (int64_t i = 1; i < n; ++i) s = s + term(i);
+  return s;
+}
+
+// batch-normalize-impl (cpu/tensor_math.clj:756-784).  inv-std-dev is rounded
+// to T; the per-element arithmetic runs in double and the store rounds once.
+template <class T>
+void bn_apply_t(const BnOffsetter& o, T* out, const T* in, const T* means, const T* variances, const T* scale,
+                const T* bias, double epsilon_) {
+  const T epsilon = (T)epsilon_;
+  const int64_t pc = o.parallel_count(), ic = o.idx_count();
+#pragma omp parallel for schedule(static)
+  for (int64_t c = 0; c < pc; ++c) {
+    const T variance = variances[c];
+    const T inv_std_dev = (T)std::sqrt(1.0 / ((double)variance + (double)epsilon));
+    const T mean = means[c], sc = scale[c], shift = bias[c];
+    for (int64_t i = 0; i < ic; ++i) {
+      const int64_t off = o(c, i);
+      const double x_hat = ((double)in[off] - (double)mean) * (double)inv_std_dev;
+      out[off] = (T)(x_hat * (double)sc + (double)shift);
+    }
+  }
+}
+
+// batch-normalize-update-impl (cpu/tensor_math.clj:820-870).
+template <class T>
+void bn_update_t(const BnOffsetter& o, const T* in, T* batch_means, T* batch_variances, T* running_means,
+                 T* running_variances, double average_factor) {
+  const T ave_factor = (T)average_factor;
+  const double ave_lerp = (double)(T)1.0 - (double)ave_factor;
+  const int64_t pc = o.parallel_count(), ic = o.idx_count();
+  const double count_val = std::max(1.0, (double)ic);
+  const double running_count_val = std::max(1.0, count_val - 1.0);
+#pragma omp parallel for schedule(static)
+  for (int64_t c = 0; c < pc; ++c) {
+    const T variance = running_variances[c], mean = running_means[c];
+    const T new_mean = (T)(sum_double_var(ic, [&](int64_t i) { return (double)in[o(c, i)]; }) / count_val);
+    const double new_var = sum_double_var(ic, [&](int64_t i) {
+      const double mean_diff = (double)new_mean - (double)in[o(c, i)];
+      return mean_diff * mean_diff;
+    });
+    batch_means[c] = new_mean;
+    batch_variances[c] = (T)(new_var / count_val);
+    running_means[c] = (T)((double)mean * ave_lerp + (double)new_mean * (double)ave_factor);
+    running_variances[c] =
+        (T)((double)variance * ave_lerp + (double)(T)(new_var / running_count_val) * (double)ave_factor);
+  }
+}
+
+// batch-normalize-gradients-impl (cpu/tensor_math.clj:903-1001).  The scaled
+// output gradient is parked, rounded to T, in the input-gradient buffer and
+// read back from there (:956-960); `output` and `bias` are not read.
+template <class T>
+void bn_gradients_t(const BnOffsetter& o, T* input_gradient, T* scale_gradient, T* bias_gradient,
+                    const T* output_gradient, const T* in, const T* means, const T* variances, const T* scale,
+                    double epsilon_) {
+  const T pow_factor = (T)(-3.0 / 2.0);
+  const T epsilon = (T)epsilon_;
+  const int64_t pc = o.parallel_count(), ic = o.idx_count();
+#pragma omp parallel for schedule(static)
+  for (int64_t c = 0; c < pc; ++c) {
+    const T sc = scale[c];
+    const double variance = (double)epsilon + (double)variances[c];
+    const double inv_std_dev = 1.0 / std::sqrt(variance);
+    const T mean = means[c];
+    const T d_var = (T)(-0.5 * std::pow(variance, (double)pow_factor));
+    bias_gradient[c] = (T)sum_double_var(ic, [&](int64_t i) { return (double)output_gradient[o(c, i)]; });
+    scale_gradient[c] = (T)sum_double_var(ic, [&](int64_t i) {
+      const int64_t off = o(c, i);
+      return (double)output_gradient[off] * (((double)in[off] - (double)mean) * inv_std_dev);
+    });
+    for (int64_t i = 0; i < ic; ++i) {
+      const int64_t off = o(c, i);
+      input_gradient[off] = (T)((double)sc * (double)output_gradient[off]);
+    }
+    const T d_var_d_out = (T)sum_double_var(ic, [&](int64_t i) {
+      const int64_t off = o(c, i);
+      return ((double)input_gradient[off] * ((double)in[off] - (double)mean)) * (double)d_var;
+    });
+    const T d_mean_d_out = (T)(
+        sum_double_var(ic, [&](int64_t i) { return (-(double)input_gradient[o(c, i)]) * inv_std_dev; }) +
+        (double)d_var_d_out *
+            (sum_double_var(ic, [&](int64_t i) { return -2.0 * ((double)in[o(c, i)] - (double)mean); }) /
+             (double)ic));
+    for (int64_t i = 0; i < ic; ++i) {
+      const int64_t off = o(c, i);
+      const double d_x_hat_d_out = (double)input_gradient[off];
+      const double input_var = (double)in[off];
+      const double one_over_index_count = 1.0 / (double)ic;
+      const double sum_part_1 = d_x_hat_d_out * inv_std_dev;
+      const double sum_part_2 = (((double)d_var_d_out * 2.0) * (input_var - (double)mean)) * one_over_index_count;
+      const double sum_part_3 = (double)d_mean_d_out * one_over_index_count;
+      input_gradient[off] = (T)((sum_part_1 + sum_part_2) + sum_part_3);
+    }
+  }
+}
+
 // cpu-adam-step-impl! (adam.clj:68-102).  The scalars are cast to the datatype
 // first; the arithmetic then runs in double.
 template <class T>
@@ -839,6 +957,86 @@ int co_softmax_spatial(void* output, const ct_dims* output_dims, const void* inp
   if (dtype == CT_F32) return softmax_t<float>((float*)output, odt, (const float*)input, idt);
   if (dtype == CT_F64) return softmax_t<double>((double*)output, odt, (const double*)input, idt);
   return fail("softmax! is only defined for float and double tensors");
+}
+
+static bool bn_counts_ok(int64_t b, int64_t c, int64_t e) { return b >= 1 && c >= 1 && e >= 1; }
+
+#define BN_FLOAT_DISPATCH(dtype, ...)                                               \
+  if ((dtype) == CT_F32) { using T = float; __VA_ARGS__; }                          \
+  else if ((dtype) == CT_F64) { using T = double; __VA_ARGS__; }                    \
+  else return fail("batch-normalization is only defined for float and double tensors")
+
+// batch-normalize-spatial! (cpu/tensor_math.clj:1566-1572); the eltwise form
+// (:1558-1564) is the same with one element per channel.
+int co_batch_normalize_spatial(void* output, const void* input, const void* means, const void* variances,
+                               const void* scale, const void* bias, double epsilon, int64_t batch_count,
+                               int64_t channel_count, int64_t element_count, int dtype) {
+  if (!bn_counts_ok(batch_count, channel_count, element_count)) return fail("batch-normalize: counts must be positive");
+  const BnOffsetter o{batch_count, channel_count, element_count};
+  BN_FLOAT_DISPATCH(dtype, bn_apply_t<T>(o, (T*)output, (const T*)input, (const T*)means, (const T*)variances,
+                                         (const T*)scale, (const T*)bias, epsilon));
+  return 0;
+}
+
+int co_batch_normalize_eltwise(void* output, const void* input, const void* means, const void* variances,
+                               const void* scale, const void* bias, double epsilon, int64_t batch_count,
+                               int64_t element_count, int dtype) {
+  return co_batch_normalize_spatial(output, input, means, variances, scale, bias, epsilon, batch_count,
+                                    element_count, 1, dtype);
+}
+
+// batch-normalize-update-and-apply-spatial! (cpu/tensor_math.clj:1592-1608):
+// the update, then the plain normalization with the batch statistics.
+int co_batch_normalize_update_and_apply_spatial(void* output, const void* input, void* batch_means,
+                                                void* batch_variances, void* running_means,
+                                                void* running_variances, double average_factor, const void* scale,
+                                                const void* bias, double epsilon, int64_t batch_count,
+                                                int64_t channel_count, int64_t element_count, int dtype) {
+  if (!bn_counts_ok(batch_count, channel_count, element_count)) return fail("batch-normalize: counts must be positive");
+  const BnOffsetter o{batch_count, channel_count, element_count};
+  BN_FLOAT_DISPATCH(dtype, {
+    bn_update_t<T>(o, (const T*)input, (T*)batch_means, (T*)batch_variances, (T*)running_means,
+                   (T*)running_variances, average_factor);
+    bn_apply_t<T>(o, (T*)output, (const T*)input, (const T*)batch_means, (const T*)batch_variances,
+                  (const T*)scale, (const T*)bias, epsilon);
+  });
+  return 0;
+}
+
+int co_batch_normalize_update_and_apply_eltwise(void* output, const void* input, void* batch_means,
+                                                void* batch_variances, void* running_means,
+                                                void* running_variances, double average_factor, const void* scale,
+                                                const void* bias, double epsilon, int64_t batch_count,
+                                                int64_t element_count, int dtype) {
+  return co_batch_normalize_update_and_apply_spatial(output, input, batch_means, batch_variances, running_means,
+                                                     running_variances, average_factor, scale, bias, epsilon,
+                                                     batch_count, element_count, 1, dtype);
+}
+
+// batch-normalize-gradients-spatial! (cpu/tensor_math.clj:1624-1638)
+int co_batch_normalize_gradients_spatial(void* input_gradient, void* scale_gradient, void* bias_gradient,
+                                         const void* output_gradient, const void* output, const void* input,
+                                         const void* batch_means, const void* batch_variances, const void* scale,
+                                         const void* bias, double epsilon, int64_t batch_count,
+                                         int64_t channel_count, int64_t element_count, int dtype) {
+  (void)output;
+  (void)bias;
+  if (!bn_counts_ok(batch_count, channel_count, element_count)) return fail("batch-normalize: counts must be positive");
+  const BnOffsetter o{batch_count, channel_count, element_count};
+  BN_FLOAT_DISPATCH(dtype, bn_gradients_t<T>(o, (T*)input_gradient, (T*)scale_gradient, (T*)bias_gradient,
+                                             (const T*)output_gradient, (const T*)input, (const T*)batch_means,
+                                             (const T*)batch_variances, (const T*)scale, epsilon));
+  return 0;
+}
+
+int co_batch_normalize_gradients_eltwise(void* input_gradient, void* scale_gradient, void* bias_gradient,
+                                         const void* output_gradient, const void* output, const void* input,
+                                         const void* batch_means, const void* batch_variances, const void* scale,
+                                         const void* bias, double epsilon, int64_t batch_count,
+                                         int64_t element_count, int dtype) {
+  return co_batch_normalize_gradients_spatial(input_gradient, scale_gradient, bias_gradient, output_gradient, output,
+                                              input, batch_means, batch_variances, scale, bias, epsilon, batch_count,
+                                              element_count, 1, dtype);
 }
 
 int co_adam_step(int dtype, double alpha, double beta1, double beta2, double epsilon,

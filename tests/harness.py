@@ -227,6 +227,42 @@ def softmax(side, out: View, inp: View, spatial=False):
     side.call("softmax_spatial" if spatial else "softmax_eltwise", *_pd(side, out), *_pd(side, inp), out.buf.dtype)
 
 
+def batch_normalize(side, out: View, inp: View, means: View, variances: View, scale: View, bias: View, epsilon,
+                    batch, channels, elements=None):
+    """elements=None selects the eltwise form ([batch, channels] with one statistic per element)."""
+    ptrs = [side.ptr(v) for v in (out, inp, means, variances, scale, bias)]
+    if elements is None:
+        side.call("batch_normalize_eltwise", *ptrs, float(epsilon), batch, channels, out.buf.dtype)
+    else:
+        side.call("batch_normalize_spatial", *ptrs, float(epsilon), batch, channels, elements, out.buf.dtype)
+
+
+def batch_normalize_update_and_apply(side, out: View, inp: View, batch_means: View, batch_variances: View,
+                                     running_means: View, running_variances: View, average_factor, scale: View,
+                                     bias: View, epsilon, batch, channels, elements=None):
+    head = [side.ptr(v) for v in (out, inp, batch_means, batch_variances, running_means, running_variances)]
+    tail = [side.ptr(scale), side.ptr(bias), float(epsilon), batch, channels]
+    if elements is None:
+        side.call("batch_normalize_update_and_apply_eltwise", *head, float(average_factor), *tail, out.buf.dtype)
+    else:
+        side.call("batch_normalize_update_and_apply_spatial", *head, float(average_factor), *tail, elements,
+                  out.buf.dtype)
+
+
+def batch_normalize_gradients(side, input_gradient: View, scale_gradient: View, bias_gradient: View,
+                              output_gradient: View, output: View, inp: View, batch_means: View,
+                              batch_variances: View, scale: View, bias: View, epsilon, batch, channels,
+                              elements=None):
+    ptrs = [side.ptr(v) for v in (input_gradient, scale_gradient, bias_gradient, output_gradient, output, inp,
+                                  batch_means, batch_variances, scale, bias)]
+    if elements is None:
+        side.call("batch_normalize_gradients_eltwise", *ptrs, float(epsilon), batch, channels,
+                  input_gradient.buf.dtype)
+    else:
+        side.call("batch_normalize_gradients_spatial", *ptrs, float(epsilon), batch, channels, elements,
+                  input_gradient.buf.dtype)
+
+
 def adam_step(side, alpha, beta1, beta2, eps, pb1, pb2, ga, grad: View, params: View, m: View, v: View, n):
     args = (grad.buf.dtype, float(alpha), float(beta1), float(beta2), float(eps), float(pb1), float(pb2), float(ga),
             side.ptr(grad), side.ptr(params), side.ptr(m), side.ptr(v), n)

@@ -163,6 +163,32 @@ class OracleStream:
         ob.call("softmax_spatial", out.ptr, C.byref(_dims(od)), inp.ptr, C.byref(_dims(idims)),
                 capi.DTYPE_CODES[out.datatype])
 
+    def batch_normalize_eltwise(self, out, inp, means, variances, scale, bias, eps, batch, elems):
+        ob.call("batch_normalize_eltwise", out.ptr, inp.ptr, means.ptr, variances.ptr, scale.ptr, bias.ptr, float(eps),
+                int(batch), int(elems), capi.DTYPE_CODES[out.datatype])
+
+    def batch_normalize_spatial(self, out, inp, means, variances, scale, bias, eps, batch, chans, elems):
+        ob.call("batch_normalize_spatial", out.ptr, inp.ptr, means.ptr, variances.ptr, scale.ptr, bias.ptr, float(eps),
+                int(batch), int(chans), int(elems), capi.DTYPE_CODES[out.datatype])
+
+    def batch_normalize_update_and_apply_eltwise(self, out, inp, bm, bv, rm, rv, af, scale, bias, eps, batch, elems):
+        ob.call("batch_normalize_update_and_apply_eltwise", out.ptr, inp.ptr, bm.ptr, bv.ptr, rm.ptr, rv.ptr, float(af),
+                scale.ptr, bias.ptr, float(eps), int(batch), int(elems), capi.DTYPE_CODES[out.datatype])
+
+    def batch_normalize_update_and_apply_spatial(self, out, inp, bm, bv, rm, rv, af, scale, bias, eps, batch, chans,
+                                                 elems):
+        ob.call("batch_normalize_update_and_apply_spatial", out.ptr, inp.ptr, bm.ptr, bv.ptr, rm.ptr, rv.ptr, float(af),
+                scale.ptr, bias.ptr, float(eps), int(batch), int(chans), int(elems), capi.DTYPE_CODES[out.datatype])
+
+    def batch_normalize_gradients_eltwise(self, ig, sg, bg, og, out, inp, bm, bv, scale, bias, eps, batch, elems):
+        ob.call("batch_normalize_gradients_eltwise", ig.ptr, sg.ptr, bg.ptr, og.ptr, out.ptr, inp.ptr, bm.ptr, bv.ptr,
+                scale.ptr, bias.ptr, float(eps), int(batch), int(elems), capi.DTYPE_CODES[ig.datatype])
+
+    def batch_normalize_gradients_spatial(self, ig, sg, bg, og, out, inp, bm, bv, scale, bias, eps, batch, chans,
+                                          elems):
+        ob.call("batch_normalize_gradients_spatial", ig.ptr, sg.ptr, bg.ptr, og.ptr, out.ptr, inp.ptr, bm.ptr, bv.ptr,
+                scale.ptr, bias.ptr, float(eps), int(batch), int(chans), int(elems), capi.DTYPE_CODES[ig.datatype])
+
     def adam_step(self, alpha, beta1, beta2, eps, pb1, pb2, ga, gradient, parameters, m, v, n):
         ob.call("adam_step", capi.DTYPE_CODES[gradient.datatype], float(alpha), float(beta1), float(beta2), float(eps),
                 float(pb1), float(pb2), float(ga), gradient.ptr, parameters.ptr, m.ptr, v.ptr, int(n))

@@ -246,6 +246,120 @@ def softmax(driver, datatype):
         equals(([0, 1] + list(ct.to_double_array(answer))) * 5, ct.to_double_array(pred_matrix))
 
 
+BN_ELTWISE_OUT = [-26.0, 4.0, 6.116036847575795, 64.0, 12.955334711889902, 12.46414739030318, 154.0,
+                  21.910669423779805, 18.812257933030565, 244.0, 30.86600413566971, 25.16036847575795]
+BN_SPATIAL_OUT = [-26.0, 4.0, 34.0, 64.0, 12.955334711889902, 15.94044628251987, 18.925557853149837,
+                  21.910669423779805, 18.812257933030565, 20.92829478060636, 23.044331628182157, 25.16036847575795,
+                  334.0, 364.0, 394.0, 424.0, 48.77667355944951, 51.76178513007948, 54.74689670070945,
+                  57.73200827133942, 44.204700103940105, 46.3207369515159, 48.436773799091696, 50.55281064666749]
+BN_UPDATE_ELTWISE_OUT = [-0.023134696804511745] * 3 + [2.6589551010651626] * 3 + [5.341044898934837] * 3 + \
+                        [8.023134696804512] * 3
+BN_UPDATE_SPATIAL_OUT = [0.3139510961275713, 0.8054242833105618, 1.2968974704935523, 1.7883706576765428] * 3 + \
+                        [6.211629342323457, 6.703102529506448, 7.194575716689438, 7.686048903872429] * 3
+
+
+def _spatial_input():
+    return ct.to_tensor(partition(3, partition(4, range(24))))
+
+
+# verify/tensor.clj:309-348
+def batch_normalize(driver, datatype):
+    with context(driver, datatype):
+        # eltwise; a variance of 0 is included to sniff out the edge case
+        inp = ct.to_tensor(partition(3, range(12)))
+        output = ct.new_tensor([4, 3])
+        means, variances = ct.to_tensor([1] * 3), ct.to_tensor(range(3))
+        scale, bias = ct.to_tensor([3] * 3), ct.to_tensor([4] * 3)
+        ct.batch_normalize(output, inp, means, variances, scale, bias, 1e-2)
+        equals(BN_ELTWISE_OUT, ct.to_double_array(output), 1e-4)
+        # spatial
+        inp = _spatial_input()
+        output = ct.new_tensor([2, 3, 4])
+        means, variances = ct.to_tensor([1] * 3), ct.to_tensor(range(3))
+        scale, bias = ct.to_tensor([3] * 3), ct.to_tensor([4] * 3)
+        ct.batch_normalize(output, inp, means, variances, scale, bias, 1e-2)
+        equals(BN_SPATIAL_OUT, ct.to_double_array(output), 1e-4)
+
+
+# verify/tensor.clj:350-429
+def batch_normalize_update_and_apply(driver, datatype):
+    with context(driver, datatype):
+        inp = ct.to_tensor(partition(3, range(12)))
+        output = ct.new_tensor([4, 3])
+        means, variances = ct.to_tensor([1] * 3), ct.to_tensor(range(3))
+        running_means, running_variances = ct.to_tensor([2] * 3), ct.to_tensor([4] * 3)
+        scale, bias = ct.to_tensor([3] * 3), ct.to_tensor([4] * 3)
+        ct.batch_normalize_update_and_apply(output, inp, means, variances, running_means, running_variances, 0.8,
+                                            scale, bias, 1e-2)
+        equals(BN_UPDATE_ELTWISE_OUT, ct.to_double_array(output), 1e-4)
+        equals([4.5, 5.5, 6.5], ct.to_double_array(means), 1e-4)
+        # the reference leaves the batch variances unchecked (cuDNN stores them as 1/sqrt); the
+        # CPU backend's value is the population variance
+        equals([11.25] * 3, ct.to_double_array(variances), 1e-4)
+        equals([4.0, 4.8, 5.6000000000000005], ct.to_double_array(running_means), 1e-4)
+        equals([12.8, 12.8, 12.8], ct.to_double_array(running_variances), 1e-4)
+        # spatial
+        inp = _spatial_input()
+        output = ct.new_tensor([2, 3, 4])
+        means, variances = ct.to_tensor([1] * 3), ct.to_tensor(range(3))
+        running_means, running_variances = ct.to_tensor([2] * 3), ct.to_tensor([4] * 3)
+        scale, bias = ct.to_tensor([3] * 3), ct.to_tensor([4] * 3)
+        ct.batch_normalize_update_and_apply(output, inp, means, variances, running_means, running_variances, 0.8,
+                                            scale, bias, 1e-2)
+        equals(BN_UPDATE_SPATIAL_OUT, ct.to_double_array(output), 1e-4)
+        equals([7.5, 11.5, 15.5], ct.to_double_array(means), 1e-4)
+        equals([6.4, 9.6, 12.8], ct.to_double_array(running_means), 1e-4)
+        equals([34.857142857142854] * 3, ct.to_double_array(running_variances), 1e-4)
+
+
+# verify/tensor.clj:432-529
+def batch_normalize_gradients(driver, datatype):
+    with context(driver, datatype):
+        inp = ct.to_tensor(partition(3, range(12)))
+        output = ct.to_tensor(partition(3, BN_ELTWISE_OUT))
+        input_gradient = ct.new_tensor([4, 3])
+        output_gradient = ct.to_tensor(partition(3, range(12)))
+        batch_means, batch_variances = ct.to_tensor([1] * 3), ct.to_tensor(range(3))
+        running_means, running_variances = ct.to_tensor([2] * 3), ct.to_tensor([4] * 3)
+        scale, bias = ct.to_tensor([3] * 3), ct.to_tensor([4] * 3)
+        scale_gradient, bias_gradient = ct.new_tensor([3]), ct.new_tensor([3])
+        ct.batch_normalize_update_and_apply(output, inp, batch_means, batch_variances, running_means,
+                                            running_variances, 0.8, scale, bias, 1e-2)
+        ct.batch_normalize_gradients(input_gradient, scale_gradient, bias_gradient, output_gradient, output, inp,
+                                     batch_means, batch_variances, scale, bias, 1e-2)
+        equals(BN_UPDATE_ELTWISE_OUT, ct.to_double_array(output), 1e-4)
+        equals([-0.003572943780465465, -0.003572943780465465, -0.003572943780465465,
+                -0.001190981260155155, -0.001190981260154711, -0.001190981260154489,
+                0.001190981260154933, 0.001190981260155155, 0.0011909812601555991,
+                0.0035729437804663533, 0.0035729437804663533, 0.0035729437804663533],
+               ct.to_double_array(input_gradient), 1e-4)
+        equals([13.410448989348373] * 3, ct.to_double_array(scale_gradient), 1e-4)
+        equals([18, 22, 26], ct.to_double_array(bias_gradient), 1e-4)
+        # spatial
+        inp = _spatial_input()
+        output = ct.new_tensor([2, 3, 4])
+        input_gradient = ct.new_tensor([2, 3, 4])
+        output_gradient = _spatial_input()
+        batch_means, batch_variances = ct.to_tensor([1] * 3), ct.to_tensor(range(3))
+        running_means, running_variances = ct.to_tensor([2] * 3), ct.to_tensor([4] * 3)
+        scale, bias = ct.to_tensor([3] * 3), ct.to_tensor([4] * 3)
+        scale_gradient, bias_gradient = ct.new_tensor([3]), ct.new_tensor([3])
+        ct.batch_normalize_update_and_apply(output, inp, batch_means, batch_variances, running_means,
+                                            running_variances, 0.8, scale, bias, 1e-2)
+        ct.batch_normalize_gradients(input_gradient, scale_gradient, bias_gradient, output_gradient, output, inp,
+                                     batch_means, batch_variances, scale, bias, 1e-2)
+        equals(BN_UPDATE_SPATIAL_OUT, ct.to_double_array(output), 1e-4)
+        equals([-9.892777519776665E-4, -8.57374051714065E-4, -7.254703514504634E-4, -5.935666511868618E-4,
+                -9.89277751978103E-4, -8.57374051714065E-4, -7.254703514500268E-4, -5.935666511868618E-4,
+                -9.89277751978103E-4, -8.57374051714065E-4, -7.254703514500268E-4, -5.935666511868618E-4,
+                5.935666511868618E-4, 7.254703514504634E-4, 8.57374051714065E-4, 9.892777519776665E-4,
+                5.935666511868618E-4, 7.254703514500268E-4, 8.57374051714065E-4, 9.89277751978103E-4,
+                5.935666511868618E-4, 7.254703514500268E-4, 8.57374051714065E-4, 9.89277751978103E-4],
+               ct.to_double_array(input_gradient), 1e-6)
+        equals([48.81966992684372] * 3, ct.to_double_array(scale_gradient), 1e-4)
+        equals([60.0, 92.0, 124.0], ct.to_double_array(bias_gradient), 1e-4)
+
+
 # verify/tensor.clj:623-645
 def ternary_op_select(driver, datatype):
     with context(driver, datatype):

@@ -616,3 +616,110 @@ def test_softmax_and_activation_gradient_errors(P):
         H.softmax(P.hip, View(x, [4, 4]), View(x, [2, 8]))
     with pytest.raises(capi.CortexHipError, match="float and double"):
         H.activation_gradient(P.hip, View(xi, [16]), View(xi, [16]), View(xi, [16]), "relu", 16)
+
+
+# ------------------------------------------------------------------ batch normalization
+# Layouts: (batch, channels) is the eltwise form, (batch, channels, elements) the spatial one.
+# They cover both statistics kernels (rows of at least 128 bytes are walked row style), vector
+# and scalar accesses, table-per-window and table-of-all-channels apply passes, and tails.
+BN_SHAPES = [(4, 3), (128, 1000), (37, 130), (1000, 64), (5, 4099), (2, 3, 4), (8, 16, 196), (4, 5, 49),
+             (3, 7, 1024), (16, 3, 4100), (2, 2, 31), (70, 33, 8), (2, 3000, 4), (33, 6, 1000), (1, 4, 64)]
+
+
+def bn_close(buf, what, code, scale_by=None):
+    """|got - want| <= tol * max|want|: the sums are taken in another order than the CPU
+    backend's left-to-right walk, so values that cancel are compared on the tensor's scale."""
+    tol = REL_TOL if code == capi.F32 else REL_TOL_F64
+    got, want = buf.download().astype(np.float64), buf.host.astype(np.float64)
+    scale = np.max(np.abs(want)) if scale_by is None else scale_by
+    err = np.max(np.abs(got - want))
+    assert err <= tol * max(scale, 1e-30), f"{what}: max abs err {err} on scale {scale}"
+
+
+def bn_setup(P, rng, code, shape):
+    b, c = shape[0], shape[1]
+    e = shape[2] if len(shape) == 3 else None
+    n = b * c * (e or 1)
+    f = NP[code]
+    t = dict(
+        x=P.buf((rng.standard_normal(n) * 2 + 5).astype(f)), out=P.buf(np.zeros(n, f)),
+        og=P.buf(rng.standard_normal(n).astype(f)), ig=P.buf(np.zeros(n, f)),
+        means=P.buf(rng.standard_normal(c).astype(f)), variances=P.buf(rng.uniform(0, 3, c).astype(f)),
+        rmeans=P.buf(rng.standard_normal(c).astype(f)), rvars=P.buf(rng.uniform(0.5, 2, c).astype(f)),
+        scale=P.buf(rng.uniform(0.5, 1.5, c).astype(f)), bias=P.buf(rng.standard_normal(c).astype(f)),
+        sg=P.buf(np.zeros(c, f)), bg=P.buf(np.zeros(c, f)))
+    V = {k: View(v, [v.init.size]) for k, v in t.items()}
+    return t, V, (b, c, e)
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("shape", BN_SHAPES, ids=str)
+def test_batch_normalize(P, code, shape):
+    rng = np.random.default_rng(40)
+    t, V, (b, c, e) = bn_setup(P, rng, code, shape)
+    t["variances"].init[0] = 0.0          # the reference's edge case
+    t["variances"].reset()
+    k = P.run(H.batch_normalize, V["out"], V["x"], V["means"], V["variances"], V["scale"], V["bias"], 1e-2, b, c, e)
+    compare(t["out"], f"batch-normalize {shape} ({k})")      # elementwise in the CPU backend's order: bit-exact
+    P.run(H.batch_normalize, V["x"], V["x"], V["means"], V["variances"], V["scale"], V["bias"], 1e-2, b, c, e)
+    compare(t["x"], f"batch-normalize {shape} in place")
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("shape", BN_SHAPES, ids=str)
+def test_batch_normalize_update_and_gradients(P, code, shape):
+    rng = np.random.default_rng(41)
+    t, V, (b, c, e) = bn_setup(P, rng, code, shape)
+    x64 = t["x"].init.astype(np.float64)
+    k = P.run(H.batch_normalize_update_and_apply, V["out"], V["x"], V["means"], V["variances"], V["rmeans"],
+              V["rvars"], 0.8, V["scale"], V["bias"], 1e-3, b, c, e)
+    assert k == ("bn_update_row" if (e or 1) * t["x"].init.itemsize >= 128 else "bn_update_col")
+    what = f"batch-normalize-update-and-apply {shape} ({k})"
+    bn_close(t["means"], what + " batch means", code, scale_by=np.max(np.abs(x64)))
+    bn_close(t["variances"], what + " batch variances", code)
+    bn_close(t["rmeans"], what + " running means", code, scale_by=np.max(np.abs(x64)))
+    bn_close(t["rvars"], what + " running variances", code)
+    bn_close(t["out"], what + " output", code)
+    # the gradient takes the statistics as given: hand both sides the oracle's
+    for name in ("means", "variances"):
+        t[name].upload(t[name].host)
+    k = P.run(H.batch_normalize_gradients, V["ig"], V["sg"], V["bg"], V["og"], V["out"], V["x"], V["means"],
+              V["variances"], V["scale"], V["bias"], 1e-3, b, c, e)
+    what = f"batch-normalize-gradients {shape} ({k})"
+    og64 = np.abs(t["og"].init.astype(np.float64))
+    per_channel = og64.reshape(b, c, e or 1).sum(axis=(0, 2)).max()
+    bn_close(t["bg"], what + " bias gradient", code, scale_by=per_channel)
+    bn_close(t["sg"], what + " scale gradient", code, scale_by=per_channel * 4)
+    bn_close(t["ig"], what + " input gradient", code, scale_by=np.max(og64))
+    # in place over the output gradient
+    P.run(H.batch_normalize_gradients, V["og"], V["sg"], V["bg"], V["og"], V["out"], V["x"], V["means"],
+          V["variances"], V["scale"], V["bias"], 1e-3, b, c, e)
+    bn_close(t["og"], what + " input gradient in place", code, scale_by=np.max(og64))
+
+
+def test_batch_normalize_offset_mean_and_misaligned(P):
+    """A channel far from zero (mean 1000, deviation 0.01) and buffers that start
+    off a 16-byte boundary."""
+    rng = np.random.default_rng(42)
+    b, c, e = 6, 5, 100
+    n = b * c * e
+    x = (rng.standard_normal(n) * 0.01 + 1000).astype(np.float32)
+    xb, ob = P.buf(np.concatenate([[0], x]).astype(np.float32)), P.buf(np.zeros(n + 3, np.float32))
+    stats = [P.buf(np.ones(c + 1, np.float32)) for _ in range(6)]
+    sv = [View(s, [c], offset=1) for s in stats]
+    P.run(H.batch_normalize_update_and_apply, View(ob, [n], offset=3), View(xb, [n], offset=1), sv[0], sv[1], sv[2],
+          sv[3], 0.5, sv[4], sv[5], 1e-4, b, c, e)
+    bn_close(stats[0], "offset mean: batch means", capi.F32)
+    bn_close(stats[1], "offset mean: batch variances", capi.F32)
+    bn_close(ob, "offset mean: output", capi.F32)
+
+
+def test_batch_normalize_errors(P):
+    x = P.buf(np.zeros(16, np.float32))
+    xi = P.buf(np.zeros(16, np.int32))
+    v = View(x, [16])
+    with pytest.raises(capi.CortexHipError, match="float and double"):
+        H.batch_normalize(P.hip, View(xi, [16]), View(xi, [16]), View(xi, [16]), View(xi, [16]), View(xi, [16]),
+                          View(xi, [16]), 1e-2, 4, 4)
+    with pytest.raises(capi.CortexHipError, match="positive"):
+        H.batch_normalize(P.hip, v, v, v, v, v, v, 1e-2, 0, 4)

@@ -518,3 +518,91 @@ def test_softmax_stores_float_exponentials_before_summing():
     e = np.exp(x.astype(np.float64) - np.float64(x.max())).astype(np.float32)
     s = np.float32(np.cumsum(e.astype(np.float64))[-1])
     H.assert_bit_exact(ob.host, e / s, "softmax staging")
+
+
+# ------------------------------------------------------------------ batch normalization
+# Pinned by the reference's stored vectors (tests/reference_suite.py) and, here, by what the
+# mathematics fixes: numpy's mean / var for the statistics, the running-average rule, a
+# normalized output, and a finite-difference derivative of the forward pass for the gradients.
+
+def _bn_buffers(rng, b, c, e, f):
+    n = b * c * e
+    t = dict(x=(rng.standard_normal(n) * 2 + 3).astype(f), out=np.zeros(n, f), og=rng.standard_normal(n).astype(f),
+             ig=np.zeros(n, f), means=np.zeros(c, f), variances=np.zeros(c, f), rmeans=rng.standard_normal(c).astype(f),
+             rvars=rng.uniform(0.5, 2, c).astype(f), scale=rng.uniform(0.5, 1.5, c).astype(f),
+             bias=rng.standard_normal(c).astype(f), sg=np.zeros(c, f), bg=np.zeros(c, f))
+    bufs = {k: H.Buf(v, gpu=False) for k, v in t.items()}
+    return bufs, {k: H.View(v, [v.init.size]) for k, v in bufs.items()}
+
+
+@pytest.mark.parametrize("layout", [(6, 5, None), (4, 3, 7)], ids=["eltwise", "spatial"])
+def test_batch_normalize_statistics_closed_form(layout):
+    b, c, e = layout
+    rng = np.random.default_rng(50)
+    bufs, V = _bn_buffers(rng, b, c, e or 1, np.float64)
+    rm0, rv0 = bufs["rmeans"].init.copy(), bufs["rvars"].init.copy()
+    H.batch_normalize_update_and_apply(H.ORACLE, V["out"], V["x"], V["means"], V["variances"], V["rmeans"], V["rvars"],
+                                       0.3, V["scale"], V["bias"], 1e-3, b, c, e)
+    x = bufs["x"].init.reshape(b, c, e or 1)
+    mean, var = x.mean(axis=(0, 2)), x.var(axis=(0, 2))
+    np.testing.assert_allclose(bufs["means"].host, mean, rtol=1e-13)
+    np.testing.assert_allclose(bufs["variances"].host, var, rtol=1e-12)
+    np.testing.assert_allclose(bufs["rmeans"].host, rm0 * 0.7 + mean * 0.3, rtol=1e-12)
+    np.testing.assert_allclose(bufs["rvars"].host, rv0 * 0.7 + x.var(axis=(0, 2), ddof=1) * 0.3, rtol=1e-12)
+    want = (x - mean[None, :, None]) / np.sqrt(var + 1e-3)[None, :, None] * bufs["scale"].init[None, :, None] \
+        + bufs["bias"].init[None, :, None]
+    np.testing.assert_allclose(bufs["out"].host.reshape(x.shape), want, rtol=1e-11, atol=1e-12)
+
+
+@pytest.mark.parametrize("layout", [(5, 4, None), (3, 2, 6)], ids=["eltwise", "spatial"])
+def test_batch_normalize_gradients_against_finite_differences(layout):
+    b, c, e = layout
+    ee = e or 1
+    rng = np.random.default_rng(51)
+    bufs, V = _bn_buffers(rng, b, c, ee, np.float64)
+    eps = 1e-3
+
+    def forward(x, scale, bias):
+        x = x.reshape(b, c, ee)
+        mean, var = x.mean(axis=(0, 2), keepdims=True), x.var(axis=(0, 2), keepdims=True)
+        return ((x - mean) / np.sqrt(var + eps) * scale[None, :, None] + bias[None, :, None]).reshape(-1)
+
+    x0, og = bufs["x"].init.copy(), bufs["og"].init.copy()
+    scale0, bias0 = bufs["scale"].init.copy(), bufs["bias"].init.copy()
+    loss = lambda x, s, bb: float(np.dot(forward(x, s, bb), og))
+    H.batch_normalize_update_and_apply(H.ORACLE, V["out"], V["x"], V["means"], V["variances"], V["rmeans"], V["rvars"],
+                                       0.3, V["scale"], V["bias"], eps, b, c, e)
+    H.batch_normalize_gradients(H.ORACLE, V["ig"], V["sg"], V["bg"], V["og"], V["out"], V["x"], V["means"],
+                                V["variances"], V["scale"], V["bias"], eps, b, c, e)
+    h = 1e-6
+    num_ig = np.zeros_like(x0)
+    for i in range(x0.size):
+        xp, xm = x0.copy(), x0.copy()
+        xp[i] += h
+        xm[i] -= h
+        num_ig[i] = (loss(xp, scale0, bias0) - loss(xm, scale0, bias0)) / (2 * h)
+    np.testing.assert_allclose(bufs["ig"].host, num_ig, rtol=1e-5, atol=1e-7)
+    for name, which in (("sg", 0), ("bg", 1)):
+        num = np.zeros(c)
+        for j in range(c):
+            d = np.zeros(c)
+            d[j] = h
+            if which == 0:
+                num[j] = (loss(x0, scale0 + d, bias0) - loss(x0, scale0 - d, bias0)) / (2 * h)
+            else:
+                num[j] = (loss(x0, scale0, bias0 + d) - loss(x0, scale0, bias0 - d)) / (2 * h)
+        np.testing.assert_allclose(bufs[name].host, num, rtol=1e-6, atol=1e-8)
+
+
+def test_batch_normalize_float_rounding_points():
+    """Where the float form rounds: the inverse standard deviation is rounded to float before it
+    is used (cpu/tensor_math.clj:772-773) and the store rounds once."""
+    x = np.array([0.1, 0.7, 1.3, 2.9], np.float32)
+    m, v, s, bb = np.float32(0.3), np.float32(0.77), np.float32(1.7), np.float32(-0.2)
+    bufs = [H.Buf(a, gpu=False) for a in (np.zeros(4, np.float32), x, np.array([m]), np.array([v]), np.array([s]),
+                                          np.array([bb]))]
+    views = [H.View(bf, [bf.init.size]) for bf in bufs]
+    H.batch_normalize(H.ORACLE, *views, 1e-2, 4, 1)
+    inv = np.float32(np.sqrt(1.0 / (np.float64(v) + np.float64(np.float32(1e-2)))))
+    want = ((x.astype(np.float64) - np.float64(m)) * np.float64(inv) * np.float64(s) + np.float64(bb)).astype(np.float32)
+    H.assert_bit_exact(bufs[0].host, want, "batch-normalize float rounding")

@@ -9,7 +9,8 @@ from oracle_backend import OracleDriver
 ALL_DTYPE_TESTS = ["assign_constant", "assign_marshal", "binary_constant_op", "binary_op", "unary_op", "channel_op",
                    "ternary_op_select", "unary_reduce", "transpose", "select", "select_transpose_interaction",
                    "indexed_tensor", "simple_stream"]
-FLOAT_TESTS = ["activation_forward", "activation_gradient", "softmax", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
+FLOAT_TESTS = ["activation_forward", "activation_gradient", "softmax", "batch_normalize",
+               "batch_normalize_update_and_apply", "batch_normalize_gradients", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
                "adam_trajectory"]
 
 
