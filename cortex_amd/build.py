@@ -30,6 +30,8 @@ SOURCES = [
     "ops_optim.hip",
     "ops_nn.hip",
     "ops_batchnorm.hip",
+    "ops_rand.hip",
+    "ops_blas.cpp",
 ]
 
 # -ffp-contract=off: the reference's CPU backend rounds after every JVM

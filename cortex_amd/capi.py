@@ -30,6 +30,7 @@ BINARY_OPS = {"+": 0, "-": 1, "*": 2, "/": 3, "min": 4, "max": 5, "bit-and": 6, 
               ">": 9, ">=": 10, "<": 11, "<=": 12}
 TERNARY_OPS = {"select": 0}
 ACTIVATION_OPS = {"logistic": 0, "tanh": 1, "relu": 2}
+DISTRIBUTIONS = {"gaussian": 0, "flat": 1}
 REDUCE_OPS = {"max": 0, "min": 1, "sum": 2, "mean": 3, "magnitude": 4, "magnitude-squared": 5}
 
 COPY_H2D, COPY_D2H, COPY_D2D = 0, 1, 2
@@ -117,6 +118,9 @@ PROTOTYPES = {
     "ct_batch_normalize_update_and_apply_spatial": [_P, _P, _P, _P, _P, _P, _P, _D, _P, _P, _D, _L, _L, _L, _I],
     "ct_batch_normalize_gradients_eltwise": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _I],
     "ct_batch_normalize_gradients_spatial": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _L, _I],
+    "ct_gemm": [_P, _P, _L, _I, _I, _D, _P, _L, _L, _L, _P, _L, _L, _D, _I],
+    "ct_gemv": [_P, _P, _L, _I, _D, _P, _L, _L, _L, _P, _L, _D, _I],
+    "ct_rand": [_P, _P, _L, _I, _I, _D, _D, C.c_uint64, C.c_uint64],
     "ct_adam_step": [_P, _I, _D, _D, _D, _D, _D, _D, _D, _P, _P, _P, _P, _L],
     "ct_adadelta_step": [_P, _I, _D, _D, _P, _P, _D, _P, _P, _L],
 }

@@ -25,6 +25,7 @@ indirectly addressed dimension.
 from __future__ import annotations
 
 import ctypes as C
+import os
 from typing import Optional, Sequence
 
 import numpy as np
@@ -298,6 +299,17 @@ class HipStream:
         capi.call("ct_softmax_spatial", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), input.ptr,
                   C.byref(_dims_struct(input_dims)), capi.DTYPE_CODES[output.datatype])
 
+    # -- gemm!, gemv! (tensor/math.clj:106-123) ---------------------------------
+    def gemm(self, c, c_colstride, trans_a, trans_b, alpha, a, a_row_count, a_col_count, a_colstride, b, b_col_count,
+             b_colstride, beta) -> None:
+        capi.call("ct_gemm", self.handle, c.ptr, int(c_colstride), int(bool(trans_a)), int(bool(trans_b)), float(alpha),
+                  a.ptr, int(a_row_count), int(a_col_count), int(a_colstride), b.ptr, int(b_col_count),
+                  int(b_colstride), float(beta), capi.DTYPE_CODES[c.datatype])
+
+    def gemv(self, c, inc_c, trans_a, alpha, a, a_row_count, a_col_count, a_colstride, x, inc_x, beta) -> None:
+        capi.call("ct_gemv", self.handle, c.ptr, int(inc_c), int(bool(trans_a)), float(alpha), a.ptr, int(a_row_count),
+                  int(a_col_count), int(a_colstride), x.ptr, int(inc_x), float(beta), capi.DTYPE_CODES[c.datatype])
+
     # -- batch normalization (tensor/math.clj:124-174); every buffer is packed --
     def batch_normalize_eltwise(self, output, input, means, variances, scale, bias, epsilon, batch_count,
                                 element_count) -> None:
@@ -341,6 +353,29 @@ class HipStream:
                   bias_gradient.ptr, output_gradient.ptr, output.ptr, input.ptr, batch_means.ptr, batch_variances.ptr,
                   scale.ptr, bias.ptr, float(epsilon), int(batch_count), int(channel_count), int(element_count),
                   capi.DTYPE_CODES[input_gradient.datatype])
+
+    # -- rand! (tensor/math.clj:237) ------------------------------------------
+    def seed_random(self, seed: int) -> None:
+        """Restarts this stream's generator.  The reference's generators are
+        seeded by their libraries (SecureRandom, cuRAND); an unseeded stream
+        draws its seed from the operating system."""
+        self._rand_seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+        self._rand_calls = 0
+
+    def rand(self, dest, dest_dims, distribution) -> None:
+        if getattr(self, "_rand_seed", None) is None:
+            self.seed_random(int.from_bytes(os.urandom(8), "little"))
+        kind = distribution["type"]
+        if kind == "gaussian":
+            a, b = distribution["mean"], distribution["variance"]
+        elif kind == "flat":
+            a, b = distribution["minimum"], distribution["maximum"]
+        else:
+            raise ValueError(f"Unrecognized distribution: {distribution}")
+        n = int(np.prod([int(v) for v in dest_dims["shape"]], dtype=np.int64))
+        capi.call("ct_rand", self.handle, dest.ptr, n, capi.DTYPE_CODES[dest.datatype], capi.DISTRIBUTIONS[kind],
+                  float(a), float(b), self._rand_seed, self._rand_calls)
+        self._rand_calls += 1
 
     # -- optimizers ---------------------------------------------------------
     def adam_step(self, alpha, beta1, beta2, epsilon, pow_beta1_t, pow_beta2_t, gradient_alpha, gradient, parameters,

@@ -513,10 +513,87 @@ def softmax(output: Tensor, input: Tensor) -> Tensor:
     return output
 
 
+# ---------------------------------------------------------------- gemm!, gemv!
+
+def _column_stride(t: Tensor) -> int:
+    """``dimensions->column-stride`` (``tensor.clj:198-204``)."""
+    strides, shp = t.dimensions["strides"], t.dimensions["shape"]
+    return int(strides[-2]) if len(strides) > 1 else int(shp[0]) if shp else 1
+
+
+def _2d_shape(t: Tensor):
+    return dims.to_2d_shape(t.dimensions)
+
+
+def gemm(C: Tensor, trans_a, trans_b, alpha, A: Tensor, B: Tensor, beta) -> Tensor:
+    """``gemm!`` (``tensor.clj:920-951``): C = alpha * (trans-a? A) * (trans-b? B) + beta * C."""
+    _external_library_check("gemm!", C, A, B)
+    a_shape = _2d_shape(A)[::-1] if trans_a else _2d_shape(A)
+    b_shape = _2d_shape(B)[::-1] if trans_b else _2d_shape(B)
+    c_shape = _2d_shape(C)
+    if a_shape[1] != b_shape[0]:
+        raise TensorError(f"A {a_shape} col count doesn't match B {b_shape} row count")
+    if a_shape[0] != c_shape[0]:
+        raise TensorError(f"C {c_shape} rows count doesn't match A {a_shape} row count")
+    if b_shape[1] != c_shape[1]:
+        raise TensorError(f"C {c_shape} col count doesn't match B {b_shape} col count")
+    check_stream().gemm(C.buffer, _column_stride(C), trans_a, trans_b, alpha, A.buffer, a_shape[0], a_shape[1],
+                        _column_stride(A), B.buffer, b_shape[1], _column_stride(B), beta)
+    return C
+
+
+def _blas_vector_increment(t: Tensor) -> int:
+    """``blas-vector-increment`` (``tensor.clj:966-972``)."""
+    if dense(t):
+        return 1
+    strides = t.dimensions["strides"]
+    return int(strides[-1]) if strides else 1
+
+
+def gemv(c: Tensor, trans_a, alpha, A: Tensor, x: Tensor, beta) -> Tensor:
+    """``gemv!`` (``tensor.clj:975-989``): c = alpha * (trans-a? A) * x + beta * c."""
+    _external_library_check("gemv!", c, A, x)
+    for t in (x, c):
+        if not (dense(t) or _num_columns(t) == 1):
+            raise TensorError("Argument is not vector-indexable")
+    a_rows, a_cols = _2d_shape(A)
+    check_stream().gemv(c.buffer, _blas_vector_increment(c), trans_a, alpha, A.buffer, a_rows, a_cols,
+                        _column_stride(A), x.buffer, _blas_vector_increment(x), beta)
+    return c
+
+
+# ---------------------------------------------------------------- rand!
+
+def gaussian_distribution(mean=0, variance=1) -> dict:
+    """``gaussian-distribution`` (``tensor.clj:989-996``)."""
+    return {"type": "gaussian", "mean": float(mean), "variance": float(variance)}
+
+
+def flat_distribution(minimum=0, maximum=1) -> dict:
+    """``flat-distribution`` (``tensor.clj:999-1013``): [minimum, maximum)."""
+    if not float(minimum) < float(maximum):
+        raise TensorError("Minimum must be less than maximum")
+    return {"type": "flat", "minimum": float(minimum), "maximum": float(maximum)}
+
+
+def rand(dest: Tensor, distribution: dict) -> Tensor:
+    """``rand!`` (``tensor.clj:1026-1044``): float tensors with simple dense buffers only."""
+    if dest.get_datatype() != "float":
+        raise TensorError("Can only generate rands into floating point buffers")
+    if not (dense(dest) and dims.access_increasing(dest.dimensions)):
+        raise TensorError("Rand generation must have simple dense buffers")
+    if distribution.get("type") not in ("gaussian", "flat"):
+        raise TensorError("Invalid distibution type")
+    check_stream().rand(dest.buffer, dest.dimensions, distribution)
+    return dest
+
+
 # ---------------------------------------------------------------- batch normalization
 
 def _num_columns(t: Tensor) -> int:
-    return int(t.shape()[-1])
+    """``dimensions->num-columns`` (``tensor.clj:207-209``): the second shape entry, 1 if there is none."""
+    shp = t.shape()
+    return int(shp[1]) if len(shp) > 1 else 1
 
 
 def as_row_vector(t: Tensor) -> Tensor:

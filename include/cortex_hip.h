@@ -86,6 +86,9 @@ typedef enum ct_activation_op_t {
   CT_ACT_LOGISTIC = 0, CT_ACT_TANH = 1, CT_ACT_RELU = 2
 } ct_activation_op_t;
 
+/* rand! distributions (src/cortex/tensor.clj:989-1017). */
+typedef enum ct_distribution_t { CT_DIST_GAUSSIAN = 0, CT_DIST_FLAT = 1 } ct_distribution_t;
+
 typedef enum ct_status {
   CT_OK = 0,
   CT_ERR_INVALID = 1,     /* bad argument: rank, dtype, op code, null pointer, shape rule */
@@ -263,6 +266,39 @@ int ct_softmax_eltwise(void* stream, void* output, const ct_dims* output_dims, c
  * channels of every (batch, element) position. */
 int ct_softmax_spatial(void* stream, void* output, const ct_dims* output_dims, const void* input,
                        const ct_dims* input_dims, int dtype);
+
+/* gemm! (tensor/math.clj:106-116; cpu/tensor_math.clj:672-700, 1534-1545;
+ * compute/math_util.clj:17-30): row-major
+ *   C[a_row_count, b_col_count] = alpha * op(A) * op(B) + beta * C,
+ * op(A) is [a_row_count, a_col_count], op(B) is [a_col_count, b_col_count]
+ * (the counts are taken after the transposition, src/cortex/tensor.clj:920-951);
+ * a column stride is the distance in elements between two stored rows.  Runs on
+ * rocBLAS, loaded on first use.  dtype is CT_F32 or CT_F64. */
+int ct_gemm(void* stream, void* c, int64_t c_colstride, int trans_a, int trans_b, double alpha,
+            const void* a, int64_t a_row_count, int64_t a_col_count, int64_t a_colstride,
+            const void* b, int64_t b_col_count, int64_t b_colstride, double beta, int dtype);
+
+/* gemv! (tensor/math.clj:117-123; cpu/tensor_math.clj:701-726, 1547-1556;
+ * compute/math_util.clj:33-41): c = alpha * op(A) * x + beta * c for the stored
+ * row-major matrix A [a_row_count, a_col_count] (counts before the
+ * transposition, src/cortex/tensor.clj:975-989) and vector increments in
+ * elements. */
+int ct_gemv(void* stream, void* c, int64_t inc_c, int trans_a, double alpha, const void* a,
+            int64_t a_row_count, int64_t a_col_count, int64_t a_colstride, const void* x,
+            int64_t inc_x, double beta, int dtype);
+
+/* rand! (tensor/math.clj:237; cpu/tensor_math.clj:1867-1890;
+ * cuda/tensor_math.clj:1246-1274): fills n values of a dense float buffer.
+ *   CT_DIST_GAUSSIAN  a = mean, b = variance
+ *   CT_DIST_FLAT      a = minimum (included), b = maximum (excluded)
+ * The reference draws from a stateful library generator, so only the
+ * distribution is specified.  Here value k is a pure function of
+ * (seed, offset, k) (Philox4x32-10, counter (k / 4, offset), key seed): the
+ * caller keeps the generator state, e.g. one seed per stream and an offset it
+ * increments per call.  dtype must be CT_F32, as in the reference
+ * (src/cortex/tensor.clj:1020-1037). */
+int ct_rand(void* stream, void* dest, int64_t n, int dtype, int distribution, double a, double b,
+            uint64_t seed, uint64_t offset);
 
 /* Batch normalization.  Every buffer is packed: input and output hold
  * batch_count x channel_count x element_count values (the eltwise forms have

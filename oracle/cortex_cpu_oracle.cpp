@@ -22,6 +22,19 @@
 //   activation-gradient!     cpu/tensor_math.clj:1318-1362
 //   softmax (both forms)     cpu/tensor_math.clj:1037-1103
 //   batch-normalize (6 forms) cpu/tensor_math.clj:731-1033, 1558-1638
+//   gemm!, gemv!             cpu/tensor_math.clj:672-726, 1534-1556 and
+//                            compute/math_util.clj:17-41 for the operand
+//                            mapping; the product itself is netlib BLAS
+//                            (com.github.fommil.netlib, not under
+//                            /root/reference) whose published definition
+//                            C = alpha op(A) op(B) + beta C is restated with a
+//                            double accumulator
+//   rand!                    cpu/tensor_math.clj:1867-1890 for the arithmetic
+//                            around the draws; the generator itself is this
+//                            build's (Philox4x32-10, Salmon et al. SC'11), pinned
+//                            by the Random123 known-answer vectors -- the
+//                            reference draws from SecureRandom / cuRAND and
+//                            fixes only the distribution
 //   Adam                     src/cortex/optimize/adam.clj:68-102
 //   Adadelta                 java/cortex/compute/optimize/AdadeltaOptimizer.java:29-64
 //
@@ -705,6 +718,59 @@ void bn_gradients_t(const BnOffsetter& o, T* input_gradient, T* scale_gradient, 
   }
 }
 
+// ---------------------------------------------------------------- gemm!, gemv!
+// gemm! through col->row-gemm (compute/math_util.clj:17-30) is the row-major
+// product C[M, N] = alpha * op(A)[M, K] * op(B)[K, N] + beta * C with row pitches
+// ("column strides" in the reference's column-major wording).  BLAS does not
+// read C when beta is zero.
+template <class T>
+void gemm_t(T* c, int64_t ldc, bool ta, bool tb, double alpha, const T* a, int64_t M, int64_t K, int64_t lda,
+            const T* b, int64_t N, int64_t ldb, double beta) {
+  const T al = (T)alpha, be = (T)beta;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < M; ++i)
+    for (int64_t j = 0; j < N; ++j) {
+      double acc = 0.0;
+      for (int64_t k = 0; k < K; ++k) {
+        const double av = (double)(ta ? a[k * lda + i] : a[i * lda + k]);
+        const double bv = (double)(tb ? b[j * ldb + k] : b[k * ldb + j]);
+        acc += av * bv;
+      }
+      const double prev = be == (T)0 ? 0.0 : (double)be * (double)c[i * ldc + j];
+      c[i * ldc + j] = (T)((double)al * acc + prev);
+    }
+}
+
+// gemv! through col->row-gemv (compute/math_util.clj:33-41): y = alpha * op(A) x + beta * y for
+// the stored row-major A[rows, cols].
+template <class T>
+void gemv_t(T* y, int64_t incy, bool ta, double alpha, const T* a, int64_t rows, int64_t cols, int64_t lda,
+            const T* x, int64_t incx, double beta) {
+  const T al = (T)alpha, be = (T)beta;
+  const int64_t out_n = ta ? cols : rows, in_n = ta ? rows : cols;
+  for (int64_t i = 0; i < out_n; ++i) {
+    double acc = 0.0;
+    for (int64_t k = 0; k < in_n; ++k) acc += (double)(ta ? a[k * lda + i] : a[i * lda + k]) * (double)x[k * incx];
+    const double prev = be == (T)0 ? 0.0 : (double)be * (double)y[i * incy];
+    y[i * incy] = (T)((double)al * acc + prev);
+  }
+}
+
+// ---------------------------------------------------------------- rand!
+// Philox4x32-10: ten rounds of two 32x32->64 multiplies, the key bumped by the
+// Weyl constants between rounds.
+inline void philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  const uint64_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = M0 * c0, p1 = M1 * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c0 = n0; c1 = (uint32_t)p1; c2 = n2; c3 = (uint32_t)p0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
 // cpu-adam-step-impl! (adam.clj:68-102).  The scalars are cast to the datatype
 // first; the arithmetic then runs in double.
 template <class T>
@@ -1037,6 +1103,88 @@ int co_batch_normalize_gradients_eltwise(void* input_gradient, void* scale_gradi
   return co_batch_normalize_gradients_spatial(input_gradient, scale_gradient, bias_gradient, output_gradient, output,
                                               input, batch_means, batch_variances, scale, bias, epsilon, batch_count,
                                               element_count, 1, dtype);
+}
+
+int co_gemm(void* c, int64_t c_colstride, int trans_a, int trans_b, double alpha, const void* a, int64_t a_row_count,
+            int64_t a_col_count, int64_t a_colstride, const void* b, int64_t b_col_count, int64_t b_colstride,
+            double beta, int dtype) {
+  if (dtype == CT_F32)
+    gemm_t<float>((float*)c, c_colstride, trans_a != 0, trans_b != 0, alpha, (const float*)a, a_row_count, a_col_count,
+                  a_colstride, (const float*)b, b_col_count, b_colstride, beta);
+  else if (dtype == CT_F64)
+    gemm_t<double>((double*)c, c_colstride, trans_a != 0, trans_b != 0, alpha, (const double*)a, a_row_count,
+                   a_col_count, a_colstride, (const double*)b, b_col_count, b_colstride, beta);
+  else
+    return fail("gemm! is only defined for float and double tensors");
+  return 0;
+}
+
+int co_gemv(void* c, int64_t inc_c, int trans_a, double alpha, const void* a, int64_t a_row_count,
+            int64_t a_col_count, int64_t a_colstride, const void* x, int64_t inc_x, double beta, int dtype) {
+  if (dtype == CT_F32)
+    gemv_t<float>((float*)c, inc_c, trans_a != 0, alpha, (const float*)a, a_row_count, a_col_count, a_colstride,
+                  (const float*)x, inc_x, beta);
+  else if (dtype == CT_F64)
+    gemv_t<double>((double*)c, inc_c, trans_a != 0, alpha, (const double*)a, a_row_count, a_col_count, a_colstride,
+                   (const double*)x, inc_x, beta);
+  else
+    return fail("gemv! is only defined for float and double tensors");
+  return 0;
+}
+
+// The library's rand!: value k of the stream (seed, offset) is word k % 4 of
+// the Philox block with counter (k / 4, offset) and key seed.  The arithmetic
+// around the draw follows cpu/tensor_math.clj:1873-1887: float parameters,
+// double arithmetic, one rounding at the store.
+int co_rand(void* dest, int64_t n, int dtype, int distribution, double a, double b, uint64_t seed,
+            uint64_t offset) {
+  if (dtype != CT_F32) return fail("Can only generate rands into floating point buffers");
+  if (n < 0) return fail("negative count");
+  float* d = (float*)dest;
+  const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  const float inv24 = 5.9604644775390625e-08f, two_pi = 6.28318530717958647692f;
+  double p0, p1;
+  if (distribution == CT_DIST_FLAT) {
+    const float minimum = (float)a, maximum = (float)b;
+    if (!(minimum < maximum)) return fail("Minimum must be less than maximum");
+    p0 = (double)minimum;
+    p1 = (double)maximum - (double)minimum;
+  } else if (distribution == CT_DIST_GAUSSIAN) {
+    if (!((float)b >= 0.0f)) return fail("negative variance");
+    p0 = (double)(float)a;
+    p1 = std::sqrt((double)(float)b);
+  } else {
+    return fail("Unrecognized distribution");
+  }
+  for (int64_t i = 0; i * 4 < n; ++i) {
+    const uint32_t ctr[4] = {(uint32_t)i, (uint32_t)((uint64_t)i >> 32), (uint32_t)offset, (uint32_t)(offset >> 32)};
+    uint32_t r[4];
+    float v[4];
+    philox4x32_10(ctr, key, r);
+    if (distribution == CT_DIST_FLAT) {
+      for (int e = 0; e < 4; ++e) {
+        const float u = (float)(r[e] >> 8) * inv24;
+        v[e] = (float)(p0 + (double)u * p1);
+      }
+    } else {
+      for (int h = 0; h < 2; ++h) {
+        const float u1 = (float)((r[2 * h] >> 8) + 1u) * inv24;
+        const float u2 = (float)(r[2 * h + 1] >> 8) * inv24;
+        const float rad = std::sqrt(-2.0f * std::log(u1));
+        const float ang = two_pi * u2;
+        v[2 * h] = (float)(p1 * (double)(rad * std::cos(ang)) + p0);
+        v[2 * h + 1] = (float)(p1 * (double)(rad * std::sin(ang)) + p0);
+      }
+    }
+    for (int e = 0; e < 4 && i * 4 + e < n; ++e) d[i * 4 + e] = v[e];
+  }
+  return 0;
+}
+
+// One Philox4x32-10 block, for the known-answer tests.
+int co_philox4x32_10(const uint32_t* counter, const uint32_t* key, uint32_t* out) {
+  philox4x32_10(counter, key, out);
+  return 0;
 }
 
 int co_adam_step(int dtype, double alpha, double beta1, double beta2, double epsilon,

@@ -263,6 +263,23 @@ def batch_normalize_gradients(side, input_gradient: View, scale_gradient: View, 
                   input_gradient.buf.dtype)
 
 
+def gemm(side, c: View, c_colstride, trans_a, trans_b, alpha, a: View, a_rows, a_cols, a_colstride, b: View, b_cols,
+         b_colstride, beta):
+    side.call("gemm", side.ptr(c), c_colstride, int(trans_a), int(trans_b), float(alpha), side.ptr(a), a_rows, a_cols,
+              a_colstride, side.ptr(b), b_cols, b_colstride, float(beta), c.buf.dtype)
+
+
+def gemv(side, c: View, inc_c, trans_a, alpha, a: View, a_rows, a_cols, a_colstride, x: View, inc_x, beta):
+    side.call("gemv", side.ptr(c), inc_c, int(trans_a), float(alpha), side.ptr(a), a_rows, a_cols, a_colstride,
+              side.ptr(x), inc_x, float(beta), c.buf.dtype)
+
+
+def rand(side, dest: View, n, distribution, a, b, seed, offset):
+    """distribution: "gaussian" (a = mean, b = variance) or "flat" (a = minimum, b = maximum)."""
+    side.call("rand", side.ptr(dest), n, dest.buf.dtype, capi.DISTRIBUTIONS[distribution], float(a), float(b),
+              int(seed), int(offset))
+
+
 def adam_step(side, alpha, beta1, beta2, eps, pb1, pb2, ga, grad: View, params: View, m: View, v: View, n):
     args = (grad.buf.dtype, float(alpha), float(beta1), float(beta2), float(eps), float(pb1), float(pb2), float(ga),
             side.ptr(grad), side.ptr(params), side.ptr(m), side.ptr(v), n)

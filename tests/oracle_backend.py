@@ -189,6 +189,28 @@ class OracleStream:
         ob.call("batch_normalize_gradients_spatial", ig.ptr, sg.ptr, bg.ptr, og.ptr, out.ptr, inp.ptr, bm.ptr, bv.ptr,
                 scale.ptr, bias.ptr, float(eps), int(batch), int(chans), int(elems), capi.DTYPE_CODES[ig.datatype])
 
+    def gemm(self, c, ldc, ta, tb, alpha, a, a_rows, a_cols, lda, b, b_cols, ldb, beta):
+        ob.call("gemm", c.ptr, int(ldc), int(bool(ta)), int(bool(tb)), float(alpha), a.ptr, int(a_rows), int(a_cols),
+                int(lda), b.ptr, int(b_cols), int(ldb), float(beta), capi.DTYPE_CODES[c.datatype])
+
+    def gemv(self, c, inc_c, ta, alpha, a, a_rows, a_cols, lda, x, inc_x, beta):
+        ob.call("gemv", c.ptr, int(inc_c), int(bool(ta)), float(alpha), a.ptr, int(a_rows), int(a_cols), int(lda),
+                x.ptr, int(inc_x), float(beta), capi.DTYPE_CODES[c.datatype])
+
+    def seed_random(self, seed):
+        self._rand_seed, self._rand_calls = int(seed) & 0xFFFFFFFFFFFFFFFF, 0
+
+    def rand(self, dest, dest_dims, distribution):
+        if getattr(self, "_rand_seed", None) is None:
+            self.seed_random(0x5EED)
+        kind = distribution["type"]
+        a, b = ((distribution["mean"], distribution["variance"]) if kind == "gaussian"
+                else (distribution["minimum"], distribution["maximum"]))
+        n = int(np.prod([int(v) for v in dest_dims["shape"]]))
+        ob.call("rand", dest.ptr, n, capi.DTYPE_CODES[dest.datatype], capi.DISTRIBUTIONS[kind], float(a), float(b),
+                self._rand_seed, self._rand_calls)
+        self._rand_calls += 1
+
     def adam_step(self, alpha, beta1, beta2, eps, pb1, pb2, ga, gradient, parameters, m, v, n):
         ob.call("adam_step", capi.DTYPE_CODES[gradient.datatype], float(alpha), float(beta1), float(beta2), float(eps),
                 float(pb1), float(pb2), float(ga), gradient.ptr, parameters.ptr, m.ptr, v.ptr, int(n))

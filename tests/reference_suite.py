@@ -246,6 +246,46 @@ def softmax(driver, datatype):
         equals(([0, 1] + list(ct.to_double_array(answer))) * 5, ct.to_double_array(pred_matrix))
 
 
+# verify/tensor.clj:252-283; also exercises sub-matrices
+def gemm(driver, datatype):
+    with context(driver, datatype):
+        tens_a = ct.to_tensor(partition(3, range(9)))
+        tens_b = ct.to_tensor(partition(3, [2] * 9))
+        tens_c = ct.to_tensor(partition(3, [10] * 9))
+        ct.gemm(tens_c, False, False, 1, tens_a, tens_b, 1)
+        equals([16.0, 16.0, 16.0, 34.0, 34.0, 34.0, 52.0, 52.0, 52.0], ct.to_double_array(tens_c))
+        ct.gemm(tens_c, False, False, 1, tens_a, tens_b, 0)
+        equals([6.0, 6.0, 6.0, 24.0, 24.0, 24.0, 42.0, 42.0, 42.0], ct.to_double_array(tens_c))
+        ct.gemm(tens_c, True, False, 1, tens_a, tens_b, 0)
+        equals([18.0, 18.0, 18.0, 24.0, 24.0, 24.0, 30.0, 30.0, 30.0], ct.to_double_array(tens_c))
+        sub_a, sub_b = ct.submatrix(tens_a, 0, 2, 0, 2), ct.submatrix(tens_b, 0, 2, 0, 2)
+        sub_c = ct.submatrix(tens_c, 0, 2, 0, 2)
+        ct.gemm(sub_c, False, False, 1, sub_a, sub_b, 0)
+        equals([2, 2, 14, 14], ct.to_double_array(sub_c))
+        equals([2.0, 2.0, 18.0, 14.0, 14.0, 24.0, 30.0, 30.0, 30.0], ct.to_double_array(tens_c))
+        sub_a, sub_b = ct.submatrix(tens_a, 1, 2, 1, 2), ct.submatrix(tens_b, 0, 2, 0, 2)
+        sub_c = ct.submatrix(tens_c, 1, 2, 1, 2)
+        ct.gemm(sub_c, False, False, 1, sub_a, sub_b, 1)
+        equals([32, 42, 60, 60], ct.to_double_array(sub_c))
+        equals([2.0, 2.0, 18.0, 14.0, 32.0, 42.0, 30.0, 60.0, 60.0], ct.to_double_array(tens_c))
+
+
+# verify/tensor.clj:286-306
+def gemv(driver, datatype):
+    with context(driver, datatype):
+        tens_a = ct.to_tensor(partition(3, range(12)))
+        tens_b = ct.to_tensor([2] * 4)
+        tens_c = ct.to_tensor(range(4))
+        ct.gemv(tens_c, False, 1, tens_a, tens_b, 1)
+        equals([6.0, 25.0, 44.0, 63.0], ct.to_double_array(tens_c))
+        ct.gemv(tens_c, False, 1, tens_a, tens_b, 0)
+        equals([6, 24, 42, 60], ct.to_double_array(tens_c))
+        tens_c_sub = ct.subvector(tens_c, 0, 3)
+        tens_a_col = ct.columns(tens_a)[1]            # [1 4 7 10], a strided vector
+        ct.gemv(tens_c_sub, True, 1, tens_a, tens_a_col, 0)
+        equals([144.0, 166.0, 188.0], ct.to_double_array(tens_c_sub))
+
+
 BN_ELTWISE_OUT = [-26.0, 4.0, 6.116036847575795, 64.0, 12.955334711889902, 12.46414739030318, 154.0,
                   21.910669423779805, 18.812257933030565, 244.0, 30.86600413566971, 25.16036847575795]
 BN_SPATIAL_OUT = [-26.0, 4.0, 34.0, 64.0, 12.955334711889902, 15.94044628251987, 18.925557853149837,
@@ -358,6 +398,22 @@ def batch_normalize_gradients(driver, datatype):
                ct.to_double_array(input_gradient), 1e-6)
         equals([48.81966992684372] * 3, ct.to_double_array(scale_gradient), 1e-4)
         equals([60.0, 92.0, 124.0], ct.to_double_array(bias_gradient), 1e-4)
+
+
+# verify/tensor.clj:1036-1063; the reference runs it with :float only
+def rand_operator(driver, datatype):
+    with context(driver, "float"):
+        test_vec = []
+        for idx in range(1, 11):
+            tens = ct.rand(ct.new_tensor([10000]), ct.gaussian_distribution(mean=idx, variance=idx))
+            values = ct.to_double_array(tens)
+            test_vec += [np.mean(values), np.var(values, ddof=1)]
+        equals([v for idx in range(1, 11) for v in (idx, idx)], test_vec, 1)
+        test_vec = []
+        for idx in range(1, 11):
+            tens = ct.rand(ct.new_tensor([10000]), ct.flat_distribution(minimum=idx - 2, maximum=idx + 2))
+            test_vec.append(np.mean(ct.to_double_array(tens)))
+        equals(list(range(1, 11)), test_vec, 1)
 
 
 # verify/tensor.clj:623-645

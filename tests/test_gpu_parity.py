@@ -723,3 +723,90 @@ def test_batch_normalize_errors(P):
                           View(xi, [16]), 1e-2, 4, 4)
     with pytest.raises(capi.CortexHipError, match="positive"):
         H.batch_normalize(P.hip, v, v, v, v, v, v, 1e-2, 0, 4)
+
+
+# ------------------------------------------------------------------ rand!
+
+@pytest.mark.parametrize("n", [1, 3, 4, 1003, 70001, 1 << 20])
+def test_rand_matches_oracle_stream(P, n):
+    buf = P.buf(np.zeros(n + 1, np.float32))
+    for view in (View(buf, [n]), View(buf, [n], offset=1)):          # aligned and off the 16-byte grid
+        k = P.run(H.rand, view, n, "flat", -2.0, 3.0, 0xC0FFEE123, 5)
+        compare(buf, f"rand flat n={n} ({k})")                       # integer work and one exact product: bit-exact
+        k = P.run(H.rand, view, n, "gaussian", 1.0, 9.0, 0xC0FFEE123, 6)
+        got, want = buf.download().astype(np.float64), buf.host.astype(np.float64)
+        # Box-Muller in float: log, sqrt, cos and sin of the device library against the host's
+        assert np.max(np.abs(got - want)) <= 3 * 2e-6 * 6, f"rand gaussian n={n} ({k})"
+
+
+def test_rand_errors(P):
+    x = P.buf(np.zeros(8, np.float64))
+    with pytest.raises(capi.CortexHipError, match="floating point buffers"):
+        H.rand(P.hip, View(x, [8]), 8, "flat", 0, 1, 1, 0)
+    y = P.buf(np.zeros(8, np.float32))
+    with pytest.raises(capi.CortexHipError, match="Minimum must be less"):
+        H.rand(P.hip, View(y, [8]), 8, "flat", 1, 1, 1, 0)
+
+
+# ------------------------------------------------------------------ gemm!, gemv! (rocBLAS)
+# The vendor library sums in the tensor's own precision and in its own order; the oracle keeps a
+# double accumulator.  Bar: |got - want| <= tol * (|alpha| sum |a||b| + |beta c|) with
+# tol = 1e-5 for float (k up to 512 terms of 2^-24 relative error each) and 1e-13 for double.
+
+GEMM_CASES = [(5, 7, 4, 9, 8, 6), (64, 64, 64, 64, 64, 64), (33, 129, 65, 140, 70, 70), (256, 512, 128, 512, 512, 128),
+              (1, 300, 1, 300, 300, 1)]
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("case", GEMM_CASES, ids=str)
+def test_gemm(P, code, ta, tb, case):
+    M, K, N, lda, ldb, ldc = case
+    rng = np.random.default_rng(70)
+    f = NP[code]
+    a_rows, a_cols = (K, M) if ta else (M, K)
+    b_rows, b_cols = (N, K) if tb else (K, N)
+    lda, ldb = max(lda, a_cols), max(ldb, b_cols)
+    a, b, c = (rng.standard_normal(s).astype(f) for s in ((a_rows, lda), (b_rows, ldb), (M, ldc)))
+    ba, bb, bc = P.buf(a), P.buf(b), P.buf(c)
+    va, vb, vc = (View(bf, [bf.init.size]) for bf in (ba, bb, bc))
+    A, B = np.abs(a[:, :a_cols].astype(np.float64)), np.abs(b[:, :b_cols].astype(np.float64))
+    for alpha, beta in ((1.0, 0.0), (1.5, -0.5)):
+        P.run(H.gemm, vc, ldc, ta, tb, alpha, va, M, K, lda, vb, N, ldb, beta)
+        bound = np.zeros((M, ldc))
+        bound[:, :N] = abs(alpha) * ((A.T if ta else A) @ (B.T if tb else B)) + abs(beta) * np.abs(c[:, :N]) + 1e-30
+        tol = 1e-5 if code == capi.F32 else 1e-13
+        got, want = bc.download().astype(np.float64).reshape(M, ldc), bc.host.astype(np.float64).reshape(M, ldc)
+        assert np.all(np.abs(got - want) <= tol * bound + 0.0), f"gemm {case} ta={ta} tb={tb}: {np.max(np.abs(got - want))}"
+        assert np.array_equal(got[:, N:], c[:, N:].astype(np.float64))      # row padding untouched
+        bc.reset()
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("ta", [False, True])
+def test_gemv(P, code, ta):
+    rng = np.random.default_rng(71)
+    f = NP[code]
+    for rows, cols, lda, incx, incy in ((6, 5, 8, 3, 2), (300, 257, 257, 1, 1), (64, 1000, 1024, 1, 5)):
+        n_in, n_out = (rows, cols) if ta else (cols, rows)
+        a, x, y = (rng.standard_normal(s).astype(f) for s in ((rows, lda), n_in * incx, n_out * incy))
+        ba, bx, by = P.buf(a), P.buf(x), P.buf(y)
+        va, vx, vy = (View(bf, [bf.init.size]) for bf in (ba, bx, by))
+        P.run(H.gemv, vy, incy, ta, 2.0, va, rows, cols, lda, vx, incx, 0.25)
+        A = np.abs(a[:, :cols].astype(np.float64))
+        bound = np.zeros(n_out * incy)
+        bound[::incy] = 2.0 * ((A.T if ta else A) @ np.abs(x[::incx].astype(np.float64))) + 0.25 * np.abs(y[::incy])
+        tol = 1e-5 if code == capi.F32 else 1e-13
+        got, want = by.download().astype(np.float64), by.host.astype(np.float64)
+        assert np.all(np.abs(got - want) <= tol * bound), f"gemv {(rows, cols)} ta={ta}: {np.max(np.abs(got - want))}"
+
+
+def test_gemm_errors(P):
+    x = P.buf(np.zeros(16, np.float32))
+    xi = P.buf(np.zeros(16, np.int32))
+    v = View(x, [16])
+    with pytest.raises(capi.CortexHipError, match="float and double"):
+        H.gemm(P.hip, View(xi, [16]), 4, False, False, 1, View(xi, [16]), 4, 4, 4, View(xi, [16]), 4, 4, 0)
+    with pytest.raises(capi.CortexHipError, match="column stride"):
+        H.gemm(P.hip, v, 2, False, False, 1, v, 4, 4, 4, v, 4, 4, 0)

@@ -606,3 +606,108 @@ def test_batch_normalize_float_rounding_points():
     inv = np.float32(np.sqrt(1.0 / (np.float64(v) + np.float64(np.float32(1e-2)))))
     want = ((x.astype(np.float64) - np.float64(m)) * np.float64(inv) * np.float64(s) + np.float64(bb)).astype(np.float32)
     H.assert_bit_exact(bufs[0].host, want, "batch-normalize float rounding")
+
+
+# ------------------------------------------------------------------ rand!
+# The generator is not the reference's (it draws from SecureRandom / cuRAND and fixes only the
+# distribution).  Philox4x32-10 is pinned by the known-answer vectors published with Random123
+# (kat_vectors: zero, all-ones and digits-of-pi inputs); the mapping to floats by its closed form
+# and by the moments of the two distributions.
+
+PHILOX_KAT = [
+    ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+    ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+    ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+     [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+]
+
+
+def _philox(counter, key):
+    import ctypes as C
+    c, k, o = (C.c_uint32 * 4)(*counter), (C.c_uint32 * 2)(*key), (C.c_uint32 * 4)()
+    H.oracle_lib().co_philox4x32_10(c, k, o)
+    return list(o)
+
+
+@pytest.mark.parametrize("counter,key,want", PHILOX_KAT)
+def test_philox_known_answers(counter, key, want):
+    assert _philox(counter, key) == want
+
+
+def test_rand_flat_is_the_philox_stream():
+    n, seed, offset = 1003, 0x0123456789ABCDEF, 7
+    buf = H.Buf(np.zeros(n, np.float32), gpu=False)
+    H.rand(H.ORACLE, H.View(buf, [n]), n, "flat", -1.5, 2.5, seed, offset)
+    key = [seed & 0xFFFFFFFF, seed >> 32]
+    words = np.array([w for i in range((n + 3) // 4) for w in _philox([i, 0, offset, 0], key)][:n], dtype=np.uint64)
+    u = (words >> np.uint64(8)).astype(np.float64) * 2.0 ** -24
+    want = (np.float64(np.float32(-1.5)) + u * (np.float64(np.float32(2.5)) - np.float64(np.float32(-1.5)))).astype(np.float32)
+    H.assert_bit_exact(buf.host, want, "flat rand")
+    assert buf.host.min() >= -1.5 and buf.host.max() < 2.5
+    # another offset or seed gives another stream; the same pair repeats
+    again = H.Buf(np.zeros(n, np.float32), gpu=False)
+    H.rand(H.ORACLE, H.View(again, [n]), n, "flat", -1.5, 2.5, seed, offset)
+    assert np.array_equal(again.host, buf.host)
+    H.rand(H.ORACLE, H.View(again, [n]), n, "flat", -1.5, 2.5, seed, offset + 1)
+    assert not np.array_equal(again.host, buf.host)
+
+
+def test_rand_moments():
+    n = 1 << 20
+    buf = H.Buf(np.zeros(n, np.float32), gpu=False)
+    H.rand(H.ORACLE, H.View(buf, [n]), n, "gaussian", 3.0, 4.0, 11, 0)
+    v = buf.host.astype(np.float64)
+    assert abs(v.mean() - 3.0) < 0.01 and abs(v.var() - 4.0) < 0.03
+    z = (v - 3.0) / 2.0
+    assert abs(np.mean(z ** 3)) < 0.02 and abs(np.mean(z ** 4) - 3.0) < 0.05      # skewness, kurtosis
+    assert abs(np.corrcoef(z[:-1], z[1:])[0, 1]) < 0.005                           # neighbours (cos / sin of one pair)
+    from scipy import stats
+    assert stats.kstest(z[:200000], "norm").pvalue > 1e-3
+    H.rand(H.ORACLE, H.View(buf, [n]), n, "flat", 0.0, 1.0, 11, 1)
+    u = buf.host.astype(np.float64)
+    assert abs(u.mean() - 0.5) < 0.002 and abs(u.var() - 1 / 12) < 0.001
+    counts = np.histogram(u, bins=64, range=(0, 1))[0]
+    assert stats.chisquare(counts).pvalue > 1e-3
+
+
+# ------------------------------------------------------------------ gemm!, gemv!
+# The product is netlib BLAS in the reference (not under /root/reference); its definition
+# C = alpha op(A) op(B) + beta C is checked against numpy's matmul in float64, with row pitches
+# wider than the rows, all four transposition pairs, and beta = 0 over a NaN-filled C.
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_gemm_matches_numpy(ta, tb):
+    rng = np.random.default_rng(60)
+    M, K, N, lda, ldb, ldc = 5, 7, 4, 9, 8, 6
+    a_rows, a_cols = (K, M) if ta else (M, K)
+    b_rows, b_cols = (N, K) if tb else (K, N)
+    a, b, c = rng.standard_normal((a_rows, lda)), rng.standard_normal((b_rows, ldb)), rng.standard_normal((M, ldc))
+    A, B = a[:, :a_cols], b[:, :b_cols]
+    want = c.copy()
+    want[:, :N] = 1.5 * (A.T if ta else A) @ (B.T if tb else B) - 0.5 * c[:, :N]
+    bufs = [H.Buf(v, gpu=False) for v in (c, a, b)]
+    vc, va, vb = (H.View(bf, [bf.init.size]) for bf in bufs)
+    H.gemm(H.ORACLE, vc, ldc, ta, tb, 1.5, va, M, K, lda, vb, N, ldb, -0.5)
+    np.testing.assert_allclose(bufs[0].host.reshape(M, ldc), want, rtol=1e-13, atol=1e-13)
+    bufs[0].host[...] = np.nan
+    H.gemm(H.ORACLE, vc, ldc, ta, tb, 1.0, va, M, K, lda, vb, N, ldb, 0.0)
+    got = bufs[0].host.reshape(M, ldc)
+    np.testing.assert_allclose(got[:, :N], (A.T if ta else A) @ (B.T if tb else B), rtol=1e-13, atol=1e-13)
+    assert np.all(np.isnan(got[:, N:]))          # the padding between rows is not touched
+
+
+@pytest.mark.parametrize("ta", [False, True])
+def test_gemv_matches_numpy(ta):
+    rng = np.random.default_rng(61)
+    rows, cols, lda, incx, incy = 6, 5, 8, 3, 2
+    a = rng.standard_normal((rows, lda))
+    n_in, n_out = (rows, cols) if ta else (cols, rows)
+    x, y = rng.standard_normal(n_in * incx), rng.standard_normal(n_out * incy)
+    A = a[:, :cols]
+    want = y.copy()
+    want[::incy] = 2.0 * ((A.T if ta else A) @ x[::incx]) + 0.25 * y[::incy]
+    bufs = [H.Buf(v, gpu=False) for v in (y, a, x)]
+    vy, va, vx = (H.View(bf, [bf.init.size]) for bf in bufs)
+    H.gemv(H.ORACLE, vy, incy, ta, 2.0, va, rows, cols, lda, vx, incx, 0.25)
+    np.testing.assert_allclose(bufs[0].host, want, rtol=1e-13, atol=1e-13)

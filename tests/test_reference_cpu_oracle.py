@@ -9,7 +9,7 @@ from oracle_backend import OracleDriver
 ALL_DTYPE_TESTS = ["assign_constant", "assign_marshal", "binary_constant_op", "binary_op", "unary_op", "channel_op",
                    "ternary_op_select", "unary_reduce", "transpose", "select", "select_transpose_interaction",
                    "indexed_tensor", "simple_stream"]
-FLOAT_TESTS = ["activation_forward", "activation_gradient", "softmax", "batch_normalize",
+FLOAT_TESTS = ["gemm", "gemv", "activation_forward", "activation_gradient", "softmax", "batch_normalize",
                "batch_normalize_update_and_apply", "batch_normalize_gradients", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
                "adam_trajectory"]
 
@@ -36,3 +36,7 @@ def test_mask(driver, datatype):
     # the reference runs the body with :int under both names
     # (test/clj/cortex/compute/cpu/tensor_test.clj:91-92)
     rs.mask(driver, "int")
+
+
+def test_rand_operator(driver):
+    rs.rand_operator(driver, "float")

@@ -35,3 +35,7 @@ def test_float_double(driver, name, datatype):
 @pytest.mark.parametrize("datatype", ["int", "long"])
 def test_mask(driver, datatype):
     rs.mask(driver, "int")
+
+
+def test_rand_operator(driver):
+    rs.rand_operator(driver, "float")
