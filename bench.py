@@ -16,7 +16,8 @@ running ``:select``, three transposed inputs), timed with HIP events recorded on
 the launch stream around every one of its launches inside the timed region.
 ``cpu_baseline`` times the CPU oracle (a C++ restatement of the cortex CPU
 backend, OpenMP) on the same step.  ``others`` reports the remaining BASELINE
-configs, each timed the same way, as additional information.
+configs and ``adjacent`` the neighbouring TensorMath methods, each timed the
+same way, as additional information.
 """
 from __future__ import annotations
 
@@ -192,6 +193,63 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
     return out
 
 
+def run_adjacent(drv, device, stream, timer, capi) -> dict:
+    """The adjacent TensorMath methods built on the same machinery (activation-gradient!,
+    softmax!, batch normalization, rand!, gemm!), timed like the BASELINE configs.  Bytes
+    are algorithmic: every operand read once, every result written once, although the
+    batch-normalization forms that need batch statistics read their operands twice."""
+    out = {}
+    rng = np.random.default_rng(9)
+
+    def entry(nbytes, ms, **more):
+        e = {"us": round(ms * 1e3, 2), "GB/s": round(gbs(nbytes, ms), 1), "frac": round(gbs(nbytes, ms) / PEAK_HBM_GBS, 4),
+             "kernel": capi.last_kernel()}
+        e.update(more)
+        return e
+
+    n = 1 << 27
+    x = upload(drv, device, stream, rng.standard_normal(n, dtype=np.float32))
+    g = upload(drv, device, stream, rng.standard_normal(n, dtype=np.float32))
+    o = device.allocate_device_buffer(n, "float")
+    ms = time_launches(timer, stream, lambda: stream.activation_gradient(o, dims([n]), g, dims([n]), x, dims([n]), "tanh", n), 20)
+    out["activation-gradient! :tanh f32 [2^27]"] = entry(12 * n, ms)
+    for k in (16, 1024):
+        rows = n // k
+        ms = time_launches(timer, stream, lambda: stream.softmax_eltwise(o, dims([rows, k]), x, dims([rows, k])), 20)
+        out[f"softmax! f32 [{rows},{k}]"] = entry(8 * n, ms)
+    b, c, e = 64, 21, 65536
+    ms = time_launches(timer, stream, lambda: stream.softmax_spatial(o, dims([b, c, e]), x, dims([b, c, e])), 20)
+    out[f"softmax! spatial f32 [{b},{c},{e}]"] = entry(8 * b * c * e, ms)
+    ms = time_launches(timer, stream, lambda: stream.rand(o, dims([n]), {"type": "gaussian", "mean": 0.0, "variance": 1.0}), 20)
+    out["rand! gaussian f32 [2^27]"] = entry(4 * n, ms)
+    ms = time_launches(timer, stream, lambda: stream.rand(o, dims([n]), {"type": "flat", "minimum": 0.0, "maximum": 1.0}), 20)
+    out["rand! flat f32 [2^27]"] = entry(4 * n, ms)
+
+    b, c, e = 64, 256, 3136
+    nn_ = b * c * e
+    st = [upload(drv, device, stream, rng.uniform(0.5, 1.5, c).astype(np.float32)) for _ in range(8)]
+    ms = time_launches(timer, stream, lambda: stream.batch_normalize_spatial(o, x, st[0], st[1], st[2], st[3], 1e-3, b, c, e), 20)
+    out[f"batch-normalize! spatial f32 [{b},{c},{e}]"] = entry(8 * nn_, ms)
+    ms = time_launches(timer, stream, lambda: stream.batch_normalize_update_and_apply_spatial(
+        o, x, st[0], st[1], st[4], st[5], 0.9, st[2], st[3], 1e-3, b, c, e), 20)
+    out[f"batch-normalize-update-and-apply! spatial f32 [{b},{c},{e}]"] = entry(8 * nn_, ms, hbm_bytes_moved=12 * nn_)
+    ms = time_launches(timer, stream, lambda: stream.batch_normalize_gradients_spatial(
+        o, st[6], st[7], g, o, x, st[0], st[1], st[2], st[3], 1e-3, b, c, e), 20)
+    out[f"batch-normalize-gradients! spatial f32 [{b},{c},{e}]"] = entry(12 * nn_, ms, hbm_bytes_moved=20 * nn_)
+
+    # gemm! is the one MFMA-bound method (rocBLAS); priced against the dense fp32 matrix peak
+    m = 8192
+    a_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))
+    b_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))
+    c_ = device.allocate_device_buffer(m * m, "float")
+    ms = time_launches(timer, stream, lambda: stream.gemm(c_, m, False, False, 1.0, a_, m, m, m, b_, m, m, 0.0), 5, warm=2)
+    tflops = 2.0 * m ** 3 / (ms * 1e-3) / 1e12
+    out[f"gemm! f32 [{m},{m}]x[{m},{m}] (rocBLAS)"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tflops, 1),
+                                                     "frac_of_fp32_matrix_peak": round(tflops / 157.3, 4),
+                                                     "kernel": capi.last_kernel()}
+    return out
+
+
 def cpu_baseline(hosts, n: int) -> dict:
     """Times the CPU oracle on one full step of the workload."""
     from cortex_amd import capi
@@ -332,6 +390,8 @@ def main() -> int:
     if not args.no_extras:
         log("timing the other BASELINE configs ...")
         result["others"] = run_extras(drv, device, stream, timer, capi)
+        log("timing the adjacent TensorMath methods ...")
+        result["adjacent"] = run_adjacent(drv, device, stream, timer, capi)
     if not args.no_cpu:
         log("timing the CPU oracle on one step ...")
         result["cpu_baseline"] = cpu_baseline(hosts, n)

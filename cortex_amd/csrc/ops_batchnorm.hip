@@ -13,7 +13,8 @@
 //   finishing pass    one wave per channel adds the partials in a fixed order
 //                     and derives the channel's constants
 //   apply pass        one flat, 128-bit vectorised elementwise pass
-// so the operands are read twice and the result written once.  Per-element
+// so the operands are read twice and the result written once (the plain
+// normalization with given statistics is the apply pass alone).  Per-element
 // arithmetic follows the CPU backend operation by operation (double, one
 // rounding at the store); only the order of the additions inside a sum differs
 // (a tree instead of left to right), which moves a double sum by a few units in
@@ -35,8 +36,9 @@ namespace {
 
 enum { kBnNormalize = 0, kBnGradient = 1 };
 constexpr int kParamStride = 8;  // doubles per channel in the parameter table
-// parameter table, normalize: mean, inv_std (rounded to T), scale, shift
-// parameter table, gradient:  mean, inv_std (double), scale, d_var, 2 * d_var_d_out, d_mean_d_out / n, 1 / n
+// constants of a channel as the apply pass holds them:
+//   normalize: mean, inv_std (rounded to T), scale, shift -- derived from the statistics vectors on the fly
+//   gradient:  mean, inv_std (double), scale, d_var, 2 * d_var_d_out, d_mean_d_out / n, 1 / n -- the parameter table
 constexpr int kUnroll = 4;
 
 template <int MODE> struct bn_nacc { static constexpr int value = MODE == kBnGradient ? 5 : 2; };
@@ -46,8 +48,13 @@ struct BnArgs {
   const void* x;    // input
   const void* og;   // output gradient (gradient mode)
   void* out;        // output, or input gradient
-  double* params;   // [channels][kParamStride]
+  double* params;   // [channels][kParamStride], gradient constants written by the finishing pass
   double* partials;
+  const void* means;      // per channel, of the tensor type: the statistics in use
+  const void* variances;
+  const void* scale;
+  const void* bias;
+  double epsilon;
   int64_t B, C, E, W;        // W = C * E, the length of one batch row
   int64_t N;                 // B * C * E
   uint32_t S;                // row segments of the statistics pass
@@ -65,8 +72,7 @@ struct BnArgs {
 struct BnFinish {
   // normalize (update) mode
   void* batch_means; void* batch_variances; void* running_means; void* running_variances;
-  const void* scale; const void* bias;
-  double average_factor, epsilon;
+  double average_factor;
   // gradient mode
   void* scale_gradient; void* bias_gradient;
 };
@@ -170,11 +176,12 @@ __global__ void __launch_bounds__(kBlock) bn_stats_row_kernel(const BnArgs a) {
   const int64_t base = (b0 * a.C + c) * a.E;
   const T* x = reinterpret_cast<const T*>(a.x) + base;
   const T* og = reinterpret_cast<const T*>(a.og) + base;
-  const double* pm = a.params + (int64_t)c * kParamStride;
   double p0;
   T scale = (T)0;
-  if constexpr (MODE == kBnGradient) { p0 = pm[0]; scale = (T)pm[2]; }
-  else p0 = (double)reinterpret_cast<const T*>(a.x)[(int64_t)c * a.E];  // pivot: the channel's first value
+  if constexpr (MODE == kBnGradient) {
+    p0 = (double)reinterpret_cast<const T*>(a.means)[c];
+    scale = reinterpret_cast<const T*>(a.scale)[c];
+  } else p0 = (double)reinterpret_cast<const T*>(a.x)[(int64_t)c * a.E];  // pivot: the channel's first value
   double acc[NACC];
 #pragma unroll
   for (int k = 0; k < NACC; ++k) acc[k] = 0.0;
@@ -235,8 +242,8 @@ __global__ void __launch_bounds__(kBlock) bn_stats_col_kernel(const BnArgs a) {
     if (live) {
       const uint32_t ch = a.e_fd.div((uint32_t)(j0 + e));
       if constexpr (MODE == kBnGradient) {
-        const double* pm = a.params + (int64_t)ch * kParamStride;
-        p0[e] = pm[0]; scale[e] = (T)pm[2];
+        p0[e] = (double)reinterpret_cast<const T*>(a.means)[ch];
+        scale[e] = reinterpret_cast<const T*>(a.scale)[ch];
       } else {
         p0[e] = (double)reinterpret_cast<const T*>(a.x)[(int64_t)ch * a.E];
       }
@@ -300,38 +307,25 @@ __global__ void __launch_bounds__(kBlock) bn_stats_col_kernel(const BnArgs a) {
 
 // ---------------------------------------------------------------- per-channel constants
 
-// Normalization with given statistics (batch-normalize-impl, :766-777).
-template <class T>
-__device__ __forceinline__ void bn_store_normalize_params(double* pm, T mean, T variance, T scale, T shift, double epsilon) {
-  const T eps = (T)epsilon;
-  pm[0] = (double)mean;
-  pm[1] = (double)(T)sqrt(1.0 / ((double)variance + (double)eps));
-  pm[2] = (double)scale;
-  pm[3] = (double)shift;
-}
-
-template <class T>
-__global__ void __launch_bounds__(kBlock) bn_prepare_normalize_kernel(double* params, const T* means, const T* variances,
-                                                                      const T* scale, const T* bias, double epsilon,
-                                                                      int64_t C) {
-  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (c < C) bn_store_normalize_params<T>(params + c * kParamStride, means[c], variances[c], scale[c], bias[c], epsilon);
-}
-
-// Gradient constants known before the sums (batch-normalize-gradients-impl, :922-931).
-template <class T>
-__global__ void __launch_bounds__(kBlock) bn_prepare_gradient_kernel(double* params, const T* means, const T* variances,
-                                                                     const T* scale, double epsilon, int64_t C) {
-  const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (c >= C) return;
-  const T eps = (T)epsilon;
-  const T pow_factor = (T)(-3.0 / 2.0);
-  const double variance = (double)eps + (double)variances[c];
-  double* pm = params + c * kParamStride;
-  pm[0] = (double)means[c];
-  pm[1] = 1.0 / sqrt(variance);
-  pm[2] = (double)scale[c];
-  pm[3] = (double)(T)(-0.5 * pow(variance, (double)pow_factor));
+// The constants of channel ch for the apply pass, NP doubles.  Normalize mode
+// derives them from the statistics vectors (batch-normalize-impl, :766-777: the
+// inverse standard deviation is rounded to T); gradient mode reads the table the
+// finishing pass wrote.
+template <class T, int MODE>
+__device__ __forceinline__ double bn_channel_constant(const BnArgs& a, uint32_t ch, int k) {
+  if constexpr (MODE == kBnGradient) {
+    return a.params[(int64_t)ch * kParamStride + k];
+  } else {
+    switch (k) {
+      case 0: return (double)reinterpret_cast<const T*>(a.means)[ch];
+      case 1: {
+        const T eps = (T)a.epsilon;
+        return (double)(T)sqrt(1.0 / ((double)reinterpret_cast<const T*>(a.variances)[ch] + (double)eps));
+      }
+      case 2: return (double)reinterpret_cast<const T*>(a.scale)[ch];
+      default: return (double)reinterpret_cast<const T*>(a.bias)[ch];
+    }
+  }
 }
 
 // One wave per channel adds the channel's partial sums (segments, and columns in
@@ -363,8 +357,16 @@ __global__ void __launch_bounds__(kBlock) bn_finish_kernel(const BnArgs a, const
   double* pm = a.params + c * kParamStride;
   const int64_t count = a.B * a.E;
   if constexpr (MODE == kBnGradient) {
-    // :932-983, with the factors put back
-    const double inv_std = pm[1], d_var = pm[3];
+    // :922-983, with the factors put back
+    const T eps = (T)a.epsilon;
+    const T pow_factor = (T)(-3.0 / 2.0);
+    const double variance = (double)eps + (double)reinterpret_cast<const T*>(a.variances)[c];
+    const double inv_std = 1.0 / sqrt(variance);
+    const double d_var = (double)(T)(-0.5 * pow(variance, (double)pow_factor));
+    pm[0] = (double)reinterpret_cast<const T*>(a.means)[c];
+    pm[1] = inv_std;
+    pm[2] = (double)reinterpret_cast<const T*>(a.scale)[c];
+    pm[3] = d_var;
     reinterpret_cast<T*>(f.bias_gradient)[c] = (T)acc[0];
     reinterpret_cast<T*>(f.scale_gradient)[c] = (T)(inv_std * acc[1]);
     const T d_var_d_out = (T)(d_var * acc[2]);
@@ -393,8 +395,6 @@ __global__ void __launch_bounds__(kBlock) bn_finish_kernel(const BnArgs a, const
     running_means[c] = (T)((double)mean * ave_lerp + (double)new_mean * (double)ave_factor);
     running_variances[c] =
         (T)((double)variance * ave_lerp + (double)(T)(new_var / running_count_val) * (double)ave_factor);
-    bn_store_normalize_params<T>(pm, new_mean, batch_variance, reinterpret_cast<const T*>(f.scale)[c],
-                                 reinterpret_cast<const T*>(f.bias)[c], f.epsilon);
   }
 }
 
@@ -429,9 +429,8 @@ __global__ void __launch_bounds__(kBlock) bn_apply_col_kernel(const BnArgs a) {
 #pragma unroll
   for (int e = 0; e < VEC; ++e) {
     const uint32_t ch = a.e_fd.div((uint32_t)(j0 + e));
-    const double* pm = a.params + (int64_t)ch * kParamStride;
 #pragma unroll
-    for (int k = 0; k < NP; ++k) p[e][k] = pm[k];
+    for (int k = 0; k < NP; ++k) p[e][k] = bn_channel_constant<T, MODE>(a, ch, k);
   }
   const int64_t b0 = (int64_t)blockIdx.y * a.apply_rows_per_seg;
   const int64_t nb = a.B - b0 < (int64_t)a.apply_rows_per_seg ? a.B - b0 : (int64_t)a.apply_rows_per_seg;
@@ -491,7 +490,7 @@ __global__ void __launch_bounds__(kBlock) bn_apply_kernel(const BnArgs a) {
     const uint32_t slot = i / NP, k = i - slot * NP;
     uint32_t q, ch;
     a.c_fd.divmod(ch_base + slot, q, ch);
-    table[i] = a.params[(int64_t)ch * kParamStride + k];
+    table[i] = bn_channel_constant<T, MODE>(a, ch, (int)k);
   }
   __syncthreads();
 #pragma unroll
@@ -659,14 +658,18 @@ void bn_launch_apply(hipStream_t s, const BnPlan& plan) {
 
 inline dim3 channel_grid(int64_t C, int per_block) { return dim3((uint32_t)((C + per_block - 1) / per_block)); }
 
+inline void bn_set_statistics(BnArgs* a, const void* means, const void* variances, const void* scale, const void* bias,
+                              double epsilon) {
+  a->means = means; a->variances = variances; a->scale = scale; a->bias = bias; a->epsilon = epsilon;
+}
+
 template <class T>
 int bn_normalize(hipStream_t s, void* output, const void* input, const void* means, const void* variances,
                  const void* scale, const void* bias, double epsilon, int64_t B, int64_t C, int64_t E) {
   BnPlan plan;
   if (int rc = bn_plan<T, kBnNormalize>(s, B, C, E, input, nullptr, output, false, &plan)) return rc;
-  note_kernel("bn_apply");
-  hipLaunchKernelGGL((bn_prepare_normalize_kernel<T>), channel_grid(C, kBlock), dim3(kBlock), 0, s, plan.a.params,
-                     (const T*)means, (const T*)variances, (const T*)scale, (const T*)bias, epsilon, C);
+  bn_set_statistics(&plan.a, means, variances, scale, bias, epsilon);
+  note_kernel(plan.col_style ? "bn_apply_col" : "bn_apply");
   bn_launch_apply<T, kBnNormalize>(s, plan);
   return after_launch(s);
 }
@@ -677,14 +680,15 @@ int bn_update_and_apply(hipStream_t s, void* output, const void* input, void* ba
                         const void* bias, double epsilon, int64_t B, int64_t C, int64_t E) {
   BnPlan plan;
   if (int rc = bn_plan<T, kBnNormalize>(s, B, C, E, input, nullptr, output, true, &plan)) return rc;
+  // the apply pass normalizes with the batch statistics the finishing pass writes
+  bn_set_statistics(&plan.a, batch_means, batch_variances, scale, bias, epsilon);
   note_kernel(plan.col_style ? "bn_update_col" : "bn_update_row");
   bn_launch_stats<T, kBnNormalize>(s, plan);
   BnFinish f;
   std::memset(&f, 0, sizeof(f));
   f.batch_means = batch_means; f.batch_variances = batch_variances;
   f.running_means = running_means; f.running_variances = running_variances;
-  f.scale = scale; f.bias = bias;
-  f.average_factor = average_factor; f.epsilon = epsilon;
+  f.average_factor = average_factor;
   hipLaunchKernelGGL((bn_finish_kernel<T, kBnNormalize>), channel_grid(C, kBlock / 64), dim3(kBlock), 0, s, plan.a, f);
   bn_launch_apply<T, kBnNormalize>(s, plan);
   return after_launch(s);
@@ -696,9 +700,8 @@ int bn_gradients(hipStream_t s, void* input_gradient, void* scale_gradient, void
                  const void* scale, double epsilon, int64_t B, int64_t C, int64_t E) {
   BnPlan plan;
   if (int rc = bn_plan<T, kBnGradient>(s, B, C, E, input, output_gradient, input_gradient, true, &plan)) return rc;
+  bn_set_statistics(&plan.a, batch_means, batch_variances, scale, nullptr, epsilon);
   note_kernel(plan.col_style ? "bn_gradients_col" : "bn_gradients_row");
-  hipLaunchKernelGGL((bn_prepare_gradient_kernel<T>), channel_grid(C, kBlock), dim3(kBlock), 0, s, plan.a.params,
-                     (const T*)batch_means, (const T*)batch_variances, (const T*)scale, epsilon, C);
   bn_launch_stats<T, kBnGradient>(s, plan);
   BnFinish f;
   std::memset(&f, 0, sizeof(f));

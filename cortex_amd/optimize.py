@@ -1,12 +1,13 @@
 """Gradient optimizers of the tensor-math path: a Python mirror of
-``src/cortex/optimize.clj:5-24``, ``src/cortex/optimize/adam.clj:116-200`` and
-``src/cortex/optimize/adadelta.clj:19-132``.
+``src/cortex/optimize.clj:5-24``, ``src/cortex/optimize/adam.clj:116-200``,
+``src/cortex/optimize/adadelta.clj:19-132`` and ``src/cortex/optimize/sgd.clj``.
 
 An optimizer object implements ``PGradientOptimizer``: ``batch_update`` is
 called once per batch, ``compute_parameters`` once per parameter buffer with
 the running ``offset`` of that buffer inside the flat optimizer state
-(``src/cortex/nn/compute_binding.clj:817-854``).  The step itself is one fused
-kernel on the backend's stream.
+(``src/cortex/nn/compute_binding.clj:817-854``).  The Adam and Adadelta steps
+are one fused kernel each on the backend's stream; SGD is, as in the reference,
+four calls of the tensor API.
 """
 from __future__ import annotations
 
@@ -23,6 +24,13 @@ def adam(**kwargs) -> dict:
 def adadelta(**kwargs) -> dict:
     """Default Adadelta description (``adadelta.clj:124-132``)."""
     out = {"type": "adadelta", "decay": 0.05, "epsilon": 1e-6}
+    out.update(kwargs)
+    return out
+
+
+def sgd(**kwargs) -> dict:
+    """Default SGD description (``sgd.clj:74-80``)."""
+    out = {"type": "sgd", "learning-rate": 0.001, "momentum": 0.9}
     out.update(kwargs)
     return out
 
@@ -88,6 +96,41 @@ class Adadelta:
                                           da.sub_buffer(offset, da.ecount() - offset), gradient_alpha, g, p, g.ecount())
 
 
+@dataclasses.dataclass
+class SGD:
+    backend: Backend
+    optimizer: dict
+    _temp: object = None   # the allocator's reusable :sgd-temp tensor (sgd.clj:27)
+
+    def batch_update(self, optimizer_parameters=None) -> "SGD":
+        return self
+
+    def compute_parameters(self, state: dict, gradient_alpha, offset: int, gradient, parameters) -> None:
+        """``tensor-sgd`` (``sgd.clj:16-40``): momentum with the look-ahead correction,
+            dxm = momentum * v;  v = dxm + learning-rate * gradient-alpha * g;
+            dx = dxm - (1 + momentum) * v;  p = p + dx
+        as one ``unary-op!`` and three ``binary-op!`` calls."""
+        from . import tensor as ct
+        from . import dimensions as dims
+
+        g, p, mv = _buffer(gradient), _buffer(parameters), _buffer(state["momentum-vals"])
+        _ensure_datatype(self.backend.datatype, g, p, mv)
+        n = g.ecount()
+        device = self.backend.stream.get_device()
+        vec = lambda buf, count: ct.Tensor(device, dims.dimensions([count]), buf)
+        momentum = float(self.optimizer["momentum"])
+        with ct.tensor_context(self.backend.stream, self.backend.datatype):
+            grad, params = vec(g, n), vec(p, p.ecount())
+            momentum_vals = vec(mv.sub_buffer(offset, n), n)
+            if self._temp is None or self._temp.ecount() < n:
+                self._temp = ct.new_tensor([n], init_value=None)
+            temp = vec(self._temp.buffer.sub_buffer(0, n), n)
+            dxm = ct.unary_op(temp, momentum, momentum_vals, "noop")
+            ct.binary_op(momentum_vals, 1.0, dxm, float(self.optimizer["learning-rate"]) * float(gradient_alpha), grad, "+")
+            dx = ct.binary_op(temp, 1.0, dxm, 1 + momentum, momentum_vals, "-")
+            ct.binary_op(params, 1.0, params, 1.0, dx, "+")
+
+
 def create_optimizer(backend: Backend, optimizer: dict):
     """``create-optimizer`` multimethod on ``[(:type backend) (:type optimizer)]``
     (``optimize.clj:19-24``)."""
@@ -98,4 +141,6 @@ def create_optimizer(backend: Backend, optimizer: dict):
         return Adam(backend, optimizer)
     if kind == "adadelta":
         return Adadelta(backend, optimizer)
+    if kind == "sgd":
+        return SGD(backend, optimizer)
     raise KeyError(f"No optimizer {kind!r} for backend {backend.type!r}")

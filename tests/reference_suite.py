@@ -672,3 +672,26 @@ def adam_trajectory(driver, datatype):
             # about-there?: sum of absolute differences below 1e-6 (src/cortex/verify/utils.clj:20-27)
             assert np.abs(guess1 - np.array(answer)).sum() < 1e-6, (guess1, answer)
             assert np.abs(guess2 - np.array([1.0, 2.0, 3.0, 4.0])).sum() < 1e-6, guess2
+
+
+# src/cortex/optimize/sgd.clj:16-40.  The reference holds no stored vector for SGD (it is only
+# exercised by MNIST training, verify/nn/train.clj); the update rule is checked in closed form.
+def sgd_closed_form(driver, datatype):
+    from cortex_amd import optimize as opt
+
+    with context(driver, datatype) as stream:
+        backend = opt.Backend(stream=stream, datatype=datatype, type=getattr(driver, "type", "hip"))
+        rng = np.random.default_rng(80)
+        p0, v0 = rng.standard_normal(6), rng.standard_normal(10)
+        params, momentum_vals = ct.to_tensor(p0), ct.to_tensor(v0)
+        optimizer = opt.create_optimizer(backend, opt.sgd(**{"learning-rate": 0.01, "momentum": 0.8}))
+        p, v = p0.copy(), v0.copy()
+        for step in range(3):
+            g = rng.standard_normal(6)
+            optimizer.compute_parameters({"momentum-vals": momentum_vals}, 0.5, 4, ct.to_tensor(g), params)
+            dxm = 0.8 * v[4:]
+            v[4:] = dxm + 0.01 * 0.5 * g
+            p = p + (dxm - 1.8 * v[4:])
+            tol = 1e-12 if datatype == "double" else 1e-5
+            equals(p, ct.to_double_array(params), tol)
+            equals(v, ct.to_double_array(momentum_vals), tol)

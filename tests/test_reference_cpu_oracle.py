@@ -11,7 +11,7 @@ ALL_DTYPE_TESTS = ["assign_constant", "assign_marshal", "binary_constant_op", "b
                    "indexed_tensor", "simple_stream"]
 FLOAT_TESTS = ["gemm", "gemv", "activation_forward", "activation_gradient", "softmax", "batch_normalize",
                "batch_normalize_update_and_apply", "batch_normalize_gradients", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
-               "adam_trajectory"]
+               "adam_trajectory", "sgd_closed_form"]
 
 
 @pytest.fixture(scope="module")
