@@ -22,7 +22,11 @@ void common_vec(const Plan& plan, const EwOperand* ops, VecArgs* a) {
   std::memset(a, 0, sizeof(*a));
   a->n_outer = c.nd - 1;
   a->streaming = is_streaming(plan, ops) ? 1u : 0u;
-  for (int d = 0; d + 1 < c.nd; ++d) a->outer_fd[d] = FastDiv((uint32_t)c.size[d + 1]);
+  for (int d = 0; d + 1 < c.nd; ++d) {
+    if (d < 2) a->outer_fd01[d] = FastDiv((uint32_t)c.size[d + 1]);
+    else a->outer_fd_hi[d - 2] = FastDiv((uint32_t)c.size[d + 1]);
+  }
+  for (int d = std::max(c.nd - 1, 0); d < 2; ++d) a->outer_fd01[d] = FastDiv(1);
   for (int k = 0; k < plan.n_ops; ++k) {
     a->ptr[k] = (char*)ops[k].ptr;
     a->cbits[k] = ops[k].cbits;
@@ -32,7 +36,10 @@ void common_vec(const Plan& plan, const EwOperand* ops, VecArgs* a) {
     for (int d = 0; d < c.nd; ++d)
       if (c.stride[k][d] == 0 && c.size[d] > 1) once = false;
     if (once) a->nt_mask |= 1u << k;
-    for (int d = 0; d + 1 < c.nd; ++d) a->outer_stride[k][d] = c.stride[k][d + 1];
+    for (int d = 0; d + 1 < c.nd; ++d) {
+      if (d < 2) a->outer_stride01[k][d] = c.stride[k][d + 1];
+      else a->outer_stride_hi[k][d - 2] = c.stride[k][d + 1];
+    }
   }
 }
 }  // namespace
@@ -56,18 +63,22 @@ int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_
   if (aligned && c.nd == 1 && inner < vmax) aligned = false;
 
   common_vec(plan, ops, main_args);
+  // The kernel decomposes a 32-bit vector index; a flat call is one row of up to
+  // kVecLaunchMax vectors per launch (launch_vec walks longer ones in pieces).
   if (!aligned) {
     *main_vec = 1;
-    main_args->inner_vecs = (uint32_t)std::min<int64_t>(inner, kLim31 - 1);
+    main_args->inner_vecs = (uint32_t)std::min<int64_t>(inner, kVecLaunchMax);
     main_args->inner_fd = FastDiv(main_args->inner_vecs);
     main_args->total_vecs = (uint64_t)inner * (uint64_t)rows;
+    CT_REQUIRE(c.nd == 1 || main_args->total_vecs < (uint64_t)kLim31, "tensor too large for 32-bit vector indexing");
     return CT_OK;
   }
   *main_vec = vmax;
   const int64_t inner_vecs = inner / vmax;
-  main_args->inner_vecs = (uint32_t)std::min<int64_t>(inner_vecs, kLim31 - 1);
+  main_args->inner_vecs = (uint32_t)std::min<int64_t>(inner_vecs, kVecLaunchMax);
   main_args->inner_fd = FastDiv(main_args->inner_vecs);
   main_args->total_vecs = (uint64_t)inner_vecs * (uint64_t)rows;
+  CT_REQUIRE(c.nd == 1 || main_args->total_vecs < (uint64_t)kLim31, "tensor too large for 32-bit vector indexing");
   const int64_t tail = inner - inner_vecs * vmax;  // only possible when flat
   if (tail > 0) {
     *has_tail = true;

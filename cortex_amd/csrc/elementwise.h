@@ -13,6 +13,8 @@
 //   ew_gen_kernel   per-element addressing with the reference's address objects
 #pragma once
 
+#include <algorithm>
+
 #include "common.h"
 #include "plan.h"
 
@@ -21,6 +23,7 @@ namespace cthip {
 template <class T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 
 constexpr int kBlock = 256;
+constexpr int64_t kVecLaunchMax = int64_t(1) << 30;  // vectors one launch of the vector kernel indexes
 
 template <class T> __device__ __forceinline__ T const_from_bits(uint64_t bits) {
   T c;
@@ -58,35 +61,43 @@ template <class T> inline uint64_t bits_of(T c) {
 
 // ------------------------------------------------------------------ VEC
 
+// The first block of members is everything a lane needs when the operands have
+// at most two outer axes; the kernel fetches it in one batch (see ew_vec_kernel).
 struct VecArgs {
   uint64_t total_vecs;
-  uint32_t inner_vecs;
   FastDiv inner_fd;
   int32_t n_outer;
-  FastDiv outer_fd[CT_MAX_DIMS - 1];
+  FastDiv outer_fd01[2];  // an absent axis has size 1 (and stride 0)
+  uint32_t unit_mask;     // bit k: operand k is unit-stride along the inner axis
+  uint32_t const_mask;    // bit k: operand k is a scalar constant
+  uint32_t nt_mask;       // bit k: operand k is read exactly once (no broadcast axis), so its loads may bypass the caches
+  uint32_t streaming;     // the call moves more data than the caches hold: non-temporal loads
   char* ptr[kMaxOps];
-  int64_t outer_stride[kMaxOps][CT_MAX_DIMS - 1];
-  uint32_t unit_mask;   // bit k: operand k is unit-stride along the inner axis
-  uint32_t const_mask;  // bit k: operand k is a scalar constant
-  uint32_t streaming;   // the call moves more data than the caches hold: non-temporal loads
-  uint32_t nt_mask;     // bit k: operand k is read exactly once (no broadcast axis), so its loads may bypass the caches
+  int64_t outer_stride01[kMaxOps][2];
   uint64_t cbits[kMaxOps];
+  // outer axes beyond the second
+  FastDiv outer_fd_hi[CT_MAX_DIMS - 3];
+  int64_t outer_stride_hi[kMaxOps][CT_MAX_DIMS - 3];
+  uint32_t inner_vecs;
 };
 
+// Operand k of one lane: a constant, VEC consecutive elements, or one element
+// broadcast along the inner axis.  vp / sp are the lane's vector and scalar
+// addresses, computed by the caller before any branch.
 template <class T, int VEC, bool STREAM>
-__device__ __forceinline__ Vec<T, VEC> vec_load(const VecArgs& a, int k, int64_t base, int64_t col) {
+__device__ __forceinline__ Vec<T, VEC> vec_load(uint32_t const_mask, uint32_t unit_mask, uint32_t nt_mask, uint64_t cbits,
+                                                int k, const Vec<T, VEC>* vp, const T* sp) {
   Vec<T, VEC> r;
-  if ((a.const_mask >> k) & 1u) {
-    const T c = const_from_bits<T>(a.cbits[k]);
+  if ((const_mask >> k) & 1u) {
+    const T c = const_from_bits<T>(cbits);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) r.v[i] = c;
-  } else if ((a.unit_mask >> k) & 1u) {
-    const Vec<T, VEC>* p = reinterpret_cast<const Vec<T, VEC>*>(reinterpret_cast<const T*>(a.ptr[k]) + base + col);
+  } else if ((unit_mask >> k) & 1u) {
     // a broadcast operand (a bias row, say) is re-read by every outer index and must stay cached
-    if (STREAM && ((a.nt_mask >> k) & 1u)) r = nt_load(p);
-    else r = *p;
+    if (STREAM && ((nt_mask >> k) & 1u)) r = nt_load(vp);
+    else r = *vp;
   } else {
-    const T c = reinterpret_cast<const T*>(a.ptr[k])[base];
+    const T c = *sp;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) r.v[i] = c;
   }
@@ -95,10 +106,19 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(const VecArgs& a, int k, int64_t
 
 // One 16-byte vector per lane.  On this part one vector per lane with many
 // resident blocks sustains more bandwidth than several vectors per lane, and
-// non-temporal loads and stores add about 8 % on streams larger than the caches.
+// non-temporal loads add a few percent on streams larger than the caches.
 // STREAM is a template parameter: a run-time choice between a plain and a
 // non-temporal access to the same address is folded into one plain access by
 // the compiler, which loses the hint.
+//
+// A wave lives about as long as one trip to memory, so every scalar fetch of a
+// kernel argument that sits between the wave's start and its first vector load
+// costs bandwidth, and the compiler fetches an argument next to its first use,
+// inside whatever branch that is.  The kernel therefore names every argument it
+// needs in one empty asm statement at the top: they are fetched in one batch
+// with one wait, and the code that follows only touches registers.  For the
+// same reason there is no special case for flat operands: the host describes
+// them as one row (absent outer axes have size 1 and stride 0).
 template <class F, int VEC, bool STREAM>
 __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs a) {
   using Out = typename F::Out;
@@ -107,30 +127,89 @@ __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs
   using In2 = typename F::In2;
   constexpr int NIN = F::NIN;
 
-  const uint64_t v = (uint64_t)blockIdx.x * (uint64_t)kBlock + threadIdx.x;
-  if (v >= a.total_vecs) return;
-  int64_t off[kMaxOps] = {0, 0, 0, 0};
+  const uint64_t total = a.total_vecs;
+  const FastDiv ifd = a.inner_fd, fd0 = a.outer_fd01[0], fd1 = a.outer_fd01[1];
+  const int32_t n_outer = a.n_outer;
+  const uint32_t unit_mask = a.unit_mask, const_mask = a.const_mask, nt_mask = a.nt_mask;
+  char* const b0 = a.ptr[0];
+  char* const b1 = a.ptr[NIN >= 1 ? 1 : 0];
+  char* const b2 = a.ptr[NIN >= 2 ? 2 : 0];
+  char* const b3 = a.ptr[NIN >= 3 ? 3 : 0];
+  const int64_t s00 = a.outer_stride01[0][0], s01 = a.outer_stride01[0][1];
+  const int64_t s10 = a.outer_stride01[NIN >= 1 ? 1 : 0][0], s11 = a.outer_stride01[NIN >= 1 ? 1 : 0][1];
+  const int64_t s20 = a.outer_stride01[NIN >= 2 ? 2 : 0][0], s21 = a.outer_stride01[NIN >= 2 ? 2 : 0][1];
+  const int64_t s30 = a.outer_stride01[NIN >= 3 ? 3 : 0][0], s31 = a.outer_stride01[NIN >= 3 ? 3 : 0][1];
+  const uint64_t c1 = a.cbits[NIN >= 1 ? 1 : 0], c2 = a.cbits[NIN >= 2 ? 2 : 0], c3 = a.cbits[NIN >= 3 ? 3 : 0];
+  asm volatile("" ::"s"(total), "s"(ifd.d), "s"(ifd.m), "s"(ifd.s), "s"(fd0.d), "s"(fd0.m), "s"(fd0.s), "s"(fd1.d),
+               "s"(fd1.m), "s"(fd1.s), "s"(n_outer), "s"(unit_mask), "s"(const_mask), "s"(nt_mask), "s"(b0), "s"(b1),
+               "s"(b2), "s"(b3), "s"(s00), "s"(s01), "s"(s10), "s"(s11), "s"(s20), "s"(s21), "s"(s30), "s"(s31),
+               "s"(c1), "s"(c2), "s"(c3));
+
+  const uint64_t v_first = (uint64_t)blockIdx.x * (uint64_t)kBlock;  // the block's first vector
+  if (v_first + threadIdx.x >= total) return;
+  // Offsets of the outer index `row` for every operand.  Called with a
+  // wave-uniform row this is scalar arithmetic.
+  auto outer_offsets = [&](uint32_t row, int64_t* off) {
+    uint32_t q0, r0, q1, r1;
+    fd0.divmod(row, q0, r0);
+    fd1.divmod(q0, q1, r1);
+    off[0] = (int64_t)r0 * s00 + (int64_t)r1 * s01;
+    off[1] = (int64_t)r0 * s10 + (int64_t)r1 * s11;
+    off[2] = (int64_t)r0 * s20 + (int64_t)r1 * s21;
+    off[3] = (int64_t)r0 * s30 + (int64_t)r1 * s31;
+    if (n_outer > 2) {
+      row = q1;
+      for (int d = 2; d < n_outer; ++d) {
+        uint32_t q, r;
+        a.outer_fd_hi[d - 2].divmod(row, q, r);
+        row = q;
+#pragma unroll
+        for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride_hi[k][d - 2];
+      }
+    }
+  };
+  int64_t off[kMaxOps];
   int64_t col;
-  if (a.n_outer == 0) {
-    col = (int64_t)v * VEC;
+  if (ifd.d >= (uint32_t)kBlock) {
+    // Rows of at least a block's width: the block's 256 vectors lie in at most two
+    // rows, whose offsets are computed once per wave on the scalar unit; a lane
+    // only picks its row.
+    uint32_t row_a, cv_a;
+    ifd.divmod((uint32_t)v_first, row_a, cv_a);
+    outer_offsets(row_a, off);
+    uint32_t cv = cv_a + threadIdx.x;
+    if (cv_a + (uint32_t)kBlock > ifd.d) {  // the block runs into the next row
+      int64_t off_b[kMaxOps];
+      outer_offsets(row_a + 1, off_b);
+      const bool next = cv >= ifd.d;
+      cv -= next ? ifd.d : 0u;
+#pragma unroll
+      for (int k = 0; k < kMaxOps; ++k) off[k] = next ? off_b[k] : off[k];
+    }
+    col = (int64_t)cv * VEC;
   } else {
     uint32_t row, cv;
-    a.inner_fd.divmod((uint32_t)v, row, cv);
+    ifd.divmod((uint32_t)v_first + threadIdx.x, row, cv);
     col = (int64_t)cv * VEC;
-    for (int d = 0; d < a.n_outer; ++d) {
-      uint32_t q, r;
-      a.outer_fd[d].divmod(row, q, r);
-      row = q;
-#pragma unroll
-      for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
-    }
+    outer_offsets(row, off);
   }
+  char* const base[kMaxOps] = {b0, b1, b2, b3};
+  const uint64_t cbits[kMaxOps] = {0, c1, c2, c3};
   Vec<In0, VEC> x0;
   Vec<In1, VEC> x1;
   Vec<In2, VEC> x2;
-  if constexpr (NIN >= 1) x0 = vec_load<In0, VEC, STREAM>(a, 1, off[1], col);
-  if constexpr (NIN >= 2) x1 = vec_load<In1, VEC, STREAM>(a, 2, off[2], col);
-  if constexpr (NIN >= 3) x2 = vec_load<In2, VEC, STREAM>(a, 3, off[3], col);
+  if constexpr (NIN >= 1) {
+    const In0* sp = reinterpret_cast<const In0*>(base[1]) + off[1];
+    x0 = vec_load<In0, VEC, STREAM>(const_mask, unit_mask, nt_mask, cbits[1], 1, reinterpret_cast<const Vec<In0, VEC>*>(sp + col), sp);
+  }
+  if constexpr (NIN >= 2) {
+    const In1* sp = reinterpret_cast<const In1*>(base[2]) + off[2];
+    x1 = vec_load<In1, VEC, STREAM>(const_mask, unit_mask, nt_mask, cbits[2], 2, reinterpret_cast<const Vec<In1, VEC>*>(sp + col), sp);
+  }
+  if constexpr (NIN >= 3) {
+    const In2* sp = reinterpret_cast<const In2*>(base[3]) + off[3];
+    x2 = vec_load<In2, VEC, STREAM>(const_mask, unit_mask, nt_mask, cbits[3], 3, reinterpret_cast<const Vec<In2, VEC>*>(sp + col), sp);
+  }
   Vec<Out, VEC> r;
 #pragma unroll
   for (int i = 0; i < VEC; ++i) {
@@ -142,7 +221,7 @@ __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs
     if constexpr (NIN >= 3) p2 = x2.v[i];
     r.v[i] = f(p0, p1, p2);
   }
-  Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(a.ptr[0]) + off[0] + col);
+  Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(base[0]) + off[0] + col);
   *dp = r;  // plain stores: non-temporal ones measured no faster here and slower for narrow inputs
 }
 
@@ -455,11 +534,29 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_b_edge, TileAr
 int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use64, uint32_t* grid);
 
 template <class F, int VEC>
-inline void launch_vec(hipStream_t s, const F& f, const VecArgs& a) {
-  if (a.total_vecs == 0) return;
+inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& a) {
   const dim3 grid((uint32_t)((a.total_vecs + kBlock - 1) / kBlock));
   if (a.streaming) hipLaunchKernelGGL((ew_vec_kernel<F, VEC, true>), grid, dim3(kBlock), 0, s, f, a);
   else hipLaunchKernelGGL((ew_vec_kernel<F, VEC, false>), grid, dim3(kBlock), 0, s, f, a);
+}
+
+// A flat call longer than one launch's 32-bit vector index is walked in pieces.
+template <class F, int VEC>
+inline void launch_vec(hipStream_t s, const F& f, const VecArgs& a) {
+  if (a.total_vecs == 0) return;
+  if (a.n_outer > 0 || a.total_vecs <= (uint64_t)kVecLaunchMax) {
+    launch_vec_once<F, VEC>(s, f, a);
+    return;
+  }
+  const size_t elem[kMaxOps] = {sizeof(typename F::Out), sizeof(typename F::In0), sizeof(typename F::In1),
+                                sizeof(typename F::In2)};
+  for (uint64_t first = 0; first < a.total_vecs; first += (uint64_t)kVecLaunchMax) {
+    VecArgs piece = a;
+    piece.total_vecs = std::min<uint64_t>((uint64_t)kVecLaunchMax, a.total_vecs - first);
+    for (int k = 0; k <= F::NIN; ++k)
+      if (((a.unit_mask >> k) & 1u) && !((a.const_mask >> k) & 1u)) piece.ptr[k] = a.ptr[k] + first * VEC * elem[k];
+    launch_vec_once<F, VEC>(s, f, piece);
+  }
 }
 
 // ops[0] is the destination; ops[1..NIN] the inputs in functor order.

@@ -810,3 +810,55 @@ def test_gemm_errors(P):
         H.gemm(P.hip, View(xi, [16]), 4, False, False, 1, View(xi, [16]), 4, 4, 4, View(xi, [16]), 4, 4, 0)
     with pytest.raises(capi.CortexHipError, match="column stride"):
         H.gemm(P.hip, v, 2, False, False, 1, v, 4, 4, 4, v, 4, 4, 0)
+
+
+# ------------------------------------------------------------------ vector kernel: rows at least a block wide
+# Blocks of 256 vectors that start in one row and end in the next, with one, two and three outer axes.
+
+@pytest.mark.parametrize("code", [capi.F32, capi.F64, capi.I16])
+def test_wide_rows_crossing_blocks(P, code):
+    rng = np.random.default_rng(90)
+    f = NP[code]
+    for shape, y_shape in (((5, 1200), (1200,)), ((5, 1200), (5, 1)), ((3, 5, 1208), (5, 1)), ((2, 3, 2, 1300), (3, 1, 1)),
+                           ((2, 2, 3, 2, 1100), (2, 1, 1, 1))):
+        n = int(np.prod(shape))
+        x, y = P.buf(values(rng, code, n)), P.buf(values(rng, code, int(np.prod(y_shape))))
+        d = P.buf(np.zeros(n, f))
+        k = P.run(H.binary_op, View(d, shape), View(x, shape), 1.0, View(y, y_shape), 1.0, "+")
+        assert k == "vec"
+        compare(d, f"binary-op! :+ {shape} + {y_shape}")
+        # pitched rows (a sub-matrix) keep two outer axes apart
+        pitch = shape[-1] + 8
+        rows = n // shape[-1]
+        xp = P.buf(values(rng, code, rows * pitch))
+        k = P.run(H.binary_op, View(d, [rows, shape[-1]]), View(xp, [rows, shape[-1]], [pitch, 1]), 1.0,
+                  View(y, [1]), 2.0, "*")
+        compare(d, f"binary-op! :* pitched {shape}")
+
+
+def test_flat_call_longer_than_one_launch():
+    """A flat call of more than 2^30 vectors (16 GiB of bytes) is walked in pieces."""
+    import ctypes as C
+    n = (1 << 34) + 4096 + 5
+    free, total = C.c_size_t(), C.c_size_t()
+    capi.call("ct_memory_info", C.byref(free), C.byref(total))
+    if free.value < 2 * n + (1 << 30):
+        pytest.skip("needs 33 GiB of free device memory")
+    a, b = C.c_void_p(), C.c_void_p()
+    capi.call("ct_malloc", C.byref(a), n)
+    capi.call("ct_malloc", C.byref(b), n)
+    try:
+        dims1 = capi.make_dims([n], [1])
+        capi.call("ct_memset", None, a, capi.I8, 7.0, n)
+        capi.call("ct_binary_op_constant", None, b, C.byref(dims1), a, C.byref(dims1), 1.0, 5.0, n, capi.BINARY_OPS["+"], 0,
+                  capi.I8)
+        capi.call("ct_stream_sync", None)
+        assert capi.last_kernel() == "vec"
+        for start in (0, (1 << 34) - 2048, (1 << 34) - 8, n - 4096):
+            out = np.zeros(4096 if start + 4096 <= n else n - start, np.int8)
+            capi.call("ct_memcpy_async", out.ctypes.data, b.value + start, out.nbytes, capi.COPY_D2H, None)
+            capi.call("ct_stream_sync", None)
+            assert np.all(out == 12), (start, out[:16])
+    finally:
+        capi.call("ct_free", a)
+        capi.call("ct_free", b)
