@@ -278,6 +278,18 @@ __device__ __forceinline__ void tile_read(T* v, const T* p, int64_t step, uint32
   }
 }
 
+// Reads this lane's share of the tile of an operand that needs no transposition:
+// element i of the lane is (a = wx, b = wy + i * rows_w), the write-phase layout.
+template <class T, int IT, bool FULL>
+__device__ __forceinline__ void tile_read_direct(T* v, const T* q, int64_t step, bool a_ok, uint32_t b_left, int wy,
+                                                 int rows_w) {
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    if (FULL || (a_ok && (uint32_t)(wy + i * rows_w) < b_left)) v[i] = q[(int64_t)i * step];
+    else v[i] = T{};
+  }
+}
+
 // Transposes the lane values through the block's single LDS tile (rows padded
 // to TB + 1 elements: conflict-free both ways).  On entry v[i] holds element
 // (a = ty + i*ROWS_R, b = tx) with tx = t % TB; on exit element
@@ -315,26 +327,7 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   const bool t0 = NIN >= 1 && ((a.lds_mask >> 1) & 1u), t1 = NIN >= 2 && ((a.lds_mask >> 2) & 1u),
              t2 = NIN >= 3 && ((a.lds_mask >> 3) & 1u);
 
-  // phase 1: every load of every transposed operand is issued before the first LDS round
-  In0 v0[IT];
-  In1 v1[IT];
-  In2 v2[IT];
-  const bool b_ok = (uint32_t)tx < b_left;
-  if constexpr (NIN >= 1)
-    if (t0) tile_read<In0, TB, FULL, STREAM>(v0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
-                                     (int64_t)ROWS_R * a.strideA[1], a_left, b_ok, ty);
-  if constexpr (NIN >= 2)
-    if (t1) tile_read<In1, TB, FULL, STREAM>(v1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
-                                     (int64_t)ROWS_R * a.strideA[2], a_left, b_ok, ty);
-  if constexpr (NIN >= 3)
-    if (t2) tile_read<In2, TB, FULL, STREAM>(v2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
-                                     (int64_t)ROWS_R * a.strideA[3], a_left, b_ok, ty);
-  bool used = false;
-  if constexpr (NIN >= 1) if (t0) { tile_transpose<In0, TB>(v0, smem, used); used = true; }
-  if constexpr (NIN >= 2) if (t1) { tile_transpose<In1, TB>(v1, smem, used); used = true; }
-  if constexpr (NIN >= 3) if (t2) { tile_transpose<In2, TB>(v2, smem, used); used = true; }
-
-  // phase 2: lane wx walks A (the destination's unit-stride axis), lane rows walk B
+  // Addresses of the write phase, formed now: nothing after the LDS rounds needs a kernel argument again.
   const bool a_ok = (uint32_t)wx < a_left;
   Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + off[0] + (int64_t)(a0 + wx) * a.strideA[0] + (int64_t)(b0 + wy) * a.strideB[0];
   const int64_t dstep = (int64_t)ROWS_W * a.strideB[0];
@@ -357,6 +350,35 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
     if ((a.const_mask >> 3) & 1u) c2 = const_from_bits<In2>(a.cbits[3]);
     else if (!t2) { q2 = reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + wx) * a.strideA[3] + (int64_t)(b0 + wy) * a.strideB[3]; s2 = (int64_t)ROWS_W * a.strideB[3]; }
   }
+
+  // phase 1: every load of every transposed operand is issued before the first LDS round
+  In0 v0[IT];
+  In1 v1[IT];
+  In2 v2[IT];
+  const bool b_ok = (uint32_t)tx < b_left;
+  if constexpr (NIN >= 1)
+    if (t0) tile_read<In0, TB, FULL, STREAM>(v0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
+                                     (int64_t)ROWS_R * a.strideA[1], a_left, b_ok, ty);
+  if constexpr (NIN >= 2)
+    if (t1) tile_read<In1, TB, FULL, STREAM>(v1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
+                                     (int64_t)ROWS_R * a.strideA[2], a_left, b_ok, ty);
+  if constexpr (NIN >= 3)
+    if (t2) tile_read<In2, TB, FULL, STREAM>(v2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
+                                     (int64_t)ROWS_R * a.strideA[3], a_left, b_ok, ty);
+  // operands that are read along A directly (not through LDS) are fetched now as well, so
+  // that their latency overlaps the transposed operands' instead of following the LDS rounds
+  if constexpr (NIN >= 1)
+    if (q0) tile_read_direct<In0, IT, FULL>(v0, q0, s0, a_ok, b_left, wy, ROWS_W);
+  if constexpr (NIN >= 2)
+    if (q1) tile_read_direct<In1, IT, FULL>(v1, q1, s1, a_ok, b_left, wy, ROWS_W);
+  if constexpr (NIN >= 3)
+    if (q2) tile_read_direct<In2, IT, FULL>(v2, q2, s2, a_ok, b_left, wy, ROWS_W);
+  bool used = false;
+  if constexpr (NIN >= 1) if (t0) { tile_transpose<In0, TB>(v0, smem, used); used = true; }
+  if constexpr (NIN >= 2) if (t1) { tile_transpose<In1, TB>(v1, smem, used); used = true; }
+  if constexpr (NIN >= 3) if (t2) { tile_transpose<In2, TB>(v2, smem, used); used = true; }
+
+  // phase 2: lane wx walks A (the destination's unit-stride axis), lane rows walk B
 #pragma unroll
   for (int i = 0; i < IT; ++i) {
     const int row = wy + i * ROWS_W;
@@ -364,9 +386,9 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
       In0 p0 = c0;
       In1 p1 = c1;
       In2 p2 = c2;
-      if constexpr (NIN >= 1) { if (t0) p0 = v0[i]; else if (q0) p0 = q0[(int64_t)i * s0]; }
-      if constexpr (NIN >= 2) { if (t1) p1 = v1[i]; else if (q1) p1 = q1[(int64_t)i * s1]; }
-      if constexpr (NIN >= 3) { if (t2) p2 = v2[i]; else if (q2) p2 = q2[(int64_t)i * s2]; }
+      if constexpr (NIN >= 1) { if (t0 || q0) p0 = v0[i]; }
+      if constexpr (NIN >= 2) { if (t1 || q1) p1 = v1[i]; }
+      if constexpr (NIN >= 3) { if (t2 || q2) p2 = v2[i]; }
       // plain stores: element-wide non-temporal stores measured slower here
       dp[(int64_t)i * dstep] = f(p0, p1, p2);
     }
@@ -381,6 +403,18 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
   constexpr int NIN = F::NIN;
   constexpr int TB = tile_b<F>::value;
   extern __shared__ __align__(16) char smem[];
+
+  // Every argument the block needs is named here so that the compiler fetches
+  // them in one batch before the first branch (see ew_vec_kernel); the code
+  // below reads the same values.
+  {
+    constexpr int K1 = NIN >= 1 ? 1 : 0, K2 = NIN >= 2 ? 2 : 0, K3 = NIN >= 3 ? 3 : 0;
+    asm volatile("" ::"s"(a.sizeA), "s"(a.sizeB), "s"(a.tilesA_fd.d), "s"(a.tilesA_fd.m), "s"(a.tilesA_fd.s),
+                 "s"(a.tilesB_fd.d), "s"(a.tilesB_fd.m), "s"(a.tilesB_fd.s), "s"(a.n_outer), "s"(a.lds_mask),
+                 "s"(a.const_mask), "s"(a.ptr[0]), "s"(a.ptr[K1]), "s"(a.ptr[K2]), "s"(a.ptr[K3]), "s"(a.strideA[0]),
+                 "s"(a.strideA[K1]), "s"(a.strideA[K2]), "s"(a.strideA[K3]), "s"(a.strideB[0]), "s"(a.strideB[K1]),
+                 "s"(a.strideB[K2]), "s"(a.strideB[K3]), "s"(a.cbits[K1]), "s"(a.cbits[K2]), "s"(a.cbits[K3]));
+  }
 
   uint32_t bid, tb, ta, q0;
   // tiles along B vary fastest: consecutive blocks read neighbouring segments

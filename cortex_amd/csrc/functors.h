@@ -11,8 +11,16 @@
 // exp, tanh and logistic on float tensors with alpha == 1 are evaluated by the
 // single-precision device routines (about 1 ulp, far inside the 2e-6 relative
 // budget of a transcendental) because the double-precision routines would make
-// these kernels compute-bound; every other float operation takes the double
-// route and is bit-identical to the CPU backend.
+// these kernels compute-bound; every other float operation is bit-identical to
+// the CPU backend.
+//
+// PLAIN functors are the float forms whose multipliers are +-1.  Then x * alpha
+// is exact in float, and one correctly rounded float operation (+ - * / sqrt,
+// floor, ceil, a comparison) equals the double operation rounded once to float
+// (a double carries more than 2 * 24 + 2 bits), so the widening is skipped.
+// Which form runs is decided on the host: a run-time flag inside the functor
+// would put a branch, and both code paths, into every unrolled element of the
+// kernels.
 #pragma once
 
 #include "common.h"
@@ -63,25 +71,29 @@ template <class T, int OP, class A> __device__ __forceinline__ T unary_value(A v
   else return jvm_cast<T>((double)v);
 }
 
-template <class T, int OP> struct UnaryF {
+template <class T, int OP, bool PLAIN = false> struct UnaryF {
   static constexpr int NIN = 1;
   using Out = T;
   using In0 = T;
   using In1 = T;
   using In2 = T;
   using A = typename acc_of<T>::type;
-  A alpha;
-  int32_t single;  // float tensor, alpha == 1, transcendental op
+  A alpha;  // 1 when PLAIN
   __device__ __forceinline__ T operator()(T x, T, T) const {
-    if constexpr (std::is_same<T, float>::value &&
-                  (OP == CT_UOP_TANH || OP == CT_UOP_LOGISTIC || OP == CT_UOP_EXP)) {
-      if (single) {
-        if constexpr (OP == CT_UOP_TANH) return tanhf(x);
-        else if constexpr (OP == CT_UOP_EXP) return expf(x);
-        else return 1.0f / (1.0f + expf(-x));
-      }
+    if constexpr (PLAIN) {
+      static_assert(std::is_same<T, float>::value, "PLAIN is a float form");
+      if constexpr (OP == CT_UOP_TANH) return tanhf(x);
+      else if constexpr (OP == CT_UOP_EXP) return expf(x);
+      else if constexpr (OP == CT_UOP_LOGISTIC) return 1.0f / (1.0f + expf(-x));
+      else if constexpr (OP == CT_UOP_FLOOR) return floorf(x);
+      else if constexpr (OP == CT_UOP_CEIL) return ceilf(x);
+      else if constexpr (OP == CT_UOP_NEGATE) return -x;
+      else if constexpr (OP == CT_UOP_SQRT) return sqrtf(x);
+      else if constexpr (OP == CT_UOP_NOOP) return x;
+      else return unary_value<T, OP, A>((A)x);
+    } else {
+      return unary_value<T, OP, A>(w_mul((A)x, alpha));
     }
-    return unary_value<T, OP, A>(w_mul((A)x, alpha));
   }
 };
 
@@ -112,7 +124,13 @@ template <class T, int OP, class A> __device__ __forceinline__ T binary_value(A 
 
 // dest = op(x * xa, y * ya).  A scalar operand is passed as a constant input
 // with alpha 1 (the caller has already folded its alpha, src/cortex/tensor.clj:680).
-template <class T, int OP> struct BinaryF {
+// PLAIN: float, xa and ya are +-1, and OP is one of binary_plain_op's.
+constexpr bool binary_plain_op(int op) {
+  return op == CT_BOP_ADD || op == CT_BOP_SUB || op == CT_BOP_MUL || op == CT_BOP_DIV || op == CT_BOP_MIN ||
+         op == CT_BOP_MAX || op == CT_BOP_EQ || op == CT_BOP_GT || op == CT_BOP_GE || op == CT_BOP_LT || op == CT_BOP_LE;
+}
+
+template <class T, int OP, bool PLAIN = false> struct BinaryF {
   static constexpr int NIN = 2;
   using Out = T;
   using In0 = T;
@@ -120,23 +138,24 @@ template <class T, int OP> struct BinaryF {
   using In2 = T;
   using A = typename acc_of<T>::type;
   A xa, ya;
-  // Float tensors whose multipliers are +-1: x*xa and y*ya are exact in float,
-  // and a single float add, subtract, multiply or divide (correctly rounded)
-  // equals the double operation rounded once to float, so the widening can be
-  // skipped.  Comparisons and min/max see the same values either way.
-  int32_t narrow;
   __device__ __forceinline__ T operator()(T x, T y, T) const {
-    if constexpr (std::is_same<T, float>::value &&
-                  (OP == CT_BOP_ADD || OP == CT_BOP_SUB || OP == CT_BOP_MUL || OP == CT_BOP_DIV)) {
-      if (narrow) {
-        const float fx = xa < 0 ? -x : x, fy = ya < 0 ? -y : y;
-        if constexpr (OP == CT_BOP_ADD) return fx + fy;
-        else if constexpr (OP == CT_BOP_SUB) return fx - fy;
-        else if constexpr (OP == CT_BOP_MUL) return fx * fy;
-        else return fx / fy;
-      }
+    if constexpr (PLAIN) {
+      static_assert(std::is_same<T, float>::value && binary_plain_op(OP), "PLAIN is a float form");
+      const float fx = xa < 0 ? -x : x, fy = ya < 0 ? -y : y;
+      if constexpr (OP == CT_BOP_ADD) return fx + fy;
+      else if constexpr (OP == CT_BOP_SUB) return fx - fy;
+      else if constexpr (OP == CT_BOP_MUL) return fx * fy;
+      else if constexpr (OP == CT_BOP_DIV) return fx / fy;
+      else if constexpr (OP == CT_BOP_MAX) return fx > fy ? fx : fy;
+      else if constexpr (OP == CT_BOP_MIN) return fx > fy ? fy : fx;
+      else if constexpr (OP == CT_BOP_EQ) return fx == fy ? 1.0f : 0.0f;
+      else if constexpr (OP == CT_BOP_GT) return fx > fy ? 1.0f : 0.0f;
+      else if constexpr (OP == CT_BOP_GE) return fx >= fy ? 1.0f : 0.0f;
+      else if constexpr (OP == CT_BOP_LT) return fx < fy ? 1.0f : 0.0f;
+      else return fx <= fy ? 1.0f : 0.0f;
+    } else {
+      return binary_value<T, OP, A>(w_mul((A)x, xa), w_mul((A)y, ya));
     }
-    return binary_value<T, OP, A>(w_mul((A)x, xa), w_mul((A)y, ya));
   }
 };
 
@@ -145,8 +164,8 @@ template <class A> inline bool unit_magnitude(A v) { return v == (A)1 || v == (A
 // ------------------------------------------------------------------ ternary select
 
 // Three tensors (cpu/tensor_math.clj:469-497): the comparison sees the
-// unrounded products.
-template <class T> struct SelectF {
+// unrounded products.  PLAIN: float with all three multipliers 1.
+template <class T, bool PLAIN = false> struct SelectF {
   static constexpr int NIN = 3;
   using Out = T;
   using In0 = T;
@@ -155,8 +174,12 @@ template <class T> struct SelectF {
   using A = typename acc_of<T>::type;
   A xa, ya, za;
   __device__ __forceinline__ T operator()(T x, T y, T z) const {
-    const A vx = w_mul(xa, (A)x);
-    return jvm_cast<T>(vx >= (A)0 ? w_mul(za, (A)z) : w_mul(ya, (A)y));
+    if constexpr (PLAIN) {
+      return x >= (T)0 ? z : y;
+    } else {
+      const A vx = w_mul(xa, (A)x);
+      return jvm_cast<T>(vx >= (A)0 ? w_mul(za, (A)z) : w_mul(ya, (A)y));
+    }
   }
 };
 

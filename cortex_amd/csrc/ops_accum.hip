@@ -252,7 +252,6 @@ int accum_run(hipStream_t s, void* dest, const ct_dims* dd, double dest_alpha, c
   // f(first, second) = op(first * xa, second * ya)
   f.xa = reverse ? (A)jvm_cast<T>(y_alpha) : (A)jvm_cast<T>(dest_alpha);
   f.ya = reverse ? (A)jvm_cast<T>(dest_alpha) : (A)jvm_cast<T>(y_alpha);
-  f.narrow = 0;  // every update is rounded to T; keep the reference's double route
   OwnerArgs a;
   std::memset(&a, 0, sizeof(a));
   if (owner_structure(*dd, *yd, n, &a)) {

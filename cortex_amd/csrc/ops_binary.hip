@@ -11,14 +11,19 @@ namespace {
 template <class T, int OP>
 int binary_run(hipStream_t s, const BinaryCall& c) {
   using A = typename acc_of<T>::type;
-  BinaryF<T, OP> f;
   // A scalar side has had its alpha folded in by the caller; its multiplier is 1.
-  f.xa = c.x ? (A)jvm_cast<T>(c.x_alpha) : (A)1;
-  f.ya = c.y ? (A)jvm_cast<T>(c.y_alpha) : (A)1;
-  f.narrow = unit_magnitude(f.xa) && unit_magnitude(f.ya);
+  const A xa = c.x ? (A)jvm_cast<T>(c.x_alpha) : (A)1;
+  const A ya = c.y ? (A)jvm_cast<T>(c.y_alpha) : (A)1;
   EwOperand ops[3] = {{c.dest, c.dest_dims, (int)sizeof(T), 0},
                       {c.x, c.x ? c.x_dims : nullptr, (int)sizeof(T), bits_of<T>(jvm_cast<T>(c.x_scalar))},
                       {c.y, c.y ? c.y_dims : nullptr, (int)sizeof(T), bits_of<T>(jvm_cast<T>(c.y_scalar))}};
+  if constexpr (std::is_same<T, float>::value && binary_plain_op(OP)) {
+    if (unit_magnitude(xa) && unit_magnitude(ya) && !c.serial) {
+      BinaryF<T, OP, true> f{xa, ya};
+      return launch_elementwise(s, f, ops, c.n);
+    }
+  }
+  BinaryF<T, OP> f{xa, ya};
   return c.serial ? launch_elementwise_serial(s, f, ops, c.n) : launch_elementwise(s, f, ops, c.n);
 }
 

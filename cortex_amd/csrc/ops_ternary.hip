@@ -47,11 +47,18 @@ int ct_ternary_op(void* stream, void* dest, const ct_dims* dest_dims, const void
   CT_REQUIRE(op == CT_TOP_SELECT, "unknown ternary operation %d", op);
   CT_DISPATCH_DTYPE(dtype, {
     using A = typename acc_of<T>::type;
-    SelectF<T> f{(A)jvm_cast<T>(x_alpha), (A)jvm_cast<T>(y_alpha), (A)jvm_cast<T>(z_alpha)};
+    const A xa = (A)jvm_cast<T>(x_alpha), ya = (A)jvm_cast<T>(y_alpha), za = (A)jvm_cast<T>(z_alpha);
     EwOperand ops[4] = {{dest, dest_dims, (int)sizeof(T), 0},
                         {x, x_dims, (int)sizeof(T), 0},
                         {y, y_dims, (int)sizeof(T), 0},
                         {z, z_dims, (int)sizeof(T), 0}};
+    if constexpr (std::is_same<T, float>::value) {
+      if (xa == (A)1 && ya == (A)1 && za == (A)1) {
+        SelectF<T, true> f{xa, ya, za};
+        return launch_elementwise(static_cast<hipStream_t>(stream), f, ops, n);
+      }
+    }
+    SelectF<T> f{xa, ya, za};
     return launch_elementwise(static_cast<hipStream_t>(stream), f, ops, n);
   });
   return CT_OK;

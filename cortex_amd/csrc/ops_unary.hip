@@ -10,11 +10,15 @@ template <class T, int OP>
 int unary_run(hipStream_t s, void* dest, const ct_dims* dd, const void* x, const ct_dims* xd, double alpha,
               int64_t n, bool serial) {
   using A = typename acc_of<T>::type;
-  UnaryF<T, OP> f;
   const T a = jvm_cast<T>(alpha);
-  f.alpha = (A)a;
-  f.single = std::is_same<T, float>::value && a == (T)1;
   EwOperand ops[2] = {{dest, dd, (int)sizeof(T), 0}, {x, xd, (int)sizeof(T), 0}};
+  if constexpr (std::is_same<T, float>::value) {
+    if (a == (T)1 && !serial) {
+      UnaryF<T, OP, true> f{(A)1};
+      return launch_elementwise(s, f, ops, n);
+    }
+  }
+  UnaryF<T, OP> f{(A)a};
   return serial ? launch_elementwise_serial(s, f, ops, n) : launch_elementwise(s, f, ops, n);
 }
 
