@@ -260,15 +260,21 @@ def cpu_baseline(hosts, n: int) -> dict:
     cont = capi.make_dims(shape, [n, 1])
     view = capi.make_dims(shape, tr)
     p = lambda a: a.ctypes.data
-    t0 = time.perf_counter()
-    ob.call("unary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, capi.UNARY_OPS["exp"], capi.F32, n * n)
-    ob.call("unary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, capi.UNARY_OPS["tanh"], capi.F32, n * n)
-    ob.call("ternary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, p(hosts[1]), C.byref(view), 1.0,
-            p(hosts[2]), C.byref(view), 1.0, n * n, 0, capi.F32)
+    def one_step():
+        ob.call("unary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, capi.UNARY_OPS["exp"], capi.F32, n * n)
+        ob.call("unary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, capi.UNARY_OPS["tanh"], capi.F32, n * n)
+        ob.call("ternary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, p(hosts[1]), C.byref(view), 1.0,
+                p(hosts[2]), C.byref(view), 1.0, n * n, 0, capi.F32)
+
+    one_step()  # first touch of the destination pages
+    steps, t0 = 0, time.perf_counter()
+    while steps < 3 or (time.perf_counter() - t0 < 10.0 and steps < 200):
+        one_step()
+        steps += 1
     dt = time.perf_counter() - t0
     step_bytes = 8 * 4 * n * n
-    return {"value": round(step_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": ob.num_threads(), "kind": "port",
-            "sample": f"1 full step (exp, tanh, select on transposed float32 [{n},{n}]) in {dt:.2f} s, "
+    return {"value": round(steps * step_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": ob.num_threads(), "kind": "port",
+            "sample": f"{steps} full steps (exp, tanh, select on transposed float32 [{n},{n}]) in {dt:.2f} s, "
                       "C++ restatement of the cortex CPU backend with OpenMP"}
 
 
