@@ -195,6 +195,13 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
   using V = Vec<T, VEC>;
   constexpr int RPB = kBlock / TPR;
   __shared__ A lds[kBlock / 64];
+  // A block lives about as long as one trip to memory (a row is a few KiB), so the
+  // arguments are fetched in one batch before the first branch: naming them in one
+  // empty asm statement makes the compiler load them here rather than next to each use.
+  asm volatile("" ::"s"(a.in), "s"(a.out), "s"(a.partials), "s"(a.k), "s"(a.n_out), "s"(a.chunk), "s"(a.split_fd.d),
+               "s"(a.split_fd.m), "s"(a.split_fd.s), "s"(a.n_split), "s"(a.n_outer), "s"(a.osize[0].d), "s"(a.osize[0].m),
+               "s"(a.osize[0].s), "s"(a.ostride[0]), "s"(a.osize[1].d), "s"(a.osize[1].m), "s"(a.osize[1].s),
+               "s"(a.ostride[1]), "s"(a.oa.identity));
   const int lane = threadIdx.x % TPR;
   const int64_t vp = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
   const bool live = vp < a.n_out * (int64_t)a.n_split;
@@ -205,8 +212,12 @@ __global__ void __launch_bounds__(kBlock) reduce_row_kernel(const RowArgs a, con
     int64_t base = (int64_t)seg * a.chunk;
     int64_t len = a.k - base;
     if (len > a.chunk) len = a.chunk;
-    uint32_t rem = p;
-    for (int d = 0; d < a.n_outer; ++d) {
+    // the first two kept axes with fixed indices (absent axes have size 1, stride 0)
+    uint32_t rem, r0, r1, q0;
+    a.osize[0].divmod(p, q0, r0);
+    a.osize[1].divmod(q0, rem, r1);
+    base += (int64_t)r0 * a.ostride[0] + (int64_t)r1 * a.ostride[1];
+    for (int d = 2; d < a.n_outer; ++d) {
       uint32_t q, r;
       a.osize[d].divmod(rem, q, r);
       rem = q;
