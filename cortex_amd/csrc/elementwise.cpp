@@ -9,19 +9,22 @@ namespace {
 constexpr int64_t kLim31 = int64_t(1) << 31;
 
 // A call whose operands together exceed what the caches can hold streams
-// through them: its accesses are marked non-temporal.
-bool is_streaming(const Plan& plan, const EwOperand* ops) {
+// through them: its loads are marked non-temporal (level 1), and from about
+// four times the last-level cache's size its stores too (level 2).
+uint32_t streaming_level(const Plan& plan, const EwOperand* ops) {
   int64_t bytes = 0;
   for (int k = 0; k < plan.n_ops; ++k)
     if (ops[k].ptr) bytes += plan.n * ops[k].elem_size;
-  return bytes >= (int64_t(64) << 20);
+  if (bytes >= (int64_t(1) << 30)) return 2;
+  return bytes >= (int64_t(64) << 20) ? 1 : 0;
 }
+bool is_streaming(const Plan& plan, const EwOperand* ops) { return streaming_level(plan, ops) > 0; }
 
 void common_vec(const Plan& plan, const EwOperand* ops, VecArgs* a) {
   const Canon& c = plan.canon;
   std::memset(a, 0, sizeof(*a));
   a->n_outer = c.nd - 1;
-  a->streaming = is_streaming(plan, ops) ? 1u : 0u;
+  a->streaming = streaming_level(plan, ops);
   for (int d = 0; d + 1 < c.nd; ++d) {
     if (d < 2) a->outer_fd01[d] = FastDiv((uint32_t)c.size[d + 1]);
     else a->outer_fd_hi[d - 2] = FastDiv((uint32_t)c.size[d + 1]);

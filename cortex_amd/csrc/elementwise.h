@@ -71,7 +71,7 @@ struct VecArgs {
   uint32_t unit_mask;     // bit k: operand k is unit-stride along the inner axis
   uint32_t const_mask;    // bit k: operand k is a scalar constant
   uint32_t nt_mask;       // bit k: operand k is read exactly once (no broadcast axis), so its loads may bypass the caches
-  uint32_t streaming;     // the call moves more data than the caches hold: non-temporal loads
+  uint32_t streaming;     // 0: the call fits the caches; 1: non-temporal loads; 2: and non-temporal stores (see ew_vec_kernel)
   char* ptr[kMaxOps];
   int64_t outer_stride01[kMaxOps][2];
   uint64_t cbits[kMaxOps];
@@ -90,7 +90,7 @@ constexpr int vec_kinds(int k1, int k2 = 0, int k3 = 0) { return k1 | (k2 << 2) 
 
 // Operand k of one lane.  vp / sp are the lane's vector and scalar addresses.
 // KIND < 0: the kind is read from the run-time masks.
-template <class T, int VEC, bool STREAM, int KIND>
+template <class T, int VEC, int STREAM, int KIND>
 __device__ __forceinline__ Vec<T, VEC> vec_load(uint32_t const_mask, uint32_t unit_mask, uint32_t nt_mask, uint64_t cbits,
                                                 int k, const Vec<T, VEC>* vp, const T* sp) {
   Vec<T, VEC> r;
@@ -103,7 +103,7 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(uint32_t const_mask, uint32_t un
     for (int i = 0; i < VEC; ++i) r.v[i] = c;
   } else if (is_unit) {
     // a broadcast operand (a bias row, say) is re-read by every outer index and must stay cached
-    if (STREAM && is_once) r = nt_load(vp);
+    if (STREAM >= 1 && is_once) r = nt_load(vp);
     else r = *vp;
   } else {
     const T c = *sp;
@@ -116,9 +116,13 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(uint32_t const_mask, uint32_t un
 // One 16-byte vector per lane.  On this part one vector per lane with many
 // resident blocks sustains more bandwidth than several vectors per lane, and
 // non-temporal loads add a few percent on streams larger than the caches.
-// STREAM is a template parameter: a run-time choice between a plain and a
+// STREAM (0: plain accesses, 1: non-temporal loads, 2: non-temporal loads and
+// stores) is a template parameter: a run-time choice between a plain and a
 // non-temporal access to the same address is folded into one plain access by
-// the compiler, which loses the hint.
+// the compiler, which loses the hint.  Measured on an in-place add: below the
+// last-level cache's size plain accesses win (92 % of peak at 256 MiB against
+// 88 % with non-temporal loads and 83 % with non-temporal stores too); at 1 GiB
+// non-temporal loads and stores together win (82 % against 73 %).
 //
 // A wave lives about as long as one trip to memory, so every scalar fetch of a
 // kernel argument that sits between the wave's start and its first vector load
@@ -132,7 +136,7 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(uint32_t const_mask, uint32_t un
 // KINDS >= 0 fixes the operand kinds at compile time (vec_kinds): the common
 // broadcast patterns then run without the operand-kind branches, which cost
 // about 3 % of a copy's bandwidth.
-template <class F, int VEC, bool STREAM, int KINDS = -1>
+template <class F, int VEC, int STREAM, int KINDS = -1>
 __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs a) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
@@ -235,7 +239,8 @@ __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs
     r.v[i] = f(p0, p1, p2);
   }
   Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(base[0]) + off[0] + col);
-  *dp = r;  // plain stores: non-temporal ones measured no faster here and slower for narrow inputs
+  if constexpr (STREAM == 2) nt_store(r, dp);
+  else *dp = r;
 }
 
 // The contiguous case: every operand is a flat unit-stride array read (or
@@ -248,7 +253,7 @@ struct FlatArgs {
   char* ptr[kMaxOps];
 };
 
-template <class F, int VEC, bool STREAM>
+template <class F, int VEC, int STREAM>
 __global__ void __launch_bounds__(kBlock) ew_flat_kernel(const F f, const FlatArgs a) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
@@ -262,15 +267,15 @@ __global__ void __launch_bounds__(kBlock) ew_flat_kernel(const F f, const FlatAr
   Vec<In2, VEC> x2;
   if constexpr (NIN >= 1) {
     const Vec<In0, VEC>* p = reinterpret_cast<const Vec<In0, VEC>*>(a.ptr[1]) + v;
-    if constexpr (STREAM) x0 = nt_load(p); else x0 = *p;
+    if constexpr (STREAM >= 1) x0 = nt_load(p); else x0 = *p;
   }
   if constexpr (NIN >= 2) {
     const Vec<In1, VEC>* p = reinterpret_cast<const Vec<In1, VEC>*>(a.ptr[2]) + v;
-    if constexpr (STREAM) x1 = nt_load(p); else x1 = *p;
+    if constexpr (STREAM >= 1) x1 = nt_load(p); else x1 = *p;
   }
   if constexpr (NIN >= 3) {
     const Vec<In2, VEC>* p = reinterpret_cast<const Vec<In2, VEC>*>(a.ptr[3]) + v;
-    if constexpr (STREAM) x2 = nt_load(p); else x2 = *p;
+    if constexpr (STREAM >= 1) x2 = nt_load(p); else x2 = *p;
   }
   Vec<Out, VEC> r;
 #pragma unroll
@@ -283,7 +288,9 @@ __global__ void __launch_bounds__(kBlock) ew_flat_kernel(const F f, const FlatAr
     if constexpr (NIN >= 3) p2 = x2.v[i];
     r.v[i] = f(p0, p1, p2);
   }
-  reinterpret_cast<Vec<Out, VEC>*>(a.ptr[0])[v] = r;
+  Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(a.ptr[0]) + v;
+  if constexpr (STREAM == 2) nt_store(r, dp);
+  else *dp = r;
 }
 
 // ------------------------------------------------------------------ TILE
@@ -641,8 +648,9 @@ inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& a) {
     FlatArgs fa;
     fa.total_vecs = a.total_vecs;
     for (int k = 0; k < kMaxOps; ++k) fa.ptr[k] = a.ptr[k];
-    if (a.streaming) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, true>), grid, dim3(kBlock), 0, s, f, fa);
-    else hipLaunchKernelGGL((ew_flat_kernel<F, VEC, false>), grid, dim3(kBlock), 0, s, f, fa);
+    if (a.streaming == 2) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 2>), grid, dim3(kBlock), 0, s, f, fa);
+    else if (a.streaming) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 1>), grid, dim3(kBlock), 0, s, f, fa);
+    else hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 0>), grid, dim3(kBlock), 0, s, f, fa);
     return;
   }
   if (VEC > 1 && a.streaming) {
@@ -656,7 +664,8 @@ inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& a) {
     }
 #define CT_VEC_KINDS(K)                                                                                  \
   if (kinds == (K)) {                                                                                    \
-    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, true, (K)>), grid, dim3(kBlock), 0, s, f, a);              \
+    if (a.streaming == 2) hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 2, (K)>), grid, dim3(kBlock), 0, s, f, a); \
+    else hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 1, (K)>), grid, dim3(kBlock), 0, s, f, a);            \
     return;                                                                                              \
   }
     if constexpr (F::NIN == 1) {
@@ -672,8 +681,8 @@ inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& a) {
     }
 #undef CT_VEC_KINDS
   }
-  if (a.streaming) hipLaunchKernelGGL((ew_vec_kernel<F, VEC, true>), grid, dim3(kBlock), 0, s, f, a);
-  else hipLaunchKernelGGL((ew_vec_kernel<F, VEC, false>), grid, dim3(kBlock), 0, s, f, a);
+  if (a.streaming) hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 1>), grid, dim3(kBlock), 0, s, f, a);
+  else hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 0>), grid, dim3(kBlock), 0, s, f, a);
 }
 
 // A flat call longer than one launch's 32-bit vector index is walked in pieces.
