@@ -18,11 +18,12 @@
 //                         rows are unit-stride and aligned)
 //   softmax_block_kernel  longer rows: one block per row, exponentials parked
 //                         in the output and scaled in a third pass
-//   softmax_lane_kernel   one lane owns a row and walks k sequentially, the
-//                         lanes of a wave take neighbouring rows (coalesced when
-//                         the row axis is unit-stride: the spatial form, where
-//                         k is the channel axis); rows of up to 32 elements stay
-//                         in registers.  Its sum runs in the reference's order.
+//   softmax_lane_kernel   one lane owns a row (or four neighbouring rows, as
+//                         128-bit accesses) and walks k sequentially, the lanes
+//                         of a wave take neighbouring rows (coalesced when the
+//                         row axis is unit-stride: the spatial form, where k is
+//                         the channel axis); rows of up to 32 elements stay in
+//                         registers.  Its sum runs in the reference's order.
 // y_i is formed as e_i * (1 / s): at most one ulp from the reference's e_i / s.
 // The reference's maximum loop reads elements 1..k-1 of the input through the
 // output's address object (cpu/tensor_math.clj:1067-1072); that only matters
@@ -211,39 +212,83 @@ __global__ void __launch_bounds__(kBlock) softmax_block_kernel(const SoftmaxArgs
 // One lane per row, the lanes of a wave on neighbouring rows.  CMAX > 0: the row
 // (k <= CMAX) stays in registers.  CMAX == 0: any k, exponentials parked in the
 // output.  The sum runs in the reference's own order.
-template <class T, int CMAX>
+template <class T, int VEC, int CMAX>
 __global__ void __launch_bounds__(kBlock) softmax_lane_kernel(const SoftmaxArgs a) {
-  const int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  // VEC > 1: the lane owns VEC neighbouring rows (positions); the row axis is unit-stride
+  // and every stride a multiple of VEC, so each channel is one aligned vector access.
+  using V = Vec<T, VEC>;
+  const int64_t r = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
   if (r >= a.n_rows) return;
   int64_t ib, ob;
   softmax_row_base(a, r, &ib, &ob);
   const T* in = reinterpret_cast<const T*>(a.in) + ib;
   T* out = reinterpret_cast<T*>(a.out) + ob;
+  auto load = [&](uint32_t i) { return *reinterpret_cast<const V*>(in + (int64_t)i * a.in_k); };
+  auto store = [&](uint32_t i, const V& v) { *reinterpret_cast<V*>(out + (int64_t)i * a.out_k) = v; };
+  T m[VEC];
+  double sum[VEC];
+  T inv[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) { m[e] = -__builtin_huge_valf(); sum[e] = 0.0; }  // identity of Math.max that lets NaN through
   if constexpr (CMAX > 0) {
-    T x[CMAX];
-    T m = -__builtin_huge_valf();
+    V x[CMAX];
 #pragma unroll
     for (int i = 0; i < CMAX; ++i)
-      if ((uint32_t)i < a.k) { x[i] = in[(int64_t)i * a.in_k]; m = jvm_max(m, x[i]); }
-    double sum = 0.0;
+      if ((uint32_t)i < a.k) {
+        x[i] = load(i);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) m[e] = jvm_max(m[e], x[i].v[e]);
+      }
 #pragma unroll
     for (int i = 0; i < CMAX; ++i)
-      if ((uint32_t)i < a.k) { x[i] = shifted_exp(x[i], m); sum += (double)x[i]; }
-    const T inv = (T)1 / (T)sum;
+      if ((uint32_t)i < a.k) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { x[i].v[e] = shifted_exp(x[i].v[e], m[e]); sum[e] += (double)x[i].v[e]; }
+      }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) inv[e] = (T)1 / (T)sum[e];
 #pragma unroll
     for (int i = 0; i < CMAX; ++i)
-      if ((uint32_t)i < a.k) out[(int64_t)i * a.out_k] = x[i] * inv;
+      if ((uint32_t)i < a.k) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[i].v[e] *= inv[e];
+        store(i, x[i]);
+      }
   } else {
-    T m = in[0];
-    for (uint32_t i = 1; i < a.k; ++i) m = jvm_max(m, in[(int64_t)i * a.in_k]);
-    double sum = 0.0;
-    for (uint32_t i = 0; i < a.k; ++i) {
-      const T e = shifted_exp(in[(int64_t)i * a.in_k], m);
-      out[(int64_t)i * a.out_k] = e;
-      sum += (double)e;
+    constexpr int U = 4;  // channels fetched ahead
+    for (uint32_t i0 = 0; i0 < a.k; i0 += U) {
+      V x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (i0 + u < a.k) x[u] = load(i0 + u);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (i0 + u < a.k) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) m[e] = jvm_max(m[e], x[u].v[e]);
+        }
     }
-    const T inv = (T)1 / (T)sum;
-    for (uint32_t i = 0; i < a.k; ++i) out[(int64_t)i * a.out_k] *= inv;
+    for (uint32_t i0 = 0; i0 < a.k; i0 += U) {
+      V x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (i0 + u < a.k) x[u] = load(i0 + u);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (i0 + u < a.k) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) { x[u].v[e] = shifted_exp(x[u].v[e], m[e]); sum[e] += (double)x[u].v[e]; }
+          store(i0 + u, x[u]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) inv[e] = (T)1 / (T)sum[e];
+    for (uint32_t i = 0; i < a.k; ++i) {
+      V x = *reinterpret_cast<const V*>(out + (int64_t)i * a.out_k);  // the lane re-reads its own stores
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) x.v[e] *= inv[e];
+      store(i, x);
+    }
   }
 }
 
@@ -279,11 +324,22 @@ int softmax_run(hipStream_t s, void* out, const RowLayout& ol, const void* in, c
   // lanes along the row axis when that is the unit-stride one (spatial form) or the rows are tiny
   const bool row_major = il.s_k == 1 || il.k == 1;
   if (il.k < 8 || (!row_major && il.s_row == 1)) {
-    const dim3 grid((uint32_t)((a.n_rows + kBlock - 1) / kBlock));
-    note_kernel(il.k <= 32 ? "softmax_lane" : "softmax_lane_loop");
-    if (il.k <= 8) hipLaunchKernelGGL((softmax_lane_kernel<T, 8>), grid, dim3(kBlock), 0, s, a);
-    else if (il.k <= 32) hipLaunchKernelGGL((softmax_lane_kernel<T, 32>), grid, dim3(kBlock), 0, s, a);
-    else hipLaunchKernelGGL((softmax_lane_kernel<T, 0>), grid, dim3(kBlock), 0, s, a);
+    constexpr int VL = 16 / (int)sizeof(T);
+    auto lanes_ok = [](const void* p, const RowLayout& l) {
+      return l.s_row == 1 && l.rows % VL == 0 && l.s_k % VL == 0 && l.s_outer % VL == 0 && (uintptr_t)p % 16 == 0;
+    };
+    const bool vec_rows = lanes_ok(in, il) && lanes_ok(out, ol);
+    const int64_t lanes = vec_rows ? a.n_rows / VL : a.n_rows;
+    const dim3 grid((uint32_t)((lanes + kBlock - 1) / kBlock));
+    note_kernel(il.k <= 32 ? (vec_rows ? "softmax_lane_vec" : "softmax_lane") : (vec_rows ? "softmax_lane_loop_vec" : "softmax_lane_loop"));
+#define CT_SM_LANE(VEC_)                                                                                  \
+  if (il.k <= 8) hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 8>), grid, dim3(kBlock), 0, s, a);       \
+  else if (il.k <= 16) hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 16>), grid, dim3(kBlock), 0, s, a); \
+  else if (il.k <= 24) hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 24>), grid, dim3(kBlock), 0, s, a); \
+  else if (il.k <= 32) hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 32>), grid, dim3(kBlock), 0, s, a); \
+  else hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 0>), grid, dim3(kBlock), 0, s, a)
+    if (vec_rows) { CT_SM_LANE(VL); } else { CT_SM_LANE(1); }
+#undef CT_SM_LANE
     return after_launch(s);
   }
   constexpr int VMAX = 16 / (int)sizeof(T);

@@ -580,14 +580,25 @@ def test_softmax_layouts(P, code):
     out = P.buf(np.zeros(b * c * e, NP[code]))
     kern = P.run(H.softmax, View(out, [b, c, e]), View(x, [b, c, e]), True)
     compare(out, f"softmax-spatial ({kern})", tol=tol)
-    assert kern == "softmax_lane"
-    c2 = 70                                       # more channels than the register-resident form holds
+    assert kern in ("softmax_lane", "softmax_lane_vec")         # 130 positions: pairs of doubles, single floats
+    c2 = 70                                       # more channels than the four-positions-per-lane form holds
     x2, out2 = P.buf((rng.standard_normal(2 * c2 * 90) * 3).astype(NP[code])), P.buf(np.zeros(2 * c2 * 90, NP[code]))
     kern2 = P.run(H.softmax, View(out2, [2, c2, 90]), View(x2, [2, c2, 90]), True)
     compare(out2, f"softmax-spatial wide ({kern2})", tol=tol)
-    assert kern2 == "softmax_lane_loop"
+    assert kern2 in ("softmax_lane_loop", "softmax_lane_loop_vec")
     got = out.download().reshape(b, c, e).astype(np.float64)
     assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
+    # position counts that allow 128-bit accesses across neighbouring positions
+    for (b3, c3, e3), want_kernel in (((3, 21, 132), "softmax_lane_vec"), ((2, 5, 64), "softmax_lane_vec"),
+                                     ((2, 13, 64), "softmax_lane_vec"), ((2, 30, 64), "softmax_lane_vec"),
+                                     ((2, 70, 96), "softmax_lane_loop_vec"), ((2, 70, 97), "softmax_lane_loop")):
+        n3 = b3 * c3 * e3
+        x3, out3 = P.buf((rng.standard_normal(n3) * 3).astype(NP[code])), P.buf(np.zeros(n3, NP[code]))
+        kern3 = P.run(H.softmax, View(out3, [b3, c3, e3]), View(x3, [b3, c3, e3]), True)
+        compare(out3, f"softmax-spatial {(b3, c3, e3)} ({kern3})", tol=tol)
+        assert kern3 == want_kernel
+        P.run(H.softmax, View(x3, [b3, c3, e3]), View(x3, [b3, c3, e3]), True)
+        compare(x3, f"softmax-spatial {(b3, c3, e3)} in place", tol=tol)
     # eltwise on three dimensions
     kern = P.run(H.softmax, View(out, [b, c, e]), View(x, [b, c, e]))
     compare(out, f"softmax 3-d eltwise ({kern})", tol=tol)
