@@ -873,3 +873,73 @@ def test_flat_call_longer_than_one_launch():
     finally:
         capi.call("ct_free", a)
         capi.call("ct_free", b)
+
+
+# ------------------------------------------------------------------ threads and streams
+
+def test_threads_on_their_own_streams(P):
+    """Several host threads drive their own streams at once, as cortex's training threads do
+    (src/cortex/verify/nn/train.clj:211-236): every call that keeps state outside its
+    arguments is in the mix (stream scratch of the split reductions, the staged sum-accumulate
+    and batch normalization; the per-thread rocBLAS handle; the thread-local error text)."""
+    import ctypes as C
+    import threading
+
+    rng = np.random.default_rng(100)
+    n_threads, rounds = 4, 6
+    r, c = 600, 520
+    work = []
+    for t in range(n_threads):
+        x = P.buf(rng.standard_normal(r * c).astype(np.float32))
+        w = dict(x=x, col=P.buf(np.zeros(c, np.float32)), row=P.buf(np.zeros(r, np.float32)),
+                 acc=P.buf(rng.standard_normal(c).astype(np.float32)), out=P.buf(np.zeros(r * c, np.float32)),
+                 stats=[P.buf(rng.uniform(0.5, 1.5, c).astype(np.float32)) for _ in range(6)],
+                 gemm=P.buf(np.zeros(c * c, np.float32)))
+        work.append(w)
+
+    def run_all(side, w):
+        V = lambda b, shape=None: View(b, shape or [b.init.size])
+        H.unary_reduce(side, View(w["col"], [c, 1]), 1.0, View(w["x"], [c, r], [1, c]), "sum")      # column reduce: partials
+        H.unary_reduce(side, View(w["row"], [r, 1]), 1.0, View(w["x"], [r, c]), "max")
+        H.binary_accum(side, View(w["acc"], [c]), 1.0, View(w["x"], [r, c]), 1.0, "+")              # staged sum
+        st = w["stats"]
+        H.batch_normalize_update_and_apply(side, V(w["out"]), V(w["x"]), V(st[0]), V(st[1]), V(st[2]), V(st[3]), 0.9,
+                                           V(st[4]), V(st[5]), 1e-3, r, c)
+        H.gemm(side, V(w["gemm"]), c, True, False, 1.0, V(w["x"]), c, r, c, V(w["x"]), c, c, 0.0)    # x^T x
+
+    for w in work:                                  # expected values, serially on the oracle
+        for _ in range(rounds):
+            run_all(H.ORACLE, w)
+
+    errors = []
+
+    def worker(w):
+        try:
+            side = H.gpu_side()
+            s = C.c_void_p()
+            capi.call("ct_set_device", 0)
+            capi.call("ct_stream_create", C.byref(s))
+            side.stream = s
+            for _ in range(rounds):
+                run_all(side, w)
+            with pytest.raises(capi.CortexHipError, match="float and double"):   # this thread's own error text
+                H.softmax(side, View(P_int, [4, 4]), View(P_int, [4, 4]))
+            capi.call("ct_stream_destroy", s)
+        except BaseException as exc:  # noqa: BLE001 -- reported in the main thread
+            errors.append(exc)
+
+    P_int = P.buf(np.zeros(16, np.int32))
+    threads = [threading.Thread(target=worker, args=(w,)) for w in work]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i, w in enumerate(work):
+        x64 = np.abs(w["x"].init.astype(np.float64))
+        bn_close(w["col"], f"thread {i} column sum", capi.F32, scale_by=x64.sum(axis=None) / c)
+        compare(w["row"], f"thread {i} row max")
+        bn_close(w["acc"], f"thread {i} accumulated sum", capi.F32, scale_by=rounds * x64.reshape(r, c).sum(axis=0).max())
+        bn_close(w["out"], f"thread {i} batch-normalized output", capi.F32)
+        got, want = w["gemm"].download().astype(np.float64), w["gemm"].host.astype(np.float64)
+        assert np.max(np.abs(got - want)) <= 1e-5 * (x64.reshape(r, c) ** 2).sum(axis=0).max()
