@@ -1,0 +1,457 @@
+"""The reference's backend-neutral layer tests, restated for the layers that
+are built purely on the tensor-math path.
+
+Every function takes ``(driver, datatype)`` and runs one forward and backward
+pass of one layer through ``cortex_amd.nn_layers`` on that driver, as
+``/root/reference/src/cortex/verify/nn/layers.clj`` (cited per function) does
+through a bound two-node network.  Expected values are the reference's own
+stored vectors where it holds any; the regularisers and loss gradients, for
+which it stores none, are checked against their closed forms.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from cortex_amd import nn_layers as nl
+from cortex_amd import tensor as ct
+from reference_suite import context, equals
+
+
+def about_there(actual, expected, eps=1e-6):
+    """``about-there?`` (src/cortex/verify/utils.clj:20-27): the sum of the
+    absolute differences stays below eps."""
+    a = np.asarray(actual, dtype=np.float64).reshape(-1)
+    e = np.asarray(expected, dtype=np.float64).reshape(-1)
+    assert a.shape == e.shape, (a.shape, e.shape)
+    assert np.abs(a - e).sum() < eps, (a, e)
+
+
+def entry(values, shape=None, with_gradient=True):
+    arr = np.asarray(values, dtype=np.float64)
+    if shape is not None:
+        arr = arr.reshape(shape)
+    out = {"buffer": ct.to_tensor(arr)}
+    if with_gradient:
+        out["gradient"] = ct.new_tensor(list(arr.shape))
+    return out
+
+
+def forward_backward(layer, parameters, inputs, outputs, output_gradients):
+    """One traversal forward and one backward (verify/nn/layers.clj:101-125)."""
+    if hasattr(layer, "prepare_forward"):
+        layer.prepare_forward(parameters, inputs, outputs)
+    layer.forward(parameters, inputs, outputs)
+    for out, og in zip(outputs, output_gradients):
+        ct.assign(out["gradient"], ct.to_tensor(np.asarray(og, dtype=np.float64).reshape(out["gradient"].shape())))
+    layer.backward(parameters, outputs, inputs)
+
+
+def single(node, batch_size, input, output_gradient, parameters=None, item_shape=None, datatype=None):
+    """``forward-backward-test`` (verify/nn/layers.clj:143-153)."""
+    input = np.asarray(input, dtype=np.float64)
+    shape = [batch_size] + list(item_shape or [input.size // batch_size])
+    layer = nl.create(node, batch_size, datatype)
+    inputs = [entry(input, shape)]
+    outputs = [{"buffer": ct.new_tensor(shape), "gradient": ct.new_tensor(shape)}]
+    forward_backward(layer, parameters or {}, inputs, outputs, [output_gradient])
+    return {"output": ct.to_double_array(outputs[0]["buffer"]).reshape(-1),
+            "input-gradient": ct.to_double_array(inputs[0]["gradient"]).reshape(-1), "layer": layer}
+
+
+# verify/nn/layers.clj:155-191
+def relu_activation(driver, datatype):
+    with context(driver, datatype):
+        for item_count, batch_size in ((10, 1), (10000, 5)):
+            r = single({"type": "relu"}, batch_size, [-1, 1] * (batch_size * item_count // 2),
+                       [1] * (batch_size * item_count))
+            assert r["output"].sum() == batch_size * item_count / 2
+            assert r["input-gradient"].sum() == batch_size * item_count / 2
+
+
+# verify/nn/layers.clj:193-235
+def linear(driver, datatype):
+    with context(driver, datatype):
+        for batch_size in (1, 10):
+            params = {"weights": entry([[1, 2], [3, 4]]), "bias": entry([0, 10])}
+            layer = nl.create({"type": "linear"}, batch_size)
+            inputs = [entry([1, 2] * batch_size, [batch_size, 2])]
+            outputs = [{"buffer": ct.new_tensor([batch_size, 2]), "gradient": ct.new_tensor([batch_size, 2])}]
+            forward_backward(layer, params, inputs, outputs, [[1, 2] * batch_size])
+            equals([5, 21] * batch_size, ct.to_double_array(outputs[0]["buffer"]))
+            equals(np.array([1, 2, 2, 4]) * batch_size, ct.to_double_array(params["weights"]["gradient"]))
+            equals(np.array([1, 2]) * batch_size, ct.to_double_array(params["bias"]["gradient"]))
+            equals([7, 10] * batch_size, ct.to_double_array(inputs[0]["gradient"]))
+
+
+# verify/nn/layers.clj:283-314
+ACTIVATION_ANSWERS = {
+    "logistic": ([0.2689414213699951, 0.7310585786300049], [-0.19661193324148185, 0.19661193324148185]),
+    "swish": ([-0.2689414213699951, 0.7310585786300049], [-0.36713290505919505, 0.835403899885462]),
+    "tanh": ([-0.7615941559557649, 0.7615941559557649], [-0.41997434161402614, 0.41997434161402614]),
+    "selu": ([-1.1113307378125625, 1.0507009873554805], [-0.5786268790075374, 1.0507009873554805]),
+}
+
+# verify/nn/layers.clj:332-381
+ACTIVATION_BATCH_ANSWERS = {
+    "logistic": ([0.0066928509242848554, 0.01798620996209156, 0.04742587317756678, 0.11920292202211755,
+                  0.2689414213699951, 0.5, 0.7310585786300049, 0.8807970779778823, 0.9525741268224334,
+                  0.9820137900379085],
+                 [-0.033240283353950774, -0.07065082485316447, -0.1355299791927364, -0.209987170807013,
+                  -0.19661193324148185, 0.0, 0.19661193324148185, 0.20998717080701323, 0.135529979192736,
+                  0.07065082485316443]),
+    "tanh": ([-0.9999092042625951, -0.999329299739067, -0.9950547536867305, -0.9640275800758169,
+              -0.7615941559557649, 0.0, 0.7615941559557649, 0.9640275800758169, 0.9950547536867305,
+              0.999329299739067],
+             [-9.079161547192634E-4, -0.005363802732103666, -0.0295981114963205, -0.14130164970632886,
+              -0.41997434161402614, 0.0, 0.41997434161402614, 0.14130164970632886, 0.0295981114963205,
+              0.005363802732103666]),
+    "swish": ([-0.03346425462142428, -0.07194483984836623, -0.14227761953270035, -0.2384058440442351,
+               -0.2689414213699951, 0.0, 0.7310585786300049, 1.7615941559557646, 2.8577223804673,
+               3.928055160151634],
+              [-2.416354975472916, -1.856234354263459, -1.2873014189882364, -0.7638334409883287,
+               -0.36713290505919505, 0.0, 0.835403899885462, 2.1475760812469877, 3.277268515997532,
+               4.220215568779826]),
+    "selu": ([-1.74625336066962, -1.7258986281898945, -1.6705687287671118, -1.520166468595695,
+              -1.1113307378125625, 0.0, 1.0507009873554805, 2.101401974710961, 3.1521029620664414,
+              4.202803949421922],
+             [-1.5332932256617793, -1.2518582388020294, -0.9923066122192254, -0.768906439142725,
+              -0.5786268790075374, 0.0, 1.0507009873554805, 2.101401974710961, 3.1521029620664414,
+              4.202803949421922]),
+}
+
+
+# verify/nn/layers.clj:316-326: a float32 backend cannot hold the reference's 1e-6 on a sum of ten
+# differences; the float tolerance is ten roundings of values below 1.2
+def activations(driver, datatype):
+    eps = 1e-6 if datatype == "double" else 10 * 1.2 * 2.0 ** -23
+    with context(driver, datatype):
+        for act_type, (forward, backward) in ACTIVATION_ANSWERS.items():
+            r = single({"type": act_type}, 1, [-1, 1] * 5, [-1, 1] * 5)
+            about_there(r["output"], forward * 5, eps)
+            about_there(r["input-gradient"], backward * 5, eps)
+
+
+# verify/nn/layers.clj:383-396
+def activations_batch(driver, datatype):
+    with context(driver, datatype):
+        for act_type, (forward, backward) in ACTIVATION_BATCH_ANSWERS.items():
+            item_range = list(range(-5, 5)) * 5
+            r = single({"type": act_type}, 5, item_range, item_range)
+            about_there(r["output"], forward * 5, 1e-3)
+            about_there(r["input-gradient"], backward * 5, 1e-3)
+
+
+# verify/nn/layers.clj:399-444: two batch sizes; the gradient passes through unchanged
+def softmax(driver, datatype):
+    with context(driver, datatype):
+        for batch_size in (1, 10):
+            values = list(range(1, 11))
+            r = single({"type": "softmax"}, batch_size, values * batch_size, values * batch_size)
+            e = np.exp(np.array(values, dtype=np.float64))
+            about_there(r["output"], np.tile(e / e.sum(), batch_size), 1e-6 * batch_size)
+            equals(values * batch_size, r["input-gradient"])
+
+
+# verify/nn/layers.clj:472-499: channels as the trailing axis of every pixel
+def softmax_channels(driver, datatype):
+    with context(driver, datatype):
+        batch_size, channels, n_pixels = 10, 4, 9
+        values = list(range(1, channels + 1)) * (n_pixels * batch_size)
+        shape = [n_pixels * channels]
+        r = single({"type": "softmax", "output-channels": channels}, batch_size, values, values, item_shape=shape)
+        e = np.exp(np.arange(1, channels + 1, dtype=np.float64))
+        about_there(r["output"], np.tile(e / e.sum(), n_pixels * batch_size), 1e-4)
+
+
+# verify/nn/layers.clj:640-672
+def dropout_bernoulli(driver, datatype):
+    with context(driver, datatype):
+        batch_size, item_count, repeat_count = 5, 20, 30
+        n = batch_size * item_count
+        node = {"type": "dropout", "distribution": "bernoulli", "probability": 0.8, "input-size": item_count}
+        layer = nl.create(node, batch_size)
+        inputs = [entry([1.0] * n, [batch_size, item_count])]
+        outputs = [{"buffer": ct.new_tensor([batch_size, item_count]),
+                    "gradient": ct.new_tensor([batch_size, item_count])}]
+        answers = []
+        for _ in range(repeat_count):
+            forward_backward(layer, {}, inputs, outputs, [[2.0] * n])
+            out = ct.to_double_array(outputs[0]["buffer"])
+            ig = ct.to_double_array(inputs[0]["gradient"])
+            # survivors carry exactly 1/p
+            assert set(np.unique(out)) <= {0.0, float(ct.to_double_array(ct.to_tensor([1.0 / 0.8]))[0])}
+            equals(2.0 * out, ig, 1e-6)
+            answers.append([out.sum(), (out == 0).sum(), ig.sum(), (ig == 0).sum()])
+        final = np.mean(np.array(answers, dtype=np.float64), axis=0)
+        assert final[1] == final[3]
+        assert abs(final[0] - n) < 3
+        assert abs(final[2] - 2.0 * n) < 10
+        # successive draws differ
+        assert len({a[0] for a in answers}) > 1
+
+
+# verify/nn/layers.clj:675-702
+def dropout_gaussian(driver, datatype):
+    with context(driver, datatype):
+        batch_size, item_count, repeat_count = 5, 100, 30
+        n = batch_size * item_count
+        node = {"type": "dropout", "distribution": "gaussian", "variance": 0.5, "input-size": item_count}
+        layer = nl.create(node, batch_size)
+        inputs = [entry([1.0] * n, [batch_size, item_count])]
+        outputs = [{"buffer": ct.new_tensor([batch_size, item_count]),
+                    "gradient": ct.new_tensor([batch_size, item_count])}]
+        answers = []
+        for _ in range(repeat_count):
+            forward_backward(layer, {}, inputs, outputs, [[2.0] * n])
+            answers.append([ct.to_double_array(outputs[0]["buffer"]).sum(),
+                            ct.to_double_array(inputs[0]["gradient"]).sum()])
+        final = np.mean(np.array(answers), axis=0)
+        assert abs(final[0] - n) < 10
+        assert abs(final[1] - 2.0 * n) < 20
+
+
+# verify/nn/layers.clj:705-763, restated without the network: training forward sets the running
+# statistics from the first batch, normalises to zero mean and unit variance per feature, and
+# inference then reproduces the training output from the running statistics
+def batch_normalization(driver, datatype):
+    with context(driver, datatype):
+        batch_size, input_size = 20, 20
+        rng = np.random.default_rng(5)
+        x = rng.standard_normal((batch_size, input_size)) * np.linspace(1, 3, input_size) + np.arange(input_size)
+        node = {"type": "batch-normalization", "mode": "elementwise", "input-size": input_size,
+                "epsilon": 1e-4, "average-factor": 0.9}
+        layer = nl.create(node, batch_size)
+        params = {"scale": entry(np.ones(input_size)), "bias": entry(np.zeros(input_size)),
+                  "means": entry(np.zeros(input_size), with_gradient=False),
+                  "variances": entry(np.zeros(input_size), with_gradient=False)}
+        inputs = [entry(x)]
+        outputs = [{"buffer": ct.new_tensor([batch_size, input_size]),
+                    "gradient": ct.new_tensor([batch_size, input_size])}]
+        og = rng.standard_normal((batch_size, input_size))
+        forward_backward(layer, params, inputs, outputs, [og])
+        out = ct.to_double_array(outputs[0]["buffer"]).reshape(batch_size, input_size)
+        tol = 1e-9 if datatype == "double" else 2e-5
+        equals(np.zeros(input_size), out.mean(axis=0), tol)
+        equals(np.ones(input_size), out.var(axis=0) * (x.var(axis=0) + 1e-4) / x.var(axis=0), 10 * tol)
+        equals(x.mean(axis=0), ct.to_double_array(params["means"]["buffer"]), 30 * tol)
+        # running variance is the unbiased one
+        equals(x.var(axis=0, ddof=1), ct.to_double_array(params["variances"]["buffer"]), 30 * tol)
+        equals(og.sum(axis=0), ct.to_double_array(params["bias"]["gradient"]), 30 * tol)
+        assert layer.local_average_factor == 0.9
+        # the gradient of a sum over the batch of normalised values is zero
+        equals(np.zeros(input_size), ct.to_double_array(inputs[0]["gradient"]).reshape(batch_size, -1).sum(axis=0),
+               30 * tol)
+
+
+# verify/nn/layers.clj:813-835
+def prelu(driver, datatype):
+    with context(driver, datatype):
+        batch_size, channel_count, input_dim = 10, 4, 3
+        input_size = input_dim * input_dim * channel_count
+        input = [-1, 1] * (input_size // 2) * batch_size
+        node = {"type": "prelu", "input-dimension": {"channels": channel_count, "height": input_dim,
+                                                     "width": input_dim}}
+        params = {"neg-scale": entry([0.25] * channel_count)}
+        r = single(node, batch_size, input, [1] * (batch_size * input_size), parameters=params,
+                   item_shape=[channel_count, input_dim, input_dim])
+        equals([-0.25 if v < 0 else 1.0 for v in input], r["output"])
+        equals([-10.0, 10.0, -10.0, 10.0], ct.to_double_array(params["neg-scale"]["gradient"]))
+        equals([0.25 if v < 0 else 1.0 for v in input], r["input-gradient"])
+
+
+# verify/nn/layers.clj:838-895
+def concatenate(driver, datatype):
+    with context(driver, datatype):
+        batch_size, item_count = 4, 5
+        left = np.arange(batch_size * item_count, dtype=np.float64).reshape(batch_size, item_count)
+        right = left + batch_size * item_count
+        for order in (("left", "right"), ("right", "left")):
+            data = {"left": left, "right": right}
+            inputs = [entry(data[k]) for k in order]
+            expected = np.concatenate([data[k] for k in order], axis=1)
+            outputs = [{"buffer": ct.new_tensor([batch_size, 2 * item_count]),
+                        "gradient": ct.new_tensor([batch_size, 2 * item_count])}]
+            layer = nl.create({"type": "concatenate"}, batch_size)
+            forward_backward(layer, {}, inputs, outputs, [expected])
+            equals(expected, ct.to_double_array(outputs[0]["buffer"]))
+            for k, e in zip(order, inputs):
+                equals(data[k], ct.to_double_array(e["gradient"]))
+
+
+# verify/nn/layers.clj:898-918
+def split(driver, datatype):
+    with context(driver, datatype):
+        input_size, batch_size = 5, 5
+        x = np.arange(batch_size * input_size, dtype=np.float64).reshape(batch_size, input_size)
+        inputs = [entry(x)]
+        outputs = [{"buffer": ct.new_tensor([batch_size, input_size]),
+                    "gradient": ct.new_tensor([batch_size, input_size])} for _ in range(2)]
+        layer = nl.create({"type": "split"}, batch_size)
+        forward_backward(layer, {}, inputs, outputs, [x, x])
+        for out in outputs:
+            equals(x, ct.to_double_array(out["buffer"]))
+        equals(2 * x, ct.to_double_array(inputs[0]["gradient"]))
+
+
+# verify/nn/layers.clj:922-953
+def join_add(driver, datatype):
+    with context(driver, datatype):
+        batch_size, item_count = 4, 5
+        left = np.arange(batch_size * item_count, dtype=np.float64).reshape(batch_size, item_count)
+        right = left + batch_size * item_count
+        inputs = [entry(left), entry(right)]
+        outputs = [{"buffer": ct.new_tensor([batch_size, item_count]),
+                    "gradient": ct.new_tensor([batch_size, item_count])}]
+        layer = nl.create({"type": "join"}, batch_size)
+        forward_backward(layer, {}, inputs, outputs, [left])
+        equals(left + right, ct.to_double_array(outputs[0]["buffer"]))
+        for e in inputs:
+            equals(left, ct.to_double_array(e["gradient"]))
+
+
+# verify/nn/layers.clj:956-987
+def join_add_ragged(driver, datatype):
+    with context(driver, datatype):
+        batch_size, counts = 4, [3, 4, 5]
+        seq = [-1, -2, 1, 4]
+        inputs = [entry([seq[i % 4] for i in range(batch_size * c)], [batch_size, c]) for c in counts]
+        outputs = [{"buffer": ct.new_tensor([batch_size, 5]), "gradient": ct.new_tensor([batch_size, 5])}]
+        layer = nl.create({"type": "join"}, batch_size)
+        forward_backward(layer, {}, inputs, outputs, [np.ones((batch_size, 5))])
+        equals([[-3.0, -6.0, 3.0, 8.0, -1.0],
+                [1.0, -2.0, 3.0, 3.0, -2.0],
+                [1.0, 6.0, -1.0, 2.0, 1.0],
+                [1.0, -2.0, 3.0, 5.0, 4.0]], ct.to_double_array(outputs[0]["buffer"]))
+        for e, c in zip(inputs, counts):
+            equals(np.ones(batch_size * c), ct.to_double_array(e["gradient"]))
+
+
+# compute/nn/layers.clj:603-660 with :operation :* — the reference stores no vector for it
+def join_multiply(driver, datatype):
+    with context(driver, datatype):
+        batch_size, counts = 3, [4, 2, 3]
+        rng = np.random.default_rng(11)
+        data = [rng.integers(-4, 5, size=(batch_size, c)).astype(np.float64) for c in counts]
+        og = rng.integers(-3, 4, size=(batch_size, 4)).astype(np.float64)
+        inputs = [entry(d) for d in data]
+        outputs = [{"buffer": ct.new_tensor([batch_size, 4]), "gradient": ct.new_tensor([batch_size, 4])}]
+        layer = nl.create({"type": "join", "operation": "*"}, batch_size)
+        forward_backward(layer, {}, inputs, outputs, [og])
+        expected = np.zeros((batch_size, 4))
+        expected[:, :2] = data[0][:, :2] * data[1][:, :2] * data[2][:, :2]
+        equals(expected, ct.to_double_array(outputs[0]["buffer"]))
+        for i, (e, c) in enumerate(zip(inputs, counts)):
+            g = np.zeros((batch_size, c))
+            others = [data[j][:, :2] for j in range(3) if j != i]
+            g[:, :2] = og[:, :2] * others[0] * others[1]
+            equals(g, ct.to_double_array(e["gradient"]))
+
+
+# loss/mse.clj:12-21, loss/softmax.clj:13-29, loss/regularization.clj:16-56: closed forms
+def loss_gradients(driver, datatype):
+    with context(driver, datatype):
+        rng = np.random.default_rng(3)
+        batch_size, n = 6, 10
+        v = rng.integers(-8, 9, size=(batch_size, n)) / 4.0
+        target = rng.integers(-8, 9, size=(batch_size, n)) / 4.0
+        tol = 1e-15 if datatype == "double" else 1e-6
+        bm = {"output": entry(v), "labels": entry(target, with_gradient=False)}
+        nl.mse_loss_gradient(bm)
+        equals(2.0 / n * (v - target), ct.to_double_array(bm["output"]["gradient"]), tol)
+        nl.softmax_loss_gradient(bm)
+        equals(v - target, ct.to_double_array(bm["output"]["gradient"]))
+
+        param = np.array([[-1.5, 0.0, 2.0], [0.25, -0.0, -3.0]])
+        g0 = np.array([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+        pe = {"output": {"buffer": ct.to_tensor(param), "gradient": ct.to_tensor(g0)}}
+        nl.L1RegularizationLoss(6).compute_loss_gradient(pe)
+        equals(g0 + np.where(param >= 0, 1.0, -1.0), ct.to_double_array(pe["output"]["gradient"]))
+        pe = {"output": {"buffer": ct.to_tensor(param), "gradient": ct.to_tensor(g0)}}
+        nl.L2RegularizationLoss().compute_loss_gradient(pe)
+        equals(g0 + param, ct.to_double_array(pe["output"]["gradient"]))
+
+
+# A two-layer network trained with the reference's call sequence end to end: linear, tanh, linear,
+# softmax, softmax loss, L2 on the weights, Adam.  Checked against the same steps in numpy.
+def train_small_network(driver, datatype):
+    from cortex_amd import optimize as opt
+
+    with context(driver, datatype) as stream:
+        backend = opt.Backend(stream=stream, datatype=datatype, type=getattr(driver, "type", "hip"))
+        rng = np.random.default_rng(17)
+        batch, n_in, n_hidden, n_out = 16, 8, 12, 4
+        w1, b1 = rng.standard_normal((n_hidden, n_in)) * 0.3, np.zeros(n_hidden)
+        w2, b2 = rng.standard_normal((n_out, n_hidden)) * 0.3, np.zeros(n_out)
+        x = rng.standard_normal((batch, n_in))
+        labels = np.eye(n_out)[rng.integers(0, n_out, size=batch)]
+        lam = 0.01
+
+        p1 = {"weights": entry(w1), "bias": entry(b1)}
+        p2 = {"weights": entry(w2), "bias": entry(b2)}
+        l1, act, l2, sm = (nl.create({"type": t}, batch) for t in ("linear", "tanh", "linear", "softmax"))
+        reg = nl.L2RegularizationLoss()
+
+        def buf(n):
+            return [{"buffer": ct.new_tensor([batch, n]), "gradient": ct.new_tensor([batch, n])}]
+        a0, a1, a2, a3, a4 = [entry(x)], buf(n_hidden), buf(n_hidden), buf(n_out), buf(n_out)
+        label_entry = entry(labels, with_gradient=False)
+        order = [p1["weights"], p1["bias"], p2["weights"], p2["bias"]]
+        total = sum(e["buffer"].ecount() for e in order)
+        state = {"m": ct.new_tensor([total]), "v": ct.new_tensor([total])}
+        optimizer = opt.create_optimizer(backend, opt.adam())
+
+        # numpy restatement of the same steps
+        ref = [w1.copy(), b1.copy(), w2.copy(), b2.copy()]
+        m, v = np.zeros(total), np.zeros(total)
+        pow1 = pow2 = 1.0
+        losses = []
+        for step in range(8):
+            for e in order:
+                ct.assign(e["gradient"], 0)
+            l1.forward(p1, a0, a1)
+            act.forward({}, a1, a2)
+            l2.forward(p2, a2, a3)
+            sm.forward({}, a3, a4)
+            nl.softmax_loss_gradient({"output": a4[0], "labels": label_entry})
+            sm.backward({}, a4, a3)
+            l2.backward(p2, a3, a2)
+            act.backward({}, a2, a1)
+            l1.backward(p1, a1, a0)
+            for p in (p1, p2):
+                # lambda scales the regulariser's gradient: gradient += lambda * weights
+                tmp = {"buffer": p["weights"]["buffer"], "gradient": ct.new_tensor(p["weights"]["buffer"].shape())}
+                reg.compute_loss_gradient({"output": tmp})
+                ct.binary_op(p["weights"]["gradient"], 1.0, p["weights"]["gradient"], lam, tmp["gradient"], "+")
+            optimizer = optimizer.batch_update(state)
+            offset = 0
+            for e in order:
+                optimizer.compute_parameters(state, 1.0 / batch, offset, ct.as_vector(e["gradient"]),
+                                             ct.as_vector(e["buffer"]))
+                offset += e["buffer"].ecount()
+
+            rw1, rb1, rw2, rb2 = ref
+            h_pre = x @ rw1.T + rb1
+            h = np.tanh(h_pre)
+            z = h @ rw2.T + rb2
+            e_z = np.exp(z - z.max(axis=1, keepdims=True))
+            prob = e_z / e_z.sum(axis=1, keepdims=True)
+            losses.append(-np.log((prob * labels).sum(axis=1)).mean())
+            dz = prob - labels
+            gw2, gb2 = dz.T @ h + lam * rw2, dz.sum(axis=0)
+            dh = (dz @ rw2) * (1 - h * h)
+            gw1, gb1 = dh.T @ x + lam * rw1, dh.sum(axis=0)
+            g = np.concatenate([a.reshape(-1) for a in (gw1, gb1, gw2, gb2)]) / batch
+            pow1, pow2 = pow1 * 0.9, pow2 * 0.999
+            m = 0.9 * m + 0.1 * g
+            v = 0.999 * v + 0.001 * g * g
+            upd = 0.001 * (m / (1 - pow1)) / (np.sqrt(v / (1 - pow2)) + 1e-8)
+            offset = 0
+            for i, a in enumerate(ref):
+                ref[i] = a - upd[offset:offset + a.size].reshape(a.shape)
+                offset += a.size
+
+            tol = 1e-11 if datatype == "double" else 2e-5
+            for e, a in zip(order, ref):
+                equals(a, ct.to_double_array(e["buffer"]), tol)
+            equals(prob, ct.to_double_array(a4[0]["buffer"]), tol)
+        assert losses[-1] < losses[0]

@@ -3,6 +3,7 @@ backend-neutral test bodies (tests/reference_suite.py) run on the oracle
 driver.  CPU only."""
 import pytest
 
+import layer_suite as ls
 import reference_suite as rs
 from oracle_backend import OracleDriver
 
@@ -12,6 +13,12 @@ ALL_DTYPE_TESTS = ["assign_constant", "assign_marshal", "binary_constant_op", "b
 FLOAT_TESTS = ["gemm", "gemv", "activation_forward", "activation_gradient", "softmax", "batch_normalize",
                "batch_normalize_update_and_apply", "batch_normalize_gradients", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
                "adam_trajectory", "sgd_closed_form"]
+
+# tests/layer_suite.py: the layers, loss gradients and regularisers built on the tensor calls
+LAYER_TESTS = ["relu_activation", "linear", "activations", "activations_batch", "softmax", "softmax_channels",
+               "dropout_bernoulli", "dropout_gaussian", "batch_normalization", "prelu",
+               "concatenate", "split", "join_add", "join_add_ragged", "join_multiply", "loss_gradients",
+               "train_small_network"]
 
 
 @pytest.fixture(scope="module")
@@ -29,6 +36,12 @@ def test_all_dtypes(driver, name, datatype):
 @pytest.mark.parametrize("name", FLOAT_TESTS)
 def test_float_double(driver, name, datatype):
     getattr(rs, name)(driver, datatype)
+
+
+@pytest.mark.parametrize("datatype", rs.FLOAT_DTYPES)
+@pytest.mark.parametrize("name", LAYER_TESTS)
+def test_layers(driver, name, datatype):
+    getattr(ls, name)(driver, datatype)
 
 
 @pytest.mark.parametrize("datatype", ["int", "long"])

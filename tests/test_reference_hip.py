@@ -1,10 +1,11 @@
-"""The reference's backend-neutral test bodies (tests/reference_suite.py) on
+"""The reference's backend-neutral test bodies (tests/reference_suite.py, tests/layer_suite.py) on
 the HIP driver, as test/clj/cortex/compute/cuda/tensor_test.clj runs them on
 the CUDA driver.  Needs a GPU."""
 import pytest
 
 import reference_suite as rs
-from test_reference_cpu_oracle import ALL_DTYPE_TESTS, FLOAT_TESTS
+import layer_suite as ls
+from test_reference_cpu_oracle import ALL_DTYPE_TESTS, FLOAT_TESTS, LAYER_TESTS
 
 pytestmark = pytest.mark.gpu
 
@@ -30,6 +31,12 @@ def test_all_dtypes(driver, name, datatype):
 @pytest.mark.parametrize("name", FLOAT_TESTS)
 def test_float_double(driver, name, datatype):
     getattr(rs, name)(driver, datatype)
+
+
+@pytest.mark.parametrize("datatype", rs.FLOAT_DTYPES)
+@pytest.mark.parametrize("name", LAYER_TESTS)
+def test_layers(driver, name, datatype):
+    getattr(ls, name)(driver, datatype)
 
 
 @pytest.mark.parametrize("datatype", ["int", "long"])
