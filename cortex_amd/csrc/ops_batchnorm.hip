@@ -35,6 +35,9 @@ using namespace cthip;
 namespace {
 
 enum { kBnNormalize = 0, kBnGradient = 1 };
+constexpr int64_t kRowApplyBytes = int64_t(32) << 20;  // plain normalize: size from which the constants get a launch of their own
+constexpr int kRowApplyMinVecs = 8;  // shortest row, in vectors, that the row kernel takes
+constexpr int kRaggedApplyMinVecs = 64;  // the same for rows that are no whole number of vectors (measured: 49-element rows lose)
 constexpr int kParamStride = 8;  // doubles per channel in the parameter table
 // constants of a channel as the apply pass holds them:
 //   normalize: mean, inv_std (rounded to T), scale, shift -- derived from the statistics vectors on the fly
@@ -67,6 +70,7 @@ struct BnArgs {
   uint32_t table_slots;      // channels held in the LDS table
   uint32_t table_full;       // the table holds every channel (indexed by channel) instead of a window of rows
   uint32_t apply_rows_per_seg;  // column-style apply: batch rows per block
+  uint32_t row_holds_vectors;   // E and the launch's first element are multiples of the vector width
 };
 
 struct BnFinish {
@@ -311,21 +315,32 @@ __global__ void __launch_bounds__(kBlock) bn_stats_col_kernel(const BnArgs a) {
 // derives them from the statistics vectors (batch-normalize-impl, :766-777: the
 // inverse standard deviation is rounded to T); gradient mode reads the table the
 // finishing pass wrote.
+// The load and the arithmetic are separate so that a caller can put other loads
+// between them.
 template <class T, int MODE>
-__device__ __forceinline__ double bn_channel_constant(const BnArgs& a, uint32_t ch, int k) {
+__device__ __forceinline__ double bn_channel_constant_load(const BnArgs& a, uint32_t ch, int k) {
   if constexpr (MODE == kBnGradient) {
     return a.params[(int64_t)ch * kParamStride + k];
   } else {
-    switch (k) {
-      case 0: return (double)reinterpret_cast<const T*>(a.means)[ch];
-      case 1: {
-        const T eps = (T)a.epsilon;
-        return (double)(T)sqrt(1.0 / ((double)reinterpret_cast<const T*>(a.variances)[ch] + (double)eps));
-      }
-      case 2: return (double)reinterpret_cast<const T*>(a.scale)[ch];
-      default: return (double)reinterpret_cast<const T*>(a.bias)[ch];
+    const void* src = k == 0 ? a.means : k == 1 ? a.variances : k == 2 ? a.scale : a.bias;
+    return (double)reinterpret_cast<const T*>(src)[ch];
+  }
+}
+
+template <class T, int MODE>
+__device__ __forceinline__ double bn_channel_constant_finish(const BnArgs& a, double raw, int k) {
+  if constexpr (MODE != kBnGradient) {
+    if (k == 1) {
+      const T eps = (T)a.epsilon;
+      return (double)(T)sqrt(1.0 / (raw + (double)eps));
     }
   }
+  return raw;
+}
+
+template <class T, int MODE>
+__device__ __forceinline__ double bn_channel_constant(const BnArgs& a, uint32_t ch, int k) {
+  return bn_channel_constant_finish<T, MODE>(a, bn_channel_constant_load<T, MODE>(a, ch, k), k);
 }
 
 // One wave per channel adds the channel's partial sums (segments, and columns in
@@ -392,6 +407,11 @@ __global__ void __launch_bounds__(kBlock) bn_finish_kernel(const BnArgs a, const
     const T batch_variance = (T)(new_var / count_val);
     reinterpret_cast<T*>(f.batch_means)[c] = new_mean;
     reinterpret_cast<T*>(f.batch_variances)[c] = batch_variance;
+    // the apply pass's constants, as bn_channel_constant derives them from the stored statistics
+    pm[0] = (double)new_mean;
+    pm[1] = bn_channel_constant_finish<T, kBnNormalize>(a, (double)batch_variance, 1);
+    pm[2] = (double)reinterpret_cast<const T*>(a.scale)[c];
+    pm[3] = (double)reinterpret_cast<const T*>(a.bias)[c];
     running_means[c] = (T)((double)mean * ave_lerp + (double)new_mean * (double)ave_factor);
     running_variances[c] =
         (T)((double)variance * ave_lerp + (double)(T)(new_var / running_count_val) * (double)ave_factor);
@@ -476,7 +496,16 @@ __global__ void __launch_bounds__(kBlock) bn_apply_kernel(const BnArgs a) {
   const T* x = reinterpret_cast<const T*>(a.x);
   const T* og = reinterpret_cast<const T*>(a.og);
   T* out = reinterpret_cast<T*>(a.out);
-  // the operands' loads are in flight while the table is filled
+  // Loads return in issue order: the first table entry's load goes out ahead of
+  // the operands', so the table is complete while the operands are still in flight.
+  const uint32_t n_table = a.table_slots * NP;
+  const uint32_t slot_t = threadIdx.x / NP, k_t = threadIdx.x - slot_t * NP;
+  double raw = 0.0;
+  if (threadIdx.x < n_table) {
+    uint32_t q, ch;
+    a.c_fd.divmod(ch_base + slot_t, q, ch);
+    raw = bn_channel_constant_load<T, MODE>(a, ch, (int)k_t);
+  }
   V xv[UNROLL], gv[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
@@ -486,7 +515,8 @@ __global__ void __launch_bounds__(kBlock) bn_apply_kernel(const BnArgs a) {
       if constexpr (MODE == kBnGradient) gv[u] = nt_load(reinterpret_cast<const V*>(og + j));
     }
   }
-  for (uint32_t i = threadIdx.x; i < a.table_slots * NP; i += kBlock) {
+  if (threadIdx.x < n_table) table[threadIdx.x] = bn_channel_constant_finish<T, MODE>(a, raw, (int)k_t);
+  for (uint32_t i = threadIdx.x + kBlock; i < n_table; i += kBlock) {
     const uint32_t slot = i / NP, k = i - slot * NP;
     uint32_t q, ch;
     a.c_fd.divmod(ch_base + slot, q, ch);
@@ -499,18 +529,142 @@ __global__ void __launch_bounds__(kBlock) bn_apply_kernel(const BnArgs a) {
     const int64_t j = blk_first + jr;
     if (j < end) {
       V r;
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        uint32_t slot = a.e_fd.div(rel0 + jr + e);  // (batch, channel) rows past row_first
+      if (VEC > 1 && a.row_holds_vectors) {
+        // a vector lies inside one (batch, channel) row: one table read serves its elements
+        uint32_t slot = a.e_fd.div(rel0 + jr);
         if (a.table_full) {
           uint32_t q;
           a.c_fd.divmod(ch_first + slot, q, slot);
         }
-        r.v[e] = bn_apply_one<T, MODE>(table + slot * NP, xv[u].v[e], MODE == kBnGradient ? gv[u].v[e] : (T)0);
+        double p[NP];
+#pragma unroll
+        for (int k = 0; k < NP; ++k) p[k] = table[slot * NP + k];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.v[e] = bn_apply_one<T, MODE>(p, xv[u].v[e], MODE == kBnGradient ? gv[u].v[e] : (T)0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          uint32_t slot = a.e_fd.div(rel0 + jr + e);  // (batch, channel) rows past row_first
+          if (a.table_full) {
+            uint32_t q;
+            a.c_fd.divmod(ch_first + slot, q, slot);
+          }
+          r.v[e] = bn_apply_one<T, MODE>(table + slot * NP, xv[u].v[e], MODE == kBnGradient ? gv[u].v[e] : (T)0);
+        }
       }
       *reinterpret_cast<V*>(out + j) = r;
     }
   }
+}
+
+// The normalize constants of every channel into the parameter table, for the
+// row kernel below when no finishing pass has written them.
+template <class T>
+__global__ void __launch_bounds__(kBlock) bn_constants_kernel(const BnArgs a) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t ch = i >> 2, k = i & 3;
+  if (ch >= a.C) return;
+  a.params[(int64_t)ch * kParamStride + k] = bn_channel_constant<T, kBnNormalize>(a, ch, (int)k);
+}
+
+// One vector per lane, constants from the parameter table: no LDS table, no
+// barrier, and waves as short as those of the plain elementwise kernels.  With
+// rows of at least a block's width the block's 256 vectors lie in at most two
+// (batch, channel) rows, so the constants are read with wave-uniform addresses
+// and a lane only picks its row's set.
+struct BnRowArgs {
+  uint64_t total_vecs;
+  FastDiv nv_fd, c_fd;   // vectors per row; channels
+  const double* params;
+  const void* x;
+  const void* og;
+  void* out;
+};
+
+template <class T, int VEC, int MODE, int STREAM, bool RAGGED = false>
+__global__ void __launch_bounds__(kBlock) bn_apply_rows_kernel(const BnRowArgs a) {
+  using V = Vec<T, VEC>;
+  constexpr int NP = bn_nparam<MODE>::value;
+  const uint64_t total = a.total_vecs;
+  const FastDiv nfd = a.nv_fd, cfd = a.c_fd;
+  const double* const params = a.params;
+  const V* const x = reinterpret_cast<const V*>(a.x);
+  const V* const og = reinterpret_cast<const V*>(MODE == kBnGradient ? a.og : a.x);
+  V* const out = reinterpret_cast<V*>(a.out);
+  asm volatile("" ::"s"(total), "s"(nfd.d), "s"(nfd.m), "s"(nfd.s), "s"(cfd.d), "s"(cfd.m), "s"(cfd.s), "s"(params),
+               "s"(x), "s"(og), "s"(out));
+  const uint64_t v_first = (uint64_t)blockIdx.x * (uint64_t)kBlock;
+  const uint64_t v = v_first + threadIdx.x;
+  if (v >= total) return;
+  V xv, gv;
+  if constexpr (STREAM >= 1) xv = nt_load(x + v); else xv = x[v];
+  if constexpr (MODE == kBnGradient) {
+    if constexpr (STREAM >= 1) gv = nt_load(og + v); else gv = og[v];
+  }
+  double p[NP];
+  if constexpr (RAGGED) {
+    // Rows of E >= VEC elements that are no whole number of vectors (nv_fd divides
+    // by E here): a vector can end in the next row, whose constants the lane then
+    // fetches as well.
+    uint32_t row, rem, q, ch;
+    nfd.divmod((uint32_t)v * VEC, row, rem);
+    cfd.divmod(row, q, ch);
+    const double* pl = params + (uint64_t)ch * kParamStride;
+#pragma unroll
+    for (int k = 0; k < NP; ++k) p[k] = pl[k];
+    const uint32_t in_row = nfd.d - rem;  // elements of the vector that lie in `row`
+    V r;
+    if (in_row < (uint32_t)VEC) {
+      const uint32_t ch_b = ch + 1 == cfd.d ? 0u : ch + 1;
+      const double* pb = params + (uint64_t)ch_b * kParamStride;
+      double p2[NP];
+#pragma unroll
+      for (int k = 0; k < NP; ++k) p2[k] = pb[k];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        double pe[NP];
+#pragma unroll
+        for (int k = 0; k < NP; ++k) pe[k] = (uint32_t)e >= in_row ? p2[k] : p[k];
+        r.v[e] = bn_apply_one<T, MODE>(pe, xv.v[e], MODE == kBnGradient ? gv.v[e] : (T)0);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) r.v[e] = bn_apply_one<T, MODE>(p, xv.v[e], MODE == kBnGradient ? gv.v[e] : (T)0);
+    }
+    if constexpr (STREAM == 2) nt_store(r, out + v);
+    else out[v] = r;
+    return;
+  }
+  if (nfd.d >= (uint32_t)kBlock) {
+    uint32_t row_a, cv_a, q, ch_a;
+    nfd.divmod((uint32_t)v_first, row_a, cv_a);
+    cfd.divmod(row_a, q, ch_a);
+    const double* pa = params + (uint64_t)ch_a * kParamStride;
+#pragma unroll
+    for (int k = 0; k < NP; ++k) p[k] = pa[k];
+    if (cv_a + (uint32_t)kBlock > nfd.d) {  // the block runs into the next row
+      const uint32_t ch_b = ch_a + 1 == cfd.d ? 0u : ch_a + 1;
+      const double* pb = params + (uint64_t)ch_b * kParamStride;
+      const bool next = cv_a + threadIdx.x >= nfd.d;
+#pragma unroll
+      for (int k = 0; k < NP; ++k) {
+        const double other = pb[k];
+        p[k] = next ? other : p[k];
+      }
+    }
+  } else {
+    // shorter rows: a lane finds its own row; its neighbours mostly read the same table entry
+    uint32_t q, ch;
+    cfd.divmod(nfd.div((uint32_t)v), q, ch);
+    const double* pl = params + (uint64_t)ch * kParamStride;
+#pragma unroll
+    for (int k = 0; k < NP; ++k) p[k] = pl[k];
+  }
+  V r;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) r.v[e] = bn_apply_one<T, MODE>(p, xv.v[e], MODE == kBnGradient ? gv.v[e] : (T)0);
+  if constexpr (STREAM == 2) nt_store(r, out + v);
+  else out[v] = r;
 }
 
 // ---------------------------------------------------------------- host side
@@ -520,6 +674,7 @@ struct BnPlan {
   bool col_style;   // few elements per channel: lanes own columns of [batch, channels * elements]
   bool vec_stats;
   bool nt_stats;    // the operands exceed the caches: the statistics pass reads them with non-temporal loads
+  bool params_ready = false;  // the parameter table holds the apply pass's constants
   dim3 stats_grid;
   size_t scratch_bytes;
 };
@@ -611,6 +766,7 @@ bool bn_try_apply_range(hipStream_t s, BnArgs a, int64_t first, int64_t count) {
   constexpr int64_t kSpan = (int64_t)kBlock * VEC * UNROLL;
   a.first = first;
   a.count = count;
+  a.row_holds_vectors = (a.E % VEC == 0 && first % VEC == 0) ? 1u : 0u;
   const int64_t window = (kSpan + a.E - 1) / a.E + 1;  // (batch, channel) rows a block's range can touch
   a.table_full = window >= a.C ? 1u : 0u;
   a.table_slots = (uint32_t)(a.table_full ? a.C : window);
@@ -647,6 +803,29 @@ void bn_launch_apply(hipStream_t s, const BnPlan& plan) {
   if (plan.col_style) {
     if (aligned && a.W % VMAX == 0) bn_launch_apply_col<T, VMAX, MODE>(s, a);
     else bn_launch_apply_col<T, 1, MODE>(s, a);
+  } else if (aligned && VMAX > 1 && a.E / VMAX >= (a.E % VMAX ? kRaggedApplyMinVecs : kRowApplyMinVecs) &&
+             a.N < (int64_t(1) << 32) && plan.params_ready) {
+    const bool ragged = a.E % VMAX != 0;
+    BnRowArgs r;
+    r.total_vecs = (uint64_t)(a.N / VMAX);
+    r.nv_fd = FastDiv((uint32_t)(ragged ? a.E : a.E / VMAX));
+    r.c_fd = FastDiv((uint32_t)a.C);
+    r.params = a.params;
+    r.x = a.x; r.og = a.og; r.out = a.out;
+    const dim3 grid((uint32_t)((r.total_vecs + kBlock - 1) / kBlock));
+    const double bytes = (double)a.N * sizeof(T) * (MODE == kBnGradient ? 3 : 2);
+    const int level = bytes >= (double)(int64_t(1) << 30) ? 2 : bytes >= (double)kStreamingBytes ? 1 : 0;
+    if (ragged) {
+      if (level == 2) hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 2, true>), grid, dim3(kBlock), 0, s, r);
+      else if (level == 1) hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 1, true>), grid, dim3(kBlock), 0, s, r);
+      else hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 0, true>), grid, dim3(kBlock), 0, s, r);
+      // the elements past the last whole vector
+      bn_launch_apply_range<T, 1, MODE>(s, a, a.N / VMAX * VMAX, a.N % VMAX);
+    } else {
+      if (level == 2) hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 2>), grid, dim3(kBlock), 0, s, r);
+      else if (level == 1) hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 1>), grid, dim3(kBlock), 0, s, r);
+      else hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 0>), grid, dim3(kBlock), 0, s, r);
+    }
   } else if (aligned && VMAX > 1) {
     const int64_t body = a.N / VMAX * VMAX;
     bn_launch_apply_range<T, VMAX, MODE>(s, a, 0, body);
@@ -670,6 +849,11 @@ int bn_normalize(hipStream_t s, void* output, const void* input, const void* mea
   if (int rc = bn_plan<T, kBnNormalize>(s, B, C, E, input, nullptr, output, false, &plan)) return rc;
   bn_set_statistics(&plan.a, means, variances, scale, bias, epsilon);
   note_kernel(plan.col_style ? "bn_apply_col" : "bn_apply");
+  // a launch of its own for the constants pays off once the tensor is large
+  if (!plan.col_style && (double)plan.a.N * sizeof(T) >= (double)kRowApplyBytes) {
+    hipLaunchKernelGGL((bn_constants_kernel<T>), dim3((uint32_t)((C * 4 + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, plan.a);
+    plan.params_ready = true;
+  }
   bn_launch_apply<T, kBnNormalize>(s, plan);
   return after_launch(s);
 }
@@ -690,6 +874,7 @@ int bn_update_and_apply(hipStream_t s, void* output, const void* input, void* ba
   f.running_means = running_means; f.running_variances = running_variances;
   f.average_factor = average_factor;
   hipLaunchKernelGGL((bn_finish_kernel<T, kBnNormalize>), channel_grid(C, kBlock / 64), dim3(kBlock), 0, s, plan.a, f);
+  plan.params_ready = true;
   bn_launch_apply<T, kBnNormalize>(s, plan);
   return after_launch(s);
 }
@@ -707,6 +892,7 @@ int bn_gradients(hipStream_t s, void* input_gradient, void* scale_gradient, void
   std::memset(&f, 0, sizeof(f));
   f.scale_gradient = scale_gradient; f.bias_gradient = bias_gradient;
   hipLaunchKernelGGL((bn_finish_kernel<T, kBnGradient>), channel_grid(C, kBlock / 64), dim3(kBlock), 0, s, plan.a, f);
+  plan.params_ready = true;
   bn_launch_apply<T, kBnGradient>(s, plan);
   return after_launch(s);
 }

@@ -634,7 +634,8 @@ def test_softmax_and_activation_gradient_errors(P):
 # They cover both statistics kernels (rows of at least 128 bytes are walked row style), vector
 # and scalar accesses, table-per-window and table-of-all-channels apply passes, and tails.
 BN_SHAPES = [(4, 3), (128, 1000), (37, 130), (1000, 64), (5, 4099), (2, 3, 4), (8, 16, 196), (4, 5, 49),
-             (3, 7, 1024), (16, 3, 4100), (2, 2, 31), (70, 33, 8), (2, 3000, 4), (33, 6, 1000), (1, 4, 64)]
+             (3, 7, 1024), (16, 3, 4100), (2, 2, 31), (70, 33, 8), (2, 3000, 4), (33, 6, 1000), (1, 4, 64),
+             (6, 10, 1023), (3, 4, 35), (9, 3, 50), (5, 3, 257), (2, 7, 513)]
 
 
 def bn_close(buf, what, code, scale_by=None):
@@ -672,6 +673,19 @@ def test_batch_normalize(P, code, shape):
     t["variances"].reset()
     k = P.run(H.batch_normalize, V["out"], V["x"], V["means"], V["variances"], V["scale"], V["bias"], 1e-2, b, c, e)
     compare(t["out"], f"batch-normalize {shape} ({k})")      # elementwise in the CPU backend's order: bit-exact
+    P.run(H.batch_normalize, V["x"], V["x"], V["means"], V["variances"], V["scale"], V["bias"], 1e-2, b, c, e)
+    compare(t["x"], f"batch-normalize {shape} in place")
+
+
+@pytest.mark.parametrize("code", FLOATS)
+def test_batch_normalize_large_rows(P, code):
+    """From 32 MiB on, the plain normalization of long rows writes its channel constants in a
+    launch of their own and reads them per row; the rows here end inside blocks."""
+    shape = (8, 64, 16400)
+    rng = np.random.default_rng(44)
+    t, V, (b, c, e) = bn_setup(P, rng, code, shape)
+    P.run(H.batch_normalize, V["out"], V["x"], V["means"], V["variances"], V["scale"], V["bias"], 1e-2, b, c, e)
+    compare(t["out"], f"batch-normalize {shape}")
     P.run(H.batch_normalize, V["x"], V["x"], V["means"], V["variances"], V["scale"], V["bias"], 1e-2, b, c, e)
     compare(t["x"], f"batch-normalize {shape} in place")
 
