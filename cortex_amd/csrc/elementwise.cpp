@@ -96,14 +96,14 @@ int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_
   return CT_OK;
 }
 
-int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_b_edge, TileArgs* a, size_t* lds_bytes,
+int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int tile_b_edge, TileArgs* a, size_t* lds_bytes,
                  uint32_t* grid) {
   const Canon& c = plan.canon;
   const int b = plan.tile_b;
   std::memset(a, 0, sizeof(*a));
   a->sizeA = (uint32_t)c.size[0];
   a->sizeB = (uint32_t)c.size[b];
-  a->tilesA = (a->sizeA + kTileA - 1) / kTileA;
+  a->tilesA = (a->sizeA + tile_a_edge - 1) / tile_a_edge;
   a->tilesB = (a->sizeB + tile_b_edge - 1) / tile_b_edge;
   a->tilesA_fd = FastDiv(a->tilesA);
   a->tilesB_fd = FastDiv(a->tilesB);
@@ -129,7 +129,7 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_b_edge, TileAr
     if (!ops[k].ptr) a->const_mask |= 1u << k;
     if (plan.via_lds[k]) {
       a->lds_mask |= 1u << k;
-      lds = std::max(lds, tile_slot_bytes((size_t)ops[k].elem_size, tile_b_edge));  // one tile, used in turn
+      lds = std::max(lds, tile_slot_bytes((size_t)ops[k].elem_size, tile_a_edge, tile_b_edge));  // one tile, used in turn
     }
   }
   *lds_bytes = lds;

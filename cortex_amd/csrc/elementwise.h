@@ -316,25 +316,30 @@ template <class F> struct elem_sizes {
   static constexpr size_t max_in = m012;
   static constexpr size_t max_all = m012 > sizeof(typename F::Out) ? m012 : sizeof(typename F::Out);
 };
-// Tile shape: kTileA elements along A (the destination's unit-stride axis) by
-// tile_b<F> elements along B (the axis the transposed inputs are unit-stride
-// along).  The read side matters most: 512-byte source segments measured
-// 83 % of peak on a transposing float copy against 76 % for 256-byte ones, while
-// shrinking the written segments from 256 to 128 bytes cost about 1 %.
-constexpr int kTileA = 32;
-template <class F> struct tile_b {
-  static constexpr int value = elem_sizes<F>::max_in > 4 ? 64 : 128;
+// Tile shape: TA elements along A (the destination's unit-stride axis) by TB
+// elements along B (the axis the transposed inputs are unit-stride along).
+// The longer edge goes to the side with more streams.  Transposed inputs in the
+// majority (or level with the directly readable streams, the destination
+// included): 32 x 128, 512-byte source segments, which measured 83 % of peak on
+// a transposing float copy against 76 % for 256-byte ones, while shrinking the
+// written segments from 256 to 128 bytes cost about 1 %.  Directly readable
+// streams in the majority (WIDE_A): the mirror image, so that they and the
+// destination move in 512-byte segments.
+template <class F, bool WIDE_A> struct tile_shape {
+  static constexpr bool wide_elem = elem_sizes<F>::max_in > 4;
+  static constexpr int ta = WIDE_A ? (wide_elem ? 64 : 128) : 32;
+  static constexpr int tb = WIDE_A ? 32 : (wide_elem ? 64 : 128);
 };
-constexpr size_t tile_slot_bytes(size_t elem, int tb) { return ((elem * kTileA * (tb + 1)) + 15) & ~size_t(15); }
+constexpr size_t tile_slot_bytes(size_t elem, int ta, int tb) { return ((elem * ta * (tb + 1)) + 15) & ~size_t(15); }
 
-// Reads this lane's share of a kTileA x TB tile of an operand that is
+// Reads this lane's share of a TA x TB tile of an operand that is
 // unit-stride along B: lane tx walks B (TB consecutive elements per source
 // row), the block's ROWS lane rows walk A.  The pointer advances by a constant
 // step.
-template <class T, int TB, bool FULL, bool STREAM>
+template <class T, int TA, int TB, bool FULL, bool STREAM>
 __device__ __forceinline__ void tile_read(T* v, const T* p, int64_t step, uint32_t a_left, bool b_ok, int ty) {
   constexpr int ROWS = kBlock / TB;
-  constexpr int IT = kTileA / ROWS;
+  constexpr int IT = TA / ROWS;
 #pragma unroll
   for (int i = 0; i < IT; ++i) {
     if (FULL || (b_ok && (uint32_t)(ty + i * ROWS) < a_left)) {
@@ -361,14 +366,14 @@ __device__ __forceinline__ void tile_read_direct(T* v, const T* q, int64_t step,
 // Transposes the lane values through the block's single LDS tile (rows padded
 // to TB + 1 elements: conflict-free both ways).  On entry v[i] holds element
 // (a = ty + i*ROWS_R, b = tx) with tx = t % TB; on exit element
-// (a = wx, b = wy + i*ROWS_W) with wx = t % kTileA.
-template <class T, int TB>
+// (a = wx, b = wy + i*ROWS_W) with wx = t % TA.
+template <class T, int TA, int TB>
 __device__ __forceinline__ void tile_transpose(T* v, char* smem, bool need_sync_before) {
-  constexpr int ROWS_R = kBlock / TB, ROWS_W = kBlock / kTileA;
-  constexpr int IT = kTileA / ROWS_R;
+  constexpr int ROWS_R = kBlock / TB, ROWS_W = kBlock / TA;
+  constexpr int IT = TA / ROWS_R;
   static_assert(IT == TB / ROWS_W, "both phases move the same number of elements per lane");
   const int tx = threadIdx.x % TB, ty = threadIdx.x / TB;
-  const int wx = threadIdx.x % kTileA, wy = threadIdx.x / kTileA;
+  const int wx = threadIdx.x % TA, wy = threadIdx.x / TA;
   T* lds = reinterpret_cast<T*>(smem);
   if (need_sync_before) __syncthreads();
 #pragma unroll
@@ -378,7 +383,7 @@ __device__ __forceinline__ void tile_transpose(T* v, char* smem, bool need_sync_
   for (int i = 0; i < IT; ++i) v[i] = lds[wx * (TB + 1) + wy + i * ROWS_W];
 }
 
-template <class F, bool FULL, bool STREAM>
+template <class F, bool FULL, bool STREAM, bool WIDE_A>
 __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const int64_t* off, uint32_t a0, uint32_t b0,
                                           char* smem) {
   using Out = typename F::Out;
@@ -386,11 +391,11 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   using In1 = typename F::In1;
   using In2 = typename F::In2;
   constexpr int NIN = F::NIN;
-  constexpr int TB = tile_b<F>::value;
-  constexpr int ROWS_R = kBlock / TB, ROWS_W = kBlock / kTileA;
-  constexpr int IT = kTileA / ROWS_R;
+  constexpr int TA = tile_shape<F, WIDE_A>::ta, TB = tile_shape<F, WIDE_A>::tb;
+  constexpr int ROWS_R = kBlock / TB, ROWS_W = kBlock / TA;
+  constexpr int IT = TA / ROWS_R;
   const int tx = threadIdx.x % TB, ty = threadIdx.x / TB;
-  const int wx = threadIdx.x % kTileA, wy = threadIdx.x / kTileA;
+  const int wx = threadIdx.x % TA, wy = threadIdx.x / TA;
   const uint32_t a_left = a.sizeA - a0, b_left = a.sizeB - b0;  // valid extent of this tile
   const bool t0 = NIN >= 1 && ((a.lds_mask >> 1) & 1u), t1 = NIN >= 2 && ((a.lds_mask >> 2) & 1u),
              t2 = NIN >= 3 && ((a.lds_mask >> 3) & 1u);
@@ -425,13 +430,13 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   In2 v2[IT];
   const bool b_ok = (uint32_t)tx < b_left;
   if constexpr (NIN >= 1)
-    if (t0) tile_read<In0, TB, FULL, STREAM>(v0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
+    if (t0) tile_read<In0, TA, TB, FULL, STREAM>(v0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1] + (int64_t)(a0 + ty) * a.strideA[1] + (b0 + tx),
                                      (int64_t)ROWS_R * a.strideA[1], a_left, b_ok, ty);
   if constexpr (NIN >= 2)
-    if (t1) tile_read<In1, TB, FULL, STREAM>(v1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
+    if (t1) tile_read<In1, TA, TB, FULL, STREAM>(v1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2] + (int64_t)(a0 + ty) * a.strideA[2] + (b0 + tx),
                                      (int64_t)ROWS_R * a.strideA[2], a_left, b_ok, ty);
   if constexpr (NIN >= 3)
-    if (t2) tile_read<In2, TB, FULL, STREAM>(v2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
+    if (t2) tile_read<In2, TA, TB, FULL, STREAM>(v2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3] + (int64_t)(a0 + ty) * a.strideA[3] + (b0 + tx),
                                      (int64_t)ROWS_R * a.strideA[3], a_left, b_ok, ty);
   // operands that are read along A directly (not through LDS) are fetched now as well, so
   // that their latency overlaps the transposed operands' instead of following the LDS rounds
@@ -442,9 +447,9 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   if constexpr (NIN >= 3)
     if (q2) tile_read_direct<In2, IT, FULL>(v2, q2, s2, a_ok, b_left, wy, ROWS_W);
   bool used = false;
-  if constexpr (NIN >= 1) if (t0) { tile_transpose<In0, TB>(v0, smem, used); used = true; }
-  if constexpr (NIN >= 2) if (t1) { tile_transpose<In1, TB>(v1, smem, used); used = true; }
-  if constexpr (NIN >= 3) if (t2) { tile_transpose<In2, TB>(v2, smem, used); used = true; }
+  if constexpr (NIN >= 1) if (t0) { tile_transpose<In0, TA, TB>(v0, smem, used); used = true; }
+  if constexpr (NIN >= 2) if (t1) { tile_transpose<In1, TA, TB>(v1, smem, used); used = true; }
+  if constexpr (NIN >= 3) if (t2) { tile_transpose<In2, TA, TB>(v2, smem, used); used = true; }
 
   // phase 2: lane wx walks A (the destination's unit-stride axis), lane rows walk B
 #pragma unroll
@@ -463,13 +468,13 @@ __device__ __forceinline__ void tile_body(const F& f, const TileArgs& a, const i
   }
 }
 
-// One block per kTileA x TB tile.  All transposed operands share one LDS tile,
+// One block per TA x TB tile.  All transposed operands share one LDS tile,
 // used in turn, so the LDS footprint (and with it the number of resident
 // blocks) does not grow with the operand count.
-template <class F, bool STREAM>
+template <class F, bool STREAM, bool WIDE_A>
 __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileArgs a) {
   constexpr int NIN = F::NIN;
-  constexpr int TB = tile_b<F>::value;
+  constexpr int TA = tile_shape<F, WIDE_A>::ta, TB = tile_shape<F, WIDE_A>::tb;
   extern __shared__ __align__(16) char smem[];
 
   // Every argument the block needs is named here so that the compiler fetches
@@ -487,9 +492,15 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
   uint32_t bid, tb, ta, q0;
   // tiles along B vary fastest: consecutive blocks read neighbouring segments
   // of the same source rows (measured 71 % of peak against 58 % with tiles
-  // along A fastest on a transposed [8192,8192] float input)
-  a.tilesB_fd.divmod(blockIdx.x, q0, tb);
-  a.tilesA_fd.divmod(q0, bid, ta);
+  // along A fastest on a transposed [8192,8192] float input); the mirrored tile
+  // takes the mirrored order
+  if constexpr (WIDE_A) {
+    a.tilesA_fd.divmod(blockIdx.x, q0, ta);
+    a.tilesB_fd.divmod(q0, bid, tb);
+  } else {
+    a.tilesB_fd.divmod(blockIdx.x, q0, tb);
+    a.tilesA_fd.divmod(q0, bid, ta);
+  }
   int64_t off[kMaxOps] = {0, 0, 0, 0};
   for (int d = 0; d < a.n_outer; ++d) {
     uint32_t q, r;
@@ -498,9 +509,9 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
 #pragma unroll
     for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
   }
-  const uint32_t a0 = ta * kTileA, b0 = tb * TB;
-  if (a0 + kTileA <= a.sizeA && b0 + TB <= a.sizeB) tile_body<F, true, STREAM>(f, a, off, a0, b0, smem);
-  else tile_body<F, false, STREAM>(f, a, off, a0, b0, smem);
+  const uint32_t a0 = ta * TA, b0 = tb * TB;
+  if (a0 + TA <= a.sizeA && b0 + TB <= a.sizeB) tile_body<F, true, STREAM, WIDE_A>(f, a, off, a0, b0, smem);
+  else tile_body<F, false, STREAM, WIDE_A>(f, a, off, a0, b0, smem);
 }
 
 // ------------------------------------------------------------------ GENERAL
@@ -631,7 +642,7 @@ struct EwOperand {
 
 int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_args, int* main_vec,
                 VecArgs* tail_args, bool* has_tail);
-int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_b_edge, TileArgs* args, size_t* lds_bytes,
+int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int tile_b_edge, TileArgs* args, size_t* lds_bytes,
                  uint32_t* grid);
 int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use64, uint32_t* grid);
 
@@ -735,10 +746,24 @@ int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t 
     TileArgs ta;
     size_t lds = 0;
     uint32_t grid = 0;
-    if (int rc = prepare_tile(plan, ops, tile_b<F>::value, &ta, &lds, &grid)) return rc;
-    note_kernel("tile");
-    if (ta.streaming) hipLaunchKernelGGL((ew_tile_kernel<F, true>), dim3(grid), dim3(kBlock), lds, s, f, ta);
-    else hipLaunchKernelGGL((ew_tile_kernel<F, false>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+    // streams read or written along A (the destination among them) against those read along B
+    int along_a = 1, along_b = 0;
+    for (int k = 1; k < plan.n_ops; ++k) {
+      if (plan.via_lds[k]) ++along_b;
+      else if (ops[k].ptr && plan.canon.stride[k][0] != 0) ++along_a;
+    }
+    const bool wide_a = along_a > along_b;
+    if (int rc = prepare_tile(plan, ops, wide_a ? tile_shape<F, true>::ta : tile_shape<F, false>::ta,
+                              wide_a ? tile_shape<F, true>::tb : tile_shape<F, false>::tb, &ta, &lds, &grid))
+      return rc;
+    note_kernel(wide_a ? "tile_wide_a" : "tile");
+    if (wide_a) {
+      if (ta.streaming) hipLaunchKernelGGL((ew_tile_kernel<F, true, true>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+      else hipLaunchKernelGGL((ew_tile_kernel<F, false, true>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+    } else {
+      if (ta.streaming) hipLaunchKernelGGL((ew_tile_kernel<F, true, false>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+      else hipLaunchKernelGGL((ew_tile_kernel<F, false, false>), dim3(grid), dim3(kBlock), lds, s, f, ta);
+    }
     return after_launch(s);
   }
   GenArgs ga;

@@ -108,7 +108,8 @@ def pat_transposed_mixed(P, rng, code, n_in):
         ins.append(View(P.buf(values(rng, code, a * b)), [a, b]))
     if n_in >= 3:
         ins.append(View(P.buf(values(rng, code, b)), [b]))
-    return View(P.buf(np.zeros(a * b, NP[code])), [a, b]), ins, "tile"
+    # streams along the destination's rows in the majority: the mirrored tile
+    return View(P.buf(np.zeros(a * b, NP[code])), [a, b]), ins, "tile_wide_a" if n_in >= 2 else "tile"
 
 
 def pat_permuted_3d(P, rng, code, n_in):
