@@ -12,12 +12,14 @@
 //   e_i = T(exp(double(x_i) - double(m)))
 //   s   = T(sum of double(e_i))
 //   y_i = e_i / s                      (a division in T)
-// Three kernels cover the layouts:
+// Four kernels cover the layouts:
 //   softmax_wave_kernel   a group of 4, 16 or 64 lanes owns a row of up to 1024
 //                         vectors, kept in registers (128-bit accesses when the
 //                         rows are unit-stride and aligned)
 //   softmax_block_kernel  longer rows: one block per row, exponentials parked
 //                         in the output and scaled in a third pass
+//   softmax_short_rows_kernel  dense rows of up to 128 bytes that are no whole
+//                         number of vectors, staged through LDS
 //   softmax_lane_kernel   one lane owns a row (or four neighbouring rows, as
 //                         128-bit accesses) and walks k sequentially, the lanes
 //                         of a wave take neighbouring rows (coalesced when the
@@ -76,12 +78,14 @@ int act_grad_typed(hipStream_t s, void* ig, const ct_dims* igd, const void* og, 
 
 // ------------------------------------------------------------------ softmax
 
-// java.lang.Math.max on the tensor's own type.
+// The running maximum of a row.  java.lang.Math.max propagates NaN and ranks
+// +0 above -0; the sign of a zero maximum cannot reach the result (x - 0 has the
+// same exponential for either zero), so only the NaN rule is kept: half the
+// instructions of the full rule, in kernels whose arithmetic is close to the
+// memory time.
 template <class T> __device__ __forceinline__ T jvm_max(T a, T b) {
-  if (a != a) return a;
-  if (b != b) return b;
-  if (a == (T)0 && b == (T)0) return __builtin_signbit(a) ? b : a;
-  return a > b ? a : b;
+  const T r = a > b ? a : b;
+  return __builtin_isunordered(a, b) ? (T)__builtin_nan("") : r;
 }
 
 // T(exp(double(x) - double(m))).  For float, x - m is formed exactly as a float
@@ -292,6 +296,48 @@ __global__ void __launch_bounds__(kBlock) softmax_lane_kernel(const SoftmaxArgs 
   }
 }
 
+// Short rows stored back to back (a dense [rows, k] block) whose length is no
+// whole number of 16-byte vectors, e.g. ten classes.  A block stages its 256
+// rows, one contiguous stretch of memory, through LDS with 128-bit accesses;
+// one lane then owns one row in LDS.  (With one lane per element the same rows
+// move 4 bytes per lane and reach under a fifth of the memory rate.)
+template <class T>
+__global__ void __launch_bounds__(kBlock) softmax_short_rows_kernel(const SoftmaxArgs a) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  using V = Vec<T, VEC>;
+  extern __shared__ __align__(16) char smem[];
+  T* tile = reinterpret_cast<T*>(smem);
+  const uint32_t k = a.k;
+  const int64_t row0 = (int64_t)blockIdx.x * kBlock;
+  const uint32_t n_rows = (uint32_t)(a.n_rows - row0 < kBlock ? a.n_rows - row0 : kBlock);
+  const uint32_t count = n_rows * k;
+  const T* in = reinterpret_cast<const T*>(a.in) + row0 * k;
+  T* out = reinterpret_cast<T*>(a.out) + row0 * k;
+  // a block's stretch starts on the 16-byte grid whenever the tensor does (256 * k elements per block)
+  const uint32_t n_vec = count / VEC;
+  for (uint32_t v = threadIdx.x; v < n_vec; v += kBlock)
+    reinterpret_cast<V*>(tile)[v] = reinterpret_cast<const V*>(in)[v];
+  for (uint32_t e = n_vec * VEC + threadIdx.x; e < count; e += kBlock) tile[e] = in[e];
+  __syncthreads();
+  if (threadIdx.x < n_rows) {
+    T* row = tile + threadIdx.x * k;
+    T m = -__builtin_huge_valf();
+    for (uint32_t j = 0; j < k; ++j) m = jvm_max(m, row[j]);
+    double sum = 0.0;
+    for (uint32_t j = 0; j < k; ++j) {
+      const T e = shifted_exp(row[j], m);
+      row[j] = e;
+      sum += (double)e;
+    }
+    const T inv = (T)1 / (T)sum;
+    for (uint32_t j = 0; j < k; ++j) row[j] *= inv;
+  }
+  __syncthreads();
+  for (uint32_t v = threadIdx.x; v < n_vec; v += kBlock)
+    reinterpret_cast<V*>(out)[v] = reinterpret_cast<const V*>(tile)[v];
+  for (uint32_t e = n_vec * VEC + threadIdx.x; e < count; e += kBlock) out[e] = tile[e];
+}
+
 struct RowLayout { int64_t outer, rows, k, s_outer, s_row, s_k; };
 
 // [rows, k] or [outer, rows, k]; spatial swaps the last two axes (dimensions.clj:473-484 with [0 2 1]).
@@ -349,6 +395,15 @@ int softmax_run(hipStream_t s, void* out, const RowLayout& ol, const void* in, c
   };
   const bool vec_ok = aligned(in, il) && aligned(out, ol);
   const int64_t nv = vec_ok ? il.k / VMAX : il.k;
+  auto dense_rows = [](const void* p, const RowLayout& l) {
+    return l.s_k == 1 && l.s_row == l.k && (l.outer == 1 || l.s_outer == l.rows * l.k) && (uintptr_t)p % 16 == 0;
+  };
+  if (!vec_ok && il.k * (int64_t)sizeof(T) <= 128 && a.n_rows >= 4 * kBlock && dense_rows(in, il) && dense_rows(out, ol)) {
+    note_kernel("softmax_short_rows");
+    hipLaunchKernelGGL((softmax_short_rows_kernel<T>), dim3((uint32_t)((a.n_rows + kBlock - 1) / kBlock)), dim3(kBlock),
+                       (size_t)kBlock * il.k * sizeof(T), s, a);
+    return after_launch(s);
+  }
 #define CT_SM(VEC, TPR, ITER)                                                                                    \
   hipLaunchKernelGGL((softmax_wave_kernel<T, VEC, TPR, ITER>),                                                  \
                      dim3((uint32_t)((a.n_rows + (kBlock / TPR) - 1) / (kBlock / TPR))), dim3(kBlock), 0, s, a)
