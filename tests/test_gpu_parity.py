@@ -589,13 +589,17 @@ def test_softmax_layouts(P, code):
     x2, out2 = P.buf((rng.standard_normal(2 * c2 * 90) * 3).astype(NP[code])), P.buf(np.zeros(2 * c2 * 90, NP[code]))
     kern2 = P.run(H.softmax, View(out2, [2, c2, 90]), View(x2, [2, c2, 90]), True)
     compare(out2, f"softmax-spatial wide ({kern2})", tol=tol)
-    assert kern2 in ("softmax_lane_loop", "softmax_lane_loop_vec")
+    # parked in LDS while the rows of one wave fit 32 KiB, else the loop form
+    lds_fits = lambda ch: ch * 64 * x.init.itemsize <= 32768
+    assert kern2 == ("softmax_lane_lds" if lds_fits(c2) else "softmax_lane_loop_vec")
     got = out.download().reshape(b, c, e).astype(np.float64)
     assert np.allclose(got.sum(axis=1), 1.0, atol=1e-5)
     # position counts that allow 128-bit accesses across neighbouring positions
     for (b3, c3, e3), want_kernel in (((3, 21, 132), "softmax_lane_vec"), ((2, 5, 64), "softmax_lane_vec"),
                                      ((2, 13, 64), "softmax_lane_vec"), ((2, 30, 64), "softmax_lane_vec"),
-                                     ((2, 70, 96), "softmax_lane_loop_vec"), ((2, 70, 97), "softmax_lane_loop")):
+                                     ((2, 64, 96), "softmax_lane_lds"),
+                                     ((2, 70, 97), "softmax_lane_lds" if lds_fits(70) else "softmax_lane_loop"),
+                                     ((2, 300, 96), "softmax_lane_loop_vec"), ((2, 300, 97), "softmax_lane_loop")):
         n3 = b3 * c3 * e3
         x3, out3 = P.buf((rng.standard_normal(n3) * 3).astype(NP[code])), P.buf(np.zeros(n3, NP[code]))
         kern3 = P.run(H.softmax, View(out3, [b3, c3, e3]), View(x3, [b3, c3, e3]), True)
