@@ -24,6 +24,10 @@ SOURCES = [
     "ops_assign.hip",
     "ops_unary.hip",
     "ops_binary.hip",
+    "ops_binary_f32.hip",
+    "ops_binary_f64.hip",
+    "ops_binary_int_narrow.hip",
+    "ops_binary_int_wide.hip",
     "ops_ternary.hip",
     "ops_accum.hip",
     "ops_reduce.hip",
