@@ -1,8 +1,7 @@
-"""The BASELINE configurations at their full sizes on the GPU: compared with the
+"""The benchmark configurations at their full sizes on the GPU: compared with the
 CPU oracle where it finishes in seconds, and through size-independent
 properties (closed forms, a checksum of checksums, selection consistency).
-Inputs follow BASELINE.md: numpy default_rng(seed), generated in float64 and
-cast.  Needs a GPU.
+Inputs: numpy default_rng(seed), generated in float64 and cast.  Needs a GPU.
 """
 import ctypes as C
 
