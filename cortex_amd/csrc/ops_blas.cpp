@@ -11,12 +11,14 @@
 //
 // rocBLAS is loaded on first use (dlopen), so the library loads, and every
 // other entry point works, on a machine without it.  One handle per host thread
-// and device; atomics are switched off so results do not depend on scheduling.
+// and device, destroyed when the thread ends; atomics are switched off so results
+// do not depend on scheduling.
 #include <dlfcn.h>
 #include <rocblas/rocblas.h>
 
 #include <map>
 #include <mutex>
+#include <thread>
 
 #include "common.h"
 
@@ -78,14 +80,32 @@ RocblasApi* rocblas_api() {
       return set_error(CT_ERR_HIP, "%s failed: %s", #expr, (api)->status_to_string(st__));              \
   } while (0)
 
+// A host thread's handles, one per device, destroyed with the thread so that a
+// pool that retires threads does not pile up rocBLAS workspaces.  The thread
+// that loaded this library (normally the main one) keeps its handles until the
+// process ends: its thread-local destructors run inside exit(), where tearing
+// down a GPU library object is not worth the risk.
+const std::thread::id g_loader_thread = std::this_thread::get_id();
+
+struct HandleCache {
+  std::map<int, rocblas_handle> handles;
+  ~HandleCache() {
+    if (std::this_thread::get_id() == g_loader_thread) return;
+    RocblasApi* api = rocblas_api();
+    if (!api->ok) return;
+    for (auto& kv : handles)
+      if (kv.second) api->destroy_handle(kv.second);
+  }
+};
+
 // The calling thread's handle for the current device, bound to `s`.
 int blas_handle(hipStream_t s, RocblasApi** api_out, rocblas_handle* out) {
   RocblasApi* api = rocblas_api();
   if (!api->ok) return set_error(CT_ERR_UNSUPPORTED, "gemm!/gemv! need rocBLAS: %s", api->why);
   int dev = 0;
   CT_HIP(hipGetDevice(&dev));
-  thread_local std::map<int, rocblas_handle> handles;
-  rocblas_handle& h = handles[dev];
+  thread_local HandleCache cache;
+  rocblas_handle& h = cache.handles[dev];
   if (!h) {
     CT_BLAS(api, api->create_handle(&h));
     CT_BLAS(api, api->set_atomics_mode(h, rocblas_atomics_not_allowed));

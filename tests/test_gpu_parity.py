@@ -965,3 +965,48 @@ def test_threads_on_their_own_streams(P):
         bn_close(w["out"], f"thread {i} batch-normalized output", capi.F32)
         got, want = w["gemm"].download().astype(np.float64), w["gemm"].host.astype(np.float64)
         assert np.max(np.abs(got - want)) <= 1e-5 * (x64.reshape(r, c) ** 2).sum(axis=0).max()
+
+
+def test_thread_exit_releases_blas_handles(P):
+    """A host thread's rocBLAS handle (and the device workspace behind it) goes away with the
+    thread: a pool that retires threads must not shrink the free device memory thread by thread."""
+    import ctypes as C
+    import threading
+
+    rng = np.random.default_rng(101)
+    m = 64
+    a = P.buf(rng.standard_normal(m * m).astype(np.float32))
+    out = P.buf(np.zeros(m * m, np.float32))
+    errors = []
+
+    def worker():
+        try:
+            side = H.gpu_side()
+            s = C.c_void_p()
+            capi.call("ct_set_device", 0)
+            capi.call("ct_stream_create", C.byref(s))
+            side.stream = s
+            V = lambda b: View(b, [b.init.size])
+            H.gemm(side, V(out), m, False, False, 1.0, V(a), m, m, m, V(a), m, m, 0.0)
+            capi.call("ct_stream_sync", s)
+            capi.call("ct_stream_destroy", s)
+        except BaseException as exc:  # noqa: BLE001 -- reported in the main thread
+            errors.append(exc)
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        capi.call("ct_memory_info", C.byref(free), C.byref(total))
+        return free.value
+
+    def one_thread():
+        t = threading.Thread(target=worker)
+        t.start()
+        t.join()
+
+    one_thread()                      # whatever the first use of the library allocates for good
+    before = free_bytes()
+    for _ in range(12):
+        one_thread()
+    assert not errors, errors
+    lost = before - free_bytes()
+    assert lost < (8 << 20), f"{lost} bytes of device memory did not come back after 12 threads"
