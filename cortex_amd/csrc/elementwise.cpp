@@ -96,8 +96,8 @@ int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_
   return CT_OK;
 }
 
-int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int tile_b_edge, TileArgs* a, size_t* lds_bytes,
-                 uint32_t* grid) {
+int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int tile_b_edge, bool wide_a, TileArgs* a,
+                 size_t* lds_bytes, uint32_t* grid) {
   const Canon& c = plan.canon;
   const int b = plan.tile_b;
   std::memset(a, 0, sizeof(*a));
@@ -105,20 +105,30 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int ti
   a->sizeB = (uint32_t)c.size[b];
   a->tilesA = (a->sizeA + tile_a_edge - 1) / tile_a_edge;
   a->tilesB = (a->sizeB + tile_b_edge - 1) / tile_b_edge;
-  a->tilesA_fd = FastDiv(a->tilesA);
-  a->tilesB_fd = FastDiv(a->tilesB);
-  int64_t blocks = (int64_t)a->tilesA * a->tilesB;
+  // Super-tiles (see ew_tile_kernel): at most 64 x 2 tiles, 32 x 4 for the mirrored tile, evened
+  // out so that the last super-tile along an axis is as full as the others.
+  const uint32_t want_a = wide_a ? 32 : 64, want_b = wide_a ? 4 : 2;
+  const uint32_t nsa = (a->tilesA + want_a - 1) / want_a, nsb = (a->tilesB + want_b - 1) / want_b;
+  a->super_a = (a->tilesA + nsa - 1) / nsa;
+  a->super_b = (a->tilesB + nsb - 1) / nsb;
+  a->per_fd = FastDiv(a->super_a * a->super_b);
+  a->sb_fd = FastDiv(a->super_b);
+  a->nsb_fd = FastDiv(nsb);
+  a->nst_fd = FastDiv(nsa * nsb);
+  int64_t supers = (int64_t)nsa * nsb;
   int no = 0;
   for (int d = 1; d < c.nd; ++d) {
     if (d == b) continue;
     a->outer_fd[no] = FastDiv((uint32_t)c.size[d]);
     for (int k = 0; k < plan.n_ops; ++k) a->outer_stride[k][no] = c.stride[k][d];
-    blocks *= c.size[d];
+    supers *= c.size[d];
     ++no;
   }
   a->n_outer = no;
   a->streaming = is_streaming(plan, ops) ? 1u : 0u;
-  CT_REQUIRE(blocks < kLim31, "internal: tile grid too large");
+  const int64_t blocks = (supers + kXcds - 1) / kXcds * kXcds * (int64_t)(a->super_a * a->super_b);
+  CT_REQUIRE(supers < kLim31 && blocks < kLim31, "internal: tile grid too large");
+  a->n_super = (uint32_t)supers;
   *grid = (uint32_t)blocks;
   size_t lds = 0;
   for (int k = 0; k < plan.n_ops; ++k) {

@@ -869,6 +869,29 @@ def test_wide_rows_crossing_blocks(P, code):
         compare(d, f"binary-op! :* pitched {shape}")
 
 
+@pytest.mark.parametrize("code", [capi.F32, capi.F64, capi.I8])
+def test_tile_super_tiles(P, code):
+    """Transposed views large enough for several super-tiles of the tile kernel's block order,
+    with tile counts that do not divide into them and an outer axis on top."""
+    rng = np.random.default_rng(91)
+    f = NP[code]
+    for outer, a, b in ((1, 2100, 300), (3, 2100, 140), (2, 90, 2200)):
+        n = outer * a * b
+        x, y, z = (P.buf(values(rng, code, n)) for _ in range(3))
+        d = P.buf(np.zeros(n, f))
+        dest = View(d, [outer, a, b])
+        tr = lambda buf: View(buf, [outer, b, a]).transpose([0, 2, 1])
+        k = P.run(H.ternary_op, dest, tr(x), 1.0, tr(y), 1.0, tr(z), 1.0)
+        assert k == "tile"
+        compare(d, f"select, three transposed {(outer, a, b)}")
+        k = P.run(H.binary_op, dest, tr(x), 1.0, View(y, [outer, a, b]), 1.0, "+")
+        assert k == "tile_wide_a"
+        compare(d, f"x^T + y {(outer, a, b)}")
+        k = P.run(H.unary_op, dest, tr(x), 1.0, "-")
+        assert k == "tile"
+        compare(d, f"negated transpose {(outer, a, b)}")
+
+
 def test_flat_call_longer_than_one_launch():
     """A flat call of more than 2^30 vectors (16 GiB of bytes) is walked in pieces."""
     import ctypes as C
