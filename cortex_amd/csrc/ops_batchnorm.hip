@@ -574,6 +574,7 @@ __global__ void __launch_bounds__(kBlock) bn_constants_kernel(const BnArgs a) {
 // and a lane only picks its row's set.
 struct BnRowArgs {
   uint64_t total_vecs;
+  uint32_t grouped_blocks;  // see xcd_grouped_unit
   FastDiv nv_fd, c_fd;   // vectors per row; channels
   const double* params;
   const void* x;
@@ -588,12 +589,13 @@ __global__ void __launch_bounds__(kBlock) bn_apply_rows_kernel(const BnRowArgs a
   const uint64_t total = a.total_vecs;
   const FastDiv nfd = a.nv_fd, cfd = a.c_fd;
   const double* const params = a.params;
+  const uint32_t grouped = a.grouped_blocks;
   const V* const x = reinterpret_cast<const V*>(a.x);
   const V* const og = reinterpret_cast<const V*>(MODE == kBnGradient ? a.og : a.x);
   V* const out = reinterpret_cast<V*>(a.out);
   asm volatile("" ::"s"(total), "s"(nfd.d), "s"(nfd.m), "s"(nfd.s), "s"(cfd.d), "s"(cfd.m), "s"(cfd.s), "s"(params),
-               "s"(x), "s"(og), "s"(out));
-  const uint64_t v_first = (uint64_t)blockIdx.x * (uint64_t)kBlock;
+               "s"(grouped), "s"(x), "s"(og), "s"(out));
+  const uint64_t v_first = (uint64_t)xcd_grouped_unit(blockIdx.x, grouped) * (uint64_t)kBlock;
   const uint64_t v = v_first + threadIdx.x;
   if (v >= total) return;
   V xv, gv;
@@ -826,6 +828,7 @@ void bn_launch_apply(hipStream_t s, const BnPlan& plan) {
     r.params = a.params;
     r.x = a.x; r.og = a.og; r.out = a.out;
     const dim3 grid((uint32_t)((r.total_vecs + kBlock - 1) / kBlock));
+    r.grouped_blocks = xcd_grouped_blocks(grid.x);
     const double bytes = (double)a.N * sizeof(T) * (MODE == kBnGradient ? 3 : 2);
     const int level = bytes >= (double)(int64_t(1) << 30) ? 2 : bytes >= (double)kStreamingBytes ? 1 : 0;
     if (ragged) {

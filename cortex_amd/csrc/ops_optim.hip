@@ -26,9 +26,9 @@ struct AdamScalars {
 
 template <class T, int VEC, int UNROLL, bool streaming>
 __global__ void __launch_bounds__(kBlock) adam_kernel(const AdamScalars s, const T* g, T* p, T* m, T* v,
-                                                      int64_t n_vecs) {
+                                                      int64_t n_vecs, uint32_t grouped_blocks) {
   using V = Vec<T, VEC>;
-  const int64_t first = (int64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x;
+  const int64_t first = (int64_t)xcd_grouped_unit(blockIdx.x, grouped_blocks) * (kBlock * UNROLL) + threadIdx.x;
   V gv[UNROLL], pv[UNROLL], mv[UNROLL], vv[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
@@ -70,9 +70,9 @@ template <class T> struct AdadeltaScalars { T ga; double decay, eps, one_minus_d
 
 template <class T, int VEC, int UNROLL, bool streaming>
 __global__ void __launch_bounds__(kBlock) adadelta_kernel(const AdadeltaScalars<T> s, const T* g, T* p, T* gacc,
-                                                          T* dacc, int64_t n_vecs) {
+                                                          T* dacc, int64_t n_vecs, uint32_t grouped_blocks) {
   using V = Vec<T, VEC>;
-  const int64_t first = (int64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x;
+  const int64_t first = (int64_t)xcd_grouped_unit(blockIdx.x, grouped_blocks) * (kBlock * UNROLL) + threadIdx.x;
   V gv[UNROLL], pv[UNROLL], av[UNROLL], dv[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
@@ -133,13 +133,13 @@ void adam_launch(hipStream_t st, const AdamScalars& s, const T* g, T* p, T* m, T
   if (n_vecs > 0) {
     const int64_t per = (int64_t)kBlock * kUnroll;
     const dim3 grid((uint32_t)((n_vecs + per - 1) / per));
-    if (streaming) hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, true>), grid, dim3(kBlock), 0, st, s, g, p, m, v, n_vecs);
-    else hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, false>), grid, dim3(kBlock), 0, st, s, g, p, m, v, n_vecs);
+    if (streaming) hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, true>), grid, dim3(kBlock), 0, st, s, g, p, m, v, n_vecs, xcd_grouped_blocks(grid.x));
+    else hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, false>), grid, dim3(kBlock), 0, st, s, g, p, m, v, n_vecs, xcd_grouped_blocks(grid.x));
   }
   const int64_t done = n_vecs * VEC;
   if (VEC > 1 && done < n)
     hipLaunchKernelGGL((adam_kernel<T, 1, 1, false>), dim3(1), dim3(kBlock), 0, st, s, g + done, p + done, m + done,
-                       v + done, n - done);
+                       v + done, n - done, 0u);
 }
 
 template <class T>
@@ -173,13 +173,13 @@ void adadelta_launch(hipStream_t st, const AdadeltaScalars<T>& s, const T* g, T*
   if (n_vecs > 0) {
     const int64_t per = (int64_t)kBlock * kUnroll;
     const dim3 grid((uint32_t)((n_vecs + per - 1) / per));
-    if (streaming) hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, true>), grid, dim3(kBlock), 0, st, s, g, p, a, d, n_vecs);
-    else hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, false>), grid, dim3(kBlock), 0, st, s, g, p, a, d, n_vecs);
+    if (streaming) hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, true>), grid, dim3(kBlock), 0, st, s, g, p, a, d, n_vecs, xcd_grouped_blocks(grid.x));
+    else hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, false>), grid, dim3(kBlock), 0, st, s, g, p, a, d, n_vecs, xcd_grouped_blocks(grid.x));
   }
   const int64_t done = n_vecs * VEC;
   if (VEC > 1 && done < n)
     hipLaunchKernelGGL((adadelta_kernel<T, 1, 1, false>), dim3(1), dim3(kBlock), 0, st, s, g + done, p + done, a + done,
-                       d + done, n - done);
+                       d + done, n - done, 0u);
 }
 
 template <class T>
