@@ -174,7 +174,9 @@ struct FastDiv {
 // optimizers' four reads and three writes in place +2 to +6; the library's own
 // flat kernels, same range of sizes: copy +0.5 to +4, x + y +1 to +6.5, a
 // three-input select -1 to +4.  Groups of 4 to 64 pieces gain as much at
-// 256 MiB but lose up to 10 points at 1 GiB.
+// 256 MiB but lose up to 10 points at 1 GiB.  The reductions, softmax and rand!
+// kernels gained nothing from the same regrouping (the double row reduction and
+// rand! lost 5 points) and keep the plain order.
 constexpr uint32_t kXcds = 8;
 constexpr uint32_t kXcdGroup = 128;
 

@@ -165,7 +165,10 @@ def softmax_channels(driver, datatype):
 
 # verify/nn/layers.clj:640-672
 def dropout_bernoulli(driver, datatype):
-    with context(driver, datatype):
+    with context(driver, datatype) as stream:
+        # the reference's bounds are about three standard deviations of the averaged sums: with
+        # the operating system's seed the test would fail once in several hundred runs
+        stream.seed_random(20)
         batch_size, item_count, repeat_count = 5, 20, 30
         n = batch_size * item_count
         node = {"type": "dropout", "distribution": "bernoulli", "probability": 0.8, "input-size": item_count}
@@ -192,7 +195,8 @@ def dropout_bernoulli(driver, datatype):
 
 # verify/nn/layers.clj:675-702
 def dropout_gaussian(driver, datatype):
-    with context(driver, datatype):
+    with context(driver, datatype) as stream:
+        stream.seed_random(21)
         batch_size, item_count, repeat_count = 5, 100, 30
         n = batch_size * item_count
         node = {"type": "dropout", "distribution": "gaussian", "variance": 0.5, "input-size": item_count}
