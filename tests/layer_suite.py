@@ -247,6 +247,71 @@ def batch_normalization(driver, datatype):
                30 * tol)
 
 
+# verify/nn/layers.clj:705-763 as the reference runs it: six batches whose every feature has mean 5
+# and (population) variance 20 exactly (src/cortex/gaussian.clj:34-47), average factor 0.8; every
+# output batch is normalized, and the running statistics settle on 5 and the sample variance
+# 20 * 20 / 19 = 21.05
+def batch_normalization_running(driver, datatype):
+    with context(driver, datatype):
+        batch_size, input_size = 20, 20
+        rng = np.random.default_rng(6)
+
+        def batch():
+            x = rng.standard_normal((batch_size, input_size))
+            x = (x - x.mean(axis=0)) / x.std(axis=0) * np.sqrt(20.0) + 5.0
+            return x
+
+        node = {"type": "batch-normalization", "mode": "elementwise", "input-size": input_size,
+                "epsilon": 1e-4, "average-factor": 0.8}
+        layer = nl.create(node, batch_size)
+        params = {"scale": entry(np.ones(input_size)), "bias": entry(np.zeros(input_size)),
+                  "means": entry(np.zeros(input_size), with_gradient=False),
+                  "variances": entry(np.zeros(input_size), with_gradient=False)}
+        outputs = [{"buffer": ct.new_tensor([batch_size, input_size]),
+                    "gradient": ct.new_tensor([batch_size, input_size])}]
+        for _ in range(6):
+            inputs = [entry(batch())]
+            forward_backward(layer, params, inputs, outputs, [np.ones((batch_size, input_size))])
+            out = ct.to_double_array(outputs[0]["buffer"]).reshape(batch_size, input_size)
+            about_there(out.mean(axis=0), np.zeros(input_size), 1e-6 if datatype == "double" else 1e-4)
+            about_there(out.var(axis=0), np.ones(input_size), 1e-3)
+        about_there([ct.to_double_array(params["means"]["buffer"]).mean()], [5.0],
+                    1e-6 if datatype == "double" else 1e-4)
+        about_there([ct.to_double_array(params["variances"]["buffer"]).mean()], [21.05], 1e-2)
+
+
+# the spatial mode of the same layer: one statistic per channel over batch and pixels
+def batch_normalization_spatial(driver, datatype):
+    with context(driver, datatype):
+        batch_size, channels, height, width = 6, 5, 4, 7
+        rng = np.random.default_rng(7)
+        x = rng.standard_normal((batch_size, channels, height * width)) * np.arange(1, channels + 1)[None, :, None] + 3
+        node = {"type": "batch-normalization", "mode": "spatial", "epsilon": 1e-4, "average-factor": 0.9,
+                "input-dimension": {"channels": channels, "height": height, "width": width}}
+        layer = nl.create(node, batch_size)
+        scale, bias = rng.uniform(0.5, 2.0, channels), rng.standard_normal(channels)
+        params = {"scale": entry(scale), "bias": entry(bias),
+                  "means": entry(np.zeros(channels), with_gradient=False),
+                  "variances": entry(np.zeros(channels), with_gradient=False)}
+        inputs = [entry(x)]
+        outputs = [{"buffer": ct.new_tensor(list(x.shape)), "gradient": ct.new_tensor(list(x.shape))}]
+        og = rng.standard_normal(x.shape)
+        forward_backward(layer, params, inputs, outputs, [og])
+        mean, var = x.mean(axis=(0, 2)), x.var(axis=(0, 2))
+        x_hat = (x - mean[None, :, None]) / np.sqrt(var + 1e-4)[None, :, None]
+        tol = 1e-10 if datatype == "double" else 3e-5
+        equals(x_hat * scale[None, :, None] + bias[None, :, None], ct.to_double_array(outputs[0]["buffer"]), tol * 10)
+        equals(og.sum(axis=(0, 2)), ct.to_double_array(params["bias"]["gradient"]), tol * 100)
+        equals((og * x_hat).sum(axis=(0, 2)), ct.to_double_array(params["scale"]["gradient"]), tol * 100)
+        n = batch_size * height * width
+        equals(var * n / (n - 1), ct.to_double_array(params["variances"]["buffer"]), tol * 100)
+        # inference reproduces the training output once the running statistics equal the batch's
+        ct.assign(params["variances"]["buffer"], ct.to_tensor(var))
+        infer_out = [{"buffer": ct.new_tensor(list(x.shape))}]
+        layer.infer(params, inputs, infer_out)
+        equals(ct.to_double_array(outputs[0]["buffer"]), ct.to_double_array(infer_out[0]["buffer"]), tol * 10)
+
+
 # verify/nn/layers.clj:813-835
 def prelu(driver, datatype):
     with context(driver, datatype):

@@ -16,7 +16,8 @@ FLOAT_TESTS = ["gemm", "gemv", "activation_forward", "activation_gradient", "sof
 
 # tests/layer_suite.py: the layers, loss gradients and regularisers built on the tensor calls
 LAYER_TESTS = ["relu_activation", "linear", "activations", "activations_batch", "softmax", "softmax_channels",
-               "dropout_bernoulli", "dropout_gaussian", "batch_normalization", "prelu",
+               "dropout_bernoulli", "dropout_gaussian", "batch_normalization", "batch_normalization_running",
+               "batch_normalization_spatial", "prelu",
                "concatenate", "split", "join_add", "join_add_ragged", "join_multiply", "loss_gradients",
                "train_small_network"]
 
