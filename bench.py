@@ -195,7 +195,7 @@ def run_extras(drv, device, stream, timer, capi) -> dict:
 
 def run_adjacent(drv, device, stream, timer, capi) -> dict:
     """The adjacent TensorMath methods built on the same machinery (activation-gradient!,
-    softmax!, batch normalization, rand!, gemm!), timed like the BASELINE configs.  Bytes
+    softmax!, batch normalization, rand!, gemv!, gemm!), timed like the BASELINE configs.  Bytes
     are algorithmic: every operand read once, every result written once, although the
     batch-normalization forms that need batch statistics read their operands twice."""
     out = {}
@@ -242,6 +242,12 @@ def run_adjacent(drv, device, stream, timer, capi) -> dict:
     a_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))
     b_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))
     c_ = device.allocate_device_buffer(m * m, "float")
+    # gemv! reads the matrix once: HBM-bound like the rest
+    xv = upload(drv, device, stream, rng.standard_normal(m, dtype=np.float32))
+    yv = device.allocate_device_buffer(m, "float")
+    for trans, label in ((False, "A x"), (True, "A^T x")):
+        ms = time_launches(timer, stream, lambda: stream.gemv(yv, 1, trans, 1.0, a_, m, m, m, xv, 1, 0.0), 20)
+        out[f"gemv! f32 [{m},{m}] {label}"] = entry(4 * m * m, ms)
     ms = time_launches(timer, stream, lambda: stream.gemm(c_, m, False, False, 1.0, a_, m, m, m, b_, m, m, 0.0), 5, warm=2)
     tflops = 2.0 * m ** 3 / (ms * 1e-3) / 1e12
     out[f"gemm! f32 [{m},{m}]x[{m},{m}] (rocBLAS)"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tflops, 1),

@@ -1,13 +1,14 @@
-// ops_blas.cpp -- gemm! and gemv! (src/cortex/tensor/math.clj:106-123) on
-// rocBLAS.  These are plain library matrix products (the reference's backends
-// call netlib BLAS and cuBLAS for them, src/cortex/compute/cpu/tensor_math.clj:672-726,
+// ops_blas.cpp -- gemm! (src/cortex/tensor/math.clj:106-114) on rocBLAS.  It is
+// a plain library matrix product (the reference's backends call netlib BLAS and
+// cuBLAS for it, src/cortex/compute/cpu/tensor_math.clj:672-726,
 // src/cortex/compute/cuda/tensor_math.clj:633-660), so the vendor library's MFMA
-// kernels are the right tool; nothing is hand-written here.
+// kernels are the right tool; nothing is hand-written here.  gemv!, which is
+// bound by memory rather than by the matrix cores, lives in ops_gemv.hip.
 //
 // The tensors are row-major and BLAS is column-major: a row-major matrix with
 // row pitch ld is the column-major matrix of its transpose with leading
 // dimension ld, and C^T = op(B)^T op(A)^T, which is the operand swap of
-// col->row-gemm / col->row-gemv (src/cortex/compute/math_util.clj:17-41).
+// col->row-gemm (src/cortex/compute/math_util.clj:17-31).
 //
 // rocBLAS is loaded on first use (dlopen), so the library loads, and every
 // other entry point works, on a machine without it.  One handle per host thread
@@ -34,8 +35,6 @@ struct RocblasApi {
   decltype(&rocblas_set_pointer_mode) set_pointer_mode = nullptr;
   decltype(&rocblas_sgemm) sgemm = nullptr;
   decltype(&rocblas_dgemm) dgemm = nullptr;
-  decltype(&rocblas_sgemv) sgemv = nullptr;
-  decltype(&rocblas_dgemv) dgemv = nullptr;
   decltype(&rocblas_status_to_string) status_to_string = nullptr;
   bool ok = false;
   char why[256] = "";
@@ -64,8 +63,6 @@ RocblasApi* rocblas_api() {
     CT_SYM(set_pointer_mode, rocblas_set_pointer_mode)
     CT_SYM(sgemm, rocblas_sgemm)
     CT_SYM(dgemm, rocblas_dgemm)
-    CT_SYM(sgemv, rocblas_sgemv)
-    CT_SYM(dgemv, rocblas_dgemv)
     CT_SYM(status_to_string, rocblas_status_to_string)
 #undef CT_SYM
     api.ok = true;
@@ -101,7 +98,7 @@ struct HandleCache {
 // The calling thread's handle for the current device, bound to `s`.
 int blas_handle(hipStream_t s, RocblasApi** api_out, rocblas_handle* out) {
   RocblasApi* api = rocblas_api();
-  if (!api->ok) return set_error(CT_ERR_UNSUPPORTED, "gemm!/gemv! need rocBLAS: %s", api->why);
+  if (!api->ok) return set_error(CT_ERR_UNSUPPORTED, "gemm! needs rocBLAS: %s", api->why);
   int dev = 0;
   CT_HIP(hipGetDevice(&dev));
   thread_local HandleCache cache;
@@ -152,34 +149,6 @@ int ct_gemm(void* stream, void* c, int64_t c_colstride, int trans_a, int trans_b
     CT_BLAS(api, api->dgemm(h, op_of(trans_b), op_of(trans_a), m, n, k, &alpha, (const double*)b,
                             (rocblas_int)b_colstride, (const double*)a, (rocblas_int)a_colstride, &beta, (double*)c,
                             (rocblas_int)c_colstride));
-  }
-  return after_launch(s);
-}
-
-int ct_gemv(void* stream, void* c, int64_t inc_c, int trans_a, double alpha, const void* a, int64_t a_row_count,
-            int64_t a_col_count, int64_t a_colstride, const void* x, int64_t inc_x, double beta, int dtype) {
-  CT_REQUIRE(dtype == CT_F32 || dtype == CT_F64, "gemv! is only defined for float and double tensors");
-  CT_REQUIRE(a && x && c, "ct_gemv: null buffer");
-  CT_REQUIRE(fits_int(a_row_count) && fits_int(a_col_count) && fits_int(a_colstride) && fits_int(inc_x) &&
-                 fits_int(inc_c) && inc_x >= 1 && inc_c >= 1,
-             "ct_gemv: a size or increment is out of range");
-  CT_REQUIRE(a_colstride >= a_col_count, "ct_gemv: A column stride is shorter than its rows");
-  if (a_row_count == 0 || a_col_count == 0) return CT_OK;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  RocblasApi* api;
-  rocblas_handle h;
-  if (int rc = blas_handle(s, &api, &h)) return rc;
-  note_kernel("rocblas_gemv");
-  // the row-major [rows, cols] matrix is the column-major [cols, rows] one: flip the transposition
-  const rocblas_operation op = op_of(!trans_a);
-  const rocblas_int m = (rocblas_int)a_col_count, n = (rocblas_int)a_row_count;
-  if (dtype == CT_F32) {
-    const float al = (float)alpha, be = (float)beta;
-    CT_BLAS(api, api->sgemv(h, op, m, n, &al, (const float*)a, (rocblas_int)a_colstride, (const float*)x,
-                            (rocblas_int)inc_x, &be, (float*)c, (rocblas_int)inc_c));
-  } else {
-    CT_BLAS(api, api->dgemv(h, op, m, n, &alpha, (const double*)a, (rocblas_int)a_colstride, (const double*)x,
-                            (rocblas_int)inc_x, &beta, (double*)c, (rocblas_int)inc_c));
   }
   return after_launch(s);
 }

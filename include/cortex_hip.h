@@ -282,7 +282,8 @@ int ct_gemm(void* stream, void* c, int64_t c_colstride, int trans_a, int trans_b
  * compute/math_util.clj:33-41): c = alpha * op(A) * x + beta * c for the stored
  * row-major matrix A [a_row_count, a_col_count] (counts before the
  * transposition, src/cortex/tensor.clj:975-989) and vector increments in
- * elements. */
+ * elements.  The library's own kernels (the product is bound by memory, not by
+ * the matrix cores); the sums run in double.  dtype is CT_F32 or CT_F64. */
 int ct_gemv(void* stream, void* c, int64_t inc_c, int trans_a, double alpha, const void* a,
             int64_t a_row_count, int64_t a_col_count, int64_t a_colstride, const void* x,
             int64_t inc_x, double beta, int dtype);

@@ -781,7 +781,7 @@ def test_rand_errors(P):
         H.rand(P.hip, View(y, [8]), 8, "flat", 1, 1, 1, 0)
 
 
-# ------------------------------------------------------------------ gemm!, gemv! (rocBLAS)
+# ------------------------------------------------------------------ gemm! (rocBLAS), gemv!
 # The vendor library sums in the tensor's own precision and in its own order; the oracle keeps a
 # double accumulator.  Bar: |got - want| <= tol * (|alpha| sum |a||b| + |beta c|) with
 # tol = 1e-5 for float (k up to 512 terms of 2^-24 relative error each) and 1e-13 for double.
@@ -816,23 +816,38 @@ def test_gemm(P, code, ta, tb, case):
         bc.reset()
 
 
+# gemv! is the library's own pair of reductions with double accumulators: it differs from the
+# oracle only in the order of the double additions, so the bar is the reductions' (2e-6 / 1e-12
+# of the sum of magnitudes), and what lies between the strided elements of y must stay untouched.
+GEMV_CASES = [(6, 5, 8, 3, 2), (300, 257, 257, 1, 1), (64, 1000, 1024, 1, 5), (2000, 64, 64, 1, 1), (3, 5000, 5000, 1, 1),
+              (1500, 260, 264, 2, 1), (700, 1028, 1028, 1, 1), (1, 1, 1, 1, 1), (129, 12, 12, 1, 3)]
+
+
 @pytest.mark.parametrize("code", FLOATS)
 @pytest.mark.parametrize("ta", [False, True])
 def test_gemv(P, code, ta):
     rng = np.random.default_rng(71)
     f = NP[code]
-    for rows, cols, lda, incx, incy in ((6, 5, 8, 3, 2), (300, 257, 257, 1, 1), (64, 1000, 1024, 1, 5)):
+    for rows, cols, lda, incx, incy in GEMV_CASES:
         n_in, n_out = (rows, cols) if ta else (cols, rows)
         a, x, y = (rng.standard_normal(s).astype(f) for s in ((rows, lda), n_in * incx, n_out * incy))
         ba, bx, by = P.buf(a), P.buf(x), P.buf(y)
         va, vx, vy = (View(bf, [bf.init.size]) for bf in (ba, bx, by))
-        P.run(H.gemv, vy, incy, ta, 2.0, va, rows, cols, lda, vx, incx, 0.25)
+        k = P.run(H.gemv, vy, incy, ta, 2.0, va, rows, cols, lda, vx, incx, 0.25)
+        assert k.startswith("gemv_cols" if ta else "gemv_rows"), k
         A = np.abs(a[:, :cols].astype(np.float64))
         bound = np.zeros(n_out * incy)
         bound[::incy] = 2.0 * ((A.T if ta else A) @ np.abs(x[::incx].astype(np.float64))) + 0.25 * np.abs(y[::incy])
-        tol = 1e-5 if code == capi.F32 else 1e-13
+        tol = 2e-6 if code == capi.F32 else 1e-12
         got, want = by.download().astype(np.float64), by.host.astype(np.float64)
         assert np.all(np.abs(got - want) <= tol * bound), f"gemv {(rows, cols)} ta={ta}: {np.max(np.abs(got - want))}"
+        # beta = 0 overwrites whatever y held, NaN included
+        by.init[::incy] = np.nan
+        by.reset()
+        P.run(H.gemv, vy, incy, ta, 1.0, va, rows, cols, lda, vx, incx, 0.0)
+        got, want = by.download().astype(np.float64), by.host.astype(np.float64)
+        assert not np.isnan(got[::incy]).any()
+        assert np.all(np.abs(got - want) <= tol * bound), f"gemv beta 0 {(rows, cols)} ta={ta}"
 
 
 def test_gemm_errors(P):
