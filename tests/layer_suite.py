@@ -14,7 +14,7 @@ import numpy as np
 
 from cortex_amd import nn_layers as nl
 from cortex_amd import tensor as ct
-from reference_suite import context, equals
+from reference_suite import GOLDEN, context, equals
 
 
 def about_there(actual, expected, eps=1e-6):
@@ -83,41 +83,9 @@ def linear(driver, datatype):
             equals([7, 10] * batch_size, ct.to_double_array(inputs[0]["gradient"]))
 
 
-# verify/nn/layers.clj:283-314
-ACTIVATION_ANSWERS = {
-    "logistic": ([0.2689414213699951, 0.7310585786300049], [-0.19661193324148185, 0.19661193324148185]),
-    "swish": ([-0.2689414213699951, 0.7310585786300049], [-0.36713290505919505, 0.835403899885462]),
-    "tanh": ([-0.7615941559557649, 0.7615941559557649], [-0.41997434161402614, 0.41997434161402614]),
-    "selu": ([-1.1113307378125625, 1.0507009873554805], [-0.5786268790075374, 1.0507009873554805]),
-}
-
-# verify/nn/layers.clj:332-381
-ACTIVATION_BATCH_ANSWERS = {
-    "logistic": ([0.0066928509242848554, 0.01798620996209156, 0.04742587317756678, 0.11920292202211755,
-                  0.2689414213699951, 0.5, 0.7310585786300049, 0.8807970779778823, 0.9525741268224334,
-                  0.9820137900379085],
-                 [-0.033240283353950774, -0.07065082485316447, -0.1355299791927364, -0.209987170807013,
-                  -0.19661193324148185, 0.0, 0.19661193324148185, 0.20998717080701323, 0.135529979192736,
-                  0.07065082485316443]),
-    "tanh": ([-0.9999092042625951, -0.999329299739067, -0.9950547536867305, -0.9640275800758169,
-              -0.7615941559557649, 0.0, 0.7615941559557649, 0.9640275800758169, 0.9950547536867305,
-              0.999329299739067],
-             [-9.079161547192634E-4, -0.005363802732103666, -0.0295981114963205, -0.14130164970632886,
-              -0.41997434161402614, 0.0, 0.41997434161402614, 0.14130164970632886, 0.0295981114963205,
-              0.005363802732103666]),
-    "swish": ([-0.03346425462142428, -0.07194483984836623, -0.14227761953270035, -0.2384058440442351,
-               -0.2689414213699951, 0.0, 0.7310585786300049, 1.7615941559557646, 2.8577223804673,
-               3.928055160151634],
-              [-2.416354975472916, -1.856234354263459, -1.2873014189882364, -0.7638334409883287,
-               -0.36713290505919505, 0.0, 0.835403899885462, 2.1475760812469877, 3.277268515997532,
-               4.220215568779826]),
-    "selu": ([-1.74625336066962, -1.7258986281898945, -1.6705687287671118, -1.520166468595695,
-              -1.1113307378125625, 0.0, 1.0507009873554805, 2.101401974710961, 3.1521029620664414,
-              4.202803949421922],
-             [-1.5332932256617793, -1.2518582388020294, -0.9923066122192254, -0.768906439142725,
-              -0.5786268790075374, 0.0, 1.0507009873554805, 2.101401974710961, 3.1521029620664414,
-              4.202803949421922]),
-}
+# verify/nn/layers.clj:283-314 and :332-381: (forward, backward) per activation
+ACTIVATION_ANSWERS = {k: tuple(v) for k, v in GOLDEN["activation_answers"]["values"].items()}
+ACTIVATION_BATCH_ANSWERS = {k: tuple(v) for k, v in GOLDEN["activation_batch_answers"]["values"].items()}
 
 
 # verify/nn/layers.clj:316-326: a float32 backend cannot hold the reference's 1e-6 on a sum of ten

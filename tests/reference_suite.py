@@ -8,13 +8,18 @@ HIP driver.  Expected values are the reference's own.
 """
 from __future__ import annotations
 
+import json
 import math
+import pathlib
 
 import numpy as np
 
 from cortex_amd import dimensions as ct_dims
 from cortex_amd import tensor as ct
 from cortex_amd.dimensions import ALL
+
+# the longer expected vectors of the reference's tests, kept as data (tests/golden/README.md)
+GOLDEN = json.loads((pathlib.Path(__file__).resolve().parent / "golden" / "reference_vectors.json").read_text())
 
 ALL_DTYPES = ["double", "float", "long", "int", "short", "byte"]   # def-all-dtype-test
 FLOAT_DTYPES = ["double", "float"]                                  # def-double-float-test
@@ -286,16 +291,10 @@ def gemv(driver, datatype):
         equals([144.0, 166.0, 188.0], ct.to_double_array(tens_c_sub))
 
 
-BN_ELTWISE_OUT = [-26.0, 4.0, 6.116036847575795, 64.0, 12.955334711889902, 12.46414739030318, 154.0,
-                  21.910669423779805, 18.812257933030565, 244.0, 30.86600413566971, 25.16036847575795]
-BN_SPATIAL_OUT = [-26.0, 4.0, 34.0, 64.0, 12.955334711889902, 15.94044628251987, 18.925557853149837,
-                  21.910669423779805, 18.812257933030565, 20.92829478060636, 23.044331628182157, 25.16036847575795,
-                  334.0, 364.0, 394.0, 424.0, 48.77667355944951, 51.76178513007948, 54.74689670070945,
-                  57.73200827133942, 44.204700103940105, 46.3207369515159, 48.436773799091696, 50.55281064666749]
-BN_UPDATE_ELTWISE_OUT = [-0.023134696804511745] * 3 + [2.6589551010651626] * 3 + [5.341044898934837] * 3 + \
-                        [8.023134696804512] * 3
-BN_UPDATE_SPATIAL_OUT = [0.3139510961275713, 0.8054242833105618, 1.2968974704935523, 1.7883706576765428] * 3 + \
-                        [6.211629342323457, 6.703102529506448, 7.194575716689438, 7.686048903872429] * 3
+BN_ELTWISE_OUT = GOLDEN["batch_normalize_eltwise"]["values"]
+BN_SPATIAL_OUT = GOLDEN["batch_normalize_spatial"]["values"]
+BN_UPDATE_ELTWISE_OUT = GOLDEN["batch_normalize_update_eltwise"]["values"]
+BN_UPDATE_SPATIAL_OUT = GOLDEN["batch_normalize_update_spatial"]["values"]
 
 
 def _spatial_input():
@@ -628,27 +627,7 @@ def simple_stream(driver, datatype):
 
 
 # compute/verify/optimize.clj:11-61
-ADAM_ANSWERS = [
-    [0.999000000005, 1.9990000000025, 2.9990000000016668, 3.99900000000125],
-    [0.9980000262138343, 1.9980000130723587, 2.998000008707231, 3.998000006527546],
-    [0.9970000960651408, 1.9970000478972731, 2.9970000319014805, 3.9970000239148513],
-    [0.9960002269257634, 1.9960001131228113, 2.9960000753397424, 3.9960000564765217],
-    [0.995000436052392, 1.9950002173334274, 2.995000144735273, 3.995000108493863],
-    [0.9940007405541528, 1.9940003690339771, 2.994000245746984, 3.9940001842069432],
-    [0.9930011573564278, 1.9930005766318695, 2.9930003839675967, 3.993000287805732],
-    [0.9920017031661642, 1.9920008484199827, 2.992000564912314, 3.992000423421624],
-    [0.9910023944389119, 1.991001192560463, 2.9910007940080785, 3.9910005951194076],
-    [0.9900032473478027, 1.9900016170695067, 2.9900010765834972, 3.990000806889731],
-    [0.9890042777546556, 1.9890021298032192, 2.9890014178594777, 3.9890010626421075],
-    [0.9880055011833645, 1.9880027384446224, 2.9880018229406398, 3.988001366198499],
-    [0.9870069327956914, 1.987003450491873, 2.98700229680753, 3.9870017212875037],
-    [0.9860085873695607, 1.986004273247733, 2.9860028443096756, 3.9860021315391725],
-    [0.9850104792799151, 1.9850052138103236, 2.9850034701594894, 3.9850026004804673],
-    [0.9840126224821667, 1.984006279065173, 2.984004178927043, 3.984003131531364],
-    [0.9830150304982433, 1.9830074756785594, 2.9830049750356973, 3.9830037280016044],
-    [0.9820177164052082, 1.9820088100921336, 2.982005862758586, 3.9820043930880837],
-    [0.9810206928263993, 1.9810102885187928, 2.981006846215933, 3.9810051298728633],
-]
+ADAM_ANSWERS = GOLDEN["adam_trajectory"]["values"]
 
 
 def adam_trajectory(driver, datatype):
