@@ -39,13 +39,19 @@ def values(rng, code, n, lo=-100, hi=100, nonzero=False):
     return v.astype(NP[code])
 
 
-def compare(buf, what, tol=None):
+def compare(buf, what, tol=None, denormal_ulps=0):
+    """tol: relative bar per element.  denormal_ulps: results below the smallest normal number of
+    the type may instead differ by that many units of the denormal grid, where one unit is a
+    large relative step."""
     got, want = buf.download(), buf.host
     if tol is None:
         H.assert_bit_exact(got, want, what)
         return
     g, w = got.astype(np.float64), want.astype(np.float64)
     ok = (np.abs(g - w) <= tol * np.abs(w)) | (np.isnan(g) & np.isnan(w)) | (g == w)
+    if denormal_ulps:
+        info = np.finfo(want.dtype)
+        ok |= (np.abs(w) < info.tiny) & (np.abs(g - w) <= denormal_ulps * float(info.smallest_subnormal))
     assert np.all(ok), f"{what}: max rel err {np.nanmax(np.abs(g - w) / np.abs(w))}"
 
 
@@ -572,6 +578,38 @@ def test_softmax_rows(P, code, shape):
         assert kern == "softmax_lane" if k < 8 else kern in ("softmax_wave", "softmax_wave_vec", "softmax_block")
     P.run(H.softmax, View(x, [rows, k]), View(x, [rows, k]))     # in place
     compare(x, f"softmax {shape} in place", tol=tol)
+
+
+@pytest.mark.parametrize("code", FLOATS)
+def test_softmax_wide_range(P, code):
+    """Rows whose entries lie hundreds below the maximum (exponentials in the denormal range and
+    below it) and rows with infinities and NaN: the float kernels' hardware-exp2 path hands the
+    far tail to the library routine, and special values behave as java.lang.Math.exp does."""
+    rng = np.random.default_rng(33)
+    tol = 2e-6 if code == capi.F32 else 1e-12
+    for rows, k in ((64, 16), (40, 1000), (300, 10), (7, 5000)):
+        v = (rng.standard_normal(rows * k) * 40).astype(NP[code])
+        v[::7] -= 60
+        x = P.buf(v)
+        out = P.buf(np.zeros(rows * k, NP[code]))
+        kern = P.run(H.softmax, View(out, [rows, k]), View(x, [rows, k]))
+        compare(out, f"softmax wide range {(rows, k)} ({kern})", tol=tol, denormal_ulps=2)
+    rows, k = 8, 12
+    v = rng.standard_normal(rows * k).astype(NP[code]).reshape(rows, k)
+    v[0, 3] = -np.inf
+    v[1, :] = -np.inf          # 0 / 0 throughout
+    v[2, 5] = np.inf           # inf - inf
+    v[3, 0] = np.nan
+    v[4, 1], v[4, 2] = -np.inf, 100.0
+    x = P.buf(v.reshape(-1))
+    out = P.buf(np.zeros(rows * k, NP[code]))
+    for shape, spatial in (([rows, k], False), ([1, rows, k], False)):
+        kern = P.run(H.softmax, View(out, shape), View(x, shape), spatial)
+        compare(out, f"softmax special values ({kern})", tol=tol)
+    xs = P.buf(np.ascontiguousarray(v.T).reshape(-1))      # the same rows along the channel axis
+    outs = P.buf(np.zeros(rows * k, NP[code]))
+    kern = P.run(H.softmax, View(outs, [1, k, rows]), View(xs, [1, k, rows]), True)
+    compare(outs, f"softmax-spatial special values ({kern})", tol=tol)
 
 
 @pytest.mark.parametrize("code", FLOATS)
