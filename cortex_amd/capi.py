@@ -31,6 +31,7 @@ BINARY_OPS = {"+": 0, "-": 1, "*": 2, "/": 3, "min": 4, "max": 5, "bit-and": 6, 
 TERNARY_OPS = {"select": 0}
 ACTIVATION_OPS = {"logistic": 0, "tanh": 1, "relu": 2}
 DISTRIBUTIONS = {"gaussian": 0, "flat": 1}
+POOL_OPS = {"max": 0, "avg": 1, "avg-exc-pad": 2}
 REDUCE_OPS = {"max": 0, "min": 1, "sum": 2, "mean": 3, "magnitude": 4, "magnitude-squared": 5}
 
 COPY_H2D, COPY_D2H, COPY_D2D = 0, 1, 2
@@ -45,6 +46,24 @@ class CtDims(C.Structure):
         ("strides", C.c_int64 * MAX_DIMS),
         ("index", C.c_void_p * MAX_DIMS),
     ]
+
+
+class CtPoolDesc(C.Structure):
+    """``ct_pool_desc``: the geometry of a pooling descriptor."""
+
+    _fields_ = [
+        ("kernel_width", C.c_int32), ("kernel_height", C.c_int32),
+        ("pad_x", C.c_int32), ("pad_y", C.c_int32),
+        ("stride_x", C.c_int32), ("stride_y", C.c_int32),
+        ("pool_op", C.c_int32),
+    ]
+
+
+def make_pool_desc(descriptor) -> CtPoolDesc:
+    """Builds a ``ct_pool_desc`` from a pooling descriptor map."""
+    return CtPoolDesc(int(descriptor["kernel-width"]), int(descriptor["kernel-height"]), int(descriptor["pad-x"]),
+                      int(descriptor["pad-y"]), int(descriptor["stride-x"]), int(descriptor["stride-y"]),
+                      POOL_OPS[descriptor["pool-op"]])
 
 
 def make_dims(shape: Sequence[int], strides: Sequence[int], index: Optional[Sequence[Optional[int]]] = None) -> CtDims:
@@ -118,6 +137,8 @@ PROTOTYPES = {
     "ct_batch_normalize_update_and_apply_spatial": [_P, _P, _P, _P, _P, _P, _P, _D, _P, _P, _D, _L, _L, _L, _I],
     "ct_batch_normalize_gradients_eltwise": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _I],
     "ct_batch_normalize_gradients_spatial": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _L, _I],
+    "ct_pooling_forward": [_P, _P, _D, _P, C.POINTER(CtPoolDesc), _L, _L, _L, _L, _L, _L, _I],
+    "ct_pooling_backward": [_P, _P, _D, _P, _P, _P, C.POINTER(CtPoolDesc), _L, _L, _L, _L, _L, _L, _I],
     "ct_gemm": [_P, _P, _L, _I, _I, _D, _P, _L, _L, _L, _P, _L, _L, _D, _I],
     "ct_gemv": [_P, _P, _L, _I, _D, _P, _L, _L, _L, _P, _L, _D, _I],
     "ct_rand": [_P, _P, _L, _I, _I, _D, _D, C.c_uint64, C.c_uint64],

@@ -299,6 +299,23 @@ class HipStream:
         capi.call("ct_softmax_spatial", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), input.ptr,
                   C.byref(_dims_struct(input_dims)), capi.DTYPE_CODES[output.datatype])
 
+    # -- pooling (tensor/math.clj:221-236); buffers are packed [batch channels height width] --
+    def pooling_forward(self, output, output_dims, output_alpha, input, input_dims, pool_descriptor) -> None:
+        batch, channels, in_h, in_w = (int(v) for v in input_dims["shape"])
+        out_h, out_w = (int(v) for v in output_dims["shape"][2:])
+        desc = capi.make_pool_desc(pool_descriptor)
+        capi.call("ct_pooling_forward", self.handle, output.ptr, float(output_alpha), input.ptr, C.byref(desc), batch,
+                  channels, in_h, in_w, out_h, out_w, capi.DTYPE_CODES[output.datatype])
+
+    def pooling_backward(self, input_grad, input_grad_dims, input_grad_alpha, input, input_dims, output, output_dims,
+                         output_grad, output_grad_dims, pool_descriptor) -> None:
+        batch, channels, in_h, in_w = (int(v) for v in input_dims["shape"])
+        out_h, out_w = (int(v) for v in output_dims["shape"][2:])
+        desc = capi.make_pool_desc(pool_descriptor)
+        capi.call("ct_pooling_backward", self.handle, input_grad.ptr, float(input_grad_alpha), input.ptr, output.ptr,
+                  output_grad.ptr, C.byref(desc), batch, channels, in_h, in_w, out_h, out_w,
+                  capi.DTYPE_CODES[output.datatype])
+
     # -- gemm!, gemv! (tensor/math.clj:106-123) ---------------------------------
     def gemm(self, c, c_colstride, trans_a, trans_b, alpha, a, a_row_count, a_col_count, a_colstride, b, b_col_count,
              b_colstride, beta) -> None:

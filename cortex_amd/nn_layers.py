@@ -313,6 +313,59 @@ class BatchNormalization:
 
 # ------------------------------------------------------------------ prelu
 
+def max_pooling(kernel_dim: int, pad: int, stride: int, input_dimension: dict, **args) -> dict:
+    """The description of a pooling layer as ``layers/max-pooling``
+    (``src/cortex/nn/layers.clj:492-511``) writes it and
+    ``build-convolutional-type-node`` (``:449-465``) completes it: square kernel,
+    padding and stride, ``:dimension-op :ceil`` and ``:pool-op :max`` unless
+    given, output dimensions from the padded-strided formula (``:421-446``)."""
+    if stride < 1:
+        raise ValueError("Convolutional layers must have stride >= 1")
+    if kernel_dim < 1:
+        raise ValueError("Convolutional layers must have kernel dimensions >= 1")
+    node = {"type": "max-pooling", "kernel-width": kernel_dim, "kernel-height": kernel_dim, "pad-x": pad,
+            "pad-y": pad, "stride-x": stride, "stride-y": stride, "num-kernels": 0, "dimension-op": "ceil"}
+    node.update({k.replace("_", "-"): v for k, v in args.items()})
+    node.setdefault("pool-op", "max")
+    if node["pool-op"] not in ct.POOL_OPERATIONS:
+        raise ValueError(f"Max pooling layers have three possible pool operations: {ct.POOL_OPERATIONS}")
+    out = ct.get_convolution_output_dimensions(node, input_dimension["width"], input_dimension["height"])
+    node["input-dimension"] = dict(input_dimension)
+    node["output-dimension"] = {"channels": input_dimension["channels"], "height": out["output-height"],
+                                "width": out["output-width"]}
+    return node
+
+
+def _conv_tensor(dimension: dict, batch_size: int, t: ct.Tensor) -> ct.Tensor:
+    """``->conv-tensor`` (``layers.clj:297-303``)."""
+    return ct.in_place_reshape(t, [batch_size, dimension["channels"], dimension["height"], dimension["width"]])
+
+
+class PoolingLayer:
+    """``PoolingLayer`` (``layers.clj:390-428``)."""
+
+    def __init__(self, layer: dict, batch_size: int, datatype: str = None):
+        self.layer, self.batch_size = layer, batch_size
+        self.pool_desc = ct.pooling_descriptor(datatype or ct.current_datatype(), layer["input-dimension"]["channels"],
+                                               layer["kernel-width"], layer["kernel-height"], layer["pad-x"],
+                                               layer["pad-y"], layer["stride-x"], layer["stride-y"],
+                                               dimension_op=layer.get("dimension-op"),
+                                               pool_op=layer.get("pool-op") or "max")
+
+    def forward(self, parameter_buffers, input_buffers, output_buffers):
+        output = _conv_tensor(self.layer["output-dimension"], self.batch_size, first_buffer(output_buffers))
+        input = _conv_tensor(self.layer["input-dimension"], self.batch_size, first_buffer(input_buffers))
+        ct.pooling_forward(output, 0.0, input, self.pool_desc)
+
+    def backward(self, parameter_buffers, output_buffers, input_buffers):
+        output = _conv_tensor(self.layer["output-dimension"], self.batch_size, first_buffer(output_buffers))
+        output_gradient = _conv_tensor(self.layer["output-dimension"], self.batch_size,
+                                       first_gradient(output_buffers))
+        input = _conv_tensor(self.layer["input-dimension"], self.batch_size, first_buffer(input_buffers))
+        input_gradient = _conv_tensor(self.layer["input-dimension"], self.batch_size, first_gradient(input_buffers))
+        ct.pooling_backward(input_gradient, 0.0, input, output, output_gradient, self.pool_desc)
+
+
 def prelu_size(layer: dict) -> int:
     """One slope per channel, or per element when there is one channel
     (``src/cortex/nn/layers.clj:241-246``)."""
@@ -478,6 +531,8 @@ def create(node: dict, batch_size: int, datatype: str = None):
         return BatchNormalization(node, datatype)
     if kind == "prelu":
         return Prelu(node, batch_size, datatype)
+    if kind == "max-pooling":
+        return PoolingLayer(node, batch_size, datatype)
     if kind == "concatenate":
         return Concatenate()
     if kind == "split":

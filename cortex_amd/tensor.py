@@ -513,6 +513,87 @@ def softmax(output: Tensor, input: Tensor) -> Tensor:
     return output
 
 
+# ---------------------------------------------------------------- pooling
+
+POOL_OPERATIONS = ("max", "avg", "avg-exc-pad")
+
+
+def _padded_strided_dimension(input_dim, pad, kernel_size, stride, dimension_op) -> int:
+    """``get-padded-strided-dimension`` (``tensor.clj:1351-1365``)."""
+    partial = (float(input_dim) + 2.0 * float(pad) - float(kernel_size)) / float(stride)
+    if dimension_op == "floor":
+        partial = math.floor(partial)
+    elif dimension_op == "ceil":
+        partial = math.ceil(partial)
+    else:
+        raise TensorError(f"No matching clause: {dimension_op}")
+    return int(partial + 1)
+
+
+def get_convolution_output_dimensions(descriptor, input_width, input_height):
+    """``get-convolution-output-dimensions`` (``tensor.clj:1368-1382``)."""
+    op = descriptor.get("dimension-op") or "floor"
+    return {"output-width": _padded_strided_dimension(input_width, descriptor["pad-x"], descriptor["kernel-width"],
+                                                      descriptor["stride-x"], op),
+            "output-height": _padded_strided_dimension(input_height, descriptor["pad-y"],
+                                                       descriptor["kernel-height"], descriptor["stride-y"], op)}
+
+
+def pooling_descriptor(datatype, channels, kern_width, kern_height, pad_x, pad_y, stride_x, stride_y, *,
+                       dimension_op="ceil", pool_op="max"):
+    """``pooling-descriptor`` (``tensor.clj:1499-1524``); the library keeps no
+    descriptor object of its own, as the CPU backend keeps none
+    (``cpu/tensor_math.clj:1794-1798``)."""
+    retval = {"in-channels": channels, "out-channels": channels, "datatype": datatype, "kernel-width": kern_width,
+              "kernel-height": kern_height, "pad-x": pad_x, "pad-y": pad_y, "stride-x": stride_x,
+              "stride-y": stride_y, "pool-op": pool_op, "dimension-op": dimension_op}
+    missing = [k for k, v in retval.items() if v is None]
+    if missing:
+        raise TensorError(f"Nil values detected in map: {missing}")
+    if pool_op not in POOL_OPERATIONS:
+        raise TensorError(f"Max pooling layers have three possible pool operations: {POOL_OPERATIONS}, got {pool_op}")
+    check_stream()
+    return retval
+
+
+def _ensure_conv_io(descriptor, input_args, output_args) -> None:
+    """``ensure-conv-io`` (``tensor.clj:1425-1451``).  As there, the output is
+    expected as [batch channels output-width output-height] and only the first
+    tensor of each list is compared."""
+    batch_size, _, in_height, in_width = input_args[0].shape()
+    out = get_convolution_output_dimensions(descriptor, in_height, in_width)
+    expected_input = [batch_size, int(descriptor["in-channels"]), in_height, in_width]
+    expected_output = [batch_size, int(descriptor["out-channels"]), out["output-width"], out["output-height"]]
+    if not all(dense(t) for t in list(input_args) + list(output_args)):
+        raise TensorError("Convolution arguments must be dense tensors")
+    if list(input_args[0].shape()) != expected_input:
+        raise TensorError(f"Input dimensions do not match expected dimensions {expected_input} "
+                          f"{list(input_args[0].shape())}")
+    if list(output_args[0].shape()) != expected_output:
+        raise TensorError(f"Output dimensions do not match expected dimensions {expected_output} "
+                          f"{list(output_args[0].shape())}")
+
+
+def pooling_forward(output: Tensor, output_alpha, input: Tensor, pool_descriptor) -> Tensor:
+    """``pooling-forward!`` (``tensor.clj:1527-1538``)."""
+    _external_library_check("pooling-forward!", output, input)
+    _ensure_conv_io(pool_descriptor, [input], [output])
+    check_stream().pooling_forward(output.buffer, output.dimensions, output_alpha, input.buffer, input.dimensions,
+                                   pool_descriptor)
+    return output
+
+
+def pooling_backward(input_gradient: Tensor, input_grad_alpha, input: Tensor, output: Tensor,
+                     output_gradient: Tensor, pool_descriptor) -> Tensor:
+    """``pooling-backward!`` (``tensor.clj:1541-1551``)."""
+    _external_library_check("pooling-backward!", input_gradient, input, output, output_gradient)
+    _ensure_conv_io(pool_descriptor, [input_gradient, input], [output, output_gradient])
+    check_stream().pooling_backward(input_gradient.buffer, input_gradient.dimensions, input_grad_alpha, input.buffer,
+                                    input.dimensions, output.buffer, output.dimensions, output_gradient.buffer,
+                                    output_gradient.dimensions, pool_descriptor)
+    return input_gradient
+
+
 # ---------------------------------------------------------------- gemm!, gemv!
 
 def _column_stride(t: Tensor) -> int:

@@ -89,6 +89,18 @@ typedef enum ct_activation_op_t {
 /* rand! distributions (src/cortex/tensor.clj:989-1017). */
 typedef enum ct_distribution_t { CT_DIST_GAUSSIAN = 0, CT_DIST_FLAT = 1 } ct_distribution_t;
 
+/* :pool-op of a pooling descriptor (src/cortex/tensor.clj:1495-1524). */
+typedef enum ct_pool_op_t { CT_POOL_MAX = 0, CT_POOL_AVG = 1, CT_POOL_AVG_EXC_PAD = 2 } ct_pool_op_t;
+
+/* The geometry of a pooling descriptor (src/cortex/tensor.clj:1499-1524): the
+ * window, the zero padding on each side and the step between windows. */
+typedef struct ct_pool_desc {
+  int32_t kernel_width, kernel_height;
+  int32_t pad_x, pad_y;
+  int32_t stride_x, stride_y;
+  int32_t pool_op; /* ct_pool_op_t */
+} ct_pool_desc;
+
 typedef enum ct_status {
   CT_OK = 0,
   CT_ERR_INVALID = 1,     /* bad argument: rank, dtype, op code, null pointer, shape rule */
@@ -357,6 +369,32 @@ int ct_batch_normalize_gradients_spatial(void* stream, void* input_gradient, voi
                                          const void* scale, const void* bias, double epsilon,
                                          int64_t batch_count, int64_t channel_count,
                                          int64_t element_count, int dtype);
+
+/* pooling-forward! / pooling-backward! (tensor/math.clj:221-236;
+ * cpu/tensor_math.clj:1153-1284, 1800-1866; window walk src/cortex/nn/impl.clj:8-96).
+ * Buffers are packed [batch_count, channel_count, height, width]; dtype is
+ * CT_F32 or CT_F64.  The taps of a window are visited row by row, those beyond
+ * the padded input are skipped, and padding reads as 0:
+ *   max          the first tap, then every tap greater than the running value
+ *                (padding takes part as 0, NaN only wins as the first tap)
+ *   avg          sum of tap / (kernel_width * kernel_height), rounded to the
+ *                tensor's type after every tap
+ *   avg-exc-pad  tap / (taps of the window inside the input), added ONTO what
+ *                `output` holds: the CPU backend never clears it
+ * The backward pass adds into input_gradient (never cleared either): for max,
+ * output_gradient of every window whose output equals this input; for the
+ * averages, output_gradient / divisor of every window covering it; windows in
+ * increasing (row, column) order.  output_alpha and input_gradient_alpha are
+ * accepted for signature parity: the CPU backend does not read them. */
+int ct_pooling_forward(void* stream, void* output, double output_alpha, const void* input,
+                       const ct_pool_desc* desc, int64_t batch_count, int64_t channel_count,
+                       int64_t in_height, int64_t in_width, int64_t out_height, int64_t out_width,
+                       int dtype);
+int ct_pooling_backward(void* stream, void* input_gradient, double input_gradient_alpha,
+                        const void* input, const void* output, const void* output_gradient,
+                        const ct_pool_desc* desc, int64_t batch_count, int64_t channel_count,
+                        int64_t in_height, int64_t in_width, int64_t out_height, int64_t out_width,
+                        int dtype);
 
 /* ------------------------------------------------- optimizers */
 

@@ -22,6 +22,8 @@
 //   activation-gradient!     cpu/tensor_math.clj:1318-1362
 //   softmax (both forms)     cpu/tensor_math.clj:1037-1103
 //   batch-normalize (6 forms) cpu/tensor_math.clj:731-1033, 1558-1638
+//   pooling (6 forms)        cpu/tensor_math.clj:1153-1284, 1800-1866 over the
+//                            window walk of src/cortex/nn/impl.clj:8-96
 //   gemm!, gemv!             cpu/tensor_math.clj:672-726, 1534-1556 and
 //                            compute/math_util.clj:17-41 for the operand
 //                            mapping; the product itself is netlib BLAS
@@ -805,6 +807,97 @@ inline void adadelta_micro(double g, double decay, double eps, double ga_in, dou
   *dx_out = dx;
 }
 
+// ------------------------------------------------------------------ pooling
+// The window walk of src/cortex/nn/impl.clj:8-96 (convolution-outer-kernel with
+// convolution-roll-unroll-inner-kernel) over one image, with the six bodies of
+// cpu/tensor_math.clj:1153-1284.  Loops and their order are the reference's: the
+// backward bodies scatter into the input gradient one tap at a time.
+
+struct PoolGeom {
+  int64_t channels, in_h, in_w, out_h, out_w;
+  int64_t kw, kh, pad_x, pad_y, stride_x, stride_y;
+};
+
+template <class Body>
+void pool_walk(const PoolGeom& g, Body body) {
+  const int64_t min_x = -g.pad_x, min_y = -g.pad_y, max_x = g.in_w + g.pad_x, max_y = g.in_h + g.pad_y;
+  for (int64_t chan = 0; chan < g.channels; ++chan) {
+    const int64_t chan_in = chan * g.in_w * g.in_h, chan_out = chan * g.out_w * g.out_h;
+    for (int64_t out_y = 0; out_y < g.out_h; ++out_y) {
+      const int64_t rel_y = out_y * g.stride_y - g.pad_y;
+      for (int64_t out_x = 0; out_x < g.out_w; ++out_x) {
+        const int64_t rel_x = out_x * g.stride_x - g.pad_x;
+        const int64_t over_x = std::max<int64_t>(0, rel_x + g.kw - g.in_w);
+        const int64_t over_y = std::max<int64_t>(0, rel_y + g.kh - g.in_h);
+        const int64_t under_x = std::min<int64_t>(rel_x, 0), under_y = std::min<int64_t>(rel_y, 0);
+        const int64_t exc_w = std::max<int64_t>(0, g.kw - over_x + under_x);
+        const int64_t exc_h = std::max<int64_t>(0, g.kh - over_y + under_y);
+        const int64_t exc_count = exc_w * exc_h;
+        const int64_t out_addr = out_y * g.out_w + out_x + chan_out;
+        for (int64_t k_y = 0; k_y < g.kh; ++k_y)
+          for (int64_t k_x = 0; k_x < g.kw; ++k_x) {
+            const int64_t in_x = rel_x + k_x, in_y = rel_y + k_y;
+            const bool input_valid = in_x >= 0 && in_x < g.in_w && in_y >= 0 && in_y < g.in_h;
+            const bool loop_valid = in_x >= min_x && in_x < max_x && in_y >= min_y && in_y < max_y;
+            if (loop_valid) body(in_y * g.in_w + in_x + chan_in, out_addr, k_y * g.kw + k_x, input_valid, exc_count);
+          }
+      }
+    }
+  }
+}
+
+template <class T>
+void pool_forward_image(T* out, const T* in, const PoolGeom& g, int op) {
+  const int64_t kernel_count = g.kw * g.kh;
+  if (op == CT_POOL_MAX) {  // :1153-1172
+    pool_walk(g, [&](int64_t ia, int64_t oa, int64_t k_idx, bool valid, int64_t) {
+      const T v = valid ? in[ia] : (T)0.0;
+      if (k_idx == 0 || v > out[oa]) out[oa] = v;
+    });
+  } else if (op == CT_POOL_AVG) {  // :1198-1219
+    pool_walk(g, [&](int64_t ia, int64_t oa, int64_t k_idx, bool valid, int64_t) {
+      const T v = valid ? in[ia] : (T)0.0;
+      const T prev = k_idx == 0 ? (T)0 : out[oa];
+      out[oa] = (T)((double)prev + (double)v / (double)kernel_count);
+    });
+  } else {  // :avg-exc-pad, :1243-1261 -- adds onto what the output holds
+    pool_walk(g, [&](int64_t ia, int64_t oa, int64_t, bool valid, int64_t exc_count) {
+      const T v = valid ? in[ia] : (T)0.0;
+      out[oa] = (T)((double)out[oa] + (double)v / (double)exc_count);
+    });
+  }
+}
+
+template <class T>
+void pool_backward_image(T* ig, const T* in, const T* out, const T* og, const PoolGeom& g, int op) {
+  const int64_t kernel_count = g.kw * g.kh;
+  if (op == CT_POOL_MAX) {  // :1175-1196
+    pool_walk(g, [&](int64_t ia, int64_t oa, int64_t, bool valid, int64_t) {
+      if (valid && in[ia] == out[oa]) ig[ia] = (T)((double)ig[ia] + (double)og[oa]);
+    });
+  } else if (op == CT_POOL_AVG) {  // :1221-1241
+    pool_walk(g, [&](int64_t ia, int64_t oa, int64_t, bool valid, int64_t) {
+      if (valid) ig[ia] = (T)((double)ig[ia] + (double)og[oa] / (double)kernel_count);
+    });
+  } else {  // :1263-1284
+    pool_walk(g, [&](int64_t ia, int64_t oa, int64_t, bool valid, int64_t exc_count) {
+      if (valid) ig[ia] = (T)((double)ig[ia] + (double)og[oa] / (double)exc_count);
+    });
+  }
+}
+
+bool pool_geom(const ct_pool_desc* d, int64_t batch, int64_t channels, int64_t in_h, int64_t in_w, int64_t out_h,
+               int64_t out_w, PoolGeom* g) {
+  if (!d || batch < 0 || channels < 0 || in_h < 0 || in_w < 0 || out_h < 0 || out_w < 0) return false;
+  if (d->kernel_width < 1 || d->kernel_height < 1 || d->stride_x < 1 || d->stride_y < 1 || d->pad_x < 0 ||
+      d->pad_y < 0)
+    return false;
+  if (d->pool_op != CT_POOL_MAX && d->pool_op != CT_POOL_AVG && d->pool_op != CT_POOL_AVG_EXC_PAD) return false;
+  *g = PoolGeom{channels, in_h, in_w, out_h, out_w, d->kernel_width, d->kernel_height, d->pad_x, d->pad_y,
+                d->stride_x, d->stride_y};
+  return true;
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------ C entry points
@@ -1177,6 +1270,48 @@ int co_rand(void* dest, int64_t n, int dtype, int distribution, double a, double
       }
     }
     for (int e = 0; e < 4 && i * 4 + e < n; ++e) d[i * 4 + e] = v[e];
+  }
+  return 0;
+}
+
+// pooling-forward! / pooling-backward! (cpu/tensor_math.clj:1800-1866): the
+// images of the batch are independent (the reference maps them with pmap); the
+// alphas are not read there and are not taken here.
+int co_pooling_forward(void* output, double, const void* input, const ct_pool_desc* desc, int64_t batch_count,
+                       int64_t channel_count, int64_t in_height, int64_t in_width, int64_t out_height,
+                       int64_t out_width, int dtype) {
+  PoolGeom g;
+  if (!pool_geom(desc, batch_count, channel_count, in_height, in_width, out_height, out_width, &g))
+    return fail("pooling: bad descriptor or counts");
+  if (dtype != CT_F32 && dtype != CT_F64) return fail("Failed to find cpu pooling op");
+  const int64_t in_img = channel_count * in_height * in_width, out_img = channel_count * out_height * out_width;
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < batch_count; ++b) {
+    if (dtype == CT_F32) pool_forward_image((float*)output + b * out_img, (const float*)input + b * in_img, g, desc->pool_op);
+    else pool_forward_image((double*)output + b * out_img, (const double*)input + b * in_img, g, desc->pool_op);
+  }
+  return 0;
+}
+
+int co_pooling_backward(void* input_gradient, double, const void* input, const void* output,
+                        const void* output_gradient, const ct_pool_desc* desc, int64_t batch_count,
+                        int64_t channel_count, int64_t in_height, int64_t in_width, int64_t out_height,
+                        int64_t out_width, int dtype) {
+  PoolGeom g;
+  if (!pool_geom(desc, batch_count, channel_count, in_height, in_width, out_height, out_width, &g))
+    return fail("pooling: bad descriptor or counts");
+  if (dtype != CT_F32 && dtype != CT_F64) return fail("Failed to find cpu pooling op");
+  const int64_t in_img = channel_count * in_height * in_width, out_img = channel_count * out_height * out_width;
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < batch_count; ++b) {
+    if (dtype == CT_F32)
+      pool_backward_image((float*)input_gradient + b * in_img, (const float*)input + b * in_img,
+                          (const float*)output + b * out_img, (const float*)output_gradient + b * out_img, g,
+                          desc->pool_op);
+    else
+      pool_backward_image((double*)input_gradient + b * in_img, (const double*)input + b * in_img,
+                          (const double*)output + b * out_img, (const double*)output_gradient + b * out_img, g,
+                          desc->pool_op);
   }
   return 0;
 }

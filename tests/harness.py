@@ -227,6 +227,23 @@ def softmax(side, out: View, inp: View, spatial=False):
     side.call("softmax_spatial" if spatial else "softmax_eltwise", *_pd(side, out), *_pd(side, inp), out.buf.dtype)
 
 
+def pool_desc(kw, kh, px, py, sx, sy, op):
+    return {"kernel-width": kw, "kernel-height": kh, "pad-x": px, "pad-y": py, "stride-x": sx, "stride-y": sy,
+            "pool-op": op}
+
+
+def pooling_forward(side, out: View, inp: View, desc, batch, channels, in_h, in_w, out_h, out_w):
+    d = capi.make_pool_desc(desc)
+    side.call("pooling_forward", side.ptr(out), 0.0, side.ptr(inp), C.byref(d), batch, channels, in_h, in_w, out_h,
+              out_w, out.buf.dtype)
+
+
+def pooling_backward(side, ig: View, inp: View, out: View, og: View, desc, batch, channels, in_h, in_w, out_h, out_w):
+    d = capi.make_pool_desc(desc)
+    side.call("pooling_backward", side.ptr(ig), 0.0, side.ptr(inp), side.ptr(out), side.ptr(og), C.byref(d), batch,
+              channels, in_h, in_w, out_h, out_w, ig.buf.dtype)
+
+
 def batch_normalize(side, out: View, inp: View, means: View, variances: View, scale: View, bias: View, epsilon,
                     batch, channels, elements=None):
     """elements=None selects the eltwise form ([batch, channels] with one statistic per element)."""

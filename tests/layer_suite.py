@@ -46,16 +46,57 @@ def forward_backward(layer, parameters, inputs, outputs, output_gradients):
     layer.backward(parameters, outputs, inputs)
 
 
-def single(node, batch_size, input, output_gradient, parameters=None, item_shape=None, datatype=None):
+def single(node, batch_size, input, output_gradient, parameters=None, item_shape=None, datatype=None,
+           output_item_shape=None):
     """``forward-backward-test`` (verify/nn/layers.clj:143-153)."""
     input = np.asarray(input, dtype=np.float64)
     shape = [batch_size] + list(item_shape or [input.size // batch_size])
+    out_shape = [batch_size] + list(output_item_shape) if output_item_shape else shape
     layer = nl.create(node, batch_size, datatype)
     inputs = [entry(input, shape)]
-    outputs = [{"buffer": ct.new_tensor(shape), "gradient": ct.new_tensor(shape)}]
+    outputs = [{"buffer": ct.new_tensor(out_shape), "gradient": ct.new_tensor(out_shape)}]
     forward_backward(layer, parameters or {}, inputs, outputs, [output_gradient])
     return {"output": ct.to_double_array(outputs[0]["buffer"]).reshape(-1),
             "input-gradient": ct.to_double_array(inputs[0]["gradient"]).reshape(-1), "layer": layer}
+
+
+def _pool(node, batch_size, input, output_gradient):
+    d = node["output-dimension"]
+    return single(node, batch_size, input, output_gradient,
+                  output_item_shape=[d["channels"] * d["height"] * d["width"]])
+
+
+# verify/nn/layers.clj:560-590: (layers/input 2 2 4) is width 2, height 2, 4 channels
+def pool_layer_basic(driver, datatype):
+    with context(driver, datatype):
+        batch_size, dimension = 10, {"channels": 4, "height": 2, "width": 2}
+        node = nl.max_pooling(2, 0, 1, dimension)
+        r = _pool(node, batch_size, list(range(1, 17)) * batch_size, [1, 2, 3, 4] * batch_size)
+        equals([4, 8, 12, 16] * batch_size, r["output"])
+        equals([v for _ in range(batch_size) for g in range(1, 5) for v in (0, 0, 0, g)], r["input-gradient"])
+        r = _pool(node, batch_size, list(range(16, 0, -1)) * batch_size, [1, 2, 3, 4] * batch_size)
+        equals([16, 12, 8, 4] * batch_size, r["output"])
+        equals([v for _ in range(batch_size) for g in range(1, 5) for v in (g, 0, 0, 0)], r["input-gradient"])
+
+
+# verify/nn/layers.clj:593-611
+def pool_layer_avg(driver, datatype):
+    with context(driver, datatype):
+        batch_size, num_channels = 10, 4
+        node = nl.max_pooling(2, 1, 1, {"channels": num_channels, "height": 2, "width": 2}, pool_op="avg")
+        r = _pool(node, batch_size, [1] * (16 * batch_size), list(range(1, 10)) * (batch_size * num_channels))
+        equals([0.25, 0.5, 0.25, 0.5, 1.0, 0.5, 0.25, 0.5, 0.25] * (batch_size * num_channels), r["output"])
+        equals([3, 4, 6, 7] * (batch_size * num_channels), r["input-gradient"])
+
+
+# verify/nn/layers.clj:614-632
+def pool_layer_avg_exc_pad(driver, datatype):
+    with context(driver, datatype):
+        batch_size, num_channels = 10, 4
+        node = nl.max_pooling(2, 1, 1, {"channels": num_channels, "height": 2, "width": 2}, pool_op="avg-exc-pad")
+        r = _pool(node, batch_size, [1] * (16 * batch_size), list(range(1, 10)) * (batch_size * num_channels))
+        equals([1] * (9 * batch_size * num_channels), r["output"])
+        equals([5.25, 8.25, 14.25, 17.25] * (batch_size * num_channels), r["input-gradient"])
 
 
 # verify/nn/layers.clj:155-191

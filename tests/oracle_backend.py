@@ -189,6 +189,19 @@ class OracleStream:
         ob.call("batch_normalize_gradients_spatial", ig.ptr, sg.ptr, bg.ptr, og.ptr, out.ptr, inp.ptr, bm.ptr, bv.ptr,
                 scale.ptr, bias.ptr, float(eps), int(batch), int(chans), int(elems), capi.DTYPE_CODES[ig.datatype])
 
+    def pooling_forward(self, out, od, out_alpha, inp, idims, desc):
+        batch, channels, in_h, in_w = (int(v) for v in idims["shape"])
+        out_h, out_w = (int(v) for v in od["shape"][2:])
+        ob.call("pooling_forward", out.ptr, float(out_alpha), inp.ptr, C.byref(capi.make_pool_desc(desc)), batch,
+                channels, in_h, in_w, out_h, out_w, capi.DTYPE_CODES[out.datatype])
+
+    def pooling_backward(self, ig, igd, ig_alpha, inp, idims, out, od, og, ogd, desc):
+        batch, channels, in_h, in_w = (int(v) for v in idims["shape"])
+        out_h, out_w = (int(v) for v in od["shape"][2:])
+        ob.call("pooling_backward", ig.ptr, float(ig_alpha), inp.ptr, out.ptr, og.ptr,
+                C.byref(capi.make_pool_desc(desc)), batch, channels, in_h, in_w, out_h, out_w,
+                capi.DTYPE_CODES[out.datatype])
+
     def gemm(self, c, ldc, ta, tb, alpha, a, a_rows, a_cols, lda, b, b_cols, ldb, beta):
         ob.call("gemm", c.ptr, int(ldc), int(bool(ta)), int(bool(tb)), float(alpha), a.ptr, int(a_rows), int(a_cols),
                 int(lda), b.ptr, int(b_cols), int(ldb), float(beta), capi.DTYPE_CODES[c.datatype])

@@ -251,6 +251,30 @@ def softmax(driver, datatype):
         equals(([0, 1] + list(ct.to_double_array(answer))) * 5, ct.to_double_array(pred_matrix))
 
 
+# verify/tensor.clj:893-1051
+def pooling_operator(driver, datatype):
+    with context(driver, datatype):
+        want = GOLDEN["pooling_operator"]
+        channels, dimension, batch_size = 4, 4, 2
+        n_elems = batch_size * channels * dimension * dimension
+        cycle = list(range(-5, 15))
+        values = [cycle[i % len(cycle)] for i in range(n_elems)]
+        inp = ct.to_tensor(np.asarray(values, dtype=np.float64).reshape(batch_size, channels, dimension, dimension))
+        descs = {op: ct.pooling_descriptor(datatype, channels, 3, 3, 1, 1, 2, 2, pool_op=op, dimension_op="floor")
+                 for op in ("max", "avg", "avg-exc-pad")}
+        out_dims = ct.get_convolution_output_dimensions(descs["max"], dimension, dimension)
+        out_shape = [batch_size, channels, out_dims["output-width"], out_dims["output-height"]]
+        assert out_shape == [2, 4, 2, 2]
+        output_gradient = ct.to_tensor(np.ones(out_shape))
+        for op, key, eps in (("max", "max", 0.0), ("avg", "avg", 1e-4), ("avg-exc-pad", "avg_exc_pad", 1e-4)):
+            output = ct.new_tensor(out_shape)
+            input_gradient = ct.new_tensor(ct.shape(inp))
+            ct.pooling_forward(output, 0.0, inp, descs[op])
+            equals(want[key + "_forward"], ct.to_double_array(output), eps)
+            ct.pooling_backward(input_gradient, 0.0, inp, output, output_gradient, descs[op])
+            equals(want[key + "_backward"], ct.to_double_array(input_gradient), 1e-4)
+
+
 # verify/tensor.clj:252-283; also exercises sub-matrices
 def gemm(driver, datatype):
     with context(driver, datatype):

@@ -824,6 +824,85 @@ def test_rand_errors(P):
 # double accumulator.  Bar: |got - want| <= tol * (|alpha| sum |a||b| + |beta c|) with
 # tol = 1e-5 for float (k up to 512 terms of 2^-24 relative error each) and 1e-13 for double.
 
+# ------------------------------------------------------------------ pooling
+# (batch, channels, height, width, kw, kh, px, py, sx, sy, dimension-op)
+POOL_CASES = [
+    (2, 4, 4, 4, 3, 3, 1, 1, 2, 2, "floor"),       # the reference's own test geometry
+    (3, 5, 17, 23, 3, 3, 1, 1, 2, 2, "ceil"),      # ragged, windows running past the padding
+    (2, 3, 32, 32, 2, 2, 0, 0, 2, 2, "floor"),     # disjoint windows
+    (2, 3, 9, 9, 2, 2, 1, 1, 1, 1, "ceil"),        # every input under four windows
+    (1, 2, 30, 19, 5, 3, 2, 1, 3, 2, "ceil"),      # rectangular window, stride and padding
+    (2, 2, 13, 13, 3, 3, 0, 0, 1, 1, "floor"),     # nine windows per input
+    (1, 3, 11, 14, 2, 2, 0, 0, 3, 3, "ceil"),      # stride beyond the window: inputs under no window
+    (1, 1, 5, 7, 7, 5, 3, 2, 1, 1, "floor"),       # window as large as the image
+    (4, 8, 56, 56, 3, 3, 1, 1, 2, 2, "floor"),
+    (1, 1, 1, 1, 1, 1, 0, 0, 1, 1, "floor"),
+]
+
+
+def pool_out_dim(n, pad, k, stride, op):
+    partial = (n + 2.0 * pad - k) / stride
+    return int((np.floor(partial) if op == "floor" else np.ceil(partial)) + 1)
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("op", list(capi.POOL_OPS))
+@pytest.mark.parametrize("case", POOL_CASES, ids=str)
+def test_pooling_bit_exact(P, code, op, case):
+    batch, channels, h, w, kw, kh, px, py, sx, sy, dim_op = case
+    oh, ow = pool_out_dim(h, py, kh, sy, dim_op), pool_out_dim(w, px, kw, sx, dim_op)
+    rng = np.random.default_rng(50)
+    n_in, n_out = batch * channels * h * w, batch * channels * oh * ow
+    # small integers: ties inside a window decide which inputs the max gradient reaches
+    x = rng.integers(-4, 5, n_in).astype(NP[code]) if op == "max" else values(rng, code, n_in)
+    if n_in > 8:
+        x[:3] = [np.nan, -0.0, 0.0]
+    inp, out = P.buf(x), P.buf(values(rng, code, n_out))       # avg-exc-pad adds onto the output
+    og, ig = P.buf(values(rng, code, n_out)), P.buf(values(rng, code, n_in))  # the gradient is added onto
+    desc = H.pool_desc(kw, kh, px, py, sx, sy, op)
+    geom = (desc, batch, channels, h, w, oh, ow)
+    k = P.run(H.pooling_forward, View(out, [n_out]), View(inp, [n_in]), *geom)
+    assert k == "pool_forward"
+    compare(out, f"pooling-forward {op} {case}")
+    k = P.run(H.pooling_backward, View(ig, [n_in]), View(inp, [n_in]), View(out, [n_out]), View(og, [n_out]), *geom)
+    assert k == "pool_backward"
+    compare(ig, f"pooling-backward {op} {case}")
+
+
+def test_pooling_first_tap_outside_padded_input(P):
+    """A stride that carries the last window past the padded input leaves no first tap to
+    reset the value: max and avg continue from what the output held (impl.clj:84-96)."""
+    rng = np.random.default_rng(51)
+    for op in capi.POOL_OPS:
+        h = w = 5
+        oh = ow = 4                      # the caller's output is larger than the formula's
+        x, prev = values(rng, capi.F32, h * w), values(rng, capi.F32, oh * ow)
+        inp, out = P.buf(x), P.buf(prev)
+        desc = H.pool_desc(2, 2, 0, 0, 2, 2, op)
+        P.run(H.pooling_forward, View(out, [oh * ow]), View(inp, [h * w]), desc, 1, 1, h, w, oh, ow)
+        compare(out, f"pooling-forward {op} with windows beyond the input")
+        og, ig = P.buf(values(rng, capi.F32, oh * ow)), P.buf(np.zeros(h * w, np.float32))
+        P.run(H.pooling_backward, View(ig, [h * w]), View(inp, [h * w]), View(out, [oh * ow]), View(og, [oh * ow]),
+              desc, 1, 1, h, w, oh, ow)
+        compare(ig, f"pooling-backward {op} with windows beyond the input")
+
+
+def test_pooling_errors(P):
+    b = P.buf(np.zeros(64, np.float32))
+    v = View(b, [64])
+    good = H.pool_desc(2, 2, 0, 0, 2, 2, "max")
+    for desc, dtype_buf in ((H.pool_desc(0, 2, 0, 0, 2, 2, "max"), b), (H.pool_desc(2, 2, 0, 0, 0, 2, "max"), b),
+                            (H.pool_desc(2, 2, -1, 0, 2, 2, "max"), b)):
+        with pytest.raises(capi.CortexHipError):
+            H.pooling_forward(P.hip, v, v, desc, 1, 1, 4, 4, 2, 2)
+    ints = P.buf(np.zeros(64, np.int32))
+    with pytest.raises(capi.CortexHipError, match="pooling op"):
+        H.pooling_forward(P.hip, View(ints, [64]), View(ints, [64]), good, 1, 1, 4, 4, 2, 2)
+    with pytest.raises(capi.CortexHipError, match="negative"):
+        H.pooling_forward(P.hip, v, v, good, -1, 1, 4, 4, 2, 2)
+    H.pooling_forward(P.hip, v, v, good, 0, 1, 4, 4, 2, 2)    # an empty batch is no error
+
+
 GEMM_CASES = [(5, 7, 4, 9, 8, 6), (64, 64, 64, 64, 64, 64), (33, 129, 65, 140, 70, 70), (256, 512, 128, 512, 512, 128),
               (1, 300, 1, 300, 300, 1)]
 

@@ -711,3 +711,70 @@ def test_gemv_matches_numpy(ta):
     vy, va, vx = (H.View(bf, [bf.init.size]) for bf in bufs)
     H.gemv(H.ORACLE, vy, incy, ta, 2.0, va, rows, cols, lda, vx, incx, 0.25)
     np.testing.assert_allclose(bufs[0].host, want, rtol=1e-13, atol=1e-13)
+
+
+# ------------------------------------------------------------------ pooling against a windowed numpy restatement
+
+POOL_GEOMETRIES = [(7, 9, 3, 3, 1, 1, 2, 2, 4, 5), (8, 8, 2, 2, 0, 0, 2, 2, 4, 4), (6, 5, 3, 2, 1, 1, 1, 2, 4, 5),
+                   (9, 9, 2, 2, 1, 1, 1, 1, 10, 10)]
+
+
+def _windows(h, w, kw, kh, px, py, sx, sy, oh, ow):
+    """Per output position: the list of (y, x, inside-the-input) taps within the padded input."""
+    for oy in range(oh):
+        for ox in range(ow):
+            taps = []
+            for ky in range(kh):
+                for kx in range(kw):
+                    y, x = oy * sy - py + ky, ox * sx - px + kx
+                    if -py <= y < h + py and -px <= x < w + px:
+                        taps.append((y, x, 0 <= y < h and 0 <= x < w))
+            yield oy, ox, taps
+
+
+@pytest.mark.parametrize("geometry", POOL_GEOMETRIES, ids=str)
+def test_pooling_matches_windowed_numpy(geometry):
+    h, w, kw, kh, px, py, sx, sy, oh, ow = geometry
+    rng = np.random.default_rng(60)
+    planes = 3
+    x = rng.standard_normal((planes, h, w))
+    og = rng.standard_normal((planes, oh, ow))
+    for op in capi.POOL_OPS:
+        want = np.zeros((planes, oh, ow))
+        want_ig = np.zeros((planes, h, w))
+        for p in range(planes):
+            for oy, ox, taps in _windows(h, w, kw, kh, px, py, sx, sy, oh, ow):
+                vals = [x[p, y, xx] if inside else 0.0 for y, xx, inside in taps]
+                inside_taps = [(y, xx) for y, xx, inside in taps if inside]
+                if op == "max":
+                    want[p, oy, ox] = max(vals)
+                    for y, xx in inside_taps:
+                        if x[p, y, xx] == want[p, oy, ox]:
+                            want_ig[p, y, xx] += og[p, oy, ox]
+                else:
+                    count = kw * kh if op == "avg" else len(inside_taps)
+                    want[p, oy, ox] = sum(vals) / count
+                    for y, xx in inside_taps:
+                        want_ig[p, y, xx] += og[p, oy, ox] / count
+        inp, out = hbuf(x.reshape(-1)), hbuf(np.zeros(planes * oh * ow))
+        grad, ig = hbuf(og.reshape(-1)), hbuf(np.zeros(planes * h * w))
+        desc = H.pool_desc(kw, kh, px, py, sx, sy, op)
+        H.pooling_forward(ORACLE, View(out, [out.host.size]), View(inp, [inp.host.size]), desc, 1, planes, h, w, oh, ow)
+        np.testing.assert_allclose(out.host.reshape(want.shape), want, rtol=1e-12, atol=1e-14, err_msg=op)
+        H.pooling_backward(ORACLE, View(ig, [ig.host.size]), View(inp, [inp.host.size]), View(out, [out.host.size]),
+                           View(grad, [grad.host.size]), desc, 1, planes, h, w, oh, ow)
+        np.testing.assert_allclose(ig.host.reshape(want_ig.shape), want_ig, rtol=1e-12, atol=1e-14, err_msg=op)
+
+
+def test_average_pooling_backward_is_the_adjoint_of_forward():
+    """<forward(x), g> = <x, backward(g)> for the two averages, which are linear maps."""
+    h, w, kw, kh, px, py, sx, sy, oh, ow = 11, 13, 3, 3, 1, 1, 2, 2, 6, 7
+    rng = np.random.default_rng(61)
+    x, g = rng.standard_normal(2 * h * w), rng.standard_normal(2 * oh * ow)
+    for op in ("avg", "avg-exc-pad"):
+        inp, out, grad, ig = hbuf(x), hbuf(np.zeros(2 * oh * ow)), hbuf(g), hbuf(np.zeros(2 * h * w))
+        desc = H.pool_desc(kw, kh, px, py, sx, sy, op)
+        H.pooling_forward(ORACLE, View(out, [out.host.size]), View(inp, [x.size]), desc, 2, 1, h, w, oh, ow)
+        H.pooling_backward(ORACLE, View(ig, [x.size]), View(inp, [x.size]), View(out, [g.size]), View(grad, [g.size]),
+                           desc, 2, 1, h, w, oh, ow)
+        assert abs(np.dot(out.host, g) - np.dot(x, ig.host)) < 1e-10
