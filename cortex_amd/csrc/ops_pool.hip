@@ -24,6 +24,25 @@
 // its gradient) plus the smaller pooled one: HBM-bound.  A launch covers at most
 // 2^31 - 1 elements of either tensor so that all index arithmetic is 32-bit with
 // multiply-high divisions; the host walks larger batches in several launches.
+//
+// Two kernel families.  The band kernels give a block a band of destination
+// rows of one plane (or several whole planes when they are small): the rows of
+// the other tensor that the band touches are one contiguous piece of memory,
+// which the block copies into LDS with aligned 16-byte loads, and the windows
+// are then read out of LDS, so that global memory sees only linear streams.  The
+// direct kernels read the windows from global memory, one lane per destination
+// element, and serve rows too long for the LDS budget.
+//
+// Division.  The averages divide every tap by an integer count d and round the
+// quotient to double before the addition.  For float tensors and d <= 255 the
+// quotient is computed as q = a * y, r = fma(-d, q, a), q' = fma(r, y, q) with
+// y = RN(1 / d): r is exact (a has 24 significant bits, d * q at most 8 + 53, and
+// the difference is below 2^9 ulp(q)), so a / d = q + r / d exactly and
+// q + r * y differs from it by less than 2^-50 ulp(q); a / d cannot lie that close
+// to a rounding boundary m of doubles without being m, because a - m * d is a
+// multiple of ulp(q) / 2, and it cannot be m, because m * d has at least 54
+// significant bits and a has 24.  So q' = RN(a / d), the value the JVM computes;
+// zeros, infinities and NaN take q itself.  Doubles and larger windows divide.
 #include <algorithm>
 
 #include "common.h"
@@ -128,6 +147,194 @@ __global__ void __launch_bounds__(kBlock) pool_backward_kernel(const PoolArgs a)
   ig[e] = acc;
 }
 
+// ------------------------------------------------------------------ band kernels
+
+struct BandArgs {
+  const void* in;
+  const void* out_values;
+  const void* out_grad;
+  void* dest;
+  int32_t in_h, in_w, out_h, out_w;
+  int32_t kw, kh, px, py, sx, sy;
+  uint32_t in_plane, out_plane;
+  uint32_t planes;     // of this launch
+  uint32_t pb;         // planes per block; above 1 a block takes whole planes
+  uint32_t br;         // destination rows per band
+  uint32_t bands;      // bands per plane
+  uint32_t cap;        // LDS elements per staged array
+  uint32_t load_prev;
+  uint32_t fast_div;   // float tensor and kw * kh <= kRecipTable - 1
+  double recip;        // RN(1 / (kw * kh))
+  FastDiv bands_fd, dest_w_fd, dest_plane_fd, sx_fd, sy_fd;
+};
+
+constexpr int kRecipTable = 256;
+
+struct alignas(16) Bytes16 { uint32_t w[4]; };
+
+// Copies src[0, len) to tile[lead, lead + len), where lead is the distance of
+// src from the 16-byte boundary below it, so that both sides of every full
+// vector are aligned.  Returns lead.
+template <class T>
+__device__ __forceinline__ uint32_t stage_linear(T* tile, const T* src, uint32_t len) {
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  const uint32_t lead = (uint32_t)((reinterpret_cast<uintptr_t>(src) / sizeof(T)) % VEC);
+  const T* base = src - lead;
+  const uint32_t end = lead + len;
+  const uint32_t nvec = (end + VEC - 1) / VEC;
+  for (uint32_t v = threadIdx.x; v < nvec; v += kBlock) {
+    const uint32_t i0 = v * VEC;
+    if (i0 >= lead && i0 + VEC <= end) {
+      *reinterpret_cast<Bytes16*>(tile + i0) = *reinterpret_cast<const Bytes16*>(base + i0);
+    } else {
+#pragma unroll
+      for (uint32_t e = 0; e < VEC; ++e)
+        if (i0 + e >= lead && i0 + e < end) tile[i0 + e] = base[i0 + e];
+    }
+  }
+  return lead;
+}
+
+// RN(a / d) for a float a and an integer 1 <= d <= 255 with y = RN(1 / d).
+__device__ __forceinline__ double quotient_by_reciprocal(double a, double d, double y) {
+  const double q = a * y;
+  const double r = fma(-d, q, a);
+  const double q2 = fma(r, y, q);
+  return (r == 0.0 || !(fabs(q) < __builtin_huge_val())) ? q : q2;
+}
+
+template <class T>
+__device__ __forceinline__ double tap_quotient(T v, double d, double y, bool fast) {
+  if (sizeof(T) == 4 && fast) return quotient_by_reciprocal((double)v, d, y);
+  return (double)v / d;
+}
+
+template <class T, int OP, int KW, int KH>
+__global__ void __launch_bounds__(kBlock) pool_forward_band_kernel(const BandArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* tile = reinterpret_cast<T*>(smem);
+  double* recips = reinterpret_cast<double*>(smem + (size_t)a.cap * sizeof(T));
+  const int32_t kw = KW ? KW : a.kw, kh = KH ? KH : a.kh;
+  uint32_t group, band;
+  a.bands_fd.divmod(blockIdx.x, group, band);
+  const uint32_t p0 = group * a.pb, np = min(a.pb, a.planes - p0);
+  const int32_t oy0 = (int32_t)(band * a.br), rows = min((int32_t)a.br, a.out_h - oy0);
+  int32_t iy_lo = 0, n_src_rows = a.in_h;
+  if (a.pb == 1) {
+    iy_lo = max(0, oy0 * a.sy - a.py);
+    n_src_rows = max(0, min(a.in_h, (oy0 + rows - 1) * a.sy - a.py + kh) - iy_lo);
+  }
+  const uint32_t len = a.pb > 1 ? np * a.in_plane : (uint32_t)(n_src_rows * a.in_w);
+  const T* src = reinterpret_cast<const T*>(a.in) + (int64_t)p0 * a.in_plane + (int64_t)iy_lo * a.in_w;
+  const uint32_t lead = stage_linear(tile, src, len);
+  if (OP == CT_POOL_AVG_EXC_PAD && a.fast_div)
+    for (int32_t i = threadIdx.x; i <= kw * kh; i += kBlock) recips[i] = 1.0 / (double)i;
+  __syncthreads();
+  const uint32_t n_dest = np * (uint32_t)(rows * a.out_w);
+  T* out = reinterpret_cast<T*>(a.dest) + (int64_t)p0 * a.out_plane + (int64_t)oy0 * a.out_w;
+  const double kernel_count = (double)(kw * kh);
+  for (uint32_t o = threadIdx.x; o < n_dest; o += kBlock) {
+    uint32_t j = 0, rr = o, oyl, ox;
+    if (a.pb > 1) a.dest_plane_fd.divmod(o, j, rr);
+    a.dest_w_fd.divmod(rr, oyl, ox);
+    const int32_t rel_x = (int32_t)ox * a.sx - a.px, rel_y = (oy0 + (int32_t)oyl) * a.sy - a.py;
+    const int32_t plane_at = (int32_t)(lead + j * a.in_plane) - iy_lo * a.in_w;
+    T acc = (OP == CT_POOL_AVG_EXC_PAD || a.load_prev) ? out[o] : (T)0;
+    double divisor = kernel_count, y = a.recip;
+    if (OP == CT_POOL_AVG_EXC_PAD) {
+      const int32_t inside = taps_inside(rel_x, kw, a.in_w) * taps_inside(rel_y, kh, a.in_h);
+      divisor = (double)inside;
+      if (a.fast_div) y = recips[inside];
+    }
+#pragma unroll
+    for (int32_t ky = 0; ky < kh; ++ky) {
+      const int32_t iy = rel_y + ky;
+      const bool row_reached = iy < a.in_h + a.py;
+      const bool row_inside = iy >= 0 && iy < a.in_h;
+#pragma unroll
+      for (int32_t kx = 0; kx < kw; ++kx) {
+        const int32_t ix = rel_x + kx;
+        if (row_reached && ix < a.in_w + a.px) {
+          const T v = (row_inside && ix >= 0 && ix < a.in_w) ? tile[plane_at + iy * a.in_w + ix] : (T)0;
+          const bool first = (ky | kx) == 0;
+          if (OP == CT_POOL_MAX) {
+            if (first || v > acc) acc = v;
+          } else if (OP == CT_POOL_AVG) {
+            acc = (T)((double)(first ? (T)0 : acc) + tap_quotient(v, divisor, y, a.fast_div));
+          } else {
+            acc = (T)((double)acc + tap_quotient(v, divisor, y, a.fast_div));
+          }
+        }
+      }
+    }
+    out[o] = acc;
+  }
+}
+
+template <class T, int OP, int KW, int KH>
+__global__ void __launch_bounds__(kBlock) pool_backward_band_kernel(const BandArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* tile_v = reinterpret_cast<T*>(smem);
+  T* tile_g = tile_v + a.cap;
+  double* recips = reinterpret_cast<double*>(smem + (size_t)2 * a.cap * sizeof(T));
+  const int32_t kw = KW ? KW : a.kw, kh = KH ? KH : a.kh;
+  uint32_t group, band;
+  a.bands_fd.divmod(blockIdx.x, group, band);
+  const uint32_t p0 = group * a.pb, np = min(a.pb, a.planes - p0);
+  const int32_t iy0 = (int32_t)(band * a.br), rows = min((int32_t)a.br, a.in_h - iy0);
+  int32_t oy_first = 0, n_src_rows = a.out_h;
+  if (a.pb == 1) {
+    const int32_t t = iy0 + a.py - kh + 1;
+    oy_first = t <= 0 ? 0 : min(a.out_h, (int32_t)a.sy_fd.div((uint32_t)(t + a.sy - 1)));
+    const int32_t oy_end = min(a.out_h, (int32_t)a.sy_fd.div((uint32_t)(iy0 + rows - 1 + a.py)) + 1);
+    n_src_rows = max(0, oy_end - oy_first);
+  }
+  const uint32_t len = a.pb > 1 ? np * a.out_plane : (uint32_t)(n_src_rows * a.out_w);
+  const int64_t src_at = (int64_t)p0 * a.out_plane + (int64_t)oy_first * a.out_w;
+  uint32_t lead_v = 0;
+  if (OP == CT_POOL_MAX) lead_v = stage_linear(tile_v, reinterpret_cast<const T*>(a.out_values) + src_at, len);
+  const uint32_t lead_g = stage_linear(tile_g, reinterpret_cast<const T*>(a.out_grad) + src_at, len);
+  if (OP == CT_POOL_AVG_EXC_PAD && a.fast_div)
+    for (int32_t i = threadIdx.x; i <= kw * kh; i += kBlock) recips[i] = 1.0 / (double)i;
+  __syncthreads();
+  const uint32_t n_dest = np * (uint32_t)(rows * a.in_w);
+  const int64_t dest_at = (int64_t)p0 * a.in_plane + (int64_t)iy0 * a.in_w;
+  T* ig = reinterpret_cast<T*>(a.dest) + dest_at;
+  const T* in = reinterpret_cast<const T*>(a.in) + dest_at;
+  const double kernel_count = (double)(kw * kh);
+  for (uint32_t o = threadIdx.x; o < n_dest; o += kBlock) {
+    uint32_t j = 0, rr = o, iyl, ix;
+    if (a.pb > 1) a.dest_plane_fd.divmod(o, j, rr);
+    a.dest_w_fd.divmod(rr, iyl, ix);
+    const int32_t ty = iy0 + (int32_t)iyl + a.py, tx = (int32_t)ix + a.px;
+    const int32_t oy_hi = min(a.out_h - 1, (int32_t)a.sy_fd.div((uint32_t)ty));
+    const int32_t ox_hi = min(a.out_w - 1, (int32_t)a.sx_fd.div((uint32_t)tx));
+    const int32_t by = ty - kh + 1, bx = tx - kw + 1;
+    const int32_t oy_lo = by <= 0 ? 0 : (int32_t)a.sy_fd.div((uint32_t)(by + a.sy - 1));
+    const int32_t ox_lo = bx <= 0 ? 0 : (int32_t)a.sx_fd.div((uint32_t)(bx + a.sx - 1));
+    const int32_t plane_at = (int32_t)(j * a.out_plane) - oy_first * a.out_w;
+    T acc = ig[o];
+    T v = (T)0;
+    if (OP == CT_POOL_MAX) v = in[o];
+    for (int32_t oy = oy_lo; oy <= oy_hi; ++oy) {
+      const int32_t exc_h = taps_inside(oy * a.sy - a.py, kh, a.in_h);
+      for (int32_t ox = ox_lo; ox <= ox_hi; ++ox) {
+        const int32_t at = plane_at + oy * a.out_w + ox;
+        const T g = tile_g[(int32_t)lead_g + at];
+        if (OP == CT_POOL_MAX) {
+          if (v == tile_v[(int32_t)lead_v + at]) acc = acc + g;
+        } else if (OP == CT_POOL_AVG) {
+          acc = (T)((double)acc + tap_quotient(g, kernel_count, a.recip, a.fast_div));
+        } else {
+          const int32_t inside = taps_inside(ox * a.sx - a.px, kw, a.in_w) * exc_h;
+          acc = (T)((double)acc + tap_quotient(g, (double)inside, a.fast_div ? recips[inside] : 0.0, a.fast_div));
+        }
+      }
+    }
+    ig[o] = acc;
+  }
+}
+
 struct PoolShape {
   int64_t planes, in_h, in_w, out_h, out_w;
 };
@@ -161,12 +368,113 @@ int check_pool(const ct_pool_desc* d, int64_t batch_count, int64_t channel_count
   return CT_OK;
 }
 
+// LDS given to the staged rows of a block: eight blocks of this size fit the
+// 160 KiB of a compute unit, which keeps it full of waves.
+constexpr uint32_t kBandLdsBytes = 20 * 1024;
+// Destination elements a block of whole small planes aims for.
+constexpr uint32_t kBandDestTarget = 16 * kBlock;
+
+struct BandPlan {
+  bool usable;
+  uint32_t pb, br, bands;
+};
+
+// Forward: `rows` destination rows read (rows - 1) * stride + k source rows.
+// Backward: `rows` destination (input) rows are covered by at most
+// (rows + k - 2) / stride + 2 source (output) rows.
+BandPlan plan_bands(bool forward, uint32_t budget, int64_t src_plane, int64_t src_w, int64_t dest_plane,
+                    int64_t dest_h, int64_t k, int64_t stride) {
+  BandPlan p{false, 1, 1, 1};
+  if (src_plane <= budget) {
+    p.usable = true;
+    const int64_t by_lds = budget / std::max<int64_t>(1, src_plane);
+    const int64_t by_dest = std::max<int64_t>(1, kBandDestTarget / std::max<int64_t>(1, dest_plane));
+    p.pb = (uint32_t)std::max<int64_t>(1, std::min(by_lds, by_dest));
+    p.br = (uint32_t)dest_h;
+    p.bands = 1;
+    return p;
+  }
+  const int64_t src_rows = budget / std::max<int64_t>(1, src_w);
+  int64_t rows;
+  if (forward) rows = src_rows >= k ? (src_rows - k) / stride + 1 : 0;
+  else rows = (src_rows - 2) * stride - k + 2;
+  if (rows < 1) return p;
+  rows = std::min(rows, dest_h);
+  p.usable = true;
+  p.bands = (uint32_t)((dest_h + rows - 1) / rows);
+  p.br = (uint32_t)((dest_h + p.bands - 1) / p.bands);
+  return p;
+}
+
+template <class T, int OP, int KW, int KH>
+void launch_band(hipStream_t s, bool forward, dim3 grid, size_t lds, const BandArgs& a) {
+  if (forward) hipLaunchKernelGGL((pool_forward_band_kernel<T, OP, KW, KH>), grid, dim3(kBlock), lds, s, a);
+  else hipLaunchKernelGGL((pool_backward_band_kernel<T, OP, KW, KH>), grid, dim3(kBlock), lds, s, a);
+}
+
+template <class T, int OP>
+void launch_band_window(hipStream_t s, bool forward, dim3 grid, size_t lds, const BandArgs& a) {
+  if (a.kw == 2 && a.kh == 2) launch_band<T, OP, 2, 2>(s, forward, grid, lds, a);
+  else if (a.kw == 3 && a.kh == 3) launch_band<T, OP, 3, 3>(s, forward, grid, lds, a);
+  else launch_band<T, OP, 0, 0>(s, forward, grid, lds, a);
+}
+
 template <class T>
 int pool_launch(hipStream_t s, bool forward, void* dest, const void* in, const void* out_values, const void* out_grad,
                 const ct_pool_desc& d, const PoolShape& sh) {
   const int64_t in_plane = sh.in_h * sh.in_w, out_plane = sh.out_h * sh.out_w;
   const int64_t dest_plane = forward ? out_plane : in_plane;
   if (sh.planes == 0 || dest_plane == 0) return CT_OK;
+  // The first tap lies inside the padded input unless the stride carries the
+  // last window past it; then max and avg continue from what the output holds.
+  const bool first_tap_inside = (sh.out_w - 1) * d.stride_x - d.pad_x < sh.in_w + d.pad_x &&
+                                (sh.out_h - 1) * d.stride_y - d.pad_y < sh.in_h + d.pad_y;
+  const int64_t limit = (int64_t(1) << 31) - 1;
+  const int64_t planes_per_launch = std::max<int64_t>(1, limit / std::max<int64_t>(1, std::max(in_plane, out_plane)));
+
+  const uint32_t arrays = forward ? 1u : 2u;
+  const uint32_t budget = kBandLdsBytes / (uint32_t)sizeof(T) / arrays;
+  const BandPlan bp = forward ? plan_bands(true, budget, in_plane, sh.in_w, out_plane, sh.out_h, d.kernel_height,
+                                           d.stride_y)
+                              : plan_bands(false, budget, out_plane, sh.out_w, in_plane, sh.in_h, d.kernel_height,
+                                           d.stride_y);
+  if (bp.usable && (forward ? in_plane : out_plane) > 0) {
+    BandArgs a{};
+    a.in_h = (int32_t)sh.in_h; a.in_w = (int32_t)sh.in_w; a.out_h = (int32_t)sh.out_h; a.out_w = (int32_t)sh.out_w;
+    a.kw = d.kernel_width; a.kh = d.kernel_height; a.px = d.pad_x; a.py = d.pad_y; a.sx = d.stride_x;
+    a.sy = d.stride_y;
+    a.in_plane = (uint32_t)in_plane; a.out_plane = (uint32_t)out_plane;
+    a.pb = bp.pb; a.br = bp.br; a.bands = bp.bands;
+    a.cap = (budget + 8u) / 4u * 4u;
+    a.load_prev = first_tap_inside ? 0u : 1u;
+    const int64_t window = (int64_t)d.kernel_width * d.kernel_height;
+    a.fast_div = (sizeof(T) == 4 && window < kRecipTable) ? 1u : 0u;
+    a.recip = 1.0 / (double)window;
+    a.bands_fd = FastDiv(bp.bands);
+    a.dest_w_fd = FastDiv((uint32_t)(forward ? sh.out_w : sh.in_w));
+    a.dest_plane_fd = FastDiv((uint32_t)dest_plane);
+    a.sx_fd = FastDiv((uint32_t)d.stride_x);
+    a.sy_fd = FastDiv((uint32_t)d.stride_y);
+    const size_t lds = (size_t)arrays * a.cap * sizeof(T) + (size_t)kRecipTable * sizeof(double);
+    note_kernel(forward ? "pool_forward_band" : "pool_backward_band");
+    for (int64_t p0 = 0; p0 < sh.planes; p0 += planes_per_launch) {
+      const int64_t np = std::min(planes_per_launch, sh.planes - p0);
+      a.planes = (uint32_t)np;
+      a.in = reinterpret_cast<const T*>(in) + p0 * in_plane;
+      a.out_values = out_values ? reinterpret_cast<const T*>(out_values) + p0 * out_plane : nullptr;
+      a.out_grad = out_grad ? reinterpret_cast<const T*>(out_grad) + p0 * out_plane : nullptr;
+      a.dest = reinterpret_cast<T*>(dest) + p0 * dest_plane;
+      const int64_t groups = (np + bp.pb - 1) / bp.pb;
+      const dim3 grid((uint32_t)(groups * bp.bands));
+      switch (d.pool_op) {
+        case CT_POOL_MAX: launch_band_window<T, CT_POOL_MAX>(s, forward, grid, lds, a); break;
+        case CT_POOL_AVG: launch_band_window<T, CT_POOL_AVG>(s, forward, grid, lds, a); break;
+        default: launch_band_window<T, CT_POOL_AVG_EXC_PAD>(s, forward, grid, lds, a); break;
+      }
+    }
+    return after_launch(s);
+  }
+
   PoolArgs a{};
   a.in_h = (int32_t)sh.in_h; a.in_w = (int32_t)sh.in_w; a.out_h = (int32_t)sh.out_h; a.out_w = (int32_t)sh.out_w;
   a.kw = d.kernel_width; a.kh = d.kernel_height; a.px = d.pad_x; a.py = d.pad_y; a.sx = d.stride_x; a.sy = d.stride_y;
@@ -175,13 +483,8 @@ int pool_launch(hipStream_t s, bool forward, void* dest, const void* in, const v
   a.row_fd = FastDiv((uint32_t)(forward ? sh.out_w : sh.in_w));
   a.sx_fd = FastDiv((uint32_t)d.stride_x);
   a.sy_fd = FastDiv((uint32_t)d.stride_y);
-  // The first tap lies inside the padded input unless the stride carries the
-  // last window past it; then max and avg continue from what the output holds.
-  const bool first_tap_inside = (sh.out_w - 1) * d.stride_x - d.pad_x < sh.in_w + d.pad_x &&
-                                (sh.out_h - 1) * d.stride_y - d.pad_y < sh.in_h + d.pad_y;
   a.load_prev = first_tap_inside ? 0u : 1u;
-  const int64_t limit = (int64_t(1) << 31) - 1;
-  const int64_t planes_per_launch = std::max<int64_t>(1, limit / std::max<int64_t>(1, std::max(in_plane, out_plane)));
+  note_kernel(forward ? "pool_forward" : "pool_backward");
   for (int64_t p0 = 0; p0 < sh.planes; p0 += planes_per_launch) {
     const int64_t np = std::min(planes_per_launch, sh.planes - p0);
     a.total = (uint32_t)(np * dest_plane);
@@ -214,7 +517,6 @@ int ct_pooling_forward(void* stream, void* output, double /*output_alpha*/, cons
     return rc;
   if (sh.planes * sh.out_h * sh.out_w == 0) return CT_OK;
   CT_REQUIRE(output != nullptr && (input != nullptr || sh.in_h * sh.in_w == 0), "pooling-forward!: null buffer");
-  note_kernel("pool_forward");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == CT_F32) return pool_launch<float>(s, true, output, input, nullptr, nullptr, *desc, sh);
   return pool_launch<double>(s, true, output, input, nullptr, nullptr, *desc, sh);
@@ -230,7 +532,6 @@ int ct_pooling_backward(void* stream, void* input_gradient, double /*input_gradi
   if (sh.planes * sh.in_h * sh.in_w == 0 || sh.out_h * sh.out_w == 0) return CT_OK;
   CT_REQUIRE(input_gradient != nullptr && input != nullptr && output != nullptr && output_gradient != nullptr,
              "pooling-backward!: null buffer");
-  note_kernel("pool_backward");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == CT_F32) return pool_launch<float>(s, false, input_gradient, input, output, output_gradient, *desc, sh);
   return pool_launch<double>(s, false, input_gradient, input, output, output_gradient, *desc, sh);

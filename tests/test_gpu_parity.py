@@ -837,6 +837,13 @@ POOL_CASES = [
     (1, 1, 5, 7, 7, 5, 3, 2, 1, 1, "floor"),       # window as large as the image
     (4, 8, 56, 56, 3, 3, 1, 1, 2, 2, "floor"),
     (1, 1, 1, 1, 1, 1, 0, 0, 1, 1, "floor"),
+    (2, 3, 120, 100, 3, 3, 1, 1, 2, 2, "floor"),   # planes beyond the LDS budget: bands of rows
+    (1, 2, 131, 97, 3, 3, 1, 1, 2, 2, "ceil"),
+    (2, 2, 90, 90, 2, 2, 0, 0, 2, 2, "floor"),
+    (1, 3, 75, 110, 3, 3, 1, 1, 1, 1, "floor"),
+    (1, 2, 100, 70, 5, 4, 2, 1, 2, 3, "ceil"),
+    (1, 1, 9, 2000, 3, 3, 1, 1, 2, 2, "floor"),    # rows beyond it: the direct kernels
+    (1, 1, 40, 300, 17, 17, 8, 8, 1, 1, "floor"),  # a window too large for the reciprocal table
 ]
 
 
@@ -862,10 +869,10 @@ def test_pooling_bit_exact(P, code, op, case):
     desc = H.pool_desc(kw, kh, px, py, sx, sy, op)
     geom = (desc, batch, channels, h, w, oh, ow)
     k = P.run(H.pooling_forward, View(out, [n_out]), View(inp, [n_in]), *geom)
-    assert k == "pool_forward"
+    assert k.startswith("pool_forward")
     compare(out, f"pooling-forward {op} {case}")
     k = P.run(H.pooling_backward, View(ig, [n_in]), View(inp, [n_in]), View(out, [n_out]), View(og, [n_out]), *geom)
-    assert k == "pool_backward"
+    assert k.startswith("pool_backward")
     compare(ig, f"pooling-backward {op} {case}")
 
 
