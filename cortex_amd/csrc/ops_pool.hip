@@ -200,7 +200,9 @@ __device__ __forceinline__ double quotient_by_reciprocal(double a, double d, dou
   const double q = a * y;
   const double r = fma(-d, q, a);
   const double q2 = fma(r, y, q);
-  return (r == 0.0 || !(fabs(q) < __builtin_huge_val())) ? q : q2;
+  // zeros (whose sign the correction would lose), infinities and NaN: q is the quotient
+  constexpr int kZeroInfNan = 0x001 | 0x002 | 0x004 | 0x020 | 0x040 | 0x200;
+  return __builtin_amdgcn_class(a, kZeroInfNan) ? q : q2;
 }
 
 template <class T>
@@ -246,15 +248,43 @@ __global__ void __launch_bounds__(kBlock) pool_forward_band_kernel(const BandArg
       divisor = (double)inside;
       if (a.fast_div) y = recips[inside];
     }
+    if constexpr (KW > 0) {
+      // Fixed window: no branches.  Every tap is read (from LDS index 0 when it
+      // lies outside the input) and takes part by selects.
+      bool col_inside[KW], col_reached[KW];
 #pragma unroll
-    for (int32_t ky = 0; ky < kh; ++ky) {
-      const int32_t iy = rel_y + ky;
-      const bool row_reached = iy < a.in_h + a.py;
-      const bool row_inside = iy >= 0 && iy < a.in_h;
+      for (int32_t kx = 0; kx < KW; ++kx) {
+        col_inside[kx] = (uint32_t)(rel_x + kx) < (uint32_t)a.in_w;
+        col_reached[kx] = rel_x + kx < a.in_w + a.px;
+      }
 #pragma unroll
-      for (int32_t kx = 0; kx < kw; ++kx) {
-        const int32_t ix = rel_x + kx;
-        if (row_reached && ix < a.in_w + a.px) {
+      for (int32_t ky = 0; ky < KH; ++ky) {
+        const int32_t iy = rel_y + ky;
+        const bool row_reached = iy < a.in_h + a.py;
+        const bool row_inside = (uint32_t)iy < (uint32_t)a.in_h;
+        const int32_t row_at = plane_at + iy * a.in_w + rel_x;
+#pragma unroll
+        for (int32_t kx = 0; kx < KW; ++kx) {
+          const bool inside = row_inside && col_inside[kx];
+          const bool reached = row_reached && col_reached[kx];
+          const T read = tile[inside ? row_at + kx : 0];
+          const T v = inside ? read : (T)0;
+          const bool first = (ky | kx) == 0;
+          T next;
+          if (OP == CT_POOL_MAX) next = (first || v > acc) ? v : acc;
+          else if (OP == CT_POOL_AVG) next = (T)((double)(first ? (T)0 : acc) + tap_quotient(v, divisor, y, a.fast_div));
+          else next = (T)((double)acc + tap_quotient(v, divisor, y, a.fast_div));
+          acc = reached ? next : acc;
+        }
+      }
+    } else {
+      for (int32_t ky = 0; ky < kh; ++ky) {
+        const int32_t iy = rel_y + ky;
+        if (iy >= a.in_h + a.py) break;
+        const bool row_inside = iy >= 0 && iy < a.in_h;
+        for (int32_t kx = 0; kx < kw; ++kx) {
+          const int32_t ix = rel_x + kx;
+          if (ix >= a.in_w + a.px) break;
           const T v = (row_inside && ix >= 0 && ix < a.in_w) ? tile[plane_at + iy * a.in_w + ix] : (T)0;
           const bool first = (ky | kx) == 0;
           if (OP == CT_POOL_MAX) {
@@ -302,10 +332,9 @@ __global__ void __launch_bounds__(kBlock) pool_backward_band_kernel(const BandAr
   T* ig = reinterpret_cast<T*>(a.dest) + dest_at;
   const T* in = reinterpret_cast<const T*>(a.in) + dest_at;
   const double kernel_count = (double)(kw * kh);
-  for (uint32_t o = threadIdx.x; o < n_dest; o += kBlock) {
-    uint32_t j = 0, rr = o, iyl, ix;
-    if (a.pb > 1) a.dest_plane_fd.divmod(o, j, rr);
-    a.dest_w_fd.divmod(rr, iyl, ix);
+  // The input gradient at row iyl of the band, column ix of plane j of the block.
+  auto gather = [&](uint32_t j, uint32_t iyl, uint32_t ix, T acc, T v) -> T {
+    // Windows o with o * stride - pad <= i < o * stride - pad + k.
     const int32_t ty = iy0 + (int32_t)iyl + a.py, tx = (int32_t)ix + a.px;
     const int32_t oy_hi = min(a.out_h - 1, (int32_t)a.sy_fd.div((uint32_t)ty));
     const int32_t ox_hi = min(a.out_w - 1, (int32_t)a.sx_fd.div((uint32_t)tx));
@@ -313,9 +342,6 @@ __global__ void __launch_bounds__(kBlock) pool_backward_band_kernel(const BandAr
     const int32_t oy_lo = by <= 0 ? 0 : (int32_t)a.sy_fd.div((uint32_t)(by + a.sy - 1));
     const int32_t ox_lo = bx <= 0 ? 0 : (int32_t)a.sx_fd.div((uint32_t)(bx + a.sx - 1));
     const int32_t plane_at = (int32_t)(j * a.out_plane) - oy_first * a.out_w;
-    T acc = ig[o];
-    T v = (T)0;
-    if (OP == CT_POOL_MAX) v = in[o];
     for (int32_t oy = oy_lo; oy <= oy_hi; ++oy) {
       const int32_t exc_h = taps_inside(oy * a.sy - a.py, kh, a.in_h);
       for (int32_t ox = ox_lo; ox <= ox_hi; ++ox) {
@@ -331,8 +357,126 @@ __global__ void __launch_bounds__(kBlock) pool_backward_band_kernel(const BandAr
         }
       }
     }
-    ig[o] = acc;
+    return acc;
+  };
+  // 16-byte pieces of the gradient (and of the input, for max) when the band
+  // starts on a 16-byte boundary of both; the remainder one element at a time.
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  struct alignas(16) Piece { T v[VEC]; };
+  const bool pieces = reinterpret_cast<uintptr_t>(ig) % 16 == 0 &&
+                      (OP != CT_POOL_MAX || reinterpret_cast<uintptr_t>(in) % 16 == 0);
+  const uint32_t n_pieces = pieces ? n_dest / VEC : 0;
+  for (uint32_t q = threadIdx.x; q < n_pieces; q += kBlock) {
+    const uint32_t o = q * VEC;
+    uint32_t j = 0, rr = o, iyl, ix;
+    if (a.pb > 1) a.dest_plane_fd.divmod(o, j, rr);
+    a.dest_w_fd.divmod(rr, iyl, ix);
+    Piece acc = *reinterpret_cast<const Piece*>(ig + o);
+    Piece vin;
+    if (OP == CT_POOL_MAX) vin = *reinterpret_cast<const Piece*>(in + o);
+#pragma unroll
+    for (uint32_t e = 0; e < VEC; ++e) {
+      acc.v[e] = gather(j, iyl, ix, acc.v[e], OP == CT_POOL_MAX ? vin.v[e] : (T)0);
+      if (++ix == (uint32_t)a.in_w) {
+        ix = 0;
+        if (++iyl == (uint32_t)rows) { iyl = 0; ++j; }
+      }
+    }
+    *reinterpret_cast<Piece*>(ig + o) = acc;
   }
+  for (uint32_t o = n_pieces * VEC + threadIdx.x; o < n_dest; o += kBlock) {
+    uint32_t j = 0, rr = o, iyl, ix;
+    if (a.pb > 1) a.dest_plane_fd.divmod(o, j, rr);
+    a.dest_w_fd.divmod(rr, iyl, ix);
+    ig[o] = gather(j, iyl, ix, ig[o], OP == CT_POOL_MAX ? in[o] : (T)0);
+  }
+}
+
+// ------------------------------------------------------------------ 2 x 2 windows that tile the input
+
+// kernel 2 x 2, stride 2, no padding, in_h = 2 * out_h, in_w = 2 * out_w, in_w a
+// multiple of 4: every input lies under exactly one window and global output
+// row R reads input rows 2 R and 2 R + 1 whatever the plane, so a lane takes two
+// neighbouring windows as 16-byte (float) pieces of the two rows.  No LDS, no
+// plane arithmetic, every access a full aligned vector.
+struct Tile2Args {
+  const void* in;
+  const void* out_values;
+  const void* out_grad;
+  void* dest;
+  uint32_t total;  // pairs of windows in this launch
+  uint32_t in_w, out_w;
+  FastDiv pairs_fd;  // pairs per output row
+};
+
+template <class T, int N>
+struct alignas(N * sizeof(T) >= 16 ? 16 : N * sizeof(T)) Run { T v[N]; };
+
+template <class T, int OP>
+__device__ __forceinline__ T tile2_forward(T prev, T t0, T t1, T t2, T t3) {
+  if (OP == CT_POOL_MAX) {
+    T acc = t0;
+    if (t1 > acc) acc = t1;
+    if (t2 > acc) acc = t2;
+    if (t3 > acc) acc = t3;
+    return acc;
+  }
+  // a quarter is exact in double, so the multiplication is the division
+  T acc = OP == CT_POOL_AVG ? (T)0 : prev;
+  acc = (T)((double)acc + (double)t0 * 0.25);
+  acc = (T)((double)acc + (double)t1 * 0.25);
+  acc = (T)((double)acc + (double)t2 * 0.25);
+  acc = (T)((double)acc + (double)t3 * 0.25);
+  return acc;
+}
+
+template <class T, int OP>
+__device__ __forceinline__ T tile2_backward(T grad_in, T x, T pooled, T grad_out) {
+  if (OP == CT_POOL_MAX) return x == pooled ? grad_in + grad_out : grad_in;
+  return (T)((double)grad_in + (double)grad_out * 0.25);
+}
+
+template <class T, int OP>
+__global__ void __launch_bounds__(kBlock) pool_tile2_forward_kernel(const Tile2Args a) {
+  const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= a.total) return;
+  uint32_t row, pair;
+  a.pairs_fd.divmod(idx, row, pair);
+  const T* top = reinterpret_cast<const T*>(a.in) + (int64_t)row * 2 * a.in_w + pair * 4;
+  const Run<T, 4> r0 = *reinterpret_cast<const Run<T, 4>*>(top);
+  const Run<T, 4> r1 = *reinterpret_cast<const Run<T, 4>*>(top + a.in_w);
+  Run<T, 2>* out = reinterpret_cast<Run<T, 2>*>(reinterpret_cast<T*>(a.dest) + (int64_t)row * a.out_w + pair * 2);
+  Run<T, 2> o;
+  if (OP == CT_POOL_AVG_EXC_PAD) o = *out;
+  o.v[0] = tile2_forward<T, OP>(o.v[0], r0.v[0], r0.v[1], r1.v[0], r1.v[1]);
+  o.v[1] = tile2_forward<T, OP>(o.v[1], r0.v[2], r0.v[3], r1.v[2], r1.v[3]);
+  *out = o;
+}
+
+template <class T, int OP>
+__global__ void __launch_bounds__(kBlock) pool_tile2_backward_kernel(const Tile2Args a) {
+  const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= a.total) return;
+  uint32_t row, pair;
+  a.pairs_fd.divmod(idx, row, pair);
+  const int64_t in_at = (int64_t)row * 2 * a.in_w + pair * 4, out_at = (int64_t)row * a.out_w + pair * 2;
+  Run<T, 4>* g0 = reinterpret_cast<Run<T, 4>*>(reinterpret_cast<T*>(a.dest) + in_at);
+  Run<T, 4>* g1 = reinterpret_cast<Run<T, 4>*>(reinterpret_cast<T*>(a.dest) + in_at + a.in_w);
+  Run<T, 4> ig0 = *g0, ig1 = *g1, x0{}, x1{};
+  Run<T, 2> pooled{};
+  if (OP == CT_POOL_MAX) {
+    x0 = *reinterpret_cast<const Run<T, 4>*>(reinterpret_cast<const T*>(a.in) + in_at);
+    x1 = *reinterpret_cast<const Run<T, 4>*>(reinterpret_cast<const T*>(a.in) + in_at + a.in_w);
+    pooled = *reinterpret_cast<const Run<T, 2>*>(reinterpret_cast<const T*>(a.out_values) + out_at);
+  }
+  const Run<T, 2> og = *reinterpret_cast<const Run<T, 2>*>(reinterpret_cast<const T*>(a.out_grad) + out_at);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    ig0.v[c] = tile2_backward<T, OP>(ig0.v[c], x0.v[c], pooled.v[c / 2], og.v[c / 2]);
+    ig1.v[c] = tile2_backward<T, OP>(ig1.v[c], x1.v[c], pooled.v[c / 2], og.v[c / 2]);
+  }
+  *g0 = ig0;
+  *g1 = ig1;
 }
 
 struct PoolShape {
@@ -368,9 +512,12 @@ int check_pool(const ct_pool_desc* d, int64_t batch_count, int64_t channel_count
   return CT_OK;
 }
 
-// LDS given to the staged rows of a block: eight blocks of this size fit the
-// 160 KiB of a compute unit, which keeps it full of waves.
-constexpr uint32_t kBandLdsBytes = 20 * 1024;
+// LDS given to the staged rows of a block.  The kernels are bound by latency and
+// instruction issue, so the waves a compute unit holds matter more than the
+// length of a band: measured on [64, 64, 224, 224] float, 3 x 3 stride 2, the
+// forward max pass reads and writes at 53 / 57 / 52 / 41 / 34 % of the HBM peak
+// with 8 / 12 / 20 / 32 / 48 KiB.
+constexpr uint32_t kBandLdsBytes = 12 * 1024;
 // Destination elements a block of whole small planes aims for.
 constexpr uint32_t kBandDestTarget = 16 * kBlock;
 
@@ -431,6 +578,37 @@ int pool_launch(hipStream_t s, bool forward, void* dest, const void* in, const v
                                 (sh.out_h - 1) * d.stride_y - d.pad_y < sh.in_h + d.pad_y;
   const int64_t limit = (int64_t(1) << 31) - 1;
   const int64_t planes_per_launch = std::max<int64_t>(1, limit / std::max<int64_t>(1, std::max(in_plane, out_plane)));
+
+  auto aligned16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool tiles2 = d.kernel_width == 2 && d.kernel_height == 2 && d.stride_x == 2 && d.stride_y == 2 &&
+                      d.pad_x == 0 && d.pad_y == 0 && sh.in_w == 2 * sh.out_w && sh.in_h == 2 * sh.out_h &&
+                      sh.in_w % 4 == 0 && aligned16(dest) && aligned16(in) && aligned16(out_values) &&
+                      aligned16(out_grad);
+  if (tiles2) {
+    Tile2Args a{};
+    a.in_w = (uint32_t)sh.in_w; a.out_w = (uint32_t)sh.out_w;
+    const int64_t pairs = sh.out_w / 2;
+    a.pairs_fd = FastDiv((uint32_t)pairs);
+    note_kernel(forward ? "pool_forward_tile2" : "pool_backward_tile2");
+    for (int64_t p0 = 0; p0 < sh.planes; p0 += planes_per_launch) {
+      const int64_t np = std::min(planes_per_launch, sh.planes - p0);
+      a.total = (uint32_t)(np * sh.out_h * pairs);
+      a.in = reinterpret_cast<const T*>(in) + p0 * in_plane;
+      a.out_values = out_values ? reinterpret_cast<const T*>(out_values) + p0 * out_plane : nullptr;
+      a.out_grad = out_grad ? reinterpret_cast<const T*>(out_grad) + p0 * out_plane : nullptr;
+      a.dest = reinterpret_cast<T*>(dest) + p0 * dest_plane;
+      const dim3 grid((a.total + kBlock - 1) / kBlock);
+#define CT_POOL(KERNEL)                                                                                       \
+  switch (d.pool_op) {                                                                                        \
+    case CT_POOL_MAX: hipLaunchKernelGGL((KERNEL<T, CT_POOL_MAX>), grid, dim3(kBlock), 0, s, a); break;       \
+    case CT_POOL_AVG: hipLaunchKernelGGL((KERNEL<T, CT_POOL_AVG>), grid, dim3(kBlock), 0, s, a); break;       \
+    default: hipLaunchKernelGGL((KERNEL<T, CT_POOL_AVG_EXC_PAD>), grid, dim3(kBlock), 0, s, a); break;        \
+  }
+      if (forward) { CT_POOL(pool_tile2_forward_kernel) } else { CT_POOL(pool_tile2_backward_kernel) }
+#undef CT_POOL
+    }
+    return after_launch(s);
+  }
 
   const uint32_t arrays = forward ? 1u : 2u;
   const uint32_t budget = kBandLdsBytes / (uint32_t)sizeof(T) / arrays;
