@@ -237,6 +237,24 @@ def run_adjacent(drv, device, stream, timer, capi) -> dict:
         o, st[6], st[7], g, o, x, st[0], st[1], st[2], st[3], 1e-3, b, c, e), 20)
     out[f"batch-normalize-gradients! spatial f32 [{b},{c},{e}]"] = entry(12 * nn_, ms, hbm_bytes_moved=20 * nn_)
 
+    # pooling: algorithmic bytes = input + output forward; gradient read and written, output gradient
+    # (and, for max, input and output) backward
+    pb, pc, ph = 32, 64, 256
+    po = ph // 2
+    in_dims, out_dims = dims([pb, pc, ph, ph]), dims([pb, pc, po, po])
+    n_out = pb * pc * po * po
+    ig = device.allocate_device_buffer(n, "float")
+    stream.memset(ig, 0, 0.0, n)
+    for kernel, pad, pool_op in ((2, 0, "max"), (3, 1, "max"), (3, 1, "avg")):
+        desc = {"kernel-width": kernel, "kernel-height": kernel, "pad-x": pad, "pad-y": pad, "stride-x": 2,
+                "stride-y": 2, "pool-op": pool_op}
+        label = f"f32 [{pb},{pc},{ph},{ph}] {kernel}x{kernel} stride 2 :{pool_op}"
+        ms = time_launches(timer, stream, lambda: stream.pooling_forward(o, out_dims, 0.0, x, in_dims, desc), 20)
+        out[f"pooling-forward! {label}"] = entry(4 * (n + n_out), ms)
+        ms = time_launches(timer, stream, lambda: stream.pooling_backward(ig, in_dims, 0.0, x, in_dims, o, out_dims, g,
+                                                                         out_dims, desc), 20)
+        out[f"pooling-backward! {label}"] = entry(4 * (2 * n + n_out) + (4 * (n + n_out) if pool_op == "max" else 0), ms)
+
     # gemm! is the one MFMA-bound method (rocBLAS); priced against the dense fp32 matrix peak
     m = 8192
     a_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))

@@ -398,13 +398,17 @@ __global__ void __launch_bounds__(kBlock) pool_backward_band_kernel(const BandAr
 // multiple of 4: every input lies under exactly one window and global output
 // row R reads input rows 2 R and 2 R + 1 whatever the plane, so a lane takes two
 // neighbouring windows as 16-byte (float) pieces of the two rows.  No LDS, no
-// plane arithmetic, every access a full aligned vector.
+// plane arithmetic, every access a full aligned vector.  Blocks take the die-
+// grouped order of the flat kernels (forward +4 points of the HBM peak, backward
+// +1 to +3 measured); the band kernels, which wait at a barrier between their
+// loads and their arithmetic, measured no gain from it and keep the plain order.
 struct Tile2Args {
   const void* in;
   const void* out_values;
   const void* out_grad;
   void* dest;
   uint32_t total;  // pairs of windows in this launch
+  uint32_t grouped_blocks;
   uint32_t in_w, out_w;
   FastDiv pairs_fd;  // pairs per output row
 };
@@ -438,7 +442,7 @@ __device__ __forceinline__ T tile2_backward(T grad_in, T x, T pooled, T grad_out
 
 template <class T, int OP>
 __global__ void __launch_bounds__(kBlock) pool_tile2_forward_kernel(const Tile2Args a) {
-  const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t idx = xcd_grouped_unit(blockIdx.x, a.grouped_blocks) * kBlock + threadIdx.x;
   if (idx >= a.total) return;
   uint32_t row, pair;
   a.pairs_fd.divmod(idx, row, pair);
@@ -455,7 +459,7 @@ __global__ void __launch_bounds__(kBlock) pool_tile2_forward_kernel(const Tile2A
 
 template <class T, int OP>
 __global__ void __launch_bounds__(kBlock) pool_tile2_backward_kernel(const Tile2Args a) {
-  const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
+  const uint32_t idx = xcd_grouped_unit(blockIdx.x, a.grouped_blocks) * kBlock + threadIdx.x;
   if (idx >= a.total) return;
   uint32_t row, pair;
   a.pairs_fd.divmod(idx, row, pair);
@@ -598,6 +602,7 @@ int pool_launch(hipStream_t s, bool forward, void* dest, const void* in, const v
       a.out_grad = out_grad ? reinterpret_cast<const T*>(out_grad) + p0 * out_plane : nullptr;
       a.dest = reinterpret_cast<T*>(dest) + p0 * dest_plane;
       const dim3 grid((a.total + kBlock - 1) / kBlock);
+      a.grouped_blocks = xcd_grouped_blocks(grid.x);
 #define CT_POOL(KERNEL)                                                                                       \
   switch (d.pool_op) {                                                                                        \
     case CT_POOL_MAX: hipLaunchKernelGGL((KERNEL<T, CT_POOL_MAX>), grid, dim3(kBlock), 0, s, a); break;       \
