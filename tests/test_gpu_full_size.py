@@ -218,3 +218,86 @@ def test_config4_image_normalise_and_int_to_double():
     assert bits_equal(dd.download(), i32.astype(np.float64))
     di.free()
     dd.free()
+
+
+def _pool(forward, desc, geom, *ptrs):
+    d = capi.make_pool_desc(desc)
+    name = "ct_pooling_forward" if forward else "ct_pooling_backward"
+    capi.call(name, None, ptrs[0], 0.0, *ptrs[1:], C.byref(d), *geom, capi.F32)
+    return capi.last_kernel()
+
+
+def test_pooling_at_image_batch_size():
+    """[32, 64, 224, 224] float (411 MB): 2 x 2 stride 2 max against numpy's window maximum and the
+    indicator of the maxima, 3 x 3 pad 1 stride 2 through window-independent properties (an average
+    of a constant image is the constant times the fraction of the window inside it; a 1 x 1 window is
+    a copy), and the two averages' backward passes as adjoints of their forward passes."""
+    batch, channels, h, w = 32, 64, 224, 224
+    planes = batch * channels
+    rng = np.random.default_rng(70)
+    x = rng.standard_normal((planes, h, w), dtype=np.float32)
+    xin = Dev(x)
+
+    # 2 x 2 windows that tile the image
+    oh, ow = h // 2, w // 2
+    desc = {"kernel-width": 2, "kernel-height": 2, "pad-x": 0, "pad-y": 0, "stride-x": 2, "stride-y": 2, "pool-op": "max"}
+    geom = (batch, channels, h, w, oh, ow)
+    out = Dev(np.zeros(planes * oh * ow, np.float32))
+    assert _pool(True, desc, geom, out.ptr, xin.ptr) == "pool_forward_tile2"
+    want = x.reshape(planes, oh, 2, ow, 2).max(axis=(2, 4))
+    got = out.download().reshape(want.shape)
+    assert bits_equal(got, want)
+    og = Dev(np.ones(planes * oh * ow, np.float32))
+    ig = Dev(np.zeros(planes * h * w, np.float32))
+    assert _pool(False, desc, geom, ig.ptr, xin.ptr, out.ptr, og.ptr) == "pool_backward_tile2"
+    indicator = (x.reshape(planes, oh, 2, ow, 2) == want[:, :, None, :, None]).astype(np.float32).reshape(-1)
+    assert bits_equal(ig.download(), indicator)
+    for b in (out, og, ig):
+        b.free()
+
+    # a 1 x 1 window is a copy for every pool op (the generic band kernel at full size)
+    geom1 = (batch, channels, h, w, h, w)
+    for op in ("max", "avg", "avg-exc-pad"):
+        desc1 = {"kernel-width": 1, "kernel-height": 1, "pad-x": 0, "pad-y": 0, "stride-x": 1, "stride-y": 1, "pool-op": op}
+        out = Dev(np.zeros(planes * h * w, np.float32))
+        _pool(True, desc1, geom1, out.ptr, xin.ptr)
+        got = out.download()
+        if op == "max":
+            assert bits_equal(got, x.reshape(-1)), op
+        else:       # 0 + -0.0 = +0.0: the averages return a negative zero as a positive one
+            assert np.array_equal(got, x.reshape(-1)) and not np.any(np.signbit(got) & (got == 0)), op
+        out.free()
+    xin.free()
+
+    # 3 x 3, pad 1, stride 2 on a constant image; adjointness on random data at a smaller batch
+    oh = ow = (h + 2 - 3) // 2 + 1
+    geom3 = (batch, channels, h, w, oh, ow)
+    ones = Dev(np.full(planes * h * w, 3.0, np.float32))
+    inside_y = np.array([min(2 * o - 1 + 3, h) - max(2 * o - 1, 0) for o in range(oh)], np.float64)
+    inside = np.outer(inside_y, inside_y)
+    for op, expect in (("max", np.full((oh, ow), 3.0)), ("avg", None), ("avg-exc-pad", np.full((oh, ow), 3.0))):
+        desc3 = {"kernel-width": 3, "kernel-height": 3, "pad-x": 1, "pad-y": 1, "stride-x": 2, "stride-y": 2, "pool-op": op}
+        out = Dev(np.zeros(planes * oh * ow, np.float32))
+        assert _pool(True, desc3, geom3, out.ptr, ones.ptr) == "pool_forward_band"
+        got = out.download().reshape(planes, oh, ow)
+        assert np.all(got == got[0]), op               # every plane alike
+        if expect is None:
+            np.testing.assert_allclose(got[0], 3.0 * inside / 9.0, rtol=1e-6)
+        else:
+            np.testing.assert_allclose(got[0], expect, rtol=1e-6)
+        out.free()
+    ones.free()
+    sub = 256
+    xs, gs = x[:sub], rng.standard_normal((sub, oh, ow), dtype=np.float32)
+    for op in ("avg", "avg-exc-pad"):
+        desc3 = {"kernel-width": 3, "kernel-height": 3, "pad-x": 1, "pad-y": 1, "stride-x": 2, "stride-y": 2, "pool-op": op}
+        xi, gi = Dev(xs), Dev(gs)
+        out, ig = Dev(np.zeros(sub * oh * ow, np.float32)), Dev(np.zeros(sub * h * w, np.float32))
+        g3 = (1, sub, h, w, oh, ow)
+        _pool(True, desc3, g3, out.ptr, xi.ptr)
+        _pool(False, desc3, g3, ig.ptr, xi.ptr, out.ptr, gi.ptr)
+        lhs = np.dot(out.download().astype(np.float64), gs.reshape(-1).astype(np.float64))
+        rhs = np.dot(xs.reshape(-1).astype(np.float64), ig.download().astype(np.float64))
+        assert abs(lhs - rhs) <= 1e-6 * np.abs(gs).sum(), (op, lhs, rhs)
+        for b in (xi, gi, out, ig):
+            b.free()
