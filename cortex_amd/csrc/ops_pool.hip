@@ -301,6 +301,155 @@ __global__ void __launch_bounds__(kBlock) pool_forward_band_kernel(const BandArg
   }
 }
 
+// Forward pass over a zero-padded tile.  When no window reaches beyond the padded
+// input, every tap is either an input element or padding that reads 0, so the
+// tile is laid out with the padding in it and the taps need no tests at all:
+// row r of the tile is input row iy_base + r as kPadCells zero cells, the row
+// itself, and zero cells up to a pitch that is a multiple of four; rows above
+// and below the input are zero, and four more zero cells follow the last row.
+// The cells to the right of a row run on into the left padding of the next.
+// Tap (k_y, k_x) of output (y, x) of the band is
+// tile[(y * stride_y + k_y) * pitch + kPadCells - pad_x + x * stride_x + k_x].
+// With rows that are whole 16-byte pieces of an aligned buffer, every piece
+// loaded from memory is stored to LDS as one piece; otherwise cell by cell.
+constexpr int32_t kPadCells = 4;
+// LDS of a padded tile: a little more than the band kernels take, so that a
+// 56 x 56 float plane with its padding (13.4 KiB) stays whole.
+constexpr uint32_t kPaddedLdsBytes = 16 * 1024;
+
+struct PaddedArgs {
+  const void* in;
+  void* dest;
+  int32_t in_h, in_w, out_h, out_w;
+  int32_t px, py, sx, sy;
+  uint32_t in_plane, out_plane;
+  uint32_t planes, pb, br, bands;
+  uint32_t pitch;         // kPadCells + in_w rounded up to a multiple of four
+  uint32_t tile_rows;     // whole planes: rows of a plane's tile
+  uint32_t cap;
+  uint32_t fast_div;
+  double recip;
+  FastDiv bands_fd, out_w_fd, out_plane_fd, in_w_fd, in_plane_fd;
+};
+
+template <class T, int OP, int KW, int KH>
+__global__ void __launch_bounds__(kBlock) pool_forward_padded_kernel(const PaddedArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* tile = reinterpret_cast<T*>(smem);
+  double* recips = reinterpret_cast<double*>(smem + (size_t)a.cap * sizeof(T));
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  uint32_t group, band;
+  a.bands_fd.divmod(blockIdx.x, group, band);
+  const uint32_t p0 = group * a.pb, np = min(a.pb, a.planes - p0);
+  const int32_t oy0 = (int32_t)(band * a.br), rows = min((int32_t)a.br, a.out_h - oy0);
+  const int32_t iy_base = oy0 * a.sy - a.py;
+  const uint32_t tile_rows = a.pb > 1 ? a.tile_rows : (uint32_t)((rows - 1) * a.sy + KH);
+  // input rows [iy_lo, iy_hi) are staged; with whole planes, all of them
+  const int32_t iy_lo = a.pb > 1 ? 0 : max(0, iy_base);
+  const int32_t iy_hi = a.pb > 1 ? a.in_h : max(iy_lo, min(a.in_h, iy_base + (int32_t)tile_rows));
+  const uint32_t top = (uint32_t)(iy_lo - iy_base);          // zero rows above the first staged one
+  const uint32_t n_rows = (uint32_t)(iy_hi - iy_lo);
+  const uint32_t plane_cells = tile_rows * a.pitch;
+  const uint32_t gap = a.pitch - (uint32_t)a.in_w;            // cells between the end of a row and the next row's data
+
+  // zeros: around every row, the rows outside the input, the cells after the last row
+  for (uint32_t jr = threadIdx.x; jr < np * tile_rows; jr += kBlock) {
+    T* row = tile + jr * a.pitch;
+#pragma unroll
+    for (int32_t c = 0; c < kPadCells; ++c) row[c] = (T)0;
+    for (uint32_t c = kPadCells + (uint32_t)a.in_w; c < a.pitch; ++c) row[c] = (T)0;
+  }
+  if (threadIdx.x < kPadCells) tile[np * plane_cells + threadIdx.x] = (T)0;
+  const uint32_t zero_rows = tile_rows - n_rows;               // `top` above, the rest below
+  for (uint32_t j = 0; j < np; ++j)
+    for (uint32_t z = 0; z < zero_rows; ++z) {
+      const uint32_t r = z < top ? z : z + n_rows;
+      for (uint32_t c = kPadCells + threadIdx.x; c < kPadCells + (uint32_t)a.in_w; c += kBlock)
+        tile[j * plane_cells + r * a.pitch + c] = (T)0;
+    }
+
+  // the staged rows are one contiguous piece of memory
+  const uint32_t len = a.pb > 1 ? np * a.in_plane : n_rows * (uint32_t)a.in_w;
+  const T* src = reinterpret_cast<const T*>(a.in) + (int64_t)p0 * a.in_plane + (int64_t)iy_lo * a.in_w;
+  const uint32_t lead = (uint32_t)((reinterpret_cast<uintptr_t>(src) / sizeof(T)) % VEC);
+  if (lead == 0 && (uint32_t)a.in_w % VEC == 0) {
+    for (uint32_t g0 = threadIdx.x * VEC; g0 < len; g0 += kBlock * VEC) {
+      const Bytes16 raw = *reinterpret_cast<const Bytes16*>(src + g0);
+      uint32_t j = 0, rr = g0, row, col;
+      if (a.pb > 1) a.in_plane_fd.divmod(g0, j, rr);
+      a.in_w_fd.divmod(rr, row, col);
+      *reinterpret_cast<Bytes16*>(tile + j * plane_cells + (row + top) * a.pitch + kPadCells + col) = raw;
+    }
+  } else {
+    const T* base = src - lead;
+    const uint32_t end = lead + len;
+    for (uint32_t v = threadIdx.x; v * VEC < end; v += kBlock) {
+      const uint32_t i0 = v * VEC;
+      T piece[VEC];
+      if (i0 >= lead && i0 + VEC <= end) {
+        const Bytes16 raw = *reinterpret_cast<const Bytes16*>(base + i0);
+        __builtin_memcpy(piece, &raw, 16);
+      } else {
+#pragma unroll
+        for (uint32_t e = 0; e < VEC; ++e) piece[e] = (i0 + e >= lead && i0 + e < end) ? base[i0 + e] : (T)0;
+      }
+      // element g of the piece of memory: plane j, row, column
+      const uint32_t g0 = i0 >= lead ? i0 - lead : 0u;
+      uint32_t j = 0, rr = g0, row, col;
+      if (a.pb > 1) a.in_plane_fd.divmod(g0, j, rr);
+      a.in_w_fd.divmod(rr, row, col);
+      uint32_t at = j * plane_cells + (row + top) * a.pitch + kPadCells + col;
+#pragma unroll
+      for (uint32_t e = 0; e < VEC; ++e) {
+        const uint32_t i = i0 + e;
+        if (i >= lead && i < end) {
+          tile[at] = piece[e];
+          ++at;
+          if (++col == (uint32_t)a.in_w) {
+            col = 0;
+            at += gap;
+            if (a.pb > 1 && ++row == (uint32_t)a.in_h) { row = 0; at += (tile_rows - (uint32_t)a.in_h) * a.pitch; }
+          }
+        }
+      }
+    }
+  }
+  if (OP == CT_POOL_AVG_EXC_PAD && a.fast_div)
+    for (int32_t i = threadIdx.x; i <= KW * KH; i += kBlock) recips[i] = 1.0 / (double)i;
+  __syncthreads();
+
+  const uint32_t n_dest = np * (uint32_t)(rows * a.out_w);
+  T* out = reinterpret_cast<T*>(a.dest) + (int64_t)p0 * a.out_plane + (int64_t)oy0 * a.out_w;
+  constexpr double kernel_count = (double)(KW * KH);
+  const uint32_t first_tap = (uint32_t)(kPadCells - a.px);
+  for (uint32_t o = threadIdx.x; o < n_dest; o += kBlock) {
+    uint32_t j = 0, rr = o, oyl, ox;
+    if (a.pb > 1) a.out_plane_fd.divmod(o, j, rr);
+    a.out_w_fd.divmod(rr, oyl, ox);
+    const T* window = tile + j * plane_cells + oyl * (uint32_t)a.sy * a.pitch + first_tap + ox * (uint32_t)a.sx;
+    T acc = OP == CT_POOL_AVG_EXC_PAD ? out[o] : (T)0;
+    double divisor = kernel_count, y = a.recip;
+    if (OP == CT_POOL_AVG_EXC_PAD) {
+      const int32_t inside = taps_inside((int32_t)ox * a.sx - a.px, KW, a.in_w) *
+                             taps_inside((oy0 + (int32_t)oyl) * a.sy - a.py, KH, a.in_h);
+      divisor = (double)inside;
+      if (a.fast_div) y = recips[inside];
+    }
+#pragma unroll
+    for (int32_t ky = 0; ky < KH; ++ky) {
+#pragma unroll
+      for (int32_t kx = 0; kx < KW; ++kx) {
+        const T v = window[ky * a.pitch + kx];
+        const bool first = (ky | kx) == 0;
+        if (OP == CT_POOL_MAX) acc = (first || v > acc) ? v : acc;
+        else if (OP == CT_POOL_AVG) acc = (T)((double)(first ? (T)0 : acc) + tap_quotient(v, divisor, y, a.fast_div));
+        else acc = (T)((double)acc + tap_quotient(v, divisor, y, a.fast_div));
+      }
+    }
+    out[o] = acc;
+  }
+}
+
 template <class T, int OP, int KW, int KH>
 __global__ void __launch_bounds__(kBlock) pool_backward_band_kernel(const BandArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -613,6 +762,73 @@ int pool_launch(hipStream_t s, bool forward, void* dest, const void* in, const v
 #undef CT_POOL
     }
     return after_launch(s);
+  }
+
+  // Forward pass of a 2 x 2 or 3 x 3 window that never reaches beyond the padded input: zero-padded tile.
+  const bool fixed_window = (d.kernel_width == 2 && d.kernel_height == 2) || (d.kernel_width == 3 && d.kernel_height == 3);
+  const int64_t reach_x = (sh.out_w - 1) * d.stride_x - d.pad_x + d.kernel_width;
+  const int64_t reach_y = (sh.out_h - 1) * d.stride_y - d.pad_y + d.kernel_height;
+  if (forward && fixed_window && in_plane > 0 && d.pad_x <= kPadCells && reach_x <= sh.in_w + d.pad_x &&
+      reach_y <= sh.in_h + d.pad_y) {
+    const int64_t budget = kPaddedLdsBytes / (int64_t)sizeof(T);
+    const int64_t pitch = (kPadCells + sh.in_w + 3) / 4 * 4;
+    const int64_t plane_rows = d.pad_y + std::max<int64_t>(sh.in_h, reach_y);
+    const int64_t plane_cells = plane_rows * pitch;
+    PaddedArgs a{};
+    bool usable = true;
+    if (plane_cells + kPadCells <= budget) {
+      const int64_t by_lds = (budget - kPadCells) / plane_cells;
+      const int64_t by_dest = std::max<int64_t>(1, kBandDestTarget / out_plane);
+      a.pb = (uint32_t)std::max<int64_t>(1, std::min(by_lds, by_dest));
+      a.br = (uint32_t)sh.out_h;
+      a.bands = 1;
+    } else {
+      const int64_t tile_rows = (budget - kPadCells) / pitch;
+      int64_t rows = tile_rows >= d.kernel_height ? (tile_rows - d.kernel_height) / d.stride_y + 1 : 0;
+      usable = rows >= 1;
+      rows = std::min<int64_t>(std::max<int64_t>(rows, 1), sh.out_h);
+      a.pb = 1;
+      a.bands = (uint32_t)((sh.out_h + rows - 1) / rows);
+      a.br = (uint32_t)((sh.out_h + a.bands - 1) / a.bands);
+    }
+    if (usable) {
+      a.in_h = (int32_t)sh.in_h; a.in_w = (int32_t)sh.in_w; a.out_h = (int32_t)sh.out_h; a.out_w = (int32_t)sh.out_w;
+      a.px = d.pad_x; a.py = d.pad_y; a.sx = d.stride_x; a.sy = d.stride_y;
+      a.in_plane = (uint32_t)in_plane; a.out_plane = (uint32_t)out_plane;
+      a.pitch = (uint32_t)pitch;
+      a.tile_rows = (uint32_t)plane_rows;
+      a.cap = ((uint32_t)budget + 8u) / 4u * 4u;
+      const int64_t window = (int64_t)d.kernel_width * d.kernel_height;
+      a.fast_div = sizeof(T) == 4 ? 1u : 0u;
+      a.recip = 1.0 / (double)window;
+      a.bands_fd = FastDiv(a.bands);
+      a.out_w_fd = FastDiv((uint32_t)sh.out_w);
+      a.out_plane_fd = FastDiv((uint32_t)out_plane);
+      a.in_w_fd = FastDiv((uint32_t)sh.in_w);
+      a.in_plane_fd = FastDiv((uint32_t)in_plane);
+      const size_t lds = (size_t)a.cap * sizeof(T) + (size_t)kRecipTable * sizeof(double);
+      note_kernel("pool_forward_padded");
+      for (int64_t p0 = 0; p0 < sh.planes; p0 += planes_per_launch) {
+        const int64_t np = std::min(planes_per_launch, sh.planes - p0);
+        a.planes = (uint32_t)np;
+        a.in = reinterpret_cast<const T*>(in) + p0 * in_plane;
+        a.dest = reinterpret_cast<T*>(dest) + p0 * dest_plane;
+        const int64_t groups = (np + a.pb - 1) / a.pb;
+        const dim3 grid((uint32_t)(groups * a.bands));
+#define CT_POOL(KW, KH)                                                                                                  \
+  switch (d.pool_op) {                                                                                                   \
+    case CT_POOL_MAX:                                                                                                    \
+      hipLaunchKernelGGL((pool_forward_padded_kernel<T, CT_POOL_MAX, KW, KH>), grid, dim3(kBlock), lds, s, a); break;    \
+    case CT_POOL_AVG:                                                                                                    \
+      hipLaunchKernelGGL((pool_forward_padded_kernel<T, CT_POOL_AVG, KW, KH>), grid, dim3(kBlock), lds, s, a); break;    \
+    default:                                                                                                             \
+      hipLaunchKernelGGL((pool_forward_padded_kernel<T, CT_POOL_AVG_EXC_PAD, KW, KH>), grid, dim3(kBlock), lds, s, a);  \
+  }
+        if (d.kernel_width == 2) { CT_POOL(2, 2) } else { CT_POOL(3, 3) }
+#undef CT_POOL
+      }
+      return after_launch(s);
+    }
   }
 
   const uint32_t arrays = forward ? 1u : 2u;

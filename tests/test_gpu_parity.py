@@ -842,6 +842,8 @@ POOL_CASES = [
     (2, 2, 90, 90, 2, 2, 0, 0, 2, 2, "floor"),
     (1, 3, 75, 110, 3, 3, 1, 1, 1, 1, "floor"),
     (1, 2, 100, 70, 5, 4, 2, 1, 2, 3, "ceil"),
+    (2, 2, 10, 10, 3, 3, 0, 0, 2, 2, "ceil"),      # the last windows reach beyond the padded input
+    (3, 4, 20, 20, 3, 3, 1, 1, 1, 1, "floor"),     # several small padded planes per block
     (1, 1, 9, 2000, 3, 3, 1, 1, 2, 2, "floor"),    # rows beyond it: the direct kernels
     (1, 1, 40, 300, 17, 17, 8, 8, 1, 1, "floor"),  # a window too large for the reciprocal table
 ]
