@@ -36,7 +36,7 @@ SOURCES = [
     "ops_batchnorm.hip",
     "ops_rand.hip",
     "ops_blas.cpp",
-    "ops_gemv.hip", "ops_pool.hip",
+    "ops_gemv.hip", "ops_pool.hip", "ops_conv.hip",
 ]
 
 # -ffp-contract=off: the reference's CPU backend rounds after every JVM

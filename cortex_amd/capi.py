@@ -59,6 +59,24 @@ class CtPoolDesc(C.Structure):
     ]
 
 
+class CtConvDesc(C.Structure):
+    """``ct_conv_desc``: the geometry of a convolution descriptor."""
+
+    _fields_ = [
+        ("in_channels", C.c_int32), ("out_channels", C.c_int32),
+        ("kernel_width", C.c_int32), ("kernel_height", C.c_int32),
+        ("pad_x", C.c_int32), ("pad_y", C.c_int32),
+        ("stride_x", C.c_int32), ("stride_y", C.c_int32),
+    ]
+
+
+def make_conv_desc(descriptor) -> CtConvDesc:
+    """Builds a ``ct_conv_desc`` from a convolution descriptor map."""
+    return CtConvDesc(int(descriptor["in-channels"]), int(descriptor["out-channels"]), int(descriptor["kernel-width"]),
+                      int(descriptor["kernel-height"]), int(descriptor["pad-x"]), int(descriptor["pad-y"]),
+                      int(descriptor["stride-x"]), int(descriptor["stride-y"]))
+
+
 def make_pool_desc(descriptor) -> CtPoolDesc:
     """Builds a ``ct_pool_desc`` from a pooling descriptor map."""
     return CtPoolDesc(int(descriptor["kernel-width"]), int(descriptor["kernel-height"]), int(descriptor["pad-x"]),
@@ -137,6 +155,9 @@ PROTOTYPES = {
     "ct_batch_normalize_update_and_apply_spatial": [_P, _P, _P, _P, _P, _P, _P, _D, _P, _P, _D, _L, _L, _L, _I],
     "ct_batch_normalize_gradients_eltwise": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _I],
     "ct_batch_normalize_gradients_spatial": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _D, _L, _L, _L, _I],
+    "ct_convolution_forward": [_P, _P, _D, _P, _P, _P, _L, C.POINTER(CtConvDesc), _L, _L, _L, _L, _L, _I],
+    "ct_convolution_backward_weights": [_P, _P, _D, _P, _P, _P, _L, C.POINTER(CtConvDesc), _L, _L, _L, _L, _L, _I],
+    "ct_convolution_backward_data": [_P, _P, _D, _P, _P, _P, _L, C.POINTER(CtConvDesc), _L, _L, _L, _L, _L, _I],
     "ct_pooling_forward": [_P, _P, _D, _P, C.POINTER(CtPoolDesc), _L, _L, _L, _L, _L, _L, _I],
     "ct_pooling_backward": [_P, _P, _D, _P, _P, _P, C.POINTER(CtPoolDesc), _L, _L, _L, _L, _L, _L, _I],
     "ct_gemm": [_P, _P, _L, _I, _I, _D, _P, _L, _L, _L, _P, _L, _L, _D, _I],

@@ -1,0 +1,294 @@
+// ops_conv.hip -- convolution-forward!, convolution-backward-weights! and
+// convolution-backward-data! (src/cortex/tensor/math.clj:185-220) with the
+// decomposition of the reference's CPU backend
+// (src/cortex/compute/cpu/tensor_math.clj:1118-1151, 1670-1792): the input is
+// unrolled into the caller's workspace, one row of in_channels * kh * kw cells
+// per output position (window walk: src/cortex/nn/impl.clj:8-96), and each
+// method is one gemm! per image around that matrix.  The two data movements are
+// the kernels of this file; the products go through ct_gemm (rocBLAS).
+//
+//   unroll     one lane per workspace cell, 16 bytes of cells per lane where a
+//              row of cells is a whole number of them: the writes, kh * kw times
+//              the volume of the reads, are linear and the reads come from the
+//              caches.  HBM-bound on the workspace it writes.
+//   roll back  the reference adds cell after cell into the input gradient while
+//              it walks the windows; here every input element gathers the cells
+//              that came from it, windows in increasing (row, column) order,
+//              which is the order in which that walk reaches the element: the
+//              same roundings, no atomics.  Reads the workspace once.
+#include <algorithm>
+
+#include "common.h"
+
+using namespace cthip;
+
+extern "C" int ct_gemm(void* stream, void* c, int64_t c_colstride, int trans_a, int trans_b, double alpha,
+                       const void* a, int64_t a_row_count, int64_t a_col_count, int64_t a_colstride, const void* b,
+                       int64_t b_col_count, int64_t b_colstride, double beta, int dtype);
+
+namespace {
+
+constexpr int kBlock = 256;
+
+struct ConvArgs {
+  const void* src;
+  void* dest;
+  uint32_t total;  // lanes' worth of work in this launch
+  int32_t in_h, in_w, out_h, out_w;
+  int32_t kw, kh, px, py, sx, sy;
+  uint32_t channels, n_cols, n_rows, in_plane;
+  FastDiv cols_fd, kk_fd, kw_fd, out_w_fd, rows_fd;  // unroll: cell -> (image, position, channel, tap)
+  FastDiv in_w_fd, in_plane_fd, image_fd, sx_fd, sy_fd;  // roll back: element -> (image, channel, row, column)
+};
+
+// workspace[image][position][channel * kh * kw + k_y * kw + k_x] = input tap or 0 in the padding
+template <class T, int VEC>
+__global__ void __launch_bounds__(kBlock) conv_unroll_kernel(const ConvArgs a) {
+  const uint32_t lane = blockIdx.x * kBlock + threadIdx.x;
+  if (lane >= a.total) return;
+  const uint32_t cell0 = lane * VEC;
+  uint32_t position_all, col;
+  a.cols_fd.divmod(cell0, position_all, col);
+  uint32_t image, position, oy, ox;
+  a.rows_fd.divmod(position_all, image, position);
+  a.out_w_fd.divmod(position, oy, ox);
+  const T* in = reinterpret_cast<const T*>(a.src) + (int64_t)image * a.channels * a.in_plane;
+  const int32_t rel_x = (int32_t)ox * a.sx - a.px, rel_y = (int32_t)oy * a.sy - a.py;
+  struct alignas(sizeof(T) * VEC) Piece { T v[VEC]; } piece;
+  uint32_t chan, tap, ky, kx;
+  a.kk_fd.divmod(col, chan, tap);
+  a.kw_fd.divmod(tap, ky, kx);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    const int32_t iy = rel_y + (int32_t)ky, ix = rel_x + (int32_t)kx;
+    const bool inside = (uint32_t)iy < (uint32_t)a.in_h && (uint32_t)ix < (uint32_t)a.in_w;
+    piece.v[e] = inside ? in[(int64_t)chan * a.in_plane + iy * a.in_w + ix] : (T)0;
+    if (++kx == (uint32_t)a.kw) {
+      kx = 0;
+      if (++ky == (uint32_t)a.kh) { ky = 0; ++chan; }
+    }
+  }
+  *reinterpret_cast<Piece*>(reinterpret_cast<T*>(a.dest) + (int64_t)cell0) = piece;
+}
+
+// input_gradient[image][channel][y][x] = sum of the workspace cells unrolled from it
+template <class T>
+__global__ void __launch_bounds__(kBlock) conv_roll_kernel(const ConvArgs a) {
+  const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+  if (e >= a.total) return;
+  uint32_t image, rest, chan, r, iy, ix;
+  a.image_fd.divmod(e, image, rest);
+  a.in_plane_fd.divmod(rest, chan, r);
+  a.in_w_fd.divmod(r, iy, ix);
+  const T* conv = reinterpret_cast<const T*>(a.src) + (int64_t)image * a.n_rows * a.n_cols + chan * (uint32_t)(a.kw * a.kh);
+  // Windows o with o * stride - pad <= i < o * stride - pad + k.
+  const int32_t ty = (int32_t)iy + a.py, tx = (int32_t)ix + a.px;
+  const int32_t oy_hi = min(a.out_h - 1, (int32_t)a.sy_fd.div((uint32_t)ty));
+  const int32_t ox_hi = min(a.out_w - 1, (int32_t)a.sx_fd.div((uint32_t)tx));
+  const int32_t by = ty - a.kh + 1, bx = tx - a.kw + 1;
+  const int32_t oy_lo = by <= 0 ? 0 : (int32_t)a.sy_fd.div((uint32_t)(by + a.sy - 1));
+  const int32_t ox_lo = bx <= 0 ? 0 : (int32_t)a.sx_fd.div((uint32_t)(bx + a.sx - 1));
+  T acc = (T)0;
+  for (int32_t oy = oy_lo; oy <= oy_hi; ++oy) {
+    const int32_t ky = ty - oy * a.sy;
+    for (int32_t ox = ox_lo; ox <= ox_hi; ++ox) {
+      const int32_t kx = tx - ox * a.sx;
+      acc = acc + conv[(int64_t)(oy * a.out_w + ox) * a.n_cols + ky * a.kw + kx];
+    }
+  }
+  reinterpret_cast<T*>(a.dest)[e] = acc;
+}
+
+struct ConvShape {
+  int64_t batch, in_h, in_w, out_h, out_w, n_rows, n_cols, in_image, out_image, conv_image;
+};
+
+int check_conv(const ct_conv_desc* d, int64_t batch_count, int64_t in_height, int64_t in_width, int64_t out_height,
+               int64_t out_width, int64_t workspace_ecount, int dtype, ConvShape* sh) {
+  CT_REQUIRE(d != nullptr, "convolution: null descriptor");
+  CT_REQUIRE(dtype == CT_F32 || dtype == CT_F64, "convolution is only defined for float and double tensors");
+  CT_REQUIRE(d->in_channels >= 1 && d->out_channels >= 1 && d->kernel_width >= 1 && d->kernel_height >= 1 &&
+                 d->stride_x >= 1 && d->stride_y >= 1 && d->pad_x >= 0 && d->pad_y >= 0,
+             "convolution: channels, kernel and stride must be positive and padding non-negative");
+  CT_REQUIRE(d->kernel_width <= 1024 && d->kernel_height <= 1024 && d->stride_x <= 1024 && d->stride_y <= 1024 &&
+                 d->pad_x <= 1024 && d->pad_y <= 1024 && d->in_channels <= 1 << 20 && d->out_channels <= 1 << 20,
+             "convolution: descriptor exceeds the supported range");
+  CT_REQUIRE(batch_count >= 0 && in_height >= 0 && in_width >= 0 && out_height >= 0 && out_width >= 0,
+             "convolution: negative count");
+  CT_REQUIRE(in_height <= 1 << 20 && in_width <= 1 << 20 && out_height <= 1 << 20 && out_width <= 1 << 20 &&
+                 batch_count <= 1 << 30,
+             "convolution: counts exceed the supported range");
+  if (out_height > 0 && out_width > 0)
+    CT_REQUIRE((out_width - 1) * d->stride_x - d->pad_x + d->kernel_width <= in_width + d->pad_x &&
+                   (out_height - 1) * d->stride_y - d->pad_y + d->kernel_height <= in_height + d->pad_y,
+               "convolution: a window reaches beyond the padded input (output dimensions must follow the floor rule)");
+  ConvShape s{};
+  s.batch = batch_count; s.in_h = in_height; s.in_w = in_width; s.out_h = out_height; s.out_w = out_width;
+  s.n_rows = out_height * out_width;
+  s.n_cols = (int64_t)d->kernel_width * d->kernel_height * d->in_channels;
+  s.in_image = (int64_t)d->in_channels * in_height * in_width;
+  s.out_image = (int64_t)d->out_channels * s.n_rows;
+  const int64_t limit = (int64_t(1) << 31) - 1;
+  CT_REQUIRE(s.n_rows <= limit && s.n_cols <= limit, "convolution: one image exceeds the supported range");
+  s.conv_image = s.n_rows * s.n_cols;
+  CT_REQUIRE(s.in_image <= limit && s.out_image <= limit && s.conv_image <= limit && s.n_cols <= limit,
+             "convolution: one image exceeds the supported range");
+  CT_REQUIRE(workspace_ecount >= batch_count * s.conv_image,
+             "convolution: workspace of %lld elements, %lld needed", (long long)workspace_ecount,
+             (long long)(batch_count * s.conv_image));
+  *sh = s;
+  return CT_OK;
+}
+
+ConvArgs conv_args(const ct_conv_desc& d, const ConvShape& sh) {
+  ConvArgs a{};
+  a.in_h = (int32_t)sh.in_h; a.in_w = (int32_t)sh.in_w; a.out_h = (int32_t)sh.out_h; a.out_w = (int32_t)sh.out_w;
+  a.kw = d.kernel_width; a.kh = d.kernel_height; a.px = d.pad_x; a.py = d.pad_y; a.sx = d.stride_x; a.sy = d.stride_y;
+  a.channels = (uint32_t)d.in_channels;
+  a.n_cols = (uint32_t)sh.n_cols; a.n_rows = (uint32_t)sh.n_rows;
+  a.in_plane = (uint32_t)(sh.in_h * sh.in_w);
+  a.cols_fd = FastDiv((uint32_t)std::max<int64_t>(1, sh.n_cols));
+  a.kk_fd = FastDiv((uint32_t)(d.kernel_width * d.kernel_height));
+  a.kw_fd = FastDiv((uint32_t)d.kernel_width);
+  a.out_w_fd = FastDiv((uint32_t)std::max<int64_t>(1, sh.out_w));
+  a.rows_fd = FastDiv((uint32_t)std::max<int64_t>(1, sh.n_rows));
+  a.in_w_fd = FastDiv((uint32_t)std::max<int64_t>(1, sh.in_w));
+  a.in_plane_fd = FastDiv(std::max<uint32_t>(1u, a.in_plane));
+  a.image_fd = FastDiv((uint32_t)std::max<int64_t>(1, sh.in_image));
+  a.sx_fd = FastDiv((uint32_t)d.stride_x);
+  a.sy_fd = FastDiv((uint32_t)d.stride_y);
+  return a;
+}
+
+// Images per launch so that a launch indexes fewer than 2^31 cells.
+int64_t images_per_launch(int64_t per_image) {
+  return std::max<int64_t>(1, ((int64_t(1) << 31) - 1) / std::max<int64_t>(1, per_image));
+}
+
+template <class T>
+void unroll(hipStream_t s, const T* input, T* workspace, const ct_conv_desc& d, const ConvShape& sh) {
+  if (sh.batch * sh.conv_image == 0) return;
+  ConvArgs a = conv_args(d, sh);
+  constexpr int VEC = 16 / sizeof(T);
+  const bool pieces = sh.n_cols % VEC == 0 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+  const int64_t step = images_per_launch(sh.conv_image);
+  for (int64_t b0 = 0; b0 < sh.batch; b0 += step) {
+    const int64_t nb = std::min(step, sh.batch - b0);
+    a.src = input + b0 * sh.in_image;
+    a.dest = workspace + b0 * sh.conv_image;
+    const int64_t cells = nb * sh.conv_image;
+    a.total = (uint32_t)(pieces ? cells / VEC : cells);
+    const dim3 grid((a.total + kBlock - 1) / kBlock);
+    if (pieces) hipLaunchKernelGGL((conv_unroll_kernel<T, VEC>), grid, dim3(kBlock), 0, s, a);
+    else hipLaunchKernelGGL((conv_unroll_kernel<T, 1>), grid, dim3(kBlock), 0, s, a);
+  }
+}
+
+template <class T>
+void roll_back(hipStream_t s, const T* workspace, T* input_gradient, const ct_conv_desc& d, const ConvShape& sh) {
+  if (sh.batch * sh.in_image == 0) return;
+  ConvArgs a = conv_args(d, sh);
+  const int64_t step = std::min(images_per_launch(sh.in_image), images_per_launch(sh.conv_image));
+  for (int64_t b0 = 0; b0 < sh.batch; b0 += step) {
+    const int64_t nb = std::min(step, sh.batch - b0);
+    a.src = workspace + b0 * sh.conv_image;
+    a.dest = input_gradient + b0 * sh.in_image;
+    a.total = (uint32_t)(nb * sh.in_image);
+    const dim3 grid((a.total + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL((conv_roll_kernel<T>), grid, dim3(kBlock), 0, s, a);
+  }
+}
+
+template <class T>
+int forward_t(void* stream, T* output, double output_alpha, const T* input, const T* weights, T* workspace,
+              const ct_conv_desc& d, const ConvShape& sh, int dtype) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  unroll(s, input, workspace, d, sh);
+  if (int rc = after_launch(s)) return rc;
+  for (int64_t b = 0; b < sh.batch; ++b)
+    if (int rc = ct_gemm(stream, output + b * sh.out_image, sh.n_rows, 0, 1, 1.0, weights, d.out_channels, sh.n_cols,
+                         sh.n_cols, workspace + b * sh.conv_image, sh.n_rows, sh.n_cols, output_alpha, dtype))
+      return rc;
+  note_kernel("conv_unroll+gemm");
+  return CT_OK;
+}
+
+template <class T>
+int backward_weights_t(void* stream, T* weight_gradient, double alpha, const T* output_gradient, T* workspace,
+                       const ct_conv_desc& d, const ConvShape& sh, int dtype) {
+  for (int64_t b = 0; b < sh.batch; ++b)
+    if (int rc = ct_gemm(stream, weight_gradient, sh.n_cols, 0, 0, 1.0, output_gradient + b * sh.out_image,
+                         d.out_channels, sh.n_rows, sh.n_rows, workspace + b * sh.conv_image, sh.n_cols, sh.n_cols,
+                         b == 0 ? alpha : 1.0, dtype))
+      return rc;
+  return CT_OK;
+}
+
+template <class T>
+int backward_data_t(void* stream, T* input_gradient, const T* output_gradient, const T* weights, T* workspace,
+                    const ct_conv_desc& d, const ConvShape& sh, int dtype) {
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  for (int64_t b = 0; b < sh.batch && sh.conv_image > 0; ++b)
+    if (int rc = ct_gemm(stream, workspace + b * sh.conv_image, sh.n_cols, 1, 0, 1.0, output_gradient + b * sh.out_image,
+                         sh.n_rows, d.out_channels, sh.n_rows, weights, sh.n_cols, sh.n_cols, 0.0, dtype))
+      return rc;
+  roll_back(s, workspace, input_gradient, d, sh);
+  note_kernel("gemm+conv_roll");
+  return after_launch(s);
+}
+
+}  // namespace
+
+extern "C" {
+
+int ct_convolution_forward(void* stream, void* output, double output_alpha, const void* input, const void* weights,
+                           void* workspace, int64_t workspace_ecount, const ct_conv_desc* desc, int64_t batch_count,
+                           int64_t in_height, int64_t in_width, int64_t out_height, int64_t out_width, int dtype) {
+  ConvShape sh;
+  if (int rc = check_conv(desc, batch_count, in_height, in_width, out_height, out_width, workspace_ecount, dtype, &sh))
+    return rc;
+  if (sh.batch * sh.out_image == 0) return CT_OK;
+  CT_REQUIRE(output && weights && workspace && (input || sh.in_image == 0), "convolution-forward!: null buffer");
+  if (dtype == CT_F32)
+    return forward_t<float>(stream, (float*)output, output_alpha, (const float*)input, (const float*)weights,
+                            (float*)workspace, *desc, sh, dtype);
+  return forward_t<double>(stream, (double*)output, output_alpha, (const double*)input, (const double*)weights,
+                           (double*)workspace, *desc, sh, dtype);
+}
+
+int ct_convolution_backward_weights(void* stream, void* weight_gradient, double weight_gradient_alpha,
+                                    const void* output_gradient, const void* /*input*/, void* workspace,
+                                    int64_t workspace_ecount, const ct_conv_desc* desc, int64_t batch_count,
+                                    int64_t in_height, int64_t in_width, int64_t out_height, int64_t out_width,
+                                    int dtype) {
+  ConvShape sh;
+  if (int rc = check_conv(desc, batch_count, in_height, in_width, out_height, out_width, workspace_ecount, dtype, &sh))
+    return rc;
+  if (sh.batch * sh.conv_image == 0) return CT_OK;
+  CT_REQUIRE(weight_gradient && output_gradient && workspace, "convolution-backward-weights!: null buffer");
+  if (dtype == CT_F32)
+    return backward_weights_t<float>(stream, (float*)weight_gradient, weight_gradient_alpha,
+                                     (const float*)output_gradient, (float*)workspace, *desc, sh, dtype);
+  return backward_weights_t<double>(stream, (double*)weight_gradient, weight_gradient_alpha,
+                                    (const double*)output_gradient, (double*)workspace, *desc, sh, dtype);
+}
+
+int ct_convolution_backward_data(void* stream, void* input_gradient, double /*input_gradient_alpha*/,
+                                 const void* output_gradient, const void* weights, void* workspace,
+                                 int64_t workspace_ecount, const ct_conv_desc* desc, int64_t batch_count,
+                                 int64_t in_height, int64_t in_width, int64_t out_height, int64_t out_width,
+                                 int dtype) {
+  ConvShape sh;
+  if (int rc = check_conv(desc, batch_count, in_height, in_width, out_height, out_width, workspace_ecount, dtype, &sh))
+    return rc;
+  if (sh.batch * sh.in_image == 0) return CT_OK;
+  CT_REQUIRE(input_gradient && (sh.conv_image == 0 || (output_gradient && weights && workspace)),
+             "convolution-backward-data!: null buffer");
+  if (dtype == CT_F32)
+    return backward_data_t<float>(stream, (float*)input_gradient, (const float*)output_gradient,
+                                  (const float*)weights, (float*)workspace, *desc, sh, dtype);
+  return backward_data_t<double>(stream, (double*)input_gradient, (const double*)output_gradient,
+                                 (const double*)weights, (double*)workspace, *desc, sh, dtype);
+}
+
+}  // extern "C"

@@ -299,6 +299,43 @@ class HipStream:
         capi.call("ct_softmax_spatial", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), input.ptr,
                   C.byref(_dims_struct(input_dims)), capi.DTYPE_CODES[output.datatype])
 
+    # -- convolution (tensor/math.clj:185-220); buffers are packed, the workspace is the caller's --
+    def convolution_descriptor(self, datatype, out_channels, in_channels, kern_width, kern_height, pad_x, pad_y,
+                               stride_x, stride_y):
+        return None   # no native object, as on the CPU backend (cpu/tensor_math.clj:1665-1668)
+
+    def choose_convolution_algorithms(self, conv_descriptor, input_width, input_height, output_width, output_height,
+                                      batch_size, max_ideal_workspace_size, use_defaults):
+        """Workspace for the unrolled input (cpu/tensor_math.clj:1670-1680)."""
+        n_cols = int(conv_descriptor["kernel-width"]) * int(conv_descriptor["kernel-height"]) * \
+            int(conv_descriptor["in-channels"])
+        return {"workspace-size": n_cols * int(output_width) * int(output_height) * int(batch_size)}
+
+    def _conv(self, name, dest, alpha, a, b, workspace, workspace_ecount, conv_descriptor, in_shape, out_shape):
+        batch, _, in_h, in_w = (int(v) for v in in_shape)
+        out_h, out_w = (int(v) for v in out_shape[2:])
+        desc = capi.make_conv_desc(conv_descriptor)
+        capi.call(name, self.handle, dest.ptr, float(alpha), a.ptr, b.ptr, workspace.ptr, int(workspace_ecount),
+                  C.byref(desc), int(out_shape[0]), in_h, in_w, out_h, out_w, capi.DTYPE_CODES[dest.datatype])
+
+    def convolution_forward(self, output, output_dims, output_alpha, input, input_dims, weights, weight_dims,
+                            workspace, workspace_ecount, conv_descriptor, algorithms) -> None:
+        self._conv("ct_convolution_forward", output, output_alpha, input, weights, workspace, workspace_ecount,
+                   conv_descriptor, input_dims["shape"], output_dims["shape"])
+
+    def convolution_backward_weights(self, weight_gradient, weight_gradient_dims, weight_gradient_alpha,
+                                     output_gradient, output_gradient_dims, input, input_dims, workspace,
+                                     workspace_ecount, conv_descriptor, algorithms) -> None:
+        self._conv("ct_convolution_backward_weights", weight_gradient, weight_gradient_alpha, output_gradient, input,
+                   workspace, workspace_ecount, conv_descriptor, input_dims["shape"], output_gradient_dims["shape"])
+
+    def convolution_backward_data(self, input_gradient, input_gradient_dims, input_gradient_alpha, output_gradient,
+                                  output_gradient_dims, weights, weights_dims, workspace, workspace_ecount,
+                                  conv_descriptor, algorithms) -> None:
+        self._conv("ct_convolution_backward_data", input_gradient, input_gradient_alpha, output_gradient, weights,
+                   workspace, workspace_ecount, conv_descriptor, input_gradient_dims["shape"],
+                   output_gradient_dims["shape"])
+
     # -- pooling (tensor/math.clj:221-236); buffers are packed [batch channels height width] --
     def pooling_forward(self, output, output_dims, output_alpha, input, input_dims, pool_descriptor) -> None:
         batch, channels, in_h, in_w = (int(v) for v in input_dims["shape"])

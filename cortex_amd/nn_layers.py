@@ -313,6 +313,66 @@ class BatchNormalization:
 
 # ------------------------------------------------------------------ prelu
 
+def convolutional(kernel_dim: int, pad: int, stride: int, num_kernels: int, input_dimension: dict) -> dict:
+    """The description of a convolutional layer as ``layers/convolutional``
+    (``src/cortex/nn/layers.clj:394-408``) writes it and ``build-convolutional-type-node``
+    (``:449-465``) completes it; the dimension operation is always ``:floor``
+    (``:467-475``).  Weights are [num-kernels, kernel-width * kernel-height * channels]
+    (``:410-413``), the bias [num-kernels]."""
+    if stride < 1:
+        raise ValueError("Convolutional layers must have stride >= 1")
+    if kernel_dim < 1:
+        raise ValueError("Convolutional layers must have kernel dimensions >= 1")
+    node = {"type": "convolutional", "kernel-width": kernel_dim, "kernel-height": kernel_dim, "pad-x": pad,
+            "pad-y": pad, "stride-x": stride, "stride-y": stride, "num-kernels": num_kernels, "dimension-op": "floor"}
+    out = ct.get_convolution_output_dimensions(node, input_dimension["width"], input_dimension["height"])
+    node["input-dimension"] = dict(input_dimension)
+    node["output-dimension"] = {"channels": num_kernels, "height": out["output-height"], "width": out["output-width"]}
+    return node
+
+
+class ConvolutionLayer:
+    """``ConvolutionLayer`` (``layers.clj:306-368``): the workspace for the
+    unrolled input lives with the layer and carries the unrolled input from the
+    forward pass to the weight gradient."""
+
+    def __init__(self, layer: dict, batch_size: int, datatype: str = None):
+        self.layer = layer
+        datatype = datatype or ct.current_datatype()
+        dimension = layer["input-dimension"]
+        self.conv_desc = ct.convolution_descriptor(datatype, layer["num-kernels"], dimension["channels"],
+                                                   layer["kernel-width"], layer["kernel-height"], layer["pad-x"],
+                                                   layer["pad-y"], layer["stride-x"], layer["stride-y"])
+        self.algorithms = ct.choose_convolution_algorithms(self.conv_desc, dimension["width"], dimension["height"],
+                                                           batch_size, 100000)
+        self.workspace = ct.new_tensor([self.algorithms["workspace-size"]], datatype)
+
+    def forward(self, parameter_buffers, input_buffers, output_buffers):
+        batch_size = _batch_size(first_buffer(input_buffers))
+        output = _conv_tensor(self.layer["output-dimension"], batch_size, first_buffer(output_buffers))
+        input = _conv_tensor(self.layer["input-dimension"], batch_size, first_buffer(input_buffers))
+        weights = parameter_buffers["weights"]["buffer"]
+        # set the bias up so that it broadcasts over the output
+        bias = ct.in_place_reshape(parameter_buffers["bias"]["buffer"], [self.conv_desc["out-channels"], 1, 1])
+        ct.convolution_forward(output, 0.0, input, weights, self.workspace, self.conv_desc, self.algorithms)
+        ct.binary_op(output, 1.0, output, 1.0, bias, "+")
+
+    def backward(self, parameter_buffers, output_buffers, input_buffers):
+        batch_size = _batch_size(first_buffer(input_buffers))
+        output_gradient = _conv_tensor(self.layer["output-dimension"], batch_size, first_gradient(output_buffers))
+        input = _conv_tensor(self.layer["input-dimension"], batch_size, first_buffer(input_buffers))
+        input_gradient = _conv_tensor(self.layer["input-dimension"], batch_size, first_gradient(input_buffers))
+        weights = parameter_buffers["weights"]["buffer"]
+        weight_gradient = parameter_buffers["weights"]["gradient"]
+        out_chan = output_gradient.shape()[1]
+        bias_gradient = ct.in_place_reshape(parameter_buffers["bias"]["gradient"], [out_chan, 1, 1])
+        ct.binary_op(bias_gradient, 1.0, output_gradient, 1.0, bias_gradient, "+")
+        ct.convolution_backward_weights(weight_gradient, 0.0, output_gradient, input, self.workspace, self.conv_desc,
+                                        self.algorithms)
+        ct.convolution_backward_data(input_gradient, 0.0, output_gradient, weights, self.workspace, self.conv_desc,
+                                     self.algorithms)
+
+
 def max_pooling(kernel_dim: int, pad: int, stride: int, input_dimension: dict, **args) -> dict:
     """The description of a pooling layer as ``layers/max-pooling``
     (``src/cortex/nn/layers.clj:492-511``) writes it and
@@ -533,6 +593,8 @@ def create(node: dict, batch_size: int, datatype: str = None):
         return Prelu(node, batch_size, datatype)
     if kind == "max-pooling":
         return PoolingLayer(node, batch_size, datatype)
+    if kind == "convolutional":
+        return ConvolutionLayer(node, batch_size, datatype)
     if kind == "concatenate":
         return Concatenate()
     if kind == "split":

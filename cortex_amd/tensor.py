@@ -513,6 +513,79 @@ def softmax(output: Tensor, input: Tensor) -> Tensor:
     return output
 
 
+# ---------------------------------------------------------------- convolution
+
+def convolution_descriptor(datatype, out_channels, in_channels, kern_width, kern_height, pad_x, pad_y, stride_x,
+                           stride_y):
+    """``convolution-descriptor`` (``tensor.clj:1320-1348``)."""
+    args = {"out-channels": out_channels, "in-channels": in_channels, "kern-width": kern_width,
+            "kern-height": kern_height, "pad-x": pad_x, "pad-y": pad_y, "stride-x": stride_x, "stride-y": stride_y}
+    missing = [k for k, v in args.items() if v is None]
+    if missing:
+        raise TensorError(f"Arguments were nil: {missing}")
+    return {"datatype": datatype, "out-channels": out_channels, "in-channels": in_channels,
+            "kernel-width": kern_width, "kernel-height": kern_height, "pad-x": pad_x, "pad-y": pad_y,
+            "stride-x": stride_x, "stride-y": stride_y,
+            "descriptor": check_stream().convolution_descriptor(datatype, out_channels, in_channels, kern_width,
+                                                                kern_height, pad_x, pad_y, stride_x, stride_y)}
+
+
+def choose_convolution_algorithms(descriptor, input_width, input_height, batch_size, max_ideal_workspace_size,
+                                  use_defaults=False):
+    """``choose-convolution-algorithms`` (``tensor.clj:1385-1401``)."""
+    out = get_convolution_output_dimensions(descriptor, input_width, input_height)
+    return check_stream().choose_convolution_algorithms(descriptor, input_width, input_height, out["output-width"],
+                                                        out["output-height"], batch_size, max_ideal_workspace_size,
+                                                        use_defaults)
+
+
+def _ensure_conv_weight_dims_match(input: Tensor, weights: Tensor, descriptor) -> None:
+    """``ensure-conv-weight-dims-match`` (``tensor.clj:1403-1423``)."""
+    out_size, in_size = as_2d_matrix(weights).shape()
+    if not dense(weights):
+        raise TensorError("Convolution weights must be dense tensors")
+    expected = int(descriptor["kernel-width"]) * int(descriptor["kernel-height"]) * int(descriptor["in-channels"])
+    if int(in_size) != expected:
+        raise TensorError(f"Weight column length does not equal kernel-width * kernel-height * in-channels: "
+                          f"{in_size} {expected}")
+    if int(out_size) != int(descriptor["out-channels"]):
+        raise TensorError(f"Weight row count does not match out-channels: {out_size} {descriptor['out-channels']}")
+
+
+def convolution_forward(output: Tensor, output_alpha, input: Tensor, weights: Tensor, workspace: Tensor,
+                        conv_descriptor, algorithms) -> Tensor:
+    """``convolution-forward!`` (``tensor.clj:1454-1467``)."""
+    _external_library_check("convolution-forward!", output, input, weights)
+    _ensure_conv_io(conv_descriptor, [input], [output])
+    check_stream().convolution_forward(output.buffer, output.dimensions, output_alpha, input.buffer, input.dimensions,
+                                       weights.buffer, weights.dimensions, workspace.buffer, ecount(workspace),
+                                       conv_descriptor, algorithms)
+    return output
+
+
+def convolution_backward_weights(weight_gradient: Tensor, weight_gradient_alpha, output_gradient: Tensor,
+                                 input: Tensor, workspace: Tensor, conv_descriptor, algorithms) -> Tensor:
+    """``convolution-backward-weights!`` (``tensor.clj:1470-1481``)."""
+    _external_library_check("convolution-backward-weights!", weight_gradient, output_gradient, input)
+    check_stream().convolution_backward_weights(weight_gradient.buffer, weight_gradient.dimensions,
+                                                weight_gradient_alpha, output_gradient.buffer,
+                                                output_gradient.dimensions, input.buffer, input.dimensions,
+                                                workspace.buffer, ecount(workspace), conv_descriptor, algorithms)
+    return weight_gradient
+
+
+def convolution_backward_data(input_gradient: Tensor, input_gradient_alpha, output_gradient: Tensor, weights: Tensor,
+                              workspace: Tensor, conv_descriptor, algorithms) -> Tensor:
+    """``convolution-backward-data!`` (``tensor.clj:1484-1496``)."""
+    _external_library_check("convolution-backward-data!", input_gradient, output_gradient, weights)
+    _ensure_conv_io(conv_descriptor, [input_gradient], [output_gradient])
+    check_stream().convolution_backward_data(input_gradient.buffer, input_gradient.dimensions, input_gradient_alpha,
+                                             output_gradient.buffer, output_gradient.dimensions, weights.buffer,
+                                             weights.dimensions, workspace.buffer, ecount(workspace),
+                                             conv_descriptor, algorithms)
+    return input_gradient
+
+
 # ---------------------------------------------------------------- pooling
 
 POOL_OPERATIONS = ("max", "avg", "avg-exc-pad")

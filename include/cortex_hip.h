@@ -370,6 +370,52 @@ int ct_batch_normalize_gradients_spatial(void* stream, void* input_gradient, voi
                                          int64_t batch_count, int64_t channel_count,
                                          int64_t element_count, int dtype);
 
+/* The geometry of a convolution descriptor (src/cortex/tensor.clj:1320-1348). */
+typedef struct ct_conv_desc {
+  int32_t in_channels, out_channels;
+  int32_t kernel_width, kernel_height;
+  int32_t pad_x, pad_y;
+  int32_t stride_x, stride_y;
+} ct_conv_desc;
+
+/* convolution-forward! / -backward-weights! / -backward-data!
+ * (tensor/math.clj:185-220), decomposed as the CPU backend decomposes them
+ * (cpu/tensor_math.clj:1118-1151, 1670-1792): the input is unrolled into the
+ * caller's workspace as [batch, out_height * out_width, in_channels *
+ * kernel_height * kernel_width] (padding reads 0), and the three methods are
+ * one gemm! per image around that matrix:
+ *   forward           output[b] = weights x unrolled[b]^T + output_alpha * output[b]
+ *   backward-weights  weight_gradient = sum over b of output_gradient[b] x unrolled[b],
+ *                     on top of weight_gradient_alpha * weight_gradient; it reads the
+ *                     workspace as the forward pass left it and not `input`
+ *   backward-data     unrolled[b] = output_gradient[b]^T x weights, rolled back into
+ *                     input_gradient by adding every cell to the input element it
+ *                     came from, windows in increasing (row, column) order;
+ *                     input_gradient is overwritten: the CPU backend replaces
+ *                     input_gradient_alpha by 0.0 (:1766)
+ * Buffers are packed: input [batch, in_channels, in_height, in_width], output
+ * [batch, out_channels, out_height, out_width], weights [out_channels,
+ * in_channels * kernel_height * kernel_width].  workspace_ecount must be at
+ * least batch * out_height * out_width * in_channels * kernel_height *
+ * kernel_width (choose-convolution-algorithms, :1670-1680).  Every window must
+ * lie inside the padded input, as the floor rule for convolution output sizes
+ * guarantees.  dtype is CT_F32 or CT_F64. */
+int ct_convolution_forward(void* stream, void* output, double output_alpha, const void* input,
+                           const void* weights, void* workspace, int64_t workspace_ecount,
+                           const ct_conv_desc* desc, int64_t batch_count, int64_t in_height,
+                           int64_t in_width, int64_t out_height, int64_t out_width, int dtype);
+int ct_convolution_backward_weights(void* stream, void* weight_gradient,
+                                    double weight_gradient_alpha, const void* output_gradient,
+                                    const void* input, void* workspace, int64_t workspace_ecount,
+                                    const ct_conv_desc* desc, int64_t batch_count,
+                                    int64_t in_height, int64_t in_width, int64_t out_height,
+                                    int64_t out_width, int dtype);
+int ct_convolution_backward_data(void* stream, void* input_gradient, double input_gradient_alpha,
+                                 const void* output_gradient, const void* weights, void* workspace,
+                                 int64_t workspace_ecount, const ct_conv_desc* desc,
+                                 int64_t batch_count, int64_t in_height, int64_t in_width,
+                                 int64_t out_height, int64_t out_width, int dtype);
+
 /* pooling-forward! / pooling-backward! (tensor/math.clj:221-236;
  * cpu/tensor_math.clj:1153-1284, 1800-1866; window walk src/cortex/nn/impl.clj:8-96).
  * Buffers are packed [batch_count, channel_count, height, width]; dtype is

@@ -22,6 +22,8 @@
 //   activation-gradient!     cpu/tensor_math.clj:1318-1362
 //   softmax (both forms)     cpu/tensor_math.clj:1037-1103
 //   batch-normalize (6 forms) cpu/tensor_math.clj:731-1033, 1558-1638
+//   convolution (3 methods)  cpu/tensor_math.clj:1118-1151, 1670-1792: unroll, gemm!,
+//                            roll back
 //   pooling (6 forms)        cpu/tensor_math.clj:1153-1284, 1800-1866 over the
 //                            window walk of src/cortex/nn/impl.clj:8-96
 //   gemm!, gemv!             cpu/tensor_math.clj:672-726, 1534-1556 and
@@ -818,6 +820,7 @@ struct PoolGeom {
   int64_t kw, kh, pad_x, pad_y, stride_x, stride_y;
 };
 
+// conv_addr (impl.clj:76-81) is passed to bodies that take six arguments.
 template <class Body>
 void pool_walk(const PoolGeom& g, Body body) {
   const int64_t min_x = -g.pad_x, min_y = -g.pad_y, max_x = g.in_w + g.pad_x, max_y = g.in_h + g.pad_y;
@@ -896,6 +899,69 @@ bool pool_geom(const ct_pool_desc* d, int64_t batch, int64_t channels, int64_t i
   *g = PoolGeom{channels, in_h, in_w, out_h, out_w, d->kernel_width, d->kernel_height, d->pad_x, d->pad_y,
                 d->stride_x, d->stride_y};
   return true;
+}
+
+// ------------------------------------------------------------------ convolution
+// planar-input->convolution! and convolution->planar-output!
+// (cpu/tensor_math.clj:1118-1151) over one image: the same window walk with
+// output-conv-addr = (out_y * out_w + out_x) * (channels * kh * kw) + chan * kh * kw
+// + k_y * kw + k_x (impl.clj:54-81).
+
+template <class T>
+void unroll_image(const T* in, T* conv, const PoolGeom& g) {
+  const int64_t kk = g.kw * g.kh, n_cols = kk * g.channels;
+  pool_walk(g, [&](int64_t ia, int64_t oa, int64_t k_idx, bool valid, int64_t) {
+    const int64_t chan = oa / (g.out_w * g.out_h), offset = oa % (g.out_w * g.out_h);
+    conv[offset * n_cols + chan * kk + k_idx] = valid ? in[ia] : (T)0.0;
+  });
+}
+
+template <class T>
+void roll_image(const T* conv, T* ig, const PoolGeom& g) {
+  const int64_t kk = g.kw * g.kh, n_cols = kk * g.channels;
+  pool_walk(g, [&](int64_t ia, int64_t oa, int64_t k_idx, bool valid, int64_t) {
+    if (!valid) return;
+    const int64_t chan = oa / (g.out_w * g.out_h), offset = oa % (g.out_w * g.out_h);
+    ig[ia] = (T)((double)conv[offset * n_cols + chan * kk + k_idx] + (double)ig[ia]);
+  });
+}
+
+bool conv_geom(const ct_conv_desc* d, int64_t batch, int64_t in_h, int64_t in_w, int64_t out_h, int64_t out_w,
+               PoolGeom* g) {
+  if (!d || batch < 0 || in_h < 0 || in_w < 0 || out_h < 0 || out_w < 0) return false;
+  if (d->in_channels < 1 || d->out_channels < 1 || d->kernel_width < 1 || d->kernel_height < 1 ||
+      d->stride_x < 1 || d->stride_y < 1 || d->pad_x < 0 || d->pad_y < 0)
+    return false;
+  *g = PoolGeom{d->in_channels, in_h, in_w, out_h, out_w, d->kernel_width, d->kernel_height, d->pad_x, d->pad_y,
+                d->stride_x, d->stride_y};
+  return true;
+}
+
+template <class T>
+int convolution_t(int which, T* dest, double alpha, const T* other, const T* weights, T* workspace,
+                  int64_t workspace_ecount, const ct_conv_desc* d, int64_t batch, const PoolGeom& g) {
+  const int64_t n_rows = g.out_h * g.out_w, n_cols = g.kw * g.kh * g.channels, out_ch = d->out_channels;
+  const int64_t in_img = g.channels * g.in_h * g.in_w, out_img = out_ch * n_rows, conv_img = n_rows * n_cols;
+  if (workspace_ecount < batch * conv_img) return fail("convolution: workspace too small");
+  if (which == 0) {  // forward (:1682-1714): dest = output, other = input
+    for (int64_t b = 0; b < batch; ++b) {
+      unroll_image(other + b * in_img, workspace + b * conv_img, g);
+      gemm_t<T>(dest + b * out_img, n_rows, false, true, 1.0, weights, out_ch, n_cols, n_cols, workspace + b * conv_img,
+                n_rows, n_cols, alpha);
+    }
+  } else if (which == 1) {  // backward-weights (:1716-1747): dest = weight gradient, other = output gradient
+    for (int64_t b = 0; b < batch; ++b)
+      gemm_t<T>(dest, n_cols, false, false, 1.0, other + b * out_img, out_ch, n_rows, n_rows, workspace + b * conv_img,
+                n_cols, n_cols, b == 0 ? alpha : 1.0);
+  } else {  // backward-data (:1749-1792): dest = input gradient, other = output gradient
+    for (int64_t i = 0; i < batch * in_img; ++i) dest[i] = (T)0;
+    for (int64_t b = 0; b < batch; ++b) {
+      gemm_t<T>(workspace + b * conv_img, n_cols, true, false, 1.0, other + b * out_img, n_rows, out_ch, n_rows, weights,
+                n_cols, n_cols, 0.0);
+      roll_image(workspace + b * conv_img, dest + b * in_img, g);
+    }
+  }
+  return 0;
 }
 
 }  // namespace
@@ -1314,6 +1380,38 @@ int co_pooling_backward(void* input_gradient, double, const void* input, const v
                           desc->pool_op);
   }
   return 0;
+}
+
+#define CONV_ENTRY(which, dest, alpha, other, weights)                                                                  \
+  PoolGeom g;                                                                                                           \
+  if (!conv_geom(desc, batch_count, in_height, in_width, out_height, out_width, &g))                                    \
+    return fail("convolution: bad descriptor or counts");                                                              \
+  if (dtype == CT_F32)                                                                                                  \
+    return convolution_t<float>(which, (float*)dest, alpha, (const float*)other, (const float*)weights,                 \
+                                (float*)workspace, workspace_ecount, desc, batch_count, g);                            \
+  if (dtype == CT_F64)                                                                                                  \
+    return convolution_t<double>(which, (double*)dest, alpha, (const double*)other, (const double*)weights,             \
+                                 (double*)workspace, workspace_ecount, desc, batch_count, g);                          \
+  return fail("convolution is only defined for float and double tensors")
+
+int co_convolution_forward(void* output, double output_alpha, const void* input, const void* weights, void* workspace,
+                           int64_t workspace_ecount, const ct_conv_desc* desc, int64_t batch_count, int64_t in_height,
+                           int64_t in_width, int64_t out_height, int64_t out_width, int dtype) {
+  CONV_ENTRY(0, output, output_alpha, input, weights);
+}
+
+int co_convolution_backward_weights(void* weight_gradient, double weight_gradient_alpha, const void* output_gradient,
+                                    const void*, void* workspace, int64_t workspace_ecount, const ct_conv_desc* desc,
+                                    int64_t batch_count, int64_t in_height, int64_t in_width, int64_t out_height,
+                                    int64_t out_width, int dtype) {
+  CONV_ENTRY(1, weight_gradient, weight_gradient_alpha, output_gradient, nullptr);
+}
+
+int co_convolution_backward_data(void* input_gradient, double, const void* output_gradient, const void* weights,
+                                 void* workspace, int64_t workspace_ecount, const ct_conv_desc* desc,
+                                 int64_t batch_count, int64_t in_height, int64_t in_width, int64_t out_height,
+                                 int64_t out_width, int dtype) {
+  CONV_ENTRY(2, input_gradient, 0.0, output_gradient, weights);
 }
 
 // One Philox4x32-10 block, for the known-answer tests.

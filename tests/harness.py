@@ -227,6 +227,20 @@ def softmax(side, out: View, inp: View, spatial=False):
     side.call("softmax_spatial" if spatial else "softmax_eltwise", *_pd(side, out), *_pd(side, inp), out.buf.dtype)
 
 
+def conv_desc(in_channels, out_channels, kw, kh, px, py, sx, sy):
+    return {"in-channels": in_channels, "out-channels": out_channels, "kernel-width": kw, "kernel-height": kh,
+            "pad-x": px, "pad-y": py, "stride-x": sx, "stride-y": sy}
+
+
+def convolution(side, which, dest: View, alpha, a: View, b: View, workspace: View, desc, batch, in_h, in_w, out_h,
+                out_w):
+    """which: "forward" (dest output, a input, b weights), "backward_weights" (dest weight gradient, a output
+    gradient, b input), "backward_data" (dest input gradient, a output gradient, b weights)."""
+    d = capi.make_conv_desc(desc)
+    side.call("convolution_" + which, side.ptr(dest), float(alpha), side.ptr(a), side.ptr(b), side.ptr(workspace),
+              int(np.prod(workspace.shape)), C.byref(d), batch, in_h, in_w, out_h, out_w, dest.buf.dtype)
+
+
 def pool_desc(kw, kh, px, py, sx, sy, op):
     return {"kernel-width": kw, "kernel-height": kh, "pad-x": px, "pad-y": py, "stride-x": sx, "stride-y": sy,
             "pool-op": op}

@@ -60,6 +60,32 @@ def single(node, batch_size, input, output_gradient, parameters=None, item_shape
             "input-gradient": ct.to_double_array(inputs[0]["gradient"]).reshape(-1), "layer": layer}
 
 
+# verify/nn/layers.clj:502-553: kernels k = 1..n of constant value k, bias 1
+def basic_conv_layer(driver, datatype):
+    with context(driver, datatype):
+        batch_size, channel_count = 10, 4
+        cases = (
+            ({"channels": 1, "height": 3, "width": 3}, list(range(1, 10)),
+             [13, 17, 25, 29, 25, 33, 49, 57, 37, 49, 73, 85, 49, 65, 97, 113], [120, 160, 240, 280], 4,
+             [1, 2, 1, 2, 4, 2, 1, 2, 1]),
+            ({"channels": 1, "height": 4, "width": 3}, list(range(1, 13)),
+             [13, 17, 25, 29, 37, 41, 25, 33, 49, 57, 73, 81, 37, 49, 73, 85, 109, 121, 49, 65, 97, 113, 145, 161],
+             [270, 330, 450, 510], 6, [1, 2, 1, 2, 4, 2, 2, 4, 2, 1, 2, 1]),
+        )
+        for dimension, item, want_output, want_weight_gradient, outputs_per_kernel, want_input_gradient in cases:
+            node = nl.convolutional(2, 0, 1, channel_count, dimension)
+            d = node["output-dimension"]
+            params = {"weights": entry([[k] * (2 * 2 * dimension["channels"]) for k in range(1, channel_count + 1)]),
+                      "bias": entry([1] * channel_count)}
+            n_out = d["channels"] * d["height"] * d["width"]
+            r = single(node, batch_size, item * batch_size, [1] * (n_out * batch_size), parameters=params,
+                       output_item_shape=[n_out])
+            equals(want_output * batch_size, r["output"])
+            equals(want_weight_gradient * 4, ct.to_double_array(params["weights"]["gradient"]))
+            equals([outputs_per_kernel * batch_size] * 4, ct.to_double_array(params["bias"]["gradient"]))
+            equals([10.0 * v for v in want_input_gradient] * batch_size, r["input-gradient"])
+
+
 def _pool(node, batch_size, input, output_gradient):
     d = node["output-dimension"]
     return single(node, batch_size, input, output_gradient,

@@ -189,6 +189,33 @@ class OracleStream:
         ob.call("batch_normalize_gradients_spatial", ig.ptr, sg.ptr, bg.ptr, og.ptr, out.ptr, inp.ptr, bm.ptr, bv.ptr,
                 scale.ptr, bias.ptr, float(eps), int(batch), int(chans), int(elems), capi.DTYPE_CODES[ig.datatype])
 
+    def convolution_descriptor(self, *args):
+        return None
+
+    def choose_convolution_algorithms(self, desc, input_width, input_height, output_width, output_height, batch_size,
+                                      max_ideal_workspace_size, use_defaults):
+        n_cols = int(desc["kernel-width"]) * int(desc["kernel-height"]) * int(desc["in-channels"])
+        return {"workspace-size": n_cols * int(output_width) * int(output_height) * int(batch_size)}
+
+    def _conv(self, name, dest, alpha, a, b, workspace, workspace_ecount, desc, in_shape, out_shape):
+        batch, _, in_h, in_w = (int(v) for v in in_shape)
+        out_h, out_w = (int(v) for v in out_shape[2:])
+        ob.call(name, dest.ptr, float(alpha), a.ptr, b.ptr, workspace.ptr, int(workspace_ecount),
+                C.byref(capi.make_conv_desc(desc)), int(out_shape[0]), in_h, in_w, out_h, out_w,
+                capi.DTYPE_CODES[dest.datatype])
+
+    def convolution_forward(self, out, od, out_alpha, inp, idims, weights, wd, workspace, ecount, desc, algorithms):
+        self._conv("convolution_forward", out, out_alpha, inp, weights, workspace, ecount, desc, idims["shape"],
+                   od["shape"])
+
+    def convolution_backward_weights(self, wg, wgd, wg_alpha, og, ogd, inp, idims, workspace, ecount, desc, algorithms):
+        self._conv("convolution_backward_weights", wg, wg_alpha, og, inp, workspace, ecount, desc, idims["shape"],
+                   ogd["shape"])
+
+    def convolution_backward_data(self, ig, igd, ig_alpha, og, ogd, weights, wd, workspace, ecount, desc, algorithms):
+        self._conv("convolution_backward_data", ig, ig_alpha, og, weights, workspace, ecount, desc, igd["shape"],
+                   ogd["shape"])
+
     def pooling_forward(self, out, od, out_alpha, inp, idims, desc):
         batch, channels, in_h, in_w = (int(v) for v in idims["shape"])
         out_h, out_w = (int(v) for v in od["shape"][2:])

@@ -251,6 +251,35 @@ def softmax(driver, datatype):
         equals(([0, 1] + list(ct.to_double_array(answer))) * 5, ct.to_double_array(pred_matrix))
 
 
+# verify/tensor.clj:808-890
+def convolution_operator(driver, datatype):
+    with context(driver, datatype):
+        want = GOLDEN["convolution_operator"]
+        batch_size, num_in_channels, num_out_channels, input_dim = 3, 4, 3, 4
+        n = input_dim * input_dim * batch_size * num_in_channels
+        inp = ct.to_tensor(np.arange(n, dtype=np.float64).reshape(batch_size, num_in_channels, input_dim, input_dim))
+        conv_desc = ct.convolution_descriptor(datatype, num_out_channels, num_in_channels, 3, 3, 0, 0, 1, 1)
+        dims_ = ct.get_convolution_output_dimensions(conv_desc, input_dim, input_dim)
+        ow, oh = dims_["output-width"], dims_["output-height"]
+        output = ct.new_tensor([batch_size, num_out_channels, oh, ow])
+        output_gradient = ct.to_tensor(np.ones([batch_size, num_out_channels, oh, ow]))
+        algorithms = ct.choose_convolution_algorithms(conv_desc, input_dim, input_dim, batch_size, 1000)
+        workspace = ct.new_tensor([algorithms["workspace-size"]])
+        weights = ct.to_tensor(np.arange(num_out_channels * 9 * num_in_channels, dtype=np.float64)
+                               .reshape(num_out_channels, 9 * num_in_channels))
+        weight_gradient = ct.new_tensor(ct.shape(weights))
+        input_gradient = ct.new_tensor(ct.shape(inp))
+        # make sure that pre-existing contents are overwritten
+        for t in (output, weight_gradient, input_gradient):
+            ct.assign(t, 1)
+        ct.convolution_forward(output, 0.0, inp, weights, workspace, conv_desc, algorithms)
+        equals(want["forward"], ct.to_double_array(output))
+        ct.convolution_backward_weights(weight_gradient, 0.0, output_gradient, inp, workspace, conv_desc, algorithms)
+        equals(want["backward_weights"], ct.to_double_array(weight_gradient))
+        ct.convolution_backward_data(input_gradient, 0.0, output_gradient, weights, workspace, conv_desc, algorithms)
+        equals(want["backward_data"], ct.to_double_array(input_gradient))
+
+
 # verify/tensor.clj:893-1051
 def pooling_operator(driver, datatype):
     with context(driver, datatype):

@@ -824,6 +824,90 @@ def test_rand_errors(P):
 # double accumulator.  Bar: |got - want| <= tol * (|alpha| sum |a||b| + |beta c|) with
 # tol = 1e-5 for float (k up to 512 terms of 2^-24 relative error each) and 1e-13 for double.
 
+# ------------------------------------------------------------------ convolution
+# (batch, in channels, out channels, height, width, kw, kh, px, py, sx, sy)
+CONV_CASES = [
+    (3, 4, 3, 4, 4, 3, 3, 0, 0, 1, 1),       # the reference's own test geometry
+    (2, 3, 5, 9, 11, 3, 3, 1, 1, 1, 1),      # 27 cells per row: cell-by-cell stores
+    (2, 4, 6, 12, 10, 3, 3, 1, 1, 2, 2),     # 36 cells per row: 16-byte stores
+    (1, 2, 3, 8, 8, 2, 2, 0, 0, 2, 2),
+    (2, 1, 4, 7, 9, 5, 3, 2, 1, 2, 1),       # rectangular window
+    (1, 8, 16, 14, 14, 1, 1, 0, 0, 1, 1),    # 1 x 1: the unrolled matrix is the transposed input
+    (4, 16, 32, 28, 28, 3, 3, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("case", CONV_CASES, ids=str)
+def test_convolution(P, code, case):
+    batch, cin, cout, h, w, kw, kh, px, py, sx, sy = case
+    oh, ow = (h + 2 * py - kh) // sy + 1, (w + 2 * px - kw) // sx + 1
+    n_cols, n_rows = cin * kh * kw, oh * ow
+    rng = np.random.default_rng(55)
+    desc = H.conv_desc(cin, cout, kw, kh, px, py, sx, sy)
+    geom = (desc, batch, h, w, oh, ow)
+    inp = P.buf(values(rng, code, batch * cin * h * w))
+    weights = P.buf(values(rng, code, cout * n_cols) / 8)
+    out = P.buf(values(rng, code, batch * cout * n_rows))            # overwritten (alpha 0), then added onto
+    work = P.buf(np.full(batch * n_rows * n_cols + 5, 7.0, NP[code]))
+    og = P.buf(values(rng, code, batch * cout * n_rows))
+    wg = P.buf(values(rng, code, cout * n_cols))
+    ig = P.buf(values(rng, code, batch * cin * h * w))
+    V = lambda b: View(b, [b.init.size])
+    tol = 2e-5 if code == capi.F32 else 1e-12
+
+    def close(buf, scale, what):
+        got, want = buf.download().astype(np.float64), buf.host.astype(np.float64)
+        assert np.all(np.abs(got - want) <= tol * scale), f"{what} {case}: {np.abs(got - want).max()} vs {tol * scale}"
+
+    x64, w64, g64 = (b.init.astype(np.float64) for b in (inp, weights, og))
+    P.run(H.convolution, "forward", V(out), 0.0, V(inp), V(weights), V(work), *geom)
+    compare(work, f"unrolled input {case}")                             # a copy: bit-exact, the slack untouched
+    scale = np.abs(w64).max() * np.abs(x64).max() * n_cols
+    close(out, scale, "convolution-forward")
+    P.run(H.convolution, "forward", V(out), 0.5, V(inp), V(weights), V(work), *geom)
+    close(out, 2 * scale, "convolution-forward onto half the output")
+    P.run(H.convolution, "backward_weights", V(wg), 0.0, V(og), V(inp), V(work), *geom)
+    close(wg, np.abs(g64).max() * np.abs(x64).max() * n_rows * batch, "convolution-backward-weights")
+    P.run(H.convolution, "backward_weights", V(wg), 1.0, V(og), V(inp), V(work), *geom)
+    close(wg, 2 * np.abs(g64).max() * np.abs(x64).max() * n_rows * batch, "convolution-backward-weights, accumulated")
+    P.run(H.convolution, "backward_data", V(ig), 0.0, V(og), V(weights), V(work), *geom)
+    close(ig, np.abs(g64).max() * np.abs(w64).max() * cout * kh * kw, "convolution-backward-data")
+
+
+def test_convolution_roll_back_is_bit_exact(P):
+    """With integer-valued operands every product and sum is exact, so the input gradient must
+    agree to the bit whatever order the gemm sums in; the gather then adds windows in the
+    reference's order."""
+    rng = np.random.default_rng(56)
+    batch, cin, cout, h, w, k = 2, 3, 4, 10, 9, 3
+    oh, ow = h - k + 1 + 2, w - k + 1 + 2      # pad 1, stride 1
+    desc = H.conv_desc(cin, cout, k, k, 1, 1, 1, 1)
+    og = P.buf(rng.integers(-3, 4, batch * cout * oh * ow).astype(np.float32))
+    weights = P.buf(rng.integers(-3, 4, cout * cin * k * k).astype(np.float32))
+    work = P.buf(np.zeros(batch * oh * ow * cin * k * k, np.float32))
+    ig = P.buf(np.ones(batch * cin * h * w, np.float32))
+    V = lambda b: View(b, [b.init.size])
+    P.run(H.convolution, "backward_data", V(ig), 0.0, V(og), V(weights), V(work), desc, batch, h, w, oh, ow)
+    compare(work, "unrolled gradient")
+    compare(ig, "input gradient")
+
+
+def test_convolution_errors(P):
+    b = P.buf(np.zeros(4096, np.float32))
+    v = View(b, [4096])
+    good = H.conv_desc(2, 3, 3, 3, 0, 0, 1, 1)
+    with pytest.raises(capi.CortexHipError, match="workspace"):
+        H.convolution(P.hip, "forward", v, 0.0, v, v, View(b, [10]), good, 1, 6, 6, 4, 4)
+    with pytest.raises(capi.CortexHipError, match="beyond the padded input"):
+        H.convolution(P.hip, "forward", v, 0.0, v, v, v, good, 1, 6, 6, 5, 5)
+    with pytest.raises(capi.CortexHipError):
+        H.convolution(P.hip, "forward", v, 0.0, v, v, v, H.conv_desc(0, 3, 3, 3, 0, 0, 1, 1), 1, 6, 6, 4, 4)
+    ints = P.buf(np.zeros(4096, np.int32))
+    with pytest.raises(capi.CortexHipError, match="float and double"):
+        H.convolution(P.hip, "forward", View(ints, [4096]), 0.0, v, v, v, good, 1, 6, 6, 4, 4)
+
+
 # ------------------------------------------------------------------ pooling
 # (batch, channels, height, width, kw, kh, px, py, sx, sy, dimension-op)
 POOL_CASES = [

@@ -778,3 +778,45 @@ def test_average_pooling_backward_is_the_adjoint_of_forward():
         H.pooling_backward(ORACLE, View(ig, [x.size]), View(inp, [x.size]), View(out, [g.size]), View(grad, [g.size]),
                            desc, 2, 1, h, w, oh, ow)
         assert abs(np.dot(out.host, g) - np.dot(x, ig.host)) < 1e-10
+
+
+# ------------------------------------------------------------------ convolution against scipy's correlation
+
+@pytest.mark.parametrize("geometry", [(5, 6, 3, 3, 0, 0, 1, 1), (7, 7, 3, 3, 1, 1, 2, 2), (6, 9, 2, 3, 1, 0, 1, 2)], ids=str)
+def test_convolution_matches_correlation(geometry):
+    from scipy.signal import correlate2d
+    h, w, kw, kh, px, py, sx, sy = geometry
+    batch, cin, cout = 2, 3, 4
+    oh, ow = (h + 2 * py - kh) // sy + 1, (w + 2 * px - kw) // sx + 1
+    rng = np.random.default_rng(62)
+    x = rng.standard_normal((batch, cin, h, w))
+    wt = rng.standard_normal((cout, cin, kh, kw))
+    g = rng.standard_normal((batch, cout, oh, ow))
+    desc = H.conv_desc(cin, cout, kw, kh, px, py, sx, sy)
+    n_rows, n_cols = oh * ow, cin * kh * kw
+    inp, weights, grad = hbuf(x.reshape(-1)), hbuf(wt.reshape(-1)), hbuf(g.reshape(-1))
+    out, work = hbuf(np.full(batch * cout * n_rows, 9.0)), hbuf(np.zeros(batch * n_rows * n_cols))
+    wg, ig = hbuf(np.full(cout * n_cols, 9.0)), hbuf(np.full(x.size, 9.0))
+    V = lambda b: View(b, [b.host.size])
+    geom = (desc, batch, h, w, oh, ow)
+    H.convolution(ORACLE, "forward", V(out), 0.0, V(inp), V(weights), V(work), *geom)
+    padded = np.pad(x, ((0, 0), (0, 0), (py, py), (px, px)))
+    want = np.zeros((batch, cout, oh, ow))
+    for b in range(batch):
+        for o in range(cout):
+            full = sum(correlate2d(padded[b, c], wt[o, c], mode="valid") for c in range(cin))
+            want[b, o] = full[::sy, ::sx][:oh, :ow]
+    np.testing.assert_allclose(out.host.reshape(want.shape), want, rtol=1e-12, atol=1e-12)
+    # the gradients as the adjoints of the forward map: <conv(x, W), g> is linear in x and in W
+    H.convolution(ORACLE, "backward_weights", V(wg), 0.0, V(grad), V(inp), V(work), *geom)
+    H.convolution(ORACLE, "backward_data", V(ig), 0.0, V(grad), V(weights), V(work), *geom)
+    inner = np.dot(want.reshape(-1), g.reshape(-1))
+    assert abs(np.dot(wg.host, wt.reshape(-1)) - inner) < 1e-9 * max(1.0, abs(inner))
+    assert abs(np.dot(ig.host, x.reshape(-1)) - inner) < 1e-9 * max(1.0, abs(inner))
+    # finite differences pin the gradients element by element, not just their projections
+    eps = 1e-6
+    for idx in (0, x.size // 2, x.size - 1):
+        bumped = x.reshape(-1).copy(); bumped[idx] += eps
+        o2, w2 = hbuf(np.zeros(out.host.size)), hbuf(np.zeros(work.host.size))
+        H.convolution(ORACLE, "forward", V(o2), 0.0, V(hbuf(bumped)), V(weights), V(w2), *geom)
+        assert abs(np.dot(o2.host - out.host, g.reshape(-1)) / eps - ig.host[idx]) < 1e-5
