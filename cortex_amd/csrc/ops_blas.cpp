@@ -35,6 +35,8 @@ struct RocblasApi {
   decltype(&rocblas_set_pointer_mode) set_pointer_mode = nullptr;
   decltype(&rocblas_sgemm) sgemm = nullptr;
   decltype(&rocblas_dgemm) dgemm = nullptr;
+  decltype(&rocblas_sgemm_strided_batched) sgemm_batched = nullptr;
+  decltype(&rocblas_dgemm_strided_batched) dgemm_batched = nullptr;
   decltype(&rocblas_status_to_string) status_to_string = nullptr;
   bool ok = false;
   char why[256] = "";
@@ -63,6 +65,8 @@ RocblasApi* rocblas_api() {
     CT_SYM(set_pointer_mode, rocblas_set_pointer_mode)
     CT_SYM(sgemm, rocblas_sgemm)
     CT_SYM(dgemm, rocblas_dgemm)
+    CT_SYM(sgemm_batched, rocblas_sgemm_strided_batched)
+    CT_SYM(dgemm_batched, rocblas_dgemm_strided_batched)
     CT_SYM(status_to_string, rocblas_status_to_string)
 #undef CT_SYM
     api.ok = true;
@@ -118,6 +122,45 @@ inline rocblas_operation op_of(bool trans) { return trans ? rocblas_operation_tr
 inline bool fits_int(int64_t v) { return v >= 0 && v <= 2147483647; }
 
 }  // namespace
+
+namespace cthip {
+
+// `batch_count` products of ct_gemm's form in one launch: product i reads
+// a + i * a_stride, b + i * b_stride and writes c + i * c_stride (strides in
+// elements; 0 shares an operand among the products).  Used by the convolution
+// methods, whose per-image products are too small to fill the device one at a time.
+int gemm_strided_batched(void* stream, void* c, int64_t c_colstride, int64_t c_stride, int trans_a, int trans_b,
+                         double alpha, const void* a, int64_t a_row_count, int64_t a_col_count, int64_t a_colstride,
+                         int64_t a_stride, const void* b, int64_t b_col_count, int64_t b_colstride, int64_t b_stride,
+                         double beta, int64_t batch_count, int dtype) {
+  CT_REQUIRE(dtype == CT_F32 || dtype == CT_F64, "gemm! is only defined for float and double tensors");
+  CT_REQUIRE(a && b && c, "gemm: null buffer");
+  CT_REQUIRE(fits_int(a_row_count) && fits_int(a_col_count) && fits_int(b_col_count) && fits_int(a_colstride) &&
+                 fits_int(b_colstride) && fits_int(c_colstride) && fits_int(batch_count),
+             "gemm: a size is negative or exceeds 2^31 - 1");
+  if (a_row_count == 0 || b_col_count == 0 || batch_count == 0) return CT_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  RocblasApi* api;
+  rocblas_handle h;
+  if (int rc = blas_handle(s, &api, &h)) return rc;
+  note_kernel("rocblas_gemm_strided_batched");
+  const rocblas_int m = (rocblas_int)b_col_count, n = (rocblas_int)a_row_count, k = (rocblas_int)a_col_count;
+  if (dtype == CT_F32) {
+    const float al = (float)alpha, be = (float)beta;
+    CT_BLAS(api, api->sgemm_batched(h, op_of(trans_b), op_of(trans_a), m, n, k, &al, (const float*)b,
+                                    (rocblas_int)b_colstride, b_stride, (const float*)a, (rocblas_int)a_colstride,
+                                    a_stride, &be, (float*)c, (rocblas_int)c_colstride, c_stride,
+                                    (rocblas_int)batch_count));
+  } else {
+    CT_BLAS(api, api->dgemm_batched(h, op_of(trans_b), op_of(trans_a), m, n, k, &alpha, (const double*)b,
+                                    (rocblas_int)b_colstride, b_stride, (const double*)a, (rocblas_int)a_colstride,
+                                    a_stride, &beta, (double*)c, (rocblas_int)c_colstride, c_stride,
+                                    (rocblas_int)batch_count));
+  }
+  return after_launch(s);
+}
+
+}  // namespace cthip
 
 extern "C" {
 

@@ -5,7 +5,11 @@
 // unrolled into the caller's workspace, one row of in_channels * kh * kw cells
 // per output position (window walk: src/cortex/nn/impl.clj:8-96), and each
 // method is one gemm! per image around that matrix.  The two data movements are
-// the kernels of this file; the products go through ct_gemm (rocBLAS).
+// the kernels of this file; the per-image products go to rocBLAS as ONE
+// strided-batched call per method (an image's product alone leaves most of the
+// device idle).  The weight gradient, which the reference accumulates image
+// after image into one matrix, is formed as per-image products in the stream's
+// scratch memory and summed over the images in double by a small kernel.
 //
 //   unroll     one lane per workspace cell, 16 bytes of cells per lane where a
 //              row of cells is a whole number of them: the writes, kh * kw times
@@ -22,9 +26,12 @@
 
 using namespace cthip;
 
-extern "C" int ct_gemm(void* stream, void* c, int64_t c_colstride, int trans_a, int trans_b, double alpha,
-                       const void* a, int64_t a_row_count, int64_t a_col_count, int64_t a_colstride, const void* b,
-                       int64_t b_col_count, int64_t b_colstride, double beta, int dtype);
+namespace cthip {
+int gemm_strided_batched(void* stream, void* c, int64_t c_colstride, int64_t c_stride, int trans_a, int trans_b,
+                         double alpha, const void* a, int64_t a_row_count, int64_t a_col_count, int64_t a_colstride,
+                         int64_t a_stride, const void* b, int64_t b_col_count, int64_t b_colstride, int64_t b_stride,
+                         double beta, int64_t batch_count, int dtype);
+}
 
 namespace {
 
@@ -205,32 +212,62 @@ int forward_t(void* stream, T* output, double output_alpha, const T* input, cons
   hipStream_t s = static_cast<hipStream_t>(stream);
   unroll(s, input, workspace, d, sh);
   if (int rc = after_launch(s)) return rc;
-  for (int64_t b = 0; b < sh.batch; ++b)
-    if (int rc = ct_gemm(stream, output + b * sh.out_image, sh.n_rows, 0, 1, 1.0, weights, d.out_channels, sh.n_cols,
-                         sh.n_cols, workspace + b * sh.conv_image, sh.n_rows, sh.n_cols, output_alpha, dtype))
-      return rc;
+  // output[b] [out_channels, n_rows] = weights [out_channels, n_cols] x unrolled[b]^T
+  if (int rc = gemm_strided_batched(stream, output, sh.n_rows, sh.out_image, 0, 1, 1.0, weights, d.out_channels,
+                                    sh.n_cols, sh.n_cols, 0, workspace, sh.n_rows, sh.n_cols, sh.conv_image,
+                                    output_alpha, sh.batch, dtype))
+    return rc;
   note_kernel("conv_unroll+gemm");
   return CT_OK;
+}
+
+// weight_gradient = T(alpha * weight_gradient + sum over the images of partial[image]), in double
+template <class T>
+__global__ void __launch_bounds__(kBlock) conv_sum_partials_kernel(T* weight_gradient, const T* partials, uint32_t n,
+                                                                    uint32_t images, double alpha) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  double acc = alpha == 0.0 ? 0.0 : alpha * (double)weight_gradient[i];
+  for (uint32_t b = 0; b < images; ++b) acc += (double)partials[(int64_t)b * n + i];
+  weight_gradient[i] = (T)acc;
 }
 
 template <class T>
 int backward_weights_t(void* stream, T* weight_gradient, double alpha, const T* output_gradient, T* workspace,
                        const ct_conv_desc& d, const ConvShape& sh, int dtype) {
-  for (int64_t b = 0; b < sh.batch; ++b)
-    if (int rc = ct_gemm(stream, weight_gradient, sh.n_cols, 0, 0, 1.0, output_gradient + b * sh.out_image,
-                         d.out_channels, sh.n_rows, sh.n_rows, workspace + b * sh.conv_image, sh.n_cols, sh.n_cols,
-                         b == 0 ? alpha : 1.0, dtype))
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t n = (int64_t)d.out_channels * sh.n_cols;
+  CT_REQUIRE(n <= (int64_t(1) << 31) - 1, "convolution: the weight matrix exceeds the supported range");
+  // images per pass: partial products of at most 256 MiB
+  const int64_t per_pass = std::max<int64_t>(1, std::min<int64_t>(sh.batch, (int64_t(256) << 20) / (n * (int64_t)sizeof(T))));
+  void* scratch = nullptr;
+  if (int rc = stream_scratch(s, (size_t)(per_pass * n) * sizeof(T), &scratch)) return rc;
+  const T al = (T)alpha;
+  for (int64_t b0 = 0; b0 < sh.batch; b0 += per_pass) {
+    const int64_t nb = std::min(per_pass, sh.batch - b0);
+    // partial[b] [out_channels, n_cols] = output_gradient[b] [out_channels, n_rows] x unrolled[b] [n_rows, n_cols]
+    if (int rc = gemm_strided_batched(stream, scratch, sh.n_cols, n, 0, 0, 1.0, output_gradient + b0 * sh.out_image,
+                                      d.out_channels, sh.n_rows, sh.n_rows, sh.out_image,
+                                      workspace + b0 * sh.conv_image, sh.n_cols, sh.n_cols, sh.conv_image, 0.0, nb,
+                                      dtype))
       return rc;
-  return CT_OK;
+    hipLaunchKernelGGL((conv_sum_partials_kernel<T>), dim3((uint32_t)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+                       weight_gradient, reinterpret_cast<const T*>(scratch), (uint32_t)n, (uint32_t)nb,
+                       b0 == 0 ? (double)al : 1.0);
+  }
+  note_kernel("gemm+conv_sum_partials");
+  return after_launch(s);
 }
 
 template <class T>
 int backward_data_t(void* stream, T* input_gradient, const T* output_gradient, const T* weights, T* workspace,
                     const ct_conv_desc& d, const ConvShape& sh, int dtype) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  for (int64_t b = 0; b < sh.batch && sh.conv_image > 0; ++b)
-    if (int rc = ct_gemm(stream, workspace + b * sh.conv_image, sh.n_cols, 1, 0, 1.0, output_gradient + b * sh.out_image,
-                         sh.n_rows, d.out_channels, sh.n_rows, weights, sh.n_cols, sh.n_cols, 0.0, dtype))
+  // unrolled[b] [n_rows, n_cols] = output_gradient[b]^T [n_rows, out_channels] x weights [out_channels, n_cols]
+  if (sh.conv_image > 0)
+    if (int rc = gemm_strided_batched(stream, workspace, sh.n_cols, sh.conv_image, 1, 0, 1.0, output_gradient, sh.n_rows,
+                                      d.out_channels, sh.n_rows, sh.out_image, weights, sh.n_cols, sh.n_cols, 0, 0.0,
+                                      sh.batch, dtype))
       return rc;
   roll_back(s, workspace, input_gradient, d, sh);
   note_kernel("gemm+conv_roll");
