@@ -255,6 +255,32 @@ def run_adjacent(drv, device, stream, timer, capi) -> dict:
                                                                          out_dims, desc), 20)
         out[f"pooling-backward! {label}"] = entry(4 * (2 * n + n_out) + (4 * (n + n_out) if pool_op == "max" else 0), ms)
 
+    # convolution as the CPU backend decomposes it (unroll, gemm!, roll back): priced like gemm!
+    cb, cc, ck, chw = 64, 64, 64, 56
+    conv_desc = {"in-channels": cc, "out-channels": ck, "kernel-width": 3, "kernel-height": 3, "pad-x": 1, "pad-y": 1,
+                 "stride-x": 1, "stride-y": 1}
+    c_in, c_out = dims([cb, cc, chw, chw]), dims([cb, ck, chw, chw])
+    n_cols, n_rows = cc * 9, chw * chw
+    w_ = upload(drv, device, stream, (rng.standard_normal(ck * n_cols, dtype=np.float32) / 24))
+    work = device.allocate_device_buffer(cb * n_rows * n_cols, "float")
+    wgrad = device.allocate_device_buffer(ck * n_cols, "float")
+    w_dims = dims([ck, n_cols])
+    conv_flops = 2.0 * cb * ck * n_rows * n_cols
+    conv_calls = (
+        ("convolution-forward!", lambda: stream.convolution_forward(o, c_out, 0.0, x, c_in, w_, w_dims, work,
+                                                                    cb * n_rows * n_cols, conv_desc, None)),
+        ("convolution-backward-weights!", lambda: stream.convolution_backward_weights(
+            wgrad, w_dims, 0.0, g, c_out, x, c_in, work, cb * n_rows * n_cols, conv_desc, None)),
+        ("convolution-backward-data!", lambda: stream.convolution_backward_data(
+            ig, c_in, 0.0, g, c_out, w_, w_dims, work, cb * n_rows * n_cols, conv_desc, None)),
+    )
+    for name, call in conv_calls:
+        ms = time_launches(timer, stream, call, 5, warm=2)
+        tflops = conv_flops / (ms * 1e-3) / 1e12
+        out[f"{name} f32 [{cb},{cc}->{ck},{chw},{chw}] 3x3 pad 1"] = {
+            "us": round(ms * 1e3, 1), "TFLOP/s": round(tflops, 1), "frac_of_fp32_matrix_peak": round(tflops / 157.3, 4),
+            "workspace_bytes": 4 * cb * n_rows * n_cols, "kernel": capi.last_kernel()}
+
     # gemm! is the one MFMA-bound method (rocBLAS); priced against the dense fp32 matrix peak
     m = 8192
     a_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))
