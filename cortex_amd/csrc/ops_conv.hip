@@ -2,24 +2,32 @@
 // convolution-backward-data! (src/cortex/tensor/math.clj:185-220) with the
 // decomposition of the reference's CPU backend
 // (src/cortex/compute/cpu/tensor_math.clj:1118-1151, 1670-1792): the input is
-// unrolled into the caller's workspace, one row of in_channels * kh * kw cells
-// per output position (window walk: src/cortex/nn/impl.clj:8-96), and each
-// method is one gemm! per image around that matrix.  The two data movements are
-// the kernels of this file; the per-image products go to rocBLAS as ONE
-// strided-batched call per method (an image's product alone leaves most of the
-// device idle).  The weight gradient, which the reference accumulates image
-// after image into one matrix, is formed as per-image products in the stream's
-// scratch memory and summed over the images in double by a small kernel.
+// unrolled into the caller's workspace (window walk: src/cortex/nn/impl.clj:8-96)
+// and each method is one gemm! per image around that matrix.
 //
-//   unroll     one lane per workspace cell, 16 bytes of cells per lane where a
-//              row of cells is a whole number of them: the writes, kh * kw times
-//              the volume of the reads, are linear and the reads come from the
-//              caches.  HBM-bound on the workspace it writes.
+// Workspace layout.  The CPU backend stores an image's unrolled input as
+// [position, in_channels * kh * kw]; here it is the transpose,
+// [in_channels * kh * kw, position] with position = out_y * out_w + out_x.  The
+// workspace is opaque to callers (they size it with choose-convolution-algorithms
+// and only hand it back), the products merely swap their transposition flags,
+// and with the positions innermost both data movements are linear on both sides:
+// neighbouring lanes read neighbouring input elements and write neighbouring
+// cells.  (With the CPU backend's layout the roll-back read 13 times its
+// algorithmic bytes from HBM and ran at 7 % of the peak, the unroll at 20 %.)
+//
+//   unroll     one lane per 16 bytes of cells of one (channel, tap) row: reads a
+//              run of input positions, writes one aligned piece.  HBM-bound on
+//              the workspace it writes, kh * kw times the input.
 //   roll back  the reference adds cell after cell into the input gradient while
 //              it walks the windows; here every input element gathers the cells
 //              that came from it, windows in increasing (row, column) order,
 //              which is the order in which that walk reaches the element: the
 //              same roundings, no atomics.  Reads the workspace once.
+//   products   ONE strided-batched rocBLAS call per method (an image's product
+//              alone leaves most of the device idle).  The weight gradient, which
+//              the reference accumulates image after image into one matrix, is
+//              formed as per-image products in the stream's scratch memory and
+//              summed over the images in double by a small kernel.
 #include <algorithm>
 
 #include "common.h"
@@ -48,31 +56,30 @@ struct ConvArgs {
   FastDiv in_w_fd, in_plane_fd, image_fd, sx_fd, sy_fd;  // roll back: element -> (image, channel, row, column)
 };
 
-// workspace[image][position][channel * kh * kw + k_y * kw + k_x] = input tap or 0 in the padding
+// workspace[image][channel * kh * kw + k_y * kw + k_x][position] = input tap or 0 in the padding
 template <class T, int VEC>
 __global__ void __launch_bounds__(kBlock) conv_unroll_kernel(const ConvArgs a) {
   const uint32_t lane = blockIdx.x * kBlock + threadIdx.x;
   if (lane >= a.total) return;
   const uint32_t cell0 = lane * VEC;
-  uint32_t position_all, col;
-  a.cols_fd.divmod(cell0, position_all, col);
-  uint32_t image, position, oy, ox;
-  a.rows_fd.divmod(position_all, image, position);
-  a.out_w_fd.divmod(position, oy, ox);
-  const T* in = reinterpret_cast<const T*>(a.src) + (int64_t)image * a.channels * a.in_plane;
-  const int32_t rel_x = (int32_t)ox * a.sx - a.px, rel_y = (int32_t)oy * a.sy - a.py;
-  struct alignas(sizeof(T) * VEC) Piece { T v[VEC]; } piece;
-  uint32_t chan, tap, ky, kx;
+  uint32_t row_all, position, image, col, chan, tap, ky, kx, oy, ox;
+  a.rows_fd.divmod(cell0, row_all, position);   // row_all = image * n_cols + col
+  a.cols_fd.divmod(row_all, image, col);
   a.kk_fd.divmod(col, chan, tap);
   a.kw_fd.divmod(tap, ky, kx);
+  a.out_w_fd.divmod(position, oy, ox);
+  const T* in = reinterpret_cast<const T*>(a.src) + ((int64_t)image * a.channels + chan) * a.in_plane;
+  struct alignas(sizeof(T) * VEC) Piece { T v[VEC]; } piece;
+  int32_t iy = (int32_t)oy * a.sy - a.py + (int32_t)ky, ix = (int32_t)ox * a.sx - a.px + (int32_t)kx;
 #pragma unroll
   for (int e = 0; e < VEC; ++e) {
-    const int32_t iy = rel_y + (int32_t)ky, ix = rel_x + (int32_t)kx;
     const bool inside = (uint32_t)iy < (uint32_t)a.in_h && (uint32_t)ix < (uint32_t)a.in_w;
-    piece.v[e] = inside ? in[(int64_t)chan * a.in_plane + iy * a.in_w + ix] : (T)0;
-    if (++kx == (uint32_t)a.kw) {
-      kx = 0;
-      if (++ky == (uint32_t)a.kh) { ky = 0; ++chan; }
+    piece.v[e] = inside ? in[iy * a.in_w + ix] : (T)0;
+    ix += a.sx;
+    if (++ox == (uint32_t)a.out_w) {
+      ox = 0;
+      ix = (int32_t)kx - a.px;
+      iy += a.sy;
     }
   }
   *reinterpret_cast<Piece*>(reinterpret_cast<T*>(a.dest) + (int64_t)cell0) = piece;
@@ -87,7 +94,8 @@ __global__ void __launch_bounds__(kBlock) conv_roll_kernel(const ConvArgs a) {
   a.image_fd.divmod(e, image, rest);
   a.in_plane_fd.divmod(rest, chan, r);
   a.in_w_fd.divmod(r, iy, ix);
-  const T* conv = reinterpret_cast<const T*>(a.src) + (int64_t)image * a.n_rows * a.n_cols + chan * (uint32_t)(a.kw * a.kh);
+  const T* conv = reinterpret_cast<const T*>(a.src) +
+                  ((int64_t)image * a.n_cols + (int64_t)chan * (uint32_t)(a.kw * a.kh)) * a.n_rows;
   // Windows o with o * stride - pad <= i < o * stride - pad + k.
   const int32_t ty = (int32_t)iy + a.py, tx = (int32_t)ix + a.px;
   const int32_t oy_hi = min(a.out_h - 1, (int32_t)a.sy_fd.div((uint32_t)ty));
@@ -100,7 +108,7 @@ __global__ void __launch_bounds__(kBlock) conv_roll_kernel(const ConvArgs a) {
     const int32_t ky = ty - oy * a.sy;
     for (int32_t ox = ox_lo; ox <= ox_hi; ++ox) {
       const int32_t kx = tx - ox * a.sx;
-      acc = acc + conv[(int64_t)(oy * a.out_w + ox) * a.n_cols + ky * a.kw + kx];
+      acc = acc + conv[(int64_t)(ky * a.kw + kx) * a.n_rows + oy * a.out_w + ox];
     }
   }
   reinterpret_cast<T*>(a.dest)[e] = acc;
@@ -177,7 +185,7 @@ void unroll(hipStream_t s, const T* input, T* workspace, const ct_conv_desc& d, 
   if (sh.batch * sh.conv_image == 0) return;
   ConvArgs a = conv_args(d, sh);
   constexpr int VEC = 16 / sizeof(T);
-  const bool pieces = sh.n_cols % VEC == 0 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+  const bool pieces = sh.n_rows % VEC == 0 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
   const int64_t step = images_per_launch(sh.conv_image);
   for (int64_t b0 = 0; b0 < sh.batch; b0 += step) {
     const int64_t nb = std::min(step, sh.batch - b0);
@@ -212,9 +220,9 @@ int forward_t(void* stream, T* output, double output_alpha, const T* input, cons
   hipStream_t s = static_cast<hipStream_t>(stream);
   unroll(s, input, workspace, d, sh);
   if (int rc = after_launch(s)) return rc;
-  // output[b] [out_channels, n_rows] = weights [out_channels, n_cols] x unrolled[b]^T
-  if (int rc = gemm_strided_batched(stream, output, sh.n_rows, sh.out_image, 0, 1, 1.0, weights, d.out_channels,
-                                    sh.n_cols, sh.n_cols, 0, workspace, sh.n_rows, sh.n_cols, sh.conv_image,
+  // output[b] [out_channels, n_rows] = weights [out_channels, n_cols] x unrolled[b] [n_cols, n_rows]
+  if (int rc = gemm_strided_batched(stream, output, sh.n_rows, sh.out_image, 0, 0, 1.0, weights, d.out_channels,
+                                    sh.n_cols, sh.n_cols, 0, workspace, sh.n_rows, sh.n_rows, sh.conv_image,
                                     output_alpha, sh.batch, dtype))
     return rc;
   note_kernel("conv_unroll+gemm");
@@ -245,10 +253,10 @@ int backward_weights_t(void* stream, T* weight_gradient, double alpha, const T* 
   const T al = (T)alpha;
   for (int64_t b0 = 0; b0 < sh.batch; b0 += per_pass) {
     const int64_t nb = std::min(per_pass, sh.batch - b0);
-    // partial[b] [out_channels, n_cols] = output_gradient[b] [out_channels, n_rows] x unrolled[b] [n_rows, n_cols]
-    if (int rc = gemm_strided_batched(stream, scratch, sh.n_cols, n, 0, 0, 1.0, output_gradient + b0 * sh.out_image,
+    // partial[b] [out_channels, n_cols] = output_gradient[b] [out_channels, n_rows] x unrolled[b]^T
+    if (int rc = gemm_strided_batched(stream, scratch, sh.n_cols, n, 0, 1, 1.0, output_gradient + b0 * sh.out_image,
                                       d.out_channels, sh.n_rows, sh.n_rows, sh.out_image,
-                                      workspace + b0 * sh.conv_image, sh.n_cols, sh.n_cols, sh.conv_image, 0.0, nb,
+                                      workspace + b0 * sh.conv_image, sh.n_cols, sh.n_rows, sh.conv_image, 0.0, nb,
                                       dtype))
       return rc;
     hipLaunchKernelGGL((conv_sum_partials_kernel<T>), dim3((uint32_t)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
@@ -263,11 +271,11 @@ template <class T>
 int backward_data_t(void* stream, T* input_gradient, const T* output_gradient, const T* weights, T* workspace,
                     const ct_conv_desc& d, const ConvShape& sh, int dtype) {
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // unrolled[b] [n_rows, n_cols] = output_gradient[b]^T [n_rows, out_channels] x weights [out_channels, n_cols]
+  // unrolled[b] [n_cols, n_rows] = weights^T [n_cols, out_channels] x output_gradient[b] [out_channels, n_rows]
   if (sh.conv_image > 0)
-    if (int rc = gemm_strided_batched(stream, workspace, sh.n_cols, sh.conv_image, 1, 0, 1.0, output_gradient, sh.n_rows,
-                                      d.out_channels, sh.n_rows, sh.out_image, weights, sh.n_cols, sh.n_cols, 0, 0.0,
-                                      sh.batch, dtype))
+    if (int rc = gemm_strided_batched(stream, workspace, sh.n_rows, sh.conv_image, 1, 0, 1.0, weights, sh.n_cols,
+                                      d.out_channels, sh.n_cols, 0, output_gradient, sh.n_rows, sh.n_rows,
+                                      sh.out_image, 0.0, sh.batch, dtype))
       return rc;
   roll_back(s, workspace, input_gradient, d, sh);
   note_kernel("gemm+conv_roll");

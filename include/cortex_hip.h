@@ -381,9 +381,10 @@ typedef struct ct_conv_desc {
 /* convolution-forward! / -backward-weights! / -backward-data!
  * (tensor/math.clj:185-220), decomposed as the CPU backend decomposes them
  * (cpu/tensor_math.clj:1118-1151, 1670-1792): the input is unrolled into the
- * caller's workspace as [batch, out_height * out_width, in_channels *
- * kernel_height * kernel_width] (padding reads 0), and the three methods are
- * one gemm! per image around that matrix:
+ * caller's workspace (padding reads 0; stored here as [batch, in_channels *
+ * kernel_height * kernel_width, out_height * out_width], the transpose of the
+ * CPU backend's per-image matrix: the workspace is opaque to callers), and the
+ * three methods are one gemm! per image around that matrix:
  *   forward           output[b] = weights x unrolled[b]^T + output_alpha * output[b]
  *   backward-weights  weight_gradient = sum over b of output_gradient[b] x unrolled[b],
  *                     on top of weight_gradient_alpha * weight_gradient; it reads the

@@ -837,6 +837,16 @@ CONV_CASES = [
 ]
 
 
+def unrolled_matches(work, batch, n_rows, n_cols, what):
+    """The library keeps an image's unrolled matrix as [cells, positions], the oracle (like the
+    reference's CPU backend) as [positions, cells]; whatever follows the matrices must be untouched."""
+    n = batch * n_rows * n_cols
+    got, want = work.download(), work.host
+    H.assert_bit_exact(np.ascontiguousarray(got[:n].reshape(batch, n_cols, n_rows).transpose(0, 2, 1)),
+                       want[:n].reshape(batch, n_rows, n_cols), what)
+    H.assert_bit_exact(got[n:], want[n:], what + " (slack)")
+
+
 @pytest.mark.parametrize("code", FLOATS)
 @pytest.mark.parametrize("case", CONV_CASES, ids=str)
 def test_convolution(P, code, case):
@@ -862,7 +872,7 @@ def test_convolution(P, code, case):
 
     x64, w64, g64 = (b.init.astype(np.float64) for b in (inp, weights, og))
     P.run(H.convolution, "forward", V(out), 0.0, V(inp), V(weights), V(work), *geom)
-    compare(work, f"unrolled input {case}")                             # a copy: bit-exact, the slack untouched
+    unrolled_matches(work, batch, n_rows, n_cols, f"unrolled input {case}")   # a copy: bit-exact, the slack untouched
     scale = np.abs(w64).max() * np.abs(x64).max() * n_cols
     close(out, scale, "convolution-forward")
     P.run(H.convolution, "forward", V(out), 0.5, V(inp), V(weights), V(work), *geom)
@@ -889,7 +899,7 @@ def test_convolution_roll_back_is_bit_exact(P):
     ig = P.buf(np.ones(batch * cin * h * w, np.float32))
     V = lambda b: View(b, [b.init.size])
     P.run(H.convolution, "backward_data", V(ig), 0.0, V(og), V(weights), V(work), desc, batch, h, w, oh, ow)
-    compare(work, "unrolled gradient")
+    unrolled_matches(work, batch, oh * ow, cin * k * k, "unrolled gradient")
     compare(ig, "input gradient")
 
 
