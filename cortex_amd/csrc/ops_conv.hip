@@ -49,6 +49,7 @@ struct ConvArgs {
   const void* src;
   void* dest;
   uint32_t total;  // lanes' worth of work in this launch
+  uint32_t grouped_blocks;
   int32_t in_h, in_w, out_h, out_w;
   int32_t kw, kh, px, py, sx, sy;
   uint32_t channels, n_cols, n_rows, in_plane;
@@ -59,7 +60,12 @@ struct ConvArgs {
 // workspace[image][channel * kh * kw + k_y * kw + k_x][position] = input tap or 0 in the padding
 template <class T, int VEC>
 __global__ void __launch_bounds__(kBlock) conv_unroll_kernel(const ConvArgs a) {
-  const uint32_t lane = blockIdx.x * kBlock + threadIdx.x;
+  // The kh * kw rows of one channel read the same input plane: in the die-grouped
+  // block order they run on one die and share its L2 (HBM reads of the input for
+  // [64, 64, 56, 56] float, 3 x 3: 3.7 times the input before, 1.2 times after).
+  // A variant that gave every block one row of cells, to decode the row on the
+  // scalar unit, left too many lanes idle at the row ends and was slower.
+  const uint32_t lane = xcd_grouped_unit(blockIdx.x, a.grouped_blocks) * kBlock + threadIdx.x;
   if (lane >= a.total) return;
   const uint32_t cell0 = lane * VEC;
   uint32_t row_all, position, image, col, chan, tap, ky, kx, oy, ox;
@@ -194,6 +200,7 @@ void unroll(hipStream_t s, const T* input, T* workspace, const ct_conv_desc& d, 
     const int64_t cells = nb * sh.conv_image;
     a.total = (uint32_t)(pieces ? cells / VEC : cells);
     const dim3 grid((a.total + kBlock - 1) / kBlock);
+    a.grouped_blocks = xcd_grouped_blocks(grid.x);
     if (pieces) hipLaunchKernelGGL((conv_unroll_kernel<T, VEC>), grid, dim3(kBlock), 0, s, a);
     else hipLaunchKernelGGL((conv_unroll_kernel<T, 1>), grid, dim3(kBlock), 0, s, a);
   }
