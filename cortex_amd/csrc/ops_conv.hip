@@ -253,21 +253,34 @@ int backward_weights_t(void* stream, T* weight_gradient, double alpha, const T* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t n = (int64_t)d.out_channels * sh.n_cols;
   CT_REQUIRE(n <= (int64_t(1) << 31) - 1, "convolution: the weight matrix exceeds the supported range");
+  // A product of few outputs over very many positions (a first layer: 64 x 27 outputs, 50176
+  // positions) would occupy one workgroup per image: the positions are cut into pieces of about
+  // kPositionsPerPiece, every piece a product of its own, and the sum takes the pieces too.
+  constexpr int64_t kPositionsPerPiece = 4096;
+  const int64_t pieces = std::max<int64_t>(1, std::min<int64_t>(64, sh.n_rows / kPositionsPerPiece));
+  const int64_t piece_len = (sh.n_rows + pieces - 1) / pieces;
   // images per pass: partial products of at most 256 MiB
-  const int64_t per_pass = std::max<int64_t>(1, std::min<int64_t>(sh.batch, (int64_t(256) << 20) / (n * (int64_t)sizeof(T))));
+  const int64_t per_pass =
+      std::max<int64_t>(1, std::min<int64_t>(sh.batch, (int64_t(256) << 20) / (pieces * n * (int64_t)sizeof(T))));
   void* scratch = nullptr;
-  if (int rc = stream_scratch(s, (size_t)(per_pass * n) * sizeof(T), &scratch)) return rc;
+  if (int rc = stream_scratch(s, (size_t)(per_pass * pieces * n) * sizeof(T), &scratch)) return rc;
   const T al = (T)alpha;
   for (int64_t b0 = 0; b0 < sh.batch; b0 += per_pass) {
     const int64_t nb = std::min(per_pass, sh.batch - b0);
-    // partial[b] [out_channels, n_cols] = output_gradient[b] [out_channels, n_rows] x unrolled[b]^T
-    if (int rc = gemm_strided_batched(stream, scratch, sh.n_cols, n, 0, 1, 1.0, output_gradient + b0 * sh.out_image,
-                                      d.out_channels, sh.n_rows, sh.n_rows, sh.out_image,
-                                      workspace + b0 * sh.conv_image, sh.n_cols, sh.n_rows, sh.conv_image, 0.0, nb,
-                                      dtype))
-      return rc;
+    int64_t used = 0;
+    for (int64_t p = 0; p < pieces; ++p) {
+      const int64_t r0 = p * piece_len, len = std::min(piece_len, sh.n_rows - r0);
+      if (len <= 0) break;
+      // partial[p][b] [out_channels, n_cols] = output_gradient[b][:, r0 : r0 + len] x unrolled[b][:, r0 : r0 + len]^T
+      if (int rc = gemm_strided_batched(stream, reinterpret_cast<T*>(scratch) + used * nb * n, sh.n_cols, n, 0, 1, 1.0,
+                                        output_gradient + b0 * sh.out_image + r0, d.out_channels, len, sh.n_rows,
+                                        sh.out_image, workspace + b0 * sh.conv_image + r0, sh.n_cols, sh.n_rows,
+                                        sh.conv_image, 0.0, nb, dtype))
+        return rc;
+      ++used;
+    }
     hipLaunchKernelGGL((conv_sum_partials_kernel<T>), dim3((uint32_t)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
-                       weight_gradient, reinterpret_cast<const T*>(scratch), (uint32_t)n, (uint32_t)nb,
+                       weight_gradient, reinterpret_cast<const T*>(scratch), (uint32_t)n, (uint32_t)(nb * used),
                        b0 == 0 ? (double)al : 1.0);
   }
   note_kernel("gemm+conv_sum_partials");
