@@ -54,3 +54,38 @@ def test_mask(driver, datatype):
 
 def test_rand_operator(driver):
     rs.rand_operator(driver, "float")
+
+
+def test_convolution_and_pooling_front_end_checks(driver):
+    """The argument checks of tensor.clj:1320-1551 that run before a backend is reached."""
+    import numpy as np
+    from cortex_amd import tensor as ct
+    with rs.context(driver, "float"):
+        desc = ct.convolution_descriptor("float", 3, 4, 3, 3, 0, 0, 1, 1)
+        assert ct.get_convolution_output_dimensions(desc, 4, 4) == {"output-width": 2, "output-height": 2}
+        algorithms = ct.choose_convolution_algorithms(desc, 4, 4, 2, 1000)
+        assert algorithms == {"workspace-size": 2 * 2 * 2 * 36}
+        inp, out = ct.new_tensor([2, 4, 4, 4]), ct.new_tensor([2, 3, 2, 2])
+        weights, work = ct.new_tensor([3, 36]), ct.new_tensor([algorithms["workspace-size"]])
+        ct.convolution_forward(out, 0.0, inp, weights, work, desc, algorithms)
+        with pytest.raises(ct.TensorError, match="Output dimensions"):
+            ct.convolution_forward(ct.new_tensor([2, 3, 3, 3]), 0.0, inp, weights, work, desc, algorithms)
+        with pytest.raises(ct.TensorError, match="Input dimensions"):
+            ct.convolution_forward(out, 0.0, ct.new_tensor([2, 5, 4, 4]), weights, work, desc, algorithms)
+        with pytest.raises(ct.TensorError, match="nil"):
+            ct.convolution_descriptor("float", 3, None, 3, 3, 0, 0, 1, 1)
+        with pytest.raises(Exception, match="workspace"):
+            ct.convolution_forward(out, 0.0, inp, weights, ct.new_tensor([10]), desc, algorithms)
+        # the two rounding rules of the output size (tensor.clj:1351-1365)
+        pool = ct.pooling_descriptor("float", 4, 2, 2, 0, 0, 2, 2)
+        assert pool["dimension-op"] == "ceil" and pool["pool-op"] == "max"
+        assert ct.get_convolution_output_dimensions(pool, 5, 5) == {"output-width": 3, "output-height": 3}
+        floor = ct.pooling_descriptor("float", 4, 2, 2, 0, 0, 2, 2, dimension_op="floor")
+        assert ct.get_convolution_output_dimensions(floor, 5, 5) == {"output-width": 2, "output-height": 2}
+        with pytest.raises(ct.TensorError, match="three possible pool operations"):
+            ct.pooling_descriptor("float", 4, 2, 2, 0, 0, 2, 2, pool_op="median")
+        with pytest.raises(ct.TensorError, match="Output dimensions"):
+            ct.pooling_forward(ct.new_tensor([2, 4, 2, 2]), 0.0, ct.new_tensor([2, 4, 5, 5]), pool)
+        ints = ct.new_tensor([2, 4, 5, 5], "int")
+        with pytest.raises(ct.TensorError):
+            ct.pooling_forward(ct.new_tensor([2, 4, 3, 3], "int"), 0.0, ints, pool)
