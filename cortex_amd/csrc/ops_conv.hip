@@ -120,6 +120,36 @@ __global__ void __launch_bounds__(kBlock) conv_roll_kernel(const ConvArgs a) {
   reinterpret_cast<T*>(a.dest)[e] = acc;
 }
 
+// The same for stride 1 and a fixed window: window (y, x) holds input (i_y, i_x) at tap
+// (i_y + pad - y, i_x + pad - x), so the taps taken in DEcreasing order are the windows in
+// increasing order, and the cell of tap (k_y, k_x) lies a constant distance from the cell
+// of tap (0, 0).  No loops, no divisions beyond the element's own decomposition.
+template <class T, int KW, int KH>
+__global__ void __launch_bounds__(kBlock) conv_roll_unit_stride_kernel(const ConvArgs a) {
+  const uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+  if (e >= a.total) return;
+  uint32_t image, rest, chan, r, iy, ix;
+  a.image_fd.divmod(e, image, rest);
+  a.in_plane_fd.divmod(rest, chan, r);
+  a.in_w_fd.divmod(r, iy, ix);
+  const int32_t ty = (int32_t)iy + a.py, tx = (int32_t)ix + a.px;
+  const T* conv = reinterpret_cast<const T*>(a.src) +
+                  ((int64_t)image * a.n_cols + (int64_t)chan * (KW * KH)) * a.n_rows + (ty * a.out_w + tx);
+  T acc = (T)0;
+#pragma unroll
+  for (int32_t ky = KH - 1; ky >= 0; --ky) {
+    const bool row_ok = (uint32_t)(ty - ky) < (uint32_t)a.out_h;
+#pragma unroll
+    for (int32_t kx = KW - 1; kx >= 0; --kx) {
+      const bool ok = row_ok && (uint32_t)(tx - kx) < (uint32_t)a.out_w;
+      const int64_t at = (int64_t)(ky * KW + kx) * a.n_rows - ky * a.out_w - kx;
+      const T cell = ok ? conv[at] : (T)0;
+      acc = ok ? acc + cell : acc;
+    }
+  }
+  reinterpret_cast<T*>(a.dest)[e] = acc;
+}
+
 struct ConvShape {
   int64_t batch, in_h, in_w, out_h, out_w, n_rows, n_cols, in_image, out_image, conv_image;
 };
@@ -217,7 +247,15 @@ void roll_back(hipStream_t s, const T* workspace, T* input_gradient, const ct_co
     a.dest = input_gradient + b0 * sh.in_image;
     a.total = (uint32_t)(nb * sh.in_image);
     const dim3 grid((a.total + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL((conv_roll_kernel<T>), grid, dim3(kBlock), 0, s, a);
+    const bool unit_stride = d.stride_x == 1 && d.stride_y == 1;
+    if (unit_stride && d.kernel_width == 3 && d.kernel_height == 3)
+      hipLaunchKernelGGL((conv_roll_unit_stride_kernel<T, 3, 3>), grid, dim3(kBlock), 0, s, a);
+    else if (unit_stride && d.kernel_width == 5 && d.kernel_height == 5)
+      hipLaunchKernelGGL((conv_roll_unit_stride_kernel<T, 5, 5>), grid, dim3(kBlock), 0, s, a);
+    else if (unit_stride && d.kernel_width == 1 && d.kernel_height == 1)
+      hipLaunchKernelGGL((conv_roll_unit_stride_kernel<T, 1, 1>), grid, dim3(kBlock), 0, s, a);
+    else
+      hipLaunchKernelGGL((conv_roll_kernel<T>), grid, dim3(kBlock), 0, s, a);
   }
 }
 

@@ -835,6 +835,7 @@ CONV_CASES = [
     (1, 8, 16, 14, 14, 1, 1, 0, 0, 1, 1),    # 1 x 1: the unrolled matrix is the transposed input
     (4, 16, 32, 28, 28, 3, 3, 1, 1, 1, 1),
     (2, 2, 3, 100, 130, 3, 3, 1, 1, 1, 1),   # 13000 positions: the weight gradient in three pieces
+    (1, 2, 2, 9, 11, 5, 5, 2, 2, 1, 1),
 ]
 
 
