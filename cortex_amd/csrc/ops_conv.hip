@@ -91,6 +91,42 @@ __global__ void __launch_bounds__(kBlock) conv_unroll_kernel(const ConvArgs a) {
   *reinterpret_cast<Piece*>(reinterpret_cast<T*>(a.dest) + (int64_t)cell0) = piece;
 }
 
+// The same for stride_x 1 and an output width that is a whole number of 16-byte pieces: the
+// cells of a piece are consecutive input elements of one input row, fetched with ONE
+// (unaligned) 16-byte load and then masked where they fall into the padding.  Only a run that
+// would leave the channel's plane (first and last row) is read element by element.
+template <class T>
+__global__ void __launch_bounds__(kBlock) conv_unroll_unit_stride_kernel(const ConvArgs a) {
+  constexpr int VEC = 16 / sizeof(T);
+  const uint32_t lane = xcd_grouped_unit(blockIdx.x, a.grouped_blocks) * kBlock + threadIdx.x;
+  if (lane >= a.total) return;
+  const uint32_t cell0 = lane * VEC;
+  uint32_t row_all, position, plane, tap, ky, kx, oy, ox;
+  a.rows_fd.divmod(cell0, row_all, position);   // row_all = (image * channels + channel) * kh * kw + tap
+  a.kk_fd.divmod(row_all, plane, tap);
+  a.kw_fd.divmod(tap, ky, kx);
+  a.out_w_fd.divmod(position, oy, ox);
+  const T* in = reinterpret_cast<const T*>(a.src) + (int64_t)plane * a.in_plane;
+  const int32_t iy = (int32_t)oy * a.sy - a.py + (int32_t)ky, ix = (int32_t)ox - a.px + (int32_t)kx;
+  struct alignas(16) Piece { T v[VEC]; } piece;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) piece.v[e] = (T)0;
+  if ((uint32_t)iy < (uint32_t)a.in_h) {
+    const int32_t at = iy * a.in_w + ix;
+    if (at >= 0 && at + VEC <= (int32_t)a.in_plane) {
+      __builtin_memcpy(&piece, in + at, 16);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        if ((uint32_t)(ix + e) >= (uint32_t)a.in_w) piece.v[e] = (T)0;
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        if ((uint32_t)(ix + e) < (uint32_t)a.in_w) piece.v[e] = in[at + e];
+    }
+  }
+  *reinterpret_cast<Piece*>(reinterpret_cast<T*>(a.dest) + (int64_t)cell0) = piece;
+}
+
 // input_gradient[image][channel][y][x] = sum of the workspace cells unrolled from it
 template <class T>
 __global__ void __launch_bounds__(kBlock) conv_roll_kernel(const ConvArgs a) {
@@ -231,7 +267,9 @@ void unroll(hipStream_t s, const T* input, T* workspace, const ct_conv_desc& d, 
     a.total = (uint32_t)(pieces ? cells / VEC : cells);
     const dim3 grid((a.total + kBlock - 1) / kBlock);
     a.grouped_blocks = xcd_grouped_blocks(grid.x);
-    if (pieces) hipLaunchKernelGGL((conv_unroll_kernel<T, VEC>), grid, dim3(kBlock), 0, s, a);
+    if (pieces && d.stride_x == 1 && sh.out_w % VEC == 0)
+      hipLaunchKernelGGL((conv_unroll_unit_stride_kernel<T>), grid, dim3(kBlock), 0, s, a);
+    else if (pieces) hipLaunchKernelGGL((conv_unroll_kernel<T, VEC>), grid, dim3(kBlock), 0, s, a);
     else hipLaunchKernelGGL((conv_unroll_kernel<T, 1>), grid, dim3(kBlock), 0, s, a);
   }
 }

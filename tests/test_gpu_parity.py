@@ -836,6 +836,8 @@ CONV_CASES = [
     (4, 16, 32, 28, 28, 3, 3, 1, 1, 1, 1),
     (2, 2, 3, 100, 130, 3, 3, 1, 1, 1, 1),   # 13000 positions: the weight gradient in three pieces
     (1, 2, 2, 9, 11, 5, 5, 2, 2, 1, 1),
+    (2, 3, 4, 10, 14, 3, 3, 0, 0, 1, 1),     # unit stride, rows of whole 16-byte pieces: one load per piece
+    (1, 2, 2, 12, 12, 3, 3, 1, 1, 1, 2),
 ]
 
 
