@@ -186,6 +186,48 @@ __global__ void __launch_bounds__(kBlock) conv_roll_unit_stride_kernel(const Con
   reinterpret_cast<T*>(a.dest)[e] = acc;
 }
 
+// The same, four (two for double) consecutive input elements of one row per lane: for a tap
+// their cells are consecutive, one (unaligned) 16-byte load, masked where a window does not
+// exist.  A run of cells that would leave the tap's row of the matrix is read cell by cell.
+template <class T, int KW, int KH>
+__global__ void __launch_bounds__(kBlock) conv_roll_unit_stride_pieces_kernel(const ConvArgs a) {
+  constexpr int VEC = 16 / sizeof(T);
+  const uint32_t lane = blockIdx.x * kBlock + threadIdx.x;
+  if (lane >= a.total) return;
+  const uint32_t e0 = lane * VEC;
+  uint32_t image, rest, chan, r, iy, ix;
+  a.image_fd.divmod(e0, image, rest);
+  a.in_plane_fd.divmod(rest, chan, r);
+  a.in_w_fd.divmod(r, iy, ix);
+  const int32_t ty = (int32_t)iy + a.py, tx = (int32_t)ix + a.px;
+  const T* conv = reinterpret_cast<const T*>(a.src) + ((int64_t)image * a.n_cols + (int64_t)chan * (KW * KH)) * a.n_rows;
+  struct alignas(16) Piece { T v[VEC]; } acc;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc.v[e] = (T)0;
+#pragma unroll
+  for (int32_t ky = KH - 1; ky >= 0; --ky) {
+    const int32_t oy = ty - ky;
+    if ((uint32_t)oy >= (uint32_t)a.out_h) continue;
+#pragma unroll
+    for (int32_t kx = KW - 1; kx >= 0; --kx) {
+      const int32_t ox = tx - kx;                       // of the first element; element e: ox + e
+      const int32_t at = oy * a.out_w + ox;             // inside the tap's row of cells
+      const T* cells = conv + (int64_t)(ky * KW + kx) * a.n_rows;
+      Piece got;
+      if (at >= 0 && at + VEC <= (int32_t)a.n_rows) {
+        __builtin_memcpy(&got, cells + at, 16);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) got.v[e] = (uint32_t)(ox + e) < (uint32_t)a.out_w ? cells[at + e] : (T)0;
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        if ((uint32_t)(ox + e) < (uint32_t)a.out_w) acc.v[e] = acc.v[e] + got.v[e];
+    }
+  }
+  *reinterpret_cast<Piece*>(reinterpret_cast<T*>(a.dest) + e0) = acc;
+}
+
 struct ConvShape {
   int64_t batch, in_h, in_w, out_h, out_w, n_rows, n_cols, in_image, out_image, conv_image;
 };
@@ -286,7 +328,21 @@ void roll_back(hipStream_t s, const T* workspace, T* input_gradient, const ct_co
     a.total = (uint32_t)(nb * sh.in_image);
     const dim3 grid((a.total + kBlock - 1) / kBlock);
     const bool unit_stride = d.stride_x == 1 && d.stride_y == 1;
-    if (unit_stride && d.kernel_width == 3 && d.kernel_height == 3)
+    constexpr int VEC = 16 / sizeof(T);
+    const bool pieces = unit_stride && sh.in_w % VEC == 0 && reinterpret_cast<uintptr_t>(input_gradient) % 16 == 0 &&
+                        d.kernel_width == d.kernel_height &&
+                        (d.kernel_width == 1 || d.kernel_width == 3 || d.kernel_width == 5);
+    if (pieces) {
+      ConvArgs p = a;
+      p.total = a.total / VEC;   // whole images: in_w, hence in_image, is a multiple of VEC
+      const dim3 pgrid((p.total + kBlock - 1) / kBlock);
+      if (d.kernel_width == 3)
+        hipLaunchKernelGGL((conv_roll_unit_stride_pieces_kernel<T, 3, 3>), pgrid, dim3(kBlock), 0, s, p);
+      else if (d.kernel_width == 5)
+        hipLaunchKernelGGL((conv_roll_unit_stride_pieces_kernel<T, 5, 5>), pgrid, dim3(kBlock), 0, s, p);
+      else
+        hipLaunchKernelGGL((conv_roll_unit_stride_pieces_kernel<T, 1, 1>), pgrid, dim3(kBlock), 0, s, p);
+    } else if (unit_stride && d.kernel_width == 3 && d.kernel_height == 3)
       hipLaunchKernelGGL((conv_roll_unit_stride_kernel<T, 3, 3>), grid, dim3(kBlock), 0, s, a);
     else if (unit_stride && d.kernel_width == 5 && d.kernel_height == 5)
       hipLaunchKernelGGL((conv_roll_unit_stride_kernel<T, 5, 5>), grid, dim3(kBlock), 0, s, a);

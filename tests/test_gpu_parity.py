@@ -894,17 +894,18 @@ def test_convolution_roll_back_is_bit_exact(P):
     agree to the bit whatever order the gemm sums in; the gather then adds windows in the
     reference's order."""
     rng = np.random.default_rng(56)
-    batch, cin, cout, h, w, k = 2, 3, 4, 10, 9, 3
-    oh, ow = h - k + 1 + 2, w - k + 1 + 2      # pad 1, stride 1
-    desc = H.conv_desc(cin, cout, k, k, 1, 1, 1, 1)
-    og = P.buf(rng.integers(-3, 4, batch * cout * oh * ow).astype(np.float32))
-    weights = P.buf(rng.integers(-3, 4, cout * cin * k * k).astype(np.float32))
-    work = P.buf(np.zeros(batch * oh * ow * cin * k * k, np.float32))
-    ig = P.buf(np.ones(batch * cin * h * w, np.float32))
     V = lambda b: View(b, [b.init.size])
-    P.run(H.convolution, "backward_data", V(ig), 0.0, V(og), V(weights), V(work), desc, batch, h, w, oh, ow)
-    unrolled_matches(work, batch, oh * ow, cin * k * k, "unrolled gradient")
-    compare(ig, "input gradient")
+    for h, w, k in ((10, 9, 3), (10, 12, 3), (8, 16, 5), (6, 8, 1)):      # rows of whole 16-byte pieces or not
+        batch, cin, cout, pad = 2, 3, 4, k // 2
+        oh, ow = h, w                                                   # "same" padding, stride 1
+        desc = H.conv_desc(cin, cout, k, k, pad, pad, 1, 1)
+        og = P.buf(rng.integers(-3, 4, batch * cout * oh * ow).astype(np.float32))
+        weights = P.buf(rng.integers(-3, 4, cout * cin * k * k).astype(np.float32))
+        work = P.buf(np.zeros(batch * oh * ow * cin * k * k, np.float32))
+        ig = P.buf(np.ones(batch * cin * h * w, np.float32))
+        P.run(H.convolution, "backward_data", V(ig), 0.0, V(og), V(weights), V(work), desc, batch, h, w, oh, ow)
+        unrolled_matches(work, batch, oh * ow, cin * k * k, f"unrolled gradient {h}x{w} k{k}")
+        compare(ig, f"input gradient {h}x{w} k{k}")
 
 
 def test_convolution_errors(P):
