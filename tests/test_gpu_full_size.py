@@ -278,7 +278,7 @@ def test_pooling_at_image_batch_size():
     for op, expect in (("max", np.full((oh, ow), 3.0)), ("avg", None), ("avg-exc-pad", np.full((oh, ow), 3.0))):
         desc3 = {"kernel-width": 3, "kernel-height": 3, "pad-x": 1, "pad-y": 1, "stride-x": 2, "stride-y": 2, "pool-op": op}
         out = Dev(np.zeros(planes * oh * ow, np.float32))
-        assert _pool(True, desc3, geom3, out.ptr, ones.ptr) == "pool_forward_padded"
+        assert _pool(True, desc3, geom3, out.ptr, ones.ptr).startswith("pool_forward")
         got = out.download().reshape(planes, oh, ow)
         assert np.all(got == got[0]), op               # every plane alike
         if expect is None:
