@@ -421,11 +421,15 @@ int softmax_run(hipStream_t s, void* out, const RowLayout& ol, const void* in, c
   const bool row_major = il.s_k == 1 || il.k == 1;
   if (il.k < 8 || (!row_major && il.s_row == 1)) {
     constexpr int VL = 16 / (int)sizeof(T);
+    // More than 16 float channels held four positions wide cost waves per compute unit: two
+    // positions per lane measured 2.5 points of the HBM peak better at 21 and 32 channels, two
+    // points worse at 4, the same at 10.
+    const bool half_vec = sizeof(T) == 4 && il.k > 16;
     auto lanes_ok = [](const void* p, const RowLayout& l) {
       return l.s_row == 1 && l.rows % VL == 0 && l.s_k % VL == 0 && l.s_outer % VL == 0 && (uintptr_t)p % 16 == 0;
     };
     const bool vec_rows = lanes_ok(in, il) && lanes_ok(out, ol);
-    const int64_t lanes = vec_rows ? a.n_rows / VL : a.n_rows;
+    const int64_t lanes = vec_rows ? a.n_rows / (half_vec ? 2 : VL) : a.n_rows;
     // Rows too long for registers are parked in LDS while at least five waves still fit a
     // compute unit.  One row per lane: four neighbouring rows per lane need four times the LDS
     // per wave and measured 32 % of peak against 56 % at 64 channels (24 % for the loop form).
@@ -444,7 +448,7 @@ int softmax_run(hipStream_t s, void* out, const RowLayout& ol, const void* in, c
   else if (il.k <= 24) hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 24>), grid, dim3(kBlock), 0, s, a); \
   else if (il.k <= 32) hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 32>), grid, dim3(kBlock), 0, s, a); \
   else hipLaunchKernelGGL((softmax_lane_kernel<T, VEC_, 0>), grid, dim3(kBlock), 0, s, a)
-    if (vec_rows) { CT_SM_LANE(VL); } else { CT_SM_LANE(1); }
+    if (vec_rows && half_vec) { CT_SM_LANE(2); } else if (vec_rows) { CT_SM_LANE(VL); } else { CT_SM_LANE(1); }
 #undef CT_SM_LANE
     return after_launch(s);
   }
