@@ -25,13 +25,20 @@
 // 2^31 - 1 elements of either tensor so that all index arithmetic is 32-bit with
 // multiply-high divisions; the host walks larger batches in several launches.
 //
-// Two kernel families.  The band kernels give a block a band of destination
-// rows of one plane (or several whole planes when they are small): the rows of
-// the other tensor that the band touches are one contiguous piece of memory,
-// which the block copies into LDS with aligned 16-byte loads, and the windows
-// are then read out of LDS, so that global memory sees only linear streams.  The
-// direct kernels read the windows from global memory, one lane per destination
-// element, and serve rows too long for the LDS budget.
+// Kernel families, most specific first:
+//   tile2    2 x 2 windows that tile the input exactly: no LDS, a lane takes two
+//            neighbouring windows as 16-byte pieces of two input rows.
+//   padded   forward, 2 x 2 and 3 x 3 windows that stay inside the padded input:
+//            a block's rows are staged in an LDS tile that holds the zero padding
+//            itself, so that the taps need no tests.
+//   band     everything else that fits the LDS budget: a block takes a band of
+//            destination rows of one plane (or several whole small planes); the
+//            rows of the other tensor that the band touches are one contiguous
+//            piece of memory, copied into LDS with aligned 16-byte loads, and the
+//            windows are read from there, so that global memory sees only linear
+//            streams.  The backward pass streams the gradient in 16-byte pieces.
+//   direct   rows too long for the LDS budget: one lane per destination element
+//            reads its windows from global memory.
 //
 // Division.  The averages divide every tap by an integer count d and round the
 // quotient to double before the addition.  For float tensors and d <= 255 the
