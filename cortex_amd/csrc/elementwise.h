@@ -566,7 +566,10 @@ __device__ __forceinline__ int64_t gen_address(const GenArgs& a, int k, I e, con
   int64_t off = 0;
   for (int d = 0; d < a.nd; ++d) {
     const int64_t s = o.shape[d];
-    if (s == 1) continue;
+    if (s == 1) {  // coordinate 0; an index tensor of one element still names the row
+      if (o.index[d]) off += (int64_t)o.index[d][0] * o.stride[d];
+      continue;
+    }
     I c;
     if (s == a.rmax[d]) c = arg[d] - arg[d + 1] * (I)a.rmax[d];
     else c = arg[d] % (I)s;

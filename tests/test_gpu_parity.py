@@ -388,6 +388,28 @@ def test_scatter_add_through_duplicate_indexes(P, code):
     assert mat.host[:9].tolist() == [0, 3, 6, 9, 12, 15, 12, 14, 16]
 
 
+@pytest.mark.parametrize("code", [capi.F32, capi.I32])
+def test_indirect_dimension_of_one_element(P, code):
+    """An index tensor of a single element still selects its row (a dimension of extent 1 is
+    otherwise skipped by the address functions)."""
+    table = P.buf(np.arange(12).astype(NP[code]))
+    idx = P.buf(np.array([2], np.int32))
+    row = View(table, [1, 4], [4, 1], index=[idx, None])
+    got = P.buf(np.zeros(4, NP[code]))
+    P.run(H.assign, View(got, [1, 4]), row)
+    compare(got, "gather of one row")
+    assert got.host.tolist() == [8, 9, 10, 11]
+    P.run(H.binary_op, row, View(got, [1, 4]), 1.0, View(got, [1, 4]), 1.0, "+")      # scatter back twice the row
+    compare(table, "scatter into one row")
+    assert table.host.tolist() == [0, 1, 2, 3, 4, 5, 6, 7, 16, 18, 20, 22]
+    P.run(H.binary_accum, row, 1.0, View(got, [1, 4]), 1.0, "+", reverse=True, requires_cas=True)
+    compare(table, "scatter-add into one row")
+    # broadcast over a batch: the one selected row against three rows
+    out = P.buf(np.zeros(12, NP[code]))
+    P.run(H.binary_op, View(out, [3, 4]), View(table, [3, 4]), 1.0, row, 1.0, "+")
+    compare(out, "one indexed row broadcast over three")
+
+
 # ------------------------------------------------------------------ reductions
 
 def reduce_scale(x64, axis, op, alpha):
