@@ -146,6 +146,7 @@ PROTOTYPES = {
     "ct_ternary_op_constant": [_P, _P, _DP, _P, _DP, _D, _P, _DP, _D, _D, _L, _I, C.POINTER(C.c_int8), _I],
     "ct_ternary_op_constant_constant": [_P, _P, _DP, _P, _DP, _D, _D, _D, _L, _I, C.POINTER(C.c_int8), _I],
     "ct_unary_reduce": [_P, _P, _DP, _D, _P, _DP, _I, _I],
+    "ct_unary_reduce_noalloc": [_P, _P, _DP, _D, _P, _DP, _I, _I],
     "ct_activation_gradient": [_P, _P, _DP, _P, _DP, _P, _DP, _I, _L, _I],
     "ct_softmax_eltwise": [_P, _P, _DP, _P, _DP, _I],
     "ct_softmax_spatial": [_P, _P, _DP, _P, _DP, _I],

@@ -33,6 +33,7 @@
 // rounding to float (the tree order differs from the reference's sequential
 // order by about k * 2^-53 relative to the sum of magnitudes).
 #include <algorithm>
+#include <mutex>
 
 #include "elementwise.h"
 
@@ -499,11 +500,30 @@ RedShape analyse(const ct_dims& in, int64_t k) {
   return r;
 }
 
+// Where a split reduction keeps its partial accumulators: the stream's growing
+// scratch block (allocated on demand), or a fixed block that is never grown.
+struct PartialStore {
+  void* fixed;         // nullptr: use the stream's scratch
+  size_t fixed_bytes;
+  const char* who;
+};
+
+int partial_store(hipStream_t st, const PartialStore& ps, size_t bytes, void** out) {
+  if (!ps.fixed) return stream_scratch(st, bytes, out);
+  if (bytes > ps.fixed_bytes)
+    return set_error(CT_ERR_INVALID,
+                     "%s: this reduction needs %zu bytes of partial accumulators; the fixed scratch holds %zu "
+                     "(use ct_unary_reduce, which allocates)",
+                     ps.who, bytes, ps.fixed_bytes);
+  *out = ps.fixed;
+  return CT_OK;
+}
+
 template <class T> bool aligned_for(const void* p, int vec) { return ((uintptr_t)p % (uintptr_t)(vec * sizeof(T))) == 0; }
 
 template <class P>
-int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, const void* in, const ct_dims* id,
-               int op) {
+int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims* od, double alpha_d, const void* in,
+               const ct_dims* id, int op) {
   using T = typename P::Elem;
   using A = typename P::Acc;
   const typename P::Alpha alpha = (typename P::Alpha)jvm_cast<T>(alpha_d);
@@ -549,7 +569,7 @@ int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, con
     a.n_split = (uint32_t)split;
     a.split_fd = FastDiv((uint32_t)split);
     if (split > 1) {
-      if (int rc = stream_scratch(st, (size_t)(split * n_out) * sizeof(A), &a.partials)) return rc;
+      if (int rc = partial_store(st, ps, (size_t)(split * n_out) * sizeof(A), &a.partials)) return rc;
     }
     const int64_t n_groups = n_out * split;
     const int64_t row_bytes = chunk * (int64_t)sizeof(T);
@@ -635,7 +655,7 @@ int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, con
     const int64_t grid = base_blocks * seg;
     if (grid < (int64_t(1) << 31)) {
       if (seg > 1) {
-        if (int rc = stream_scratch(st, (size_t)(seg * n_out) * sizeof(A), &a.partials)) return rc;
+        if (int rc = partial_store(st, ps, (size_t)(seg * n_out) * sizeof(A), &a.partials)) return rc;
       }
       note_kernel(vec_ok ? "reduce_col_vec" : "reduce_col");
       if (vec_ok) hipLaunchKernelGGL((reduce_col_kernel<P, VMAX>), dim3((uint32_t)grid), dim3(kColBlock), 0, st, a, alpha);
@@ -662,23 +682,24 @@ int reduce_run(hipStream_t st, void* out, const ct_dims* od, double alpha_d, con
 }
 
 template <class T, int RK>
-int reduce_typed(hipStream_t st, void* out, const ct_dims* od, double alpha, const void* in, const ct_dims* id, int op) {
+int reduce_typed(hipStream_t st, const PartialStore& ps, void* out, const ct_dims* od, double alpha, const void* in,
+                 const ct_dims* id, int op) {
   if constexpr (std::is_floating_point<T>::value && (RK == RK_MAX || RK == RK_MIN)) {
-    if (jvm_cast<T>(alpha) == (T)1) return reduce_run<RedKeyed<T, RK>>(st, out, od, alpha, in, id, op);
+    if (jvm_cast<T>(alpha) == (T)1) return reduce_run<RedKeyed<T, RK>>(st, ps, out, od, alpha, in, id, op);
   }
-  return reduce_run<RedWide<T, RK>>(st, out, od, alpha, in, id, op);
+  return reduce_run<RedWide<T, RK>>(st, ps, out, od, alpha, in, id, op);
 }
 
 template <class T>
-int reduce_dispatch(hipStream_t st, void* out, const ct_dims* od, double alpha, const void* in, const ct_dims* id,
-                    int op) {
+int reduce_dispatch(hipStream_t st, const PartialStore& ps, void* out, const ct_dims* od, double alpha, const void* in,
+                    const ct_dims* id, int op) {
   switch (op) {
-    case CT_ROP_MAX: return reduce_typed<T, RK_MAX>(st, out, od, alpha, in, id, op);
-    case CT_ROP_MIN: return reduce_typed<T, RK_MIN>(st, out, od, alpha, in, id, op);
-    case CT_ROP_SUM: return reduce_typed<T, RK_SUM>(st, out, od, alpha, in, id, op);
-    case CT_ROP_MEAN: return reduce_typed<T, RK_MEAN>(st, out, od, alpha, in, id, op);
-    case CT_ROP_MAGNITUDE: return reduce_typed<T, RK_MAG>(st, out, od, alpha, in, id, op);
-    case CT_ROP_MAGNITUDE_SQUARED: return reduce_typed<T, RK_SUMSQ>(st, out, od, alpha, in, id, op);
+    case CT_ROP_MAX: return reduce_typed<T, RK_MAX>(st, ps, out, od, alpha, in, id, op);
+    case CT_ROP_MIN: return reduce_typed<T, RK_MIN>(st, ps, out, od, alpha, in, id, op);
+    case CT_ROP_SUM: return reduce_typed<T, RK_SUM>(st, ps, out, od, alpha, in, id, op);
+    case CT_ROP_MEAN: return reduce_typed<T, RK_MEAN>(st, ps, out, od, alpha, in, id, op);
+    case CT_ROP_MAGNITUDE: return reduce_typed<T, RK_MAG>(st, ps, out, od, alpha, in, id, op);
+    case CT_ROP_MAGNITUDE_SQUARED: return reduce_typed<T, RK_SUMSQ>(st, ps, out, od, alpha, in, id, op);
     default: return set_error(CT_ERR_INVALID, "unknown reduction operation %d", op);
   }
 }
@@ -690,6 +711,63 @@ extern "C" int ct_unary_reduce(void* stream, void* output, const ct_dims* output
   CT_REQUIRE(output && input, "ct_unary_reduce: null buffer");
   if (int rc = check_dims(output_dims, "output")) return rc;
   if (int rc = check_dims(input_dims, "input")) return rc;
-  CT_DISPATCH_DTYPE(dtype, return reduce_dispatch<T>(static_cast<hipStream_t>(stream), output, output_dims, input_alpha, input, input_dims, op));
+  const PartialStore ps{nullptr, 0, "ct_unary_reduce"};
+  CT_DISPATCH_DTYPE(dtype, return reduce_dispatch<T>(static_cast<hipStream_t>(stream), ps, output, output_dims, input_alpha, input, input_dims, op));
+  return CT_OK;
+}
+
+// ------------------------------------------------------------------ the entry point that allocates nothing
+//
+// Same kernels and the same plan as ct_unary_reduce, so the results are the
+// same bits; the partial accumulators of a split reduction live in a fixed
+// array in device memory instead of the stream's growing scratch block.  Every
+// device the library runs on holds its own copy of the array, at its own
+// address, until the process ends.  The array's name below is a host-side
+// stand-in, not a device address: host code only ever uses the address that
+// hipGetSymbolAddress returned for the current device.
+//
+// The partials are written in full by the first kernel of a call before the
+// finishing kernel reads them, so nothing in the array has to start at zero.
+// Calls on one device share the array: two calls that overlap in time on one
+// device (different streams, or different host threads) race.
+
+namespace {
+
+constexpr size_t kFixedScratchBytes = size_t(2) << 20;
+constexpr int kFixedScratchDevices = 64;
+
+static __device__ __align__(256) unsigned char scratch[kFixedScratchBytes];
+
+std::mutex g_fixed_mutex;
+void* g_fixed_ptr[kFixedScratchDevices] = {};
+
+// Device address of `scratch` on the current device, resolved once per device.
+int fixed_scratch(void** out) {
+  int dev = 0;
+  CT_HIP(hipGetDevice(&dev));
+  CT_REQUIRE(dev >= 0 && dev < kFixedScratchDevices, "ct_unary_reduce_noalloc: device %d outside 0..%d", dev,
+             kFixedScratchDevices - 1);
+  std::lock_guard<std::mutex> lock(g_fixed_mutex);
+  if (!g_fixed_ptr[dev]) {
+    void* ptr = nullptr;
+    CT_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    CT_REQUIRE(ptr != nullptr, "ct_unary_reduce_noalloc: the scratch array has no address on device %d", dev);
+    g_fixed_ptr[dev] = ptr;
+  }
+  *out = g_fixed_ptr[dev];
+  return CT_OK;
+}
+
+}  // namespace
+
+extern "C" int ct_unary_reduce_noalloc(void* stream, void* output, const ct_dims* output_dims, double input_alpha,
+                                       const void* input, const ct_dims* input_dims, int op, int dtype) {
+  CT_REQUIRE(output && input, "ct_unary_reduce_noalloc: null buffer");
+  if (int rc = check_dims(output_dims, "output")) return rc;
+  if (int rc = check_dims(input_dims, "input")) return rc;
+  void* ptr = nullptr;
+  if (int rc = fixed_scratch(&ptr)) return rc;
+  const PartialStore ps{ptr, kFixedScratchBytes, "ct_unary_reduce_noalloc"};
+  CT_DISPATCH_DTYPE(dtype, return reduce_dispatch<T>(static_cast<hipStream_t>(stream), ps, output, output_dims, input_alpha, input, input_dims, op));
   return CT_OK;
 }

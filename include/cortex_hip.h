@@ -254,6 +254,23 @@ int ct_ternary_op_constant_constant(void* stream, void* dest, const ct_dims* des
 int ct_unary_reduce(void* stream, void* output, const ct_dims* output_dims, double input_alpha,
                     const void* input, const ct_dims* input_dims, int op, int dtype);
 
+/* The same reduction for callers that cannot allocate device memory while they
+ * run: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference.  It runs ct_unary_reduce's
+ * kernels with ct_unary_reduce's plan, so the results are the same bits, but
+ * the partial accumulators of a split reduction (a column reduction through a
+ * transposed view, a few very long rows) live in a fixed 2 MiB array that every
+ * device the library runs on holds until the process ends, and the call makes
+ * no hipMalloc / hipFree.  A reduction whose partial accumulators need more
+ * than 2 MiB fails with CT_ERR_INVALID and launches nothing.  All calls on one
+ * device share the array: calls that overlap in time on one device (two
+ * streams, two host threads) race; calls on one stream are ordered and safe.
+ * The first call on a device resolves the array's address; make that call
+ * before a graph capture starts. */
+int ct_unary_reduce_noalloc(void* stream, void* output, const ct_dims* output_dims,
+                            double input_alpha, const void* input, const ct_dims* input_dims,
+                            int op, int dtype);
+
 /* ------------------------------------------------- neural-network tensor ops */
 
 /* activation-gradient! (tensor/math.clj:176-181; cpu/tensor_math.clj:1318-1362):

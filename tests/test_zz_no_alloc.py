@@ -1,0 +1,110 @@
+"""ct_unary_reduce_noalloc: the reduction entry point that allocates nothing.
+
+Its partial accumulators live in a fixed array in device memory, shared by all
+calls on a device and holding whatever the previous call left there.  Every
+case below therefore runs two calls in a row through the C ABI, the second on
+a smaller input, and compares each output with ct_unary_reduce's on the same
+input: both run the same kernels with the same plan, so the bar is bit-exact
+for every datatype.  The oracle is checked as well (max / min and integers
+bit-exact, float sums to 2e-6 of the sum of magnitudes, 1e-12 for doubles).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness as H
+from cortex_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+def _reduce(entry, side, out: H.View, alpha, inp: H.View, op):
+    capi.call(entry, side.stream, side.ptr(out), C.byref(side.dims(out)), float(alpha), side.ptr(inp),
+              C.byref(side.dims(inp)), capi.REDUCE_OPS[op], out.buf.dtype)
+    capi.call("ct_stream_sync", side.stream)
+
+
+def _check(pair, data: np.ndarray, shape, strides, op, alpha=1.0):
+    """Reduces the last axis of the view (shape, strides) of `data` through both entry points."""
+    n_out = int(np.prod(shape[:-1]))
+    src = pair.buf(data)
+    want = pair.buf(np.zeros(n_out, data.dtype))
+    got = pair.buf(np.full(n_out, 77, data.dtype))
+    view = H.View(src, shape, strides)
+    out_shape = list(shape[:-1]) + [1]
+    H.unary_reduce(H.ORACLE, H.View(want, out_shape), alpha, view, op)
+    _reduce("ct_unary_reduce", pair.hip, H.View(want, out_shape), alpha, view, op)
+    kernel = capi.last_kernel()
+    _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(got, out_shape), alpha, view, op)
+    assert capi.last_kernel() == kernel
+    what = f"{op} {data.dtype} view {shape} strides {strides} ({kernel})"
+    H.assert_bit_exact(got.download(), want.download(), "noalloc vs ct_unary_reduce: " + what)
+    oracle = want.host
+    if data.dtype.kind != "f" or op in ("max", "min"):
+        H.assert_bit_exact(got.download(), oracle, "noalloc vs oracle: " + what)
+    else:
+        k = shape[-1]
+        scale = np.abs(view.gather_host(src.init).astype(np.float64) * alpha)
+        scale = (scale ** 2 if op.startswith("magnitude") else scale).reshape(n_out, k).sum(axis=1)
+        if op == "magnitude":
+            scale = np.sqrt(scale)
+        if op == "mean":
+            scale = scale / k
+        tol = 2e-6 if data.dtype == np.float32 else 1e-12
+        err = np.abs(got.download().astype(np.float64) - oracle.astype(np.float64))
+        assert np.all(err <= tol * np.maximum(scale, 1e-30)), what
+    return kernel
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int8])
+@pytest.mark.parametrize("op", ["sum", "max", "magnitude-squared", "mean"])
+def test_column_reduction_twice_second_smaller(pair_factory, dtype, op):
+    rng = np.random.default_rng(11)
+    with pair_factory() as pair:
+        for rows, cols in ((2048, 1024), (640, 384)):  # the second call is smaller and meets the first one's leftovers
+            if np.dtype(dtype).kind == "f":
+                data = rng.standard_normal(rows * cols).astype(dtype)
+            else:
+                info = np.iinfo(dtype)
+                data = rng.integers(info.min, info.max, rows * cols, dtype=np.int64).astype(dtype)
+            kernel = _check(pair, data, [cols, rows], [1, cols], op)
+            assert kernel.startswith("reduce_col"), kernel
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_split_rows_twice_second_smaller(pair_factory, dtype):
+    """A few very long rows: each row is cut into chunks whose partials go through the fixed array."""
+    rng = np.random.default_rng(12)
+    with pair_factory() as pair:
+        for rows, cols in ((3, 1 << 20), (2, 1 << 18)):
+            data = rng.standard_normal(rows * cols).astype(dtype)
+            for op in ("sum", "min", "magnitude"):
+                _check(pair, data, [rows, cols], [cols, 1], op, alpha=1.0 if op == "min" else 0.5)
+
+
+def test_unsplit_shapes_and_ragged_views(pair_factory):
+    """Shapes that need no partial accumulators run unchanged."""
+    rng = np.random.default_rng(13)
+    with pair_factory() as pair:
+        data = rng.standard_normal(4096 * 96).astype(np.float32)
+        _check(pair, data, [4096, 96], [96, 1], "sum")
+        _check(pair, data, [96, 4096], [1, 96], "max")
+        _check(pair, data, [7, 13, 5], [65, 5, 1], "mean")
+        _check(pair, data[:1], [1, 1], [1, 1], "sum")
+
+
+def test_rejects_what_the_fixed_array_cannot_hold(pair_factory):
+    """64 Ki byte-wide columns cut into 8 segments need 4 MiB of long accumulators: refused, nothing launched."""
+    rows, cols = 1024, 65536
+    with pair_factory() as pair:
+        data = np.random.default_rng(14).integers(-128, 128, rows * cols, dtype=np.int64).astype(np.int8)
+        src = pair.buf(data)
+        out = pair.buf(np.full(cols, 5, np.int8))
+        view = H.View(src, [cols, rows], [1, cols])
+        with pytest.raises(capi.CortexHipError) as err:
+            _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")
+        assert err.value.status == 1 and "fixed scratch holds 2097152" in err.value.message
+        assert np.all(out.download() == 5)
+        _reduce("ct_unary_reduce", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")  # the allocating form takes it
+        assert np.array_equal(out.download(), data.reshape(rows, cols).astype(np.int64).sum(axis=0).astype(np.int8))
