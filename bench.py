@@ -1,29 +1,46 @@
 #!/usr/bin/env python3
 """Benchmark of the tensor-math hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sections a,b,...] [--no-cpu]
+    python bench.py --profile-plan FILE ...        (under rocprofv3: marks the segments of the run)
+    python bench.py --summarize DIR [--out DIR2]   (turns rocprofv3 output into profiles/ summaries)
 
-One step is one pass of BASELINE.json configs[1] over its synthetic input:
-``unary-op! :exp``, ``unary-op! :tanh`` and ``ternary-op! :select`` on
-transposed views (strides [1, 8192]) of float32 [8192, 8192] tensors, output
-contiguous.  Inputs are resident in HBM before the timed region.  The line
-printed at the end follows the driver's contract; ``value`` is algorithmic
-bytes per second (each input element read once, each output element written
-once) over the K timed steps.
+The metric is achieved HBM bandwidth of ``binary-op!``, ``unary-reduce!`` and the
+Adam step.  One step is one pass of those three workloads at their BASELINE
+shapes over synthetic inputs that are resident in HBM before the timed region:
 
-``roofline`` describes the dominant kernel of the step (the LDS-tiled kernel
-running ``:select``, three transposed inputs), timed with HIP events recorded on
-the launch stream around every one of its launches inside the timed region.
+    configs[3]  fused Adam step over 2^28 float32 parameters (the dominant kernel)
+    configs[2]  unary-reduce! :sum :max :magnitude-squared over the last axis of
+                float32 [16384,4096] and over axis 0 through a transposed view, and
+                the same six reductions of float64 [4096,4096]
+    configs[0]  binary-op! :+ of float32 [1024,1024] with a broadcast [1024] row
+
+``value`` is the algorithmic bytes of one step (each input element read once,
+each output element written once) over the step's time.  ``roofline`` describes
+the Adam kernel, timed with HIP events recorded on the launch stream around each
+of its launches inside the timed region.  ``ops`` carries a roofline-shaped block
+for every workload of the step (and the Adadelta step of configs[3]), each timed
+on its own, back to back.  ``others`` holds BASELINE configs[1] and [4] and the
+scaled form of configs[0]; ``patterns`` the access patterns off the three fast
+kernel families; ``adjacent`` the neighbouring TensorMath methods.
 ``cpu_baseline`` times the CPU oracle (a C++ restatement of the cortex CPU
-backend, OpenMP) on the same step.  ``others`` reports the remaining BASELINE
-configs and ``adjacent`` the neighbouring TensorMath methods, each timed the
-same way, as additional information.
+backend, OpenMP) on the same step.
+
+``traffic`` figures are HBM bytes per call measured with rocprofv3 counters and
+stored in ``profiles/traffic.json`` together with a hash of the kernel sources
+they were measured on; when the sources have changed since, the run reports
+``null`` and says so.
 """
 from __future__ import annotations
 
 import argparse
+import collections
+import csv
 import ctypes as C
+import glob
+import hashlib
 import json
+import re
 import sys
 import time
 from pathlib import Path
@@ -34,11 +51,41 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
+SECTIONS = ("headline", "others", "patterns", "adjacent")
 
 
 def log(msg: str) -> None:
     print(msg, file=sys.stderr, flush=True)
 
+
+# ----------------------------------------------------------------------------- sources hash / stored traffic
+
+def csrc_hash() -> str:
+    """SHA-256 over the kernel sources and the C header, in name order."""
+    h = hashlib.sha256()
+    files = sorted(p for p in (ROOT / "cortex_amd" / "csrc").iterdir() if p.suffix in (".hip", ".h", ".cpp"))
+    for p in files + [ROOT / "include" / "cortex_hip.h"]:
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
+    return h.hexdigest()
+
+
+def load_traffic():
+    """Stored rocprofv3 traffic per workload key, or ({}, reason) when it does not describe these sources."""
+    tfile = ROOT / "profiles" / "traffic.json"
+    if not tfile.exists():
+        return {}, "profiles/traffic.json is missing"
+    try:
+        stored = json.loads(tfile.read_text())
+    except (ValueError, OSError) as err:
+        return {}, f"profiles/traffic.json unreadable: {err}"
+    if stored.get("csrc_sha256") != csrc_hash():
+        return {}, ("the kernel sources changed since profiles/traffic.json was measured "
+                    f"(stored {str(stored.get('csrc_sha256'))[:12]}, now {csrc_hash()[:12]}): traffic not reported")
+    return stored.get("ops", {}), None
+
+
+# ----------------------------------------------------------------------------- timing helpers
 
 class Timer:
     """HIP-event timing on one stream."""
@@ -62,18 +109,6 @@ class Timer:
             self.capi.call("ct_event_destroy", e)
 
 
-def upload(driver_mod, device, stream, array: np.ndarray):
-    """Copies a numpy array into a fresh device buffer."""
-    flat = np.ascontiguousarray(array).reshape(-1)
-    dt = driver_mod.DATATYPE_OF_NUMPY[flat.dtype]
-    buf = device.allocate_device_buffer(flat.size, dt)
-    from cortex_amd import capi
-
-    capi.call("ct_memcpy_async", buf.ptr, flat.ctypes.data, flat.nbytes, capi.COPY_H2D, stream.handle)
-    stream.sync()
-    return buf
-
-
 def dims(shape, strides=None):
     if strides is None:
         strides, m = [], 1
@@ -83,327 +118,586 @@ def dims(shape, strides=None):
     return {"shape": list(shape), "strides": list(strides)}
 
 
-def time_launches(timer, stream, fn, iters: int, warm: int = 2):
-    """Average duration in ms of `fn` (one or more launches) over `iters` runs."""
-    for _ in range(warm):
-        fn()
-    stream.sync()
-    e0 = timer.mark()
-    for _ in range(iters):
-        fn()
-    e1 = timer.mark()
-    ms = timer.elapsed_ms(e0, e1) / iters
-    timer.free(e0, e1)
-    return ms
-
-
 def gbs(nbytes: float, ms: float) -> float:
     return nbytes / (ms * 1e-3) / 1e9
 
 
-def run_extras(drv, device, stream, timer, capi) -> dict:
-    """BASELINE configs 0, 2, 3, 4 (additional information, not the headline).
+class Op:
+    """One timed call of the library: `fn()` issues it on the bench stream."""
 
-    Buffers are not released between configs: on this board a large buffer
-    allocated after frees can land less favourably and cost several percent of
-    bandwidth, which would make the figures depend on the order of the configs."""
-    out = {}
-    rng = np.random.default_rng(0)
+    def __init__(self, key, label, nbytes, fn, iters=20, config=None):
+        self.key, self.label, self.nbytes, self.fn, self.iters, self.config = key, label, nbytes, fn, iters, config
+        self.kernel = ""
 
-    def entry(nbytes, ms):
-        return {"us": round(ms * 1e3, 2), "GB/s": round(gbs(nbytes, ms), 1), "frac": round(gbs(nbytes, ms) / PEAK_HBM_GBS, 4),
-                "kernel": capi.last_kernel()}
 
-    # configs[0]: bias add [1024,1024] + [1024] (8 MiB: cache resident, launch bound)
-    x = upload(drv, device, stream, rng.uniform(-1, 1, 1024 * 1024).astype(np.float32))
-    b = upload(drv, device, stream, rng.uniform(-1, 1, 1024).astype(np.float32))
-    d = device.allocate_device_buffer(1024 * 1024, "float")
-    ms = time_launches(timer, stream, lambda: stream.binary_op(d, dims([1024, 1024]), x, dims([1024, 1024]), 1.0, b,
-                                                               dims([1024]), 1.0, 1024 * 1024, "+"), 200)
-    out["config0 binary-op! :+ [1024,1024]+[1024]"] = entry(8392704, ms)
-    # the same op at a size that exercises HBM
-    n = 16384
-    x = upload(drv, device, stream, rng.standard_normal(n * n, dtype=np.float32))
-    b = upload(drv, device, stream, rng.uniform(-1, 1, n).astype(np.float32))
-    d = device.allocate_device_buffer(n * n, "float")
-    ms = time_launches(timer, stream, lambda: stream.binary_op(d, dims([n, n]), x, dims([n, n]), 1.0, b, dims([n]), 1.0,
-                                                               n * n, "+"), 20)
-    out["config0 scaled binary-op! :+ [16384,16384]+[16384]"] = entry(8 * n * n + 4 * n, ms)
+class Bench:
+    def __init__(self, plan_path=None):
+        from cortex_amd import capi, driver as drv
 
-    # configs[2]: unary-reduce!
-    r, c = 16384, 4096
-    x = upload(drv, device, stream, np.random.default_rng(4).standard_normal(r * c, dtype=np.float32))
-    o_rows = device.allocate_device_buffer(r, "float")
-    o_cols = device.allocate_device_buffer(c, "float")
-    for op in ("sum", "max", "magnitude-squared"):
-        ms = time_launches(timer, stream, lambda: stream.unary_reduce(o_rows, dims([r, 1]), 1.0, x, dims([r, c]), op), 20)
-        out[f"config2 unary-reduce! :{op} last axis f32 [16384,4096]"] = entry(4 * r * c + 4 * r, ms)
-        ms = time_launches(timer, stream, lambda: stream.unary_reduce(o_cols, dims([c, 1]), 1.0, x, dims([c, r], [1, c]), op), 20)
-        out[f"config2 unary-reduce! :{op} axis 0 (transposed view) f32"] = entry(4 * r * c + 4 * c, ms)
-    r = c = 4096
-    x = upload(drv, device, stream, np.random.default_rng(5).standard_normal(r * c))
-    o = device.allocate_device_buffer(r, "double")
-    for op in ("sum", "max", "magnitude-squared"):
-        ms = time_launches(timer, stream, lambda: stream.unary_reduce(o, dims([r, 1]), 1.0, x, dims([r, c]), op), 20)
-        out[f"config2 unary-reduce! :{op} last axis f64 [4096,4096]"] = entry(8 * r * c + 8 * r, ms)
-        ms = time_launches(timer, stream, lambda: stream.unary_reduce(o, dims([c, 1]), 1.0, x, dims([c, r], [1, c]), op), 20)
-        out[f"config2 unary-reduce! :{op} axis 0 (transposed view) f64"] = entry(8 * r * c + 8 * r, ms)
+        self.capi, self.drv = capi, drv
+        self.driver = drv.HipDriver()
+        self.device = self.driver.default_device()
+        self.device.make_current()
+        self.stream = self.device.create_stream()
+        self.timer = Timer(capi, self.stream)
+        self.traffic, self.traffic_note = load_traffic()
+        self.plan = [] if plan_path else None
+        self.plan_path = plan_path
+        self.marker_buf = self.device.allocate_device_buffer(256, "byte") if plan_path else None
+        # Buffers stay allocated until the end: on this board a large buffer allocated after frees can land
+        # less favourably and cost several percent of bandwidth, which would make figures depend on the order.
+        self.keep = []
 
-    # configs[3]: Adam and Adadelta over 2^28 float parameters
-    n = 1 << 28
-    g6 = np.random.default_rng(6)
-    p = upload(drv, device, stream, g6.uniform(-0.05, 0.05, n).astype(np.float32))
-    g = upload(drv, device, stream, g6.standard_normal(n, dtype=np.float32) * np.float32(1e-3))
-    m = device.allocate_device_buffer(n, "float")
-    v = device.allocate_device_buffer(n, "float")
-    stream.memset(m, 0, 0.0, n)
-    stream.memset(v, 0, 1e-6, n)
+    # -- profile plan: under rocprofv3 every segment of the run starts with a marker launch (a one-byte
+    # fill) so that the dispatches of the trace can be attributed to workloads by order alone
+    def segment(self, key, label, calls, nbytes):
+        if self.plan is None:
+            return
+        self.stream.memset(self.marker_buf, 0, 1, 1)
+        self.plan.append({"key": key, "label": label, "calls": calls, "algorithmic_bytes": nbytes})
+
+    def save_plan(self):
+        if self.plan is not None:
+            Path(self.plan_path).write_text(json.dumps({"csrc_sha256": csrc_hash(), "segments": self.plan}, indent=1))
+
+    def upload(self, array: np.ndarray):
+        flat = np.ascontiguousarray(array).reshape(-1)
+        dt = self.drv.DATATYPE_OF_NUMPY[flat.dtype]
+        buf = self.device.allocate_device_buffer(flat.size, dt)
+        self.capi.call("ct_memcpy_async", buf.ptr, flat.ctypes.data, flat.nbytes, self.capi.COPY_H2D, self.stream.handle)
+        self.stream.sync()
+        return buf
+
+    def alloc(self, n, dt):
+        return self.device.allocate_device_buffer(n, dt)
+
+    def time_op(self, op: Op, warm: int = 2) -> dict:
+        """Average duration of `op` over op.iters back-to-back calls, as a roofline-shaped block."""
+        # the marker precedes the warm-up calls, which therefore count among the segment's dispatches
+        self.segment(op.key, op.label, op.iters + warm, op.nbytes)
+        for _ in range(warm):
+            op.fn()
+        self.stream.sync()
+        op.kernel = self.capi.last_kernel()
+        t0 = time.perf_counter()
+        e0 = self.timer.mark()
+        for _ in range(op.iters):
+            op.fn()
+        e1 = self.timer.mark()
+        host_ms = (time.perf_counter() - t0) * 1e3 / op.iters  # submission only: nothing has been waited for yet
+        ms = self.timer.elapsed_ms(e0, e1) / op.iters
+        self.timer.free(e0, e1)
+        return self.block(op, ms, host_us=host_ms * 1e3)
+
+    def block(self, op: Op, ms: float, **more) -> dict:
+        rate = gbs(op.nbytes, ms)
+        stored = self.traffic.get(op.key)
+        b = {"bound": "hbm", "achieved": round(rate, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+             "frac": round(rate / PEAK_HBM_GBS, 4), "traffic": stored["traffic"] if stored else None,
+             "avg_call_us": round(ms * 1e3, 2), "algorithmic_bytes_per_call": op.nbytes, "kernel": op.kernel}
+        if stored:
+            b["kernel_us_rocprof"] = stored.get("kernel_us")
+        for k, v in more.items():
+            b[k] = round(v, 2) if isinstance(v, float) else v
+        return b
+
+
+# ----------------------------------------------------------------------------- the step: configs[3], [2], [0]
+
+def pow_betas(t=10):
     pb1 = pb2 = 1.0
-    for _ in range(10):
+    for _ in range(t):
         pb1 *= 0.9
         pb2 *= 0.999
-    ms = time_launches(timer, stream, lambda: stream.adam_step(1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 1.0, g, p, m, v, n), 10)
-    out["config3 Adam step 2^28 f32"] = entry(28 * n, ms)
-    stream.memset(m, 0, 0.0, n)
-    stream.memset(v, 0, 0.0, n)
-    ms = time_launches(timer, stream, lambda: stream.adadelta_step(0.05, 1e-6, m, v, 1.0, g, p, n), 10)
-    out["config3 Adadelta step 2^28 f32"] = entry(28 * n, ms)
+    return pb1, pb2
 
+
+class StepData:
+    """Host arrays of the step's workloads (also used by the CPU baseline)."""
+
+    def __init__(self, adam_n: int):
+        log("generating inputs (numpy default_rng, seeds 0, 4, 5, 6) ...")
+        g0 = np.random.default_rng(0)
+        self.x0 = g0.uniform(-1, 1, 1024 * 1024).astype(np.float32)
+        self.b0 = g0.uniform(-1, 1, 1024).astype(np.float32)
+        self.red32 = np.random.default_rng(4).standard_normal(16384 * 4096, dtype=np.float32)
+        self.red64 = np.random.default_rng(5).standard_normal(4096 * 4096)
+        g6 = np.random.default_rng(6)
+        self.adam_n = adam_n
+        self.p = g6.uniform(-0.05, 0.05, adam_n).astype(np.float32)
+        self.g = g6.standard_normal(adam_n, dtype=np.float32) * np.float32(1e-3)
+
+
+REDUCE_OPS = ("sum", "max", "magnitude-squared")
+
+
+def build_step(b: Bench, data: StepData):
+    """The workloads of one step, in the order they run.  Returns (ops, adam_op, extra_ops)."""
+    s = b.stream
+    ops = []
+    # configs[3]: Adam
+    n = data.adam_n
+    p, g = b.upload(data.p), b.upload(data.g)
+    m, v = b.alloc(n, "float"), b.alloc(n, "float")
+    s.memset(m, 0, 0.0, n)
+    s.memset(v, 0, 1e-6, n)
+    pb1, pb2 = pow_betas()
+    adam = Op("c3_adam", f"configs[3] Adam step, {n} float32 parameters", 28 * n,
+              lambda: s.adam_step(1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 1.0, g, p, m, v, n), iters=10)
+    ops.append(adam)
+    # configs[2]: reductions
+    r, c = 16384, 4096
+    x32 = b.upload(data.red32)
+    o_rows, o_cols = b.alloc(r, "float"), b.alloc(c, "float")
+    for op in REDUCE_OPS:
+        ops.append(Op(f"c2_{op}_rows_f32", f"configs[2] unary-reduce! :{op} last axis of float32 [{r},{c}]", 4 * r * c + 4 * r,
+                      lambda op=op: s.unary_reduce(o_rows, dims([r, 1]), 1.0, x32, dims([r, c]), op)))
+        ops.append(Op(f"c2_{op}_cols_f32", f"configs[2] unary-reduce! :{op} axis 0 of float32 [{r},{c}] (transposed view)",
+                      4 * r * c + 4 * c,
+                      lambda op=op: s.unary_reduce(o_cols, dims([c, 1]), 1.0, x32, dims([c, r], [1, c]), op)))
+    q = 4096
+    x64 = b.upload(data.red64)
+    o64 = b.alloc(q, "double")
+    for op in REDUCE_OPS:
+        ops.append(Op(f"c2_{op}_rows_f64", f"configs[2] unary-reduce! :{op} last axis of float64 [{q},{q}]", 8 * q * q + 8 * q,
+                      lambda op=op: s.unary_reduce(o64, dims([q, 1]), 1.0, x64, dims([q, q]), op)))
+        ops.append(Op(f"c2_{op}_cols_f64", f"configs[2] unary-reduce! :{op} axis 0 of float64 [{q},{q}] (transposed view)",
+                      8 * q * q + 8 * q,
+                      lambda op=op: s.unary_reduce(o64, dims([q, 1]), 1.0, x64, dims([q, q], [1, q]), op)))
+    # configs[0]: bias add at its stated shape (8 MiB: cache resident, launch bound)
+    x0, b0 = b.upload(data.x0), b.upload(data.b0)
+    d0 = b.alloc(1024 * 1024, "float")
+    ops.append(Op("c0_bias_add", "configs[0] binary-op! :+ float32 [1024,1024] + [1024] row", 8392704,
+                  lambda: s.binary_op(d0, dims([1024, 1024]), x0, dims([1024, 1024]), 1.0, b0, dims([1024]), 1.0,
+                                      1024 * 1024, "+"), iters=200))
+    # the Adadelta step of configs[3]: timed on its own, not part of the step (the metric names Adam)
+    acc_g, acc_d = b.alloc(n, "float"), b.alloc(n, "float")
+    s.memset(acc_g, 0, 0.0, n)
+    s.memset(acc_d, 0, 0.0, n)
+    adadelta = Op("c3_adadelta", f"configs[3] Adadelta step, {n} float32 parameters", 28 * n,
+                  lambda: s.adadelta_step(0.05, 1e-6, acc_g, acc_d, 1.0, g, p, n), iters=10)
+    return ops, adam, [adadelta]
+
+
+# ----------------------------------------------------------------------------- others: configs[0] scaled, [1], [4]
+
+def build_others(b: Bench):
+    s = b.stream
+    ops = []
+    rng = np.random.default_rng(0)
+    n = 16384
+    x = b.upload(rng.standard_normal(n * n, dtype=np.float32))
+    bias = b.upload(rng.uniform(-1, 1, n).astype(np.float32))
+    d = b.alloc(n * n, "float")
+    ops.append(Op("c0_bias_add_scaled", "configs[0] scaled: binary-op! :+ float32 [16384,16384] + [16384] row", 8 * n * n + 4 * n,
+                  lambda: s.binary_op(d, dims([n, n]), x, dims([n, n]), 1.0, bias, dims([n]), 1.0, n * n, "+")))
+    # configs[1]: transposed views of [8192,8192]
+    e = 8192
+    ee = e * e
+    xs = [b.upload(np.random.default_rng(seed).standard_normal(ee).astype(np.float32)) for seed in (1, 2, 3)]
+    cont, view = dims([e, e]), dims([e, e], [1, e])
+    dest = d  # reuse (larger than needed)
+    ops.append(Op("c1_exp_t", "configs[1] unary-op! :exp on a transposed float32 [8192,8192] view", 8 * ee,
+                  lambda: s.unary_op(dest, cont, xs[0], view, 1.0, "exp", ee)))
+    ops.append(Op("c1_tanh_t", "configs[1] unary-op! :tanh on a transposed float32 [8192,8192] view", 8 * ee,
+                  lambda: s.unary_op(dest, cont, xs[0], view, 1.0, "tanh", ee)))
+    ops.append(Op("c1_select_t", "configs[1] ternary-op! :select, three transposed float32 [8192,8192] views", 16 * ee,
+                  lambda: s.ternary_op(dest, cont, xs[0], view, 1.0, xs[1], view, 1.0, xs[2], view, 1.0, ee, "select")))
+    ops.append(Op("calibration_copy", "calibration: unary-op! :noop, contiguous float32 [8192,8192] (256 MiB in, 256 MiB out)", 8 * ee,
+                  lambda: s.unary_op(dest, cont, xs[0], cont, 1.0, "noop", ee)))
     # configs[4]: mixed-dtype image normalise
     shp = [256, 3, 224, 224]
-    n = int(np.prod(shp))
-    u8 = upload(drv, device, stream, np.random.default_rng(7).integers(0, 256, n, dtype=np.uint8))
-    f = device.allocate_device_buffer(n, "float")
-    f2 = device.allocate_device_buffer(n, "float")
-    mean = upload(drv, device, stream, (np.array([0.485, 0.456, 0.406]) * 255).astype(np.float32))
-    std = upload(drv, device, stream, (np.array([0.229, 0.224, 0.225]) * 255).astype(np.float32))
-    ms = time_launches(timer, stream, lambda: stream.assign(f, dims(shp), u8, dims(shp), n), 20)
-    out["config4 assign! u8->f32 [256,3,224,224]"] = entry(5 * n, ms)
-    ms = time_launches(timer, stream, lambda: stream.binary_op(f2, dims(shp), f, dims(shp), 1.0, mean, dims([3, 1, 1]),
-                                                               -1.0, n, "+"), 20)
-    out["config4 binary-op! :- per-channel mean"] = entry(8 * n + 12, ms)
-    ms = time_launches(timer, stream, lambda: stream.binary_op(f2, dims(shp), f, dims(shp), 1.0, std, dims([3, 1, 1]),
-                                                               1.0, n, "/"), 20)
-    out["config4 binary-op! :/ per-channel std"] = entry(8 * n + 12, ms)
-    n = 1 << 26
-    i32 = upload(drv, device, stream, np.random.default_rng(8).integers(-2 ** 31, 2 ** 31, n, dtype=np.int64).astype(np.int32))
-    f64 = device.allocate_device_buffer(n, "double")
-    ms = time_launches(timer, stream, lambda: stream.assign(f64, dims([n]), i32, dims([n]), n), 20)
-    out["config4 assign! i32->f64 [64M]"] = entry(12 * n, ms)
-    return out
+    ni = int(np.prod(shp))
+    u8 = b.upload(np.random.default_rng(7).integers(0, 256, ni, dtype=np.uint8))
+    f, f2 = b.alloc(ni, "float"), b.alloc(ni, "float")
+    mean = b.upload((np.array([0.485, 0.456, 0.406]) * 255).astype(np.float32))
+    std = b.upload((np.array([0.229, 0.224, 0.225]) * 255).astype(np.float32))
+    ops.append(Op("c4_u8_f32", "configs[4] assign! uint8 -> float32 [256,3,224,224]", 5 * ni,
+                  lambda: s.assign(f, dims(shp), u8, dims(shp), ni)))
+    ops.append(Op("c4_sub_mean", "configs[4] binary-op! :- per-channel mean [3,1,1]", 8 * ni + 12,
+                  lambda: s.binary_op(f2, dims(shp), f, dims(shp), 1.0, mean, dims([3, 1, 1]), -1.0, ni, "+")))
+    ops.append(Op("c4_div_std", "configs[4] binary-op! :/ per-channel std [3,1,1]", 8 * ni + 12,
+                  lambda: s.binary_op(f2, dims(shp), f, dims(shp), 1.0, std, dims([3, 1, 1]), 1.0, ni, "/")))
+    nv = 1 << 26
+    i32 = b.upload(np.random.default_rng(8).integers(-2 ** 31, 2 ** 31, nv, dtype=np.int64).astype(np.int32))
+    f64 = b.alloc(nv, "double")
+    ops.append(Op("c4_i32_f64", "configs[4] assign! int32 -> float64 [64M]", 12 * nv,
+                  lambda: s.assign(f64, dims([nv]), i32, dims([nv]), nv)))
+    return ops
 
 
-def run_adjacent(drv, device, stream, timer, capi) -> dict:
-    """The adjacent TensorMath methods built on the same machinery (activation-gradient!,
-    softmax!, batch normalization, rand!, gemv!, gemm!), timed like the BASELINE configs.  Bytes
-    are algorithmic: every operand read once, every result written once, although the
+# ----------------------------------------------------------------------------- patterns off the fast families
+
+class _Tensor:
+    """What the driver's dimension maps accept as an index tensor: an object with a `.buffer`."""
+
+    def __init__(self, buffer):
+        self.buffer = buffer
+
+
+def build_patterns(b: Bench):
+    """Access patterns that real cortex callers produce beside the contiguous / broadcast / transposed
+    ones (the census of the tensor layer's callers): gather and scatter-add through an index tensor
+    (center loss), strided vectors (ct/columns, select :all k), planar <-> interleaved images, and
+    accumulation into a broadcast destination with an op other than :+."""
+    s = b.stream
+    ops = []
+    rng = np.random.default_rng(21)
+    # center loss (loss/center.clj:32, 75, 92): rows of [1000,512] centers selected by 4096 labels
+    n_cls, width, batch = 1000, 512, 4096
+    centers = b.upload(rng.standard_normal(n_cls * width, dtype=np.float32))
+    labels = b.upload(rng.integers(0, n_cls, batch, dtype=np.int64).astype(np.int32))
+    feats = b.upload(rng.standard_normal(batch * width, dtype=np.float32))
+    gathered = b.alloc(batch * width, "float")
+    idx_dims = {"shape": [_Tensor(labels), width], "strides": [width, 1]}
+    ops.append(Op("p_gather_rows", f"assign! gather: float32 [{batch},{width}] <- centers [{n_cls},{width}] through {batch} labels",
+                  8 * batch * width + 4 * batch,
+                  lambda: s.assign(gathered, dims([batch, width]), centers, idx_dims, batch * width)))
+    ops.append(Op("p_scatter_add_rows", f"binary-op! :+ scatter-add: centers [{n_cls},{width}] (indexed by {batch} labels) += float32 [{batch},{width}]",
+                  4 * batch * width + 8 * min(batch, n_cls) * width + 4 * batch,
+                  lambda: s.binary_accum(centers, idx_dims, 1.0, feats, dims([batch, width]), 1e-3, batch * width, "+", False, True),
+                  iters=5))
+    # large gather: 2^16 rows of 1024 floats out of 2^15
+    rows_src, rows_out, w2 = 1 << 15, 1 << 16, 1024
+    table = b.upload(rng.standard_normal(rows_src * w2, dtype=np.float32))
+    picks = b.upload(rng.integers(0, rows_src, rows_out, dtype=np.int64).astype(np.int32))
+    out2 = b.alloc(rows_out * w2, "float")
+    big_idx = {"shape": [_Tensor(picks), w2], "strides": [w2, 1]}
+    ops.append(Op("p_gather_rows_large", f"assign! gather: float32 [{rows_out},{w2}] <- table [{rows_src},{w2}] through an index tensor",
+                  8 * rows_out * w2 + 4 * rows_out,
+                  lambda: s.assign(out2, dims([rows_out, w2]), table, big_idx, rows_out * w2)))
+    # strided vector: one column of a [2^22, 16] matrix (ct/columns, select :all k)
+    rows_v, pitch = 1 << 22, 16
+    mat = b.upload(rng.standard_normal(rows_v * pitch, dtype=np.float32))
+    colv = b.alloc(rows_v, "float")
+    ops.append(Op("p_strided_vector", f"assign! strided vector: float32 [{rows_v}] <- column of [{rows_v},{pitch}] (stride {pitch})",
+                  8 * rows_v,  # the elements asked for; the lines they sit in are 16 times that
+                  lambda: s.assign(colv, dims([rows_v]), mat, dims([rows_v], [pitch]), rows_v)))
+    # planar <-> interleaved images (verify/tensor.clj:668-684, 785-805)
+    nb, hh, ww, ch = 256, 224, 224, 3
+    npx = nb * hh * ww * ch
+    inter = b.upload(rng.standard_normal(npx, dtype=np.float32))
+    planar = b.alloc(npx, "float")
+    planar_dims = dims([nb, ch, hh, ww])
+    inter_as_planar = dims([nb, ch, hh, ww], [hh * ww * ch, 1, ww * ch, ch])
+    ops.append(Op("p_interleaved_to_planar", f"assign! planar [{nb},{ch},{hh},{ww}] <- interleaved [{nb},{hh},{ww},{ch}] float32",
+                  8 * npx, lambda: s.assign(planar, planar_dims, inter, inter_as_planar, npx)))
+    inter_dims = dims([nb, hh, ww, ch])
+    planar_as_inter = dims([nb, hh, ww, ch], [ch * hh * ww, ww, 1, hh * ww])
+    ops.append(Op("p_planar_to_interleaved", f"assign! interleaved [{nb},{hh},{ww},{ch}] <- planar [{nb},{ch},{hh},{ww}] float32",
+                  8 * npx, lambda: s.assign(inter, inter_dims, planar, planar_as_inter, npx)))
+    # accumulate into a broadcast destination with :max (owner kernel) and with :+ (staged sums)
+    bb, kk = 16384, 4096
+    y = b.upload(rng.standard_normal(bb * kk, dtype=np.float32))
+    acc = b.alloc(kk, "float")
+    s.memset(acc, 0, 0.0, kk)
+    ops.append(Op("p_accum_max_rows", f"binary-op! :max accumulate: float32 [{kk}] <- max over rows of [{bb},{kk}]",
+                  4 * bb * kk + 8 * kk,
+                  lambda: s.binary_accum(acc, dims([kk]), 1.0, y, dims([bb, kk]), 1.0, bb * kk, "max", False, True), iters=10))
+    ops.append(Op("p_accum_sum_rows", f"binary-op! :+ accumulate (bias gradient): float32 [{kk}] += rows of [{bb},{kk}]",
+                  4 * bb * kk + 8 * kk,
+                  lambda: s.binary_accum(acc, dims([kk]), 1.0, y, dims([bb, kk]), 1.0, bb * kk, "+", False, True)))
+    return ops
+
+
+# ----------------------------------------------------------------------------- adjacent TensorMath methods
+
+def build_adjacent(b: Bench):
+    """activation-gradient!, softmax!, batch normalization, rand!, gemv!: HBM-bound like the hot path.
+    Bytes are algorithmic (every operand read once, every result written once) although the
     batch-normalization forms that need batch statistics read their operands twice."""
-    out = {}
+    s = b.stream
+    ops = []
     rng = np.random.default_rng(9)
-
-    def entry(nbytes, ms, **more):
-        e = {"us": round(ms * 1e3, 2), "GB/s": round(gbs(nbytes, ms), 1), "frac": round(gbs(nbytes, ms) / PEAK_HBM_GBS, 4),
-             "kernel": capi.last_kernel()}
-        e.update(more)
-        return e
-
     n = 1 << 27
-    x = upload(drv, device, stream, rng.standard_normal(n, dtype=np.float32))
-    g = upload(drv, device, stream, rng.standard_normal(n, dtype=np.float32))
-    o = device.allocate_device_buffer(n, "float")
-    ms = time_launches(timer, stream, lambda: stream.activation_gradient(o, dims([n]), g, dims([n]), x, dims([n]), "tanh", n), 20)
-    out["activation-gradient! :tanh f32 [2^27]"] = entry(12 * n, ms)
+    x = b.upload(rng.standard_normal(n, dtype=np.float32))
+    g = b.upload(rng.standard_normal(n, dtype=np.float32))
+    o = b.alloc(n, "float")
+    ops.append(Op("a_actgrad_tanh", "activation-gradient! :tanh float32 [2^27]", 12 * n,
+                  lambda: s.activation_gradient(o, dims([n]), g, dims([n]), x, dims([n]), "tanh", n)))
     for k in (16, 1024):
         rows = n // k
-        ms = time_launches(timer, stream, lambda: stream.softmax_eltwise(o, dims([rows, k]), x, dims([rows, k])), 20)
-        out[f"softmax! f32 [{rows},{k}]"] = entry(8 * n, ms)
-    b, c, e = 64, 21, 65536
-    ms = time_launches(timer, stream, lambda: stream.softmax_spatial(o, dims([b, c, e]), x, dims([b, c, e])), 20)
-    out[f"softmax! spatial f32 [{b},{c},{e}]"] = entry(8 * b * c * e, ms)
-    ms = time_launches(timer, stream, lambda: stream.rand(o, dims([n]), {"type": "gaussian", "mean": 0.0, "variance": 1.0}), 20)
-    out["rand! gaussian f32 [2^27]"] = entry(4 * n, ms)
-    ms = time_launches(timer, stream, lambda: stream.rand(o, dims([n]), {"type": "flat", "minimum": 0.0, "maximum": 1.0}), 20)
-    out["rand! flat f32 [2^27]"] = entry(4 * n, ms)
-
-    b, c, e = 64, 256, 3136
-    nn_ = b * c * e
-    st = [upload(drv, device, stream, rng.uniform(0.5, 1.5, c).astype(np.float32)) for _ in range(8)]
-    ms = time_launches(timer, stream, lambda: stream.batch_normalize_spatial(o, x, st[0], st[1], st[2], st[3], 1e-3, b, c, e), 20)
-    out[f"batch-normalize! spatial f32 [{b},{c},{e}]"] = entry(8 * nn_, ms)
-    ms = time_launches(timer, stream, lambda: stream.batch_normalize_update_and_apply_spatial(
-        o, x, st[0], st[1], st[4], st[5], 0.9, st[2], st[3], 1e-3, b, c, e), 20)
-    out[f"batch-normalize-update-and-apply! spatial f32 [{b},{c},{e}]"] = entry(8 * nn_, ms, hbm_bytes_moved=12 * nn_)
-    ms = time_launches(timer, stream, lambda: stream.batch_normalize_gradients_spatial(
-        o, st[6], st[7], g, o, x, st[0], st[1], st[2], st[3], 1e-3, b, c, e), 20)
-    out[f"batch-normalize-gradients! spatial f32 [{b},{c},{e}]"] = entry(12 * nn_, ms, hbm_bytes_moved=20 * nn_)
-
-    # pooling: algorithmic bytes = input + output forward; gradient read and written, output gradient
-    # (and, for max, input and output) backward
-    pb, pc, ph = 32, 64, 256
-    po = ph // 2
-    in_dims, out_dims = dims([pb, pc, ph, ph]), dims([pb, pc, po, po])
-    n_out = pb * pc * po * po
-    ig = device.allocate_device_buffer(n, "float")
-    stream.memset(ig, 0, 0.0, n)
-    for kernel, pad, pool_op in ((2, 0, "max"), (3, 1, "max"), (3, 1, "avg")):
-        desc = {"kernel-width": kernel, "kernel-height": kernel, "pad-x": pad, "pad-y": pad, "stride-x": 2,
-                "stride-y": 2, "pool-op": pool_op}
-        label = f"f32 [{pb},{pc},{ph},{ph}] {kernel}x{kernel} stride 2 :{pool_op}"
-        ms = time_launches(timer, stream, lambda: stream.pooling_forward(o, out_dims, 0.0, x, in_dims, desc), 20)
-        out[f"pooling-forward! {label}"] = entry(4 * (n + n_out), ms)
-        ms = time_launches(timer, stream, lambda: stream.pooling_backward(ig, in_dims, 0.0, x, in_dims, o, out_dims, g,
-                                                                         out_dims, desc), 20)
-        out[f"pooling-backward! {label}"] = entry(4 * (2 * n + n_out) + (4 * (n + n_out) if pool_op == "max" else 0), ms)
-
-    # convolution as the CPU backend decomposes it (unroll, gemm!, roll back): priced like gemm!
-    cb, cc, ck, chw = 64, 64, 64, 56
-    conv_desc = {"in-channels": cc, "out-channels": ck, "kernel-width": 3, "kernel-height": 3, "pad-x": 1, "pad-y": 1,
-                 "stride-x": 1, "stride-y": 1}
-    c_in, c_out = dims([cb, cc, chw, chw]), dims([cb, ck, chw, chw])
-    n_cols, n_rows = cc * 9, chw * chw
-    w_ = upload(drv, device, stream, (rng.standard_normal(ck * n_cols, dtype=np.float32) / 24))
-    work = device.allocate_device_buffer(cb * n_rows * n_cols, "float")
-    wgrad = device.allocate_device_buffer(ck * n_cols, "float")
-    w_dims = dims([ck, n_cols])
-    conv_flops = 2.0 * cb * ck * n_rows * n_cols
-    conv_calls = (
-        ("convolution-forward!", lambda: stream.convolution_forward(o, c_out, 0.0, x, c_in, w_, w_dims, work,
-                                                                    cb * n_rows * n_cols, conv_desc, None)),
-        ("convolution-backward-weights!", lambda: stream.convolution_backward_weights(
-            wgrad, w_dims, 0.0, g, c_out, x, c_in, work, cb * n_rows * n_cols, conv_desc, None)),
-        ("convolution-backward-data!", lambda: stream.convolution_backward_data(
-            ig, c_in, 0.0, g, c_out, w_, w_dims, work, cb * n_rows * n_cols, conv_desc, None)),
-    )
-    for name, call in conv_calls:
-        ms = time_launches(timer, stream, call, 5, warm=2)
-        tflops = conv_flops / (ms * 1e-3) / 1e12
-        out[f"{name} f32 [{cb},{cc}->{ck},{chw},{chw}] 3x3 pad 1"] = {
-            "us": round(ms * 1e3, 1), "TFLOP/s": round(tflops, 1), "frac_of_fp32_matrix_peak": round(tflops / 157.3, 4),
-            "workspace_bytes": 4 * cb * n_rows * n_cols, "kernel": capi.last_kernel()}
-
-    # gemm! is the one MFMA-bound method (rocBLAS); priced against the dense fp32 matrix peak
-    m = 8192
-    a_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))
-    b_ = upload(drv, device, stream, rng.standard_normal(m * m, dtype=np.float32))
-    c_ = device.allocate_device_buffer(m * m, "float")
-    # gemv! reads the matrix once: HBM-bound like the rest
-    xv = upload(drv, device, stream, rng.standard_normal(m, dtype=np.float32))
-    yv = device.allocate_device_buffer(m, "float")
+        ops.append(Op(f"a_softmax_{k}", f"softmax! float32 [{rows},{k}]", 8 * n,
+                      lambda rows=rows, k=k: s.softmax_eltwise(o, dims([rows, k]), x, dims([rows, k]))))
+    bq, cq, eq = 64, 21, 65536
+    ops.append(Op("a_softmax_spatial", f"softmax! spatial float32 [{bq},{cq},{eq}]", 8 * bq * cq * eq,
+                  lambda: s.softmax_spatial(o, dims([bq, cq, eq]), x, dims([bq, cq, eq]))))
+    ops.append(Op("a_rand_gaussian", "rand! gaussian float32 [2^27]", 4 * n,
+                  lambda: s.rand(o, dims([n]), {"type": "gaussian", "mean": 0.0, "variance": 1.0})))
+    ops.append(Op("a_rand_flat", "rand! flat float32 [2^27]", 4 * n,
+                  lambda: s.rand(o, dims([n]), {"type": "flat", "minimum": 0.0, "maximum": 1.0})))
+    bb, cc, ee = 64, 256, 3136
+    nn_ = bb * cc * ee
+    st = [b.upload(rng.uniform(0.5, 1.5, cc).astype(np.float32)) for _ in range(8)]
+    ops.append(Op("a_bn_apply", f"batch-normalize! spatial float32 [{bb},{cc},{ee}]", 8 * nn_,
+                  lambda: s.batch_normalize_spatial(o, x, st[0], st[1], st[2], st[3], 1e-3, bb, cc, ee)))
+    ops.append(Op("a_bn_update", f"batch-normalize-update-and-apply! spatial float32 [{bb},{cc},{ee}] (moves 12 B/element)", 8 * nn_,
+                  lambda: s.batch_normalize_update_and_apply_spatial(o, x, st[0], st[1], st[4], st[5], 0.9, st[2], st[3],
+                                                                     1e-3, bb, cc, ee)))
+    ops.append(Op("a_bn_gradients", f"batch-normalize-gradients! spatial float32 [{bb},{cc},{ee}] (moves 20 B/element)", 12 * nn_,
+                  lambda: s.batch_normalize_gradients_spatial(o, st[6], st[7], g, o, x, st[0], st[1], st[2], st[3], 1e-3,
+                                                              bb, cc, ee)))
+    mm = 8192
+    a_ = b.upload(rng.standard_normal(mm * mm, dtype=np.float32))
+    xv = b.upload(rng.standard_normal(mm, dtype=np.float32))
+    yv = b.alloc(mm, "float")
     for trans, label in ((False, "A x"), (True, "A^T x")):
-        ms = time_launches(timer, stream, lambda: stream.gemv(yv, 1, trans, 1.0, a_, m, m, m, xv, 1, 0.0), 20)
-        out[f"gemv! f32 [{m},{m}] {label}"] = entry(4 * m * m, ms)
-    ms = time_launches(timer, stream, lambda: stream.gemm(c_, m, False, False, 1.0, a_, m, m, m, b_, m, m, 0.0), 5, warm=2)
-    tflops = 2.0 * m ** 3 / (ms * 1e-3) / 1e12
-    out[f"gemm! f32 [{m},{m}]x[{m},{m}] (rocBLAS)"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tflops, 1),
-                                                     "frac_of_fp32_matrix_peak": round(tflops / 157.3, 4),
-                                                     "kernel": capi.last_kernel()}
-    return out
+        ops.append(Op(f"a_gemv_{'t' if trans else 'n'}", f"gemv! float32 [{mm},{mm}] {label}", 4 * mm * mm,
+                      lambda trans=trans: s.gemv(yv, 1, trans, 1.0, a_, mm, mm, mm, xv, 1, 0.0)))
+    return ops
 
 
-def cpu_baseline(hosts, n: int) -> dict:
-    """Times the CPU oracle on one full step of the workload."""
+# ----------------------------------------------------------------------------- CPU baseline
+
+def cpu_baseline(data: StepData) -> dict:
+    """Times the CPU oracle on full steps of the same workload (about ten seconds)."""
     from cortex_amd import capi
     from oracle import binding as ob
 
-    shape, tr = [n, n], [1, n]
-    dest = np.zeros(n * n, np.float32)
-    cont = capi.make_dims(shape, [n, 1])
-    view = capi.make_dims(shape, tr)
-    p = lambda a: a.ctypes.data
-    def one_step():
-        ob.call("unary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, capi.UNARY_OPS["exp"], capi.F32, n * n)
-        ob.call("unary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, capi.UNARY_OPS["tanh"], capi.F32, n * n)
-        ob.call("ternary_op", p(dest), C.byref(cont), p(hosts[0]), C.byref(view), 1.0, p(hosts[1]), C.byref(view), 1.0,
-                p(hosts[2]), C.byref(view), 1.0, n * n, 0, capi.F32)
+    p_ = lambda a: a.ctypes.data
+    n = data.adam_n
+    params, grads = data.p.copy(), data.g
+    m = np.zeros(n, np.float32)
+    v = np.full(n, 1e-6, np.float32)
+    pb1, pb2 = pow_betas()
+    r, c, q = 16384, 4096, 4096
+    o32, o64 = np.zeros(r, np.float32), np.zeros(q, np.float64)
+    d0 = np.zeros(1024 * 1024, np.float32)
+    D = lambda shape, strides: C.byref(capi.make_dims(shape, strides))
 
-    one_step()  # first touch of the destination pages
+    def one_step():
+        ob.call("adam_step", capi.F32, 1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 1.0, p_(grads), p_(params), p_(m), p_(v), n)
+        for op in REDUCE_OPS:
+            code = capi.REDUCE_OPS[op]
+            ob.call("unary_reduce", p_(o32), D([r, 1], [1, 1]), 1.0, p_(data.red32), D([r, c], [c, 1]), code, capi.F32)
+            ob.call("unary_reduce", p_(o32), D([c, 1], [1, 1]), 1.0, p_(data.red32), D([c, r], [1, c]), code, capi.F32)
+        for op in REDUCE_OPS:
+            code = capi.REDUCE_OPS[op]
+            ob.call("unary_reduce", p_(o64), D([q, 1], [1, 1]), 1.0, p_(data.red64), D([q, q], [q, 1]), code, capi.F64)
+            ob.call("unary_reduce", p_(o64), D([q, 1], [1, 1]), 1.0, p_(data.red64), D([q, q], [1, q]), code, capi.F64)
+        ob.call("binary_op", p_(d0), D([1024, 1024], [1024, 1]), p_(data.x0), D([1024, 1024], [1024, 1]), 1.0, p_(data.b0),
+                D([1024], [1]), 1.0, 1024 * 1024, capi.BINARY_OPS["+"], capi.F32)
+
+    one_step()  # first touch of the output pages
     steps, t0 = 0, time.perf_counter()
-    while steps < 3 or (time.perf_counter() - t0 < 10.0 and steps < 200):
+    while steps < 2 or (time.perf_counter() - t0 < 10.0 and steps < 100):
         one_step()
         steps += 1
     dt = time.perf_counter() - t0
-    step_bytes = 8 * 4 * n * n
+    step_bytes = 28 * n + 6 * (4 * r * c) + 3 * 4 * (r + c) + 6 * (8 * q * q + 8 * q) + 8392704
     return {"value": round(steps * step_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": ob.num_threads(), "kind": "port",
-            "sample": f"{steps} full steps (exp, tanh, select on transposed float32 [{n},{n}]) in {dt:.2f} s, "
-                      "C++ restatement of the cortex CPU backend with OpenMP"}
+            "sample": f"{steps} full steps (Adam over {n} float32 parameters, the twelve configs[2] reductions, the configs[0] "
+                      f"bias add) in {dt:.2f} s; C++ restatement of the cortex CPU backend, OpenMP over the index space the "
+                      "reference hands to parallel-for"}
 
+
+# ----------------------------------------------------------------------------- rocprofv3 output -> profiles/
+
+def short_kernel_name(n: str) -> str:
+    n = re.sub(r"^void ", "", n.strip('"')).replace("(anonymous namespace)::", "").replace("cthip::", "")
+    depth = 0
+    for i, ch in enumerate(n):
+        if ch == "<":
+            depth += 1
+        elif ch == ">":
+            depth -= 1
+        elif ch == "(" and depth == 0:
+            return n[:i]
+    return n
+
+
+MARKER = re.compile(r"ConstantF<signed char>")
+
+
+def _segments(rows, plan, value_of):
+    """Splits the dispatches (in dispatch order) at the marker launches; returns, per plan segment,
+    {kernel short name: [values]} in first-seen order."""
+    out, cur = [], None
+    for row in rows:
+        name = short_kernel_name(row["Kernel_Name"])
+        if MARKER.search(name):
+            cur = collections.OrderedDict()
+            out.append(cur)
+            continue
+        if cur is not None:
+            cur.setdefault(name, []).append(value_of(row))
+    if len(out) != len(plan):
+        raise SystemExit(f"profile has {len(out)} marked segments, the plan lists {len(plan)}")
+    return out
+
+
+def _read_sorted(path, key):
+    with open(path) as fh:
+        rows = list(csv.DictReader(fh))
+    rows.sort(key=lambda r_: int(r_[key]))
+    return rows
+
+
+def summarize(prof_dir: str, out_dir: str) -> None:
+    """Reads DIR/{trace,fetch,write}/*.csv and DIR/{trace,fetch,write}_plan.json (written by three runs of
+    this program under rocprofv3, see the header of the summary) and writes OUT/bench_trace_and_traffic.txt
+    and OUT/traffic.json."""
+    d, out = Path(prof_dir), Path(out_dir)
+    out.mkdir(parents=True, exist_ok=True)
+    plans = {k: json.loads((d / f"{k}_plan.json").read_text()) for k in ("trace", "fetch", "write")}
+    shas = {p["csrc_sha256"] for p in plans.values()}
+    if len(shas) != 1:
+        raise SystemExit("the three profile runs were made on different sources")
+    trace = _segments(_read_sorted(glob.glob(str(d / "trace" / "*kernel_trace.csv"))[0], "Start_Timestamp"),
+                      plans["trace"]["segments"],
+                      lambda r_: (int(r_["End_Timestamp"]) - int(r_["Start_Timestamp"])) / 1e3)
+    pmc = {}
+    for kind in ("fetch", "write"):
+        pmc[kind] = _segments(_read_sorted(glob.glob(str(d / kind / "*counter_collection.csv"))[0], "Dispatch_Id"),
+                              plans[kind]["segments"], lambda r_: float(r_["Counter_Value"]))
+
+    def seg_index(plan, key):
+        return [i for i, s_ in enumerate(plan["segments"]) if s_["key"] == key]
+
+    cal_f = pmc["fetch"][seg_index(plans["fetch"], "calibration_copy")[0]]
+    cal_w = pmc["write"][seg_index(plans["write"], "calibration_copy")[0]]
+    cal_kib = 8192 * 8192 * 4 / 1024
+    f_raw = float(np.mean(next(iter(cal_f.values()))))
+    w_raw = float(np.mean(next(iter(cal_w.values()))))
+    f_fac, w_fac = cal_kib / f_raw, cal_kib / w_raw
+
+    lines = []
+    traffic = {}
+    for i, seg in enumerate(plans["trace"]["segments"]):
+        key, calls, alg = seg["key"], seg["calls"], seg["algorithmic_bytes"]
+        if key.startswith("_"):
+            continue
+        kernels = trace[i]
+        fi, wi = seg_index(plans["fetch"], key), seg_index(plans["write"], key)
+        fseg = pmc["fetch"][fi[0]] if fi else {}
+        wseg = pmc["write"][wi[0]] if wi else {}
+        fcalls = plans["fetch"]["segments"][fi[0]]["calls"] if fi else 1
+        wcalls = plans["write"]["segments"][wi[0]]["calls"] if wi else 1
+        per_call_us, per_call_bytes = 0.0, 0.0
+        rows = []
+        for name, durs in kernels.items():
+            per = len(durs) / calls
+            fk = float(np.sum(fseg.get(name, [0.0]))) / fcalls
+            wk = float(np.sum(wseg.get(name, [0.0]))) / wcalls
+            per_call_us += float(np.sum(durs)) / calls
+            per_call_bytes += (fk * f_fac + wk * w_fac) * 1024
+            rows.append("      %-78s %6.2f/call %9.2f %9.2f %9.2f %12.1f %12.1f" % (
+                name[:78], per, float(np.mean(durs)), float(np.min(durs)), float(np.max(durs)), fk, wk))
+        if key == "step":
+            lines.append("%s\n    %d steps; kernels of the timed region (avg / min / max us per dispatch; FETCH / WRITE KiB per step):" % (seg["label"], calls))
+            lines.extend(rows)
+            continue
+        rate = alg / per_call_us / 1e3 if per_call_us > 0 else 0.0
+        lines.append("%s\n    key %s: %d calls, kernel time %.2f us per call = %.0f GB/s = %.1f %% of 8 TB/s; HBM traffic %.0f bytes per call "
+                     "= %.4f x the %d algorithmic bytes" % (seg["label"], key, calls, per_call_us, rate, rate / 80,
+                                                            per_call_bytes, per_call_bytes / alg, alg))
+        lines.extend(rows)
+        traffic[key] = {"traffic": int(round(per_call_bytes)), "kernel_us": round(per_call_us, 2),
+                        "kernels": list(kernels.keys()), "algorithmic_bytes": alg}
+
+    sha = shas.pop()
+    head = f"""rocprofv3 summary of bench.py on one MI355X (gfx950): every workload of the step, the other BASELINE configs, the
+access patterns off the fast kernel families and the adjacent TensorMath methods.  Kernel sources sha256 {sha[:16]}.
+
+Commands (from the repository root, one rocprofv3 run each; P = gpurun_out/prof):
+  cd /tmp && export TMPDIR=/tmp && cd <repo>
+  rocprofv3 --kernel-trace --stats --output-format csv -d P/trace -o bench -- python3 bench.py --steps 20 --no-cpu --profile-plan P/trace_plan.json
+  rocprofv3 --pmc FETCH_SIZE --output-format csv -d P/fetch -o bench -- python3 bench.py --steps 3 --warmup 1 --no-cpu --profile-plan P/fetch_plan.json
+  rocprofv3 --pmc WRITE_SIZE --output-format csv -d P/write -o bench -- python3 bench.py --steps 3 --warmup 1 --no-cpu --profile-plan P/write_plan.json
+  python3 bench.py --summarize P --out profiles
+
+With --profile-plan every timed segment of the run starts with a one-byte fill, and the dispatches between two such markers
+belong to one workload: durations and counters are attributed by dispatch order, not by kernel name.
+Per kernel: launches per call, then avg / min / max duration in microseconds (kernel trace), then FETCH_SIZE and WRITE_SIZE
+in KiB per call.  HBM traffic = FETCH x {f_fac:.4f} + WRITE x {w_fac:.4f}: the factors make the calibration copy (exactly
+{cal_kib:.0f} KiB each way) read {cal_kib:.0f}; FETCH_SIZE reported {f_raw:.1f} KiB for it (it counts half the bytes on this part),
+WRITE_SIZE {w_raw:.1f} KiB.  GB/s = algorithmic bytes / summed kernel time of one call; bench.py's own HIP-event figures
+(avg_call_us) also contain the gaps between dispatches.
+
+"""
+    (out / "bench_trace_and_traffic.txt").write_text(head + "\n".join(lines) + "\n")
+    (out / "traffic.json").write_text(json.dumps({
+        "csrc_sha256": sha, "fetch_factor": round(f_fac, 6), "write_factor": round(w_fac, 6),
+        "source": "profiles/bench_trace_and_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the calibration copy)",
+        "ops": traffic}, indent=1) + "\n")
+    print((out / "bench_trace_and_traffic.txt").read_text())
+
+
+# ----------------------------------------------------------------------------- main
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--no-extras", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--sections", default=",".join(SECTIONS), help="comma-separated subset of " + ",".join(SECTIONS))
+    ap.add_argument("--no-extras", action="store_true", help="only the headline step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--size", type=int, default=8192, help="edge of the square tensors (8192 is the benchmark)")
+    ap.add_argument("--adam-n", type=int, default=1 << 28, help="Adam parameter count (2^28 is the benchmark)")
+    ap.add_argument("--profile-plan", default=None, help="write the segment plan here and mark segments (for rocprofv3 runs)")
+    ap.add_argument("--summarize", default=None, help="directory holding trace/ fetch/ write/ rocprofv3 output")
+    ap.add_argument("--out", default=str(ROOT / "profiles"))
     args = ap.parse_args()
+    if args.summarize:
+        summarize(args.summarize, args.out)
+        return 0
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no cross-GPU exchange); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         return 2
+    sections = ["headline"] if args.no_extras else [s_ for s_ in args.sections.split(",") if s_]
 
-    from cortex_amd import capi, driver as drv
+    b = Bench(args.profile_plan)
+    data = StepData(args.adam_n)
+    step_ops, adam, extra = build_step(b, data)
+    step_bytes = sum(op.nbytes for op in step_ops)
 
-    driver = drv.HipDriver()
-    device = driver.default_device()
-    device.make_current()
-    stream = device.create_stream()
-    timer = Timer(capi, stream)
-    n = args.size
-
-    log("generating inputs (numpy default_rng, seeds 1-3) ...")
-    hosts = [np.random.default_rng(seed).standard_normal(n * n).astype(np.float32) for seed in (1, 2, 3)]
-    xs = [upload(drv, device, stream, h) for h in hosts]
-    dest = device.allocate_device_buffer(n * n, "float")
-    cont, view = dims([n, n]), dims([n, n], [1, n])
-    nn = n * n
-
-    sel_events = []
+    adam_events = []
 
     def step(record: bool) -> None:
-        stream.unary_op(dest, cont, xs[0], view, 1.0, "exp", nn)
-        stream.unary_op(dest, cont, xs[0], view, 1.0, "tanh", nn)
-        e0 = timer.mark() if record else None
-        stream.ternary_op(dest, cont, xs[0], view, 1.0, xs[1], view, 1.0, xs[2], view, 1.0, nn, "select")
-        if record:
-            sel_events.append((e0, timer.mark()))
+        for op in step_ops:
+            if record and op is adam:
+                e0 = b.timer.mark()
+                op.fn()
+                adam_events.append((e0, b.timer.mark()))
+            else:
+                op.fn()
 
     for _ in range(args.warmup):
         step(False)
-    stream.sync()
-    dominant_kernel = capi.last_kernel()
+    b.stream.sync()
+    b.segment("step", "the timed region: Adam, twelve reductions, bias add per step", args.steps, step_bytes)
     t_host0 = time.perf_counter()
-    e_start = timer.mark()
+    e_start = b.timer.mark()
     for _ in range(args.steps):
         step(True)
-    e_stop = timer.mark()
-    total_ms = timer.elapsed_ms(e_start, e_stop)
-    stream.sync()
+    e_stop = b.timer.mark()
+    total_ms = b.timer.elapsed_ms(e_start, e_stop)
+    b.stream.sync()
     wall_ms = (time.perf_counter() - t_host0) * 1e3
-    sel_ms = [timer.elapsed_ms(a, b) for a, b in sel_events]
-    for a, b in sel_events:
-        timer.free(a, b)
-    timer.free(e_start, e_stop)
+    adam_ms = float(np.mean([b.timer.elapsed_ms(a_, b_) for a_, b_ in adam_events]))
+    for a_, b_ in adam_events:
+        b.timer.free(a_, b_)
+    b.timer.free(e_start, e_stop)
 
-    step_bytes = 2 * 4 * nn + 2 * 4 * nn + 4 * 4 * nn  # exp + tanh + select
     ms_per_step = total_ms / args.steps
     value = gbs(step_bytes, ms_per_step)
-    sel_avg = float(np.mean(sel_ms))
-    achieved = gbs(4 * 4 * nn, sel_avg)
 
-    traffic = None
-    tfile = ROOT / "profiles" / "traffic.json"
-    if tfile.exists():
-        try:
-            traffic = json.loads(tfile.read_text()).get("ew_tile_kernel_select_f32_8192")
-        except (ValueError, OSError):
-            traffic = None
-
-    # per-op times of the other two kernels of the step
-    ms_exp = time_launches(timer, stream, lambda: stream.unary_op(dest, cont, xs[0], view, 1.0, "exp", nn), 20)
-    ms_tanh = time_launches(timer, stream, lambda: stream.unary_op(dest, cont, xs[0], view, 1.0, "tanh", nn), 20)
-    # a plain contiguous copy of the same size: the reference point for the hardware counters
-    ms_copy = time_launches(timer, stream, lambda: stream.unary_op(dest, cont, xs[0], cont, 1.0, "noop", nn), 20)
+    log("timing every workload of the step on its own ...")
+    ops_out = collections.OrderedDict()
+    for op in step_ops + extra:
+        ops_out[op.label] = b.time_op(op)
+    adam.kernel = ops_out[adam.label]["kernel"]
+    roof = b.block(adam, adam_ms)
+    roof["kernel"] = f"adam_kernel<float, 4, 1, true> ({adam.kernel})"
+    roof["avg_launch_us"] = roof.pop("avg_call_us")
+    roof["algorithmic_bytes_per_launch"] = roof.pop("algorithmic_bytes_per_call")
+    if b.traffic_note:
+        roof["traffic_note"] = b.traffic_note
+    c0 = ops_out[step_ops[-1].label]
+    c0["note"] = ("8 MiB, cache resident: avg_call_us is the GPU timeline per call with launches back to back, host_us the "
+                  "time this program needs to submit one call (Python + ctypes + launch); when the two agree the loop is "
+                  "bound by the host, and kernel_us_rocprof is what the kernel itself takes")
 
     result = {
         "metric": "achieved HBM GB/s (% of MI355X peak) for binary-op!, unary-reduce!, Adam step",
@@ -419,39 +713,35 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "configs[1]: unary-op! :exp, unary-op! :tanh and ternary-op! :select on transposed views "
-                        f"(strides [1,{n}]) of float32 [{n},{n}], inputs N(0,1) seeds 1-3, output contiguous",
+            "workload": f"configs[3] fused Adam step over {args.adam_n} float32 parameters + configs[2] unary-reduce! :sum :max "
+                        ":magnitude-squared over the last axis and over axis 0 (transposed view) of float32 [16384,4096] and of "
+                        "float64 [4096,4096] + configs[0] binary-op! :+ float32 [1024,1024] with a broadcast [1024] row; "
+                        "numpy default_rng seeds 6, 4, 5, 0",
             "algorithmic_bytes_per_step": step_bytes,
             "frac_of_peak": round(value / PEAK_HBM_GBS, 4),
             "host_wall_ms_per_step": round(wall_ms / args.steps, 4),
+            "csrc_sha256": csrc_hash()[:16],
         },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": f"ew_tile_kernel<SelectF<float>> ({dominant_kernel})",
-            "achieved": round(achieved, 1),
-            "peak": PEAK_HBM_GBS,
-            "unit": "GB/s",
-            "frac": round(achieved / PEAK_HBM_GBS, 4),
-            "traffic": traffic,
-            "avg_launch_us": round(sel_avg * 1e3, 2),
-            "algorithmic_bytes_per_launch": 4 * 4 * nn,
-        },
-        "kernels": {
-            "unary-op! :exp (transposed)": {"us": round(ms_exp * 1e3, 2), "GB/s": round(gbs(8 * nn, ms_exp), 1)},
-            "unary-op! :tanh (transposed)": {"us": round(ms_tanh * 1e3, 2), "GB/s": round(gbs(8 * nn, ms_tanh), 1)},
-            "unary-op! :noop (contiguous copy, calibration)": {"us": round(ms_copy * 1e3, 2), "GB/s": round(gbs(8 * nn, ms_copy), 1)},
-            "ternary-op! :select (3 transposed)": {"us": round(sel_avg * 1e3, 2), "GB/s": round(achieved, 1)},
-        },
+        "roofline": roof,
+        "ops": ops_out,
     }
-    if not args.no_extras:
-        log("timing the other BASELINE configs ...")
-        result["others"] = run_extras(drv, device, stream, timer, capi)
-        log("timing the adjacent TensorMath methods ...")
-        result["adjacent"] = run_adjacent(drv, device, stream, timer, capi)
+    builders = {"others": build_others, "patterns": build_patterns, "adjacent": build_adjacent}
+    for name in ("others", "patterns", "adjacent"):
+        if name not in sections:
+            continue
+        log(f"timing section '{name}' ...")
+        sect = collections.OrderedDict()
+        b.segment("_setup_" + name, "fills that prepare the section's buffers", 1, 1)
+        section_ops = builders[name](b)
+        b.keep.append(section_ops)
+        for op in section_ops:
+            sect[op.label] = b.time_op(op)
+        result[name] = sect
+    b.save_plan()
     if not args.no_cpu:
-        log("timing the CPU oracle on one step ...")
-        result["cpu_baseline"] = cpu_baseline(hosts, n)
-    stream.release()
+        log("timing the CPU oracle on the step ...")
+        result["cpu_baseline"] = cpu_baseline(data)
+    b.stream.release()
     print(json.dumps(result))
     return 0
 

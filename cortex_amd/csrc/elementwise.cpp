@@ -42,6 +42,11 @@ void common_vec(const Plan& plan, const EwOperand* ops, VecArgs* a) {
     for (int d = 0; d + 1 < c.nd; ++d) {
       if (d < 2) a->outer_stride01[k][d] = c.stride[k][d + 1];
       else a->outer_stride_hi[k][d - 2] = c.stride[k][d + 1];
+      if (d < 2 && c.any_index && c.index[k][d + 1]) {
+        a->outer_index[k][d] = c.index[k][d + 1];
+        a->indexed = 1;
+        a->nt_mask &= ~(1u << k);
+      }
     }
   }
 }

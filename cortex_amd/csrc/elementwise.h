@@ -80,6 +80,10 @@ struct VecArgs {
   FastDiv outer_fd_hi[CT_MAX_DIMS - 3];
   int64_t outer_stride_hi[kMaxOps][CT_MAX_DIMS - 3];
   uint32_t inner_vecs;
+  // Row gather / scatter: outer_index[k][d] != nullptr makes operand k take its offset along outer
+  // axis d (one of the first two) as index[coordinate] * stride.  Read by the INDEXED kernels only.
+  const int32_t* outer_index[kMaxOps][2];
+  uint32_t indexed;  // some outer_index entry is set
 };
 
 // Kinds of an input operand of the vector kernel.
@@ -137,7 +141,12 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(uint32_t const_mask, uint32_t un
 // KINDS >= 0 fixes the operand kinds at compile time (vec_kinds): the common
 // broadcast patterns then run without the operand-kind branches, which cost
 // about 3 % of a copy's bandwidth.
-template <class F, int VEC, int STREAM, int KINDS = -1>
+//
+// INDEXED: one of the first two outer axes of an operand may go through an
+// index tensor (select rows by label, scatter rows back): the row's coordinate
+// is replaced by index[coordinate] before it meets the stride.  For rows at
+// least a block wide the look-up is one scalar load per wave.
+template <class F, int VEC, int STREAM, int KINDS = -1, bool INDEXED = false>
 __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs a) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
@@ -172,10 +181,23 @@ __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs
     uint32_t q0, r0, q1, r1;
     fd0.divmod(row, q0, r0);
     fd1.divmod(q0, q1, r1);
-    off[0] = (int64_t)r0 * s00 + (int64_t)r1 * s01;
-    off[1] = (int64_t)r0 * s10 + (int64_t)r1 * s11;
-    off[2] = (int64_t)r0 * s20 + (int64_t)r1 * s21;
-    off[3] = (int64_t)r0 * s30 + (int64_t)r1 * s31;
+    if constexpr (INDEXED) {
+#pragma unroll
+      for (int k = 0; k <= NIN; ++k) {
+        const int32_t* i0 = a.outer_index[k][0];
+        const int32_t* i1 = a.outer_index[k][1];
+        const int64_t c0 = i0 ? (int64_t)i0[r0] : (int64_t)r0;
+        const int64_t c1 = i1 ? (int64_t)i1[r1] : (int64_t)r1;
+        off[k] = c0 * a.outer_stride01[k][0] + c1 * a.outer_stride01[k][1];
+      }
+#pragma unroll
+      for (int k = NIN + 1; k < kMaxOps; ++k) off[k] = 0;
+    } else {
+      off[0] = (int64_t)r0 * s00 + (int64_t)r1 * s01;
+      off[1] = (int64_t)r0 * s10 + (int64_t)r1 * s11;
+      off[2] = (int64_t)r0 * s20 + (int64_t)r1 * s21;
+      off[3] = (int64_t)r0 * s30 + (int64_t)r1 * s31;
+    }
     if (n_outer > 2) {
       row = q1;
       for (int d = 2; d < n_outer; ++d) {
@@ -680,7 +702,7 @@ int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use
 // Flat, every tensor operand unit-stride and no constants: the contiguous form.
 inline bool vec_is_flat(const VecArgs& a, int nin) {
   const uint32_t all = (2u << nin) - 1u;
-  return a.n_outer == 0 && a.const_mask == 0 && (a.unit_mask & all) == all;
+  return a.n_outer == 0 && a.const_mask == 0 && (a.unit_mask & all) == all && !a.indexed;
 }
 
 template <class F, int VEC>
@@ -696,6 +718,13 @@ inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& args) {
     if (a.streaming == 2) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 2>), grid, dim3(kBlock), 0, s, f, fa);
     else if (a.streaming) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 1>), grid, dim3(kBlock), 0, s, f, fa);
     else hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 0>), grid, dim3(kBlock), 0, s, f, fa);
+    return;
+  }
+  if (a.indexed) {
+    // gathered rows are re-read wherever labels repeat and scattered rows are not written in
+    // order: plain accesses, plain block order
+    a.grouped_blocks = 0;
+    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 0, -1, true>), grid, dim3(kBlock), 0, s, f, a);
     return;
   }
   if (VEC > 1 && a.streaming) {

@@ -22,12 +22,26 @@
 // way); float/double results are sums formed in double, closer to the exact sum
 // than the reference's value-by-value accumulation (which the reference itself
 // only checks to 1e-4, src/cortex/verify/tensor.clj:188-191).
-// Indirectly indexed destinations fall back to the serial kernel.
+//
+// Indirectly indexed destinations (scatter-add of rows through a label tensor,
+// src/cortex/loss/center.clj:92; src/cortex/verify/tensor.clj:1162-1174): two
+// updates collide exactly when their coordinates along the indexed axis name
+// the same index value and all other coordinates agree.  The positions of the
+// index tensor are sorted by value, stably, so the positions of one value are
+// adjacent and still in increasing order; then one lane per (value, element of
+// the remaining axes) applies that destination element's updates in increasing
+// position, which is increasing e: accum_grouped_kernel.  Bit-identical to the
+// serial loop for every op.  Up to 8192 index entries are ranked by one small
+// kernel; longer index tensors go through the vendor radix sort (hipCUB, a
+// stable LSD sort).  Shapes outside that pattern (reduced axes next to an
+// indexed one, an indexed y) keep the serial kernel.
 #include <algorithm>
 
 #include "elementwise.h"
 #include "functors.h"
 #include "ops.h"
+
+#include <hipcub/device/device_radix_sort.hpp>
 
 using namespace cthip;
 
@@ -44,13 +58,26 @@ struct OwnerArgs {
   FastDiv rsize[CT_MAX_DIMS];   // reduced axes, fastest first
   int64_t ry_stride[CT_MAX_DIMS];
   int32_t reverse;
+  // STAGED form: `reduced` holds, per destination element, the reduction of its updates
+  // (unary-reduce! :max / :min of y * y_alpha), addressed through kt_stride per kept axis
+  const void* reduced;
+  int64_t kt_stride[CT_MAX_DIMS];
 };
 
-template <class T, int OP>
-__global__ void __launch_bounds__(kBlock) accum_owner_kernel(const BinaryF<T, OP> f, const OwnerArgs a) {
+// STAGED (:max and :min with dest_alpha 1): the updates of every destination element have
+// already been reduced, with java.lang.Math.max / min, into a.reduced.  Where that value is
+// an ordinary non-zero number it is also what the serial chain of (x > y ? x : y) steps leaves
+// (equal non-zero values are the same bits, so which of them a tie keeps does not show), and
+// one step with it finishes the element; f_unit is f with the update's multiplier set to 1,
+// since the reduction has applied it.  Where it is a NaN or a zero the chain's outcome depends
+// on the order of the updates (a NaN restarts or freezes it, and +0 against -0 is a tie that
+// the later or the earlier operand wins), and the lane walks the updates as the serial loop does.
+template <class T, int OP, bool STAGED>
+__global__ void __launch_bounds__(kBlock) accum_owner_kernel(const BinaryF<T, OP> f, const BinaryF<T, OP> f_unit,
+                                                             const OwnerArgs a) {
   const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (t >= a.n_dest) return;
-  int64_t doff = 0, ybase = 0;
+  int64_t doff = 0, ybase = 0, toff = 0;
   uint32_t rem = (uint32_t)t;
   for (int d = 0; d < a.n_kept; ++d) {
     uint32_t q, r;
@@ -58,10 +85,20 @@ __global__ void __launch_bounds__(kBlock) accum_owner_kernel(const BinaryF<T, OP
     rem = q;
     doff += (int64_t)r * a.kd_stride[d];
     ybase += (int64_t)r * a.ky_stride[d];
+    if constexpr (STAGED) toff += (int64_t)r * a.kt_stride[d];
   }
   T* dp = reinterpret_cast<T*>(a.dest) + doff;
   const T* yp = reinterpret_cast<const T*>(a.y) + ybase;
   T acc = *dp;
+  if constexpr (STAGED) {
+    const T red = reinterpret_cast<const T*>(a.reduced)[toff];
+    bool ordinary = true;
+    if constexpr (std::is_floating_point<T>::value) ordinary = red == red && red != (T)0;
+    if (ordinary) {
+      *dp = a.reverse ? f_unit(red, acc, acc) : f_unit(acc, red, red);
+      return;
+    }
+  }
   uint32_t i = 0;
   if (a.n_redax == 1) {
     // one broadcast axis: fetch eight updates ahead, apply them in order
@@ -144,29 +181,256 @@ bool owner_structure(const ct_dims& dd, const ct_dims& yd, int64_t n, OwnerArgs*
   return true;
 }
 
+// ------------------------------------------------------------------ indexed destinations
+
+struct GroupedArgs {
+  void* dest;
+  const void* y;
+  const int32_t* skey;   // index values, sorted
+  const int32_t* perm;   // the position each sorted entry came from
+  uint32_t n_index;      // entries of the index tensor
+  uint32_t kept_vecs;    // vectors of the remaining axes per index entry
+  FastDiv kept_fd;       // kept_vecs
+  int64_t d_gstride, y_gstride;  // strides of the indexed axis
+  int32_t n_kept;
+  FastDiv ksize[CT_MAX_DIMS];    // remaining axes, fastest first (axis 0 counted in vectors)
+  int64_t kd_stride[CT_MAX_DIMS], ky_stride[CT_MAX_DIMS];
+  int32_t reverse;
+};
+
+// rank[i] = number of entries that sort before entry i (smaller value, or equal value and
+// smaller position): a stable counting rank, quadratic but one launch.  Entry i is then
+// stored at its rank.  A block ranks 64 entries: lane l of every wave owns entry l of the
+// block, the block's four waves each count over a quarter of every tile of the index tensor
+// (read from LDS four values at a time; the reads are wave-uniform), and the four counts meet
+// in LDS.
+constexpr int kRankTile = 4096;  // entries staged in LDS at a time; a multiple of 16
+constexpr uint32_t kRankMaxEntries = 8192;
+__global__ void __launch_bounds__(kBlock) index_rank_kernel(const int32_t* index, uint32_t n, int32_t* skey, int32_t* perm) {
+  __shared__ __align__(16) int32_t tile[kRankTile];
+  __shared__ uint32_t part[3][64];
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+  const uint32_t i = blockIdx.x * 64u + lane;
+  const int32_t mine = i < n ? index[i] : 0;
+  uint32_t rank = 0;
+  for (uint32_t base = 0; base < n; base += kRankTile) {
+    const uint32_t len = n - base < (uint32_t)kRankTile ? n - base : (uint32_t)kRankTile;
+    __syncthreads();
+    for (uint32_t j = threadIdx.x; j < (uint32_t)kRankTile; j += kBlock) tile[j] = j < len ? index[base + j] : INT32_MAX;
+    __syncthreads();
+    // this wave's quarter of the tile, in groups of four; padding entries (INT32_MAX at positions
+    // >= n) never count: they are neither smaller nor, at a larger position, equal-and-earlier
+    const uint32_t q0 = wave * (kRankTile / 4), q1 = q0 + kRankTile / 4;
+    if (q0 < len) {
+#pragma unroll 4
+      for (uint32_t j = q0; j < q1; j += 4) {
+        const int4 o = *reinterpret_cast<const int4*>(&tile[j]);
+        const uint32_t pos = base + j;
+        rank += (o.x < mine || (o.x == mine && pos < i)) ? 1u : 0u;
+        rank += (o.y < mine || (o.y == mine && pos + 1 < i)) ? 1u : 0u;
+        rank += (o.z < mine || (o.z == mine && pos + 2 < i)) ? 1u : 0u;
+        rank += (o.w < mine || (o.w == mine && pos + 3 < i)) ? 1u : 0u;
+      }
+    }
+  }
+  if (wave > 0) part[wave - 1][lane] = rank;
+  __syncthreads();
+  if (wave == 0 && i < n) {
+    rank += part[0][lane] + part[1][lane] + part[2][lane];
+    skey[rank] = mine;
+    perm[rank] = (int32_t)i;
+  }
+}
+
+__global__ void __launch_bounds__(kBlock) iota_kernel(int32_t* out, uint32_t n) {
+  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) out[i] = (int32_t)i;
+}
+
+// One lane per (sorted index entry, vector of the remaining axes).  A lane whose entry is
+// not the first of its value leaves at once; the first walks the run of equal values,
+// fetching kAhead updates before it applies them in order.
+template <class T, int OP, int VEC>
+__global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, OP> f, const GroupedArgs a) {
+  using V = Vec<T, VEC>;
+  const uint64_t t = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (t >= (uint64_t)a.n_index * a.kept_vecs) return;
+  uint32_t i, kv;
+  if (a.kept_vecs >= 1u << 31 || t >= (uint64_t(1) << 32)) {
+    i = (uint32_t)(t / a.kept_vecs);
+    kv = (uint32_t)(t % a.kept_vecs);
+  } else {
+    a.kept_fd.divmod((uint32_t)t, i, kv);
+  }
+  const int32_t key = a.skey[i];
+  if (i > 0 && a.skey[i - 1] == key) return;
+  int64_t doff = (int64_t)key * a.d_gstride, yoff = 0;
+  uint32_t rem = kv;
+  for (int d = 0; d < a.n_kept; ++d) {
+    uint32_t q, r;
+    a.ksize[d].divmod(rem, q, r);
+    rem = q;
+    const int64_t c = d == 0 ? (int64_t)r * VEC : (int64_t)r;
+    doff += c * a.kd_stride[d];
+    yoff += c * a.ky_stride[d];
+  }
+  V* dp = reinterpret_cast<V*>(reinterpret_cast<T*>(a.dest) + doff);
+  const T* yb = reinterpret_cast<const T*>(a.y) + yoff;
+  const bool y_unit = a.ky_stride[0] == 1 || VEC == 1;
+  V acc = *dp;
+  constexpr int kAhead = 4;
+  uint32_t j = i;
+  for (;;) {
+    V upd[kAhead];
+    int cnt = 0;
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      if (cnt == u && j + u < a.n_index && a.skey[j + u] == key) {
+        const T* yp = yb + (int64_t)a.perm[j + u] * a.y_gstride;
+        if (y_unit) {
+          upd[u] = *reinterpret_cast<const V*>(yp);
+        } else {  // y broadcast along the vectorised axis
+          const T yv = *yp;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) upd[u].v[e] = yv;
+        }
+        cnt = u + 1;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      if (u < cnt) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          acc.v[e] = a.reverse ? f(upd[u].v[e], acc.v[e], acc.v[e]) : f(acc.v[e], upd[u].v[e], upd[u].v[e]);
+      }
+    }
+    if (cnt < kAhead) break;
+    j += kAhead;
+  }
+  *dp = acc;
+}
+
+// Recognises "one indexed axis in the destination, every other axis kept, y direct".
+// Fills everything of GroupedArgs except the sorted index and the pointers; *index_out is the
+// destination's index tensor, *vec_ok whether axis 0 may be walked in 16-byte vectors.
+template <class T>
+bool grouped_structure(const ct_dims& dd, const ct_dims& yd, const void* dest, const void* y, int64_t n, GroupedArgs* a,
+                       const int32_t** index_out, bool* vec_ok) {
+  if (!dims_direct(yd)) return false;
+  const int rank = std::max(dd.ndim, yd.ndim);
+  int gi = -1;
+  struct Ax { int64_t size, ds, ys; } kept[CT_MAX_DIMS];
+  int nk = 0;
+  int64_t total = 1;
+  for (int i = rank - 1; i >= 0; --i) {  // fastest first
+    const int di = i - (rank - dd.ndim), yi = i - (rank - yd.ndim);
+    const int64_t dshape = di >= 0 ? dd.shape[di] : 1, dstr = di >= 0 ? dd.strides[di] : 0;
+    const int64_t yshape = yi >= 0 ? yd.shape[yi] : 1, ystr = yi >= 0 ? yd.strides[yi] : 0;
+    const int32_t* idx = di >= 0 ? dd.index[di] : nullptr;
+    const int64_t mx = std::max(dshape, yshape);
+    if (mx >= (int64_t(1) << 31)) return false;
+    total *= mx;
+    if (idx) {
+      if (gi >= 0 || dshape != mx || (yshape != 1 && yshape != mx)) return false;
+      gi = i;
+      a->n_index = (uint32_t)dshape;
+      a->d_gstride = dstr;
+      a->y_gstride = yshape == 1 ? 0 : ystr;
+      *index_out = idx;
+      continue;
+    }
+    if (mx == 1) continue;
+    if (dshape != mx || dstr <= 0 || (yshape != 1 && yshape != mx)) return false;
+    kept[nk++] = Ax{mx, dstr, yshape == 1 ? 0 : ystr};
+  }
+  if (gi < 0 || total != n) return false;
+  // kept axes must not overlap one another in the destination
+  {
+    int order[CT_MAX_DIMS];
+    for (int i = 0; i < nk; ++i) order[i] = i;
+    std::sort(order, order + nk, [&](int l, int r) { return kept[l].ds < kept[r].ds; });
+    int64_t span = 1;
+    for (int i = 0; i < nk; ++i) {
+      if (kept[order[i]].ds < span) return false;
+      span = kept[order[i]].ds * (kept[order[i]].size - 1) + span;
+    }
+  }
+  if (nk == 0) kept[nk++] = Ax{1, 1, 1};
+  constexpr int VMAX = 16 / (int)sizeof(T);
+  bool v = VMAX > 1 && kept[0].ds == 1 && (kept[0].ys == 1 || kept[0].ys == 0) && kept[0].size % VMAX == 0 &&
+           a->d_gstride % VMAX == 0 && a->y_gstride % VMAX == 0 && ((uintptr_t)dest % 16) == 0 && ((uintptr_t)y % 16) == 0;
+  for (int i = 1; v && i < nk; ++i) v = kept[i].ds % VMAX == 0 && kept[i].ys % VMAX == 0;
+  *vec_ok = v;
+  const int vec = v ? VMAX : 1;
+  int64_t kv = 1;
+  a->n_kept = nk;
+  for (int i = 0; i < nk; ++i) {
+    const int64_t sz = i == 0 ? kept[i].size / vec : kept[i].size;
+    a->ksize[i] = FastDiv((uint32_t)sz);
+    a->kd_stride[i] = kept[i].ds;
+    a->ky_stride[i] = kept[i].ys;
+    kv *= sz;
+  }
+  if (kv >= (int64_t(1) << 31)) return false;
+  a->kept_vecs = (uint32_t)kv;
+  a->kept_fd = FastDiv((uint32_t)kv);
+  return ((int64_t)a->n_index * kv + kBlock - 1) / kBlock < (int64_t(1) << 31);
+}
+
+// Sorts the index tensor's positions by value (stable) into the stream's scratch.
+int sort_index(hipStream_t s, const int32_t* index, uint32_t n, const int32_t** skey, const int32_t** perm) {
+  void* block = nullptr;
+  if (n <= kRankMaxEntries) {
+    if (int rc = stream_scratch(s, (size_t)n * 8, &block, kScratchAccumA)) return rc;
+    int32_t* k = static_cast<int32_t*>(block);
+    hipLaunchKernelGGL(index_rank_kernel, dim3((n + 63) / 64), dim3(kBlock), 0, s, index, n, k, k + n);
+    *skey = k;
+    *perm = k + n;
+    return CT_OK;
+  }
+  size_t temp_bytes = 0;
+  const size_t arrays = ((size_t)n * 4 + 255) / 256 * 256;
+  CT_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, index, (int32_t*)nullptr, (const int32_t*)nullptr,
+                                            (int32_t*)nullptr, (int)n, 0, 32, s));
+  if (int rc = stream_scratch(s, 3 * arrays + temp_bytes, &block, kScratchAccumA)) return rc;
+  char* base = static_cast<char*>(block);
+  int32_t* k = reinterpret_cast<int32_t*>(base);
+  int32_t* p = reinterpret_cast<int32_t*>(base + arrays);
+  int32_t* iota = reinterpret_cast<int32_t*>(base + 2 * arrays);
+  hipLaunchKernelGGL(iota_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, s, iota, n);
+  CT_HIP(hipcub::DeviceRadixSort::SortPairs(base + 3 * arrays, temp_bytes, index, k, (const int32_t*)iota, p, (int)n, 0, 32, s));
+  *skey = k;
+  *perm = p;
+  return CT_OK;
+}
+
 struct StageAxis {
   int64_t size, ystride, dstride;
   bool kept;
+  int id;  // kept axes: position in OwnerArgs::ksize
 };
 
 constexpr int64_t kStagedMinUpdates = 64;     // per destination element
 constexpr int64_t kStagedMinElements = 16384;  // of y
 
-// dest += sum over the broadcast axes of y*y_alpha, as staged unary-reduce!
-// passes plus one in-place binary-op!.  Sets *handled to false (and does
-// nothing) when y is itself broadcast along some axis.
-int accum_sum_staged(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, size_t elem_bytes, bool* handled) {
+// Reduces y * y_alpha over the broadcast axes with unary-reduce! `rop`, innermost group of
+// axes first, through the stream's two accumulate scratch blocks.  On success *result is the
+// last temporary (one value per destination element) and ax[0..*nax) the kept axes, slowest
+// first, with .ystride the temporary's stride.  *handled is false (and nothing ran) when y
+// is itself broadcast along some axis.
+int stage_reduce(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, size_t elem_bytes, int rop,
+                 bool* handled, const void** result, StageAxis* ax, int* nax_out) {
   *handled = false;
-  StageAxis ax[CT_MAX_DIMS];
   int nax = 0;
   for (int d = 0; d < a.n_kept; ++d) {
     if (a.ky_stride[d] <= 0) return CT_OK;
-    ax[nax++] = StageAxis{(int64_t)a.ksize[d].d, a.ky_stride[d], a.kd_stride[d], true};
+    ax[nax++] = StageAxis{(int64_t)a.ksize[d].d, a.ky_stride[d], a.kd_stride[d], true, d};
   }
   for (int d = 0; d < a.n_redax; ++d) {
     if (a.rsize[d].d == 1) continue;
     if (a.ry_stride[d] <= 0) return CT_OK;
-    ax[nax++] = StageAxis{(int64_t)a.rsize[d].d, a.ry_stride[d], 0, false};
+    ax[nax++] = StageAxis{(int64_t)a.rsize[d].d, a.ry_stride[d], 0, false, -1};
   }
   if (nax > CT_MAX_DIMS) return CT_OK;
   std::sort(ax, ax + nax, [](const StageAxis& l, const StageAxis& r) { return l.ystride > r.ystride; });  // slowest first
@@ -215,14 +479,26 @@ int accum_sum_staged(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtyp
     od.strides[nrest] = 1;
     void* tmp = nullptr;
     if (int rc = stream_scratch(s, (size_t)n_out * elem_bytes, &tmp, slot)) return rc;
-    if (int rc = ct_unary_reduce((void*)s, tmp, &od, alpha, cur, &id, CT_ROP_SUM, dtype)) return rc;
+    if (int rc = ct_unary_reduce((void*)s, tmp, &od, alpha, cur, &id, rop, dtype)) return rc;
     cur = tmp;
     alpha = 1.0;
     slot = slot == kScratchAccumA ? kScratchAccumB : kScratchAccumA;
     nax = nrest;
     for (int i = 0; i < nrest; ++i) ax[i] = rest[i];
   }
+  *result = cur;
+  *nax_out = nax;
+  return CT_OK;
+}
 
+// dest += sum over the broadcast axes of y*y_alpha, as staged unary-reduce! :sum passes plus
+// one in-place binary-op!.
+int accum_sum_staged(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, size_t elem_bytes, bool* handled) {
+  StageAxis ax[CT_MAX_DIMS];
+  int nax = 0;
+  const void* cur = nullptr;
+  if (int rc = stage_reduce(s, a, y_alpha, dtype, elem_bytes, CT_ROP_SUM, handled, &cur, ax, &nax)) return rc;
+  if (!*handled) return CT_OK;
   ct_dims dd, td;
   std::memset(&dd, 0, sizeof(dd));
   std::memset(&td, 0, sizeof(td));
@@ -265,9 +541,50 @@ int accum_run(hipStream_t s, void* dest, const ct_dims* dd, double dest_alpha, c
         if (handled) return CT_OK;
       }
     }
+    if constexpr (OP == CT_BOP_MAX || OP == CT_BOP_MIN) {
+      // max / min of the updates first, at the reduce kernels' rate, then one step per destination
+      // element.  Floats: rounding to T is monotonic, so it commutes with max / min for any y_alpha.
+      // Integers: the chain narrows to T after every step, which commutes only when nothing is
+      // multiplied (y_alpha 1).
+      const bool alpha_ok = std::is_floating_point<T>::value || jvm_cast<T>(y_alpha) == (T)1;
+      if (jvm_cast<T>(dest_alpha) == (T)1 && alpha_ok && a.n_red >= kStagedMinUpdates && n >= kStagedMinElements) {
+        StageAxis ax[CT_MAX_DIMS];
+        int nax = 0;
+        bool handled = false;
+        const void* reduced = nullptr;
+        const int rop = OP == CT_BOP_MAX ? CT_ROP_MAX : CT_ROP_MIN;
+        if (int rc = stage_reduce(s, a, y_alpha, dtype, sizeof(T), rop, &handled, &reduced, ax, &nax)) return rc;
+        if (handled) {
+          a.reduced = reduced;
+          for (int i = 0; i < nax; ++i) a.kt_stride[ax[i].id] = ax[i].ystride;
+          BinaryF<T, OP> f_unit = f;
+          if (reverse) f_unit.xa = (A)1; else f_unit.ya = (A)1;
+          note_kernel("accum_staged_extreme");
+          hipLaunchKernelGGL((accum_owner_kernel<T, OP, true>), dim3((uint32_t)((a.n_dest + kBlock - 1) / kBlock)),
+                             dim3(kBlock), 0, s, f, f_unit, a);
+          return after_launch(s);
+        }
+      }
+    }
     note_kernel("accum_owner");
-    hipLaunchKernelGGL((accum_owner_kernel<T, OP>), dim3((uint32_t)((a.n_dest + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       s, f, a);
+    hipLaunchKernelGGL((accum_owner_kernel<T, OP, false>), dim3((uint32_t)((a.n_dest + kBlock - 1) / kBlock)), dim3(kBlock),
+                       0, s, f, f, a);
+    return after_launch(s);
+  }
+  GroupedArgs g;
+  std::memset(&g, 0, sizeof(g));
+  const int32_t* index = nullptr;
+  bool vec_ok = false;
+  if (grouped_structure<T>(*dd, *yd, dest, y, n, &g, &index, &vec_ok)) {
+    if (int rc = sort_index(s, index, g.n_index, &g.skey, &g.perm)) return rc;
+    g.dest = dest;
+    g.y = y;
+    g.reverse = reverse ? 1 : 0;
+    const dim3 grid((uint32_t)(((int64_t)g.n_index * g.kept_vecs + kBlock - 1) / kBlock));
+    constexpr int VMAX = 16 / (int)sizeof(T);
+    note_kernel(vec_ok ? "accum_grouped_vec" : "accum_grouped");
+    if (vec_ok) hipLaunchKernelGGL((accum_grouped_kernel<T, OP, VMAX>), grid, dim3(kBlock), 0, s, f, g);
+    else hipLaunchKernelGGL((accum_grouped_kernel<T, OP, 1>), grid, dim3(kBlock), 0, s, f, g);
     return after_launch(s);
   }
   EwOperand ops[3] = {{dest, dd, (int)sizeof(T), 0},

@@ -14,6 +14,19 @@
 // every access is a 128-bit coalesced load or store when the four buffers are
 // 16-byte aligned; m and v may sit at an arbitrary element offset of the flat
 // optimizer state, in which case narrower vectors are used.
+//
+// Launch shape.  Four read streams and three write streams over the same four
+// buffers are bound by how well the memory controllers can batch the mix, not
+// by the kernel: with no arithmetic at all the same accesses run at the same
+// rate.  Measured at 2^28 floats per buffer (percent of the 8 TB/s peak): one
+// read stream 94, one write stream 84, copy 84, 2 reads + 1 write 83.5, 3 + 1
+// 82, 4 + 1 80, 4 + 2 80, 4 + 3 78 (in place or into separate buffers alike),
+// 4 + 4 76.  Within that, blocks of one wave in plain block order measured
+// best: 79.0 against 77.3 for 256-lane blocks dealt to the dies in groups
+// (256-lane blocks in plain order 77.4, 128-lane 76; two vectors per lane
+// 74-76; a persistent grid-stride loop with prefetch 58-66; die groups of 16 /
+// 32 / 64 blocks 63 / 67 / 69).  The non-temporal bit on loads and on stores
+// is worth 9 points each (70 and 71.5 without); the scope bits change nothing.
 #include "elementwise.h"
 
 using namespace cthip;
@@ -24,11 +37,14 @@ struct AdamScalars {
   double alpha, beta1, beta2, eps, one_minus_beta1, one_minus_beta2, one_minus_pb1, one_minus_pb2, ga;
 };
 
+constexpr int kOptBlock = 64;  // one wave per block
+
 template <class T, int VEC, int UNROLL, bool streaming>
-__global__ void __launch_bounds__(kBlock) adam_kernel(const AdamScalars s, const T* g, T* p, T* m, T* v,
-                                                      int64_t n_vecs, uint32_t grouped_blocks) {
+__global__ void __launch_bounds__(kOptBlock) adam_kernel(const AdamScalars s, const T* g, T* p, T* m, T* v,
+                                                         int64_t n_vecs) {
   using V = Vec<T, VEC>;
-  const int64_t first = (int64_t)xcd_grouped_unit(blockIdx.x, grouped_blocks) * (kBlock * UNROLL) + threadIdx.x;
+  constexpr int kBlock = kOptBlock;
+  const int64_t first = (int64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x;
   V gv[UNROLL], pv[UNROLL], mv[UNROLL], vv[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
@@ -69,10 +85,11 @@ __global__ void __launch_bounds__(kBlock) adam_kernel(const AdamScalars s, const
 template <class T> struct AdadeltaScalars { T ga; double decay, eps, one_minus_decay; };
 
 template <class T, int VEC, int UNROLL, bool streaming>
-__global__ void __launch_bounds__(kBlock) adadelta_kernel(const AdadeltaScalars<T> s, const T* g, T* p, T* gacc,
-                                                          T* dacc, int64_t n_vecs, uint32_t grouped_blocks) {
+__global__ void __launch_bounds__(kOptBlock) adadelta_kernel(const AdadeltaScalars<T> s, const T* g, T* p, T* gacc,
+                                                             T* dacc, int64_t n_vecs) {
   using V = Vec<T, VEC>;
-  const int64_t first = (int64_t)xcd_grouped_unit(blockIdx.x, grouped_blocks) * (kBlock * UNROLL) + threadIdx.x;
+  constexpr int kBlock = kOptBlock;
+  const int64_t first = (int64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x;
   V gv[UNROLL], pv[UNROLL], av[UNROLL], dv[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
@@ -121,25 +138,22 @@ template <class T> int common_vec_width(const void* a, const void* b, const void
   return vec;
 }
 
-// One vector per lane per buffer and non-temporal accesses measured fastest for
-// this 4-read / 3-write stream mix (about 76 % of peak against 67 % with plain
-// stores or two vectors per lane).
-constexpr int kUnroll = 1;
+constexpr int kUnroll = 1;  // one vector per lane per buffer
 
 template <class T, int VEC>
 void adam_launch(hipStream_t st, const AdamScalars& s, const T* g, T* p, T* m, T* v, int64_t n) {
   const bool streaming = n * 7 * (int64_t)sizeof(T) >= (int64_t(64) << 20);
   const int64_t n_vecs = n / VEC;
   if (n_vecs > 0) {
-    const int64_t per = (int64_t)kBlock * kUnroll;
+    const int64_t per = (int64_t)kOptBlock * kUnroll;
     const dim3 grid((uint32_t)((n_vecs + per - 1) / per));
-    if (streaming) hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, true>), grid, dim3(kBlock), 0, st, s, g, p, m, v, n_vecs, xcd_grouped_blocks(grid.x));
-    else hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, false>), grid, dim3(kBlock), 0, st, s, g, p, m, v, n_vecs, xcd_grouped_blocks(grid.x));
+    if (streaming) hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, true>), grid, dim3(kOptBlock), 0, st, s, g, p, m, v, n_vecs);
+    else hipLaunchKernelGGL((adam_kernel<T, VEC, kUnroll, false>), grid, dim3(kOptBlock), 0, st, s, g, p, m, v, n_vecs);
   }
   const int64_t done = n_vecs * VEC;
   if (VEC > 1 && done < n)
-    hipLaunchKernelGGL((adam_kernel<T, 1, 1, false>), dim3(1), dim3(kBlock), 0, st, s, g + done, p + done, m + done,
-                       v + done, n - done, 0u);
+    hipLaunchKernelGGL((adam_kernel<T, 1, 1, false>), dim3(1), dim3(kOptBlock), 0, st, s, g + done, p + done, m + done,
+                       v + done, n - done);
 }
 
 template <class T>
@@ -171,15 +185,15 @@ void adadelta_launch(hipStream_t st, const AdadeltaScalars<T>& s, const T* g, T*
   const bool streaming = n * 7 * (int64_t)sizeof(T) >= (int64_t(64) << 20);
   const int64_t n_vecs = n / VEC;
   if (n_vecs > 0) {
-    const int64_t per = (int64_t)kBlock * kUnroll;
+    const int64_t per = (int64_t)kOptBlock * kUnroll;
     const dim3 grid((uint32_t)((n_vecs + per - 1) / per));
-    if (streaming) hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, true>), grid, dim3(kBlock), 0, st, s, g, p, a, d, n_vecs, xcd_grouped_blocks(grid.x));
-    else hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, false>), grid, dim3(kBlock), 0, st, s, g, p, a, d, n_vecs, xcd_grouped_blocks(grid.x));
+    if (streaming) hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, true>), grid, dim3(kOptBlock), 0, st, s, g, p, a, d, n_vecs);
+    else hipLaunchKernelGGL((adadelta_kernel<T, VEC, kUnroll, false>), grid, dim3(kOptBlock), 0, st, s, g, p, a, d, n_vecs);
   }
   const int64_t done = n_vecs * VEC;
   if (VEC > 1 && done < n)
-    hipLaunchKernelGGL((adadelta_kernel<T, 1, 1, false>), dim3(1), dim3(kBlock), 0, st, s, g + done, p + done, a + done,
-                       d + done, n - done, 0u);
+    hipLaunchKernelGGL((adadelta_kernel<T, 1, 1, false>), dim3(1), dim3(kOptBlock), 0, st, s, g + done, p + done, a + done,
+                       d + done, n - done);
 }
 
 template <class T>

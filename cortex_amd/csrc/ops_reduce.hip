@@ -406,32 +406,59 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
   }
 }
 
-// LPO lanes share one output's partials (64 when there are many segments).
+// Combines the partial accumulators of a split reduction.  The launch is small
+// (a few KiB to a MiB of partials) and sits on the critical path between two
+// calls, so it is shaped for latency: LPO lanes share one output, every lane
+// issues all of its loads (at most kFinishLoads) before the first combine when
+// the segments allow, and the lanes of an output combine with shuffles.  The
+// lanes of a wave are laid out output-fastest (lane = seg_lane * (64 / LPO) +
+// output), so one load instruction reads runs of consecutive partials.
+constexpr int kFinishLoads = 4;
+
 template <class P, int LPO>
 __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs a) {
   using T = typename P::Elem;
   using A = typename P::Acc;
-  const int lane = threadIdx.x % LPO;
-  const int64_t p = (int64_t)blockIdx.x * (kBlock / LPO) + threadIdx.x / LPO;
+  constexpr int PPW = 64 / LPO;  // outputs per wave
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sl = lane / PPW, pl = lane % PPW;
+  const int64_t p = ((int64_t)blockIdx.x * (kBlock / 64) + wave) * PPW + pl;
   const bool live = p < a.n_out;
   const A* part = reinterpret_cast<const A*>(a.partials);
   A acc = P::identity();
-  if (live)
-#pragma unroll 8
-    for (uint32_t s = lane; s < a.n_seg; s += LPO) acc = P::combine(acc, part[(int64_t)s * a.n_out + p]);
+  if (live) {
+    if (a.n_seg <= (uint32_t)(kFinishLoads * LPO)) {
+      A x[kFinishLoads];
 #pragma unroll
-  for (int m = LPO / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
-  if (live && lane == 0) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+      for (int j = 0; j < kFinishLoads; ++j) {
+        const uint32_t s = (uint32_t)(sl + j * LPO);
+        if (s < a.n_seg) x[j] = part[(int64_t)s * a.n_out + p];
+      }
+#pragma unroll
+      for (int j = 0; j < kFinishLoads; ++j)
+        if ((uint32_t)(sl + j * LPO) < a.n_seg) acc = P::combine(acc, x[j]);
+    } else {
+#pragma unroll 8
+      for (uint32_t s = sl; s < a.n_seg; s += LPO) acc = P::combine(acc, part[(int64_t)s * a.n_out + p]);
+    }
+  }
+#pragma unroll
+  for (int m = 32; m >= PPW; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
+  if (live && sl == 0) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
 }
 
 template <class P>
 void launch_finish(hipStream_t st, const FinishArgs& f) {
-  if (f.n_seg >= 64 || (f.n_seg >= 8 && f.n_out <= 256))
-    hipLaunchKernelGGL((reduce_finish_kernel<P, 64>), dim3((uint32_t)((f.n_out + kBlock / 64 - 1) / (kBlock / 64))),
-                       dim3(kBlock), 0, st, f);
-  else
-    hipLaunchKernelGGL((reduce_finish_kernel<P, 1>), dim3((uint32_t)((f.n_out + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       st, f);
+#define CT_FINISH(LPO)                                                                                              \
+  hipLaunchKernelGGL((reduce_finish_kernel<P, LPO>),                                                                \
+                     dim3((uint32_t)((f.n_out + (kBlock / 64) * (64 / LPO) - 1) / ((kBlock / 64) * (64 / LPO)))),   \
+                     dim3(kBlock), 0, st, f)
+  // as few lanes per output as keep every lane at kFinishLoads loads or fewer
+  if (f.n_seg <= kFinishLoads) CT_FINISH(1);
+  else if (f.n_seg <= 4 * kFinishLoads) CT_FINISH(4);
+  else if (f.n_seg <= 16 * kFinishLoads) CT_FINISH(16);
+  else CT_FINISH(64);
+#undef CT_FINISH
 }
 
 struct AnyArgs {

@@ -160,7 +160,9 @@ int build_plan(const OperandIn* ops, int n_ops, int64_t n, Plan* plan, bool refe
   for (int k = 0; regular && k < n_ops; ++k) {
     if (!ops[k].dims) continue;
     for (int i = 0; regular && i < rank; ++i) {
-      if (pd[k].index[i]) regular = false;
+      // an indexed axis stays regular only as a full axis of more than one entry (the vector
+      // kernel's row gather / scatter); anything else goes to the reference's address objects
+      if (pd[k].index[i] && (pd[k].shape[i] != mx[i] || mx[i] == 1)) regular = false;
       else if (pd[k].shape[i] != mx[i] && pd[k].shape[i] != 1) regular = false;
       else if (pd[k].shape[i] != 1 && pd[k].stride[i] < 0) regular = false;
       else if (k == 0 && pd[k].shape[i] != mx[i]) regular = false;
@@ -168,41 +170,57 @@ int build_plan(const OperandIn* ops, int n_ops, int64_t n, Plan* plan, bool refe
   }
   plan->regular = regular;
 
-  if (regular) {
+  // `regular` may be withdrawn below (indexed axes that the vector kernel cannot take); the loop
+  // runs once.
+  while (regular) {
     Canon& c = plan->canon;
     c.nd = 0;
+    c.any_index = false;
     for (int i = rank - 1; i >= 0; --i) {
       if (mx[i] == 1) continue;
       c.size[c.nd] = mx[i];
-      for (int k = 0; k < n_ops; ++k)
+      for (int k = 0; k < n_ops; ++k) {
         c.stride[k][c.nd] = (!ops[k].dims || pd[k].shape[i] == 1) ? 0 : pd[k].stride[i];
+        c.index[k][c.nd] = ops[k].dims ? pd[k].index[i] : nullptr;
+        if (c.index[k][c.nd]) c.any_index = true;
+      }
       ++c.nd;
     }
     if (c.nd == 0) {  // a single element
       c.nd = 1;
       c.size[0] = 1;
-      for (int k = 0; k < n_ops; ++k) c.stride[k][0] = ops[k].dims ? 1 : 0;
+      for (int k = 0; k < n_ops; ++k) { c.stride[k][0] = ops[k].dims ? 1 : 0; c.index[k][0] = nullptr; }
     }
     // order axes by destination stride (stable insertion sort)
     for (int i = 1; i < c.nd; ++i)
       for (int j = i; j > 0 && c.stride[0][j - 1] > c.stride[0][j]; --j) {
         std::swap(c.size[j - 1], c.size[j]);
-        for (int k = 0; k < n_ops; ++k) std::swap(c.stride[k][j - 1], c.stride[k][j]);
+        for (int k = 0; k < n_ops; ++k) {
+          std::swap(c.stride[k][j - 1], c.stride[k][j]);
+          std::swap(c.index[k][j - 1], c.index[k][j]);
+        }
       }
-    // merge axis j into axis j-1 when every operand's strides chain
+    // merge axis j into axis j-1 when every operand's strides chain (an indexed axis never merges)
     int w = 0;
     for (int j = 1; j < c.nd; ++j) {
       bool chain = true;
-      for (int k = 0; chain && k < n_ops; ++k) chain = c.stride[k][j] == c.stride[k][w] * c.size[w];
+      for (int k = 0; chain && k < n_ops; ++k)
+        chain = c.stride[k][j] == c.stride[k][w] * c.size[w] && !c.index[k][j] && !c.index[k][w];
       if (chain) {
         c.size[w] *= c.size[j];
       } else {
         ++w;
         c.size[w] = c.size[j];
-        for (int k = 0; k < n_ops; ++k) c.stride[k][w] = c.stride[k][j];
+        for (int k = 0; k < n_ops; ++k) { c.stride[k][w] = c.stride[k][j]; c.index[k][w] = c.index[k][j]; }
       }
     }
     c.nd = w + 1;
+    // indexed axes must be among the first two outer axes, never the innermost
+    bool index_ok = true;
+    for (int k = 0; k < n_ops; ++k)
+      for (int i = 0; i < c.nd; ++i)
+        if (c.index[k][i] && (i == 0 || i > 2)) index_ok = false;
+    if (!index_ok) { regular = false; plan->regular = false; break; }
 
     // ---- classify
     bool fits32 = n < (int64_t(1) << 31);
@@ -213,7 +231,7 @@ int build_plan(const OperandIn* ops, int n_ops, int64_t n, Plan* plan, bool refe
       for (int k = 1; k < n_ops; ++k)
         if (c.stride[k][0] != 0 && c.stride[k][0] != 1) all_unit = false;
       if (all_unit) { plan->kind = PK_VEC; return CT_OK; }
-      if (fits32) {
+      if (fits32 && !c.any_index) {
         int b = -1;
         bool ok = true;
         for (int k = 1; ok && k < n_ops; ++k) {
@@ -232,6 +250,7 @@ int build_plan(const OperandIn* ops, int n_ops, int64_t n, Plan* plan, bool refe
         for (int k = 0; k < kMaxOps; ++k) plan->via_lds[k] = false;
       }
     }
+    if (c.any_index) { regular = false; plan->regular = false; break; }
     // regular but neither vectorisable nor tileable: per-element addressing
     // over the merged axes
     plan->kind = PK_GENERAL;

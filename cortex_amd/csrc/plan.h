@@ -10,6 +10,8 @@
 // selects one of three kernel families:
 //   VEC      every operand is unit-stride or broadcast along the innermost
 //            axis: 128-bit coalesced loads/stores, address math per vector.
+//            One of the first two outer axes of an operand may be addressed
+//            through an index tensor (row gather / scatter).
 //   TILE     the destination is unit-stride along axis A while some input is
 //            unit-stride along another axis B (a transposed view): LDS tile.
 //   GENERAL  anything else, including indirect (index tensor) dimensions and
@@ -30,11 +32,15 @@ struct OperandIn {
 };
 
 // Canonical (merged) iteration space, fastest axis first.  stride 0 marks a
-// broadcast axis of that operand.
+// broadcast axis of that operand.  index[k][d] != nullptr: operand k addresses
+// axis d through an index tensor (coordinate c contributes index[c] * stride);
+// such an axis is never merged with another and is never the innermost one.
 struct Canon {
   int nd;
   int64_t size[CT_MAX_DIMS];
   int64_t stride[kMaxOps][CT_MAX_DIMS];
+  const int32_t* index[kMaxOps][CT_MAX_DIMS];
+  bool any_index;
 };
 
 // One operand of the GENERAL kernel: the four address objects of the CPU
