@@ -151,6 +151,78 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int ti
   return CT_OK;
 }
 
+bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* a, int* n_short, int* ppt, uint32_t* grid) {
+  const Canon& c = plan.canon;
+  if (c.any_index || c.nd < 2 || c.stride[0][0] != 1) return false;
+  // Axis 0 is the destination's unit-stride axis.  Either it is the long axis (planar destination) and
+  // some other axis is the short one, or it is the short axis and the destination is laced along the
+  // axis whose destination stride equals the short extent.
+  int ls = -1, ll = -1;
+  if (c.size[0] >= 2 && c.size[0] <= kLaceMaxShort) {
+    for (int i = 1; i < c.nd && ll < 0; ++i)
+      if (c.stride[0][i] == c.size[0]) ll = i;
+    if (ll >= 0) ls = 0;
+  }
+  if (ls < 0) {
+    // planar destination: the short axis is the one along which some input is unit-stride
+    for (int k = 1; k < plan.n_ops && ls < 0; ++k) {
+      if (!ops[k].ptr) continue;
+      for (int i = 1; i < c.nd; ++i)
+        if (c.stride[k][i] == 1 && c.size[i] >= 2 && c.size[i] <= kLaceMaxShort) { ls = i; break; }
+    }
+    ll = 0;
+  }
+  if (ls < 0 || ll < 0 || ls == ll) return false;
+  const int64_t n_s = c.size[ls], n_l = c.size[ll];
+  if (n_l < 16 || n_l >= kLim31) return false;
+  std::memset(a, 0, sizeof(*a));
+  bool any_laced = false, any_planar = false;
+  for (int k = 0; k < plan.n_ops; ++k) {
+    a->ptr[k] = (char*)ops[k].ptr;
+    a->cbits[k] = ops[k].cbits;
+    if (!ops[k].ptr) { a->const_mask |= 1u << k; continue; }
+    if (c.stride[k][ls] == 1 && c.stride[k][ll] == n_s) {
+      a->laced_mask |= 1u << k;
+      any_laced = true;
+    } else if (c.stride[k][ll] == 1 && c.stride[k][ls] > 0) {
+      a->plane_stride[k] = c.stride[k][ls];
+      any_planar = true;
+    } else {
+      return false;
+    }
+  }
+  if (!any_laced || !any_planar) return false;
+  int64_t rows = 1;
+  int no = 0;
+  for (int d = 0; d < c.nd; ++d) {
+    if (d == ls || d == ll) continue;
+    if (c.size[d] >= kLim31) return false;
+    a->outer_fd[no] = FastDiv((uint32_t)c.size[d]);
+    for (int k = 0; k < plan.n_ops; ++k) a->outer_stride[k][no] = c.stride[k][d];
+    rows *= c.size[d];
+    ++no;
+  }
+  a->n_outer = no;
+  // full-width vectors need every piece a lane touches to start on a vector boundary
+  bool vec = vmax > 1 && n_l % vmax == 0;
+  for (int k = 0; vec && k < plan.n_ops; ++k) {
+    if (!ops[k].ptr) continue;
+    if (((uintptr_t)ops[k].ptr % (uintptr_t)(vmax * ops[k].elem_size)) != 0) vec = false;
+    if (a->plane_stride[k] % vmax != 0) vec = false;
+    for (int d = 0; vec && d < no; ++d)
+      if (a->outer_stride[k][d] % vmax != 0) vec = false;
+  }
+  *ppt = vec ? vmax : 1;
+  *n_short = (int)n_s;
+  const int64_t per_block = (int64_t)kBlock * *ppt;
+  const int64_t per_row = (n_l + per_block - 1) / per_block;
+  if (per_row * rows >= kLim31) return false;
+  a->n_long = (uint32_t)n_l;
+  a->per_row_fd = FastDiv((uint32_t)per_row);
+  *grid = (uint32_t)(per_row * rows);
+  return true;
+}
+
 int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* a, bool* use64, uint32_t* grid) {
   const GenPlan& g = plan.gen;
   std::memset(a, 0, sizeof(*a));

@@ -563,6 +563,158 @@ __global__ void __launch_bounds__(kBlock) ew_tile_kernel(const F f, const TileAr
   else tile_body<F, false, STREAM, SHAPE>(f, a, off, a0, b0, smem);
 }
 
+// ------------------------------------------------------------------ LACE (planar <-> interleaved)
+
+// A short axis S (2..4 entries: the channels of an image) and a long axis L (the pixels).  An
+// operand is either PLANAR, unit-stride along L with any stride along S ([C,H,W]), or LACED,
+// unit-stride along S with stride |S| along L ([H,W,C]); a call mixes the two (an image going
+// from one layout to the other).  Neither the vector kernel (no common unit-stride axis) nor
+// the tile kernel (an edge of 3) fits.
+//
+// A block takes kBlock * PPT consecutive positions of L with all of S.  In registers a lane
+// holds its PPT positions plane by plane (S vectors of PPT elements).  A planar operand is
+// read or written as exactly those vectors.  A laced operand's share of the block is one
+// contiguous run of S * kBlock vectors: the lanes move it with fully coalesced vector accesses
+// (lane i takes vectors i, i + kBlock, ...) and it changes layout on its way through LDS, kept
+// there plane by plane: the laced side touches LDS element by element (position = flat / S,
+// entry = flat % S, S a compile-time constant), the planar side vector by vector.
+struct LaceArgs {
+  uint32_t n_long;                 // |L|
+  FastDiv per_row_fd;              // blocks per outer row: ceil(|L| / (kBlock * PPT))
+  int32_t n_outer;
+  FastDiv outer_fd[CT_MAX_DIMS - 2];
+  char* ptr[kMaxOps];
+  int64_t outer_stride[kMaxOps][CT_MAX_DIMS - 2];
+  int64_t plane_stride[kMaxOps];   // planar operands: stride along S
+  uint32_t laced_mask;             // bit k: operand k is laced
+  uint32_t const_mask;
+  uint64_t cbits[kMaxOps];
+};
+
+constexpr int kLaceMaxShort = 4;
+constexpr int kLacePadBytes = 16;  // between the planes in LDS: shifts the banks, keeps vectors aligned
+
+template <int S, int PPT> constexpr size_t lace_lds_bytes(size_t elem) { return S * (kBlock * PPT * elem + kLacePadBytes); }
+
+// Reads one input of the block into registers, plane by plane: x[c].v[p] is entry c of the lane's position p.
+template <class T, int S, int PPT>
+__device__ __forceinline__ void lace_load(Vec<T, PPT>* x, const T* base, int64_t plane_stride, bool laced, uint32_t l_blk,
+                                          uint32_t n_here, char* smem) {
+  constexpr uint32_t kPlaneBytes = kBlock * PPT * sizeof(T) + kLacePadBytes;
+  const uint32_t lp = threadIdx.x * PPT;
+  const bool live = lp < n_here;
+  if (!laced) {
+    if (live) {
+#pragma unroll
+      for (int c = 0; c < S; ++c) x[c] = nt_load(reinterpret_cast<const Vec<T, PPT>*>(base + c * plane_stride + l_blk + lp));
+    }
+    return;
+  }
+  const Vec<T, PPT>* run = reinterpret_cast<const Vec<T, PPT>*>(base + (int64_t)l_blk * S);
+  const uint32_t n_vecs = n_here * S / PPT;
+  Vec<T, PPT> v[S];
+#pragma unroll
+  for (int j = 0; j < S; ++j)
+    if (threadIdx.x + j * kBlock < n_vecs) v[j] = nt_load(run + threadIdx.x + j * kBlock);
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    const uint32_t vi = threadIdx.x + j * kBlock;
+    if (vi < n_vecs) {
+#pragma unroll
+      for (int e = 0; e < PPT; ++e) {
+        const uint32_t flat = vi * PPT + e;
+        *reinterpret_cast<T*>(smem + (flat % S) * kPlaneBytes + (flat / S) * sizeof(T)) = v[j].v[e];
+      }
+    }
+  }
+  __syncthreads();
+  if (live) {
+#pragma unroll
+    for (int c = 0; c < S; ++c) x[c] = *reinterpret_cast<const Vec<T, PPT>*>(smem + c * kPlaneBytes + lp * sizeof(T));
+  }
+  __syncthreads();  // the tile is free for the next operand
+}
+
+template <class F, int S, int PPT>
+__global__ void __launch_bounds__(kBlock) ew_lace_kernel(const F f, const LaceArgs a) {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+  __shared__ __align__(16) char smem[lace_lds_bytes<S, PPT>(elem_sizes<F>::max_all)];
+  uint32_t row, lb;
+  a.per_row_fd.divmod(blockIdx.x, row, lb);
+  int64_t off[kMaxOps] = {0, 0, 0, 0};
+  for (int d = 0; d < a.n_outer; ++d) {
+    uint32_t q, r;
+    a.outer_fd[d].divmod(row, q, r);
+    row = q;
+#pragma unroll
+    for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)r * a.outer_stride[k][d];
+  }
+  const uint32_t l_blk = lb * (uint32_t)(kBlock * PPT);
+  const uint32_t left = a.n_long - l_blk;
+  const uint32_t n_here = left < (uint32_t)(kBlock * PPT) ? left : (uint32_t)(kBlock * PPT);  // a multiple of PPT
+  const uint32_t lp = threadIdx.x * PPT;
+  const bool live = lp < n_here;
+
+  Vec<In0, PPT> x0[S];
+  Vec<In1, PPT> x1[S];
+  Vec<In2, PPT> x2[S];
+  const bool c0 = (a.const_mask >> 1) & 1u, c1 = (a.const_mask >> 2) & 1u, c2 = (a.const_mask >> 3) & 1u;
+  if constexpr (NIN >= 1)
+    if (!c0) lace_load<In0, S, PPT>(x0, reinterpret_cast<const In0*>(a.ptr[1]) + off[1], a.plane_stride[1], (a.laced_mask >> 1) & 1u, l_blk, n_here, smem);
+  if constexpr (NIN >= 2)
+    if (!c1) lace_load<In1, S, PPT>(x1, reinterpret_cast<const In1*>(a.ptr[2]) + off[2], a.plane_stride[2], (a.laced_mask >> 2) & 1u, l_blk, n_here, smem);
+  if constexpr (NIN >= 3)
+    if (!c2) lace_load<In2, S, PPT>(x2, reinterpret_cast<const In2*>(a.ptr[3]) + off[3], a.plane_stride[3], (a.laced_mask >> 3) & 1u, l_blk, n_here, smem);
+
+  Vec<Out, PPT> o[S];
+#pragma unroll
+  for (int c = 0; c < S; ++c)
+#pragma unroll
+    for (int p = 0; p < PPT; ++p) {
+      In0 p0{};
+      In1 p1{};
+      In2 p2{};
+      if constexpr (NIN >= 1) p0 = c0 ? const_from_bits<In0>(a.cbits[1]) : x0[c].v[p];
+      if constexpr (NIN >= 2) p1 = c1 ? const_from_bits<In1>(a.cbits[2]) : x1[c].v[p];
+      if constexpr (NIN >= 3) p2 = c2 ? const_from_bits<In2>(a.cbits[3]) : x2[c].v[p];
+      o[c].v[p] = f(p0, p1, p2);
+    }
+
+  Out* dbase = reinterpret_cast<Out*>(a.ptr[0]) + off[0];
+  if (!(a.laced_mask & 1u)) {
+    if (live) {
+#pragma unroll
+      for (int c = 0; c < S; ++c) *reinterpret_cast<Vec<Out, PPT>*>(dbase + c * a.plane_stride[0] + l_blk + lp) = o[c];
+    }
+    return;
+  }
+  constexpr uint32_t kPlaneBytes = kBlock * PPT * sizeof(Out) + kLacePadBytes;
+  if (live) {
+#pragma unroll
+    for (int c = 0; c < S; ++c) *reinterpret_cast<Vec<Out, PPT>*>(smem + c * kPlaneBytes + lp * sizeof(Out)) = o[c];
+  }
+  __syncthreads();
+  Vec<Out, PPT>* run = reinterpret_cast<Vec<Out, PPT>*>(dbase + (int64_t)l_blk * S);
+  const uint32_t n_vecs = n_here * S / PPT;
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    const uint32_t vi = threadIdx.x + j * kBlock;
+    if (vi < n_vecs) {
+      Vec<Out, PPT> v;
+#pragma unroll
+      for (int e = 0; e < PPT; ++e) {
+        const uint32_t flat = vi * PPT + e;
+        v.v[e] = *reinterpret_cast<const Out*>(smem + (flat % S) * kPlaneBytes + (flat / S) * sizeof(Out));
+      }
+      run[vi] = v;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ GENERAL
 
 struct GenArgs {
@@ -698,6 +850,14 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int ti
                  size_t* lds_bytes,
                  uint32_t* grid);
 int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use64, uint32_t* grid);
+// Recognises the planar <-> interleaved pattern in a regular plan that neither the vector nor the
+// tile kernel took.  Returns false when it does not apply; otherwise fills the arguments, the
+// short axis' extent (2..kLaceMaxShort) and the vector width (vmax or 1) and the grid.
+bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* args, int* n_short, int* ppt, uint32_t* grid);
+
+// Functors that the lace kernel is built for declare `static constexpr bool kLace = true`.
+template <class F, class = void> struct has_lace : std::false_type {};
+template <class F> struct has_lace<F, std::enable_if_t<F::kLace>> : std::true_type {};
 
 // Flat, every tensor operand unit-stride and no constants: the contiguous form.
 inline bool vec_is_flat(const VecArgs& a, int nin) {
@@ -836,6 +996,27 @@ int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t 
     CT_TILE_LAUNCH(TS_WIDE_B);
 #undef CT_TILE_LAUNCH
     return after_launch(s);
+  }
+  if constexpr (has_lace<F>::value) {
+    LaceArgs la;
+    int n_short = 0, ppt = 1;
+    uint32_t lgrid = 0;
+    if (plan.regular && prepare_lace(plan, ops, VMAX, &la, &n_short, &ppt, &lgrid)) {
+      note_kernel(ppt > 1 ? "lace" : "lace1");
+#define CT_LACE(S_)                                                                                          \
+  case S_:                                                                                                   \
+    if (ppt > 1) hipLaunchKernelGGL((ew_lace_kernel<F, S_, VMAX>), dim3(lgrid), dim3(kBlock), 0, s, f, la);  \
+    else hipLaunchKernelGGL((ew_lace_kernel<F, S_, 1>), dim3(lgrid), dim3(kBlock), 0, s, f, la);             \
+    break
+      switch (n_short) {
+        CT_LACE(2);
+        CT_LACE(3);
+        CT_LACE(4);
+        default: return set_error(CT_ERR_INVALID, "internal: lace extent %d", n_short);
+      }
+#undef CT_LACE
+      return after_launch(s);
+    }
   }
   GenArgs ga;
   bool use64 = false;

@@ -31,6 +31,7 @@ namespace cthip {
 
 template <class D, class S> struct AssignF {
   static constexpr int NIN = 1;
+  static constexpr bool kLace = true;  // planar <-> interleaved images go through ew_lace_kernel
   using Out = D;
   using In0 = S;
   using In1 = D;

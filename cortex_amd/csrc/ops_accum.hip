@@ -198,47 +198,36 @@ struct GroupedArgs {
   int32_t reverse;
 };
 
-// rank[i] = number of entries that sort before entry i (smaller value, or equal value and
-// smaller position): a stable counting rank, quadratic but one launch.  Entry i is then
-// stored at its rank.  A block ranks 64 entries: lane l of every wave owns entry l of the
-// block, the block's four waves each count over a quarter of every tile of the index tensor
-// (read from LDS four values at a time; the reads are wave-uniform), and the four counts meet
-// in LDS.
-constexpr int kRankTile = 4096;  // entries staged in LDS at a time; a multiple of 16
+// rank[i] = number of entries that sort before entry i, where entries are ordered by
+// (value bits, position): a stable counting rank, quadratic but one short launch.  Entry i is
+// then stored at its rank.  (Any total order on the values will do: equal values must end up
+// adjacent and in increasing position, nothing more.)  One wave per entry: its lanes walk the
+// index tensor 64 entries at a time (coalesced; the tensor is a few KiB and stays cached),
+// each lane counts the entries that precede i among those it sees, and the lanes' counts
+// meet in a shuffle sum.
 constexpr uint32_t kRankMaxEntries = 8192;
-__global__ void __launch_bounds__(kBlock) index_rank_kernel(const int32_t* index, uint32_t n, int32_t* skey, int32_t* perm) {
-  __shared__ __align__(16) int32_t tile[kRankTile];
-  __shared__ uint32_t part[3][64];
-  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-  const uint32_t i = blockIdx.x * 64u + lane;
-  const int32_t mine = i < n ? index[i] : 0;
-  uint32_t rank = 0;
-  for (uint32_t base = 0; base < n; base += kRankTile) {
-    const uint32_t len = n - base < (uint32_t)kRankTile ? n - base : (uint32_t)kRankTile;
-    __syncthreads();
-    for (uint32_t j = threadIdx.x; j < (uint32_t)kRankTile; j += kBlock) tile[j] = j < len ? index[base + j] : INT32_MAX;
-    __syncthreads();
-    // this wave's quarter of the tile, in groups of four; padding entries (INT32_MAX at positions
-    // >= n) never count: they are neither smaller nor, at a larger position, equal-and-earlier
-    const uint32_t q0 = wave * (kRankTile / 4), q1 = q0 + kRankTile / 4;
-    if (q0 < len) {
-#pragma unroll 4
-      for (uint32_t j = q0; j < q1; j += 4) {
-        const int4 o = *reinterpret_cast<const int4*>(&tile[j]);
-        const uint32_t pos = base + j;
-        rank += (o.x < mine || (o.x == mine && pos < i)) ? 1u : 0u;
-        rank += (o.y < mine || (o.y == mine && pos + 1 < i)) ? 1u : 0u;
-        rank += (o.z < mine || (o.z == mine && pos + 2 < i)) ? 1u : 0u;
-        rank += (o.w < mine || (o.w == mine && pos + 3 < i)) ? 1u : 0u;
-      }
-    }
+__global__ void __launch_bounds__(kBlock) index_rank_kernel(const int32_t* __restrict__ index, uint32_t n,
+                                                            int32_t* __restrict__ skey, int32_t* __restrict__ perm) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t i = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const int32_t mine = index[i];
+  const uint64_t mine64 = ((uint64_t)(uint32_t)mine << 32) | i;
+  uint32_t count = 0;
+  uint32_t j = lane;
+  for (; j + 3 * 64 < n; j += 4 * 64) {
+    const int32_t v0 = index[j], v1 = index[j + 64], v2 = index[j + 128], v3 = index[j + 192];
+    count += (((uint64_t)(uint32_t)v0 << 32) | j) < mine64 ? 1u : 0u;
+    count += (((uint64_t)(uint32_t)v1 << 32) | (j + 64)) < mine64 ? 1u : 0u;
+    count += (((uint64_t)(uint32_t)v2 << 32) | (j + 128)) < mine64 ? 1u : 0u;
+    count += (((uint64_t)(uint32_t)v3 << 32) | (j + 192)) < mine64 ? 1u : 0u;
   }
-  if (wave > 0) part[wave - 1][lane] = rank;
-  __syncthreads();
-  if (wave == 0 && i < n) {
-    rank += part[0][lane] + part[1][lane] + part[2][lane];
-    skey[rank] = mine;
-    perm[rank] = (int32_t)i;
+  for (; j < n; j += 64) count += (((uint64_t)(uint32_t)index[j] << 32) | j) < mine64 ? 1u : 0u;
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) count += __shfl_xor(count, m, 64);
+  if (lane == 0) {
+    skey[count] = mine;
+    perm[count] = (int32_t)i;
   }
 }
 
@@ -384,7 +373,7 @@ int sort_index(hipStream_t s, const int32_t* index, uint32_t n, const int32_t** 
   if (n <= kRankMaxEntries) {
     if (int rc = stream_scratch(s, (size_t)n * 8, &block, kScratchAccumA)) return rc;
     int32_t* k = static_cast<int32_t*>(block);
-    hipLaunchKernelGGL(index_rank_kernel, dim3((n + 63) / 64), dim3(kBlock), 0, s, index, n, k, k + n);
+    hipLaunchKernelGGL(index_rank_kernel, dim3((n + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, s, index, n, k, k + n);
     *skey = k;
     *perm = k + n;
     return CT_OK;
