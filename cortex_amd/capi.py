@@ -164,6 +164,7 @@ PROTOTYPES = {
     "ct_gemm": [_P, _P, _L, _I, _I, _D, _P, _L, _L, _L, _P, _L, _L, _D, _I],
     "ct_gemv": [_P, _P, _L, _I, _D, _P, _L, _L, _L, _P, _L, _D, _I],
     "ct_rand": [_P, _P, _L, _I, _I, _D, _D, C.c_uint64, C.c_uint64],
+    "ct_dropout_bernoulli_mask": [_P, _P, _I, _P, _L, _D, C.c_uint64, C.c_uint64],
     "ct_adam_step": [_P, _I, _D, _D, _D, _D, _D, _D, _D, _P, _P, _P, _P, _L],
     "ct_adadelta_step": [_P, _I, _D, _D, _P, _P, _D, _P, _P, _L],
 }

@@ -28,7 +28,15 @@ int binary_run(hipStream_t s, const BinaryCall& c) {
     }
   }
   BinaryF<T, OP> f{xa, ya};
-  return c.serial ? launch_elementwise_serial(s, f, ops, c.n) : launch_elementwise(s, f, ops, c.n);
+  if constexpr (OP == CT_BOP_DIV && !std::is_floating_point<T>::value) {
+    if (int rc = device_error_word(&f.div0)) return rc;
+    if (int rc = arm_device_error_word(s, f.div0)) return rc;
+  }
+  const int rc = c.serial ? launch_elementwise_serial(s, f, ops, c.n) : launch_elementwise(s, f, ops, c.n);
+  if constexpr (OP == CT_BOP_DIV && !std::is_floating_point<T>::value) {
+    if (rc == CT_OK) return check_device_errors("binary-op! :/");
+  }
+  return rc;
 }
 
 template <class T>

@@ -30,6 +30,18 @@ void release_stream_scratch(hipStream_t s);
 
 inline void note_kernel(const char* name) { *last_kernel_slot() = name; }
 
+// A word of device memory per device that kernels set, with a plain store, when they meet a
+// condition the reference's CPU backend would throw on (an integer division by zero).  It is
+// allocated on the first call that may need it.  check_device_errors reads and clears it when
+// debug-sync mode is on (the stream has been synchronised by then) and turns a set word into
+// CT_ERR_INVALID; without debug-sync the word is never read and the call succeeds with 0
+// stored where the division by zero happened.
+int device_error_word(uint32_t** out);
+int check_device_errors(const char* what);
+// In debug-sync mode, clears the word on stream `s` ahead of a launch that may set it, so that
+// what check_device_errors finds afterwards was set by that launch.
+int arm_device_error_word(hipStream_t s, uint32_t* word);
+
 #define CT_HIP(expr)                                                                          \
   do {                                                                                        \
     hipError_t e__ = (expr);                                                                  \

@@ -69,6 +69,53 @@ void release_stream_scratch(hipStream_t s) {
   }
 }
 
+namespace {
+std::mutex g_error_word_mutex;
+std::map<int, uint32_t*> g_error_word;
+}  // namespace
+
+int device_error_word(uint32_t** out) {
+  int dev = 0;
+  CT_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_error_word_mutex);
+  uint32_t*& w = g_error_word[dev];
+  if (!w) {
+    void* p = nullptr;
+    CT_HIP(hipMalloc(&p, 256));
+    hipError_t rc = hipMemset(p, 0, 256);
+    if (rc != hipSuccess) {
+      (void)hipFree(p);
+      return set_error(CT_ERR_HIP, "hipMemset failed: %s", hipGetErrorString(rc));
+    }
+    w = static_cast<uint32_t*>(p);
+  }
+  *out = w;
+  return CT_OK;
+}
+
+int arm_device_error_word(hipStream_t s, uint32_t* word) {
+  if (debug_sync() && word) CT_HIP(hipMemsetAsync(word, 0, sizeof(uint32_t), s));
+  return CT_OK;
+}
+
+int check_device_errors(const char* what) {
+  if (!debug_sync()) return CT_OK;
+  int dev = 0;
+  CT_HIP(hipGetDevice(&dev));
+  uint32_t* w = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_error_word_mutex);
+    auto it = g_error_word.find(dev);
+    if (it == g_error_word.end()) return CT_OK;
+    w = it->second;
+  }
+  uint32_t value = 0;
+  CT_HIP(hipMemcpy(&value, w, sizeof(value), hipMemcpyDeviceToHost));
+  if (value == 0) return CT_OK;
+  CT_HIP(hipMemset(w, 0, sizeof(value)));
+  return set_error(CT_ERR_INVALID, "%s: Divide by zero", what);
+}
+
 int set_error(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);

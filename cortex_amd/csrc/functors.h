@@ -103,14 +103,18 @@ template <class T, int OP, bool PLAIN = false> struct UnaryF {
 __device__ __forceinline__ int32_t jvm_unchecked_int(int64_t v) { return (int32_t)(uint32_t)(uint64_t)v; }
 __device__ __forceinline__ int32_t jvm_unchecked_int(double v) { return jvm_d2i(v); }
 
-// perform-operation-impl (cpu/tensor_math.clj:278-304).
-template <class T, int OP, class A> __device__ __forceinline__ T binary_value(A x, A y) {
+// perform-operation-impl (cpu/tensor_math.clj:278-304).  An integer division by zero, where the
+// reference throws ArithmeticException, stores 0 and sets *div0 (when given).
+template <class T, int OP, class A> __device__ __forceinline__ T binary_value(A x, A y, uint32_t* div0 = nullptr) {
   if constexpr (OP == CT_BOP_ADD) return jvm_cast<T>(w_add(x, y));
   else if constexpr (OP == CT_BOP_SUB) return jvm_cast<T>(w_sub(x, y));
   else if constexpr (OP == CT_BOP_MUL) return jvm_cast<T>(w_mul(x, y));
   else if constexpr (OP == CT_BOP_DIV) {
     if constexpr (std::is_same<A, double>::value) return jvm_cast<T>(x / y);
-    else return jvm_ratio_cast<T>(x, y);
+    else {
+      if (y == 0 && div0) *div0 = 1u;
+      return jvm_ratio_cast<T>(x, y);
+    }
   }
   else if constexpr (OP == CT_BOP_MAX) return jvm_cast<T>(x > y ? x : y);
   else if constexpr (OP == CT_BOP_MIN) return jvm_cast<T>(x > y ? y : x);
@@ -139,6 +143,7 @@ template <class T, int OP, bool PLAIN = false> struct BinaryF {
   using In2 = T;
   using A = typename acc_of<T>::type;
   A xa, ya;
+  uint32_t* div0 = nullptr;  // integer :/ only: the device's error word (see device_error_word)
   __device__ __forceinline__ T operator()(T x, T y, T) const {
     if constexpr (PLAIN) {
       static_assert(std::is_same<T, float>::value && binary_plain_op(OP), "PLAIN is a float form");
@@ -155,7 +160,7 @@ template <class T, int OP, bool PLAIN = false> struct BinaryF {
       else if constexpr (OP == CT_BOP_LT) return fx < fy ? 1.0f : 0.0f;
       else return fx <= fy ? 1.0f : 0.0f;
     } else {
-      return binary_value<T, OP, A>(w_mul((A)x, xa), w_mul((A)y, ya));
+      return binary_value<T, OP, A>(w_mul((A)x, xa), w_mul((A)y, ya), div0);
     }
   }
 };

@@ -510,6 +510,10 @@ int accum_sum_staged(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtyp
 }
 
 template <class T, int OP>
+int accum_run_with(hipStream_t s, BinaryF<T, OP> f, void* dest, const ct_dims* dd, double dest_alpha, const void* y,
+                   const ct_dims* yd, double y_alpha, int64_t n, bool reverse, int dtype);
+
+template <class T, int OP>
 int accum_run(hipStream_t s, void* dest, const ct_dims* dd, double dest_alpha, const void* y, const ct_dims* yd,
               double y_alpha, int64_t n, bool reverse, int dtype) {
   using A = typename acc_of<T>::type;
@@ -517,6 +521,20 @@ int accum_run(hipStream_t s, void* dest, const ct_dims* dd, double dest_alpha, c
   // f(first, second) = op(first * xa, second * ya)
   f.xa = reverse ? (A)jvm_cast<T>(y_alpha) : (A)jvm_cast<T>(dest_alpha);
   f.ya = reverse ? (A)jvm_cast<T>(dest_alpha) : (A)jvm_cast<T>(y_alpha);
+  if constexpr (OP == CT_BOP_DIV && !std::is_floating_point<T>::value) {
+    if (int rc = device_error_word(&f.div0)) return rc;
+    if (int rc = arm_device_error_word(s, f.div0)) return rc;
+    const int rc = accum_run_with(s, f, dest, dd, dest_alpha, y, yd, y_alpha, n, reverse, dtype);
+    return rc == CT_OK ? check_device_errors("binary-accum! :/") : rc;
+  } else {
+    return accum_run_with(s, f, dest, dd, dest_alpha, y, yd, y_alpha, n, reverse, dtype);
+  }
+}
+
+template <class T, int OP>
+int accum_run_with(hipStream_t s, BinaryF<T, OP> f, void* dest, const ct_dims* dd, double dest_alpha, const void* y,
+                   const ct_dims* yd, double y_alpha, int64_t n, bool reverse, int dtype) {
+  using A = typename acc_of<T>::type;
   OwnerArgs a;
   std::memset(&a, 0, sizeof(a));
   if (owner_structure(*dd, *yd, n, &a)) {

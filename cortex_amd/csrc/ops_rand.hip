@@ -91,9 +91,89 @@ __global__ void __launch_bounds__(kBlock) rand_kernel(const RandArgs a) {
   }
 }
 
+// The bernoulli dropout mask in one pass (src/cortex/compute/nn/layers.clj:170-195): the
+// reference draws rand! flat over [p - 1, p) into a float buffer, assign!s it into the
+// multiplier buffer (a conversion when the network runs in double) and turns it into the mask
+// with ternary-op! :select, (x >= 0) ? 1 / p : 0.  One lane draws the same Philox block as
+// rand_kernel, forms the same float, converts it as assign! does and selects: the stored
+// values are those of the three calls, bit for bit.
+template <class T, bool KEEP_RAND, bool ALIGNED>
+__global__ void __launch_bounds__(kBlock) dropout_mask_kernel(const RandArgs a, T* mult, const T keep_value,
+                                                              const T drop_value) {
+  const uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t first = (int64_t)i * 4;
+  if (first >= a.n) return;
+  Vec<float, 4> r;
+  rand_block<CT_DIST_FLAT>(a, i, r.v);
+  Vec<T, 4> m;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const T x = jvm_convert<T, float>(r.v[e]);          // assign!
+    m.v[e] = ((double)x >= 0.0) ? keep_value : drop_value;  // select on x * 1.0
+  }
+  if (ALIGNED && first + 4 <= a.n) {
+    if constexpr (KEEP_RAND) *reinterpret_cast<Vec<float, 4>*>(a.dest + first) = r;
+    if constexpr (sizeof(T) == 4) {
+      *reinterpret_cast<Vec<T, 4>*>(mult + first) = m;
+    } else {
+      *reinterpret_cast<Vec<T, 2>*>(mult + first) = Vec<T, 2>{{m.v[0], m.v[1]}};
+      *reinterpret_cast<Vec<T, 2>*>(mult + first + 2) = Vec<T, 2>{{m.v[2], m.v[3]}};
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (first + e < a.n) {
+        if constexpr (KEEP_RAND) a.dest[first + e] = r.v[e];
+        mult[first + e] = m.v[e];
+      }
+  }
+}
+
+template <class T>
+int dropout_mask_run(hipStream_t s, RandArgs r, void* mult, double probability) {
+  // the constants as the reference's front end hands them to the backend: already multiplied by
+  // their alphas in double (src/cortex/tensor.clj:802-803), then cast to the tensor's datatype
+  const T keep_value = jvm_cast<T>(1.0 * (1.0 / probability));
+  const T drop_value = jvm_cast<T>(0.0 * 0.0);
+  const bool keep_rand = r.dest != nullptr && (void*)r.dest != mult;
+  const bool aligned = (uintptr_t)mult % 16 == 0 && (!keep_rand || (uintptr_t)r.dest % 16 == 0);
+  const dim3 grid((uint32_t)(((r.n + 3) / 4 + kBlock - 1) / kBlock));
+  T* m = reinterpret_cast<T*>(mult);
+  note_kernel("dropout_mask");
+#define CT_DROPOUT(KEEP, AL) hipLaunchKernelGGL((dropout_mask_kernel<T, KEEP, AL>), grid, dim3(kBlock), 0, s, r, m, keep_value, drop_value)
+  if (keep_rand) { if (aligned) CT_DROPOUT(true, true); else CT_DROPOUT(true, false); }
+  else { if (aligned) CT_DROPOUT(false, true); else CT_DROPOUT(false, false); }
+#undef CT_DROPOUT
+  return after_launch(s);
+}
+
 }  // namespace
 
 extern "C" {
+
+int ct_dropout_bernoulli_mask(void* stream, void* mult_buffer, int dtype, void* rand_buffer, int64_t n,
+                              double probability, uint64_t seed, uint64_t offset) {
+  CT_REQUIRE(dtype == CT_F32 || dtype == CT_F64, "ct_dropout_bernoulli_mask: datatype must be float or double");
+  CT_REQUIRE(n >= 0, "ct_dropout_bernoulli_mask: negative count");
+  if (n == 0) return CT_OK;
+  CT_REQUIRE(mult_buffer != nullptr, "ct_dropout_bernoulli_mask: null buffer");
+  CT_REQUIRE(n < (int64_t(1) << 40), "ct_dropout_bernoulli_mask: count exceeds the supported range");
+  // the layer's distribution: maximum = (float probability), minimum = maximum - 1.0, then rand!'s own
+  // rounding of both bounds to float (compute/nn/layers.clj:179-182; ct_rand)
+  const double maximum_d = (double)(float)probability;
+  const float minimum = (float)(maximum_d - 1.0), maximum = (float)maximum_d;
+  CT_REQUIRE(minimum < maximum, "Minimum must be less than maximum");
+  RandArgs r;
+  r.dest = reinterpret_cast<float*>(rand_buffer);
+  r.n = n;
+  r.seed_lo = (uint32_t)seed; r.seed_hi = (uint32_t)(seed >> 32);
+  r.off_lo = (uint32_t)offset; r.off_hi = (uint32_t)(offset >> 32);
+  r.p0 = (double)minimum;
+  r.p1 = (double)maximum - (double)minimum;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == CT_F32) return dropout_mask_run<float>(s, r, mult_buffer, probability);
+  return dropout_mask_run<double>(s, r, mult_buffer, probability);
+}
 
 int ct_rand(void* stream, void* dest, int64_t n, int dtype, int distribution, double a, double b, uint64_t seed,
             uint64_t offset) {

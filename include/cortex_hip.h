@@ -120,7 +120,11 @@ const char* ct_last_error(void);
 
 /* When on, every entry point synchronises its stream before returning so an
  * asynchronous fault surfaces at the call that caused it.  Mirrors
- * *cuda-library-debug-execution* (src/cortex/compute/cuda/driver.clj:88-93). */
+ * *cuda-library-debug-execution* (src/cortex/compute/cuda/driver.clj:88-93).
+ * In this mode an integer division by zero inside binary-op! / binary-accum! :/
+ * is reported by the call that met it: CT_ERR_INVALID, "Divide by zero", where the
+ * reference's CPU backend throws ArithmeticException (cpu/tensor_math.clj:278-304).
+ * With the mode off such a call succeeds and stores 0 for those elements. */
 int ct_set_debug_sync(int on);
 
 /* Name of the kernel family chosen by the most recent tensor call on this
@@ -329,6 +333,18 @@ int ct_gemv(void* stream, void* c, int64_t inc_c, int trans_a, double alpha, con
  * (src/cortex/tensor.clj:1020-1037). */
 int ct_rand(void* stream, void* dest, int64_t n, int dtype, int distribution, double a, double b,
             uint64_t seed, uint64_t offset);
+
+/* The bernoulli dropout mask of src/cortex/compute/nn/layers.clj:170-195 in one launch.  The
+ * reference builds it from three tensor calls: rand! with the flat distribution over
+ * [probability - 1, probability) into rand_buffer (float32), assign! into mult_buffer (the
+ * network's datatype), ternary-op-constant-constant! :select turning every value x of
+ * mult_buffer into (x >= 0) ? 1 / probability : 0.  This entry point stores what those three
+ * calls store, bit for bit, for the same (seed, offset): mult_buffer receives the mask, and
+ * rand_buffer, when it is neither NULL nor mult_buffer itself, the random draws.  dtype (of
+ * mult_buffer) is CT_F32 or CT_F64.  A backend whose dropout layer may call it saves two
+ * passes over the buffer; the three-call chain stays available and gives the same result. */
+int ct_dropout_bernoulli_mask(void* stream, void* mult_buffer, int dtype, void* rand_buffer,
+                              int64_t n, double probability, uint64_t seed, uint64_t offset);
 
 /* Batch normalization.  Every buffer is packed: input and output hold
  * batch_count x channel_count x element_count values (the eltwise forms have

@@ -1,0 +1,100 @@
+"""The fused bernoulli dropout mask against the reference's three-call chain (rand!, assign!,
+ternary-op! :select; src/cortex/compute/nn/layers.clj:170-195), and the integer division by zero
+that the reference's CPU backend throws on (src/cortex/compute/cpu/tensor_math.clj:278-304)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import harness as H
+from cortex_amd import capi
+from harness import View
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def P(pair_factory):
+    with pair_factory() as pair:
+        yield pair
+
+
+def fused(pair, mult: View, rand, n, probability, seed, offset):
+    side = pair.hip
+    capi.call("ct_dropout_bernoulli_mask", side.stream, side.ptr(mult), mult.buf.dtype,
+              side.ptr(rand) if rand is not None else None, n, float(probability), seed, offset)
+    capi.call("ct_stream_sync", side.stream)
+
+
+@pytest.mark.parametrize("n,offset_elems", [(1, 0), (5, 0), (4096, 0), (1000003, 0), (777, 1), (4099, 3)])
+@pytest.mark.parametrize("probability", [0.5, 0.9, 0.3])
+def test_dropout_mask_equals_the_three_call_chain(P, n, offset_elems, probability):
+    seed, offset = 1234567, 42
+    maximum = float(np.float32(probability))
+    minimum = maximum - 1.0
+    for code in (capi.F32, capi.F64):
+        np_t = H.NP_DTYPES[code]
+        total = n + offset_elems + 4
+        # the chain, on the oracle and on the device: rand! -> assign! -> select
+        rand_chain = P.buf(np.zeros(total, np.float32))
+        mult_chain = rand_chain if code == capi.F32 else P.buf(np.zeros(total, np_t))
+        rv, mv = View(rand_chain, [n], offset=offset_elems), View(mult_chain, [n], offset=offset_elems)
+        P.run(H.rand, rv, n, "flat", minimum, maximum, seed, offset)
+        if mult_chain is not rand_chain:
+            P.run(H.assign, mv, rv)
+        P.run(H.ternary_op_constant_constant, mv, mv, 1.0, 0.0 * 0.0, 1.0 * (1.0 / probability), [0, 1, 2])
+        H.assert_bit_exact(mult_chain.download(), mult_chain.host, "three-call chain, device against oracle")
+        # the fused call, with and without a separate buffer for the draws
+        mult_f = P.buf(np.zeros(total, np_t))
+        rand_f = P.buf(np.zeros(total, np.float32)) if code == capi.F64 else None
+        fused(P, View(mult_f, [n], offset=offset_elems), View(rand_f, [n], offset=offset_elems) if rand_f else None, n,
+              probability, seed, offset)
+        assert capi.last_kernel() == "dropout_mask"
+        H.assert_bit_exact(mult_f.download(), mult_chain.host, f"fused mask {np_t.__name__} n={n} p={probability}")
+        if rand_f is not None:
+            H.assert_bit_exact(rand_f.download(), rand_chain.host, "draws kept by the fused call")
+        kept = mult_chain.host[offset_elems:offset_elems + n]
+        assert set(np.unique(kept)) <= {np_t(0), np_t(1.0 / probability)}
+        if n >= 4096:
+            assert abs(np.count_nonzero(kept) / n - probability) < 0.05
+
+
+def test_dropout_mask_rejects_bad_arguments(P):
+    buf = P.buf(np.zeros(16, np.int32))
+    with pytest.raises(capi.CortexHipError, match="float or double"):
+        fused(P, View(buf, [16]), None, 16, 0.5, 1, 0)
+
+
+@pytest.mark.parametrize("code", [capi.I32, capi.I8, capi.I64])
+def test_integer_division_by_zero_is_reported_in_debug_sync_mode(P, code):
+    np_t = H.NP_DTYPES[code]
+    x = P.buf(np.arange(1, 65).astype(np_t))
+    y = P.buf(np.where(np.arange(64) % 7 == 3, 0, 2).astype(np_t))
+    d = P.buf(np.full(64, 9, np_t))
+    with pytest.raises(H.OracleError, match="Divide by zero"):
+        H.binary_op(H.ORACLE, View(d, [64]), View(x, [64]), 1.0, View(y, [64]), 1.0, "/")
+    with pytest.raises(capi.CortexHipError) as err:
+        H.binary_op(P.hip, View(d, [64]), View(x, [64]), 1.0, View(y, [64]), 1.0, "/")
+    assert err.value.status == 1 and "Divide by zero" in err.value.message
+    got = d.download()
+    want = np.where(y.init == 0, 0, x.init // 2).astype(np_t)
+    assert np.array_equal(got, want)          # the other elements are computed; the offending ones hold 0
+    # the flag was cleared: a clean division passes, and so does an unrelated call
+    y2 = P.buf(np.full(64, 3, np_t))
+    H.binary_op(P.hip, View(d, [64]), View(x, [64]), 1.0, View(y2, [64]), 1.0, "/")
+    assert np.array_equal(d.download(), (x.init // 3).astype(np_t))
+    # constant and accumulate forms
+    with pytest.raises(capi.CortexHipError, match="Divide by zero"):
+        H.binary_op_constant(P.hip, View(d, [64]), View(x, [64]), 1.0, 0.0, "/")
+    with pytest.raises(capi.CortexHipError, match="Divide by zero"):
+        H.binary_accum(P.hip, View(d, [8]), 1.0, View(y, [8, 8]), 1.0, "/", requires_cas=True)
+    # with debug-sync off the same call succeeds (0 where the division by zero happened)
+    capi.call("ct_set_debug_sync", 0)
+    try:
+        H.binary_op(P.hip, View(d, [64]), View(x, [64]), 1.0, View(y, [64]), 1.0, "/")
+        assert np.array_equal(d.download(), want)
+    finally:
+        capi.call("ct_set_debug_sync", 1)
+    # what that call left in the device's error word does not surface at a later, clean division
+    H.binary_op(P.hip, View(d, [64]), View(x, [64]), 1.0, View(y2, [64]), 1.0, "/")
+    assert np.array_equal(d.download(), (x.init // 3).astype(np_t))
