@@ -1,0 +1,169 @@
+"""The Clojure glue under clojure/src cannot be executed here (no JVM).  What can be checked on
+the text is checked: every file reads as balanced Clojure forms, every `ct_*` entry point it
+invokes is declared in include/cortex_hip.h with exactly as many parameters as the call passes
+arguments, every TensorMath method of the reference's protocol is implemented with the protocol's
+arity, and every entry point of the header is reachable from the glue."""
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+GLUE = sorted((ROOT / "clojure" / "src" / "cortex" / "compute" / "hip").glob("*.clj"))
+HEADER = ROOT / "include" / "cortex_hip.h"
+
+OPEN, CLOSE = "([{", ")]}"
+PAIR = dict(zip(CLOSE, OPEN))
+
+
+def read_forms(text: str):
+    """A small Clojure reader: returns the top-level forms as nested lists of tokens.  Strings are
+    kept as ('str', value); comments and whitespace are dropped.  Raises on unbalanced input."""
+    pos, n = 0, len(text)
+    stack = [[]]
+    opened = []
+    while pos < n:
+        ch = text[pos]
+        if ch in " \t\r\n,":
+            pos += 1
+        elif ch == ";":
+            while pos < n and text[pos] != "\n":
+                pos += 1
+        elif ch == '"':
+            end = pos + 1
+            while text[end] != '"':
+                end += 2 if text[end] == "\\" else 1
+            stack[-1].append(("str", text[pos + 1:end]))
+            pos = end + 1
+        elif ch == "\\":                       # character literal
+            m = re.match(r"\\(newline|space|tab|.)", text[pos:])
+            stack[-1].append(m.group(0))
+            pos += len(m.group(0))
+        elif ch in OPEN:
+            opened.append((ch, pos))
+            new = [ch]
+            stack[-1].append(new)
+            stack.append(new)
+            pos += 1
+        elif ch in CLOSE:
+            assert opened, f"unmatched {ch!r} at offset {pos}"
+            o, where = opened.pop()
+            assert o == PAIR[ch], f"{o!r} opened at offset {where} is closed by {ch!r} at offset {pos}"
+            stack.pop()
+            pos += 1
+        elif ch in "'`~@^#":                   # reader macros: prefix the next form; #{ and #( open collections
+            if ch == "#" and pos + 1 < n and text[pos + 1] == "_":
+                pos += 2
+            else:
+                pos += 1
+        else:
+            m = re.match(r"[^\s,;\"()\[\]{}]+", text[pos:])
+            stack[-1].append(m.group(0))
+            pos += len(m.group(0))
+    assert not opened, f"{opened[-1][0]!r} opened at offset {opened[-1][1]} is never closed"
+    return stack[0]
+
+
+def walk(form):
+    if isinstance(form, list):
+        yield form
+        for item in form:
+            yield from walk(item)
+
+
+def header_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:int|const char\*)\s+(ct_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        params = m.group(2).strip()
+        out[m.group(1)] = 0 if params in ("", "void") else len([p for p in params.split(",") if p.strip()])
+    return out
+
+
+def glue_calls():
+    """(file, function name, argument count) for every (call! "ct_..." ...) form."""
+    calls = []
+    for path in GLUE:
+        for form in walk(read_forms(path.read_text())):
+            if len(form) >= 3 and form[0] == "(" and form[1] == "call!" and isinstance(form[2], tuple):
+                calls.append((path.name, form[2][1], len(form) - 3))
+    return calls
+
+
+def test_glue_files_exist_and_read_as_balanced_forms():
+    names = {p.name for p in GLUE}
+    assert {"ffi.clj", "driver.clj", "tensor_math.clj", "backend.clj", "optimize.clj", "context.clj"} <= names
+    for path in GLUE:
+        forms = read_forms(path.read_text())
+        assert forms and forms[0][1] == "ns", path
+        assert forms[0][2].startswith("cortex.compute.hip."), path
+
+
+def test_every_native_call_matches_the_header():
+    declared = header_functions()
+    assert len(declared) > 50
+    calls = glue_calls()
+    assert len(calls) > 50
+    for file, name, argc in calls:
+        assert name in declared, f"{file}: {name} is not declared in include/cortex_hip.h"
+        assert argc == declared[name], f"{file}: {name} is called with {argc} arguments, the header declares {declared[name]}"
+
+
+def test_every_entry_point_is_bound():
+    declared = set(header_functions())
+    text = "".join(p.read_text() for p in GLUE)
+    named = set(re.findall(r'"(ct_[a-z0-9_]+)"', text))
+    assert declared - named == set(), sorted(declared - named)
+
+
+def reference_protocol_arities():
+    """Method name -> parameter count of cortex.tensor.math/TensorMath, read from the reference when it
+    is present (it is not on the GPU box); the stored copy of the counts otherwise."""
+    ref = Path("/root/reference/src/cortex/tensor/math.clj")
+    if not ref.exists():
+        return None
+    proto = [f for f in read_forms(ref.read_text()) if f[:2] == ["(", "defprotocol"]][0]
+    return {m[1]: len(m[2]) - 1 for m in proto if isinstance(m, list) and m[0] == "(" and isinstance(m[2], list)}
+
+
+# name -> number of parameters (stream included), src/cortex/tensor/math.clj:11-252
+TENSOR_MATH = {
+    "assign-constant!": 5, "assign!": 6, "unary-accum!": 6, "unary-op!": 8, "binary-accum-constant!": 8,
+    "binary-op-constant!": 10, "binary-accum!": 11, "binary-op!": 11, "ternary-op!": 14, "ternary-op-constant!": 13,
+    "ternary-op-constant-constant!": 11, "unary-reduce!": 7, "gemm!": 14, "gemv!": 12,
+    "batch-normalize-eltwise!": 10, "batch-normalize-spatial!": 11, "batch-normalize-update-and-apply-eltwise!": 13,
+    "batch-normalize-update-and-apply-spatial!": 14, "batch-normalize-gradients-eltwise!": 14,
+    "batch-normalize-gradients-spatial!": 15, "activation-gradient!": 9, "softmax-eltwise!": 5, "softmax-spatial!": 5,
+    "convolution-descriptor": 10, "choose-convolution-algorithms": 9, "convolution-forward!": 12,
+    "convolution-backward-weights!": 12, "convolution-backward-data!": 12, "pooling-descriptor": 10,
+    "pooling-forward!": 7, "pooling-backward!": 11, "rand!": 4, "lrn-descriptor": 5, "lrn-forward!": 6,
+    "lrn-backward!": 10,
+}
+
+
+def test_stored_protocol_arities_are_the_references():
+    live = reference_protocol_arities()
+    if live is None:
+        pytest.skip("the reference is not mounted here")
+    assert live == TENSOR_MATH
+
+
+def test_tensor_math_is_extended_with_the_protocols_arities():
+    forms = read_forms((ROOT / "clojure/src/cortex/compute/hip/tensor_math.clj").read_text())
+    ext = [f for f in forms if f[:3] == ["(", "extend-type", "HipStream"]]
+    assert len(ext) == 1
+    assert ext[0][3] == "tm/TensorMath"
+    methods = {m[1]: len(m[2]) - 1 for m in ext[0][4:] if isinstance(m, list) and m[0] == "("}
+    assert methods == TENSOR_MATH
+
+
+def test_driver_protocols_are_implemented():
+    text = (ROOT / "clojure/src/cortex/compute/hip/driver.clj").read_text()
+    for method in ("get-devices", "allocate-host-buffer-impl", "memory-info-impl", "create-stream-impl",
+                   "allocate-device-buffer-impl", "allocate-rand-buffer-impl", "sub-buffer-impl", "alias?",
+                   "partially-alias?", "copy-host->device", "copy-device->host", "copy-device->device", "memset",
+                   "create-event", "sync-event", "wait-for-event", "get-driver", "get-device"):
+        assert re.search(r"\(" + re.escape(method) + r"\s+\[", text), method
+    opt = (ROOT / "clojure/src/cortex/compute/hip/optimize.clj").read_text()
+    for key in ("[:hip :adam]", "[:hip :adadelta]", "[:hip :sgd]"):
+        assert "(defmethod create-optimizer " + key in opt
