@@ -604,7 +604,7 @@ def summarize(prof_dir: str, out_dir: str) -> None:
                                                             per_call_bytes, per_call_bytes / alg, alg))
         lines.extend(rows)
         traffic[key] = {"traffic": int(round(per_call_bytes)), "kernel_us": round(per_call_us, 2),
-                        "kernels": list(kernels.keys()), "algorithmic_bytes": alg}
+                        "kernels": [name[:100] for name in kernels], "algorithmic_bytes": alg}
 
     sha = shas.pop()
     head = f"""rocprofv3 summary of bench.py on one MI355X (gfx950): every workload of the step, the other BASELINE configs, the

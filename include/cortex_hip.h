@@ -13,7 +13,11 @@
  *     src/cortex/compute/cuda/driver.clj:40-49.)
  *   - A stream is an opaque handle; NULL selects the device's default stream.
  *     Calls on one stream are ordered and asynchronous with respect to the
- *     host, as on the reference's CUDA backend.
+ *     host, as on the reference's CUDA backend.  One host thread issues calls
+ *     on a given stream at a time: calls that take two launches keep their
+ *     intermediate values in scratch memory owned by the stream, and calls
+ *     from two threads on one stream could interleave between the launches.
+ *     Different threads on different streams are independent.
  *   - Buffers are raw device pointers.  A sub-buffer is pointer arithmetic by
  *     the caller (src/cortex/compute/cuda/driver.clj:502-506).
  *   - Dimensions are given in ELEMENTS, slowest dimension first, exactly as the
