@@ -4,6 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sections a,b,...] [--no-cpu]
     python bench.py --profile-plan FILE ...        (under rocprofv3: marks the segments of the run)
     python bench.py --summarize DIR [--out DIR2]   (turns rocprofv3 output into profiles/ summaries)
+    python bench.py --summarize-counters RUN [--out DIR2]   (per-workload averages of any --pmc run)
 
 The metric is achieved HBM bandwidth of ``binary-op!``, ``unary-reduce!`` and the
 Adam step.  One step is one pass of those three workloads at their BASELINE
@@ -634,6 +635,33 @@ WRITE_SIZE {w_raw:.1f} KiB.  GB/s = algorithmic bytes / summed kernel time of on
     print((out / "bench_trace_and_traffic.txt").read_text())
 
 
+def summarize_counters(run_dir: str, out_file: str) -> None:
+    """Averages every counter of one `rocprofv3 --pmc ...` run of this program per workload and kernel:
+    reads RUN/plan.json (written by --profile-plan) and RUN/*counter_collection.csv, writes a text table."""
+    d = Path(run_dir)
+    plan = json.loads((d / "plan.json").read_text())["segments"]
+    rows = _read_sorted(glob.glob(str(d / "*counter_collection.csv"))[0], "Dispatch_Id")
+    dispatches = collections.OrderedDict()
+    for r_ in rows:
+        rec = dispatches.setdefault(int(r_["Dispatch_Id"]), {"Kernel_Name": r_["Kernel_Name"], "c": {}})
+        rec["c"][r_["Counter_Name"]] = float(r_["Counter_Value"])
+    per_counter = {}
+    names = sorted({c for rec in dispatches.values() for c in rec["c"]})
+    for c in names:
+        segs = _segments(dispatches.values(), plan, lambda rec, c=c: rec["c"].get(c, 0.0))
+        per_counter[c] = segs
+    lines = ["per dispatch averages; columns: " + "  ".join(names), ""]
+    for i, seg in enumerate(plan):
+        if seg["key"].startswith("_") or seg["key"] == "step":
+            continue
+        kernels = per_counter[names[0]][i]
+        for kname in kernels:
+            vals = ["%.4g" % float(np.mean(per_counter[c][i].get(kname, [0.0]))) for c in names]
+            lines.append("%-22s %-60s %s" % (seg["key"], kname[:60], "  ".join(vals)))
+    Path(out_file).write_text("\n".join(lines) + "\n")
+    print("\n".join(lines))
+
+
 # ----------------------------------------------------------------------------- main
 
 def main() -> int:
@@ -647,10 +675,15 @@ def main() -> int:
     ap.add_argument("--adam-n", type=int, default=1 << 28, help="Adam parameter count (2^28 is the benchmark)")
     ap.add_argument("--profile-plan", default=None, help="write the segment plan here and mark segments (for rocprofv3 runs)")
     ap.add_argument("--summarize", default=None, help="directory holding trace/ fetch/ write/ rocprofv3 output")
+    ap.add_argument("--summarize-counters", default=None,
+                    help="directory of one rocprofv3 --pmc run (plan.json + *counter_collection.csv): per-workload averages")
     ap.add_argument("--out", default=str(ROOT / "profiles"))
     args = ap.parse_args()
     if args.summarize:
         summarize(args.summarize, args.out)
+        return 0
+    if args.summarize_counters:
+        summarize_counters(args.summarize_counters, str(Path(args.out) / "counters.txt"))
         return 0
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no cross-GPU exchange); "
