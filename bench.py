@@ -435,6 +435,15 @@ def build_adjacent(b: Bench):
                   lambda: s.rand(o, dims([n]), {"type": "gaussian", "mean": 0.0, "variance": 1.0})))
     ops.append(Op("a_rand_flat", "rand! flat float32 [2^27]", 4 * n,
                   lambda: s.rand(o, dims([n]), {"type": "flat", "minimum": 0.0, "maximum": 1.0})))
+    # the bernoulli dropout mask (compute/nn/layers.clj:170-195): the reference's chain of tensor calls (rand!, then
+    # ternary-op! :select in place; assign! drops out when the network runs in float) against the one-launch form
+    prob = 0.9
+    def chain():
+        s.rand(o, dims([n]), {"type": "flat", "minimum": float(np.float32(prob)) - 1.0, "maximum": float(np.float32(prob))})
+        s.ternary_op_constant_constant(o, dims([n]), o, dims([n]), 1.0, 0.0, 1.0 / prob, n, "select", ["x", "y", "z"])
+    ops.append(Op("a_dropout_chain", "dropout mask float32 [2^27]: rand! + ternary-op! :select (the reference's chain; moves 12 B/element)", 4 * n, chain))
+    ops.append(Op("a_dropout_fused", "dropout mask float32 [2^27]: ct_dropout_bernoulli_mask (one launch, same stored values)", 4 * n,
+                  lambda: s.dropout_bernoulli_mask(o, None, prob)))
     bb, cc, ee = 64, 256, 3136
     nn_ = bb * cc * ee
     st = [b.upload(rng.uniform(0.5, 1.5, cc).astype(np.float32)) for _ in range(8)]

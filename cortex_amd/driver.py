@@ -431,6 +431,19 @@ class HipStream:
                   float(a), float(b), self._rand_seed, self._rand_calls)
         self._rand_calls += 1
 
+    def dropout_bernoulli_mask(self, mult_buffer, rand_buffer, probability) -> None:
+        """The three tensor calls of ``dropout-prepare-forward!`` (``compute/nn/layers.clj:170-195``: ``rand!``,
+        ``assign!``, ``ternary-op! :select``) as one launch with the same stored values.  ``rand_buffer`` may be
+        None (or ``mult_buffer`` itself) when the draws need not be kept.  Advances the stream's generator state
+        as one ``rand!`` call does."""
+        if getattr(self, "_rand_seed", None) is None:
+            self.seed_random(int.from_bytes(os.urandom(8), "little"))
+        seed, offset = self._rand_seed, self._rand_calls
+        self._rand_calls += 1
+        capi.call("ct_dropout_bernoulli_mask", self.handle, mult_buffer.ptr, capi.DTYPE_CODES[mult_buffer.datatype],
+                  None if rand_buffer is None else rand_buffer.ptr, int(mult_buffer.ecount()), float(probability),
+                  seed, offset)
+
     # -- optimizers ---------------------------------------------------------
     def adam_step(self, alpha, beta1, beta2, epsilon, pow_beta1_t, pow_beta2_t, gradient_alpha, gradient, parameters,
                   m, v, n) -> None:

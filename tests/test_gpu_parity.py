@@ -503,7 +503,10 @@ def test_reduce_kernel_selection(P):
     rng = np.random.default_rng(10)
     x = P.buf(rng.standard_normal(64 * 4096).astype(np.float32))
     out = P.buf(np.zeros(4096, np.float32))
-    assert P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 4096]), "sum") == "reduce_row256_vec"
+    assert P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 4096]), "sum") == "reduce_row512_vec"
+    compare(out, "rows of 16 KiB", tol=2e-6)
+    assert P.run(H.unary_reduce, View(out, [128, 1]), 1.0, View(x, [128, 2048]), "sum") == "reduce_row256_vec"
+    compare(out, "rows of 8 KiB", tol=2e-6)
     assert P.run(H.unary_reduce, View(out, [1024, 1]), 1.0, View(x, [1024, 256]), "sum") == "reduce_row_small_vec"
     assert P.run(H.unary_reduce, View(out, [4096, 1]), 1.0, View(x, [4096, 63]), "sum") == "reduce_row_small"
     compare(out, "unaligned short rows", tol=2e-6)
