@@ -187,6 +187,11 @@
   [stream]
   (call! "ct_stream_sync" (:handle stream)))
 
+(defn reserve-scratch!
+  "Grow the stream's scratch blocks now, so that later calls neither allocate nor synchronise."
+  [stream partial-bytes accumulate-bytes]
+  (call! "ct_stream_reserve_scratch" (:handle stream) (long partial-bytes) (long accumulate-bytes)))
+
 (defn timed-event
   "An event that keeps a timestamp, for `elapsed-ms`."
   [stream]

@@ -125,6 +125,7 @@ PROTOTYPES = {
     "ct_host_free": [_P],
     "ct_stream_create": [C.POINTER(_P)],
     "ct_stream_destroy": [_P],
+    "ct_stream_reserve_scratch": [_P, C.c_size_t, C.c_size_t],
     "ct_stream_sync": [_P],
     "ct_event_record": [C.POINTER(_P), _P],
     "ct_event_record_timed": [C.POINTER(_P), _P],

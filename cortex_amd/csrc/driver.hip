@@ -202,6 +202,17 @@ int ct_stream_destroy(void* stream) {
   return CT_OK;
 }
 
+int ct_stream_reserve_scratch(void* stream, size_t partial_bytes, size_t accumulate_bytes) {
+  void* unused = nullptr;
+  if (partial_bytes)
+    if (int rc = stream_scratch((hipStream_t)stream, partial_bytes, &unused, kScratchReduce)) return rc;
+  if (accumulate_bytes) {
+    if (int rc = stream_scratch((hipStream_t)stream, accumulate_bytes, &unused, kScratchAccumA)) return rc;
+    if (int rc = stream_scratch((hipStream_t)stream, accumulate_bytes, &unused, kScratchAccumB)) return rc;
+  }
+  return CT_OK;
+}
+
 int ct_stream_sync(void* stream) {
   CT_HIP(hipStreamSynchronize((hipStream_t)stream));
   return CT_OK;

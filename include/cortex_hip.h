@@ -159,6 +159,19 @@ int ct_host_free(void* ptr);
 /* PDevice create-stream-impl (cuda/driver.clj:589-600). */
 int ct_stream_create(void** stream);
 int ct_stream_destroy(void* stream);
+/* Grows the stream's scratch blocks ahead of time.  No reference counterpart.  Calls that take two
+ * launches keep their intermediate values in scratch memory owned by the stream, which grows on
+ * demand: a call that has to grow a block synchronises the stream, frees the old block and
+ * allocates a new one.  A caller that wants no allocation and no synchronisation inside later
+ * calls (a latency-critical loop, a stream about to be captured into a graph) reserves once:
+ * partial_bytes for the partial results of split reductions, matrix-vector products, convolution
+ * passes and batch-normalization statistics (reductions never need more than 16 MiB),
+ * accumulate_bytes for each of the two blocks that accumulations into a broadcast or indexed
+ * destination stage their temporaries through (at most the destination's size times the updates'
+ * outermost extent; 12 bytes per index entry plus the sort's workspace for indexed rows).
+ * Zero leaves a block as it is. */
+int ct_stream_reserve_scratch(void* stream, size_t partial_bytes, size_t accumulate_bytes);
+
 /* Blocks the host until the stream drains: sync-stream
  * (compute/driver.clj:217-221). */
 int ct_stream_sync(void* stream);

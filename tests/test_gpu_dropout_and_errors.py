@@ -98,3 +98,22 @@ def test_integer_division_by_zero_is_reported_in_debug_sync_mode(P, code):
     # what that call left in the device's error word does not surface at a later, clean division
     H.binary_op(P.hip, View(d, [64]), View(x, [64]), 1.0, View(y2, [64]), 1.0, "/")
     assert np.array_equal(d.download(), (x.init // 3).astype(np_t))
+
+
+def test_reserved_scratch_serves_later_calls(P):
+    """After a reservation a split reduction and a scatter-add give the results they give without one."""
+    capi.call("ct_stream_reserve_scratch", P.hip.stream, 16 << 20, 8 << 20)
+    capi.call("ct_stream_reserve_scratch", P.hip.stream, 0, 0)
+    rng = np.random.default_rng(21)
+    rows, cols = 4096, 512
+    data = P.buf(rng.standard_normal(rows * cols).astype(np.float32))
+    out = P.buf(np.zeros(cols, np.float32))
+    P.run(H.unary_reduce, View(out, [cols, 1]), 1.0, View(data, [cols, rows], [1, cols]), "max")
+    assert capi.last_kernel().startswith("reduce_col")
+    H.assert_bit_exact(out.download(), out.host, "column max after a reservation")
+    table = P.buf(rng.integers(-50, 50, 64 * 32).astype(np.float32))
+    updates = P.buf(rng.integers(-50, 50, 4096 * 32).astype(np.float32))
+    index = P.buf(rng.integers(0, 64, 4096).astype(np.int32))
+    P.run(H.binary_accum, View(table, [4096, 32], [32, 1], index=[index, None]), 1.0, View(updates, [4096, 32]), 1.0, "+")
+    assert capi.last_kernel().startswith("accum_grouped")
+    H.assert_bit_exact(table.download(), table.host, "scatter-add after a reservation")
