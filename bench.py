@@ -511,6 +511,32 @@ def cpu_baseline(data: StepData) -> dict:
 
 # ----------------------------------------------------------------------------- rocprofv3 output -> profiles/
 
+def c_caller_rates() -> dict | None:
+    """Builds tests/c_abi/callrate.c against the library and runs it as a child process: what a call
+    costs a compiled caller (no interpreter between the loop and the C ABI).  None when it cannot be built."""
+    import subprocess
+    import tempfile
+    src = ROOT / "tests" / "c_abi" / "callrate.c"
+    libdir = ROOT / "cortex_amd"
+    with tempfile.TemporaryDirectory() as tmp:
+        exe = Path(tmp) / "callrate"
+        cmd = ["gcc", "-std=c99", "-O1", f"-I{ROOT / 'include'}", str(src), "-o", str(exe), f"-L{libdir}", "-lcortex_hip",
+               "-lm", f"-Wl,-rpath,{libdir}"]
+        try:
+            if subprocess.run(cmd, capture_output=True, text=True, timeout=120).returncode != 0:
+                return None
+            res = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+            if res.returncode != 0:
+                return None
+            out = json.loads(res.stdout.strip().splitlines()[-1])
+        except (OSError, ValueError, subprocess.SubprocessError):
+            return None
+    out["note"] = ("a C99 loop over the C ABI (tests/c_abi/callrate.c), run as a child process: host_us is the loop's own time per "
+                   "call, sustained_us includes the final wait for the stream; the interpreter's share of ops[...].host_us is the "
+                   "difference to these")
+    return out
+
+
 def short_kernel_name(n: str) -> str:
     n = re.sub(r"^void ", "", n.strip('"')).replace("(anonymous namespace)::", "").replace("cthip::", "")
     depth = 0
@@ -791,6 +817,9 @@ def main() -> int:
             sect[op.label] = b.time_op(op)
         result[name] = sect
     b.save_plan()
+    if not args.profile_plan and not args.no_extras:
+        log("timing a compiled caller of the C ABI ...")
+        result["c_caller"] = c_caller_rates()
     if not args.no_cpu:
         log("timing the CPU oracle on the step ...")
         result["cpu_baseline"] = cpu_baseline(data)

@@ -192,6 +192,11 @@
   [stream partial-bytes accumulate-bytes]
   (call! "ct_stream_reserve_scratch" (:handle stream) (long partial-bytes) (long accumulate-bytes)))
 
+(defn check-index-range!
+  "Throws unless every entry of the int index buffer lies in [0, limit). Synchronises the stream."
+  [stream index-buffer n-entries limit]
+  (call! "ct_check_index_range" (:handle stream) (->ptr index-buffer) (long n-entries) (long limit)))
+
 (defn timed-event
   "An event that keeps a timestamp, for `elapsed-ms`."
   [stream]

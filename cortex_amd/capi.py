@@ -126,6 +126,7 @@ PROTOTYPES = {
     "ct_stream_create": [C.POINTER(_P)],
     "ct_stream_destroy": [_P],
     "ct_stream_reserve_scratch": [_P, C.c_size_t, C.c_size_t],
+    "ct_check_index_range": [_P, _P, _L, _L],
     "ct_stream_sync": [_P],
     "ct_event_record": [C.POINTER(_P), _P],
     "ct_event_record_timed": [C.POINTER(_P), _P],

@@ -124,6 +124,17 @@ int set_error(int code, const char* fmt, ...) {
   return code;
 }
 
+namespace {
+// Lowest position whose entry lies outside [0, limit), kept with an unsigned minimum.
+__global__ void __launch_bounds__(kBlock) index_check_kernel(const int32_t* index, uint32_t n, int64_t limit,
+                                                             uint32_t* first_bad) {
+  for (uint32_t i = blockIdx.x * kBlock + threadIdx.x; i < n; i += gridDim.x * kBlock) {
+    const int64_t v = index[i];
+    if (v < 0 || v >= limit) atomicMin(first_bad, i);
+  }
+}
+}  // namespace
+
 }  // namespace cthip
 
 using namespace cthip;
@@ -211,6 +222,28 @@ int ct_stream_reserve_scratch(void* stream, size_t partial_bytes, size_t accumul
     if (int rc = stream_scratch((hipStream_t)stream, accumulate_bytes, &unused, kScratchAccumB)) return rc;
   }
   return CT_OK;
+}
+
+int ct_check_index_range(void* stream, const int32_t* index, int64_t n, int64_t limit) {
+  if (n < 0 || n >= (int64_t(1) << 31)) return set_error(CT_ERR_INVALID, "ct_check_index_range: %lld entries", (long long)n);
+  if (n == 0) return CT_OK;
+  if (!index) return set_error(CT_ERR_INVALID, "ct_check_index_range: null index tensor");
+  hipStream_t s = (hipStream_t)stream;
+  uint32_t* word = nullptr;
+  if (int rc = device_error_word(&word)) return rc;
+  uint32_t* first_bad = word + 1;  // the word itself belongs to the divide-by-zero check
+  CT_HIP(hipMemsetAsync(first_bad, 0xFF, sizeof(uint32_t), s));
+  const uint32_t blocks = (uint32_t)std::min<int64_t>((n + kBlock - 1) / kBlock, 4096);
+  hipLaunchKernelGGL(index_check_kernel, dim3(blocks), dim3(kBlock), 0, s, index, (uint32_t)n, limit, first_bad);
+  CT_HIP(hipGetLastError());
+  uint32_t at = 0;
+  CT_HIP(hipMemcpyAsync(&at, first_bad, sizeof(at), hipMemcpyDeviceToHost, s));
+  CT_HIP(hipStreamSynchronize(s));
+  if (at == 0xFFFFFFFFu) return CT_OK;
+  int32_t value = 0;
+  CT_HIP(hipMemcpy(&value, index + at, sizeof(value), hipMemcpyDeviceToHost));
+  return set_error(CT_ERR_INVALID, "Index out of range: entry %u of the index tensor is %d, outside [0, %lld)", at, value,
+                   (long long)limit);
 }
 
 int ct_stream_sync(void* stream) {

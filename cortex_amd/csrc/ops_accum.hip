@@ -251,8 +251,20 @@ __global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, 
   } else {
     a.kept_fd.divmod((uint32_t)t, i, kv);
   }
-  const int32_t key = a.skey[i];
-  if (i > 0 && a.skey[i - 1] == key) return;
+  // The first kAhead sorted entries and their positions are fetched before the run's extent
+  // is known, so that a run of up to kAhead updates costs two dependent trips to memory
+  // (entries, then updates) instead of three.
+  constexpr int kAhead = 4;
+  int32_t ks[kAhead], ps[kAhead];
+#pragma unroll
+  for (int u = 0; u < kAhead; ++u) {
+    const uint32_t at = i + u < a.n_index ? i + u : a.n_index - 1;
+    ks[u] = a.skey[at];
+    ps[u] = a.perm[at];
+  }
+  const int32_t before = a.skey[i > 0 ? i - 1 : 0];
+  const int32_t key = ks[0];
+  if (i > 0 && before == key) return;
   int64_t doff = (int64_t)key * a.d_gstride, yoff = 0;
   uint32_t rem = kv;
   for (int d = 0; d < a.n_kept; ++d) {
@@ -266,18 +278,18 @@ __global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, 
   V* dp = reinterpret_cast<V*>(reinterpret_cast<T*>(a.dest) + doff);
   const T* yb = reinterpret_cast<const T*>(a.y) + yoff;
   const bool y_unit = a.ky_stride[0] == 1 || VEC == 1;
+  const bool y_once = a.y_gstride != 0;  // every update is read by one lane only
   V acc = *dp;
-  constexpr int kAhead = 4;
   uint32_t j = i;
   for (;;) {
     V upd[kAhead];
     int cnt = 0;
 #pragma unroll
     for (int u = 0; u < kAhead; ++u) {
-      if (cnt == u && j + u < a.n_index && a.skey[j + u] == key) {
-        const T* yp = yb + (int64_t)a.perm[j + u] * a.y_gstride;
+      if (cnt == u && j + u < a.n_index && ks[u] == key) {
+        const T* yp = yb + (int64_t)ps[u] * a.y_gstride;
         if (y_unit) {
-          upd[u] = *reinterpret_cast<const V*>(yp);
+          upd[u] = y_once ? nt_load(reinterpret_cast<const V*>(yp)) : *reinterpret_cast<const V*>(yp);
         } else {  // y broadcast along the vectorised axis
           const T yv = *yp;
 #pragma unroll
@@ -296,6 +308,12 @@ __global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, 
     }
     if (cnt < kAhead) break;
     j += kAhead;
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const uint32_t at = j + u < a.n_index ? j + u : a.n_index - 1;
+      ks[u] = a.skey[at];
+      ps[u] = a.perm[at];
+    }
   }
   *dp = acc;
 }

@@ -172,6 +172,17 @@ int ct_stream_destroy(void* stream);
  * Zero leaves a block as it is. */
 int ct_stream_reserve_scratch(void* stream, size_t partial_bytes, size_t accumulate_bytes);
 
+/* Checks that every entry of an index tensor (the :indexes of a dimension, src/cortex/tensor/
+ * dimensions.clj:150-190) lies in [0, limit), limit being the extent of the dimension that the
+ * entries select from.  The tensor calls themselves do not check: an entry outside the buffer
+ * makes the JVM backend throw an array-bounds exception and makes a GPU kernel read or write
+ * memory it does not own.  A descriptor carries no extent for an indexed dimension, so the caller
+ * that builds the selection (which knows the extent) calls this when it wants the check, for
+ * instance whenever ct_set_debug_sync is on.  Runs after the work already queued on the stream,
+ * waits for the stream, and returns CT_ERR_INVALID "Index out of range: entry ..." naming the
+ * first offending position; nothing is dereferenced through a bad entry.  n < 2^31. */
+int ct_check_index_range(void* stream, const int32_t* index, int64_t n, int64_t limit);
+
 /* Blocks the host until the stream drains: sync-stream
  * (compute/driver.clj:217-221). */
 int ct_stream_sync(void* stream);

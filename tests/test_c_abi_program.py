@@ -12,8 +12,8 @@ SRC = ROOT / "tests" / "c_abi" / "roundtrip.c"
 LIBDIR = ROOT / "cortex_amd"
 
 
-def build(out: pathlib.Path) -> None:
-    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-O1", f"-I{ROOT / 'include'}", str(SRC),
+def build(out: pathlib.Path, src: pathlib.Path = SRC) -> None:
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-O1", f"-I{ROOT / 'include'}", str(src),
            "-o", str(out), f"-L{LIBDIR}", "-lcortex_hip", "-lm", f"-Wl,-rpath,{LIBDIR}"]
     res = subprocess.run(cmd, capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
@@ -22,6 +22,7 @@ def build(out: pathlib.Path) -> None:
 def test_c99_caller_compiles_and_links(tmp_path):
     assert (LIBDIR / "libcortex_hip.so").exists(), "build the library first: python -m cortex_amd.build"
     build(tmp_path / "roundtrip")
+    build(tmp_path / "callrate", ROOT / "tests" / "c_abi" / "callrate.c")
 
 
 @pytest.mark.gpu

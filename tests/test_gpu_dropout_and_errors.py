@@ -117,3 +117,23 @@ def test_reserved_scratch_serves_later_calls(P):
     P.run(H.binary_accum, View(table, [4096, 32], [32, 1], index=[index, None]), 1.0, View(updates, [4096, 32]), 1.0, "+")
     assert capi.last_kernel().startswith("accum_grouped")
     H.assert_bit_exact(table.download(), table.host, "scatter-add after a reservation")
+
+
+def test_index_range_check_names_the_first_bad_entry(P):
+    """ct_check_index_range accepts entries in [0, limit) and reports the first one outside without using it."""
+    rng = np.random.default_rng(22)
+    for n in (1, 77, 5000, 300001):
+        good = rng.integers(0, 1000, n).astype(np.int32)
+        buf = P.buf(good)
+        capi.call("ct_check_index_range", P.hip.stream, P.hip.ptr(View(buf, [n])), n, 1000)
+        for bad_value, where in ((1000, n // 2), (-1, n - 1), (2**31 - 1, 0)):
+            bad = good.copy()
+            bad[where] = bad_value
+            if where + 3 < n:
+                bad[where + 3] = -7  # a later offender must not be the one reported
+            bbuf = P.buf(bad)
+            with pytest.raises(capi.CortexHipError) as err:
+                capi.call("ct_check_index_range", P.hip.stream, P.hip.ptr(View(bbuf, [n])), n, 1000)
+            assert err.value.status == 1
+            assert f"entry {where} of the index tensor is {bad_value}, outside [0, 1000)" in err.value.message
+    capi.call("ct_check_index_range", P.hip.stream, None, 0, 10)
