@@ -231,6 +231,31 @@ def test_unary_ops_all_dtypes(P, code, op):
     compare(xb, f"accum {op} ({k})", tol=tol)
 
 
+def test_float_tanh_dense_sweep(P):
+    """unary-op! :tanh on float tensors runs a single-precision form of its own: a dense sweep of its
+    argument range (the polynomial below 0.4, the seam, the exponential form up to saturation, tiny and
+    huge arguments, both signs) against the oracle's double tanh rounded to float, to the 2e-6 relative
+    bar of a transcendental and to the 6e-7 the form is built for."""
+    pos = np.concatenate([np.linspace(0.0, 0.45, 1 << 21), np.linspace(0.35, 12.0, 1 << 22), np.logspace(-44, -2, 1 << 18),
+                          np.logspace(1, 38, 1 << 16),
+                          np.array([0.4, np.nextafter(np.float32(0.4), np.float32(0)), 88.0, 1e38, np.inf, 0.0])])
+    x = np.concatenate([pos, -pos]).astype(np.float32)
+    n = x.size
+    xb, db = P.buf(x), P.buf(np.zeros(n, np.float32))
+    k = P.run(H.unary_op, View(db, [n]), View(xb, [n]), 1.0, "tanh")
+    got, want = db.download().astype(np.float64), db.host.astype(np.float64)
+    assert np.array_equal(np.signbit(got), np.signbit(want)), k
+    exact = np.tanh(x.astype(np.float64))
+    scale = np.maximum(np.abs(exact), np.finfo(np.float32).tiny)  # denormal results: one denormal step is allowed
+    rel = np.abs(got - exact) / scale
+    worst = int(np.argmax(rel))
+    assert rel[worst] <= 6e-7, (float(x[worst]), got[worst], exact[worst], float(rel[worst]))
+    assert np.all(np.abs(got - want) <= REL_TOL * np.maximum(np.abs(want), np.finfo(np.float32).tiny))
+    nan = P.buf(np.array([np.nan, -np.nan], np.float32))
+    P.run(H.unary_op, View(nan, [2]), View(nan, [2]), 1.0, "tanh")
+    assert np.all(np.isnan(nan.download()))
+
+
 @pytest.mark.parametrize("code", H.ALL_DTYPES)
 @pytest.mark.parametrize("op", list(capi.BINARY_OPS))
 def test_binary_ops_all_dtypes(P, code, op):
