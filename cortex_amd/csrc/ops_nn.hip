@@ -78,29 +78,31 @@ int act_grad_typed(hipStream_t s, void* ig, const ct_dims* igd, const void* og, 
 
 // ------------------------------------------------------------------ softmax
 
-// The running maximum of a row.  java.lang.Math.max propagates NaN and ranks
-// +0 above -0; the sign of a zero maximum cannot reach the result (x - 0 has the
-// same exponential for either zero), so only the NaN rule is kept: half the
-// instructions of the full rule, in kernels whose arithmetic is close to the
-// memory time.
+// The running maximum of a row.  java.lang.Math.max propagates NaN, the hardware's maximum
+// returns the other operand.  The difference cannot reach the result: a NaN element has a NaN
+// exponential whatever is subtracted from it, the row sum is NaN with it, and every element
+// of the row comes out NaN, as it does in the reference (where the maximum itself is NaN).
+// Nor can the sign of a zero maximum.  One instruction per element instead of four, in kernels
+// whose arithmetic, not memory, sets the pace.
 template <class T> __device__ __forceinline__ T jvm_max(T a, T b) {
-  const T r = a > b ? a : b;
-  return __builtin_isunordered(a, b) ? (T)__builtin_nan("") : r;
+  if constexpr (std::is_same<T, float>::value) return __builtin_fmaxf(a, b);
+  else return __builtin_fmax(a, b);
 }
 
-// T(exp(double(x) - double(m))).  For float, x - m is formed exactly as a float
-// head h and tail t (an error-free sum), exp(h + t) = exp(h) * (1 + t) to well
-// below half an ulp, and expf is accurate to about an ulp; a plain float
-// subtraction alone would lose up to |x - m| * 2^-24 relative (3e-6 at a
-// difference of 50).  Infinite operands make the tail meaningless: it is dropped.
+// T(exp(double(x) - double(m))), x <= m.  For float: the difference and its product with
+// log2(e) are formed in double (exact to 1e-16), split into an integer n and a fraction in
+// [-0.5, 0.5]; the hardware's exp2 (1 ulp) takes the fraction as a float (its rounding moves
+// the result by 1e-8 relative) and ldexp applies n.  About a dozen instructions against
+// two dozen for an error-free float difference plus the library's expf; the result is
+// within 1 ulp of the reference's.  n is clamped at -300 (the result is 0 long before), which
+// also keeps it a number when the operand is NaN or -infinity: those reach exp2 through the
+// fraction (NaN - n = NaN, -inf - n = -inf) and give NaN and 0.
 template <class T> __device__ __forceinline__ T shifted_exp(T x, T m) {
   if constexpr (std::is_same<T, float>::value) {
-    const float h = x - m;
-    const float bb = h - x;
-    float t = (x - (h - bb)) + (-m - bb);
-    if (!(fabsf(t) < __builtin_huge_valf())) t = 0.0f;
-    const float e = expf(h);
-    return fmaf(e, t, e);
+    const double a = ((double)x - (double)m) * 1.4426950408889634;
+    const double n = __builtin_fmax(__builtin_rint(a), -300.0);
+    const float frac = (float)(a - n);
+    return __builtin_ldexpf(__builtin_amdgcn_exp2f(frac), (int)n);
   } else {
     return exp(x - m);
   }
