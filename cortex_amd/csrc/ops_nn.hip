@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(kBlock) softmax_wave_kernel(const SoftmaxArgs 
   for (int j = 0; j < ITER; ++j) {
     const uint32_t i = lane + j * TPR;
     if (live && i < nv) {
-      if constexpr (VEC > 1) x[j] = *reinterpret_cast<const V*>(in + (int64_t)i * VEC);
+      if constexpr (VEC > 1) x[j] = nt_load(reinterpret_cast<const V*>(in + (int64_t)i * VEC));  // read once
       else x[j].v[0] = in[(int64_t)i * a.in_k];
 #pragma unroll
       for (int e = 0; e < VEC; ++e) m = jvm_max(m, x[j].v[e]);
@@ -241,7 +241,7 @@ __global__ void __launch_bounds__(kBlock) softmax_lane_kernel(const SoftmaxArgs 
 #pragma unroll
     for (int i = 0; i < CMAX; ++i)
       if ((uint32_t)i < a.k) {
-        x[i] = load(i);
+        x[i] = nt_load(reinterpret_cast<const V*>(in + (int64_t)i * a.in_k));  // read once
 #pragma unroll
         for (int e = 0; e < VEC; ++e) m[e] = jvm_max(m[e], x[i].v[e]);
       }
