@@ -150,8 +150,9 @@ bool owner_structure(const ct_dims& dd, const ct_dims& yd, int64_t n, OwnerArgs*
     if (mx[i] == 1) continue;
     if ((dshape[i] != 1 && dshape[i] != mx[i]) || (yshape[i] != 1 && yshape[i] != mx[i])) return false;
     const int64_t ys = yshape[i] == 1 ? 0 : ystr[i];
-    if (dshape[i] == mx[i]) {
-      if (dstr[i] <= 0) return false;
+    if (dstr[i] < 0) return false;
+    // a destination axis of stride 0 addresses like a broadcast one: every coordinate is one element
+    if (dshape[i] == mx[i] && dstr[i] != 0) {
       a->ksize[a->n_kept] = FastDiv((uint32_t)mx[i]);
       a->kd_stride[a->n_kept] = dstr[i];
       a->ky_stride[a->n_kept] = ys;

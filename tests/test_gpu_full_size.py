@@ -301,3 +301,113 @@ def test_pooling_at_image_batch_size():
         assert abs(lhs - rhs) <= 1e-6 * np.abs(gs).sum(), (op, lhs, rhs)
         for b in (xi, gi, out, ig):
             b.free()
+
+
+def test_indexed_rows_at_benchmark_size():
+    """The row gather and the scatter-add of bench.py's access-pattern section at their full sizes:
+    65536 rows of 1024 floats through an index tensor into / out of a [32768, 1024] table.  The gather
+    against numpy's fancy indexing; the scatter-add against the oracle's serial loop (bit for bit) and,
+    with integer-valued floats whose sums are exact in any order, against numpy's add.at."""
+    rows, table_rows, width = 65536, 32768, 1024
+    rng = np.random.default_rng(81)
+    idx = rng.integers(0, table_rows, rows).astype(np.int32)
+    idx[:4096] = 7  # one long run of equal values
+    table = rng.standard_normal((table_rows, width)).astype(np.float32)
+    upd = rng.integers(-64, 65, (rows, width)).astype(np.float32)
+    d_idx, d_table, d_upd = Dev(idx), Dev(table), Dev(upd)
+    out = Dev(np.zeros(rows * width, np.float32))
+    picked = capi.make_dims([rows, width], [width, 1], [d_idx.ptr, None])
+    capi.call("ct_assign", None, out.ptr, C.byref(dims([rows, width])), capi.F32, d_table.ptr, C.byref(picked), capi.F32,
+              rows * width)
+    assert capi.last_kernel() == "vec"
+    assert bits_equal(out.download().reshape(rows, width), table[idx])
+    out.free()
+
+    capi.call("ct_binary_accum", None, d_table.ptr, C.byref(picked), 1.0, d_upd.ptr, C.byref(dims([rows, width])), 1.0,
+              rows * width, capi.BINARY_OPS["+"], 0, 1, capi.F32)
+    assert capi.last_kernel() == "accum_grouped_vec"
+    got = d_table.download().reshape(table_rows, width)
+    want = table.copy().reshape(-1)
+    host_picked = capi.make_dims([rows, width], [width, 1], [idx.ctypes.data, None])
+    ob.call("binary_accum", want.ctypes.data, C.byref(host_picked), 1.0, upd.ctypes.data, C.byref(dims([rows, width])), 1.0,
+            rows * width, capi.BINARY_OPS["+"], 0, 1, capi.F32)
+    assert bits_equal(got.reshape(-1), want)
+    # exact arithmetic: integer updates into an integer-valued table sum to the same value in any order
+    itable = np.rint(table * 8).astype(np.float32)
+    d_itable = Dev(itable)
+    capi.call("ct_binary_accum", None, d_itable.ptr, C.byref(picked), 1.0, d_upd.ptr, C.byref(dims([rows, width])), 1.0,
+              rows * width, capi.BINARY_OPS["+"], 0, 1, capi.F32)
+    sums = itable.astype(np.float64)
+    np.add.at(sums, idx, upd.astype(np.float64))
+    assert np.array_equal(d_itable.download().reshape(table_rows, width).astype(np.float64), sums)
+    for t in (d_idx, d_table, d_upd, d_itable):
+        t.free()
+
+
+def test_planar_and_interleaved_images_at_benchmark_size():
+    """[256, 3, 224, 224] planar <-> [256, 224, 224, 3] interleaved, float and u8 -> float: numpy's
+    transpose is the closed form, and there and back is the identity."""
+    n, c, h, w = 256, 3, 224, 224
+    rng = np.random.default_rng(82)
+    planar = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    d_planar, d_inter, d_back = Dev(planar), Dev(np.zeros(planar.size, np.float32)), Dev(np.zeros(planar.size, np.float32))
+    inter_as_planar = dims([n, c, h, w], [h * w * c, 1, w * c, c])  # the interleaved buffer addressed [n, c, y, x]
+    cont = dims([n, c, h, w])
+    capi.call("ct_assign", None, d_inter.ptr, C.byref(inter_as_planar), capi.F32, d_planar.ptr, C.byref(cont), capi.F32,
+              planar.size)
+    assert capi.last_kernel() == "lace"
+    assert bits_equal(d_inter.download().reshape(n, h, w, c), planar.transpose(0, 2, 3, 1))
+    capi.call("ct_assign", None, d_back.ptr, C.byref(cont), capi.F32, d_inter.ptr, C.byref(inter_as_planar), capi.F32,
+              planar.size)
+    assert capi.last_kernel() == "lace"
+    assert bits_equal(d_back.download(), planar.reshape(-1))
+    pixels = rng.integers(0, 256, (n, h, w, c)).astype(np.uint8)
+    d_pix = Dev(pixels)
+    capi.call("ct_assign", None, d_back.ptr, C.byref(cont), capi.F32, d_pix.ptr, C.byref(inter_as_planar), capi.U8,
+              planar.size)
+    assert capi.last_kernel() == "lace"
+    assert bits_equal(d_back.download().reshape(n, c, h, w), pixels.transpose(0, 3, 1, 2).astype(np.float32))
+    for t in (d_planar, d_inter, d_back, d_pix):
+        t.free()
+
+
+def test_broadcast_accumulates_at_benchmark_size():
+    """[4096] <- max / + over the 16384 rows of a [16384, 4096] float matrix (the staged forms) against
+    the oracle's serial chain: bit for bit for :max; for :+ bit for bit on integer-valued data (exact in
+    any order) and within 2e-6 of the sum of magnitudes on gaussian data."""
+    rows, cols = 16384, 4096
+    rng = np.random.default_rng(83)
+    y = rng.standard_normal((rows, cols)).astype(np.float32)
+    y[5, 17] = np.nan
+    y[9, 33] = 0.0
+    y[:, 33] = np.minimum(y[:, 33], 0.0)  # a column whose maximum is a zero: the order of +-0 decides
+    start = rng.standard_normal(cols).astype(np.float32)
+    start[33] = -1.0
+    y[0, 33] = -0.0
+    d_y = Dev(y)
+    row_view, full = dims([rows, cols], [0, 1]), dims([rows, cols])
+    for op in ("max", "+"):
+        d_acc = Dev(start)
+        capi.call("ct_binary_accum", None, d_acc.ptr, C.byref(row_view), 1.0, d_y.ptr, C.byref(full), 1.0, rows * cols,
+                  capi.BINARY_OPS[op], 0, 1, capi.F32)
+        kernel = capi.last_kernel()
+        got = d_acc.download()
+        want = start.copy()
+        ob.call("binary_accum", want.ctypes.data, C.byref(row_view), 1.0, y.ctypes.data, C.byref(full), 1.0, rows * cols,
+                capi.BINARY_OPS[op], 0, 1, capi.F32)
+        if op == "max":
+            assert kernel == "accum_staged_extreme", kernel
+            assert bits_equal(got, want)
+        else:
+            assert kernel == "accum_staged_sum", kernel
+            scale = np.abs(start.astype(np.float64)) + np.abs(np.nan_to_num(y.astype(np.float64))).sum(axis=0)
+            ok = np.abs(got.astype(np.float64) - want) <= 2e-6 * scale
+            assert np.all(ok | (np.isnan(got) & np.isnan(want)))
+        d_acc.free()
+    whole = rng.integers(-8, 9, (rows, cols)).astype(np.float32)
+    d_whole, d_acc = Dev(whole), Dev(np.zeros(cols, np.float32))
+    capi.call("ct_binary_accum", None, d_acc.ptr, C.byref(row_view), 1.0, d_whole.ptr, C.byref(full), 1.0, rows * cols,
+              capi.BINARY_OPS["+"], 0, 1, capi.F32)
+    assert np.array_equal(d_acc.download().astype(np.float64), whole.astype(np.float64).sum(axis=0))
+    for t in (d_y, d_whole, d_acc):
+        t.free()

@@ -371,6 +371,7 @@ STAGED_LAYOUTS = [
     ([50], [3], [700, 50], [64, 1]),                     # strided destination, padded rows
     ([33, 1], None, [33, 900], [1, 33]),                 # y is a transposed view
     ([4, 1, 5], None, [4, 1000, 5], None),               # reduced axis in the middle
+    ([500, 40], [0, 1], [500, 40], None),                # a destination axis of stride 0 is a broadcast axis
 ]
 
 
