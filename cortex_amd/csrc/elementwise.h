@@ -146,7 +146,7 @@ __device__ __forceinline__ Vec<T, VEC> vec_load(uint32_t const_mask, uint32_t un
 // index tensor (select rows by label, scatter rows back): the row's coordinate
 // is replaced by index[coordinate] before it meets the stride.  For rows at
 // least a block wide the look-up is one scalar load per wave.
-template <class F, int VEC, int STREAM, int KINDS = -1, bool INDEXED = false>
+template <class F, int VEC, int STREAM, int KINDS = -1, bool INDEXED = false, int PER = 1>
 __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs a) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
@@ -173,8 +173,9 @@ __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs
                "s"(b2), "s"(b3), "s"(s00), "s"(s01), "s"(s10), "s"(s11), "s"(s20), "s"(s21), "s"(s30), "s"(s31),
                "s"(c1), "s"(c2), "s"(c3));
 
-  const uint64_t v_first = (uint64_t)xcd_grouped_unit(blockIdx.x, grouped) * (uint64_t)kBlock;  // the block's first vector
-  if (v_first + threadIdx.x >= total) return;
+  // the block's first vector; a lane takes vector threadIdx.x of each of the block's PER runs of kBlock vectors
+  const uint64_t v_block = (uint64_t)xcd_grouped_unit(blockIdx.x, grouped) * (uint64_t)(kBlock * PER);
+  if (v_block + threadIdx.x >= total) return;
   // Offsets of the outer index `row` for every operand.  Called with a
   // wave-uniform row this is scalar arithmetic.
   auto outer_offsets = [&](uint32_t row, int64_t* off) {
@@ -209,62 +210,82 @@ __global__ void __launch_bounds__(kBlock) ew_vec_kernel(const F f, const VecArgs
       }
     }
   };
-  int64_t off[kMaxOps];
-  int64_t col;
-  if (ifd.d >= (uint32_t)kBlock) {
-    // Rows of at least a block's width: the block's 256 vectors lie in at most two
-    // rows, whose offsets are computed once per wave on the scalar unit; a lane
-    // only picks its row.
-    uint32_t row_a, cv_a;
-    ifd.divmod((uint32_t)v_first, row_a, cv_a);
-    outer_offsets(row_a, off);
-    uint32_t cv = cv_a + threadIdx.x;
-    if (cv_a + (uint32_t)kBlock > ifd.d) {  // the block runs into the next row
-      int64_t off_b[kMaxOps];
-      outer_offsets(row_a + 1, off_b);
-      const bool next = cv >= ifd.d;
-      cv -= next ? ifd.d : 0u;
+  struct Where { int64_t off[kMaxOps]; int64_t col; };
+  auto locate = [&](uint64_t v_first, Where& w) {
+    int64_t* const off = w.off;
+    int64_t col;
+    if (ifd.d >= (uint32_t)kBlock) {
+      // Rows of at least a block's width: the block's 256 vectors lie in at most two
+      // rows, whose offsets are computed once per wave on the scalar unit; a lane
+      // only picks its row.
+      uint32_t row_a, cv_a;
+      ifd.divmod((uint32_t)v_first, row_a, cv_a);
+      outer_offsets(row_a, off);
+      uint32_t cv = cv_a + threadIdx.x;
+      if (cv_a + (uint32_t)kBlock > ifd.d) {  // the block runs into the next row
+        int64_t off_b[kMaxOps];
+        outer_offsets(row_a + 1, off_b);
+        const bool next = cv >= ifd.d;
+        cv -= next ? ifd.d : 0u;
 #pragma unroll
-      for (int k = 0; k < kMaxOps; ++k) off[k] = next ? off_b[k] : off[k];
+        for (int k = 0; k < kMaxOps; ++k) off[k] = next ? off_b[k] : off[k];
+      }
+      col = (int64_t)cv * VEC;
+    } else {
+      uint32_t row, cv;
+      ifd.divmod((uint32_t)v_first + threadIdx.x, row, cv);
+      col = (int64_t)cv * VEC;
+      outer_offsets(row, off);
     }
-    col = (int64_t)cv * VEC;
-  } else {
-    uint32_t row, cv;
-    ifd.divmod((uint32_t)v_first + threadIdx.x, row, cv);
-    col = (int64_t)cv * VEC;
-    outer_offsets(row, off);
-  }
+    w.col = col;
+  };
   char* const base[kMaxOps] = {b0, b1, b2, b3};
   const uint64_t cbits[kMaxOps] = {0, c1, c2, c3};
-  Vec<In0, VEC> x0;
-  Vec<In1, VEC> x1;
-  Vec<In2, VEC> x2;
-  if constexpr (NIN >= 1) {
-    const In0* sp = reinterpret_cast<const In0*>(base[1]) + off[1];
-    x0 = vec_load<In0, VEC, STREAM, (KINDS < 0 ? -1 : (KINDS & 3))>(const_mask, unit_mask, nt_mask, cbits[1], 1, reinterpret_cast<const Vec<In0, VEC>*>(sp + col), sp);
-  }
-  if constexpr (NIN >= 2) {
-    const In1* sp = reinterpret_cast<const In1*>(base[2]) + off[2];
-    x1 = vec_load<In1, VEC, STREAM, (KINDS < 0 ? -1 : ((KINDS >> 2) & 3))>(const_mask, unit_mask, nt_mask, cbits[2], 2, reinterpret_cast<const Vec<In1, VEC>*>(sp + col), sp);
-  }
-  if constexpr (NIN >= 3) {
-    const In2* sp = reinterpret_cast<const In2*>(base[3]) + off[3];
-    x2 = vec_load<In2, VEC, STREAM, (KINDS < 0 ? -1 : ((KINDS >> 4) & 3))>(const_mask, unit_mask, nt_mask, cbits[3], 3, reinterpret_cast<const Vec<In2, VEC>*>(sp + col), sp);
-  }
-  Vec<Out, VEC> r;
+  Where w[PER];
+  bool live[PER];
+  Vec<In0, VEC> x0[PER];
+  Vec<In1, VEC> x1[PER];
+  Vec<In2, VEC> x2[PER];
+  // every load of the lane's PER vectors is issued before its first store
 #pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    In0 p0{};
-    In1 p1{};
-    In2 p2{};
-    if constexpr (NIN >= 1) p0 = x0.v[i];
-    if constexpr (NIN >= 2) p1 = x1.v[i];
-    if constexpr (NIN >= 3) p2 = x2.v[i];
-    r.v[i] = f(p0, p1, p2);
+  for (int h = 0; h < PER; ++h) {
+    const uint64_t v_first = v_block + (uint64_t)h * kBlock;
+    live[h] = h == 0 || v_first + threadIdx.x < total;
+    if (!live[h]) continue;
+    locate(v_first, w[h]);
+    const int64_t* const off = w[h].off;
+    const int64_t col = w[h].col;
+    if constexpr (NIN >= 1) {
+      const In0* sp = reinterpret_cast<const In0*>(base[1]) + off[1];
+      x0[h] = vec_load<In0, VEC, STREAM, (KINDS < 0 ? -1 : (KINDS & 3))>(const_mask, unit_mask, nt_mask, cbits[1], 1, reinterpret_cast<const Vec<In0, VEC>*>(sp + col), sp);
+    }
+    if constexpr (NIN >= 2) {
+      const In1* sp = reinterpret_cast<const In1*>(base[2]) + off[2];
+      x1[h] = vec_load<In1, VEC, STREAM, (KINDS < 0 ? -1 : ((KINDS >> 2) & 3))>(const_mask, unit_mask, nt_mask, cbits[2], 2, reinterpret_cast<const Vec<In1, VEC>*>(sp + col), sp);
+    }
+    if constexpr (NIN >= 3) {
+      const In2* sp = reinterpret_cast<const In2*>(base[3]) + off[3];
+      x2[h] = vec_load<In2, VEC, STREAM, (KINDS < 0 ? -1 : ((KINDS >> 4) & 3))>(const_mask, unit_mask, nt_mask, cbits[3], 3, reinterpret_cast<const Vec<In2, VEC>*>(sp + col), sp);
+    }
   }
-  Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(base[0]) + off[0] + col);
-  if constexpr (STREAM == 2) nt_store(r, dp);
-  else *dp = r;
+#pragma unroll
+  for (int h = 0; h < PER; ++h) {
+    if (!live[h]) continue;
+    Vec<Out, VEC> r;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      In0 p0{};
+      In1 p1{};
+      In2 p2{};
+      if constexpr (NIN >= 1) p0 = x0[h].v[i];
+      if constexpr (NIN >= 2) p1 = x1[h].v[i];
+      if constexpr (NIN >= 3) p2 = x2[h].v[i];
+      r.v[i] = f(p0, p1, p2);
+    }
+    Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(reinterpret_cast<Out*>(base[0]) + w[h].off[0] + w[h].col);
+    if constexpr (STREAM == 2) nt_store(r, dp);
+    else *dp = r;
+  }
 }
 
 // The contiguous case: every operand is a flat unit-stride array read (or
@@ -882,9 +903,14 @@ inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& args) {
   }
   if (a.indexed) {
     // gathered rows are re-read wherever labels repeat and scattered rows are not written in
-    // order: plain accesses, plain block order
+    // order: plain accesses, plain block order.  Four vectors per lane (from four rows when a row is
+    // a block wide): a lane's look-ups and then its row loads are in flight together, which hides
+    // the extra trip to memory that the look-up costs.  Gathering 65536 rows of 4 KiB: one vector
+    // per lane 69 % of peak, two 73 %, four 79 %, eight 73 %.
     a.grouped_blocks = 0;
-    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 0, -1, true>), grid, dim3(kBlock), 0, s, f, a);
+    constexpr int kPer = 4;
+    const dim3 grid_per((uint32_t)((args.total_vecs + kBlock * kPer - 1) / (kBlock * kPer)));
+    hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 0, -1, true, kPer>), grid_per, dim3(kBlock), 0, s, f, a);
     return;
   }
   if (VEC > 1 && a.streaming) {
