@@ -232,6 +232,8 @@ int ct_check_index_range(void* stream, const int32_t* index, int64_t n, int64_t 
   uint32_t* word = nullptr;
   if (int rc = device_error_word(&word)) return rc;
   uint32_t* first_bad = word + 1;  // the word itself belongs to the divide-by-zero check
+  static std::mutex one_check_at_a_time;  // concurrent checks on one device would share first_bad
+  std::lock_guard<std::mutex> lock(one_check_at_a_time);
   CT_HIP(hipMemsetAsync(first_bad, 0xFF, sizeof(uint32_t), s));
   const uint32_t blocks = (uint32_t)std::min<int64_t>((n + kBlock - 1) / kBlock, 4096);
   hipLaunchKernelGGL(index_check_kernel, dim3(blocks), dim3(kBlock), 0, s, index, (uint32_t)n, limit, first_bad);
