@@ -191,7 +191,8 @@ struct GroupedArgs {
   const int32_t* perm;   // the position each sorted entry came from
   uint32_t n_index;      // entries of the index tensor
   uint32_t kept_vecs;    // vectors of the remaining axes per index entry
-  FastDiv kept_fd;       // kept_vecs
+  uint32_t lane_vecs;    // lanes per index entry: kept_vecs, or half of it (rounded up) with two vectors per lane
+  FastDiv lane_fd;       // lane_vecs
   int64_t d_gstride, y_gstride;  // strides of the indexed axis
   int32_t n_kept;
   FastDiv ksize[CT_MAX_DIMS];    // remaining axes, fastest first (axis 0 counted in vectors)
@@ -237,20 +238,21 @@ __global__ void __launch_bounds__(kBlock) iota_kernel(int32_t* out, uint32_t n) 
   if (i < n) out[i] = (int32_t)i;
 }
 
-// One lane per (sorted index entry, vector of the remaining axes).  A lane whose entry is
-// not the first of its value leaves at once; the first walks the run of equal values,
-// fetching kAhead updates before it applies them in order.
-template <class T, int OP, int VEC>
+// One lane per (sorted index entry, PER vectors of the remaining axes, lane_vecs apart).  A lane
+// whose entry is not the first of its value leaves at once; the first walks the run of equal
+// values, fetching kAhead updates before it applies them in order.  PER = 2 puts twice the bytes
+// behind one look-up of the sorted entries.
+template <class T, int OP, int VEC, int PER>
 __global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, OP> f, const GroupedArgs a) {
   using V = Vec<T, VEC>;
   const uint64_t t = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (t >= (uint64_t)a.n_index * a.kept_vecs) return;
+  if (t >= (uint64_t)a.n_index * a.lane_vecs) return;
   uint32_t i, kv;
-  if (a.kept_vecs >= 1u << 31 || t >= (uint64_t(1) << 32)) {
-    i = (uint32_t)(t / a.kept_vecs);
-    kv = (uint32_t)(t % a.kept_vecs);
+  if (a.lane_vecs >= 1u << 31 || t >= (uint64_t(1) << 32)) {
+    i = (uint32_t)(t / a.lane_vecs);
+    kv = (uint32_t)(t % a.lane_vecs);
   } else {
-    a.kept_fd.divmod((uint32_t)t, i, kv);
+    a.lane_fd.divmod((uint32_t)t, i, kv);
   }
   // The first kAhead sorted entries and their positions are fetched before the run's extent
   // is known, so that a run of up to kAhead updates costs two dependent trips to memory
@@ -266,35 +268,47 @@ __global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, 
   const int32_t before = a.skey[i > 0 ? i - 1 : 0];
   const int32_t key = ks[0];
   if (i > 0 && before == key) return;
-  int64_t doff = (int64_t)key * a.d_gstride, yoff = 0;
-  uint32_t rem = kv;
-  for (int d = 0; d < a.n_kept; ++d) {
-    uint32_t q, r;
-    a.ksize[d].divmod(rem, q, r);
-    rem = q;
-    const int64_t c = d == 0 ? (int64_t)r * VEC : (int64_t)r;
-    doff += c * a.kd_stride[d];
-    yoff += c * a.ky_stride[d];
+  V* dp[PER];
+  const T* yb[PER];
+  bool live[PER];
+  V acc[PER];
+#pragma unroll
+  for (int h = 0; h < PER; ++h) {
+    uint32_t rem = kv + (uint32_t)h * a.lane_vecs;
+    live[h] = h == 0 || rem < a.kept_vecs;
+    int64_t doff = (int64_t)key * a.d_gstride, yoff = 0;
+    for (int d = 0; d < a.n_kept; ++d) {
+      uint32_t q, r;
+      a.ksize[d].divmod(rem, q, r);
+      rem = q;
+      const int64_t c = d == 0 ? (int64_t)r * VEC : (int64_t)r;
+      doff += c * a.kd_stride[d];
+      yoff += c * a.ky_stride[d];
+    }
+    dp[h] = reinterpret_cast<V*>(reinterpret_cast<T*>(a.dest) + doff);
+    yb[h] = reinterpret_cast<const T*>(a.y) + yoff;
+    if (live[h]) acc[h] = *dp[h];
   }
-  V* dp = reinterpret_cast<V*>(reinterpret_cast<T*>(a.dest) + doff);
-  const T* yb = reinterpret_cast<const T*>(a.y) + yoff;
   const bool y_unit = a.ky_stride[0] == 1 || VEC == 1;
   const bool y_once = a.y_gstride != 0;  // every update is read by one lane only
-  V acc = *dp;
   uint32_t j = i;
   for (;;) {
-    V upd[kAhead];
+    V upd[kAhead][PER];
     int cnt = 0;
 #pragma unroll
     for (int u = 0; u < kAhead; ++u) {
       if (cnt == u && j + u < a.n_index && ks[u] == key) {
-        const T* yp = yb + (int64_t)ps[u] * a.y_gstride;
-        if (y_unit) {
-          upd[u] = y_once ? nt_load(reinterpret_cast<const V*>(yp)) : *reinterpret_cast<const V*>(yp);
-        } else {  // y broadcast along the vectorised axis
-          const T yv = *yp;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) upd[u].v[e] = yv;
+        for (int h = 0; h < PER; ++h) {
+          if (!live[h]) continue;
+          const T* yp = yb[h] + (int64_t)ps[u] * a.y_gstride;
+          if (y_unit) {
+            upd[u][h] = y_once ? nt_load(reinterpret_cast<const V*>(yp)) : *reinterpret_cast<const V*>(yp);
+          } else {  // y broadcast along the vectorised axis
+            const T yv = *yp;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) upd[u][h].v[e] = yv;
+          }
         }
         cnt = u + 1;
       }
@@ -303,8 +317,12 @@ __global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, 
     for (int u = 0; u < kAhead; ++u) {
       if (u < cnt) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e)
-          acc.v[e] = a.reverse ? f(upd[u].v[e], acc.v[e], acc.v[e]) : f(acc.v[e], upd[u].v[e], upd[u].v[e]);
+        for (int h = 0; h < PER; ++h) {
+          if (!live[h]) continue;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e)
+            acc[h].v[e] = a.reverse ? f(upd[u][h].v[e], acc[h].v[e], acc[h].v[e]) : f(acc[h].v[e], upd[u][h].v[e], upd[u][h].v[e]);
+        }
       }
     }
     if (cnt < kAhead) break;
@@ -316,7 +334,9 @@ __global__ void __launch_bounds__(kBlock) accum_grouped_kernel(const BinaryF<T, 
       ps[u] = a.perm[at];
     }
   }
-  *dp = acc;
+#pragma unroll
+  for (int h = 0; h < PER; ++h)
+    if (live[h]) *dp[h] = acc[h];
 }
 
 // Recognises "one indexed axis in the destination, every other axis kept, y direct".
@@ -382,7 +402,8 @@ bool grouped_structure(const ct_dims& dd, const ct_dims& yd, const void* dest, c
   }
   if (kv >= (int64_t(1) << 31)) return false;
   a->kept_vecs = (uint32_t)kv;
-  a->kept_fd = FastDiv((uint32_t)kv);
+  a->lane_vecs = (uint32_t)kv;
+  a->lane_fd = FastDiv((uint32_t)kv);
   return ((int64_t)a->n_index * kv + kBlock - 1) / kBlock < (int64_t(1) << 31);
 }
 
@@ -606,11 +627,20 @@ int accum_run_with(hipStream_t s, BinaryF<T, OP> f, void* dest, const ct_dims* d
     g.dest = dest;
     g.y = y;
     g.reverse = reverse ? 1 : 0;
-    const dim3 grid((uint32_t)(((int64_t)g.n_index * g.kept_vecs + kBlock - 1) / kBlock));
     constexpr int VMAX = 16 / (int)sizeof(T);
+    // rows of at least a block of vectors: two vectors per lane, half a row apart (the accumulate
+    // of 65536 rows of 4 KiB: 95 us with one vector per lane, 88 with two, 130 with four)
+    constexpr int kPer = 2;
+    const bool several = vec_ok && g.kept_vecs >= 256;
+    if (several) {
+      g.lane_vecs = (g.kept_vecs + kPer - 1) / kPer;
+      g.lane_fd = FastDiv(g.lane_vecs);
+    }
+    const dim3 grid((uint32_t)(((int64_t)g.n_index * g.lane_vecs + kBlock - 1) / kBlock));
     note_kernel(vec_ok ? "accum_grouped_vec" : "accum_grouped");
-    if (vec_ok) hipLaunchKernelGGL((accum_grouped_kernel<T, OP, VMAX>), grid, dim3(kBlock), 0, s, f, g);
-    else hipLaunchKernelGGL((accum_grouped_kernel<T, OP, 1>), grid, dim3(kBlock), 0, s, f, g);
+    if (several) hipLaunchKernelGGL((accum_grouped_kernel<T, OP, VMAX, kPer>), grid, dim3(kBlock), 0, s, f, g);
+    else if (vec_ok) hipLaunchKernelGGL((accum_grouped_kernel<T, OP, VMAX, 1>), grid, dim3(kBlock), 0, s, f, g);
+    else hipLaunchKernelGGL((accum_grouped_kernel<T, OP, 1, 1>), grid, dim3(kBlock), 0, s, f, g);
     return after_launch(s);
   }
   EwOperand ops[3] = {{dest, dd, (int)sizeof(T), 0},
