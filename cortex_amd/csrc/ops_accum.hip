@@ -32,8 +32,8 @@
 // the remaining axes) applies that destination element's updates in increasing
 // position, which is increasing e: accum_grouped_kernel.  Bit-identical to the
 // serial loop for every op.  Up to 8192 index entries are ranked by one small
-// kernel; longer index tensors go through the vendor radix sort (hipCUB, a
-// stable LSD sort).  Shapes outside that pattern (reduced axes next to an
+// kernel; longer index tensors go through the vendor sort (rocPRIM's
+// radix_sort_pairs, stable, the positions fed from a counting iterator).  Shapes outside that pattern (reduced axes next to an
 // indexed one, an indexed y) keep the serial kernel.
 #include <algorithm>
 
@@ -41,7 +41,8 @@
 #include "functors.h"
 #include "ops.h"
 
-#include <hipcub/device/device_radix_sort.hpp>
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
 
 using namespace cthip;
 
@@ -233,11 +234,6 @@ __global__ void __launch_bounds__(kBlock) index_rank_kernel(const int32_t* __res
   }
 }
 
-__global__ void __launch_bounds__(kBlock) iota_kernel(int32_t* out, uint32_t n) {
-  const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
-  if (i < n) out[i] = (int32_t)i;
-}
-
 // One lane per (sorted index entry, PER vectors of the remaining axes, lane_vecs apart).  A lane
 // whose entry is not the first of its value leaves at once; the first walks the run of equal
 // values, fetching kAhead updates before it applies them in order.  PER = 2 puts twice the bytes
@@ -418,17 +414,16 @@ int sort_index(hipStream_t s, const int32_t* index, uint32_t n, const int32_t** 
     *perm = k + n;
     return CT_OK;
   }
+  // the positions come from a counting iterator, so no array of them has to be written first
   size_t temp_bytes = 0;
   const size_t arrays = ((size_t)n * 4 + 255) / 256 * 256;
-  CT_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, temp_bytes, index, (int32_t*)nullptr, (const int32_t*)nullptr,
-                                            (int32_t*)nullptr, (int)n, 0, 32, s));
-  if (int rc = stream_scratch(s, 3 * arrays + temp_bytes, &block, kScratchAccumA)) return rc;
+  const rocprim::counting_iterator<int32_t> positions(0);
+  CT_HIP(rocprim::radix_sort_pairs(nullptr, temp_bytes, index, (int32_t*)nullptr, positions, (int32_t*)nullptr, n, 0u, 32u, s));
+  if (int rc = stream_scratch(s, 2 * arrays + temp_bytes, &block, kScratchAccumA)) return rc;
   char* base = static_cast<char*>(block);
   int32_t* k = reinterpret_cast<int32_t*>(base);
   int32_t* p = reinterpret_cast<int32_t*>(base + arrays);
-  int32_t* iota = reinterpret_cast<int32_t*>(base + 2 * arrays);
-  hipLaunchKernelGGL(iota_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, s, iota, n);
-  CT_HIP(hipcub::DeviceRadixSort::SortPairs(base + 3 * arrays, temp_bytes, index, k, (const int32_t*)iota, p, (int)n, 0, 32, s));
+  CT_HIP(rocprim::radix_sort_pairs(base + 2 * arrays, temp_bytes, index, k, positions, p, n, 0u, 32u, s));
   *skey = k;
   *perm = p;
   return CT_OK;
