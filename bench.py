@@ -52,7 +52,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
-SECTIONS = ("headline", "others", "patterns", "adjacent")
+SECTIONS = ("headline", "others", "variants", "patterns", "adjacent")
 
 
 def log(msg: str) -> None:
@@ -324,6 +324,37 @@ def build_others(b: Bench):
     f64 = b.alloc(nv, "double")
     ops.append(Op("c4_i32_f64", "configs[4] assign! int32 -> float64 [64M]", 12 * nv,
                   lambda: s.assign(f64, dims([nv]), i32, dims([nv]), nv)))
+    return ops
+
+
+# ----------------------------------------------------------------------------- the constant and accumulate forms
+
+def build_variants(b: Bench):
+    """The TensorMath methods of the path that no BASELINE config names: assign-constant!, the accumulate (in place)
+    forms and the forms that take constants, each over 2^26 contiguous float32 (256 MiB per stream)."""
+    s = b.stream
+    n = 1 << 26
+    rng = np.random.default_rng(10)
+    x = b.upload(rng.standard_normal(n, dtype=np.float32))
+    y = b.upload(rng.standard_normal(n, dtype=np.float32))
+    d = b.alloc(n, "float")
+    flat = dims([n])
+    ops = [
+        Op("v_assign_constant", "assign-constant! float32 [2^26] (a write stream)", 4 * n,
+           lambda: s.assign_constant(d, flat, 1.5, n)),
+        Op("v_unary_accum", "unary-accum! :logistic float32 [2^26] (in place)", 8 * n,
+           lambda: s.unary_accum(d, flat, 1.0, "logistic", n)),
+        Op("v_binary_op_constant", "binary-op-constant! :* float32 [2^26], x * 0.5 with alpha 2", 8 * n,
+           lambda: s.binary_op_constant(d, flat, x, flat, 2.0, 0.5, n, "*", False)),
+        Op("v_binary_accum_constant", "binary-accum-constant! :max float32 [2^26] (in place, relu)", 8 * n,
+           lambda: s.binary_accum_constant(d, flat, 1.0, 0.0, n, "max", False)),
+        Op("v_binary_accum_same_shape", "binary-accum! :+ float32 [2^26] += y (destination is the max shape: no ordering needed)", 12 * n,
+           lambda: s.binary_accum(d, flat, 1.0, y, flat, 1.0, n, "+", False, False)),
+        Op("v_ternary_constant", "ternary-op! :select float32 [2^26], x >= 0 ? y : 0 (one constant)", 12 * n,
+           lambda: s.ternary_op_constant(d, flat, x, flat, 1.0, y, flat, 1.0, 0.0, n, "select", ["x", "z", "y"])),
+        Op("v_ternary_constant_constant", "ternary-op! :select float32 [2^26], x >= 0 ? 1 : 0 (two constants)", 8 * n,
+           lambda: s.ternary_op_constant_constant(d, flat, x, flat, 1.0, 0.0, 1.0, n, "select", ["x", "y", "z"])),
+    ]
     return ops
 
 
@@ -804,8 +835,8 @@ def main() -> int:
         "roofline": roof,
         "ops": ops_out,
     }
-    builders = {"others": build_others, "patterns": build_patterns, "adjacent": build_adjacent}
-    for name in ("others", "patterns", "adjacent"):
+    builders = {"others": build_others, "variants": build_variants, "patterns": build_patterns, "adjacent": build_adjacent}
+    for name in ("others", "variants", "patterns", "adjacent"):
         if name not in sections:
             continue
         log(f"timing section '{name}' ...")

@@ -232,4 +232,43 @@ template <class T> struct SelectRoutedF {
   }
 };
 
+// The constant forms with the condition in a tensor, which is what callers write (a mask
+// x >= 0 ? 1/p : 0, a clamp x >= 0 ? x : 0): the constants travel in the functor, so the call
+// has one or two inputs and runs on the kernels of a unary or binary op, and nothing is routed
+// per element.  Same value rules as SelectRoutedF.  PLAIN: float with every multiplier 1.
+//   SelectCCF          x >= 0 ? cz : cy
+//   SelectTCF<false>   x >= 0 ? cz : q      (q is the y argument)
+//   SelectTCF<true>    x >= 0 ? q  : cy     (q is the z argument)
+template <class T, bool PLAIN = false> struct SelectCCF {
+  static constexpr int NIN = 1;
+  using Out = T;
+  using In0 = T;
+  using In1 = T;
+  using In2 = T;
+  using A = typename acc_of<T>::type;
+  A xa;
+  T cy, cz;
+  __device__ __forceinline__ T operator()(T x, T, T) const {
+    const T vx = PLAIN ? x : jvm_cast<T>(w_mul(xa, (A)x));
+    return ((A)vx >= (A)0) ? cz : cy;
+  }
+};
+
+template <class T, bool Q_IS_Z, bool PLAIN = false> struct SelectTCF {
+  static constexpr int NIN = 2;
+  using Out = T;
+  using In0 = T;
+  using In1 = T;
+  using In2 = T;
+  using A = typename acc_of<T>::type;
+  A xa, qa;
+  T c;
+  __device__ __forceinline__ T operator()(T x, T q, T) const {
+    const T vx = PLAIN ? x : jvm_cast<T>(w_mul(xa, (A)x));
+    const T vq = PLAIN ? q : jvm_cast<T>(w_mul(qa, (A)q));
+    const bool pass = (A)vx >= (A)0;
+    return Q_IS_Z ? (pass ? vq : c) : (pass ? c : vq);
+  }
+};
+
 }  // namespace cthip

@@ -36,6 +36,56 @@ int routed_select(hipStream_t s, void* dest, const ct_dims* dd, const void* cons
   }
   return launch_elementwise(s, f, ops, n);
 }
+
+// Role of slot k: which of x (0), y (1), z (2) it is routed to.
+int role_of(const int8_t* arg_idx, int slot) {
+  for (int r = 0; r < 3; ++r)
+    if (arg_idx[r] == slot) return r;
+  return -1;
+}
+
+// x in the tensor, both results constant.  Returns false when the routing is another one.
+template <class T>
+bool select_cc(hipStream_t s, void* dest, const ct_dims* dd, const void* a, const ct_dims* ad, double a_alpha,
+               const double* constants, const int8_t* arg_idx, int64_t n, int* rc) {
+  using A = typename acc_of<T>::type;
+  if (role_of(arg_idx, 0) != 0) return false;
+  const T cy = jvm_cast<T>(constants[arg_idx[1] - 1]), cz = jvm_cast<T>(constants[arg_idx[2] - 1]);
+  const A xa = (A)jvm_cast<T>(a_alpha);
+  EwOperand ops[2] = {{dest, dd, (int)sizeof(T), 0}, {a, ad, (int)sizeof(T), 0}};
+  if constexpr (std::is_same<T, float>::value) {
+    if (xa == (A)1) {
+      *rc = launch_elementwise(s, SelectCCF<T, true>{xa, cy, cz}, ops, n);
+      return true;
+    }
+  }
+  *rc = launch_elementwise(s, SelectCCF<T>{xa, cy, cz}, ops, n);
+  return true;
+}
+
+// x in a tensor, one result in the other tensor, the other result constant.
+template <class T>
+bool select_tc(hipStream_t s, void* dest, const ct_dims* dd, const void* const* t, const ct_dims* const* td,
+               const double* alpha, double constant, const int8_t* arg_idx, int64_t n, int* rc) {
+  using A = typename acc_of<T>::type;
+  const int xs = arg_idx[0];  // the slot that holds x
+  if (xs > 1 || role_of(arg_idx, 2) == 0) return false;
+  const int qs = 1 - xs;      // the other tensor
+  const bool q_is_z = role_of(arg_idx, qs) == 2;
+  const A xa = (A)jvm_cast<T>(alpha[xs]), qa = (A)jvm_cast<T>(alpha[qs]);
+  const T c = jvm_cast<T>(constant);
+  EwOperand ops[3] = {{dest, dd, (int)sizeof(T), 0}, {t[xs], td[xs], (int)sizeof(T), 0}, {t[qs], td[qs], (int)sizeof(T), 0}};
+  if constexpr (std::is_same<T, float>::value) {
+    if (xa == (A)1 && qa == (A)1) {
+      *rc = q_is_z ? launch_elementwise(s, SelectTCF<T, true, true>{xa, qa, c}, ops, n)
+                   : launch_elementwise(s, SelectTCF<T, false, true>{xa, qa, c}, ops, n);
+      return true;
+    }
+  }
+  *rc = q_is_z ? launch_elementwise(s, SelectTCF<T, true>{xa, qa, c}, ops, n)
+               : launch_elementwise(s, SelectTCF<T, false>{xa, qa, c}, ops, n);
+  return true;
+}
 }  // namespace
 
 extern "C" {
@@ -75,7 +125,11 @@ int ct_ternary_op_constant(void* stream, void* dest, const ct_dims* dest_dims, c
   const ct_dims* td[2] = {a_dims, b_dims};
   const double al[2] = {a_alpha, b_alpha};
   const double cs[1] = {constant};
-  CT_DISPATCH_DTYPE(dtype, return routed_select<T>(static_cast<hipStream_t>(stream), dest, dest_dims, t, td, al, 2, cs, arg_idx, n));
+  CT_DISPATCH_DTYPE(dtype, {
+    int rc = CT_OK;
+    if (select_tc<T>(static_cast<hipStream_t>(stream), dest, dest_dims, t, td, al, constant, arg_idx, n, &rc)) return rc;
+    return routed_select<T>(static_cast<hipStream_t>(stream), dest, dest_dims, t, td, al, 2, cs, arg_idx, n);
+  });
   return CT_OK;
 }
 
@@ -89,7 +143,11 @@ int ct_ternary_op_constant_constant(void* stream, void* dest, const ct_dims* des
   const ct_dims* td[1] = {a_dims};
   const double al[1] = {a_alpha};
   const double cs[2] = {const_1, const_2};
-  CT_DISPATCH_DTYPE(dtype, return routed_select<T>(static_cast<hipStream_t>(stream), dest, dest_dims, t, td, al, 1, cs, arg_idx, n));
+  CT_DISPATCH_DTYPE(dtype, {
+    int rc = CT_OK;
+    if (select_cc<T>(static_cast<hipStream_t>(stream), dest, dest_dims, a, a_dims, a_alpha, cs, arg_idx, n, &rc)) return rc;
+    return routed_select<T>(static_cast<hipStream_t>(stream), dest, dest_dims, t, td, al, 1, cs, arg_idx, n);
+  });
   return CT_OK;
 }
 
