@@ -299,44 +299,57 @@ struct FlatArgs {
   char* ptr[kMaxOps];
 };
 
-template <class F, int VEC, int STREAM>
+// PER > 1 (a conversion between element widths, where the narrow side moves only 16 / ratio
+// bytes per lane and vector): a lane takes PER vectors, kBlock apart, and issues all of its
+// loads before the first store.
+template <class F, int VEC, int STREAM, int PER = 1>
 __global__ void __launch_bounds__(kBlock) ew_flat_kernel(const F f, const FlatArgs a) {
   using Out = typename F::Out;
   using In0 = typename F::In0;
   using In1 = typename F::In1;
   using In2 = typename F::In2;
   constexpr int NIN = F::NIN;
-  const uint64_t v = (uint64_t)xcd_grouped_unit(blockIdx.x, a.grouped_blocks) * (uint64_t)kBlock + threadIdx.x;
-  if (v >= a.total_vecs) return;
-  Vec<In0, VEC> x0;
-  Vec<In1, VEC> x1;
-  Vec<In2, VEC> x2;
-  if constexpr (NIN >= 1) {
-    const Vec<In0, VEC>* p = reinterpret_cast<const Vec<In0, VEC>*>(a.ptr[1]) + v;
-    if constexpr (STREAM >= 1) x0 = nt_load(p); else x0 = *p;
-  }
-  if constexpr (NIN >= 2) {
-    const Vec<In1, VEC>* p = reinterpret_cast<const Vec<In1, VEC>*>(a.ptr[2]) + v;
-    if constexpr (STREAM >= 1) x1 = nt_load(p); else x1 = *p;
-  }
-  if constexpr (NIN >= 3) {
-    const Vec<In2, VEC>* p = reinterpret_cast<const Vec<In2, VEC>*>(a.ptr[3]) + v;
-    if constexpr (STREAM >= 1) x2 = nt_load(p); else x2 = *p;
-  }
-  Vec<Out, VEC> r;
+  const uint64_t v0 = (uint64_t)xcd_grouped_unit(blockIdx.x, a.grouped_blocks) * (uint64_t)(kBlock * PER) + threadIdx.x;
+  if (v0 >= a.total_vecs) return;
+  Vec<In0, VEC> x0[PER];
+  Vec<In1, VEC> x1[PER];
+  Vec<In2, VEC> x2[PER];
 #pragma unroll
-  for (int i = 0; i < VEC; ++i) {
-    In0 p0{};
-    In1 p1{};
-    In2 p2{};
-    if constexpr (NIN >= 1) p0 = x0.v[i];
-    if constexpr (NIN >= 2) p1 = x1.v[i];
-    if constexpr (NIN >= 3) p2 = x2.v[i];
-    r.v[i] = f(p0, p1, p2);
+  for (int h = 0; h < PER; ++h) {
+    const uint64_t v = v0 + (uint64_t)h * kBlock;
+    if (h > 0 && v >= a.total_vecs) break;
+    if constexpr (NIN >= 1) {
+      const Vec<In0, VEC>* p = reinterpret_cast<const Vec<In0, VEC>*>(a.ptr[1]) + v;
+      if constexpr (STREAM >= 1) x0[h] = nt_load(p); else x0[h] = *p;
+    }
+    if constexpr (NIN >= 2) {
+      const Vec<In1, VEC>* p = reinterpret_cast<const Vec<In1, VEC>*>(a.ptr[2]) + v;
+      if constexpr (STREAM >= 1) x1[h] = nt_load(p); else x1[h] = *p;
+    }
+    if constexpr (NIN >= 3) {
+      const Vec<In2, VEC>* p = reinterpret_cast<const Vec<In2, VEC>*>(a.ptr[3]) + v;
+      if constexpr (STREAM >= 1) x2[h] = nt_load(p); else x2[h] = *p;
+    }
   }
-  Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(a.ptr[0]) + v;
-  if constexpr (STREAM == 2) nt_store(r, dp);
-  else *dp = r;
+#pragma unroll
+  for (int h = 0; h < PER; ++h) {
+    const uint64_t v = v0 + (uint64_t)h * kBlock;
+    if (h > 0 && v >= a.total_vecs) break;
+    Vec<Out, VEC> r;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      In0 p0{};
+      In1 p1{};
+      In2 p2{};
+      if constexpr (NIN >= 1) p0 = x0[h].v[i];
+      if constexpr (NIN >= 2) p1 = x1[h].v[i];
+      if constexpr (NIN >= 3) p2 = x2[h].v[i];
+      r.v[i] = f(p0, p1, p2);
+    }
+    Vec<Out, VEC>* dp = reinterpret_cast<Vec<Out, VEC>*>(a.ptr[0]) + v;
+    if constexpr (STREAM == 2) nt_store(r, dp);
+    else *dp = r;
+  }
 }
 
 // ------------------------------------------------------------------ TILE
@@ -881,6 +894,19 @@ template <class F, class = void> struct has_lace : std::false_type {};
 template <class F> struct has_lace<F, std::enable_if_t<F::kLace>> : std::true_type {};
 
 // Flat, every tensor operand unit-stride and no constants: the contiguous form.
+// Vectors per lane of the flat kernel: 1 when every operand has the same element width.  A
+// conversion moves only 16 / ratio bytes per lane and vector on its narrow side; a narrowing one
+// (wide loads, narrow stores) takes ratio vectors per lane, at most 4, a widening one 2.
+template <class F> constexpr int flat_vectors_per_lane() {
+  size_t mn = sizeof(typename F::Out), mx = sizeof(typename F::Out);
+  if (F::NIN >= 1) { mn = sizeof(typename F::In0) < mn ? sizeof(typename F::In0) : mn; mx = sizeof(typename F::In0) > mx ? sizeof(typename F::In0) : mx; }
+  if (F::NIN >= 2) { mn = sizeof(typename F::In1) < mn ? sizeof(typename F::In1) : mn; mx = sizeof(typename F::In1) > mx ? sizeof(typename F::In1) : mx; }
+  if (F::NIN >= 3) { mn = sizeof(typename F::In2) < mn ? sizeof(typename F::In2) : mn; mx = sizeof(typename F::In2) > mx ? sizeof(typename F::In2) : mx; }
+  const int ratio = (int)(mx / mn);
+  const int most = sizeof(typename F::Out) < mx ? 4 : 2;
+  return ratio < 1 ? 1 : (ratio > most ? most : ratio);
+}
+
 inline bool vec_is_flat(const VecArgs& a, int nin) {
   const uint32_t all = (2u << nin) - 1u;
   return a.n_outer == 0 && a.const_mask == 0 && (a.unit_mask & all) == all && !a.indexed;
@@ -896,9 +922,12 @@ inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& args) {
     fa.total_vecs = a.total_vecs;
     fa.grouped_blocks = xcd_grouped_blocks(grid.x);
     for (int k = 0; k < kMaxOps; ++k) fa.ptr[k] = a.ptr[k];
-    if (a.streaming == 2) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 2>), grid, dim3(kBlock), 0, s, f, fa);
-    else if (a.streaming) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 1>), grid, dim3(kBlock), 0, s, f, fa);
-    else hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 0>), grid, dim3(kBlock), 0, s, f, fa);
+    constexpr int kPer = flat_vectors_per_lane<F>();
+    const dim3 fgrid((uint32_t)((args.total_vecs + kBlock * kPer - 1) / (kBlock * kPer)));
+    fa.grouped_blocks = xcd_grouped_blocks(fgrid.x);
+    if (a.streaming == 2) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 2, kPer>), fgrid, dim3(kBlock), 0, s, f, fa);
+    else if (a.streaming) hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 1, kPer>), fgrid, dim3(kBlock), 0, s, f, fa);
+    else hipLaunchKernelGGL((ew_flat_kernel<F, VEC, 0, kPer>), fgrid, dim3(kBlock), 0, s, f, fa);
     return;
   }
   if (a.indexed) {
