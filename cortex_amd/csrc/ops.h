@@ -23,4 +23,9 @@ struct BinaryCall {
 
 int run_binary(hipStream_t s, int dtype, const BinaryCall& c);
 
+// output += unary-reduce!(input * input_alpha): the reduction's kernels with the addition (both
+// values widened, one rounding, as binary-op! :+ forms it) applied where they store their results.
+int unary_reduce_accumulate(hipStream_t stream, void* output, const ct_dims* output_dims, double input_alpha,
+                            const void* input, const ct_dims* input_dims, int op, int dtype);
+
 }  // namespace cthip

@@ -444,7 +444,7 @@ constexpr int64_t kStagedMinElements = 16384;  // of y
 // first, with .ystride the temporary's stride.  *handled is false (and nothing ran) when y
 // is itself broadcast along some axis.
 int stage_reduce(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, size_t elem_bytes, int rop,
-                 bool* handled, const void** result, StageAxis* ax, int* nax_out) {
+                 bool* handled, const void** result, StageAxis* ax, int* nax_out, bool add_into_dest = false) {
   *handled = false;
   int nax = 0;
   for (int d = 0; d < a.n_kept; ++d) {
@@ -501,6 +501,18 @@ int stage_reduce(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, s
     id.strides[nrest] = gstride;
     od.shape[nrest] = 1;
     od.strides[nrest] = 1;
+    bool last = add_into_dest;
+    for (int i = 0; i < nrest; ++i) last = last && rest[i].kept;
+    if (last) {
+      // nothing is left to reduce after this pass: it adds straight into the destination (the
+      // rest are the kept axes, addressed with the destination's strides), which saves the
+      // temporary and the launch of the final add
+      for (int i = 0; i < nrest; ++i) od.strides[i] = rest[i].dstride;
+      if (int rc = unary_reduce_accumulate(s, a.dest, &od, alpha, cur, &id, rop, dtype)) return rc;
+      *result = nullptr;
+      *nax_out = nrest;
+      return CT_OK;
+    }
     void* tmp = nullptr;
     if (int rc = stream_scratch(s, (size_t)n_out * elem_bytes, &tmp, slot)) return rc;
     if (int rc = ct_unary_reduce((void*)s, tmp, &od, alpha, cur, &id, rop, dtype)) return rc;
@@ -521,8 +533,12 @@ int accum_sum_staged(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtyp
   StageAxis ax[CT_MAX_DIMS];
   int nax = 0;
   const void* cur = nullptr;
-  if (int rc = stage_reduce(s, a, y_alpha, dtype, elem_bytes, CT_ROP_SUM, handled, &cur, ax, &nax)) return rc;
+  if (int rc = stage_reduce(s, a, y_alpha, dtype, elem_bytes, CT_ROP_SUM, handled, &cur, ax, &nax, true)) return rc;
   if (!*handled) return CT_OK;
+  if (!cur) {  // the last pass has added into the destination
+    note_kernel("accum_staged_sum");
+    return CT_OK;
+  }
   ct_dims dd, td;
   std::memset(&dd, 0, sizeof(dd));
   std::memset(&td, 0, sizeof(td));

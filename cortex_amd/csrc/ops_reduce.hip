@@ -36,6 +36,7 @@
 #include <mutex>
 
 #include "elementwise.h"
+#include "ops.h"
 
 using namespace cthip;
 
@@ -153,12 +154,25 @@ template <class T, int RK> struct RedKeyed {
 
 struct OutAddr {
   int32_t identity;  // output address == logical index
+  int32_t accumulate;  // the result is added to what the output holds (the last pass of a staged binary-accum! :+)
   int32_t nd;
   GenOperand op;
   int64_t rmax[CT_MAX_DIMS];
 };
 __device__ __forceinline__ int64_t out_address(const OutAddr& o, int64_t p) {
   return o.identity ? p : ref_address(o.op, o.nd, o.rmax, p);
+}
+
+// Stores output p.  With oa.accumulate the stored value is old + result, formed as binary-op! :+
+// forms it (both widened, one rounding): what a separate in-place add of the result would leave.
+template <class P>
+__device__ __forceinline__ void store_output(void* out, const OutAddr& oa, int64_t p, const typename P::Acc& acc, int64_t k) {
+  using T = typename P::Elem;
+  using W = typename acc_of<T>::type;
+  T* const o = reinterpret_cast<T*>(out) + out_address(oa, p);
+  T r = P::finish(acc, k);
+  if (oa.accumulate) r = jvm_cast<T>(w_add((W)*o, (W)r));
+  *o = r;
 }
 
 // Partial accumulators of a reduction split over several blocks:
@@ -255,7 +269,7 @@ __global__ void __launch_bounds__(BS) reduce_row_kernel(const RowArgs a, const t
     }
   }
   if (live && lane == 0) {
-    if (a.n_split == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+    if (a.n_split == 1) store_output<P>(a.out, a.oa, p, acc, a.k);
     else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc;
   }
 }
@@ -308,7 +322,7 @@ __global__ void __launch_bounds__(kBlock) reduce_row_small_kernel(const RowArgs 
     }
 #pragma unroll
     for (int m = TPR / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
-    if (p < a.n_out && lane == 0) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+    if (p < a.n_out && lane == 0) store_output<P>(a.out, a.oa, p, acc, a.k);
   }
 }
 
@@ -400,7 +414,7 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
 #pragma unroll
       for (int w = 0; w < WAVES - 1; ++w) acc[e] = P::combine(acc[e], lds[w][e * 64 + lane]);
       const int64_t p = pbase + (int64_t)(col + e) * a.u_pmul;
-      if (a.n_seg == 1) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc[e], a.k);
+      if (a.n_seg == 1) store_output<P>(a.out, a.oa, p, acc[e], a.k);
       else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc[e];
     }
   }
@@ -444,7 +458,7 @@ __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs 
   }
 #pragma unroll
   for (int m = 32; m >= PPW; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
-  if (live && sl == 0) reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+  if (live && sl == 0) store_output<P>(a.out, a.oa, p, acc, a.k);
 }
 
 template <class P>
@@ -484,7 +498,7 @@ __global__ void __launch_bounds__(kBlock) reduce_any_kernel(const AnyArgs a, con
   A acc = P::value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start)], alpha);
   for (int64_t i = 1; i < a.k; ++i)
     acc = P::combine(acc, P::value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start + i)], alpha));
-  reinterpret_cast<T*>(a.out)[out_address(a.oa, p)] = P::finish(acc, a.k);
+  store_output<P>(a.out, a.oa, p, acc, a.k);
 }
 
 // ------------------------------------------------------------------ host planning
@@ -533,6 +547,7 @@ struct PartialStore {
   void* fixed;         // nullptr: use the stream's scratch
   size_t fixed_bytes;
   const char* who;
+  bool accumulate = false;  // add the result to the output instead of replacing it
 };
 
 int partial_store(hipStream_t st, const PartialStore& ps, size_t bytes, void** out) {
@@ -565,6 +580,7 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
   if (int rc = reference_operand_own(od, &oa.op, oa.rmax, &out_rank)) return rc;
   oa.nd = out_rank;
   oa.identity = oa.op.mode == 0;
+  oa.accumulate = ps.accumulate ? 1 : 0;
 
   constexpr int VMAX = 16 / (int)sizeof(T);
   const RedShape rs = analyse(*id, k);
@@ -748,6 +764,15 @@ extern "C" int ct_unary_reduce(void* stream, void* output, const ct_dims* output
   if (int rc = check_dims(input_dims, "input")) return rc;
   const PartialStore ps{nullptr, 0, "ct_unary_reduce"};
   CT_DISPATCH_DTYPE(dtype, return reduce_dispatch<T>(static_cast<hipStream_t>(stream), ps, output, output_dims, input_alpha, input, input_dims, op));
+  return CT_OK;
+}
+
+// output += reduction, with the addition formed as binary-op! :+ forms it.  The last pass of
+// the staged binary-accum! :+ (ops_accum.hip).
+int cthip::unary_reduce_accumulate(hipStream_t stream, void* output, const ct_dims* output_dims, double input_alpha,
+                                   const void* input, const ct_dims* input_dims, int op, int dtype) {
+  const PartialStore ps{nullptr, 0, "binary-accum!", true};
+  CT_DISPATCH_DTYPE(dtype, return reduce_dispatch<T>(stream, ps, output, output_dims, input_alpha, input, input_dims, op));
   return CT_OK;
 }
 
