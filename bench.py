@@ -802,6 +802,9 @@ def main() -> int:
     roof["kernel"] = f"adam_kernel<float, 4, 1, true> ({adam.kernel})"
     roof["avg_launch_us"] = roof.pop("avg_call_us")
     roof["algorithmic_bytes_per_launch"] = roof.pop("algorithmic_bytes_per_call")
+    roof["note"] = ("four read streams and three write streams over four buffers: the bare mix with the arithmetic removed "
+                    "runs at 77-78 % of peak on this board against 84-89 % for a copy (sweep in DESIGN.md section 5; memory-side "
+                    "counters in profiles/memory_counters_adam_vs_copy.txt)")
     if b.traffic_note:
         roof["traffic_note"] = b.traffic_note
     c0 = ops_out[step_ops[-1].label]
