@@ -153,6 +153,51 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int ti
   return CT_OK;
 }
 
+// Rows that are no whole number of vectors, big operands dense over the whole call: see
+// ew_ragged_kernel.  False when the call has another shape.
+bool prepare_ragged(const Plan& plan, const EwOperand* ops, int vmax, RaggedArgs* a) {
+  const Canon& c = plan.canon;
+  if (c.any_index || c.nd < 2 || vmax < 2) return false;
+  const int64_t inner = c.size[0];
+  if (inner < vmax || inner % vmax == 0 || plan.n >= kLim31 || plan.n < 4096) return false;
+  std::memset(a, 0, sizeof(*a));
+  a->n = (uint32_t)plan.n;
+  a->inner_fd = FastDiv((uint32_t)inner);
+  a->n_outer = c.nd - 1;
+  for (int d = 1; d < c.nd; ++d) a->outer_fd[d - 1] = FastDiv((uint32_t)c.size[d]);
+  a->streaming = streaming_level(plan, ops) > 0 ? 1u : 0u;
+  for (int k = 0; k < plan.n_ops; ++k) {
+    a->ptr[k] = (char*)ops[k].ptr;
+    a->cbits[k] = ops[k].cbits;
+    if (!ops[k].ptr) {
+      if (k == 0) return false;
+      a->const_mask |= 1u << k;
+      continue;
+    }
+    if (c.stride[k][0] == 1) {
+      bool dense = true, periodic = true;
+      int64_t expect = inner;
+      for (int d = 1; d < c.nd; ++d) {
+        if (c.stride[k][d] != expect) dense = false;
+        if (c.stride[k][d] != 0) periodic = false;
+        expect *= c.size[d];
+      }
+      if (dense) {
+        if (((uintptr_t)ops[k].ptr % (uintptr_t)(vmax * ops[k].elem_size)) != 0) return false;
+        a->dense_mask |= 1u << k;
+      } else if (!periodic || k == 0) {
+        return false;
+      }
+    } else if (c.stride[k][0] == 0 && k != 0) {
+      a->scalar_mask |= 1u << k;
+      for (int d = 1; d < c.nd; ++d) a->outer_stride[k][d - 1] = c.stride[k][d];
+    } else {
+      return false;
+    }
+  }
+  return (a->dense_mask & 1u) != 0;
+}
+
 bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* a, int* n_short, int* ppt, uint32_t* grid) {
   const Canon& c = plan.canon;
   if (c.any_index || c.nd < 2 || c.stride[0][0] != 1) return false;

@@ -352,6 +352,110 @@ __global__ void __launch_bounds__(kBlock) ew_flat_kernel(const F f, const FlatAr
   }
 }
 
+// ------------------------------------------------------------------ RAGGED ROWS
+//
+// Rows that are no whole number of vectors (49 pixels of a 7 x 7 image under a per-channel bias,
+// ten classes under a per-row scale) used to run one element per lane.  When the big operands are
+// dense over the whole call, their flat offset is the element number whatever the row length, and
+// a lane can take an aligned 16-byte vector of them that may straddle the end of a row: at most
+// one row boundary falls into a vector (rows are at least a vector long).  The small operands are
+// fetched per element: a per-row value (constant along the row: any outer strides) for the row or
+// the next one, a row vector (the same row for every outer index) at its column.
+struct RaggedArgs {
+  uint32_t n;                 // elements; < 2^31
+  FastDiv inner_fd;           // row length
+  int32_t n_outer;
+  FastDiv outer_fd[CT_MAX_DIMS - 1];
+  uint32_t dense_mask;        // bit k: operand k is dense (offset = element number)
+  uint32_t scalar_mask;       // bit k: one value per row
+  uint32_t const_mask;        // bit k: a constant; every other input is a row vector
+  uint32_t streaming;
+  char* ptr[kMaxOps];
+  uint64_t cbits[kMaxOps];
+  int64_t outer_stride[kMaxOps][CT_MAX_DIMS - 1];
+};
+
+template <class F, int VEC, bool NT>
+__global__ void __launch_bounds__(kBlock) ew_ragged_kernel(const F f, const RaggedArgs a) {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+  const uint32_t e0 = (blockIdx.x * kBlock + threadIdx.x) * (uint32_t)VEC;
+  if (e0 >= a.n) return;
+  uint32_t row, col;
+  a.inner_fd.divmod(e0, row, col);
+  const uint32_t inner = a.inner_fd.d;
+  const uint32_t in_row = inner - col;  // elements of the vector that belong to `row`
+  const bool whole = e0 + VEC <= a.n;
+  // offset of a per-row operand for a row
+  auto row_offset = [&](int k, uint32_t r) {
+    int64_t off = 0;
+    for (int d = 0; d < a.n_outer; ++d) {
+      uint32_t q, c;
+      a.outer_fd[d].divmod(r, q, c);
+      r = q;
+      off += (int64_t)c * a.outer_stride[k][d];
+    }
+    return off;
+  };
+  auto fetch = [&](int k, auto* typed, auto& x) {
+    using T = typename std::remove_cv<typename std::remove_pointer<decltype(typed)>::type>::type;
+    const T* base = reinterpret_cast<const T*>(a.ptr[k]);
+    if ((a.const_mask >> k) & 1u) {
+      const T c = const_from_bits<T>(a.cbits[k]);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) x.v[i] = c;
+    } else if ((a.dense_mask >> k) & 1u) {
+      if (whole) {
+        const Vec<T, VEC>* vp = reinterpret_cast<const Vec<T, VEC>*>(base + e0);
+        if constexpr (NT) x = nt_load(vp); else x = *vp;
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = e0 + i < a.n ? base[e0 + i] : T{};
+      }
+    } else if ((a.scalar_mask >> k) & 1u) {
+      const T cur = base[row_offset(k, row)];
+      T next = cur;
+      if (in_row < (uint32_t)VEC && e0 + in_row < a.n) next = base[row_offset(k, row + 1)];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) x.v[i] = (uint32_t)i < in_row ? cur : next;
+    } else {  // a row vector
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const uint32_t c = (uint32_t)i < in_row ? col + i : (uint32_t)i - in_row;
+        x.v[i] = base[c];
+      }
+    }
+  };
+  Vec<In0, VEC> x0;
+  Vec<In1, VEC> x1;
+  Vec<In2, VEC> x2;
+  if constexpr (NIN >= 1) fetch(1, (const In0*)nullptr, x0);
+  if constexpr (NIN >= 2) fetch(2, (const In1*)nullptr, x1);
+  if constexpr (NIN >= 3) fetch(3, (const In2*)nullptr, x2);
+  Vec<Out, VEC> r;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    In0 p0{};
+    In1 p1{};
+    In2 p2{};
+    if constexpr (NIN >= 1) p0 = x0.v[i];
+    if constexpr (NIN >= 2) p1 = x1.v[i];
+    if constexpr (NIN >= 3) p2 = x2.v[i];
+    r.v[i] = f(p0, p1, p2);
+  }
+  Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + e0;
+  if (whole) {
+    *reinterpret_cast<Vec<Out, VEC>*>(dp) = r;
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+      if (e0 + i < a.n) dp[i] = r.v[i];
+  }
+}
+
 // ------------------------------------------------------------------ TILE
 
 struct TileArgs {
@@ -888,6 +992,7 @@ int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use
 // tile kernel took.  Returns false when it does not apply; otherwise fills the arguments, the
 // short axis' extent (2..kLaceMaxShort) and the vector width (vmax or 1) and the grid.
 bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* args, int* n_short, int* ppt, uint32_t* grid);
+bool prepare_ragged(const Plan& plan, const EwOperand* ops, int vmax, RaggedArgs* args);
 
 // Functors that the lace kernel is built for declare `static constexpr bool kLace = true`.
 template <class F, class = void> struct has_lace : std::false_type {};
@@ -1017,6 +1122,16 @@ int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t 
     int vec = 1;
     bool has_tail = false;
     if (int rc = prepare_vec(plan, ops, VMAX, &main_args, &vec, &tail_args, &has_tail)) return rc;
+    if constexpr (VMAX > 1) {
+      RaggedArgs ra;
+      if (vec == 1 && prepare_ragged(plan, ops, VMAX, &ra)) {
+        note_kernel("ragged");
+        const dim3 grid((uint32_t)(((int64_t)ra.n + (int64_t)VMAX * kBlock - 1) / ((int64_t)VMAX * kBlock)));
+        if (ra.streaming) hipLaunchKernelGGL((ew_ragged_kernel<F, VMAX, true>), grid, dim3(kBlock), 0, s, f, ra);
+        else hipLaunchKernelGGL((ew_ragged_kernel<F, VMAX, false>), grid, dim3(kBlock), 0, s, f, ra);
+        return after_launch(s);
+      }
+    }
     if (vec == VMAX && VMAX > 1) {
       note_kernel("vec");
       launch_vec<F, VMAX>(s, f, main_args);

@@ -431,7 +431,6 @@ constexpr int kFinishLoads = 4;
 
 template <class P, int LPO>
 __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs a) {
-  using T = typename P::Elem;
   using A = typename P::Acc;
   constexpr int PPW = 64 / LPO;  // outputs per wave
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
