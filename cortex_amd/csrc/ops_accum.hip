@@ -437,6 +437,29 @@ struct StageAxis {
 
 constexpr int64_t kStagedMinUpdates = 64;     // per destination element
 constexpr int64_t kStagedMinElements = 16384;  // of y
+constexpr int64_t kStagedShortGroup = 64;      // a first pass over rows shorter than this is avoided
+
+// Merges neighbouring kept axes of a pass (all but the last, reduced one) that chain in the input
+// and in the output alike, so that the reduction sees [512, 49, 256] rather than [512, 7, 7, 256].
+void merge_chained(ct_dims* id, ct_dims* od) {
+  const int last = id->ndim - 1;
+  int w = 0;
+  for (int i = 0; i < last; ++i) {
+    if (w > 0 && id->strides[w - 1] == id->strides[i] * id->shape[i] && od->strides[w - 1] == od->strides[i] * od->shape[i]) {
+      id->shape[w - 1] *= id->shape[i];
+      od->shape[w - 1] = id->shape[w - 1];
+      id->strides[w - 1] = id->strides[i];
+      od->strides[w - 1] = od->strides[i];
+    } else {
+      id->shape[w] = id->shape[i]; id->strides[w] = id->strides[i];
+      od->shape[w] = od->shape[i]; od->strides[w] = od->strides[i];
+      ++w;
+    }
+  }
+  id->shape[w] = id->shape[last]; id->strides[w] = id->strides[last];
+  od->shape[w] = od->shape[last]; od->strides[w] = od->strides[last];
+  id->ndim = od->ndim = w + 1;
+}
 
 // Reduces y * y_alpha over the broadcast axes with unary-reduce! `rop`, innermost group of
 // axes first, through the stream's two accumulate scratch blocks.  On success *result is the
@@ -470,7 +493,7 @@ int stage_reduce(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, s
       if (!ax[i].kept) { g = i; break; }
     if (g < 0) break;
     int64_t gsize = ax[g].size;
-    const int64_t gstride = ax[g].ystride;
+    int64_t gstride = ax[g].ystride;
     bool taken[CT_MAX_DIMS] = {false};
     taken[g] = true;
     for (int i = g - 1; i >= 0; --i) {
@@ -478,6 +501,21 @@ int stage_reduce(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, s
       if (ax[i].ystride != gstride * gsize) break;
       gsize *= ax[i].size;
       taken[i] = true;
+    }
+    // A short innermost group (the 49 pixels of a 7 x 7 image under a per-channel sum) makes a
+    // poor first pass: rows of a few elements, seldom a whole number of vectors.  When a slower
+    // broadcast axis is left (the batch), that one goes first instead: a reduction down the
+    // columns of long contiguous rows, after which the short rows are a small tensor.
+    if (gsize < kStagedShortGroup) {
+      int outer = -1;
+      for (int i = 0; i < nax; ++i)
+        if (!ax[i].kept && !taken[i]) { outer = i; break; }
+      if (outer >= 0) {
+        for (int i = 0; i < nax; ++i) taken[i] = false;
+        taken[outer] = true;
+        gsize = ax[outer].size;
+        gstride = ax[outer].ystride;
+      }
     }
     ct_dims id, od;
     std::memset(&id, 0, sizeof(id));
@@ -508,6 +546,7 @@ int stage_reduce(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, s
       // rest are the kept axes, addressed with the destination's strides), which saves the
       // temporary and the launch of the final add
       for (int i = 0; i < nrest; ++i) od.strides[i] = rest[i].dstride;
+      merge_chained(&id, &od);
       if (int rc = unary_reduce_accumulate(s, a.dest, &od, alpha, cur, &id, rop, dtype)) return rc;
       *result = nullptr;
       *nax_out = nrest;
@@ -515,6 +554,7 @@ int stage_reduce(hipStream_t s, const OwnerArgs& a, double y_alpha, int dtype, s
     }
     void* tmp = nullptr;
     if (int rc = stream_scratch(s, (size_t)n_out * elem_bytes, &tmp, slot)) return rc;
+    merge_chained(&id, &od);
     if (int rc = ct_unary_reduce((void*)s, tmp, &od, alpha, cur, &id, rop, dtype)) return rc;
     cur = tmp;
     alpha = 1.0;

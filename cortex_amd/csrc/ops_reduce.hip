@@ -531,8 +531,14 @@ RedShape analyse(const ct_dims& in, int64_t k) {
     else { r.fast = false; return r; }
   }
   r.rstride = have ? rstr : 1;
+  // kept axes, slowest first; neighbours that chain ([512, 7, 7] with strides [49, 7, 1]) are one axis
   for (int i = 0; i < j; ++i) {
     if (in.shape[i] == 1) continue;
+    if (r.n_kept > 0 && r.kstride[r.n_kept - 1] == in.strides[i] * in.shape[i]) {
+      r.ksize[r.n_kept - 1] *= in.shape[i];
+      r.kstride[r.n_kept - 1] = in.strides[i];
+      continue;
+    }
     r.ksize[r.n_kept] = in.shape[i];
     r.kstride[r.n_kept] = in.strides[i];
     ++r.n_kept;

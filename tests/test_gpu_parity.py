@@ -231,6 +231,18 @@ def test_unary_ops_all_dtypes(P, code, op):
     compare(xb, f"accum {op} ({k})", tol=tol)
 
 
+def test_reduce_view_with_chained_kept_axes_stays_on_the_column_kernel(P):
+    """[channels, 7, 7, batch] with the batch axis slowest in memory: the three kept axes chain into one."""
+    rng = np.random.default_rng(61)
+    batch, channels = 64, 24
+    x = P.buf((rng.random(batch * channels * 49) + 0.5).astype(np.float32))
+    out = P.buf(np.zeros(channels * 49, np.float32))
+    k = P.run(H.unary_reduce, View(out, [channels, 7, 7, 1]), 1.0,
+              View(x, [channels, 7, 7, batch], [49, 7, 1, channels * 49]), "sum")
+    assert k.startswith("reduce_col"), k
+    compare(out, f"sum over the batch axis ({k})", tol=REL_TOL)
+
+
 def test_float_tanh_dense_sweep(P):
     """unary-op! :tanh on float tensors runs a single-precision form of its own: a dense sweep of its
     argument range (the polynomial below 0.4, the seam, the exponential form up to saturation, tiny and
@@ -372,6 +384,7 @@ STAGED_LAYOUTS = [
     ([33, 1], None, [33, 900], [1, 33]),                 # y is a transposed view
     ([4, 1, 5], None, [4, 1000, 5], None),               # reduced axis in the middle
     ([500, 40], [0, 1], [500, 40], None),                # a destination axis of stride 0 is a broadcast axis
+    ([12, 1, 1], None, [40, 12, 7, 7], None),            # short innermost group: the batch axis is reduced first
 ]
 
 
