@@ -420,6 +420,47 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
   }
 }
 
+// Short rows stored back to back (a dense [rows, k] block of at most 128 bytes per row) whose
+// length is no whole number of 16-byte vectors, ten classes say.  A block stages its 256 rows, one
+// contiguous stretch of memory, through LDS with 128-bit accesses; one lane then owns a row in LDS
+// and accumulates it from the first element to the last, the reference's order.  (With a lane
+// group per row and 4-byte loads the same rows reach a sixth of the memory rate.)
+struct ShortRowsArgs {
+  const void* in;
+  void* out;
+  int64_t n_out;
+  uint32_t k;
+  OutAddr oa;
+};
+
+template <class P>
+__global__ void __launch_bounds__(kBlock) reduce_short_rows_kernel(const ShortRowsArgs a, const typename P::Alpha alpha) {
+  using T = typename P::Elem;
+  using A = typename P::Acc;
+  constexpr int VEC = 16 / (int)sizeof(T);
+  using V = Vec<T, VEC>;
+  extern __shared__ __align__(16) char smem[];
+  T* tile = reinterpret_cast<T*>(smem);
+  const uint32_t k = a.k;
+  const int64_t row0 = (int64_t)blockIdx.x * kBlock;
+  const uint32_t n_rows = (uint32_t)(a.n_out - row0 < kBlock ? a.n_out - row0 : kBlock);
+  const uint32_t count = n_rows * k;
+  const T* in = reinterpret_cast<const T*>(a.in) + row0 * k;
+  // a block's stretch starts on the 16-byte grid whenever the tensor does (256 * k elements per block)
+  const uint32_t n_vec = count / VEC;
+  for (uint32_t v = threadIdx.x; v < n_vec; v += kBlock)
+    reinterpret_cast<V*>(tile)[v] = nt_load(reinterpret_cast<const V*>(in) + v);
+  for (uint32_t e = n_vec * VEC + threadIdx.x; e < count; e += kBlock) tile[e] = in[e];
+  __syncthreads();
+  if (threadIdx.x < n_rows) {
+    const T* row = tile + threadIdx.x * k;
+    A acc = P::identity();
+    for (uint32_t j = 0; j < k; ++j) acc = P::combine(acc, P::value(row[j], alpha));
+    store_output<P>(a.out, a.oa, row0 + threadIdx.x, acc, (int64_t)k);
+  }
+}
+
+
 // Combines the partial accumulators of a split reduction.  The launch is small
 // (a few KiB to a MiB of partials) and sits on the critical path between two
 // calls, so it is shaped for latency: LPO lanes share one output, every lane
@@ -641,7 +682,15 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
   else if (nv <= 128) CT_ROW_SMALL(VEC, 64, 2);   \
   else CT_ROW_SMALL(VEC, 64, 4)
     const int64_t nv = vec_ok ? k / VMAX : k;
-    if (split == 1 && nv <= 256) {
+    if (VMAX > 1 && !vec_ok && k % VMAX != 0 && k * (int64_t)sizeof(T) <= 128 && k >= 2 && rs.n_kept == 1 &&
+        rs.kstride[0] == k && aligned_for<T>(in, VMAX) && n_out >= 1024) {
+      ShortRowsArgs sa;
+      std::memset(&sa, 0, sizeof(sa));
+      sa.in = in; sa.out = out; sa.n_out = n_out; sa.k = (uint32_t)k; sa.oa = oa;
+      note_kernel("reduce_short_rows");
+      hipLaunchKernelGGL((reduce_short_rows_kernel<P>), dim3((uint32_t)((n_out + kBlock - 1) / kBlock)), dim3(kBlock),
+                         (size_t)kBlock * k * sizeof(T), st, sa, alpha);
+    } else if (split == 1 && nv <= 256) {
       note_kernel(vec_ok ? "reduce_row_small_vec" : "reduce_row_small");
       if (vec_ok) { CT_ROW_SMALL_SHAPES(VMAX); } else { CT_ROW_SMALL_SHAPES(1); }
     } else if (vec_ok && row_bytes >= 16384) {

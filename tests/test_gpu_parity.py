@@ -243,6 +243,29 @@ def test_reduce_view_with_chained_kept_axes_stays_on_the_column_kernel(P):
     compare(out, f"sum over the batch axis ({k})", tol=REL_TOL)
 
 
+@pytest.mark.parametrize("code", H.ALL_DTYPES)
+def test_reduce_short_ragged_rows(P, code):
+    """Dense rows of ten (seven, thirty-one ...) elements, no whole number of vectors: staged through LDS,
+    one lane per row, accumulated first element to last as the reference does."""
+    rng = np.random.default_rng(62)
+    vmax = 16 // NP[code]().itemsize
+    for rows, k in ((5000, 10), (1024, 7), (3001, 31), (1500, 3), (2048, 9)):
+        if k % vmax == 0 or k * NP[code]().itemsize > 128:
+            continue
+        x = P.buf(values(rng, code, rows * k, -50, 50))
+        if code in FLOATS:
+            x.init[5 * k + 1] = np.nan
+            x.init[7 * k: 8 * k] = 0.0
+            x.init[7 * k + 2] = -0.0
+            x = P.buf(x.init)
+        out = P.buf(np.zeros(rows, NP[code]))
+        for op, alpha in (("sum", 1.0), ("max", 1.0), ("min", 1.0), ("mean", 1.0), ("magnitude", 0.5), ("magnitude-squared", 1.0)):
+            kname = P.run(H.unary_reduce, View(out, [rows, 1]), alpha, View(x, [rows, k]), op)
+            assert kname == "reduce_short_rows", (kname, rows, k)
+            compare(out, f"{op} rows of {k} ({kname})", tol=None if (code not in FLOATS or op in ("max", "min")) else
+                    (REL_TOL if code == capi.F32 else REL_TOL_F64))
+
+
 def test_float_tanh_dense_sweep(P):
     """unary-op! :tanh on float tensors runs a single-precision form of its own: a dense sweep of its
     argument range (the polynomial below 0.4, the seam, the exponential form up to saturation, tiny and
