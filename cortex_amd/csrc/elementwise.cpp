@@ -153,6 +153,29 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int ti
   return CT_OK;
 }
 
+// Vectors that start anywhere (ew_vecu_kernel): rows of at least one vector whose starts or
+// lengths keep them off the 16-byte grid.  False for small calls, indexed axes and rows shorter
+// than a vector, which stay with one element per lane.
+bool prepare_vecu(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* a, uint32_t* inner_elems) {
+  const Canon& c = plan.canon;
+  if (c.any_index || vmax < 2 || plan.n < 4096) return false;
+  const int64_t inner = c.size[0];
+  if (inner < vmax || inner >= kLim31) return false;
+  bool any_unit = false;
+  for (int k = 0; k < plan.n_ops; ++k) any_unit = any_unit || (ops[k].ptr && c.stride[k][0] == 1);
+  if (!any_unit) return false;
+  int64_t rows = 1;
+  for (int d = 1; d < c.nd; ++d) rows *= c.size[d];
+  const int64_t inner_vecs = (inner + vmax - 1) / vmax;
+  if (inner_vecs * rows >= kLim31) return false;
+  common_vec(plan, ops, a);
+  a->inner_vecs = (uint32_t)inner_vecs;
+  a->inner_fd = FastDiv((uint32_t)inner_vecs);
+  a->total_vecs = (uint64_t)(inner_vecs * rows);
+  *inner_elems = (uint32_t)inner;
+  return true;
+}
+
 // Rows that are no whole number of vectors, big operands dense over the whole call: see
 // ew_ragged_kernel.  False when the call has another shape.
 bool prepare_ragged(const Plan& plan, const EwOperand* ops, int vmax, RaggedArgs* a) {

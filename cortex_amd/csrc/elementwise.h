@@ -352,6 +352,91 @@ __global__ void __launch_bounds__(kBlock) ew_flat_kernel(const F f, const FlatAr
   }
 }
 
+// ------------------------------------------------------------------ UNALIGNED VECTORS
+//
+// Rows whose starts are not on the 16-byte grid (a [rows, 999] block of a pitch-1024 matrix
+// copied to a contiguous one, a sub-buffer that starts at an odd element) or whose length is no
+// whole number of vectors used to run one element per lane.  Global memory accesses only need
+// the element's alignment, so a lane takes a vector that starts anywhere; the last lane of a row
+// takes what is left of the row element by element.  a.inner_fd counts vectors per row, rounded up.
+template <class T, int N> struct alignas(sizeof(T)) UVec { T v[N]; };
+
+template <class F, int VEC>
+__global__ void __launch_bounds__(kBlock) ew_vecu_kernel(const F f, const VecArgs a, const uint32_t inner_elems) {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  constexpr int NIN = F::NIN;
+  const uint64_t v = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (v >= a.total_vecs) return;
+  uint32_t row, cv;
+  a.inner_fd.divmod((uint32_t)v, row, cv);
+  const uint32_t col = cv * (uint32_t)VEC;
+  const uint32_t left = inner_elems - col;
+  const bool whole = left >= (uint32_t)VEC;
+  int64_t off[kMaxOps] = {0, 0, 0, 0};
+  {
+    uint32_t r = row;
+    for (int d = 0; d < a.n_outer; ++d) {
+      uint32_t q, c;
+      (d < 2 ? a.outer_fd01[d] : a.outer_fd_hi[d - 2]).divmod(r, q, c);
+      r = q;
+#pragma unroll
+      for (int k = 0; k <= NIN; ++k) off[k] += (int64_t)c * (d < 2 ? a.outer_stride01[k][d] : a.outer_stride_hi[k][d - 2]);
+    }
+  }
+  auto fetch = [&](int k, auto* typed, auto& x) {
+    using T = typename std::remove_cv<typename std::remove_pointer<decltype(typed)>::type>::type;
+    if ((a.const_mask >> k) & 1u) {
+      const T c = const_from_bits<T>(a.cbits[k]);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) x.v[i] = c;
+      return;
+    }
+    const T* sp = reinterpret_cast<const T*>(a.ptr[k]) + off[k];
+    if ((a.unit_mask >> k) & 1u) {
+      if (whole) {
+        const UVec<T, VEC> u = *reinterpret_cast<const UVec<T, VEC>*>(sp + col);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = u.v[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = (uint32_t)i < left ? sp[col + i] : T{};
+      }
+    } else {
+      const T c = *sp;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) x.v[i] = c;
+    }
+  };
+  Vec<In0, VEC> x0;
+  Vec<In1, VEC> x1;
+  Vec<In2, VEC> x2;
+  if constexpr (NIN >= 1) fetch(1, (const In0*)nullptr, x0);
+  if constexpr (NIN >= 2) fetch(2, (const In1*)nullptr, x1);
+  if constexpr (NIN >= 3) fetch(3, (const In2*)nullptr, x2);
+  UVec<Out, VEC> r;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    In0 p0{};
+    In1 p1{};
+    In2 p2{};
+    if constexpr (NIN >= 1) p0 = x0.v[i];
+    if constexpr (NIN >= 2) p1 = x1.v[i];
+    if constexpr (NIN >= 3) p2 = x2.v[i];
+    r.v[i] = f(p0, p1, p2);
+  }
+  Out* dp = reinterpret_cast<Out*>(a.ptr[0]) + off[0] + col;
+  if (whole) {
+    *reinterpret_cast<UVec<Out, VEC>*>(dp) = r;
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+      if ((uint32_t)i < left) dp[i] = r.v[i];
+  }
+}
+
 // ------------------------------------------------------------------ RAGGED ROWS
 //
 // Rows that are no whole number of vectors (49 pixels of a 7 x 7 image under a per-channel bias,
@@ -993,6 +1078,7 @@ int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use
 // short axis' extent (2..kLaceMaxShort) and the vector width (vmax or 1) and the grid.
 bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* args, int* n_short, int* ppt, uint32_t* grid);
 bool prepare_ragged(const Plan& plan, const EwOperand* ops, int vmax, RaggedArgs* args);
+bool prepare_vecu(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* args, uint32_t* inner_elems);
 
 // Functors that the lace kernel is built for declare `static constexpr bool kLace = true`.
 template <class F, class = void> struct has_lace : std::false_type {};
@@ -1129,6 +1215,16 @@ int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t 
         const dim3 grid((uint32_t)(((int64_t)ra.n + (int64_t)VMAX * kBlock - 1) / ((int64_t)VMAX * kBlock)));
         if (ra.streaming) hipLaunchKernelGGL((ew_ragged_kernel<F, VMAX, true>), grid, dim3(kBlock), 0, s, f, ra);
         else hipLaunchKernelGGL((ew_ragged_kernel<F, VMAX, false>), grid, dim3(kBlock), 0, s, f, ra);
+        return after_launch(s);
+      }
+    }
+    if constexpr (VMAX > 1) {
+      VecArgs ua;
+      uint32_t inner_elems = 0;
+      if (vec == 1 && prepare_vecu(plan, ops, VMAX, &ua, &inner_elems)) {
+        note_kernel("vecu");
+        hipLaunchKernelGGL((ew_vecu_kernel<F, VMAX>), dim3((uint32_t)((ua.total_vecs + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+                           f, ua, inner_elems);
         return after_launch(s);
       }
     }

@@ -93,3 +93,46 @@ def test_three_outer_axes_and_mixed_widths(P):
     pix = P.buf(rng.integers(0, 256, n).astype(np.uint8))
     k = P.run(H.assign, View(d, shape), View(pix, shape))
     exact(d, f"assign u8 -> f32 {shape} ({k})")
+
+
+@pytest.mark.parametrize("code", [capi.F32, capi.F64, capi.I16, capi.I8, capi.I64])
+def test_rows_off_the_vector_grid(P, code):
+    """Odd-width blocks of a pitched matrix (ct/submatrix, src/cortex/tensor.clj:490-513), sub-buffers that start at
+    an odd element, rows one element longer than a vector: vectors that start anywhere (ew_vecu_kernel)."""
+    rng = np.random.default_rng(94)
+    vmax = 16 // NP[code]().itemsize
+    for rows, width, pitch, offset in ((70, 999, 1024, 0), (129, 67, 80, 3), (4100, vmax + 1, vmax + 3, 1), (33, 200, 200, 5)):
+        if width < vmax:
+            continue
+        n = rows * width
+        src = P.buf(values(rng, code, rows * pitch + offset + 8))
+        other = P.buf(values(rng, code, rows * pitch + offset + 8))
+        dense = P.buf(np.zeros(n, NP[code]))
+        pitched = P.buf(values(rng, code, rows * pitch + offset + 8))
+        sub = lambda b: View(b, [rows, width], [pitch, 1], offset=offset)
+        k = P.run(H.assign, View(dense, [rows, width]), sub(src))
+        exact(dense, f"copy out of a pitched block [{rows},{width}]/{pitch}+{offset} ({k})")
+        if n >= 4096 and (width % vmax or pitch % vmax or offset % vmax):
+            assert k == "vecu", (k, rows, width, pitch, offset)
+        k = P.run(H.binary_op, sub(pitched), sub(src), 1.0, sub(other), -1.0, "+")
+        exact(pitched, f"pitched block minus pitched block ({k})")
+        k = P.run(H.binary_op, sub(pitched), sub(pitched), 1.0, View(dense, [rows, width]), 2.0, "max")
+        exact(pitched, f"in place against a dense block ({k})")
+        per_row = P.buf(values(rng, code, rows))
+        k = P.run(H.binary_op, sub(pitched), sub(src), 1.0, View(per_row, [rows, 1]), 1.0, "*")
+        exact(pitched, f"pitched block times a per-row value ({k})")
+        k = P.run(H.binary_op_constant, sub(pitched), sub(src), 1.0, 3.0, "+")
+        exact(pitched, f"pitched block plus a constant ({k})")
+
+
+def test_conversion_off_the_vector_grid(P):
+    rng = np.random.default_rng(95)
+    rows, width, pitch = 100, 333, 340
+    pix = P.buf(rng.integers(0, 256, rows * pitch + 4).astype(np.uint8))
+    out = P.buf(np.zeros(rows * width, np.float32))
+    k = P.run(H.assign, View(out, [rows, width]), View(pix, [rows, width], [pitch, 1], offset=1))
+    exact(out, f"u8 block to float ({k})")
+    assert k == "vecu", k
+    back = P.buf(np.zeros(rows * pitch + 4, np.int16))
+    k = P.run(H.assign, View(back, [rows, width], [pitch, 1], offset=3), View(out, [rows, width]))
+    exact(back, f"float to a pitched short block ({k})")
