@@ -1134,7 +1134,10 @@ inline void launch_vec_once(hipStream_t s, const F& f, const VecArgs& args) {
     hipLaunchKernelGGL((ew_vec_kernel<F, VEC, 0, -1, true, kPer>), grid_per, dim3(kBlock), 0, s, f, a);
     return;
   }
-  if (VEC > 1) {
+  // The compile-time operand kinds are worth a few percent of memory bandwidth; integer tensors,
+  // whose arithmetic sets their pace, keep the one general form (an eighth of the library's size
+  // was specialisations of integer functors).
+  if constexpr (VEC > 1 && std::is_floating_point<typename F::Out>::value) {
     // the operand kinds of this call, in vec_kinds' encoding
     int kinds = 0;
     for (int k = 1; k <= F::NIN; ++k) {
