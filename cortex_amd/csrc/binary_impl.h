@@ -14,7 +14,7 @@ template <class T> int binary_dispatch(hipStream_t s, const BinaryCall& c);
 namespace binary_detail {
 template <class T, int OP>
 int binary_run(hipStream_t s, const BinaryCall& c) {
-  using A = typename acc_of<T>::type;
+  using A = typename ew_acc_of<T>::type;
   // A scalar side has had its alpha folded in by the caller; its multiplier is 1.
   const A xa = c.x ? (A)jvm_cast<T>(c.x_alpha) : (A)1;
   const A ya = c.y ? (A)jvm_cast<T>(c.y_alpha) : (A)1;

@@ -82,6 +82,17 @@ template <class T> struct acc_of {
   using type = typename std::conditional<std::is_floating_point<T>::value, double, int64_t>::type;
 };
 
+// The accumulator of the elementwise functors.  For byte and short tensors an int does what the
+// reference's long does: every operand and multiplier has been cast to T first, so products of
+// two fit in 32 bits exactly (what max, min, the comparisons and the division see), and sums,
+// differences and products of those are truncated to T at the store, which gives the same bits
+// from arithmetic modulo 2^32 as from arithmetic modulo 2^64.  (Reductions keep the long: a mean
+// divides the untruncated sum.)
+template <class T> struct ew_acc_of {
+  using type = typename std::conditional<std::is_floating_point<T>::value, double,
+                                         typename std::conditional<(sizeof(T) <= 2), int32_t, int64_t>::type>::type;
+};
+
 // Runs `body` with T bound to the C type of datatype `dt`.
 #define CT_DISPATCH_DTYPE(dt, ...)                                              \
   switch (dt) {                                                                 \
@@ -120,6 +131,10 @@ template <class T> CT_HD T jvm_cast(int64_t v) {
   if constexpr (std::is_floating_point<T>::value) return (T)v;
   else return (T)(uint64_t)v;
 }
+template <class T> CT_HD T jvm_cast(int32_t v) {
+  if constexpr (std::is_floating_point<T>::value) return (T)v;
+  else return (T)(uint32_t)v;
+}
 // Result of a double computation stored into T; byte and short go through int.
 template <class T> CT_HD T jvm_cast(double v) {
   if constexpr (std::is_same<T, double>::value) return v;
@@ -138,6 +153,10 @@ CT_HD int64_t w_mul(int64_t a, int64_t b) { return (int64_t)((uint64_t)a * (uint
 CT_HD int64_t w_add(int64_t a, int64_t b) { return (int64_t)((uint64_t)a + (uint64_t)b); }
 CT_HD int64_t w_sub(int64_t a, int64_t b) { return (int64_t)((uint64_t)a - (uint64_t)b); }
 CT_HD int64_t w_neg(int64_t a) { return (int64_t)(0ull - (uint64_t)a); }
+CT_HD int32_t w_mul(int32_t a, int32_t b) { return (int32_t)((uint32_t)a * (uint32_t)b); }
+CT_HD int32_t w_add(int32_t a, int32_t b) { return (int32_t)((uint32_t)a + (uint32_t)b); }
+CT_HD int32_t w_sub(int32_t a, int32_t b) { return (int32_t)((uint32_t)a - (uint32_t)b); }
+CT_HD int32_t w_neg(int32_t a) { return (int32_t)(0u - (uint32_t)a); }
 CT_HD double w_mul(double a, double b) { return a * b; }
 CT_HD double w_add(double a, double b) { return a + b; }
 CT_HD double w_sub(double a, double b) { return a - b; }
@@ -152,6 +171,14 @@ template <class T> CT_HD T jvm_ratio_cast(int64_t n, int64_t d) {
   if (n == INT64_MIN && d == -1) return jvm_cast<T>(n);
   const int64_t q = n / d;
   if (std::is_same<T, int64_t>::value || q * d == n) return jvm_cast<T>(q);
+  return jvm_cast<T>((double)q);
+}
+
+// The same for the int accumulator of byte and short tensors (|n|, |d| <= 2^30: no overflow case).
+template <class T> CT_HD T jvm_ratio_cast(int32_t n, int32_t d) {
+  if (d == 0) return (T)0;
+  const int32_t q = n / d;
+  if (q * d == n) return jvm_cast<T>(q);
   return jvm_cast<T>((double)q);
 }
 

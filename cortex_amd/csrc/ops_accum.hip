@@ -607,7 +607,7 @@ int accum_run_with(hipStream_t s, BinaryF<T, OP> f, void* dest, const ct_dims* d
 template <class T, int OP>
 int accum_run(hipStream_t s, void* dest, const ct_dims* dd, double dest_alpha, const void* y, const ct_dims* yd,
               double y_alpha, int64_t n, bool reverse, int dtype) {
-  using A = typename acc_of<T>::type;
+  using A = typename ew_acc_of<T>::type;
   BinaryF<T, OP> f;
   // f(first, second) = op(first * xa, second * ya)
   f.xa = reverse ? (A)jvm_cast<T>(y_alpha) : (A)jvm_cast<T>(dest_alpha);
@@ -625,7 +625,7 @@ int accum_run(hipStream_t s, void* dest, const ct_dims* dd, double dest_alpha, c
 template <class T, int OP>
 int accum_run_with(hipStream_t s, BinaryF<T, OP> f, void* dest, const ct_dims* dd, double dest_alpha, const void* y,
                    const ct_dims* yd, double y_alpha, int64_t n, bool reverse, int dtype) {
-  using A = typename acc_of<T>::type;
+  using A = typename ew_acc_of<T>::type;
   OwnerArgs a;
   std::memset(&a, 0, sizeof(a));
   if (owner_structure(*dd, *yd, n, &a)) {

@@ -20,7 +20,7 @@ bool valid_arg_idx(const int8_t* a) {
 template <class T>
 int routed_select(hipStream_t s, void* dest, const ct_dims* dd, const void* const* t, const ct_dims* const* td,
                   const double* alpha, int n_tensors, const double* constants, const int8_t* arg_idx, int64_t n) {
-  using A = typename acc_of<T>::type;
+  using A = typename ew_acc_of<T>::type;
   SelectRoutedF<T> f;
   EwOperand ops[4];
   ops[0] = {dest, dd, (int)sizeof(T), 0};
@@ -48,7 +48,7 @@ int role_of(const int8_t* arg_idx, int slot) {
 template <class T>
 bool select_cc(hipStream_t s, void* dest, const ct_dims* dd, const void* a, const ct_dims* ad, double a_alpha,
                const double* constants, const int8_t* arg_idx, int64_t n, int* rc) {
-  using A = typename acc_of<T>::type;
+  using A = typename ew_acc_of<T>::type;
   if (role_of(arg_idx, 0) != 0) return false;
   const T cy = jvm_cast<T>(constants[arg_idx[1] - 1]), cz = jvm_cast<T>(constants[arg_idx[2] - 1]);
   const A xa = (A)jvm_cast<T>(a_alpha);
@@ -67,7 +67,7 @@ bool select_cc(hipStream_t s, void* dest, const ct_dims* dd, const void* a, cons
 template <class T>
 bool select_tc(hipStream_t s, void* dest, const ct_dims* dd, const void* const* t, const ct_dims* const* td,
                const double* alpha, double constant, const int8_t* arg_idx, int64_t n, int* rc) {
-  using A = typename acc_of<T>::type;
+  using A = typename ew_acc_of<T>::type;
   const int xs = arg_idx[0];  // the slot that holds x
   if (xs > 1 || role_of(arg_idx, 2) == 0) return false;
   const int qs = 1 - xs;      // the other tensor
@@ -96,7 +96,7 @@ int ct_ternary_op(void* stream, void* dest, const ct_dims* dest_dims, const void
   CT_REQUIRE(dest && x && y && z, "ct_ternary_op: null buffer");
   CT_REQUIRE(op == CT_TOP_SELECT, "unknown ternary operation %d", op);
   CT_DISPATCH_DTYPE(dtype, {
-    using A = typename acc_of<T>::type;
+    using A = typename ew_acc_of<T>::type;
     const A xa = (A)jvm_cast<T>(x_alpha), ya = (A)jvm_cast<T>(y_alpha), za = (A)jvm_cast<T>(z_alpha);
     EwOperand ops[4] = {{dest, dest_dims, (int)sizeof(T), 0},
                         {x, x_dims, (int)sizeof(T), 0},

@@ -9,7 +9,7 @@ namespace {
 template <class T, int OP>
 int unary_run(hipStream_t s, void* dest, const ct_dims* dd, const void* x, const ct_dims* xd, double alpha,
               int64_t n, bool serial) {
-  using A = typename acc_of<T>::type;
+  using A = typename ew_acc_of<T>::type;
   const T a = jvm_cast<T>(alpha);
   EwOperand ops[2] = {{dest, dd, (int)sizeof(T), 0}, {x, xd, (int)sizeof(T), 0}};
   if constexpr (std::is_same<T, float>::value) {
