@@ -215,6 +215,66 @@ __global__ void __launch_bounds__(kBlock) softmax_block_kernel(const SoftmaxArgs
   for (uint32_t i = threadIdx.x; i < a.k; i += kBlock) out[(int64_t)i * a.out_k] *= inv;  // each lane re-reads its own stores
 }
 
+// One block per row of up to kBlock * ITER vectors, kept in registers like the wave kernel's rows
+// (one read, one write), with the two reductions carried across the four waves through LDS.
+// Unit-stride, aligned rows only.
+template <class T, int VEC, int ITER>
+__global__ void __launch_bounds__(kBlock) softmax_block_reg_kernel(const SoftmaxArgs a) {
+  using V = Vec<T, VEC>;
+  __shared__ double lds[kBlock / 64];
+  int64_t ib, ob;
+  softmax_row_base(a, blockIdx.x, &ib, &ob);
+  const T* in = reinterpret_cast<const T*>(a.in) + ib;
+  T* out = reinterpret_cast<T*>(a.out) + ob;
+  const uint32_t nv = a.k / VEC;
+  const int wave = threadIdx.x >> 6;
+  V x[ITER];
+  T m = -__builtin_huge_valf();
+#pragma unroll
+  for (int j = 0; j < ITER; ++j) {
+    const uint32_t i = threadIdx.x + j * kBlock;
+    if (i < nv) {
+      x[j] = nt_load(reinterpret_cast<const V*>(in + (int64_t)i * VEC));
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) m = jvm_max(m, x[j].v[e]);
+    }
+  }
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) m = jvm_max(m, (T)__shfl_xor(m, s, 64));
+  if ((threadIdx.x & 63) == 0) lds[wave] = (double)m;
+  __syncthreads();
+  m = (T)lds[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / 64; ++w) m = jvm_max(m, (T)lds[w]);
+  __syncthreads();
+  double sum = 0.0;
+#pragma unroll
+  for (int j = 0; j < ITER; ++j) {
+    const uint32_t i = threadIdx.x + j * kBlock;
+    if (i < nv) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) { x[j].v[e] = shifted_exp(x[j].v[e], m); sum += (double)x[j].v[e]; }
+    }
+  }
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) sum += __shfl_xor(sum, s, 64);
+  if ((threadIdx.x & 63) == 0) lds[wave] = sum;
+  __syncthreads();
+  sum = lds[0];
+#pragma unroll
+  for (int w = 1; w < kBlock / 64; ++w) sum += lds[w];
+  const T inv = (T)1 / (T)sum;
+#pragma unroll
+  for (int j = 0; j < ITER; ++j) {
+    const uint32_t i = threadIdx.x + j * kBlock;
+    if (i < nv) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) x[j].v[e] *= inv;
+      *reinterpret_cast<V*>(out + (int64_t)i * VEC) = x[j];
+    }
+  }
+}
+
 // One lane per row, the lanes of a wave on neighbouring rows.  CMAX > 0: the row
 // (k <= CMAX) stays in registers.  CMAX == 0: any k, exponentials parked in the
 // output.  The sum runs in the reference's own order.
@@ -485,6 +545,10 @@ int softmax_run(hipStream_t s, void* out, const RowLayout& ol, const void* in, c
   if (nv <= 1024) {
     note_kernel(vec_ok ? "softmax_wave_vec" : "softmax_wave");
     if (vec_ok) { CT_SM_SHAPES(VMAX); } else { CT_SM_SHAPES(1); }
+  } else if (vec_ok && VMAX > 1 && nv <= 16 * kBlock) {
+    note_kernel("softmax_block_reg");
+    if (nv <= 8 * kBlock) hipLaunchKernelGGL((softmax_block_reg_kernel<T, VMAX, 8>), dim3((uint32_t)a.n_rows), dim3(kBlock), 0, s, a);
+    else hipLaunchKernelGGL((softmax_block_reg_kernel<T, VMAX, 16>), dim3((uint32_t)a.n_rows), dim3(kBlock), 0, s, a);
   } else {
     note_kernel("softmax_block");
     hipLaunchKernelGGL((softmax_block_kernel<T>), dim3((uint32_t)a.n_rows), dim3(kBlock), 0, s, a);
