@@ -683,7 +683,10 @@ struct BnPlan {
 
 constexpr int64_t kRowStyleMinBytes = 128;           // (batch, channel) rows at least this long are walked row style
 constexpr size_t kMaxPartialBytes = size_t(32) << 20;
-constexpr size_t kStreamingBytes = size_t(64) << 20;
+// From this many bytes of operands on, loads are non-temporal: half the 256 MiB last-level cache.
+// The update of a [64, C, 3136] float tensor: 103 MB runs 53 -> 50 us with plain loads, 206 MB
+// 99 -> 116 us.
+constexpr size_t kStreamingBytes = size_t(128) << 20;
 
 template <class T, int MODE>
 int bn_plan(hipStream_t s, int64_t B, int64_t C, int64_t E, const void* x, const void* og, void* out, bool need_stats,
@@ -830,7 +833,8 @@ void bn_launch_apply(hipStream_t s, const BnPlan& plan) {
     const dim3 grid((uint32_t)((r.total_vecs + kBlock - 1) / kBlock));
     r.grouped_blocks = xcd_grouped_blocks(grid.x);
     const double bytes = (double)a.N * sizeof(T) * (MODE == kBnGradient ? 3 : 2);
-    const int level = bytes >= (double)(int64_t(1) << 30) ? 2 : bytes >= (double)kStreamingBytes ? 1 : 0;
+    // the apply pass is an elementwise call: non-temporal loads from the last-level cache's size on
+    const int level = bytes >= (double)(int64_t(1) << 30) ? 2 : bytes >= (double)(int64_t(256) << 20) ? 1 : 0;
     if (ragged) {
       if (level == 2) hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 2, true>), grid, dim3(kBlock), 0, s, r);
       else if (level == 1) hipLaunchKernelGGL((bn_apply_rows_kernel<T, VMAX, MODE, 1, true>), grid, dim3(kBlock), 0, s, r);
