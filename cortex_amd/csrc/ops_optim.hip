@@ -38,6 +38,10 @@ struct AdamScalars {
 };
 
 constexpr int kOptBlock = 64;  // one wave per block
+// The four buffers of a step together up to this size (the last-level cache) are read and written
+// with plain accesses, larger ones with non-temporal ones.  Adam on float: 16 M parameters
+// (256 MiB) 86 % of peak plain against 77 % non-temporal, 24 M (384 MiB) 70 % against 77 %.
+constexpr int64_t kOptCacheBytes = int64_t(256) << 20;
 
 template <class T, int VEC, int UNROLL, bool streaming>
 __global__ void __launch_bounds__(kOptBlock) adam_kernel(const AdamScalars s, const T* g, T* p, T* m, T* v,
@@ -142,7 +146,7 @@ constexpr int kUnroll = 1;  // one vector per lane per buffer
 
 template <class T, int VEC>
 void adam_launch(hipStream_t st, const AdamScalars& s, const T* g, T* p, T* m, T* v, int64_t n) {
-  const bool streaming = n * 7 * (int64_t)sizeof(T) >= (int64_t(64) << 20);
+  const bool streaming = n * 4 * (int64_t)sizeof(T) > kOptCacheBytes;
   const int64_t n_vecs = n / VEC;
   if (n_vecs > 0) {
     const int64_t per = (int64_t)kOptBlock * kUnroll;
@@ -182,7 +186,7 @@ int adam_typed(hipStream_t st, double alpha, double beta1, double beta2, double 
 
 template <class T, int VEC>
 void adadelta_launch(hipStream_t st, const AdadeltaScalars<T>& s, const T* g, T* p, T* a, T* d, int64_t n) {
-  const bool streaming = n * 7 * (int64_t)sizeof(T) >= (int64_t(64) << 20);
+  const bool streaming = n * 4 * (int64_t)sizeof(T) > kOptCacheBytes;
   const int64_t n_vecs = n / VEC;
   if (n_vecs > 0) {
     const int64_t per = (int64_t)kOptBlock * kUnroll;
