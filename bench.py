@@ -52,7 +52,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
-SECTIONS = ("headline", "others", "variants", "patterns", "adjacent")
+SECTIONS = ("headline", "others", "midsize", "variants", "patterns", "adjacent")
 
 
 def log(msg: str) -> None:
@@ -325,6 +325,43 @@ def build_others(b: Bench):
     ops.append(Op("c4_i32_f64", "configs[4] assign! int32 -> float64 [64M]", 12 * nv,
                   lambda: s.assign(f64, dims([nv]), i32, dims([nv]), nv)))
     return ops
+
+
+# ----------------------------------------------------------------------------- the same methods at layer sizes
+
+def build_midsize(b: Bench):
+    """The methods of the step at the sizes of one layer of a network (a [4096,4096] float matrix, 64 MiB): the operands
+    fit the 256 MiB last-level cache, the calls last 10-70 us, and launch ramps and second launches weigh more than at
+    the benchmark's sizes."""
+    s = b.stream
+    side = 4096
+    n = side * side
+    rng = np.random.default_rng(11)
+    x = b.upload(rng.standard_normal(n, dtype=np.float32))
+    g = b.upload(rng.standard_normal(n, dtype=np.float32) * 1e-3)
+    m, v, d = b.alloc(n, "float"), b.alloc(n, "float"), b.alloc(n, "float")
+    bias = b.upload(rng.standard_normal(side, dtype=np.float32))
+    out = b.alloc(side, "float")
+    sq, tr = dims([side, side]), dims([side, side], [1, side])
+    pb1, pb2 = pow_betas()
+    return [
+        Op("m_adam", "Adam step, 2^24 float32 parameters", 28 * n,
+           lambda: s.adam_step(1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 1.0, g, x, m, v, n)),
+        Op("m_bias_add", "binary-op! :+ float32 [4096,4096] + [4096] row", 8 * n + 4 * side,
+           lambda: s.binary_op(d, sq, x, sq, 1.0, bias, dims([side]), 1.0, n, "+")),
+        Op("m_sum_rows", "unary-reduce! :sum last axis of float32 [4096,4096]", 4 * n + 4 * side,
+           lambda: s.unary_reduce(out, dims([side, 1]), 1.0, x, sq, "sum")),
+        Op("m_sum_cols", "unary-reduce! :sum axis 0 of float32 [4096,4096] (transposed view)", 4 * n + 4 * side,
+           lambda: s.unary_reduce(out, dims([side, 1]), 1.0, x, tr, "sum")),
+        Op("m_bias_gradient", "binary-op! :+ accumulate (bias gradient): float32 [4096] += rows of [4096,4096]", 4 * n + 8 * side,
+           lambda: s.binary_accum(out, dims([side]), 1.0, x, sq, 1.0, n, "+", False, True)),
+        Op("m_exp_t", "unary-op! :exp on a transposed float32 [4096,4096] view", 8 * n,
+           lambda: s.unary_op(d, sq, x, tr, 1.0, "exp", n)),
+        Op("m_select_t", "ternary-op! :select, three transposed float32 [4096,4096] views", 16 * n,
+           lambda: s.ternary_op(d, sq, x, tr, 1.0, g, tr, 1.0, m, tr, 1.0, n, "select")),
+        Op("m_softmax", "softmax! float32 [16384,1024]", 8 * n,
+           lambda: s.softmax_eltwise(d, dims([16384, 1024]), x, dims([16384, 1024]))),
+    ]
 
 
 # ----------------------------------------------------------------------------- the constant and accumulate forms
@@ -838,8 +875,8 @@ def main() -> int:
         "roofline": roof,
         "ops": ops_out,
     }
-    builders = {"others": build_others, "variants": build_variants, "patterns": build_patterns, "adjacent": build_adjacent}
-    for name in ("others", "variants", "patterns", "adjacent"):
+    builders = {"others": build_others, "midsize": build_midsize, "variants": build_variants, "patterns": build_patterns, "adjacent": build_adjacent}
+    for name in ("others", "midsize", "variants", "patterns", "adjacent"):
         if name not in sections:
             continue
         log(f"timing section '{name}' ...")
