@@ -33,6 +33,8 @@
 // rounding to float (the tree order differs from the reference's sequential
 // order by about k * 2^-53 relative to the sum of magnitudes).
 #include <algorithm>
+#include <cstdlib>
+#include <limits>
 #include <mutex>
 
 #include "elementwise.h"
@@ -61,20 +63,25 @@ __device__ __forceinline__ double jmin(double a, double b) {
 }
 __device__ __forceinline__ int64_t jmax(int64_t a, int64_t b) { return a > b ? a : b; }
 __device__ __forceinline__ int64_t jmin(int64_t a, int64_t b) { return a < b ? a : b; }
+__device__ __forceinline__ int32_t jmax(int32_t a, int32_t b) { return a > b ? a : b; }
+__device__ __forceinline__ int32_t jmin(int32_t a, int32_t b) { return a < b ? a : b; }
 
 // Reduction policy with the reference's accumulator: a double for float and
 // double tensors, a long for integer tensors (cpu/tensor_math.clj:588-629).
-template <class T, int RK> struct RedWide {
+// ACC = int: byte and short tensors whose reduction cannot leave 32 bits (the host checks: max
+// and min always, sums and means while count * largest product stays below 2^31); the value is the
+// one the long would hold, at a third of the instructions.
+template <class T, int RK, class ACC = typename acc_of<T>::type> struct RedWide {
   using Elem = T;
-  using Acc = typename acc_of<T>::type;
+  using Acc = ACC;
   using Alpha = Acc;
   static __device__ __forceinline__ Acc identity() {
     if constexpr (RK == RK_MAX) {
       if constexpr (std::is_same<Acc, double>::value) return -__builtin_huge_val();
-      else return INT64_MIN;
+      else return std::numeric_limits<Acc>::min();
     } else if constexpr (RK == RK_MIN) {
       if constexpr (std::is_same<Acc, double>::value) return __builtin_huge_val();
-      else return INT64_MAX;
+      else return std::numeric_limits<Acc>::max();
     } else {
       // -0.0 is the additive identity that keeps a sum of negative zeros negative,
       // as the reference's first-element seed does
@@ -83,7 +90,9 @@ template <class T, int RK> struct RedWide {
     }
   }
   static __device__ __forceinline__ Acc value(T x, Alpha alpha) {
-    const Acc v = w_mul(alpha, (Acc)x);
+    Acc v;
+    if constexpr (std::is_same<Acc, int32_t>::value) v = w_mul((Acc)(T)alpha, (Acc)x);  // both in T's range: a 24-bit multiply
+    else v = w_mul(alpha, (Acc)x);
     if constexpr (RK == RK_SUMSQ || RK == RK_MAG) return w_mul(v, v);
     else return v;
   }
@@ -96,7 +105,7 @@ template <class T, int RK> struct RedWide {
   static __device__ __forceinline__ T finish(Acc acc, int64_t count) {
     if constexpr (RK == RK_MEAN) {
       if constexpr (std::is_same<Acc, double>::value) return jvm_cast<T>(acc / (double)count);
-      else return jvm_ratio_cast<T>(acc, count);
+      else return jvm_ratio_cast<T>((int64_t)acc, count);
     } else if constexpr (RK == RK_MAG) {
       return jvm_cast<T>(sqrt((double)acc));
     } else {
@@ -105,6 +114,7 @@ template <class T, int RK> struct RedWide {
   }
   static __device__ __forceinline__ Acc shfl(Acc v, int mask) {
     if constexpr (std::is_same<Acc, double>::value) return __shfl_xor(v, mask, 64);
+    else if constexpr (std::is_same<Acc, int32_t>::value) return __shfl_xor(v, mask, 64);
     else return (Acc)__shfl_xor((long long)v, mask, 64);
   }
 };
@@ -791,6 +801,16 @@ int reduce_typed(hipStream_t st, const PartialStore& ps, void* out, const ct_dim
                  const ct_dims* id, int op) {
   if constexpr (std::is_floating_point<T>::value && (RK == RK_MAX || RK == RK_MIN)) {
     if (jvm_cast<T>(alpha) == (T)1) return reduce_run<RedKeyed<T, RK>>(st, ps, out, od, alpha, in, id, op);
+  }
+  if constexpr (std::is_integral<T>::value && sizeof(T) <= 2 && (RK == RK_MAX || RK == RK_MIN || RK == RK_SUM || RK == RK_MEAN)) {
+    // the largest magnitude an element times the multiplier can have, and how many of them a sum adds
+    const int64_t a_abs = std::llabs((long long)jvm_cast<T>(alpha));
+    const int64_t x_abs = std::is_signed<T>::value ? (int64_t(1) << (8 * sizeof(T) - 1)) : (int64_t(1) << (8 * sizeof(T))) - 1;
+    const int64_t n_out = dims_ecount(*od), total = dims_ecount(*id);
+    const int64_t count = n_out > 0 ? total / n_out : 0;
+    const bool fits = (RK == RK_MAX || RK == RK_MIN) ? a_abs * x_abs < (int64_t(1) << 31)
+                                                    : (count > 0 && a_abs * x_abs < (int64_t(1) << 31) / count);
+    if (fits) return reduce_run<RedWide<T, RK, int32_t>>(st, ps, out, od, alpha, in, id, op);
   }
   return reduce_run<RedWide<T, RK>>(st, ps, out, od, alpha, in, id, op);
 }

@@ -266,6 +266,42 @@ def test_reduce_short_ragged_rows(P, code):
                     (REL_TOL if code == capi.F32 else REL_TOL_F64))
 
 
+@pytest.mark.parametrize("code", [capi.I8, capi.U8, capi.I16])
+def test_narrow_integer_reductions_at_the_edge_of_32_bits(P, code):
+    """Byte and short reductions run on int accumulators while the host can prove that the result stays inside
+    32 bits, on long ones otherwise: extreme elements, the largest multipliers, and row lengths on both sides of
+    the bound, against the oracle's long arithmetic."""
+    dt = NP[code]
+    info = np.iinfo(dt)
+    rng = np.random.default_rng(63)
+    big_alpha = float(info.max)
+    # sum: count * |alpha| * max|x| crosses 2^31 between these two row lengths
+    per = int(max(abs(info.min), info.max)) * int(info.max)
+    edge = (1 << 31) // per
+    for k in sorted({max(1, edge - 3), edge + 5, 4096}):
+        rows = 3
+        x = np.full(rows * k, info.min, dt)
+        x[k:2 * k] = info.max
+        x[2 * k:] = rng.integers(info.min, int(info.max) + 1, k).astype(dt)
+        xb = P.buf(x)
+        out = P.buf(np.zeros(rows, dt))
+        for op in ("sum", "mean", "max", "min"):
+            for alpha in (big_alpha, 1.0, -1.0):
+                kname = P.run(H.unary_reduce, View(out, [rows, 1]), alpha, View(xb, [rows, k]), op)
+                compare(out, f"{op} alpha {alpha} rows of {k} ({kname})")
+        # down the columns of the same data viewed [k, rows]^T is a strided reduce of three rows: skip; a real column case:
+    cols, rows = 512, 700
+    x = rng.integers(info.min, int(info.max) + 1, rows * cols).astype(dt)
+    x[:cols] = info.min
+    xb = P.buf(x)
+    out = P.buf(np.zeros(cols, dt))
+    for op in ("sum", "mean", "max", "min"):
+        for alpha in (big_alpha, 1.0):
+            kname = P.run(H.unary_reduce, View(out, [cols, 1]), alpha, View(xb, [cols, rows], [1, cols]), op)
+            assert kname.startswith("reduce_col"), kname
+            compare(out, f"column {op} alpha {alpha} ({kname})")
+
+
 def test_float_tanh_dense_sweep(P):
     """unary-op! :tanh on float tensors runs a single-precision form of its own: a dense sweep of its
     argument range (the polynomial below 0.4, the seam, the exponential form up to saturation, tiny and

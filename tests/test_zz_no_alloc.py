@@ -95,7 +95,8 @@ def test_unsplit_shapes_and_ragged_views(pair_factory):
 
 
 def test_rejects_what_the_fixed_array_cannot_hold(pair_factory):
-    """64 Ki byte-wide columns cut into 8 segments need 4 MiB of long accumulators: refused, nothing launched."""
+    """64 Ki byte-wide columns cut into 8 segments need 4 MiB of long accumulators (a sum of squares; plain sums
+    of bytes run on int accumulators and fit): refused, nothing launched."""
     rows, cols = 1024, 65536
     with pair_factory() as pair:
         data = np.random.default_rng(14).integers(-128, 128, rows * cols, dtype=np.int64).astype(np.int8)
@@ -103,8 +104,11 @@ def test_rejects_what_the_fixed_array_cannot_hold(pair_factory):
         out = pair.buf(np.full(cols, 5, np.int8))
         view = H.View(src, [cols, rows], [1, cols])
         with pytest.raises(capi.CortexHipError) as err:
-            _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")
+            _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "magnitude-squared")
         assert err.value.status == 1 and "fixed scratch holds 2097152" in err.value.message
         assert np.all(out.download() == 5)
-        _reduce("ct_unary_reduce", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")  # the allocating form takes it
+        _reduce("ct_unary_reduce", pair.hip, H.View(out, [cols, 1]), 1.0, view, "magnitude-squared")  # the allocating form takes it
+        squares = (data.reshape(rows, cols).astype(np.int64) ** 2).sum(axis=0)
+        assert np.array_equal(out.download(), squares.astype(np.int8))
+        _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")  # int accumulators: 2 MiB, fits
         assert np.array_equal(out.download(), data.reshape(rows, cols).astype(np.int64).sum(axis=0).astype(np.int8))
