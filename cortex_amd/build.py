@@ -31,6 +31,7 @@ SOURCES = [
     "ops_ternary.hip",
     "ops_accum.hip",
     "ops_reduce.hip",
+    "ops_reduce_int.hip",
     "ops_optim.hip",
     "ops_nn.hip",
     "ops_batchnorm.hip",
