@@ -71,7 +71,7 @@ __device__ __forceinline__ int32_t jmin(int32_t a, int32_t b) { return a < b ? a
 // Reduction policy with the reference's accumulator: a double for float and
 // double tensors, a long for integer tensors (cpu/tensor_math.clj:588-629).
 // ACC = int: byte and short tensors whose reduction cannot leave 32 bits (the host checks: max
-// and min always, sums and means while count * largest product stays below 2^31); the value is the
+// and min always, sums, means and sums of squares while count * largest term stays below 2^31); the value is the
 // one the long would hold, at a third of the instructions.
 template <class T, int RK, class ACC = typename acc_of<T>::type> struct RedWide {
   using Elem = T;
@@ -804,14 +804,15 @@ int reduce_typed(hipStream_t st, const PartialStore& ps, void* out, const ct_dim
   if constexpr (std::is_floating_point<T>::value && (RK == RK_MAX || RK == RK_MIN)) {
     if (jvm_cast<T>(alpha) == (T)1) return reduce_run<RedKeyed<T, RK>>(st, ps, out, od, alpha, in, id, op);
   }
-  if constexpr (std::is_integral<T>::value && sizeof(T) <= 2 && (RK == RK_MAX || RK == RK_MIN || RK == RK_SUM || RK == RK_MEAN)) {
+  if constexpr (std::is_integral<T>::value && sizeof(T) <= 2) {
     // the largest magnitude an element times the multiplier can have, and how many of them a sum adds
     const int64_t a_abs = std::llabs((long long)jvm_cast<T>(alpha));
     const int64_t x_abs = std::is_signed<T>::value ? (int64_t(1) << (8 * sizeof(T) - 1)) : (int64_t(1) << (8 * sizeof(T))) - 1;
     const int64_t n_out = dims_ecount(*od), total = dims_ecount(*id);
     const int64_t count = n_out > 0 ? total / n_out : 0;
-    const bool fits = (RK == RK_MAX || RK == RK_MIN) ? a_abs * x_abs < (int64_t(1) << 31)
-                                                    : (count > 0 && a_abs * x_abs < (int64_t(1) << 31) / count);
+    const int64_t term = (RK == RK_SUMSQ || RK == RK_MAG) ? (a_abs * x_abs) * (a_abs * x_abs) : a_abs * x_abs;  // < 2^62
+    const bool fits = (RK == RK_MAX || RK == RK_MIN) ? term < (int64_t(1) << 31)
+                                                    : (count > 0 && term < (int64_t(1) << 31) / count);
     if (fits) return reduce_run<RedWide<T, RK, int32_t>>(st, ps, out, od, alpha, in, id, op);
   }
   return reduce_run<RedWide<T, RK>>(st, ps, out, od, alpha, in, id, op);

@@ -285,7 +285,7 @@ def test_narrow_integer_reductions_at_the_edge_of_32_bits(P, code):
         x[2 * k:] = rng.integers(info.min, int(info.max) + 1, k).astype(dt)
         xb = P.buf(x)
         out = P.buf(np.zeros(rows, dt))
-        for op in ("sum", "mean", "max", "min"):
+        for op in ("sum", "mean", "max", "min", "magnitude-squared", "magnitude"):
             for alpha in (big_alpha, 1.0, -1.0):
                 kname = P.run(H.unary_reduce, View(out, [rows, 1]), alpha, View(xb, [rows, k]), op)
                 compare(out, f"{op} alpha {alpha} rows of {k} ({kname})")
@@ -295,7 +295,7 @@ def test_narrow_integer_reductions_at_the_edge_of_32_bits(P, code):
     x[:cols] = info.min
     xb = P.buf(x)
     out = P.buf(np.zeros(cols, dt))
-    for op in ("sum", "mean", "max", "min"):
+    for op in ("sum", "mean", "max", "min", "magnitude-squared", "magnitude"):
         for alpha in (big_alpha, 1.0):
             kname = P.run(H.unary_reduce, View(out, [cols, 1]), alpha, View(xb, [cols, rows], [1, cols]), op)
             assert kname.startswith("reduce_col"), kname

@@ -95,20 +95,21 @@ def test_unsplit_shapes_and_ragged_views(pair_factory):
 
 
 def test_rejects_what_the_fixed_array_cannot_hold(pair_factory):
-    """64 Ki byte-wide columns cut into 8 segments need 4 MiB of long accumulators (a sum of squares; plain sums
-    of bytes run on int accumulators and fit): refused, nothing launched."""
-    rows, cols = 1024, 65536
+    """1024 byte-wide columns of 132200 rows under a multiplier of 127: the sums can leave 32 bits, so they run on
+    long accumulators, and the 512 row segments need 4 MiB of them: refused, nothing launched.  With a
+    multiplier of 1 the same reduction runs on int accumulators, 2 MiB, and fits."""
+    rows, cols = 132200, 1024
     with pair_factory() as pair:
         data = np.random.default_rng(14).integers(-128, 128, rows * cols, dtype=np.int64).astype(np.int8)
         src = pair.buf(data)
         out = pair.buf(np.full(cols, 5, np.int8))
         view = H.View(src, [cols, rows], [1, cols])
         with pytest.raises(capi.CortexHipError) as err:
-            _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "magnitude-squared")
+            _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 127.0, view, "sum")
         assert err.value.status == 1 and "fixed scratch holds 2097152" in err.value.message
         assert np.all(out.download() == 5)
-        _reduce("ct_unary_reduce", pair.hip, H.View(out, [cols, 1]), 1.0, view, "magnitude-squared")  # the allocating form takes it
-        squares = (data.reshape(rows, cols).astype(np.int64) ** 2).sum(axis=0)
-        assert np.array_equal(out.download(), squares.astype(np.int8))
-        _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")  # int accumulators: 2 MiB, fits
-        assert np.array_equal(out.download(), data.reshape(rows, cols).astype(np.int64).sum(axis=0).astype(np.int8))
+        _reduce("ct_unary_reduce", pair.hip, H.View(out, [cols, 1]), 127.0, view, "sum")  # the allocating form takes it
+        sums = data.reshape(rows, cols).astype(np.int64).sum(axis=0)
+        assert np.array_equal(out.download(), (sums * 127).astype(np.int8))
+        _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")  # int accumulators: fits
+        assert np.array_equal(out.download(), sums.astype(np.int8))
