@@ -68,8 +68,28 @@ __device__ __forceinline__ int64_t jvm_round(double v) {
   return jvm_d2l(r);
 }
 
-// perform-unary-op-impl (cpu/tensor_math.clj:211-223) on v = x * alpha.
+// exp of a double argument to float accuracy (about 1 ulp of the float result): v * log2(e) is split
+// in double into an integer n and a fraction in [-0.5, 0.5]; the hardware's exp2 takes the fraction
+// as a float and ldexp applies n.  n is clamped to +-300, which keeps it a number for NaN and
+// infinite arguments; those reach exp2 through the fraction and come out NaN, +infinity and 0.
+__device__ __forceinline__ float exp_f32_of(double v) {
+  const double a = v * 1.4426950408889634;
+  const double n = __builtin_fmin(__builtin_fmax(__builtin_rint(a), -300.0), 300.0);
+  return __builtin_ldexpf(__builtin_amdgcn_exp2f((float)(a - n)), (int)n);
+}
+
+__device__ __forceinline__ float tanh_f32(float x);
+
+// perform-unary-op-impl (cpu/tensor_math.clj:211-223) on v = x * alpha.  Float tensors with a
+// multiplier other than 1 take the transcendental ops through the single-precision forms too
+// (the product itself is formed in double): inside the 2e-6 relative bar, and memory-bound where
+// the double routines were not.
 template <class T, int OP, class A> __device__ __forceinline__ T unary_value(A v) {
+  if constexpr (std::is_same<T, float>::value && std::is_same<A, double>::value) {
+    if constexpr (OP == CT_UOP_EXP) return exp_f32_of(v);
+    else if constexpr (OP == CT_UOP_TANH) return tanh_f32((float)v);
+    else if constexpr (OP == CT_UOP_LOGISTIC) return 1.0f / (1.0f + exp_f32_of(-v));
+  }
   if constexpr (OP == CT_UOP_FLOOR) return jvm_cast<T>(floor((double)v));
   else if constexpr (OP == CT_UOP_CEIL) return jvm_cast<T>(ceil((double)v));
   else if constexpr (OP == CT_UOP_ROUND) return jvm_cast<T>(jvm_round((double)v));
