@@ -705,9 +705,11 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
     } else if (split == 1 && nv <= 256) {
       note_kernel(vec_ok ? "reduce_row_small_vec" : "reduce_row_small");
       if (vec_ok) { CT_ROW_SMALL_SHAPES(VMAX); } else { CT_ROW_SMALL_SHAPES(1); }
-    } else if (vec_ok && row_bytes >= 16384) {
+    } else if (vec_ok && (row_bytes >= 32768 || (row_bytes >= 16384 && n_groups * row_bytes >= (int64_t(192) << 20)))) {
       // 512 lanes per row: a 16 KiB row is in flight at once, two loads per lane.  Measured on float
-      // [16384,4096]: 92 % of peak against 85-89 % for 256 lanes (two rounds of two loads)
+      // [16384,4096]: 92 % of peak against 85-89 % for 256 lanes (two rounds of two loads).  With a
+      // quarter of the rows, [4096,4096], 256 lanes are ahead (10.4 us against 11.5), hence the
+      // size condition on 16 KiB rows; rows of 32 KiB (double [4096,4096]) take 512 lanes at any size.
       note_kernel("reduce_row512_vec");
       CT_ROW_WIDE(VMAX);
     } else if (row_bytes >= 4096) {

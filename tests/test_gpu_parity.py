@@ -601,8 +601,11 @@ def test_reduce_kernel_selection(P):
     rng = np.random.default_rng(10)
     x = P.buf(rng.standard_normal(64 * 4096).astype(np.float32))
     out = P.buf(np.zeros(4096, np.float32))
-    assert P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 4096]), "sum") == "reduce_row512_vec"
-    compare(out, "rows of 16 KiB", tol=2e-6)
+    wide = P.buf(rng.standard_normal(2048 * 8192).astype(np.float32))
+    assert P.run(H.unary_reduce, View(out, [2048, 1]), 1.0, View(wide, [2048, 8192]), "sum") == "reduce_row512_vec"
+    compare(out, "rows of 32 KiB", tol=2e-6)
+    assert P.run(H.unary_reduce, View(out, [64, 1]), 1.0, View(x, [64, 4096]), "sum") == "reduce_row256_vec"
+    compare(out, "rows of 16 KiB, a small tensor", tol=2e-6)
     assert P.run(H.unary_reduce, View(out, [128, 1]), 1.0, View(x, [128, 2048]), "sum") == "reduce_row256_vec"
     compare(out, "rows of 8 KiB", tol=2e-6)
     assert P.run(H.unary_reduce, View(out, [1024, 1]), 1.0, View(x, [1024, 256]), "sum") == "reduce_row_small_vec"
