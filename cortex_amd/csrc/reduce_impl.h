@@ -762,7 +762,11 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
     // (one round of resident blocks measured better than several shorter ones);
     // a segment is a whole number of load batches; partials capped at 16 MiB.
     constexpr int64_t kRowQuantum = 128;  // 16 waves x 8 loads in flight
-    const int64_t want_seg = std::max<int64_t>(1, std::min<int64_t>(512 / base_blocks, k / kRowQuantum));
+    // Between one and two blocks per compute unit, segments of two load batches are preferred to
+    // twice as many of one: float [4096,4096] 10.6 us with 16 segments against 11.6 with 32.
+    const int64_t most = std::max<int64_t>(1, std::min<int64_t>(512 / base_blocks, k / kRowQuantum));
+    const int64_t least = std::max<int64_t>(1, std::min<int64_t>(most, (256 + base_blocks - 1) / base_blocks));
+    const int64_t want_seg = std::min(most, std::max(least, k / (2 * kRowQuantum)));
     int64_t rows = ((k + want_seg - 1) / want_seg + kRowQuantum - 1) / kRowQuantum * kRowQuantum;
     const int64_t seg_cap = std::max<int64_t>(1, (int64_t(16) << 20) / (n_out * (int64_t)sizeof(A)));
     if ((k + rows - 1) / rows > seg_cap) rows = (k + seg_cap - 1) / seg_cap;
