@@ -2,6 +2,7 @@
 #include "elementwise.h"
 
 #include <algorithm>
+#include <vector>
 
 namespace cthip {
 
@@ -151,6 +152,55 @@ int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int ti
   }
   *lds_bytes = lds;
   return CT_OK;
+}
+
+// Cuts a call along its slowest axis of more than one element into pieces of at most `limit`
+// elements: operands that span the axis get a shorter shape and a later start (in the index tensor
+// when the axis is indexed), operands that broadcast along it stay as they are.  False when the
+// call has another form (a count that is not the product of the largest shape, a commensurate
+// operand).  When the trailing axes alone exceed the limit a piece is one coordinate of the axis,
+// and the launcher cuts it again along the next axis.
+bool split_leading(const EwOperand* ops, int n_ops, int64_t n, int64_t limit, std::vector<EwPiece>* pieces) {
+  int rank = 0;
+  for (int k = 0; k < n_ops; ++k)
+    if (ops[k].ptr && ops[k].dims) rank = std::max(rank, ops[k].dims->ndim);
+  if (rank == 0) return false;
+  int64_t mx[CT_MAX_DIMS];
+  for (int d = 0; d < rank; ++d) mx[d] = 1;
+  for (int k = 0; k < n_ops; ++k) {
+    if (!ops[k].ptr || !ops[k].dims) continue;
+    const ct_dims& dm = *ops[k].dims;
+    for (int i = 0; i < dm.ndim; ++i) mx[i + rank - dm.ndim] = std::max<int64_t>(mx[i + rank - dm.ndim], dm.shape[i]);
+  }
+  int lead = 0;
+  while (lead < rank && mx[lead] == 1) ++lead;
+  if (lead == rank) return false;
+  int64_t rest = 1, total = 1;
+  for (int d = lead + 1; d < rank; ++d) rest *= mx[d];
+  for (int d = 0; d < rank; ++d) total *= mx[d];
+  if (total != n) return false;
+  const int64_t per = std::max<int64_t>(1, limit / rest);
+  for (int64_t c0 = 0; c0 < mx[lead]; c0 += per) {
+    const int64_t c1 = std::min(mx[lead], c0 + per);
+    EwPiece piece;
+    piece.n = (c1 - c0) * rest;
+    for (int k = 0; k < n_ops; ++k) {
+      piece.ptr[k] = ops[k].ptr;
+      if (!ops[k].ptr || !ops[k].dims) { std::memset(&piece.dims[k], 0, sizeof(ct_dims)); continue; }
+      piece.dims[k] = *ops[k].dims;
+      const int di = lead - (rank - ops[k].dims->ndim);
+      if (di < 0 || piece.dims[k].shape[di] == 1) {
+        if (k == 0) return false;  // a destination that repeats along the axis is not cut here
+        continue;
+      }
+      if (piece.dims[k].shape[di] != mx[lead]) return false;
+      piece.dims[k].shape[di] = c1 - c0;
+      if (piece.dims[k].index[di]) piece.dims[k].index[di] += c0;
+      else piece.ptr[k] = static_cast<const char*>(ops[k].ptr) + c0 * piece.dims[k].strides[di] * ops[k].elem_size;
+    }
+    pieces->push_back(piece);
+  }
+  return true;
 }
 
 // Vectors that start anywhere (ew_vecu_kernel): rows of at least one vector whose starts or

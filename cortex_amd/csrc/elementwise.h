@@ -14,6 +14,7 @@
 #pragma once
 
 #include <algorithm>
+#include <vector>
 
 #include "common.h"
 #include "plan.h"
@@ -1067,6 +1068,15 @@ struct EwOperand {
   uint64_t cbits;       // constant value, already in the operand's element type
 };
 
+// A call of 2^31 elements or more is cut into pieces along its slowest axis (split_leading), each
+// run on its own: the kernels index with 32 bits.
+struct EwPiece {
+  const void* ptr[kMaxOps];
+  ct_dims dims[kMaxOps];
+  int64_t n;
+};
+bool split_leading(const EwOperand* ops, int n_ops, int64_t n, int64_t limit, std::vector<EwPiece>* pieces);
+
 int prepare_vec(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* main_args, int* main_vec,
                 VecArgs* tail_args, bool* has_tail);
 int prepare_tile(const Plan& plan, const EwOperand* ops, int tile_a_edge, int tile_b_edge, bool wide_a, TileArgs* args,
@@ -1199,6 +1209,20 @@ template <class F>
 int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t n) {
   constexpr int NIN = F::NIN;
   if (n == 0) return CT_OK;
+  if (n >= (int64_t(1) << 31)) {
+    // Beyond what a 32-bit index counts the fast kernels do not apply as they are (only the
+    // per-element one has a 64-bit form, at a hundredth of the memory rate): the call is run as
+    // pieces of at most 2^30 elements along its slowest axis, each on the kernel of its shape.
+    std::vector<EwPiece> pieces;
+    if (split_leading(ops, NIN + 1, n, int64_t(1) << 30, &pieces)) {
+      for (const EwPiece& piece : pieces) {
+        EwOperand sub[kMaxOps];
+        for (int k = 0; k <= NIN; ++k) sub[k] = {piece.ptr[k], ops[k].dims ? &piece.dims[k] : nullptr, ops[k].elem_size, ops[k].cbits};
+        if (int rc = launch_elementwise(s, f, sub, piece.n)) return rc;
+      }
+      return CT_OK;
+    }
+  }
   OperandIn in[kMaxOps];
   for (int k = 0; k <= NIN; ++k) in[k] = {ops[k].ptr, ops[k].dims, ops[k].elem_size};
   Plan plan;

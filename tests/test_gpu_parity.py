@@ -1327,6 +1327,44 @@ def test_flat_call_longer_than_one_launch():
         capi.call("ct_free", b)
 
 
+@pytest.mark.parametrize("rows,cols", [((1 << 15) + 3, 1 << 17), (2, (1 << 31) + 48)], ids=["many_rows", "two_long_rows"])
+def test_rows_and_columns_call_beyond_32_bit_indexing(rows, cols):
+    """A byte matrix of 2^31 elements or more plus a bias row: more than the kernels' 32-bit indices
+    count, so the call is cut along its slowest axis into pieces of at most 2^30 elements (8192 rows of
+    2^17; a row longer than that is cut again along the row).  Rows at the start, on both sides of piece
+    boundaries and at the end are copied back and compared, and the pieces run on the vector kernel."""
+    import ctypes as C
+    n = rows * cols
+    free, total = C.c_size_t(), C.c_size_t()
+    capi.call("ct_memory_info", C.byref(free), C.byref(total))
+    if free.value < 2 * n + (2 << 30):
+        pytest.skip("needs %d GiB of free device memory" % ((2 * n >> 30) + 2))
+    a, b, bias = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    capi.call("ct_malloc", C.byref(a), n)
+    capi.call("ct_malloc", C.byref(b), n)
+    capi.call("ct_malloc", C.byref(bias), cols)
+    try:
+        host_bias = (np.arange(cols) % 11).astype(np.int8)
+        capi.call("ct_memcpy_async", bias, host_bias.ctypes.data, cols, capi.COPY_H2D, None)
+        capi.call("ct_memset", None, a, capi.I8, 7.0, n)
+        capi.call("ct_memset", None, b, capi.I8, 0.0, n)
+        full, row = capi.make_dims([rows, cols], [cols, 1]), capi.make_dims([cols], [1])
+        capi.call("ct_binary_op", None, b, C.byref(full), a, C.byref(full), 1.0, bias, C.byref(row), 1.0, n,
+                  capi.BINARY_OPS["+"], capi.I8)
+        capi.call("ct_stream_sync", None)
+        assert capi.last_kernel() == "vec"
+        want = (7 + host_bias).astype(np.int8)
+        picks = {0, 1, 8191, 8192, 8193, 16384, rows // 2 - 1, rows // 2, rows - 8193, rows - 1}
+        for r in sorted(p for p in picks if 0 <= p < rows):
+            out = np.zeros(cols, np.int8)
+            capi.call("ct_memcpy_async", out.ctypes.data, b.value + r * cols, cols, capi.COPY_D2H, None)
+            capi.call("ct_stream_sync", None)
+            assert np.array_equal(out, want), (r, np.flatnonzero(out != want)[:8])
+    finally:
+        for p in (a, b, bias):
+            capi.call("ct_free", p)
+
+
 # ------------------------------------------------------------------ threads and streams
 
 def test_threads_on_their_own_streams(P):
