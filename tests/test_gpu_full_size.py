@@ -411,3 +411,42 @@ def test_broadcast_accumulates_at_benchmark_size():
     assert np.array_equal(d_acc.download().astype(np.float64), whole.astype(np.float64).sum(axis=0))
     for t in (d_y, d_whole, d_acc):
         t.free()
+
+
+def test_matrix_of_2_31_elements_built_and_reduced():
+    """A float matrix of 65536 x 32768 (2^31 elements, 8 GiB: one element more than a 32-bit index
+    counts) is built on the device as column[r] + row[c] (r % 5 and c % 7, so that every sum below is an
+    integer under 2^24 and exact in any order), then summed along its rows and, through the transposed
+    view, along its columns; both results are compared with their closed forms.  The build runs as
+    pieces on the vector kernel, the sums on the row and column kernels."""
+    rows, cols = 1 << 16, 1 << 15
+    n = rows * cols
+    free, total = C.c_size_t(), C.c_size_t()
+    capi.call("ct_memory_info", C.byref(free), C.byref(total))
+    if free.value < 4 * n + (2 << 30):
+        pytest.skip("needs 10 GiB of free device memory")
+    col_vals = (np.arange(rows) % 5).astype(np.float32)
+    row_vals = (np.arange(cols) % 7).astype(np.float32)
+    d_col, d_row = Dev(col_vals), Dev(row_vals)
+    d_rsum, d_csum = Dev(np.zeros(rows, np.float32)), Dev(np.zeros(cols, np.float32))
+    big = C.c_void_p()
+    capi.call("ct_malloc", C.byref(big), 4 * n)
+    try:
+        full = dims([rows, cols])
+        capi.call("ct_binary_op", None, big, C.byref(full), d_col.ptr, C.byref(dims([rows, 1])), 1.0, d_row.ptr,
+                  C.byref(dims([cols])), 1.0, n, capi.BINARY_OPS["+"], capi.F32)
+        assert capi.last_kernel() == "vec"
+        capi.call("ct_unary_reduce", None, d_rsum.ptr, C.byref(dims([rows, 1])), 1.0, big, C.byref(full),
+                  capi.REDUCE_OPS["sum"], capi.F32)
+        assert capi.last_kernel() == "reduce_row512_vec"
+        capi.call("ct_unary_reduce", None, d_csum.ptr, C.byref(dims([cols, 1])), 1.0, big,
+                  C.byref(dims([cols, rows], [1, cols])), capi.REDUCE_OPS["sum"], capi.F32)
+        assert capi.last_kernel() == "reduce_col_vec"
+        want_r = cols * col_vals.astype(np.float64) + row_vals.astype(np.float64).sum()
+        want_c = rows * row_vals.astype(np.float64) + col_vals.astype(np.float64).sum()
+        assert np.array_equal(d_rsum.download().astype(np.float64), want_r)
+        assert np.array_equal(d_csum.download().astype(np.float64), want_c)
+    finally:
+        capi.call("ct_free", big)
+        for t in (d_col, d_row, d_rsum, d_csum):
+            t.free()
