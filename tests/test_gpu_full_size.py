@@ -450,3 +450,41 @@ def test_matrix_of_2_31_elements_built_and_reduced():
         capi.call("ct_free", big)
         for t in (d_col, d_row, d_rsum, d_csum):
             t.free()
+
+
+def test_indexed_rows_of_2_31_bytes_gathered_and_scattered():
+    """65541 rows of 32768 bytes picked from a [1000, 32768] table through an index tensor (2^31 + 163840
+    elements): the gather runs as pieces of 32768 rows whose index pointers advance with them, and rows
+    on both sides of the piece boundaries are compared with the table.  The gathered rows are then
+    scatter-added into a zeroed table through the same index: row t ends as (its number of
+    occurrences) x (table row t) in wrapping byte arithmetic, whatever the order."""
+    rows, table_rows, width = (1 << 16) + 5, 1000, 1 << 15
+    n = rows * width
+    free, total = C.c_size_t(), C.c_size_t()
+    capi.call("ct_memory_info", C.byref(free), C.byref(total))
+    if free.value < n + (2 << 30):
+        pytest.skip("needs 4 GiB of free device memory")
+    idx = ((np.arange(rows, dtype=np.int64) * 7) % table_rows).astype(np.int32)
+    table = ((np.arange(table_rows)[:, None] + np.arange(width)[None, :]) % 100).astype(np.int8)
+    d_idx, d_table, d_sums = Dev(idx), Dev(table), Dev(np.zeros(table_rows * width, np.int8))
+    out = C.c_void_p()
+    capi.call("ct_malloc", C.byref(out), n)
+    try:
+        picked = capi.make_dims([rows, width], [width, 1], [d_idx.ptr, None])
+        capi.call("ct_assign", None, out, C.byref(dims([rows, width])), capi.I8, d_table.ptr, C.byref(picked), capi.I8, n)
+        assert capi.last_kernel() == "vec"
+        for r in (0, 1, 32767, 32768, 32769, 65535, 65536, rows - 1):
+            got = np.zeros(width, np.int8)
+            capi.call("ct_memcpy_async", got.ctypes.data, out.value + r * width, width, capi.COPY_D2H, None)
+            capi.call("ct_stream_sync", None)
+            assert np.array_equal(got, table[idx[r]]), r
+        capi.call("ct_binary_accum", None, d_sums.ptr, C.byref(picked), 1.0, out, C.byref(dims([rows, width])), 1.0, n,
+                  capi.BINARY_OPS["+"], 0, 1, capi.I8)
+        assert capi.last_kernel() == "accum_grouped_vec"
+        counts = np.bincount(idx, minlength=table_rows).astype(np.int64)
+        want = (counts[:, None] * table.astype(np.int64)).astype(np.int8)
+        assert np.array_equal(d_sums.download().reshape(table_rows, width), want)
+    finally:
+        capi.call("ct_free", out)
+        for t in (d_idx, d_table, d_sums):
+            t.free()
