@@ -480,7 +480,7 @@ def build_patterns(b: Bench):
 # ----------------------------------------------------------------------------- adjacent TensorMath methods
 
 def build_adjacent(b: Bench):
-    """activation-gradient!, softmax!, batch normalization, rand!, gemv!: HBM-bound like the hot path.
+    """activation-gradient!, softmax!, batch normalization, rand!, local response normalization, gemv!: HBM-bound like the hot path.
     Bytes are algorithmic (every operand read once, every result written once) although the
     batch-normalization forms that need batch statistics read their operands twice."""
     s = b.stream
@@ -523,6 +523,15 @@ def build_adjacent(b: Bench):
     ops.append(Op("a_bn_gradients", f"batch-normalize-gradients! spatial float32 [{bb},{cc},{ee}] (moves 20 B/element)", 12 * nn_,
                   lambda: s.batch_normalize_gradients_spatial(o, st[6], st[7], g, o, x, st[0], st[1], st[2], st[3], 1e-3,
                                                               bb, cc, ee)))
+    # local response normalization across the channels (AlexNet's n 5, k 2, alpha 1e-4, beta 0.75: the reference's defaults)
+    lrn = {"n": 5, "k": 2.0, "alpha": 1e-4, "beta": 0.75}
+    hw = 56
+    o2 = b.alloc(nn_, "float")
+    ops.append(Op("a_lrn_forward", f"lrn-forward! float32 [{bb},{cc},{hw},{hw}] n 5", 8 * nn_,
+                  lambda: s.lrn_forward(o, dims([bb, cc, hw, hw]), x, dims([bb, cc, hw, hw]), lrn)))
+    ops.append(Op("a_lrn_backward", f"lrn-backward! float32 [{bb},{cc},{hw},{hw}] n 5", 16 * nn_,
+                  lambda: s.lrn_backward(o2, dims([bb, cc, hw, hw]), o, dims([bb, cc, hw, hw]), x, dims([bb, cc, hw, hw]),
+                                         g, dims([bb, cc, hw, hw]), lrn)))
     mm = 8192
     a_ = b.upload(rng.standard_normal(mm * mm, dtype=np.float32))
     xv = b.upload(rng.standard_normal(mm, dtype=np.float32))

@@ -37,9 +37,6 @@
 (defn- arg-indexes [arg-order]
   (ffi/arg-indexes->native (cpu-tm/arg-order->indexes arg-order)))   ; cpu/tensor_math.clj:500-504
 
-(defn- unsupported [method]
-  (throw (ex-info (str (name method) " is unsupported on :hip") {:method method})))
-
 (extend-type HipStream
   tm/TensorMath
 
@@ -279,12 +276,25 @@
              (int kind) (double a) (double b) (long seed) (long calls))))
 
   ;; ------------------------------------------------------------ local response normalisation (tensor/math.clj:240-252)
-  ;; cuDNN-only in the reference (src/cortex/tensor.clj:1554-1557): the CPU backend has no form of it
-  (lrn-descriptor [stream n k alpha beta] (unsupported :lrn-descriptor))
-  (lrn-forward! [stream output output-dims input input-dims lrn-descriptor] (unsupported :lrn-forward!))
+  ;; cuDNN-only in the reference (src/cortex/tensor.clj:1554-1557; cuda/tensor_math.clj:1277-1335).
+  ;; The descriptor is a plain map: the library keeps no native object for it.
+  (lrn-descriptor [stream n k alpha beta]
+    {:n (long n) :k (double k) :alpha (double alpha) :beta (double beta)})
+
+  (lrn-forward! [stream output output-dims input input-dims lrn-descriptor]
+    (select-device! stream)
+    (let [{:keys [n k alpha beta]} lrn-descriptor]
+      (call! "ct_lrn_forward" (:handle stream) (->ptr output) (dims output-dims) (->ptr input) (dims input-dims)
+             (int n) (double k) (double alpha) (double beta) (dtype-code output))))
+
   (lrn-backward! [stream input-gradient input-grad-dims output output-dims input input-dims
                   output-gradient output-grad-dims lrn-descriptor]
-    (unsupported :lrn-backward!)))
+    (select-device! stream)
+    (let [{:keys [n k alpha beta]} lrn-descriptor]
+      (call! "ct_lrn_backward" (:handle stream) (->ptr input-gradient) (dims input-grad-dims)
+             (->ptr output) (dims output-dims) (->ptr input) (dims input-dims)
+             (->ptr output-gradient) (dims output-grad-dims)
+             (int n) (double k) (double alpha) (double beta) (dtype-code output)))))
 
 ;; ---------------------------------------------------------------- entry points beyond the protocol
 

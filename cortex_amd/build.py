@@ -37,7 +37,7 @@ SOURCES = [
     "ops_batchnorm.hip",
     "ops_rand.hip",
     "ops_blas.cpp",
-    "ops_gemv.hip", "ops_pool.hip", "ops_conv.hip",
+    "ops_gemv.hip", "ops_pool.hip", "ops_conv.hip", "ops_lrn.hip",
 ]
 
 # -ffp-contract=off: the reference's CPU backend rounds after every JVM

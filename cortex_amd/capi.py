@@ -163,6 +163,8 @@ PROTOTYPES = {
     "ct_convolution_backward_data": [_P, _P, _D, _P, _P, _P, _L, C.POINTER(CtConvDesc), _L, _L, _L, _L, _L, _I],
     "ct_pooling_forward": [_P, _P, _D, _P, C.POINTER(CtPoolDesc), _L, _L, _L, _L, _L, _L, _I],
     "ct_pooling_backward": [_P, _P, _D, _P, _P, _P, C.POINTER(CtPoolDesc), _L, _L, _L, _L, _L, _L, _I],
+    "ct_lrn_forward": [_P, _P, _DP, _P, _DP, _I, _D, _D, _D, _I],
+    "ct_lrn_backward": [_P, _P, _DP, _P, _DP, _P, _DP, _P, _DP, _I, _D, _D, _D, _I],
     "ct_gemm": [_P, _P, _L, _I, _I, _D, _P, _L, _L, _L, _P, _L, _L, _D, _I],
     "ct_gemv": [_P, _P, _L, _I, _D, _P, _L, _L, _L, _P, _L, _D, _I],
     "ct_rand": [_P, _P, _L, _I, _I, _D, _D, C.c_uint64, C.c_uint64],

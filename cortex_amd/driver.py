@@ -353,6 +353,21 @@ class HipStream:
                   output_grad.ptr, C.byref(desc), batch, channels, in_h, in_w, out_h, out_w,
                   capi.DTYPE_CODES[output.datatype])
 
+    # -- local response normalization (tensor/math.clj:240-252); the descriptor is a plain map --
+    def lrn_forward(self, output, output_dims, input, input_dims, lrn_descriptor) -> None:
+        d = lrn_descriptor
+        capi.call("ct_lrn_forward", self.handle, output.ptr, C.byref(_dims_struct(output_dims)), input.ptr,
+                  C.byref(_dims_struct(input_dims)), int(d["n"]), float(d["k"]), float(d["alpha"]), float(d["beta"]),
+                  capi.DTYPE_CODES[output.datatype])
+
+    def lrn_backward(self, input_grad, input_grad_dims, output, output_dims, input, input_dims, output_grad,
+                     output_grad_dims, lrn_descriptor) -> None:
+        d = lrn_descriptor
+        capi.call("ct_lrn_backward", self.handle, input_grad.ptr, C.byref(_dims_struct(input_grad_dims)), output.ptr,
+                  C.byref(_dims_struct(output_dims)), input.ptr, C.byref(_dims_struct(input_dims)), output_grad.ptr,
+                  C.byref(_dims_struct(output_grad_dims)), int(d["n"]), float(d["k"]), float(d["alpha"]),
+                  float(d["beta"]), capi.DTYPE_CODES[output.datatype])
+
     # -- gemm!, gemv! (tensor/math.clj:106-123) ---------------------------------
     def gemm(self, c, c_colstride, trans_a, trans_b, alpha, a, a_row_count, a_col_count, a_colstride, b, b_col_count,
              b_colstride, beta) -> None:

@@ -426,6 +426,37 @@ class PoolingLayer:
         ct.pooling_backward(input_gradient, 0.0, input, output, output_gradient, self.pool_desc)
 
 
+def local_response_normalization(input_dimension: dict, *, k=2, n=5, alpha=1e-4, beta=0.75, **args) -> dict:
+    """The description ``layers/local-response-normalization``
+    (``src/cortex/nn/layers.clj:586-594``) writes, with its defaults; the output
+    has the input's dimensions."""
+    node = {"type": "local-response-normalization", "k": k, "n": n, "alpha": alpha, "beta": beta}
+    node.update({key.replace("_", "-"): v for key, v in args.items()})
+    node["input-dimension"] = dict(input_dimension)
+    node["output-dimension"] = dict(input_dimension)
+    return node
+
+
+class LocalResponseNormalization:
+    """``LocalResponseNormalization`` (``layers.clj:363-388``)."""
+
+    def __init__(self, layer: dict, batch_size: int):
+        self.layer, self.batch_size = layer, batch_size
+        self.lrn_desc = ct.lrn_descriptor(n=layer["n"], k=layer["k"], alpha=layer["alpha"], beta=layer["beta"])
+
+    def forward(self, parameter_buffers, input_buffers, output_buffers):
+        output = _conv_tensor(self.layer["output-dimension"], self.batch_size, first_buffer(output_buffers))
+        input = _conv_tensor(self.layer["input-dimension"], self.batch_size, first_buffer(input_buffers))
+        ct.lrn_forward(output, input, self.lrn_desc)
+
+    def backward(self, parameter_buffers, output_buffers, input_buffers):
+        output = _conv_tensor(self.layer["output-dimension"], self.batch_size, first_buffer(output_buffers))
+        input = _conv_tensor(self.layer["input-dimension"], self.batch_size, first_buffer(input_buffers))
+        output_gradient = _conv_tensor(self.layer["output-dimension"], self.batch_size, first_gradient(output_buffers))
+        input_gradient = _conv_tensor(self.layer["output-dimension"], self.batch_size, first_gradient(input_buffers))
+        ct.lrn_backward(input_gradient, output, input, output_gradient, self.lrn_desc)
+
+
 def prelu_size(layer: dict) -> int:
     """One slope per channel, or per element when there is one channel
     (``src/cortex/nn/layers.clj:241-246``)."""
@@ -595,6 +626,8 @@ def create(node: dict, batch_size: int, datatype: str = None):
         return PoolingLayer(node, batch_size, datatype)
     if kind == "convolutional":
         return ConvolutionLayer(node, batch_size, datatype)
+    if kind == "local-response-normalization":
+        return LocalResponseNormalization(node, batch_size)
     if kind == "concatenate":
         return Concatenate()
     if kind == "split":

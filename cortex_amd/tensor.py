@@ -667,6 +667,42 @@ def pooling_backward(input_gradient: Tensor, input_grad_alpha, input: Tensor, ou
     return input_gradient
 
 
+# ---------------------------------------------------------------- local response normalization
+
+def lrn_descriptor(*, n=5, k=2, alpha=1e-4, beta=0.75) -> dict:
+    """``lrn-descriptor`` (``tensor.clj:1554-1560``): the window and the three
+    constants, with the reference's defaults.  The library keeps no native
+    object for it."""
+    return {"n": int(n), "k": float(k), "alpha": float(alpha), "beta": float(beta)}
+
+
+def _lrn_shapes(*named) -> None:
+    first = named[0][1].shape()
+    if any(t.shape() != first for _, t in named[1:]):
+        raise TensorError("Input and output shapes must match " + str({name: t.shape() for name, t in named}))
+    if len(first) < 3:
+        raise TensorError(f"tensor must be of at least rank 3: {first}")
+
+
+def lrn_forward(output: Tensor, input: Tensor, lrn_desc: dict) -> Tensor:
+    """``lrn-forward!`` (``tensor.clj:1563-1583``): every value divided by
+    ``(k + alpha / n * sum of squares over the n neighbouring channels) ** beta``."""
+    _lrn_shapes(("input-shape", input), ("output-shape", output))
+    _external_library_check("lrn-forward", output, input)
+    check_stream().lrn_forward(output.buffer, output.dimensions, input.buffer, input.dimensions, lrn_desc)
+    return output
+
+
+def lrn_backward(input_gradient: Tensor, output: Tensor, input: Tensor, output_gradient: Tensor, lrn_desc: dict) -> Tensor:
+    """``lrn-backward!`` (``tensor.clj:1586-1616``)."""
+    _lrn_shapes(("input-shape", input), ("output-shape", output), ("in-grad-shape", input_gradient),
+                ("out-grad-shape", output_gradient))
+    _external_library_check("lrn-forward", output, input, input_gradient, output_gradient)
+    check_stream().lrn_backward(input_gradient.buffer, input_gradient.dimensions, output.buffer, output.dimensions,
+                                input.buffer, input.dimensions, output_gradient.buffer, output_gradient.dimensions, lrn_desc)
+    return input_gradient
+
+
 # ---------------------------------------------------------------- gemm!, gemv!
 
 def _column_stride(t: Tensor) -> int:

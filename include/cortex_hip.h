@@ -504,6 +504,30 @@ int ct_pooling_backward(void* stream, void* input_gradient, double input_gradien
                         int64_t in_height, int64_t in_width, int64_t out_height, int64_t out_width,
                         int dtype);
 
+/* lrn-forward! / lrn-backward! (tensor/math.clj:240-252; tensor.clj:1554-1616;
+ * cuda/tensor_math.clj:1277-1335, where cuDNN's cross-channel LRN does the
+ * work: the reference's CPU backend has no form of it).  Tensors are
+ * [batch, channels, height, width] or one image [channels, height, width], of
+ * equal shapes, each with its own strides; n, k, alpha and beta are the
+ * fields of the reference's lrn-descriptor (1 <= n <= 16, k > 0).  With
+ * behind = (n - 1) / 2 and window(c) = [c - behind, c + n - 1 - behind]
+ * clipped to the channels:
+ *   s[c]  = k + (alpha / n) * sum over window(c) of input^2
+ *   output[c] = input[c] * s[c]^-beta
+ *   input_gradient[c] = output_gradient[c] * s[c]^-beta
+ *       - (2 alpha beta / n) * input[c]
+ *         * sum over window(c) of output_gradient[c'] * output[c'] / s[c']
+ * (the same window in both directions, as the stored results of
+ * src/cortex/verify/tensor.clj:1105-1123 for n = 2 require).
+ * dtype is CT_F32 or CT_F64. */
+int ct_lrn_forward(void* stream, void* output, const ct_dims* output_dims, const void* input,
+                   const ct_dims* input_dims, int n, double k, double alpha, double beta, int dtype);
+int ct_lrn_backward(void* stream, void* input_gradient, const ct_dims* input_gradient_dims,
+                    const void* output, const ct_dims* output_dims, const void* input,
+                    const ct_dims* input_dims, const void* output_gradient,
+                    const ct_dims* output_gradient_dims, int n, double k, double alpha, double beta,
+                    int dtype);
+
 /* ------------------------------------------------- optimizers */
 
 /* Adam step (src/cortex/optimize/adam.clj:68-102, 116-134; resources/adam.cu).

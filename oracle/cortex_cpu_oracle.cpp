@@ -39,6 +39,8 @@
 //                            by the Random123 known-answer vectors -- the
 //                            reference draws from SecureRandom / cuRAND and
 //                            fixes only the distribution
+//   local response           no CPU form in the reference: cuDNN's published cross-channel LRN,
+//   normalization            called from cuda/tensor_math.clj:1277-1335
 //   Adam                     src/cortex/optimize/adam.clj:68-102
 //   Adadelta                 java/cortex/compute/optimize/AdadeltaOptimizer.java:29-64
 //
@@ -970,6 +972,100 @@ int convolution_t(int which, T* dest, double alpha, const T* other, const T* wei
 // Same argument lists as the library's entry points in include/cortex_hip.h
 // minus the stream; pointers are host pointers.
 
+// ------------------------------------------------------------------ local response normalization
+// lrn-forward! / lrn-backward! (tensor/math.clj:240-252; tensor.clj:1554-1616).  The reference has
+// no CPU form: its only implementation hands the tensors to cuDNN's cross-channel LRN
+// (cuda/tensor_math.clj:271-281, 1277-1335: cudnnLRNCrossChannelForward / Backward, mode
+// CUDNN_LRN_CROSS_CHANNEL_DIM1, through org.bytedeco.javacpp-presets/cuda 8.0-1.2, project.clj:12),
+// a closed library that is not under /root/reference.  What is restated here is that routine's
+// published definition (cuDNN library guide, cudnnSetLRNDescriptor / cudnnLRNCrossChannelForward;
+// the operator of Krizhevsky, Sutskever, Hinton 2012, section 3.3):
+//   window(c) = [c - floor((n-1)/2), c + n - 1 - floor((n-1)/2)], clipped to the channels
+//   s[c]      = k + (alpha / n) * sum over window(c) of x^2
+//   y[c]      = x[c] * s[c]^-beta
+//   dx[c]     = dy[c] * s[c]^-beta
+//               - (2 alpha beta / n) * x[c] * sum over window(c) of dy[c'] y[c'] / s[c']
+// evaluated in double and rounded once.  The backward sum runs over window(c) itself: for an even n,
+// whose window is not centred, the exact derivative would run over the mirrored window, and the
+// stored results for n = 2 below are those of the unmirrored one.  Tensors are [batch, channels, height, width] with any
+// strides; a rank-3 tensor is one image (cuda/driver.clj:1094-1123 pads shapes to four entries).
+// Pinned by the stored vectors of src/cortex/verify/tensor.clj:1088-1140 (n = 1, 2, 3 with
+// k = alpha = beta = 1; they fix the window's placement in both directions and both formulas) and,
+// for the other parameters, by central differences of the forward pass for odd n, where the
+// backward pass is the exact derivative (tests/test_oracle_closed_forms.py).
+struct LrnView {
+  int64_t size[4], stride[4];
+};
+
+bool lrn_view(const Dims& d, LrnView* v) {
+  if (d.nd < 3 || d.nd > 4 || !direct(d)) return false;
+  for (int i = 0; i < 4; ++i) { v->size[i] = 1; v->stride[i] = 0; }
+  for (int i = 0; i < d.nd; ++i) {
+    v->size[i + 4 - d.nd] = d.shape[i];
+    v->stride[i + 4 - d.nd] = d.strides[i];
+  }
+  return true;
+}
+
+bool lrn_same_shape(const LrnView& a, const LrnView& b) {
+  for (int i = 0; i < 4; ++i)
+    if (a.size[i] != b.size[i]) return false;
+  return true;
+}
+
+inline int64_t lrn_at(const LrnView& v, int64_t b, int64_t c, int64_t y, int64_t x) {
+  return b * v.stride[0] + c * v.stride[1] + y * v.stride[2] + x * v.stride[3];
+}
+
+template <class T>
+double lrn_scale(const T* in, const LrnView& iv, int64_t b, int64_t c, int64_t y, int64_t x, int n, double k, double alpha) {
+  const int64_t behind = (n - 1) / 2, ahead = n - 1 - behind;
+  double sum = 0.0;
+  for (int64_t w = std::max<int64_t>(0, c - behind); w <= std::min<int64_t>(iv.size[1] - 1, c + ahead); ++w) {
+    const double v = (double)in[lrn_at(iv, b, w, y, x)];
+    sum += v * v;
+  }
+  return k + (alpha / (double)n) * sum;
+}
+
+template <class T>
+int lrn_forward_t(T* out, const LrnView& ov, const T* in, const LrnView& iv, int n, double k, double alpha, double beta) {
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t b = 0; b < iv.size[0]; ++b)
+    for (int64_t c = 0; c < iv.size[1]; ++c)
+      for (int64_t y = 0; y < iv.size[2]; ++y)
+        for (int64_t x = 0; x < iv.size[3]; ++x) {
+          const double s = lrn_scale(in, iv, b, c, y, x, n, k, alpha);
+          out[lrn_at(ov, b, c, y, x)] = (T)((double)in[lrn_at(iv, b, c, y, x)] * std::pow(s, -beta));
+        }
+  return 0;
+}
+
+template <class T>
+int lrn_backward_t(T* ig, const LrnView& gv, const T* out, const LrnView& ov, const T* in, const LrnView& iv, const T* og,
+                   const LrnView& dv, int n, double k, double alpha, double beta) {
+  const int64_t behind = (n - 1) / 2, ahead = n - 1 - behind;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t b = 0; b < iv.size[0]; ++b)
+    for (int64_t c = 0; c < iv.size[1]; ++c)
+      for (int64_t y = 0; y < iv.size[2]; ++y)
+        for (int64_t x = 0; x < iv.size[3]; ++x) {
+          double cross = 0.0;
+          for (int64_t w = std::max<int64_t>(0, c - behind); w <= std::min<int64_t>(iv.size[1] - 1, c + ahead); ++w)
+            cross += (double)og[lrn_at(dv, b, w, y, x)] * (double)out[lrn_at(ov, b, w, y, x)] /
+                     lrn_scale(in, iv, b, w, y, x, n, k, alpha);
+          const double s = lrn_scale(in, iv, b, c, y, x, n, k, alpha);
+          const double direct_term = (double)og[lrn_at(dv, b, c, y, x)] * std::pow(s, -beta);
+          ig[lrn_at(gv, b, c, y, x)] =
+              (T)(direct_term - (2.0 * alpha * beta / (double)n) * (double)in[lrn_at(iv, b, c, y, x)] * cross);
+        }
+  return 0;
+}
+
+bool lrn_params_ok(int n, double k, double alpha, double beta) {
+  return n >= 1 && n <= 16 && k > 0.0 && std::isfinite(alpha) && std::isfinite(beta);
+}
+
 #define LOAD(name, src)        \
   Dims name;                   \
   if (!load_dims(src, &name)) return fail("bad dimensions: " #src)
@@ -1412,6 +1508,41 @@ int co_convolution_backward_data(void* input_gradient, double, const void* outpu
                                  int64_t batch_count, int64_t in_height, int64_t in_width, int64_t out_height,
                                  int64_t out_width, int dtype) {
   CONV_ENTRY(2, input_gradient, 0.0, output_gradient, weights);
+}
+
+int co_lrn_forward(void* output, const ct_dims* output_dims, const void* input, const ct_dims* input_dims, int n, double k,
+                   double alpha, double beta, int dtype) {
+  LOAD(od, output_dims);
+  LOAD(id, input_dims);
+  LrnView ov, iv;
+  if (!lrn_view(od, &ov) || !lrn_view(id, &iv)) return fail("lrn: tensor must be of rank 3 or 4 with direct dimensions");
+  if (!lrn_same_shape(ov, iv)) return fail("lrn: Input and output shapes must match");
+  if (!lrn_params_ok(n, k, alpha, beta)) return fail("lrn: bad descriptor");
+  if (dtype == CT_F32) return lrn_forward_t<float>((float*)output, ov, (const float*)input, iv, n, k, alpha, beta);
+  if (dtype == CT_F64) return lrn_forward_t<double>((double*)output, ov, (const double*)input, iv, n, k, alpha, beta);
+  return fail("lrn-forward is only defined for float and double tensors");
+}
+
+int co_lrn_backward(void* input_gradient, const ct_dims* input_gradient_dims, const void* output, const ct_dims* output_dims,
+                    const void* input, const ct_dims* input_dims, const void* output_gradient,
+                    const ct_dims* output_gradient_dims, int n, double k, double alpha, double beta, int dtype) {
+  LOAD(gd, input_gradient_dims);
+  LOAD(od, output_dims);
+  LOAD(id, input_dims);
+  LOAD(dd, output_gradient_dims);
+  LrnView gv, ov, iv, dv;
+  if (!lrn_view(gd, &gv) || !lrn_view(od, &ov) || !lrn_view(id, &iv) || !lrn_view(dd, &dv))
+    return fail("lrn: tensor must be of rank 3 or 4 with direct dimensions");
+  if (!lrn_same_shape(gv, iv) || !lrn_same_shape(ov, iv) || !lrn_same_shape(dv, iv))
+    return fail("lrn: Input and output shapes must match");
+  if (!lrn_params_ok(n, k, alpha, beta)) return fail("lrn: bad descriptor");
+  if (dtype == CT_F32)
+    return lrn_backward_t<float>((float*)input_gradient, gv, (const float*)output, ov, (const float*)input, iv,
+                                 (const float*)output_gradient, dv, n, k, alpha, beta);
+  if (dtype == CT_F64)
+    return lrn_backward_t<double>((double*)input_gradient, gv, (const double*)output, ov, (const double*)input, iv,
+                                  (const double*)output_gradient, dv, n, k, alpha, beta);
+  return fail("lrn-backward is only defined for float and double tensors");
 }
 
 // One Philox4x32-10 block, for the known-answer tests.

@@ -258,6 +258,15 @@ def pooling_backward(side, ig: View, inp: View, out: View, og: View, desc, batch
               channels, in_h, in_w, out_h, out_w, ig.buf.dtype)
 
 
+def lrn_forward(side, out: View, inp: View, n, k, alpha, beta):
+    side.call("lrn_forward", *_pd(side, out), *_pd(side, inp), int(n), float(k), float(alpha), float(beta), out.buf.dtype)
+
+
+def lrn_backward(side, ig: View, out: View, inp: View, og: View, n, k, alpha, beta):
+    side.call("lrn_backward", *_pd(side, ig), *_pd(side, out), *_pd(side, inp), *_pd(side, og), int(n), float(k),
+              float(alpha), float(beta), out.buf.dtype)
+
+
 def batch_normalize(side, out: View, inp: View, means: View, variances: View, scale: View, bias: View, epsilon,
                     batch, channels, elements=None):
     """elements=None selects the eltwise form ([batch, channels] with one statistic per element)."""

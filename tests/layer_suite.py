@@ -105,6 +105,20 @@ def pool_layer_basic(driver, datatype):
         equals([v for _ in range(batch_size) for g in range(1, 5) for v in (g, 0, 0, 0)], r["input-gradient"])
 
 
+# verify/nn/layers.clj:766-812: (layers/input 2 2 3) under k = alpha = beta = 1
+def lrn_forward(driver, datatype):
+    with context(driver, datatype):
+        batch_size, dimension = 2, {"channels": 3, "height": 2, "width": 2}
+        values = [float(v) for v in range(12)] * batch_size
+        want = GOLDEN["lrn_operator"]
+        for lrn_n in (1, 2, 3):
+            node = nl.local_response_normalization(dimension, n=lrn_n, k=1, alpha=1, beta=1)
+            r = single(node, batch_size, values, [1.0] * len(values), item_shape=[3, 2, 2])
+            expected = [v / (1 + v * v) for v in values] if lrn_n == 1 else want[f"n{lrn_n}_output"] * batch_size
+            equals(expected, r["output"], 1e-4)
+            equals(want[f"n{lrn_n}_input_gradient"] * batch_size, r["input-gradient"], 1e-4)
+
+
 # verify/nn/layers.clj:593-611
 def pool_layer_avg(driver, datatype):
     with context(driver, datatype):

@@ -229,6 +229,15 @@ class OracleStream:
                 C.byref(capi.make_pool_desc(desc)), batch, channels, in_h, in_w, out_h, out_w,
                 capi.DTYPE_CODES[out.datatype])
 
+    def lrn_forward(self, out, od, inp, idims, desc):
+        ob.call("lrn_forward", out.ptr, C.byref(_dims(od)), inp.ptr, C.byref(_dims(idims)), int(desc["n"]),
+                float(desc["k"]), float(desc["alpha"]), float(desc["beta"]), capi.DTYPE_CODES[out.datatype])
+
+    def lrn_backward(self, ig, igd, out, od, inp, idims, og, ogd, desc):
+        ob.call("lrn_backward", ig.ptr, C.byref(_dims(igd)), out.ptr, C.byref(_dims(od)), inp.ptr, C.byref(_dims(idims)),
+                og.ptr, C.byref(_dims(ogd)), int(desc["n"]), float(desc["k"]), float(desc["alpha"]), float(desc["beta"]),
+                capi.DTYPE_CODES[out.datatype])
+
     def gemm(self, c, ldc, ta, tb, alpha, a, a_rows, a_cols, lda, b, b_cols, ldb, beta):
         ob.call("gemm", c.ptr, int(ldc), int(bool(ta)), int(bool(tb)), float(alpha), a.ptr, int(a_rows), int(a_cols),
                 int(lda), b.ptr, int(b_cols), int(ldb), float(beta), capi.DTYPE_CODES[c.datatype])

@@ -304,6 +304,27 @@ def pooling_operator(driver, datatype):
             equals(want[key + "_backward"], ct.to_double_array(input_gradient), 1e-4)
 
 
+# verify/tensor.clj:1068-1140
+def lrn_operator(driver, datatype):
+    with context(driver, datatype):
+        want = GOLDEN["lrn_operator"]
+        batch_size, channels, dim = 2, 3, 2
+        n_input = channels * dim * dim
+        input_data = [float(v) for v in range(n_input)] * batch_size
+        for lrn_n in (1, 2, 3):
+            inp = ct.to_tensor(np.asarray(input_data).reshape(batch_size, channels, dim, dim))
+            output_gradient = ct.to_tensor(np.ones((batch_size, channels, dim, dim)))
+            output, input_gradient = ct.new_tensor(ct.shape(inp)), ct.new_tensor(ct.shape(inp))
+            desc = ct.lrn_descriptor(n=lrn_n, k=1, alpha=1, beta=1)
+            ct.lrn_forward(output, inp, desc)
+            ct.lrn_backward(input_gradient, output, inp, output_gradient, desc)
+            if lrn_n == 1:
+                equals([v / (1 + v * v) for v in input_data], ct.to_double_array(output), 1e-4)
+            else:
+                equals(want[f"n{lrn_n}_output"] * batch_size, ct.to_double_array(output), 1e-4)
+            equals(want[f"n{lrn_n}_input_gradient"] * batch_size, ct.to_double_array(input_gradient), 1e-4)
+
+
 # verify/tensor.clj:252-283; also exercises sub-matrices
 def gemm(driver, datatype):
     with context(driver, datatype):

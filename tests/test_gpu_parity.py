@@ -3,6 +3,8 @@ ABI, on identical seeded inputs.  Bar: bit-exact for integer work, for
 assign / convert / select / indexing and for the non-transcendental float ops;
 <= 2e-6 relative for exp / tanh / logistic and for reductions.  Needs a GPU.
 """
+import re
+
 import numpy as np
 import pytest
 
@@ -745,6 +747,82 @@ def test_softmax_rows(P, code, shape):
         assert kern == "softmax_lane" if k < 8 else kern in ("softmax_wave", "softmax_wave_vec", "softmax_block", "softmax_block_reg")
     P.run(H.softmax, View(x, [rows, k]), View(x, [rows, k]))     # in place
     compare(x, f"softmax {shape} in place", tol=tol)
+
+
+# shape [batch, channels, height, width] (or one image), window, k, alpha, beta
+LRN_CASES = [((2, 3, 2, 2), 1, 1.0, 1.0, 1.0), ((2, 3, 2, 2), 2, 1.0, 1.0, 1.0), ((2, 3, 2, 2), 3, 1.0, 1.0, 1.0),
+             ((3, 96, 8, 8), 5, 2.0, 1e-4, 0.75), ((2, 70, 7, 9), 5, 2.0, 1e-2, 0.75), ((1, 33, 5, 4), 4, 1.0, 0.5, 0.5),
+             ((2, 40, 16, 16), 16, 1.5, 0.3, 0.6), ((2, 5, 3, 3), 16, 1.0, 1.0, 1.0), ((4, 64, 1, 1), 9, 1.0, 0.1, 2.0),
+             ((37, 12, 12), 6, 1.0, 1.0, 0.75), ((2, 65, 10, 26), 7, 1e-3, 5.0, 0.9), ((1, 1, 4, 4), 3, 2.0, 1.0, 0.75)]
+
+
+@pytest.mark.parametrize("code", FLOATS)
+@pytest.mark.parametrize("case", LRN_CASES, ids=str)
+def test_lrn_forward_and_backward(P, code, case):
+    """Local response normalization against the oracle: the reference's own small cases, windows of
+    every parity up to 16 (wider than the channel count included), channel counts off the 32-channel
+    blocks, planes that are and are not whole vectors, one-image rank-3 tensors.  The float kernels
+    take the power through the hardware exp2 / log2 and the reciprocal: 4e-6 of the result, relative to
+    the larger of the two terms of the gradient; double tensors 1e-12."""
+    shape, n, k, alpha, beta = case
+    rng = np.random.default_rng(61)
+    count = int(np.prod(shape))
+    x = P.buf((rng.standard_normal(count) * 3).astype(NP[code]))
+    dy = P.buf(rng.standard_normal(count).astype(NP[code]))
+    y = P.buf(np.zeros(count, NP[code]))
+    dx = P.buf(np.zeros(count, NP[code]))
+    tol = 4e-6 if code == capi.F32 else 1e-12
+    kern = P.run(H.lrn_forward, View(y, shape), View(x, shape), n, k, alpha, beta)
+    plane = int(np.prod(shape[-2:]))
+    assert kern == ("lrn_forward_vec" if plane % (16 // x.init.itemsize) == 0 else "lrn_forward")
+    compare(y, f"lrn forward {case}", tol=tol)
+    y.upload(y.host)   # both sides differentiate the same stored output
+    kern = P.run(H.lrn_backward, View(dx, shape), View(y, shape), View(x, shape), View(dy, shape), n, k, alpha, beta)
+    assert kern == ("lrn_backward_vec" if plane % (16 // x.init.itemsize) == 0 else "lrn_backward")
+    got, want = dx.download().astype(np.float64), dx.host.astype(np.float64)
+    # the gradient is a difference of two terms: the bar is relative to their magnitudes
+    xs = x.host.astype(np.float64).reshape((-1,) + tuple(shape[-3:]))
+    ys, gs = y.host.astype(np.float64).reshape(xs.shape), dy.host.astype(np.float64).reshape(xs.shape)
+    behind = (n - 1) // 2
+    ahead = n - 1 - behind
+    sq = np.pad(xs * xs, ((0, 0), (behind, ahead), (0, 0), (0, 0)))
+    scale = k + alpha / n * sum(sq[:, w:w + xs.shape[1]] for w in range(n))
+    ratio = np.pad(np.abs(gs * ys) / scale, ((0, 0), (behind, ahead), (0, 0), (0, 0)))
+    cross = sum(ratio[:, w:w + xs.shape[1]] for w in range(n))
+    bar = tol * (np.abs(gs) * scale ** -beta + 2 * alpha * beta / n * np.abs(xs) * cross)
+    assert np.all(np.abs(got - want) <= bar.reshape(-1) + 1e-300), f"lrn backward {case}: {np.max(np.abs(got - want) / (bar.reshape(-1) + 1e-300)) * tol}"
+
+
+@pytest.mark.parametrize("code", FLOATS)
+def test_lrn_strided_tensors_and_errors(P, code):
+    """Every tensor with its own strides (padded planes, padded channels, a transposed plane), which
+    takes the one-element-per-lane kernels, and the calls the library refuses."""
+    rng = np.random.default_rng(62)
+    b, c, h, w = 2, 35, 6, 8
+    tol = 4e-6 if code == capi.F32 else 1e-12
+    big = b * (c + 2) * (h + 1) * (w + 3)
+    x = P.buf((rng.standard_normal(big) * 2).astype(NP[code]))
+    y = P.buf(np.zeros(big, NP[code]))
+    dy = P.buf(rng.standard_normal(b * c * h * w).astype(NP[code]))
+    dx = P.buf(np.zeros(b * c * h * w, NP[code]))
+    xv = View(x, [b, c, h, w], [(c + 2) * (h + 1) * (w + 3), (h + 1) * (w + 3), w + 3, 1], offset=5)
+    yv = View(y, [b, c, h, w], [(c + 1) * h * w + 7, h * w, 1, h])       # planes stored column by column
+    kern = P.run(H.lrn_forward, yv, xv, 5, 2.0, 1e-2, 0.75)
+    assert kern == "lrn_forward"
+    compare(y, "lrn forward strided", tol=tol)
+    y.upload(y.host)
+    kern = P.run(H.lrn_backward, View(dx, [b, c, h, w]), yv, xv, View(dy, [b, c, h, w]), 5, 2.0, 1e-2, 0.75)
+    assert kern == "lrn_backward"
+    compare(dx, "lrn backward strided", tol=2e-4 if code == capi.F32 else 1e-10)
+    shape = [b, c, h, w]
+    for bad, text in (((View(y, [b, c, h, w]), View(x, [b, c, h * w]), 5, 2.0, 1e-4, 0.75), "shapes must match"),
+                      ((View(y, [b * c, h * w]), View(x, [b * c, h * w]), 5, 2.0, 1e-4, 0.75), "at least rank 3"),
+                      ((View(y, shape), View(x, shape), 0, 2.0, 1e-4, 0.75), "outside [1, 16]"),
+                      ((View(y, shape), View(x, shape), 17, 2.0, 1e-4, 0.75), "outside [1, 16]"),
+                      ((View(y, shape), View(x, shape), 5, 0.0, 1e-4, 0.75), "below 1e-5"),
+                      ((View(x, shape), View(x, shape), 5, 2.0, 1e-4, 0.75), "may not be the input")):
+        with pytest.raises(capi.CortexHipError, match=re.escape(text)):
+            H.lrn_forward(P.hip, *bad)
 
 
 @pytest.mark.parametrize("code", FLOATS)

@@ -820,3 +820,90 @@ def test_convolution_matches_correlation(geometry):
         o2, w2 = hbuf(np.zeros(out.host.size)), hbuf(np.zeros(work.host.size))
         H.convolution(ORACLE, "forward", V(o2), 0.0, V(hbuf(bumped)), V(weights), V(w2), *geom)
         assert abs(np.dot(o2.host - out.host, g.reshape(-1)) / eps - ig.host[idx]) < 1e-5
+
+
+# ------------------------------------------------------------------ local response normalization
+# The reference's stored vectors (tests/reference_suite.py lrn_operator) fix k = alpha = beta = 1 and
+# n = 1, 2, 3 on three channels.  These pin the other parameters through what the mathematics fixes.
+
+def _lrn(x, dy, n, k, alpha, beta):
+    xb, gb = hbuf(x.reshape(-1)), hbuf(dy.reshape(-1))
+    yb, db = hbuf(np.zeros(x.size)), hbuf(np.zeros(x.size))
+    shape = list(x.shape)
+    H.lrn_forward(ORACLE, View(yb, shape), View(xb, shape), n, k, alpha, beta)
+    H.lrn_backward(ORACLE, View(db, shape), View(yb, shape), View(xb, shape), View(gb, shape), n, k, alpha, beta)
+    return yb.host.reshape(x.shape), db.host.reshape(x.shape)
+
+
+def test_lrn_window_of_one_is_elementwise():
+    """n = 1: y = x (k + alpha x^2)^-beta and its derivative, element by element."""
+    rng = np.random.default_rng(71)
+    x, dy = rng.standard_normal((2, 5, 3, 4)) * 2, rng.standard_normal((2, 5, 3, 4))
+    k, alpha, beta = 1.7, 0.3, 0.75
+    y, dx = _lrn(x, dy, 1, k, alpha, beta)
+    s = k + alpha * x * x
+    np.testing.assert_allclose(y, x * s ** -beta, rtol=1e-14)
+    np.testing.assert_allclose(dx, dy * (s ** -beta - 2 * alpha * beta * x * x * s ** (-beta - 1)), rtol=1e-12, atol=1e-15)
+
+
+def test_lrn_window_wider_than_the_channels_sees_all_of_them():
+    """With n >= 2 C - 1 every window, clipped to the channels, is all of them: one scale per pixel,
+    k + alpha / n * (sum over all channels of x^2)."""
+    rng = np.random.default_rng(72)
+    x = rng.standard_normal((3, 4, 2, 5))
+    for n in (7, 8, 16):
+        y, _ = _lrn(x, np.ones_like(x), n, 2.0, 0.5, 0.6)
+        s = 2.0 + 0.5 / n * (x * x).sum(axis=1, keepdims=True)
+        np.testing.assert_allclose(y, x * s ** -0.6, rtol=1e-14)
+
+
+def test_lrn_window_placement_by_impulse_response():
+    """One non-zero channel c0: the scales that rise above k are exactly those of the channels whose
+    window holds c0, c0 - ahead <= c <= c0 + behind with behind = (n - 1) // 2 (cuDNN's lookBehind) and
+    ahead = n - 1 - behind."""
+    channels, c0 = 12, 6
+    for n in range(1, 9):
+        x = np.full((1, channels, 1, 1), 1e-3)
+        x[0, c0] = 10.0
+        y, _ = _lrn(x, np.ones_like(x), n, 1.0, 1.0, 1.0)
+        scale = (x / y).reshape(-1)            # s, since beta = 1
+        behind = (n - 1) // 2
+        ahead = n - 1 - behind
+        raised = {c for c in range(channels) if scale[c] > 2.0}
+        assert raised == set(range(c0 - ahead, c0 + behind + 1)), (n, raised)
+
+
+@pytest.mark.parametrize("n", [1, 3, 5, 7, 15])
+def test_lrn_backward_against_central_differences(n):
+    """For an odd n the window is centred and the backward pass is the exact derivative of
+    sum(dy * forward(x)): checked against central differences in double.  (For an even n the stored
+    vectors of the reference fix the unmirrored window, which is not that derivative.)"""
+    rng = np.random.default_rng(73 + n)
+    shape = (2, 9, 2, 3)
+    x, dy = rng.standard_normal(shape), rng.standard_normal(shape)
+    k, alpha, beta = 1.3, 0.8, 0.75
+    _, dx = _lrn(x, dy, n, k, alpha, beta)
+    h = 1e-6
+    numeric = np.zeros(shape)
+    for idx in np.ndindex(*shape):
+        hi, lo = x.copy(), x.copy()
+        hi[idx] += h
+        lo[idx] -= h
+        numeric[idx] = ((dy * _lrn(hi, dy, n, k, alpha, beta)[0]).sum() - (dy * _lrn(lo, dy, n, k, alpha, beta)[0]).sum()) / (2 * h)
+    np.testing.assert_allclose(dx, numeric, rtol=2e-6, atol=2e-8)
+
+
+def test_lrn_rank_three_is_one_image_and_strides_are_honoured():
+    rng = np.random.default_rng(74)
+    x = rng.standard_normal((6, 3, 4))
+    y3, _ = _lrn(x, np.ones_like(x), 3, 1.0, 1.0, 0.5)
+    y4, _ = _lrn(x.reshape(1, 6, 3, 4), np.ones((1, 6, 3, 4)), 3, 1.0, 1.0, 0.5)
+    assert np.array_equal(y3.reshape(-1), y4.reshape(-1))
+    # the same tensor stored channels-last: [b, c, h, w] strides [h w c, 1, w c, c]
+    b, c, hh, w = 2, 5, 3, 4
+    x = rng.standard_normal((b, c, hh, w))
+    want, _ = _lrn(x, np.ones_like(x), 3, 1.0, 1.0, 0.5)
+    xb, yb = hbuf(np.ascontiguousarray(x.transpose(0, 2, 3, 1)).reshape(-1)), hbuf(np.zeros(x.size))
+    strides = [hh * w * c, 1, w * c, c]
+    H.lrn_forward(ORACLE, View(yb, [b, c, hh, w], strides), View(xb, [b, c, hh, w], strides), 3, 1.0, 1.0, 0.5)
+    assert np.array_equal(yb.host.reshape(b, hh, w, c).transpose(0, 3, 1, 2), want)

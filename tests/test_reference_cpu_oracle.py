@@ -11,13 +11,13 @@ ALL_DTYPE_TESTS = ["assign_constant", "assign_marshal", "binary_constant_op", "b
                    "ternary_op_select", "unary_reduce", "transpose", "select", "select_transpose_interaction",
                    "indexed_tensor", "simple_stream"]
 FLOAT_TESTS = ["gemm", "gemv", "activation_forward", "activation_gradient", "softmax", "batch_normalize",
-               "batch_normalize_update_and_apply", "batch_normalize_gradients", "convolution_operator", "pooling_operator", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
+               "batch_normalize_update_and_apply", "batch_normalize_gradients", "convolution_operator", "pooling_operator", "lrn_operator", "magnitude_and_mag_squared", "constrain_inside_hypersphere", "operations_sugar",
                "adam_trajectory", "sgd_closed_form"]
 
 # tests/layer_suite.py: the layers, loss gradients and regularisers built on the tensor calls
 LAYER_TESTS = ["relu_activation", "linear", "activations", "activations_batch", "softmax", "softmax_channels",
                "dropout_bernoulli", "dropout_gaussian", "batch_normalization", "batch_normalization_running",
-               "batch_normalization_spatial", "prelu", "basic_conv_layer", "pool_layer_basic", "pool_layer_avg", "pool_layer_avg_exc_pad",
+               "batch_normalization_spatial", "prelu", "basic_conv_layer", "pool_layer_basic", "pool_layer_avg", "pool_layer_avg_exc_pad", "lrn_forward",
                "concatenate", "split", "join_add", "join_add_ragged", "join_multiply", "loss_gradients",
                "train_small_network"]
 
