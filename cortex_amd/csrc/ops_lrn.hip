@@ -15,15 +15,18 @@
 // definition here.
 //
 // Both directions are streams: 8 bytes per float element forward (read x, write y), 16 backward
-// (read x, y, dy, write dx).  A block takes 32 channels of 64 pixel vectors of one image and keeps
-// the rows it needs in LDS: the 32 + n - 1 rows of x around its channels (forward), or the
-// 32 + 2 (n - 1) rows of x and the 32 + n - 1 rows of dy y / s (backward).  Every lane issues all
-// of its loads before the first use, a lane's LDS accesses are 16 bytes wide and conflict-free
+// (read x, y, dy, write dx).  A block takes CH = 16 or 32 channels of 64 pixel vectors of one image
+// and keeps the rows it needs in LDS: the CH + n - 1 rows of x around its channels (forward), or
+// the CH + 2 (n - 1) rows of x and the CH + n - 1 rows of dy y / s (backward).  The x rows go from
+// global memory straight into LDS (global_load_lds_dwordx4), all of a wave's rows issued at once;
+// a lane's LDS accesses are 16 bytes wide and conflict-free
 // (a wave reads one contiguous 1 KiB row), and the window sums are re-formed from their n terms
 // for every channel: a running sum with subtraction would carry the error of large neighbours
-// into small windows.  The sums run in double (the squares of floats are exact there); the power
-// for float tensors is exp2(-beta * log2 s) with s split into exponent and fraction so that its
-// relative error stays near two units in the last place over the whole range of s.
+// into small windows.  Double tensors compute in double throughout.  Float tensors compute in float
+// on the hardware's exp2 / log2 / reciprocal units (about 20 instructions per element; the same
+// arithmetic in double is 45 and bounds the kernel instead of memory), with a double path for
+// the values where that would cost accuracy (see lrn_scales): results stay within 4e-6 of the
+// double evaluation, relative to the terms that form them.
 #include <atomic>
 
 #include "elementwise.h"
@@ -31,12 +34,16 @@
 namespace cthip {
 namespace {
 
-constexpr int kLrnChannels = 32;   // output channels per block
 constexpr int kLrnMaxWindow = 16;  // cuDNN's CUDNN_LRN_MAX_N
-constexpr int kLrnWaves = kBlock / 64;
-// rows of the wider of the two register-resident tiles a wave walks: 32 + 16 - 1 channels over 4 waves
-constexpr int kLrnRowsPerWave = (kLrnChannels + kLrnMaxWindow - 1 + kLrnWaves - 1) / kLrnWaves;
-constexpr int kLrnXRowsPerWave = (kLrnChannels + 2 * (kLrnMaxWindow - 1) + kLrnWaves - 1) / kLrnWaves;
+constexpr int kLrnWaves = kBlock / 64;  // of the forward kernel
+
+// Output channels per block.  Sixteen keep four to eight blocks on a compute unit, which hides the
+// tiles' load-then-compute phases behind each other; the extra rows read around them (n - 1 of
+// 16 + n - 1) come out of the caches.  Windows past 8 take 32.  Measured on float
+// [64,256,56,56], n 5: forward 73 us with 16 channels against 77 with 32 and 99-106 with 64;
+// backward, where LDS holds two tiles, 165 against 175 (eight waves per block; 194 / 217 with
+// four, 183 / 202 with sixteen).
+inline int lrn_channels_per_block(bool vec_ok, int n) { return vec_ok && n <= 8 ? 16 : 32; }
 
 struct LrnOperand {
   const void* ptr;
@@ -51,6 +58,7 @@ struct LrnArgs {
   uint32_t p_tiles, c_chunks;
   FastDiv p_tiles_fd, c_chunks_fd, width_fd;
   double k, alpha_over_n, beta, cross_scale;  // cross_scale = 2 alpha beta / n
+  float k_f, alpha_over_n_f, beta_f, cross_scale_f;
   int32_t beta_is_one;
 };
 
@@ -72,17 +80,6 @@ template <class T> __device__ __forceinline__ T lrn_power(double s, double beta,
   }
 }
 
-// 1 / s in double precision for double tensors, to float precision otherwise, as a double.
-template <class T> __device__ __forceinline__ double lrn_reciprocal(double s) {
-  if constexpr (std::is_same<T, double>::value) {
-    return 1.0 / s;
-  } else {
-    int e;
-    const float m = (float)frexp(s, &e);
-    return ldexp((double)__builtin_amdgcn_rcpf(m), -e);
-  }
-}
-
 template <int VEC> __device__ __forceinline__ int64_t lrn_pixel_offset(const LrnOperand& t, const FastDiv& width_fd, uint32_t pv) {
   if constexpr (VEC > 1) {
     return (int64_t)pv * VEC;  // planes are contiguous on this path
@@ -93,14 +90,78 @@ template <int VEC> __device__ __forceinline__ int64_t lrn_pixel_offset(const Lrn
   }
 }
 
+// The scale s of one lane's vector at tile row `first` (the window is rows first .. first + n - 1
+// of the x tile) and s^-beta.  Double tensors sum and take the power in double.  Float tensors sum
+// the squares with float multiply-adds (no term cancels: n - 1 roundings at most) and take
+// exp2(-beta log2 s) on the hardware units while |beta log2 s| <= 16, where the error of the
+// product in the exponent stays under 1.5e-6 of the result; beyond that, and for sums past the
+// float range, the lane recomputes the sum in double and splits s as lrn_power does.
+template <class T, int VEC>
+__device__ __forceinline__ void lrn_scales(const LrnArgs& a, const Vec<T, VEC>* xt, int first, int lane, T* scale, T* power) {
+  using V = Vec<T, VEC>;
+  if constexpr (std::is_same<T, double>::value) {
+    double sum[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sum[e] = 0.0;
+    for (int w = 0; w < a.window; ++w) {
+      const V t = xt[(first + w) * 64 + lane];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum[e] += t.v[e] * t.v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      scale[e] = a.k + a.alpha_over_n * sum[e];
+      power[e] = lrn_power<double>(scale[e], a.beta, a.beta_is_one != 0);
+    }
+  } else {
+    float sum[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sum[e] = 0.0f;
+    for (int w = 0; w < a.window; ++w) {
+      const V t = xt[(first + w) * 64 + lane];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum[e] = __builtin_fmaf(t.v[e], t.v[e], sum[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float s = __builtin_fmaf(a.alpha_over_n_f, sum[e], a.k_f);
+      const float exponent = -a.beta_f * __builtin_amdgcn_logf(s);
+      if (s < 1e30f && __builtin_fabsf(exponent) <= 16.0f) {
+        scale[e] = s;
+        power[e] = __builtin_amdgcn_exp2f(exponent);
+      } else {
+        double wide = 0.0;
+        for (int w = 0; w < a.window; ++w) {
+          const double t = (double)xt[(first + w) * 64 + lane].v[e];
+          wide += t * t;
+        }
+        const double sd = a.k + a.alpha_over_n * wide;
+        scale[e] = (float)sd;  // may round to infinity: its reciprocal is then 0, as the exact quotient rounds
+        power[e] = lrn_power<float>(sd, a.beta, a.beta_is_one != 0);
+      }
+    }
+  }
+}
+
 __device__ __forceinline__ void lrn_block_place(const LrnArgs& a, uint32_t* image, uint32_t* chunk, uint32_t* tile) {
   uint32_t q;
   a.p_tiles_fd.divmod(blockIdx.x, q, *tile);
   a.c_chunks_fd.divmod(q, *image, *chunk);
 }
 
-template <class T, int VEC>
+// One row of a tile straight from global memory into LDS (gfx950's global_load_lds_dwordx4): the
+// wave's 64 lanes bring 16 bytes each to consecutive places after `row`, with no register in
+// between and no LDS store instruction.  `row` is the same for the whole wave; lanes that are
+// switched off leave their places as they were.
+template <class V> __device__ __forceinline__ void lrn_row_to_lds(const V* from, V* row) {
+  static_assert(sizeof(V) == 16, "direct loads into LDS move 16 bytes per lane here");
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)from,
+                                   (__attribute__((address_space(3))) void*)row, 16, 0, 0);
+}
+
+template <class T, int VEC, int CH>
 __global__ void __launch_bounds__(kBlock) lrn_forward_kernel(const LrnArgs a) {
+  constexpr int kRows = (CH + kLrnMaxWindow - 1 + kLrnWaves - 1) / kLrnWaves;
   using V = Vec<T, VEC>;
   extern __shared__ __align__(16) char lrn_smem[];
   V* xt = reinterpret_cast<V*>(lrn_smem);  // [rows_x][64]
@@ -109,57 +170,63 @@ __global__ void __launch_bounds__(kBlock) lrn_forward_kernel(const LrnArgs a) {
   lrn_block_place(a, &image, &chunk, &tile);
   const uint32_t pv = tile * 64 + lane;
   const bool live = pv < a.pixel_vecs;
-  const int c0 = (int)chunk * kLrnChannels;
-  const int rows_x = kLrnChannels + a.window - 1;
+  const int c0 = (int)chunk * CH;
+  const int rows_x = CH + a.window - 1;
   const T* xp = reinterpret_cast<const T*>(a.x.ptr) + (int64_t)image * a.x.sb + lrn_pixel_offset<VEC>(a.x, a.width_fd, live ? pv : 0);
-  V held[kLrnRowsPerWave];
+  if constexpr (VEC > 1) {
+    V zero;
 #pragma unroll
-  for (int q = 0; q < kLrnRowsPerWave; ++q) {
-    const int j = wave + q * kLrnWaves;
-    const int c = c0 - a.behind + j;
+    for (int e = 0; e < VEC; ++e) zero.v[e] = (T)0;
+    for (int j = wave; j < rows_x; j += kLrnWaves) {
+      const int c = c0 - a.behind + j;
+      if (c >= 0 && c < a.channels) {
+        if (live) lrn_row_to_lds(reinterpret_cast<const V*>(xp + (int64_t)c * a.x.sc), xt + j * 64);
+      } else {
+        xt[j * 64 + lane] = zero;
+      }
+    }
+  } else {
+    V held[kRows];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) held[q].v[e] = (T)0;
-    if (j < rows_x && live && c >= 0 && c < a.channels) held[q] = *reinterpret_cast<const V*>(xp + (int64_t)c * a.x.sc);
-  }
+    for (int q = 0; q < kRows; ++q) {
+      const int j = wave + q * kLrnWaves;
+      const int c = c0 - a.behind + j;
+      held[q].v[0] = (T)0;
+      if (j < rows_x && live && c >= 0 && c < a.channels) held[q] = *reinterpret_cast<const V*>(xp + (int64_t)c * a.x.sc);
+    }
 #pragma unroll
-  for (int q = 0; q < kLrnRowsPerWave; ++q) {
-    const int j = wave + q * kLrnWaves;
-    if (j < rows_x) xt[j * 64 + lane] = held[q];
+    for (int q = 0; q < kRows; ++q) {
+      const int j = wave + q * kLrnWaves;
+      if (j < rows_x) xt[j * 64 + lane] = held[q];
+    }
   }
   __syncthreads();
   if (!live) return;
   T* yp = reinterpret_cast<T*>(const_cast<void*>(a.y.ptr)) + (int64_t)image * a.y.sb + lrn_pixel_offset<VEC>(a.y, a.width_fd, pv);
 #pragma unroll
-  for (int q = 0; q < kLrnChannels / kLrnWaves; ++q) {
+  for (int q = 0; q < CH / kLrnWaves; ++q) {
     const int i = wave + q * kLrnWaves;
     const int c = c0 + i;
     if (c >= a.channels) break;
-    double sum[VEC];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) sum[e] = 0.0;
-    for (int w = 0; w < a.window; ++w) {
-      const V t = xt[(i + w) * 64 + lane];
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) sum[e] += (double)t.v[e] * (double)t.v[e];
-    }
+    T scale[VEC], power[VEC];
+    lrn_scales<T, VEC>(a, xt, i, lane, scale, power);
     const V centre = xt[(i + a.behind) * 64 + lane];
     V out;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      const double s = a.k + a.alpha_over_n * sum[e];
-      out.v[e] = (T)(centre.v[e] * lrn_power<T>(s, a.beta, a.beta_is_one != 0));
-    }
+    for (int e = 0; e < VEC; ++e) out.v[e] = centre.v[e] * power[e];
     *reinterpret_cast<V*>(yp + (int64_t)c * a.y.sc) = out;
   }
 }
 
-template <class T, int VEC>
-__global__ void __launch_bounds__(kBlock) lrn_backward_kernel(const LrnArgs a) {
+template <class T, int VEC, int CH, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) lrn_backward_kernel(const LrnArgs a) {
+  constexpr int kRows = (CH + kLrnMaxWindow - 1 + WAVES - 1) / WAVES;
+  constexpr int kXRows = (CH + 2 * (kLrnMaxWindow - 1) + WAVES - 1) / WAVES;
   using V = Vec<T, VEC>;
   using R = Vec<T, VEC>;  // dy y / s, kept in the tensor's type
   extern __shared__ __align__(16) char lrn_smem[];
-  const int rows_x = kLrnChannels + 2 * (a.window - 1);
-  const int rows_r = kLrnChannels + a.window - 1;
+  const int rows_x = CH + 2 * (a.window - 1);
+  const int rows_r = CH + a.window - 1;
   V* xt = reinterpret_cast<V*>(lrn_smem);  // [rows_x][64], row j is channel c0 - 2 behind + j
   R* rt = reinterpret_cast<R*>(xt + rows_x * 64);  // [rows_r][64], row j is channel c0 - behind + j
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -167,23 +234,38 @@ __global__ void __launch_bounds__(kBlock) lrn_backward_kernel(const LrnArgs a) {
   lrn_block_place(a, &image, &chunk, &tile);
   const uint32_t pv = tile * 64 + lane;
   const bool live = pv < a.pixel_vecs;
-  const int c0 = (int)chunk * kLrnChannels;
+  const int c0 = (int)chunk * CH;
   const uint32_t pv0 = live ? pv : 0;
   const T* xp = reinterpret_cast<const T*>(a.x.ptr) + (int64_t)image * a.x.sb + lrn_pixel_offset<VEC>(a.x, a.width_fd, pv0);
   const T* yp = reinterpret_cast<const T*>(a.y.ptr) + (int64_t)image * a.y.sb + lrn_pixel_offset<VEC>(a.y, a.width_fd, pv0);
   const T* gp = reinterpret_cast<const T*>(a.dy.ptr) + (int64_t)image * a.dy.sb + lrn_pixel_offset<VEC>(a.dy, a.width_fd, pv0);
-  V xheld[kLrnXRowsPerWave], yheld[kLrnRowsPerWave], gheld[kLrnRowsPerWave];
+  V yheld[kRows], gheld[kRows];
+  if constexpr (VEC > 1) {
+    V zero;
 #pragma unroll
-  for (int q = 0; q < kLrnXRowsPerWave; ++q) {
-    const int j = wave + q * kLrnWaves;
-    const int c = c0 - 2 * a.behind + j;
+    for (int e = 0; e < VEC; ++e) zero.v[e] = (T)0;
+    for (int j = wave; j < rows_x; j += WAVES) {
+      const int c = c0 - 2 * a.behind + j;
+      if (c >= 0 && c < a.channels) {
+        if (live) lrn_row_to_lds(reinterpret_cast<const V*>(xp + (int64_t)c * a.x.sc), xt + j * 64);
+      } else {
+        xt[j * 64 + lane] = zero;
+      }
+    }
+  }
+  V xheld[VEC > 1 ? 1 : kXRows];
+  if constexpr (VEC == 1) {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) xheld[q].v[e] = (T)0;
-    if (j < rows_x && live && c >= 0 && c < a.channels) xheld[q] = *reinterpret_cast<const V*>(xp + (int64_t)c * a.x.sc);
+    for (int q = 0; q < kXRows; ++q) {
+      const int j = wave + q * WAVES;
+      const int c = c0 - 2 * a.behind + j;
+      xheld[q].v[0] = (T)0;
+      if (j < rows_x && live && c >= 0 && c < a.channels) xheld[q] = *reinterpret_cast<const V*>(xp + (int64_t)c * a.x.sc);
+    }
   }
 #pragma unroll
-  for (int q = 0; q < kLrnRowsPerWave; ++q) {
-    const int j = wave + q * kLrnWaves;
+  for (int q = 0; q < kRows; ++q) {
+    const int j = wave + q * WAVES;
     const int c = c0 - a.behind + j;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) { yheld[q].v[e] = (T)0; gheld[q].v[e] = (T)0; }
@@ -192,35 +274,31 @@ __global__ void __launch_bounds__(kBlock) lrn_backward_kernel(const LrnArgs a) {
       gheld[q] = *reinterpret_cast<const V*>(gp + (int64_t)c * a.dy.sc);
     }
   }
+  if constexpr (VEC == 1) {
 #pragma unroll
-  for (int q = 0; q < kLrnXRowsPerWave; ++q) {
-    const int j = wave + q * kLrnWaves;
-    if (j < rows_x) xt[j * 64 + lane] = xheld[q];
+    for (int q = 0; q < kXRows; ++q) {
+      const int j = wave + q * WAVES;
+      if (j < rows_x) xt[j * 64 + lane] = xheld[q];
+    }
   }
   __syncthreads();
   // dy y / s of this wave's rows goes to LDS; dy s^-beta stays in gheld for the rows that are outputs
 #pragma unroll
-  for (int q = 0; q < kLrnRowsPerWave; ++q) {
-    const int j = wave + q * kLrnWaves;
+  for (int q = 0; q < kRows; ++q) {
+    const int j = wave + q * WAVES;
     if (j >= rows_r) break;
     const int c = c0 - a.behind + j;
     R ratio;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) ratio.v[e] = (T)0;
     if (live && c >= 0 && c < a.channels) {
-      double sum[VEC];
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) sum[e] = 0.0;
-      for (int w = 0; w < a.window; ++w) {
-        const V t = xt[(j + w) * 64 + lane];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) sum[e] += (double)t.v[e] * (double)t.v[e];
-      }
+      T scale[VEC], power[VEC];
+      lrn_scales<T, VEC>(a, xt, j, lane, scale, power);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        const double s = a.k + a.alpha_over_n * sum[e];
-        ratio.v[e] = (T)((double)gheld[q].v[e] * (double)yheld[q].v[e] * lrn_reciprocal<T>(s));
-        gheld[q].v[e] = (T)(gheld[q].v[e] * lrn_power<T>(s, a.beta, a.beta_is_one != 0));
+        if constexpr (std::is_same<T, double>::value) ratio.v[e] = gheld[q].v[e] * yheld[q].v[e] / scale[e];
+        else ratio.v[e] = gheld[q].v[e] * yheld[q].v[e] * __builtin_amdgcn_rcpf(scale[e]);
+        gheld[q].v[e] = gheld[q].v[e] * power[e];
       }
     }
     rt[j * 64 + lane] = ratio;
@@ -229,25 +307,27 @@ __global__ void __launch_bounds__(kBlock) lrn_backward_kernel(const LrnArgs a) {
   if (!live) return;
   T* dp = reinterpret_cast<T*>(const_cast<void*>(a.dx.ptr)) + (int64_t)image * a.dx.sb + lrn_pixel_offset<VEC>(a.dx, a.width_fd, pv);
 #pragma unroll
-  for (int q = 0; q < kLrnRowsPerWave; ++q) {
-    const int j = wave + q * kLrnWaves;
+  for (int q = 0; q < kRows; ++q) {
+    const int j = wave + q * WAVES;
     if (j >= rows_r) break;
     const int i = j - a.behind;  // output row: channel c0 + i
     const int c = c0 + i;
-    if (i < 0 || i >= kLrnChannels || c >= a.channels) continue;
-    double cross[VEC];
+    if (i < 0 || i >= CH || c >= a.channels) continue;
+    T cross[VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) cross[e] = 0.0;
+    for (int e = 0; e < VEC; ++e) cross[e] = (T)0;
     for (int w = 0; w < a.window; ++w) {
       const R t = rt[(i + w) * 64 + lane];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) cross[e] += (double)t.v[e];
+      for (int e = 0; e < VEC; ++e) cross[e] += t.v[e];
     }
     const V centre = xt[(i + 2 * a.behind) * 64 + lane];
     V out;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e)
-      out.v[e] = (T)((double)gheld[q].v[e] - a.cross_scale * (double)centre.v[e] * cross[e]);
+    for (int e = 0; e < VEC; ++e) {
+      if constexpr (std::is_same<T, double>::value) out.v[e] = gheld[q].v[e] - a.cross_scale * centre.v[e] * cross[e];
+      else out.v[e] = gheld[q].v[e] - a.cross_scale_f * centre.v[e] * cross[e];
+    }
     *reinterpret_cast<V*>(dp + (int64_t)c * a.dx.sc) = out;
   }
 }
@@ -286,7 +366,7 @@ template <class T> bool lrn_vector_ok(const LrnOperand& t, const LrnShape& s, in
          ((uintptr_t)t.ptr % (uintptr_t)(vec * sizeof(T))) == 0;
 }
 
-int lrn_fill(LrnArgs* a, const LrnShape& s, int n, double k, double alpha, double beta, int vec) {
+int lrn_fill(LrnArgs* a, const LrnShape& s, int n, double k, double alpha, double beta, int vec, int ch) {
   CT_REQUIRE(n >= 1 && n <= kLrnMaxWindow, "lrn: n = %d is outside [1, %d]", n, kLrnMaxWindow);
   CT_REQUIRE(k >= 1e-5, "lrn: k = %g is below 1e-5", k);  // cuDNN's CUDNN_LRN_MIN_K
   CT_REQUIRE(alpha == alpha && beta == beta && alpha - alpha == 0.0 && beta - beta == 0.0, "lrn: alpha and beta must be finite");
@@ -299,7 +379,7 @@ int lrn_fill(LrnArgs* a, const LrnShape& s, int n, double k, double alpha, doubl
   a->pixels = (uint32_t)pixels;
   a->pixel_vecs = (uint32_t)(pixels / vec);
   a->p_tiles = (a->pixel_vecs + 63) / 64;
-  a->c_chunks = (uint32_t)((s.size[1] + kLrnChannels - 1) / kLrnChannels);
+  a->c_chunks = (uint32_t)((s.size[1] + ch - 1) / ch);
   a->p_tiles_fd = FastDiv(a->p_tiles);
   a->c_chunks_fd = FastDiv(a->c_chunks);
   a->width_fd = FastDiv((uint32_t)s.size[3]);
@@ -308,6 +388,10 @@ int lrn_fill(LrnArgs* a, const LrnShape& s, int n, double k, double alpha, doubl
   a->beta = beta;
   a->cross_scale = 2.0 * alpha * beta / (double)n;
   a->beta_is_one = beta == 1.0 ? 1 : 0;
+  a->k_f = (float)k;
+  a->alpha_over_n_f = (float)a->alpha_over_n;
+  a->beta_f = (float)beta;
+  a->cross_scale_f = (float)a->cross_scale;
   const int64_t grid = (int64_t)a->p_tiles * a->c_chunks * s.size[0];
   CT_REQUIRE(grid < (int64_t(1) << 31), "lrn: tensor too large");
   return CT_OK;
@@ -315,7 +399,7 @@ int lrn_fill(LrnArgs* a, const LrnShape& s, int n, double k, double alpha, doubl
 
 // A launch may ask for more than 64 KiB of dynamic LDS only after the kernel's limit has been
 // raised, once per kernel and device (the backward tiles of wide windows need up to 109 KiB).
-constexpr size_t kLrnBackwardMaxLds = (size_t)(2 * kLrnChannels + 3 * (kLrnMaxWindow - 1)) * 64 * 16;
+constexpr size_t kLrnBackwardMaxLds = (size_t)(2 * 32 + 3 * (kLrnMaxWindow - 1)) * 64 * 16;
 template <auto Kernel> int lrn_allow_lds(size_t bytes) {
   static std::atomic<uint64_t> raised{0};
   int dev = 0;
@@ -332,12 +416,14 @@ int lrn_forward_run(hipStream_t st, LrnArgs& a, const LrnShape& s, int n, double
   constexpr int VMAX = 16 / (int)sizeof(T);
   const bool vec_ok = lrn_vector_ok<T>(a.x, s, VMAX) && lrn_vector_ok<T>(a.y, s, VMAX);
   const int vec = vec_ok ? VMAX : 1;
-  if (int rc = lrn_fill(&a, s, n, k, alpha, beta, vec)) return rc;
+  const int ch = lrn_channels_per_block(vec_ok, n);
+  if (int rc = lrn_fill(&a, s, n, k, alpha, beta, vec, ch)) return rc;
   const dim3 grid((uint32_t)((int64_t)a.p_tiles * a.c_chunks * s.size[0]));
-  const size_t lds = (size_t)(kLrnChannels + n - 1) * 64 * vec * sizeof(T);
+  const size_t lds = (size_t)(ch + n - 1) * 64 * vec * sizeof(T);  // at most 47 KiB
   note_kernel(vec_ok ? "lrn_forward_vec" : "lrn_forward");
-  if (vec_ok) hipLaunchKernelGGL((lrn_forward_kernel<T, VMAX>), grid, dim3(kBlock), lds, st, a);
-  else hipLaunchKernelGGL((lrn_forward_kernel<T, 1>), grid, dim3(kBlock), lds, st, a);
+  if (!vec_ok) hipLaunchKernelGGL((lrn_forward_kernel<T, 1, 32>), grid, dim3(kBlock), lds, st, a);
+  else if (ch == 16) hipLaunchKernelGGL((lrn_forward_kernel<T, VMAX, 16>), grid, dim3(kBlock), lds, st, a);
+  else hipLaunchKernelGGL((lrn_forward_kernel<T, VMAX, 32>), grid, dim3(kBlock), lds, st, a);
   return after_launch(st);
 }
 
@@ -347,15 +433,19 @@ int lrn_backward_run(hipStream_t st, LrnArgs& a, const LrnShape& s, int n, doubl
   const bool vec_ok = lrn_vector_ok<T>(a.x, s, VMAX) && lrn_vector_ok<T>(a.y, s, VMAX) && lrn_vector_ok<T>(a.dy, s, VMAX) &&
                       lrn_vector_ok<T>(a.dx, s, VMAX);
   const int vec = vec_ok ? VMAX : 1;
-  if (int rc = lrn_fill(&a, s, n, k, alpha, beta, vec)) return rc;
+  const int ch = lrn_channels_per_block(vec_ok, n);
+  if (int rc = lrn_fill(&a, s, n, k, alpha, beta, vec, ch)) return rc;
   const dim3 grid((uint32_t)((int64_t)a.p_tiles * a.c_chunks * s.size[0]));
-  const size_t lds = (size_t)(2 * kLrnChannels + 3 * (n - 1)) * 64 * vec * sizeof(T);
+  const size_t lds = (size_t)(2 * ch + 3 * (n - 1)) * 64 * vec * sizeof(T);
   note_kernel(vec_ok ? "lrn_backward_vec" : "lrn_backward");
-  if (vec_ok) {
-    if (int rc = lrn_allow_lds<lrn_backward_kernel<T, VMAX>>(kLrnBackwardMaxLds)) return rc;
-    hipLaunchKernelGGL((lrn_backward_kernel<T, VMAX>), grid, dim3(kBlock), lds, st, a);
+  if (!vec_ok) {
+    hipLaunchKernelGGL((lrn_backward_kernel<T, 1, 32, 4>), grid, dim3(4 * 64), lds, st, a);
+  } else if (ch == 16) {
+    if (int rc = lrn_allow_lds<lrn_backward_kernel<T, VMAX, 16, 8>>(kLrnBackwardMaxLds)) return rc;
+    hipLaunchKernelGGL((lrn_backward_kernel<T, VMAX, 16, 8>), grid, dim3(8 * 64), lds, st, a);
   } else {
-    hipLaunchKernelGGL((lrn_backward_kernel<T, 1>), grid, dim3(kBlock), lds, st, a);
+    if (int rc = lrn_allow_lds<lrn_backward_kernel<T, VMAX, 32, 8>>(kLrnBackwardMaxLds)) return rc;
+    hipLaunchKernelGGL((lrn_backward_kernel<T, VMAX, 32, 8>), grid, dim3(8 * 64), lds, st, a);
   }
   return after_launch(st);
 }

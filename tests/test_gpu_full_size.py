@@ -488,3 +488,41 @@ def test_indexed_rows_of_2_31_bytes_gathered_and_scattered():
         capi.call("ct_free", out)
         for t in (d_idx, d_table, d_sums):
             t.free()
+
+
+def test_lrn_at_benchmark_size():
+    """lrn-forward! and lrn-backward! on bench.py's [64, 256, 56, 56] float tensor (n 5, k 2, alpha 1e-4,
+    beta 0.75: the reference's defaults) against the oracle; alpha 1e-2 as well so that the window sums
+    weigh as much as k.  Forward within 4e-6 of the result; backward within 4e-6 of the magnitudes of
+    its two terms (bounded here by |dy| s^-beta + 2 alpha beta |x| max|dy y| / k)."""
+    shape = [64, 256, 56, 56]
+    count = int(np.prod(shape))
+    rng = np.random.default_rng(91)
+    x = (rng.standard_normal(count, dtype=np.float32) * 4).astype(np.float32)
+    dy = rng.standard_normal(count, dtype=np.float32)
+    d_x, d_dy = Dev(x), Dev(dy)
+    d_y, d_dx = Dev(np.zeros(count, np.float32)), Dev(np.zeros(count, np.float32))
+    dm = dims(shape)
+    try:
+        for alpha in (1e-4, 1e-2):
+            capi.call("ct_lrn_forward", None, d_y.ptr, C.byref(dm), d_x.ptr, C.byref(dm), 5, 2.0, alpha, 0.75, capi.F32)
+            assert capi.last_kernel() == "lrn_forward_vec"
+            want_y = np.zeros(count, np.float32)
+            ob.call("lrn_forward", want_y.ctypes.data, C.byref(dm), x.ctypes.data, C.byref(dm), 5, 2.0, alpha, 0.75, capi.F32)
+            got_y = d_y.download()
+            assert np.all(np.abs(got_y.astype(np.float64) - want_y) <= 4e-6 * np.abs(want_y.astype(np.float64)))
+            d_y.host[:] = want_y   # both sides differentiate the same stored output
+            capi.call("ct_memcpy_async", d_y.ptr, want_y.ctypes.data, want_y.nbytes, capi.COPY_H2D, None)
+            capi.call("ct_lrn_backward", None, d_dx.ptr, C.byref(dm), d_y.ptr, C.byref(dm), d_x.ptr, C.byref(dm), d_dy.ptr,
+                      C.byref(dm), 5, 2.0, alpha, 0.75, capi.F32)
+            assert capi.last_kernel() == "lrn_backward_vec"
+            want_dx = np.zeros(count, np.float32)
+            ob.call("lrn_backward", want_dx.ctypes.data, C.byref(dm), want_y.ctypes.data, C.byref(dm), x.ctypes.data,
+                    C.byref(dm), dy.ctypes.data, C.byref(dm), 5, 2.0, alpha, 0.75, capi.F32)
+            got_dx = d_dx.download().astype(np.float64)
+            bar = 4e-6 * (np.abs(dy.astype(np.float64)) + 2 * alpha * 0.75 * np.abs(x.astype(np.float64)) *
+                          float(np.max(np.abs(dy.astype(np.float64) * want_y))) / 2.0)
+            assert np.all(np.abs(got_dx - want_dx) <= bar)
+    finally:
+        for t in (d_x, d_dy, d_y, d_dx):
+            t.free()
