@@ -62,22 +62,21 @@ struct LrnArgs {
   int32_t beta_is_one;
 };
 
-// s^-beta for s > 0.  Float tensors: s = m 2^e with m in [1/2, 1); -beta (e + log2 m) is split into
-// an integer and a fraction in [-1/2, 1/2] in double, and the hardware exp2 of the fraction is
-// scaled by the integer.  Double tensors take the library's pow.
-template <class T> __device__ __forceinline__ T lrn_power(double s, double beta, bool beta_is_one) {
-  if constexpr (std::is_same<T, double>::value) {
-    return beta_is_one ? 1.0 / s : pow(s, -beta);
-  } else {
-    int e;
-    const float m = (float)frexp(s, &e);  // [1/2, 1)
-    if (beta_is_one) return __builtin_ldexpf(__builtin_amdgcn_rcpf(m), -e);
-    const double a = -beta * ((double)e + (double)__builtin_amdgcn_logf(m));
-    const double whole = __builtin_rint(a);
-    const float frac = (float)(a - whole);
-    const double clipped = __builtin_fmin(__builtin_fmax(whole, -300.0), 300.0);
-    return __builtin_ldexpf(__builtin_amdgcn_exp2f(frac), (int)clipped);
-  }
+// s^-beta for s > 0, for the lanes of float tensors that leave the hardware path (see lrn_scales):
+// s = m 2^e with m in [1/2, 1); -beta (e + log2 m) is split into an integer and a fraction in
+// [-1/2, 1/2] in double, and the hardware exp2 of the fraction is scaled by the integer.  The
+// result stays a double: it may lie far outside the float range while its product with a large
+// or small tensor value lies inside.
+__device__ __forceinline__ double lrn_power_wide(double s, double beta, bool beta_is_one) {
+  if (s > 1.7e308) return beta > 0.0 ? 0.0 : (beta < 0.0 ? s : 1.0);  // an infinite scale: pow(inf, -beta)
+  int e;
+  const float m = (float)frexp(s, &e);  // [1/2, 1)
+  if (beta_is_one) return ldexp((double)__builtin_amdgcn_rcpf(m), -e);
+  const double a = -beta * ((double)e + (double)__builtin_amdgcn_logf(m));
+  const double whole = __builtin_rint(a);
+  const float frac = (float)(a - whole);
+  const double clipped = __builtin_fmin(__builtin_fmax(whole, -2000.0), 2000.0);
+  return ldexp((double)__builtin_amdgcn_exp2f(frac), (int)clipped);
 }
 
 template <int VEC> __device__ __forceinline__ int64_t lrn_pixel_offset(const LrnOperand& t, const FastDiv& width_fd, uint32_t pv) {
@@ -94,10 +93,12 @@ template <int VEC> __device__ __forceinline__ int64_t lrn_pixel_offset(const Lrn
 // of the x tile) and s^-beta.  Double tensors sum and take the power in double.  Float tensors sum
 // the squares with float multiply-adds (no term cancels: n - 1 roundings at most) and take
 // exp2(-beta log2 s) on the hardware units while |beta log2 s| <= 16, where the error of the
-// product in the exponent stays under 1.5e-6 of the result; beyond that, and for sums past the
-// float range, the lane recomputes the sum in double and splits s as lrn_power does.
+// product in the exponent stays under 1.5e-6 of the result.  Beyond that, and for sums past the
+// float range, wide[e] is set to the scale recomputed in double (0 otherwise) and the caller forms
+// its products with lrn_power_wide in double.
 template <class T, int VEC>
-__device__ __forceinline__ void lrn_scales(const LrnArgs& a, const Vec<T, VEC>* xt, int first, int lane, T* scale, T* power) {
+__device__ __forceinline__ void lrn_scales(const LrnArgs& a, const Vec<T, VEC>* xt, int first, int lane, T* scale, T* power,
+                                           double* wide) {
   using V = Vec<T, VEC>;
   if constexpr (std::is_same<T, double>::value) {
     double sum[VEC];
@@ -111,7 +112,8 @@ __device__ __forceinline__ void lrn_scales(const LrnArgs& a, const Vec<T, VEC>* 
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       scale[e] = a.k + a.alpha_over_n * sum[e];
-      power[e] = lrn_power<double>(scale[e], a.beta, a.beta_is_one != 0);
+      power[e] = a.beta_is_one ? 1.0 / scale[e] : pow(scale[e], -a.beta);
+      wide[e] = 0.0;
     }
   } else {
     float sum[VEC];
@@ -126,18 +128,16 @@ __device__ __forceinline__ void lrn_scales(const LrnArgs& a, const Vec<T, VEC>* 
     for (int e = 0; e < VEC; ++e) {
       const float s = __builtin_fmaf(a.alpha_over_n_f, sum[e], a.k_f);
       const float exponent = -a.beta_f * __builtin_amdgcn_logf(s);
-      if (s < 1e30f && __builtin_fabsf(exponent) <= 16.0f) {
-        scale[e] = s;
-        power[e] = __builtin_amdgcn_exp2f(exponent);
-      } else {
-        double wide = 0.0;
+      scale[e] = s;
+      power[e] = __builtin_amdgcn_exp2f(exponent);
+      wide[e] = 0.0;
+      if (!(s < 1e30f && __builtin_fabsf(exponent) <= 16.0f)) {
+        double total = 0.0;
         for (int w = 0; w < a.window; ++w) {
           const double t = (double)xt[(first + w) * 64 + lane].v[e];
-          wide += t * t;
+          total += t * t;
         }
-        const double sd = a.k + a.alpha_over_n * wide;
-        scale[e] = (float)sd;  // may round to infinity: its reciprocal is then 0, as the exact quotient rounds
-        power[e] = lrn_power<float>(sd, a.beta, a.beta_is_one != 0);
+        wide[e] = a.k + a.alpha_over_n * total;
       }
     }
   }
@@ -221,11 +221,15 @@ __global__ void __launch_bounds__(kBlock) lrn_forward_kernel(const LrnArgs a) {
     const int c = c0 + i;
     if (c >= a.channels) break;
     T scale[VEC], power[VEC];
-    lrn_scales<T, VEC>(a, xt, i, lane, scale, power);
+    double wide[VEC];
+    lrn_scales<T, VEC>(a, xt, i, lane, scale, power, wide);
     const V centre = xt[(i + a.behind) * 64 + lane];
     V out;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) out.v[e] = centre.v[e] * power[e];
+    for (int e = 0; e < VEC; ++e) {
+      out.v[e] = centre.v[e] * power[e];
+      if (wide[e] != 0.0) out.v[e] = (T)((double)centre.v[e] * lrn_power_wide(wide[e], a.beta, a.beta_is_one != 0));
+    }
     *reinterpret_cast<V*>(yp + (int64_t)c * a.y.sc) = out;
   }
 }
@@ -305,12 +309,18 @@ __global__ void __launch_bounds__(WAVES * 64) lrn_backward_kernel(const LrnArgs 
     for (int e = 0; e < VEC; ++e) ratio.v[e] = (T)0;
     if (live && c >= 0 && c < a.channels) {
       T scale[VEC], power[VEC];
-      lrn_scales<T, VEC>(a, xt, j, lane, scale, power);
+      double wide[VEC];
+      lrn_scales<T, VEC>(a, xt, j, lane, scale, power, wide);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        if constexpr (std::is_same<T, double>::value) ratio.v[e] = gheld[q].v[e] * yheld[q].v[e] / scale[e];
-        else ratio.v[e] = gheld[q].v[e] * yheld[q].v[e] * __builtin_amdgcn_rcpf(scale[e]);
-        gheld[q].v[e] = gheld[q].v[e] * power[e];
+        const T g = gheld[q].v[e];
+        if constexpr (std::is_same<T, double>::value) ratio.v[e] = g * yheld[q].v[e] / scale[e];
+        else ratio.v[e] = g * yheld[q].v[e] * __builtin_amdgcn_rcpf(scale[e]);
+        gheld[q].v[e] = g * power[e];
+        if (wide[e] != 0.0) {
+          ratio.v[e] = (T)((double)g * (double)yheld[q].v[e] / wide[e]);
+          gheld[q].v[e] = (T)((double)g * lrn_power_wide(wide[e], a.beta, a.beta_is_one != 0));
+        }
       }
     }
     rt[j * 64 + lane] = ratio;

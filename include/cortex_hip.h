@@ -518,7 +518,9 @@ int ct_pooling_backward(void* stream, void* input_gradient, double input_gradien
  *       - (2 alpha beta / n) * input[c]
  *         * sum over window(c) of output_gradient[c'] * output[c'] / s[c']
  * (the same window in both directions, as the stored results of
- * src/cortex/verify/tensor.clj:1105-1123 for n = 2 require).
+ * src/cortex/verify/tensor.clj:1105-1123 for n = 2 require).  The backward
+ * pass keeps output_gradient * output / s of every channel in the tensor's
+ * type before summing: for float tensors a quotient below 1e-45 counts as 0.
  * dtype is CT_F32 or CT_F64. */
 int ct_lrn_forward(void* stream, void* output, const ct_dims* output_dims, const void* input,
                    const ct_dims* input_dims, int n, double k, double alpha, double beta, int dtype);

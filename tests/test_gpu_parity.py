@@ -779,18 +779,69 @@ def test_lrn_forward_and_backward(P, code, case):
     y.upload(y.host)   # both sides differentiate the same stored output
     kern = P.run(H.lrn_backward, View(dx, shape), View(y, shape), View(x, shape), View(dy, shape), n, k, alpha, beta)
     assert kern == ("lrn_backward_vec" if plane % (16 // x.init.itemsize) == 0 else "lrn_backward")
+    assert_lrn_gradient(dx, x, y, dy, case, tol)
+
+
+def assert_lrn_gradient(dx, x, y, dy, case, tol):
+    """The gradient is a difference of two terms, dy s^-beta and (2 alpha beta / n) x sum(dy y / s):
+    the bar is `tol` of the sum of their magnitudes, formed here in double."""
+    shape, n, k, alpha, beta = case
     got, want = dx.download().astype(np.float64), dx.host.astype(np.float64)
-    # the gradient is a difference of two terms: the bar is relative to their magnitudes
     xs = x.host.astype(np.float64).reshape((-1,) + tuple(shape[-3:]))
     ys, gs = y.host.astype(np.float64).reshape(xs.shape), dy.host.astype(np.float64).reshape(xs.shape)
     behind = (n - 1) // 2
     ahead = n - 1 - behind
-    sq = np.pad(xs * xs, ((0, 0), (behind, ahead), (0, 0), (0, 0)))
-    scale = k + alpha / n * sum(sq[:, w:w + xs.shape[1]] for w in range(n))
-    ratio = np.pad(np.abs(gs * ys) / scale, ((0, 0), (behind, ahead), (0, 0), (0, 0)))
-    cross = sum(ratio[:, w:w + xs.shape[1]] for w in range(n))
-    bar = tol * (np.abs(gs) * scale ** -beta + 2 * alpha * beta / n * np.abs(xs) * cross)
-    assert np.all(np.abs(got - want) <= bar.reshape(-1) + 1e-300), f"lrn backward {case}: {np.max(np.abs(got - want) / (bar.reshape(-1) + 1e-300)) * tol}"
+    with np.errstate(over="ignore", invalid="ignore"):
+        sq = np.pad(xs * xs, ((0, 0), (behind, ahead), (0, 0), (0, 0)))
+        scale = k + alpha / n * sum(sq[:, w:w + xs.shape[1]] for w in range(n))
+        ratio = np.pad(np.abs(gs * ys) / scale, ((0, 0), (behind, ahead), (0, 0), (0, 0)))
+        cross = sum(ratio[:, w:w + xs.shape[1]] for w in range(n))
+        bar = tol * (np.abs(gs) * scale ** -beta + 2 * alpha * beta / n * np.abs(xs) * cross)
+    tiny = float(np.finfo(dx.host.dtype).smallest_subnormal)
+    worst = np.max(np.abs(got - want) / (bar.reshape(-1) + 2 * tiny))
+    assert worst <= 1.0, f"lrn backward {case}: {worst * tol} of the terms' magnitudes"
+
+
+@pytest.mark.parametrize("code", FLOATS)
+def test_lrn_wide_range(P, code):
+    """Inputs from 1e-20 to 1e20 in neighbouring channels, a large beta and a tiny k: the scales run
+    from 1e-5 to past the float range (where the float kernels leave their hardware exp2 / log2 path
+    for the double one), and the window sums must not carry a large neighbour's error into a window
+    of small values.  NaN and infinite inputs give what the double evaluation gives.  The backward pass
+    is run over twelve orders of magnitude (see below)."""
+    rng = np.random.default_rng(63)
+    b, c, h, w = 2, 24, 4, 4
+    tol = 4e-6 if code == capi.F32 else 1e-12
+    mags = 10.0 ** rng.integers(-20, 21, (b, c, 1, 1)).astype(np.float64)
+    v = (rng.standard_normal((b, c, h, w)) * mags).astype(NP[code])
+    for n, k, alpha, beta in ((5, 1e-5, 1.0, 0.75), (3, 2.0, 1e-4, 3.0), (8, 1.0, 10.0, 0.5)):
+        x = P.buf(v.reshape(-1))
+        y = P.buf(np.zeros(v.size, NP[code]))
+        P.run(H.lrn_forward, View(y, [b, c, h, w]), View(x, [b, c, h, w]), n, k, alpha, beta)
+        compare(y, f"lrn forward wide range n {n} beta {beta}", tol=tol, denormal_ulps=2)
+    # The backward pass keeps dy y / s of every channel in the tensor's type: for float tensors the
+    # range of neighbouring channels is held to twelve orders of magnitude here, so that no such
+    # quotient leaves the float range while its product with a neighbour's x still counts.
+    mags = 10.0 ** rng.integers(-6, 7, (b, c, 1, 1)).astype(np.float64)
+    v = (rng.standard_normal((b, c, h, w)) * mags).astype(NP[code])
+    for n, k, alpha, beta in ((5, 1e-5, 1.0, 0.75), (3, 2.0, 1e-4, 3.0), (8, 1.0, 10.0, 0.5)):
+        x = P.buf(v.reshape(-1))
+        y = P.buf(np.zeros(v.size, NP[code]))
+        P.run(H.lrn_forward, View(y, [b, c, h, w]), View(x, [b, c, h, w]), n, k, alpha, beta)
+        y.upload(y.host)
+        dy = P.buf(rng.standard_normal(v.size).astype(NP[code]))
+        dx = P.buf(np.zeros(v.size, NP[code]))
+        P.run(H.lrn_backward, View(dx, [b, c, h, w]), View(y, [b, c, h, w]), View(x, [b, c, h, w]), View(dy, [b, c, h, w]),
+              n, k, alpha, beta)
+        assert_lrn_gradient(dx, x, y, dy, ([b, c, h, w], n, k, alpha, beta), tol)
+    special = v.copy()
+    special[0, 3, 1, 1] = np.nan
+    special[0, 9, 2, 2] = np.inf
+    special[1, 5, 0, 3] = -np.inf
+    x = P.buf(special.reshape(-1))
+    y = P.buf(np.zeros(v.size, NP[code]))
+    P.run(H.lrn_forward, View(y, [b, c, h, w]), View(x, [b, c, h, w]), 5, 2.0, 1e-4, 0.75)
+    compare(y, "lrn forward with NaN and infinities", tol=tol, denormal_ulps=2)
 
 
 @pytest.mark.parametrize("code", FLOATS)
