@@ -99,6 +99,7 @@ ACCUM_CASES = [
     (4096, 1000, 128, "accum_grouped_vec"),
     (20000, 50, 8, "accum_grouped_vec"),      # more index entries than the ranking kernel takes: radix sort
     (9000, 9000, 4, "accum_grouped_vec"),     # no duplicates at all
+    (131075, 40000, 4, "accum_grouped_vec"),  # many entries, few duplicates, a count off every power of two
     (300, 1, 20, "accum_grouped_vec"),        # every row lands on one destination row
 ]
 
