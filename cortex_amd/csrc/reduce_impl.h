@@ -432,6 +432,68 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
   }
 }
 
+// Few rows under many columns ([16, 4194304] summed over its rows): every lane owns VEC columns
+// and walks all k rows itself, first to last as the reference does, eight loads in flight.  No
+// segments, no LDS, no second launch; a block of 256 lanes covers 256 * VEC consecutive columns.
+// (With the kernel above a block of sixteen waves would meet for one row each: 30 % of the memory
+// rate on that shape against 56-60 % here, and 66-78 % where the row pitch is no power of two:
+// [16, 4198400], [64, 1050624], [32, 2000000].  Sixteen loads in flight change nothing.)  ColArgs as above with n_strips counted in blocks of 256 lanes;
+// vec_out: the results of a lane are neighbours in the output and go out as one vector.
+template <class P, int VEC>
+__global__ void __launch_bounds__(kBlock) reduce_col_thin_kernel(const ColArgs a, const typename P::Alpha alpha, const int vec_out) {
+  using T = typename P::Elem;
+  using A = typename P::Acc;
+  using V = Vec<T, VEC>;
+  uint32_t rest, strip;
+  a.strips_fd.divmod(blockIdx.x, rest, strip);
+  int64_t base = 0, pbase = 0;
+  for (int d = 0; d < a.n_rest; ++d) {
+    uint32_t q, r;
+    a.rsize[d].divmod(rest, q, r);
+    rest = q;
+    base += (int64_t)r * a.rstride_in[d];
+    pbase += (int64_t)r * a.r_pmul[d];
+  }
+  const uint32_t col = (strip * kBlock + threadIdx.x) * VEC;
+  if (col >= a.u) return;
+  A acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = P::identity();
+  const T* p = reinterpret_cast<const T*>(a.in) + base + col;
+  constexpr int UN = 8;
+  int64_t r = 0;
+  for (; r + UN <= a.k; r += UN, p += UN * a.rstride) {
+    V x[UN];
+#pragma unroll
+    for (int j = 0; j < UN; ++j) x[j] = nt_load(reinterpret_cast<const V*>(p + j * a.rstride));
+#pragma unroll
+    for (int j = 0; j < UN; ++j)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
+  }
+  if (r < a.k) {
+    V x[UN];
+#pragma unroll
+    for (int j = 0; j < UN; ++j)
+      if (r + j < a.k) x[j] = nt_load(reinterpret_cast<const V*>(p + j * a.rstride));
+#pragma unroll
+    for (int j = 0; j < UN; ++j)
+      if (r + j < a.k) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
+      }
+  }
+  if (vec_out) {
+    V out;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) out.v[e] = P::finish(acc[e], a.k);
+    *reinterpret_cast<V*>(reinterpret_cast<T*>(a.out) + pbase + col) = out;
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) store_output<P>(a.out, a.oa, pbase + (int64_t)(col + e) * a.u_pmul, acc[e], a.k);
+  }
+}
+
 // Short rows stored back to back (a dense [rows, k] block of at most 128 bytes per row) whose
 // length is no whole number of 16-byte vectors, ten classes say.  A block stages its 256 rows, one
 // contiguous stretch of memory, through LDS with 128-bit accesses; one lane then owns a row in LDS
@@ -756,6 +818,19 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
       ++a.n_rest;
     }
     const int vec = vec_ok ? VMAX : 1;
+    // few rows, and columns enough for four blocks per compute unit without cutting the rows
+    const int64_t thin_strips = ((int64_t)a.u + kBlock * vec - 1) / (kBlock * vec);
+    if (k <= 128 && thin_strips * rest_count >= 1024 && thin_strips * rest_count < (int64_t(1) << 31)) {
+      a.n_strips = (uint32_t)thin_strips;
+      a.n_seg = 1;
+      a.strips_fd = FastDiv(a.n_strips);
+      const int vec_out = oa.identity && !oa.accumulate && a.u_pmul == 1 && aligned_for<T>(out, vec) ? 1 : 0;
+      note_kernel(vec_ok ? "reduce_col_thin_vec" : "reduce_col_thin");
+      const dim3 grid((uint32_t)(thin_strips * rest_count));
+      if (vec_ok) hipLaunchKernelGGL((reduce_col_thin_kernel<P, VMAX>), grid, dim3(kBlock), 0, st, a, alpha, vec_out);
+      else hipLaunchKernelGGL((reduce_col_thin_kernel<P, 1>), grid, dim3(kBlock), 0, st, a, alpha, vec_out);
+      return after_launch(st);
+    }
     a.n_strips = (a.u + 64 * vec - 1) / (64 * vec);
     const int64_t base_blocks = (int64_t)a.n_strips * rest_count;
     // Rows are cut into segments until about two blocks per compute unit exist

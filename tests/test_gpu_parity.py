@@ -620,6 +620,37 @@ def test_reduce_kernel_selection(P):
     compare(out, "indexed reduce")
 
 
+@pytest.mark.parametrize("code", [capi.F32, capi.F64, capi.I8, capi.I32])
+@pytest.mark.parametrize("rows,cols", [(16, 1 << 20), (1, 1 << 20), (128, 300000), (7, 262147), (129, 300000)], ids=str)
+def test_few_rows_under_many_columns(P, code, rows, cols):
+    """Column reductions of few rows ([16, 2^20] summed over the 16): a lane owns its columns and
+    walks the rows in the reference's order (no segments, no second launch) up to 128 rows; column
+    counts off the vector grid, one row, and one row more than the kernel takes."""
+    rng = np.random.default_rng(12)
+    x = values(rng, code, rows * cols, -9, 9)
+    xb = P.buf(x)
+    for op in ("sum", "max", "magnitude-squared", "mean"):
+        out = P.buf(np.zeros(cols, NP[code]))
+        k = P.run(H.unary_reduce, View(out, [cols, 1]), 1.0, View(xb, [rows, cols]).transpose([1, 0]), op)
+        check_reduce(out, x.reshape(rows, cols).astype(np.float64), 0, op, 1.0, code, f"thin cols {(rows, cols)} {op} ({k})")
+        vmax = 16 // x.itemsize
+        vec = vmax if cols % vmax == 0 else 1
+        if rows == 1:
+            pass                                              # nothing to reduce: the planner sees rows of one element
+        elif rows <= 128 and -(-cols // (256 * vec)) >= 1024:   # columns enough for four blocks per compute unit
+            assert k == ("reduce_col_thin_vec" if vec > 1 else "reduce_col_thin"), k
+        else:
+            assert k.startswith("reduce_col") and "thin" not in k, k
+    # kept axes on both sides of the reduced one: [3, 5, 400000] summed over the 5
+    if code == capi.F32:
+        b3 = P.buf(values(rng, code, 3 * 5 * 400000, -9, 9))
+        out = P.buf(np.zeros(3 * 400000, NP[code]))
+        k = P.run(H.unary_reduce, View(out, [3, 400000, 1]), 1.0, View(b3, [3, 5, 400000]).transpose([0, 2, 1]), "sum")
+        assert k == "reduce_col_thin_vec", k
+        check_reduce(out, np.moveaxis(b3.init.reshape(3, 5, 400000).astype(np.float64), 1, 2).reshape(3 * 400000, 5), 1, "sum",
+                     1.0, code, "thin cols with an outer kept axis")
+
+
 def test_reduce_nan_propagates_and_signed_zero(P):
     x = np.zeros((4, 512), np.float32)
     x[0, 100] = np.nan
