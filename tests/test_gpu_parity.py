@@ -651,6 +651,34 @@ def test_few_rows_under_many_columns(P, code, rows, cols):
                      1.0, code, "thin cols with an outer kept axis")
 
 
+@pytest.mark.parametrize("code", FLOATS)
+def test_extremes_of_a_large_tensor_under_a_multiplier(P, code):
+    """:max / :min with a multiplier other than 1 on 64 MiB and more: the multiplier-free kernel runs on
+    the raw values (the opposite extreme for a negative multiplier) and its results are multiplied, which
+    must leave the reference's bits: rows with NaN, infinities of both signs, zeros of both signs, a row
+    whose extreme overflows the type once multiplied."""
+    rng = np.random.default_rng(14)
+    rows, cols = 4096, 4096 if code == capi.F32 else 2048
+    x = rng.standard_normal((rows, cols)).astype(NP[code])
+    x[0, 100] = np.nan
+    x[1, 7], x[2, 9] = np.inf, -np.inf
+    x[3, :] = 0.0
+    x[3, ::3] = -0.0
+    x[4, :] = -0.0
+    x[5, 11] = np.finfo(NP[code]).max
+    x[6, 13] = -np.finfo(NP[code]).max
+    xb = P.buf(x)
+    for alpha in (0.5, -2.0, 3.0, -1.0):
+        for op in ("max", "min"):
+            out = P.buf(np.zeros(rows, NP[code]))
+            P.run(H.unary_reduce, View(out, [rows, 1]), alpha, View(xb, [rows, cols]), op)
+            with np.errstate(all="ignore"):
+                H.assert_bit_exact(out.download(), out.host, f"{op} of rows under {alpha}")
+            out2 = P.buf(np.zeros(cols, NP[code]))
+            P.run(H.unary_reduce, View(out2, [cols, 1]), alpha, View(xb, [rows, cols]).transpose([1, 0]), op)
+            H.assert_bit_exact(out2.download(), out2.host, f"{op} of columns under {alpha}")
+
+
 def test_reduce_nan_propagates_and_signed_zero(P):
     x = np.zeros((4, 512), np.float32)
     x[0, 100] = np.nan
