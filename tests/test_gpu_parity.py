@@ -329,6 +329,41 @@ def test_float_tanh_dense_sweep(P):
     assert np.all(np.isnan(nan.download()))
 
 
+def test_double_tanh_dense_sweep(P):
+    """unary-op! :tanh on double tensors is 1 - 2 / (exp(2|x|) + 1) from 0.05 on and an odd polynomial
+    below: a dense sweep of both pieces, the seam, tiny and huge arguments and both signs against the
+    oracle's library tanh, to 1e-14 of the result (the transcendental bar for doubles is 1e-12)."""
+    pos = np.concatenate([np.linspace(0.0, 0.07, 1 << 20), np.linspace(0.04, 25.0, 1 << 21), np.logspace(-300, -2, 1 << 16),
+                          np.logspace(1.3, 300, 1 << 14),
+                          np.array([0.05, np.nextafter(0.05, 0.0), np.nextafter(0.05, 1.0), 19.0, 19.06, 19.07, 20.0, 354.0,
+                                    355.0, 710.0, np.inf, 0.0])])
+    x = np.concatenate([pos, -pos])
+    n = x.size
+    xb, db = P.buf(x), P.buf(np.zeros(n, np.float64))
+    P.run(H.unary_op, View(db, [n]), View(xb, [n]), 1.0, "tanh")
+    got, want = db.download(), db.host
+    assert np.array_equal(np.signbit(got), np.signbit(want))
+    rel = np.abs(got - want) / np.maximum(np.abs(want), np.finfo(np.float64).tiny)
+    worst = int(np.argmax(rel))
+    assert rel[worst] <= 1e-14, (float(x[worst]), got[worst], want[worst], float(rel[worst]))
+    nan = P.buf(np.array([np.nan, -np.nan]))
+    P.run(H.unary_op, View(nan, [2]), View(nan, [2]), 1.0, "tanh")
+    assert np.all(np.isnan(nan.download()))
+
+
+@pytest.mark.parametrize("code", [capi.I8, capi.I16, capi.I32, capi.I64])
+def test_integer_tanh_truncates_like_the_reference(P, code):
+    """On integer tensors tanh(x * alpha) is truncated to the tensor's type: 0 until the double result
+    is exactly +-1, which happens between |x * alpha| = 19 and 20.  Every value from -128 to 127 under
+    multipliers 1, -1 and 3, bit for bit."""
+    x = np.arange(-128, 128).astype(NP[code])
+    for alpha in (1.0, -1.0, 3.0):
+        xb, db = P.buf(x), P.buf(np.zeros(x.size, NP[code]))
+        P.run(H.unary_op, View(db, [x.size]), View(xb, [x.size]), alpha, "tanh")
+        H.assert_bit_exact(db.download(), db.host, f"integer tanh alpha {alpha}")
+        assert set(np.unique(db.host).tolist()) <= {-1, 0, 1}
+
+
 @pytest.mark.parametrize("code", H.ALL_DTYPES)
 @pytest.mark.parametrize("op", list(capi.BINARY_OPS))
 def test_binary_ops_all_dtypes(P, code, op):
