@@ -168,6 +168,15 @@ CT_HD double w_neg(double a) { return -a; }
 // reference throws ArithmeticException; a kernel cannot).
 template <class T> CT_HD T jvm_ratio_cast(int64_t n, int64_t d) {
   if (d == 0) return (T)0;
+  if ((int64_t)(int32_t)n == n && (int64_t)(int32_t)d == d) {
+    // Both fit 32 bits (int tensors under multipliers of 1, small longs): a 32-bit division is a
+    // fifth of the instructions of the 64-bit one (int [2^26] x / y: 37 -> 6x % of the memory rate).
+    // -2^31 / -1 = 2^31 is an exact quotient and takes the truncating cast like any other.
+    if (d == -1) return jvm_cast<T>(-n);
+    const int32_t q = (int32_t)n / (int32_t)d;
+    if (std::is_same<T, int64_t>::value || (int64_t)q * d == n) return jvm_cast<T>((int64_t)q);
+    return jvm_cast<T>((double)q);
+  }
   if (n == INT64_MIN && d == -1) return jvm_cast<T>(n);
   const int64_t q = n / d;
   if (std::is_same<T, int64_t>::value || q * d == n) return jvm_cast<T>(q);

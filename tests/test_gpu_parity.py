@@ -329,6 +329,28 @@ def test_float_tanh_dense_sweep(P):
     assert np.all(np.isnan(nan.download()))
 
 
+@pytest.mark.parametrize("code", [capi.I32, capi.I64])
+def test_integer_division_edges(P, code):
+    """Integer :/ truncates toward zero and wraps like the JVM's long division followed by the narrowing
+    cast: the most negative value over -1 and over 1, operands on both sides of the 32-bit range (longs
+    whose operands fit 32 bits divide in 32 bits), inexact quotients of either sign, multipliers that push
+    int operands past 32 bits."""
+    info = np.iinfo(NP[code])
+    edge = [info.min, info.min + 1, info.max, info.max - 1, -(1 << 31), -(1 << 31) - 1, -(1 << 31) + 1, (1 << 31) - 1, 1 << 31,
+            (1 << 31) + 1, -7, 7, -1, 1, 100, -100, 3, -3, (1 << 40) + 5, -(1 << 40) - 5]
+    edge = [v for v in edge if info.min <= v <= info.max]
+    divisors = [-1, 1, 2, -2, 3, -3, 7, -7, 1 << 16, -(1 << 16), (1 << 31) - 1, -(1 << 31), info.max, info.min]
+    divisors = [v for v in divisors if info.min <= v <= info.max]
+    xs = np.array([a for a in edge for _ in divisors], dtype=NP[code])
+    ys = np.array([d for _ in edge for d in divisors], dtype=NP[code])
+    n = xs.size
+    xb, yb = P.buf(xs), P.buf(ys)
+    for xa, ya in ((1.0, 1.0), (-1.0, 1.0), (3.0, 1.0), (65536.0, -3.0)):
+        out = P.buf(np.zeros(n, NP[code]))
+        P.run(H.binary_op, View(out, [n]), View(xb, [n]), xa, View(yb, [n]), ya, "/")
+        H.assert_bit_exact(out.download(), out.host, f"integer / with alphas {xa}, {ya}")
+
+
 def test_double_tanh_dense_sweep(P):
     """unary-op! :tanh on double tensors is 1 - 2 / (exp(2|x|) + 1) from 0.05 on and an odd polynomial
     below: a dense sweep of both pieces, the seam, tiny and huge arguments and both signs against the
