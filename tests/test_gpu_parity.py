@@ -706,6 +706,12 @@ def test_few_rows_under_many_columns(P, code, rows, cols):
         assert k == "reduce_col_thin_vec", k
         check_reduce(out, np.moveaxis(b3.init.reshape(3, 5, 400000).astype(np.float64), 1, 2).reshape(3 * 400000, 5), 1, "sum",
                      1.0, code, "thin cols with an outer kept axis")
+        # the unit-stride kept axis first in the output's order: [400000, 3] results from a [3, 5, 400000] buffer
+        out = P.buf(np.zeros(3 * 400000, NP[code]))
+        k = P.run(H.unary_reduce, View(out, [400000, 3, 1]), 1.0, View(b3, [3, 5, 400000]).transpose([2, 0, 1]), "max")
+        assert k == "reduce_col_thin_vec", k
+        check_reduce(out, np.transpose(b3.init.reshape(3, 5, 400000), (2, 0, 1)).reshape(400000 * 3, 5).astype(np.float64), 1,
+                     "max", 1.0, code, "thin cols, unit axis first in the output")
 
 
 @pytest.mark.parametrize("code", FLOATS)
