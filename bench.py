@@ -853,8 +853,8 @@ def main() -> int:
                     "counters in profiles/memory_counters_adam_vs_copy.txt)")
     stored_us = roof.get("kernel_us_rocprof")
     if stored_us and abs(roof["avg_launch_us"] - stored_us) > 0.025 * stored_us:
-        roof["note"] += ("; the boxes of this pool fall into two groups on which this kernel binary takes 1168-1177 us and "
-                         "1213-1221 us: kernel_us_rocprof (profiles/) was taken on one group and this run is on the other")
+        roof["note"] += ("; the boxes of this pool fall into two groups on which this kernel binary takes about 1170 us and "
+                         "about 1220 us: kernel_us_rocprof (profiles/) was taken on one group and this run is on the other")
     if b.traffic_note:
         roof["traffic_note"] = b.traffic_note
     c0 = ops_out[step_ops[-1].label]
