@@ -81,8 +81,8 @@ def load_traffic():
     except (ValueError, OSError) as err:
         return {}, f"profiles/traffic.json unreadable: {err}"
     if stored.get("csrc_sha256") != csrc_hash():
-        return {}, ("the kernel sources changed since profiles/traffic.json was measured "
-                    f"(stored {str(stored.get('csrc_sha256'))[:12]}, now {csrc_hash()[:12]}): traffic not reported")
+        return {}, ("kernel sources changed since profiles/traffic.json was measured "
+                    f"({str(stored.get('csrc_sha256'))[:8]} -> {csrc_hash()[:8]}): traffic not reported")
     return stored.get("ops", {}), None
 
 
@@ -191,16 +191,65 @@ class Bench:
         return self.block(op, ms, host_us=host_ms * 1e3)
 
     def block(self, op: Op, ms: float, **more) -> dict:
-        rate = gbs(op.nbytes, ms)
-        stored = self.traffic.get(op.key)
-        b = {"bound": "hbm", "achieved": round(rate, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-             "frac": round(rate / PEAK_HBM_GBS, 4), "traffic": stored["traffic"] if stored else None,
-             "avg_call_us": round(ms * 1e3, 2), "algorithmic_bytes_per_call": op.nbytes, "kernel": op.kernel}
-        if stored:
-            b["kernel_us_rocprof"] = stored.get("kernel_us")
-        for k, v in more.items():
-            b[k] = round(v, 2) if isinstance(v, float) else v
-        return b
+        return roofline_block(op, ms, self.traffic.get(op.key), **more)
+
+
+def roofline_block(op: Op, ms: float, stored: dict | None, **more) -> dict:
+    """A roofline-shaped record of one workload: `ms` per call, `stored` its entry of profiles/traffic.json or None."""
+    rate = gbs(op.nbytes, ms)
+    b = {"key": op.key, "bound": "hbm", "achieved": round(rate, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+         "frac": round(rate / PEAK_HBM_GBS, 4), "traffic": stored["traffic"] if stored else None,
+         "avg_call_us": round(ms * 1e3, 2), "algorithmic_bytes_per_call": op.nbytes, "kernel": op.kernel}
+    if stored:
+        b["kernel_us_rocprof"] = stored.get("kernel_us")
+    for k, v in more.items():
+        b[k] = round(v, 2) if isinstance(v, float) else v
+    return b
+
+
+def headline(steps: int, warmup: int, adam_n: int, step_bytes: int, ms_per_step: float, wall_ms_per_step: float) -> dict:
+    """The fields of the result that the benchmark contract names, up to `config`."""
+    value = gbs(step_bytes, ms_per_step)
+    return collections.OrderedDict([
+        ("metric", "achieved HBM GB/s (% of MI355X peak) for binary-op!, unary-reduce!, Adam step"),
+        ("value", round(value, 1)),
+        ("unit", "GB/s"),
+        ("n_gpus", 1),
+        ("steps", steps),
+        ("warmup", warmup),
+        ("ms_per_step", round(ms_per_step, 4)),
+        ("higher_is_better", True),
+        ("scaling", "weak"),
+        ("vs_baseline", None),
+        ("dtype", "f32"),
+        ("data", "synthetic"),
+        ("config", {
+            "workload": f"configs[3] fused Adam step over {adam_n} float32 parameters + configs[2] unary-reduce! :sum :max "
+                        ":magnitude-squared over the last axis and over axis 0 (transposed view) of float32 [16384,4096] and of "
+                        "float64 [4096,4096] + configs[0] binary-op! :+ float32 [1024,1024] with a broadcast [1024] row; "
+                        "numpy default_rng seeds 6, 4, 5, 0",
+            "algorithmic_bytes_per_step": step_bytes,
+            "frac_of_peak": round(value / PEAK_HBM_GBS, 4),
+            "host_wall_ms_per_step": round(wall_ms_per_step, 4),
+            "csrc_sha256": csrc_hash()[:16],
+        }),
+    ])
+
+
+def adam_roofline(adam: Op, adam_ms: float, stored: dict | None, traffic_note: str | None) -> dict:
+    """The `roofline` object: the Adam kernel, `adam_ms` the average of the event pairs around its launches."""
+    roof = roofline_block(adam, adam_ms, stored)
+    del roof["key"]
+    roof["kernel"] = f"adam_kernel<float, 4, 1, true> ({adam.kernel})"
+    roof["avg_launch_us"] = roof.pop("avg_call_us")
+    roof["algorithmic_bytes_per_launch"] = roof.pop("algorithmic_bytes_per_call")
+    roof["note"] = "4 read + 3 write streams; the bare mix without arithmetic reaches 77-78 % of peak here, a copy 84-89 %"
+    stored_us = roof.get("kernel_us_rocprof")
+    if stored_us and abs(roof["avg_launch_us"] - stored_us) > 0.025 * stored_us:
+        roof["note"] += "; kernel_us_rocprof is from the other of the pool's two groups of boxes"
+    if traffic_note:
+        roof["traffic_note"] = traffic_note
+    return roof
 
 
 # ----------------------------------------------------------------------------- the step: configs[3], [2], [0]
@@ -776,6 +825,47 @@ def summarize_counters(run_dir: str, out_file: str) -> None:
 
 # ----------------------------------------------------------------------------- main
 
+# ----------------------------------------------------------------------------- the one line on stdout
+
+FINAL_LINE_LIMIT = 4096  # characters; what reads the line keeps only the end of this program's output
+
+# (section, key of the workload inside it) per BASELINE config, in the order the configs are listed
+CONFIG_FRACS = (
+    ("c0_bias_add_1024", "ops", "c0_bias_add"), ("c0_bias_add_16384", "others", "c0_bias_add_scaled"),
+    ("c1_exp_t", "others", "c1_exp_t"), ("c1_tanh_t", "others", "c1_tanh_t"), ("c1_select_t", "others", "c1_select_t"),
+    ("c2_sum_rows_f32", "ops", "c2_sum_rows_f32"), ("c2_sum_cols_f32", "ops", "c2_sum_cols_f32"),
+    ("c2_max_rows_f32", "ops", "c2_max_rows_f32"), ("c2_max_cols_f32", "ops", "c2_max_cols_f32"),
+    ("c2_magsq_rows_f32", "ops", "c2_magnitude-squared_rows_f32"), ("c2_magsq_cols_f32", "ops", "c2_magnitude-squared_cols_f32"),
+    ("c2_sum_rows_f64", "ops", "c2_sum_rows_f64"), ("c2_sum_cols_f64", "ops", "c2_sum_cols_f64"),
+    ("c2_max_rows_f64", "ops", "c2_max_rows_f64"), ("c2_max_cols_f64", "ops", "c2_max_cols_f64"),
+    ("c2_magsq_rows_f64", "ops", "c2_magnitude-squared_rows_f64"), ("c2_magsq_cols_f64", "ops", "c2_magnitude-squared_cols_f64"),
+    ("c3_adam", "ops", "c3_adam"), ("c3_adadelta", "ops", "c3_adadelta"),
+    ("c4_u8_f32", "others", "c4_u8_f32"), ("c4_sub_mean", "others", "c4_sub_mean"), ("c4_div_std", "others", "c4_div_std"),
+    ("c4_i32_f64", "others", "c4_i32_f64"),
+)
+
+
+def final_line(result: dict) -> dict:
+    """The object printed as the last line of stdout: the headline fields, `roofline`, `cpu_baseline` and one fraction
+    of the HBM peak per BASELINE config (each workload timed on its own, back to back).  Everything else the run
+    measured stays in the detail file.  Raises if the line would outgrow FINAL_LINE_LIMIT."""
+    head = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+            "dtype", "data", "config", "roofline")
+    out = collections.OrderedDict((k, result[k]) for k in head)
+    if result.get("cpu_baseline") is not None:
+        out["cpu_baseline"] = result["cpu_baseline"]
+    fracs = collections.OrderedDict()
+    for name, section, key in CONFIG_FRACS:
+        block = next((blk for blk in result.get(section, {}).values() if blk.get("key") == key), None)
+        if block is not None:
+            fracs[name] = block["frac"]
+    out["frac_of_peak_by_config"] = fracs
+    size = len(json.dumps(out))
+    if size >= FINAL_LINE_LIMIT:
+        raise RuntimeError(f"the final line has {size} characters; the limit is {FINAL_LINE_LIMIT}")
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -790,6 +880,8 @@ def main() -> int:
     ap.add_argument("--summarize-counters", default=None,
                     help="directory of one rocprofv3 --pmc run (plan.json + *counter_collection.csv): per-workload averages")
     ap.add_argument("--out", default=str(ROOT / "profiles"))
+    ap.add_argument("--detail", default=str(ROOT / "gpurun_out" / "bench_detail.json"),
+                    help="file that receives every section in full (the last stdout line carries the headline only)")
     args = ap.parse_args()
     if args.summarize:
         summarize(args.summarize, args.out)
@@ -844,50 +936,15 @@ def main() -> int:
     for op in step_ops + extra:
         ops_out[op.label] = b.time_op(op)
     adam.kernel = ops_out[adam.label]["kernel"]
-    roof = b.block(adam, adam_ms)
-    roof["kernel"] = f"adam_kernel<float, 4, 1, true> ({adam.kernel})"
-    roof["avg_launch_us"] = roof.pop("avg_call_us")
-    roof["algorithmic_bytes_per_launch"] = roof.pop("algorithmic_bytes_per_call")
-    roof["note"] = ("four read streams and three write streams over four buffers: the bare mix with the arithmetic removed "
-                    "runs at 77-78 % of peak on this board against 84-89 % for a copy (sweep in DESIGN.md section 5; memory-side "
-                    "counters in profiles/memory_counters_adam_vs_copy.txt)")
-    stored_us = roof.get("kernel_us_rocprof")
-    if stored_us and abs(roof["avg_launch_us"] - stored_us) > 0.025 * stored_us:
-        roof["note"] += ("; the boxes of this pool fall into two groups on which this kernel binary takes about 1170 us and "
-                         "about 1220 us: kernel_us_rocprof (profiles/) was taken on one group and this run is on the other")
-    if b.traffic_note:
-        roof["traffic_note"] = b.traffic_note
+    roof = adam_roofline(adam, adam_ms, b.traffic.get(adam.key), b.traffic_note)
     c0 = ops_out[step_ops[-1].label]
     c0["note"] = ("8 MiB, cache resident: avg_call_us is the GPU timeline per call with launches back to back, host_us the "
                   "time this program needs to submit one call (Python + ctypes + launch); when the two agree the loop is "
                   "bound by the host, and kernel_us_rocprof is what the kernel itself takes")
 
-    result = {
-        "metric": "achieved HBM GB/s (% of MI355X peak) for binary-op!, unary-reduce!, Adam step",
-        "value": round(value, 1),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {
-            "workload": f"configs[3] fused Adam step over {args.adam_n} float32 parameters + configs[2] unary-reduce! :sum :max "
-                        ":magnitude-squared over the last axis and over axis 0 (transposed view) of float32 [16384,4096] and of "
-                        "float64 [4096,4096] + configs[0] binary-op! :+ float32 [1024,1024] with a broadcast [1024] row; "
-                        "numpy default_rng seeds 6, 4, 5, 0",
-            "algorithmic_bytes_per_step": step_bytes,
-            "frac_of_peak": round(value / PEAK_HBM_GBS, 4),
-            "host_wall_ms_per_step": round(wall_ms / args.steps, 4),
-            "csrc_sha256": csrc_hash()[:16],
-        },
-        "roofline": roof,
-        "ops": ops_out,
-    }
+    result = headline(args.steps, args.warmup, args.adam_n, step_bytes, ms_per_step, wall_ms / args.steps)
+    result["roofline"] = roof
+    result["ops"] = ops_out
     builders = {"others": build_others, "midsize": build_midsize, "variants": build_variants, "patterns": build_patterns, "adjacent": build_adjacent}
     for name in ("others", "midsize", "variants", "patterns", "adjacent"):
         if name not in sections:
@@ -908,7 +965,14 @@ def main() -> int:
         log("timing the CPU oracle on the step ...")
         result["cpu_baseline"] = cpu_baseline(data)
     b.stream.release()
-    print(json.dumps(result))
+    detail = Path(args.detail)
+    try:
+        detail.parent.mkdir(parents=True, exist_ok=True)
+        detail.write_text(json.dumps(result, indent=1))
+        log(f"every section in full: {detail}")
+    except OSError as err:
+        log(f"could not write {detail}: {err}")
+    print(json.dumps(final_line(result)))
     return 0
 
 
