@@ -369,16 +369,28 @@ bool grouped_structure(const ct_dims& dd, const ct_dims& yd, const void* dest, c
     kept[nk++] = Ax{mx, dstr, yshape == 1 ? 0 : ystr};
   }
   if (gi < 0 || total != n) return false;
-  // kept axes must not overlap one another in the destination
+  // Kept axes must not overlap one another in the destination, and rows selected by different index
+  // values must not share addresses either (different lanes own them): the kept axes that are finer
+  // than the indexed axis have to fit inside one step of it.  A view whose rows overlap (a sliding
+  // window, a non-positive row stride) keeps the serial kernel, which applies the updates one by one.
+  // Kept axes coarser than the indexed axis are taken at their word: index values address the extent
+  // of their own dimension, which lies inside one step of the next coarser axis in any dense layout.
   {
+    if (a->d_gstride <= 0) return false;
     int order[CT_MAX_DIMS];
     for (int i = 0; i < nk; ++i) order[i] = i;
     std::sort(order, order + nk, [&](int l, int r) { return kept[l].ds < kept[r].ds; });
     int64_t span = 1;
+    bool indexed_placed = false;
     for (int i = 0; i < nk; ++i) {
+      if (!indexed_placed && kept[order[i]].ds >= a->d_gstride) {
+        if (a->d_gstride < span) return false;
+        indexed_placed = true;
+      }
       if (kept[order[i]].ds < span) return false;
       span = kept[order[i]].ds * (kept[order[i]].size - 1) + span;
     }
+    if (!indexed_placed && a->d_gstride < span) return false;
   }
   if (nk == 0) kept[nk++] = Ax{1, 1, 1};
   constexpr int VMAX = 16 / (int)sizeof(T);

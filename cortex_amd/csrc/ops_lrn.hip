@@ -171,6 +171,12 @@ template <class V> __device__ __forceinline__ void lrn_row_to_lds(const V* from,
                                    (__attribute__((address_space(3))) void*)row, 16, 0, 0);
 }
 
+// A direct load into LDS is a vector-memory operation: it is counted by vmcnt, not by lgkmcnt, and
+// the barrier waits for neither.  The rows one wave brings in are read by the other waves, so every
+// wave waits for its own outstanding vector-memory loads before it reaches the barrier; only then
+// does the barrier order those LDS writes before the other waves' reads.
+__device__ __forceinline__ void lrn_wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 template <class T, int VEC, int CH>
 __global__ void __launch_bounds__(kBlock) lrn_forward_kernel(const LrnArgs a) {
   constexpr int kRows = (CH + kLrnMaxWindow - 1 + kLrnWaves - 1) / kLrnWaves;
@@ -212,6 +218,7 @@ __global__ void __launch_bounds__(kBlock) lrn_forward_kernel(const LrnArgs a) {
       if (j < rows_x) xt[j * 64 + lane] = held[q];
     }
   }
+  if constexpr (VEC > 1) lrn_wait_direct_loads();
   __syncthreads();
   if (!live) return;
   T* yp = reinterpret_cast<T*>(const_cast<void*>(a.y.ptr)) + (int64_t)image * a.y.sb + lrn_pixel_offset<VEC>(a.y, a.width_fd, pv);
@@ -297,6 +304,7 @@ __global__ void __launch_bounds__(WAVES * 64) lrn_backward_kernel(const LrnArgs 
       if (j < rows_x) xt[j * 64 + lane] = xheld[q];
     }
   }
+  if constexpr (VEC > 1) lrn_wait_direct_loads();
   __syncthreads();
   // dy y / s of this wave's rows goes to LDS; dy s^-beta stays in gheld for the rows that are outputs
 #pragma unroll
@@ -498,6 +506,8 @@ extern "C" int ct_lrn_backward(void* stream, void* input_gradient, const ct_dims
                                const void* output_gradient, const ct_dims* output_gradient_dims, int n, double k,
                                double alpha, double beta, int dtype) {
   CT_REQUIRE(input_gradient && output && input && output_gradient, "lrn-backward!: null buffer");
+  CT_REQUIRE(input_gradient != output_gradient && input_gradient != output && input_gradient != input,
+             "lrn-backward!: the input gradient may not be one of the tensors read (neighbouring channels read them)");
   LrnArgs a;
   std::memset(&a, 0, sizeof(a));
   LrnShape si, so, sg, sd;

@@ -521,6 +521,9 @@ int ct_pooling_backward(void* stream, void* input_gradient, double input_gradien
  * src/cortex/verify/tensor.clj:1105-1123 for n = 2 require).  The backward
  * pass keeps output_gradient * output / s of every channel in the tensor's
  * type before summing: for float tensors a quotient below 1e-45 counts as 0.
+ * A channel's result needs its neighbours' operands, so neither call works in
+ * place: output == input, or an input_gradient that is the same buffer as
+ * output_gradient, output or input, is refused with CT_ERR_INVALID.
  * dtype is CT_F32 or CT_F64. */
 int ct_lrn_forward(void* stream, void* output, const ct_dims* output_dims, const void* input,
                    const ct_dims* input_dims, int n, double k, double alpha, double beta, int dtype);

@@ -166,3 +166,11 @@ def test_accumulate_indexed_layouts(P, code):
               requires_cas=True)
     exact(small, f"indexed and reduced ({k})")
     assert k == "serial", k
+    # rows that overlap in the destination (a sliding window: the row step is half a row): two index values
+    # share addresses, so the updates must go one by one, as the reference applies them
+    window = P.buf(values(rng, code, (classes + 1) * (width // 2)))
+    yw = P.buf(values(rng, code, rows * width, -9, 9))
+    k = P.run(H.binary_accum, View(window, [rows, width], [width // 2, 1], index=[idx, None]), 1.0, View(yw, [rows, width]), 1.0,
+              "+", requires_cas=True)
+    exact(window, f"overlapping indexed rows ({k})")
+    assert k == "serial", k

@@ -996,6 +996,10 @@ def test_lrn_strided_tensors_and_errors(P, code):
                       ((View(x, shape), View(x, shape), 5, 2.0, 1e-4, 0.75), "may not be the input")):
         with pytest.raises(capi.CortexHipError, match=re.escape(text)):
             H.lrn_forward(P.hip, *bad)
+    g = View(dy, shape)
+    for dest in (g, View(y, shape), View(x, shape)):   # an in-place gradient would race with the neighbours' reads
+        with pytest.raises(capi.CortexHipError, match=re.escape("may not be one of the tensors read")):
+            H.lrn_backward(P.hip, dest, View(y, shape), View(x, shape), g, 5, 2.0, 1e-4, 0.75)
 
 
 @pytest.mark.parametrize("code", FLOATS)

@@ -113,3 +113,55 @@ def test_rejects_what_the_fixed_array_cannot_hold(pair_factory):
         assert np.array_equal(out.download(), (sums * 127).astype(np.int8))
         _reduce("ct_unary_reduce_noalloc", pair.hip, H.View(out, [cols, 1]), 1.0, view, "sum")  # int accumulators: fits
         assert np.array_equal(out.download(), sums.astype(np.int8))
+
+
+def test_float_extreme_under_a_multiplier_on_a_large_input(pair_factory):
+    """Float :max / :min with a multiplier other than 1 on 32 MiB and more run the multiplier-free kernel and a
+    small multiplying launch: two launches through the fixed array, second call smaller (below 32 MiB it is the
+    widening form, one kernel family)."""
+    rng = np.random.default_rng(15)
+    with pair_factory() as pair:
+        for rows, cols in ((8192, 1024), (4096, 512)):
+            data = rng.standard_normal(rows * cols).astype(np.float32)
+            for op, alpha in (("max", 0.5), ("min", -3.0)):
+                kernel = _check(pair, data, [cols, rows], [1, cols], op, alpha=alpha)
+                if rows == 8192:  # the last launch is the multiplying one, an elementwise kernel
+                    assert not kernel.startswith("reduce"), kernel
+                else:
+                    assert kernel.startswith("reduce_col"), kernel
+
+
+def test_allocates_nothing_on_a_fresh_stream(pair_factory):
+    """The property the entry point exists for: on a stream whose scratch has never been grown, a split column
+    reduction and a split row reduction through it leave the device's free memory where it was."""
+    rows, cols = 16384, 1024
+    free0, free1, free2, total = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
+    with pair_factory() as pair:
+        data = np.random.default_rng(16).standard_normal(rows * cols).astype(np.float32)
+        src = pair.buf(data)
+        out = pair.buf(np.zeros(cols, np.float32))
+        few = pair.buf(np.zeros(4, np.float32))
+        fresh = C.c_void_p()
+        capi.call("ct_stream_create", C.byref(fresh))
+        try:
+            side = H.Side(gpu=True)
+            side.stream = fresh
+            col_view, row_view = H.View(src, [cols, rows], [1, cols]), H.View(src, [4, rows * cols // 4])
+            capi.call("ct_stream_sync", fresh)
+            capi.call("ct_memory_info", C.byref(free0), C.byref(total))
+            for op in ("sum", "max"):
+                _reduce("ct_unary_reduce_noalloc", side, H.View(out, [cols, 1]), 1.0, col_view, op)
+                assert capi.last_kernel().startswith("reduce_col"), capi.last_kernel()
+                _reduce("ct_unary_reduce_noalloc", side, H.View(few, [4, 1]), 1.0, row_view, op)
+            capi.call("ct_memory_info", C.byref(free1), C.byref(total))
+            assert free1.value == free0.value, (free0.value, free1.value)
+            want = data.reshape(rows, cols).max(axis=0)
+            assert np.array_equal(out.download(), want)
+            # the probe does see an allocation of the size a stream's scratch starts with
+            block = C.c_void_p()
+            capi.call("ct_malloc", C.byref(block), 1 << 20)
+            capi.call("ct_memory_info", C.byref(free2), C.byref(total))
+            capi.call("ct_free", block)
+            assert free2.value < free1.value, "ct_memory_info did not register a 1 MiB allocation"
+        finally:
+            capi.call("ct_stream_destroy", fresh)
