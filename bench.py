@@ -523,6 +523,17 @@ def build_patterns(b: Bench):
     ops.append(Op("p_accum_sum_rows", f"binary-op! :+ accumulate (bias gradient): float32 [{kk}] += rows of [{bb},{kk}]",
                   4 * bb * kk + 8 * kk,
                   lambda: s.binary_accum(acc, dims([kk]), 1.0, y, dims([bb, kk]), 1.0, bb * kk, "+", False, True)))
+    # the same destination under operations with no staged form: every destination element is a serial chain of
+    # 16384 steps, each rounded to float (streamed through LDS, one lane per chain)
+    ones = b.upload((1.0 + 1e-3 * rng.standard_normal(bb * kk)).astype(np.float32))
+    ops.append(Op("p_accum_mul_rows", f"binary-op! :* accumulate: float32 [{kk}] <- product over rows of [{bb},{kk}] (one float "
+                                      "multiplication per step of a chain)",
+                  4 * bb * kk + 8 * kk,
+                  lambda: s.binary_accum(acc, dims([kk]), 1.0, ones, dims([bb, kk]), 1.0, bb * kk, "*", False, True), iters=10))
+    ops.append(Op("p_accum_decay_rows", f"binary-op! :+ accumulate with dest_alpha 0.9: float32 [{kk}] <- rows of [{bb},{kk}] "
+                                        "(a step is widen, multiply, add, round: four dependent instructions)",
+                  4 * bb * kk + 8 * kk,
+                  lambda: s.binary_accum(acc, dims([kk]), 0.9, y, dims([bb, kk]), 1.0, bb * kk, "+", False, True), iters=10))
     return ops
 
 

@@ -183,6 +183,67 @@ bool owner_structure(const ct_dims& dd, const ct_dims& yd, int64_t n, OwnerArgs*
   return true;
 }
 
+// Whether the streamed form (ops_accum_stream.hip) takes this call, and its description if so.
+// It wants long chains (the owner kernel above is at its best with many short ones: a lane per
+// chain is then enough lanes, and neighbouring lanes read neighbouring addresses), y on the
+// 16-byte grid, and one of two arrangements: the chains unit-stride in y under one (merged)
+// broadcast axis, or the steps unit-stride in y under at most one further broadcast axis.
+constexpr int64_t kStreamMinSteps = 128;
+constexpr int64_t kStreamMaxChains = int64_t(1) << 18;
+
+template <class T> bool stream_structure(const OwnerArgs& a, AccumStreamCall* c) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  if (a.n_red < kStreamMinSteps || a.n_dest > kStreamMaxChains) return false;
+  if (((uintptr_t)a.y % 16) != 0) return false;
+  // broadcast axes, fastest first, neighbours that chain merged
+  int64_t rs[CT_MAX_DIMS], rst[CT_MAX_DIMS];
+  int nr = 0;
+  for (int d = 0; d < a.n_redax; ++d) {
+    const int64_t size = a.rsize[d].d, st = a.ry_stride[d];
+    if (size == 1) continue;
+    if (st < 0) return false;
+    if (nr > 0 && st == rst[nr - 1] * rs[nr - 1]) rs[nr - 1] *= size;
+    else { rs[nr] = size; rst[nr] = st; ++nr; }
+  }
+  if (nr == 0 || nr > 2) return false;
+  std::memset(c, 0, sizeof(*c));
+  c->dest = a.dest;
+  c->y = a.y;
+  c->n_red = a.n_red;
+  int strip = -1;
+  if (nr == 1 && rst[0] != 1) {
+    // chains unit-stride
+    for (int d = 0; d < a.n_kept; ++d)
+      if (a.ky_stride[d] == 1) strip = d;
+    if (strip < 0 || a.ksize[strip].d % VEC != 0 || rst[0] % VEC != 0) return false;
+    c->steps_unit_stride = false;
+    c->pitch = rst[0];
+  } else {
+    // steps unit-stride; the strip runs along the kept axis whose chains lie closest in y
+    if (rst[0] != 1 || rs[0] % VEC != 0) return false;
+    if (nr == 2 && rst[1] % VEC != 0) return false;
+    for (int d = 0; d < a.n_kept; ++d)
+      if (a.ky_stride[d] < 0) return false;
+      else if (strip < 0 || a.ky_stride[d] < a.ky_stride[strip]) strip = d;
+    if (strip >= 0 && a.ky_stride[strip] % VEC != 0) return false;
+    c->steps_unit_stride = true;
+    c->pitch = strip >= 0 ? a.ky_stride[strip] : 0;
+    c->n_inner = rs[0];
+    c->outer_stride = nr == 2 ? rst[1] : 0;
+  }
+  c->u = strip >= 0 ? (int64_t)a.ksize[strip].d : 1;
+  c->d_ustride = strip >= 0 ? a.kd_stride[strip] : 0;
+  for (int d = 0; d < a.n_kept; ++d) {
+    if (d == strip) continue;
+    if (a.ky_stride[d] < 0 || a.ky_stride[d] % VEC != 0) return false;
+    c->rsize[c->n_rest] = a.ksize[d].d;
+    c->rd_stride[c->n_rest] = a.kd_stride[d];
+    c->ry_stride[c->n_rest] = a.ky_stride[d];
+    ++c->n_rest;
+  }
+  return true;
+}
+
 // ------------------------------------------------------------------ indexed destinations
 
 struct GroupedArgs {
@@ -674,6 +735,18 @@ int accum_run_with(hipStream_t s, BinaryF<T, OP> f, void* dest, const ct_dims* d
                              dim3(kBlock), 0, s, f, f_unit, a);
           return after_launch(s);
         }
+      }
+    }
+    {
+      AccumStreamCall sc;
+      if (stream_structure<T>(a, &sc)) {
+        sc.dest_alpha = dest_alpha;
+        sc.y_alpha = y_alpha;
+        sc.reverse = reverse;
+        sc.op = OP;
+        sc.dtype = dtype;
+        sc.div0 = f.div0;
+        return accum_stream(s, sc);
       }
     }
     note_kernel("accum_owner");

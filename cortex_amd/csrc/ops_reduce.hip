@@ -1,6 +1,6 @@
 // ops_reduce.hip -- unary-reduce! (src/cortex/tensor/math.clj:104-108;
 // src/cortex/compute/cpu/tensor_math.clj:582-663): the entry points, and the kernels of float and double
-// tensors (reduce_impl.h; the integer tensors' are instantiated in ops_reduce_int.hip).
+// tensors (reduce_impl.h; the integer tensors are instantiated in ops_reduce_int*.hip).
 #include "reduce_impl.h"
 
 using namespace cthip;

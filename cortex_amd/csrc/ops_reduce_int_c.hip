@@ -1,0 +1,10 @@
+// ops_reduce_int_c.hip -- unary-reduce! for the short and int tensors (see reduce_impl.h); the integer tensors are
+// spread over three translation units so that they compile side by side.
+#include "reduce_impl.h"
+
+namespace cthip {
+namespace reduce_detail {
+template int reduce_dispatch<int16_t>(hipStream_t, const PartialStore&, void*, const ct_dims*, double, const void*, const ct_dims*, int);
+template int reduce_dispatch<int32_t>(hipStream_t, const PartialStore&, void*, const ct_dims*, double, const void*, const ct_dims*, int);
+}  // namespace reduce_detail
+}  // namespace cthip

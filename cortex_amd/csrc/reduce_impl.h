@@ -77,6 +77,7 @@ template <class T, int RK, class ACC = typename acc_of<T>::type> struct RedWide 
   using Elem = T;
   using Acc = ACC;
   using Alpha = Acc;
+  __device__ __forceinline__ explicit RedWide(int) {}
   static __device__ __forceinline__ Acc identity() {
     if constexpr (RK == RK_MAX) {
       if constexpr (std::is_same<Acc, double>::value) return -__builtin_huge_val();
@@ -132,6 +133,7 @@ template <class T, int RK> struct RedKeyed {
   using K = typename std::conditional<sizeof(T) == 4, int32_t, int64_t>::type;
   struct Acc { K hi, lo; };
   using Alpha = typename acc_of<T>::type;  // unused: alpha is 1
+  __device__ __forceinline__ explicit RedKeyed(int) {}
   static constexpr K kMag = sizeof(T) == 4 ? (K)0x7fffffff : (K)0x7fffffffffffffffLL;
   static constexpr K kPosInf = sizeof(T) == 4 ? (K)0x7f800000 : (K)0x7ff0000000000000LL;
   static constexpr K kNegInf = sizeof(T) == 4 ? (K)(int32_t)0x807fffff : (K)0x800fffffffffffffLL;
@@ -164,9 +166,65 @@ template <class T, int RK> struct RedKeyed {
   }
 };
 
+// Integer tensors choose the reduction at run time inside three policies, so that one set of kernels
+// per (datatype, accumulator) serves two reductions instead of one (the integer reductions were a
+// quarter of the library's code).  Both read the ct_reduce_op_t code the kernel's arguments
+// carry; it is uniform over the launch, so the choices below are scalar selects.
+//
+// max / min: for two's-complement integers min(a, b) = ~max(~a, ~b), so :min complements every
+// value on the way in and the result on the way out (one exclusive-or each) and both run as max.
+template <class T, class ACC = typename acc_of<T>::type> struct RedIntExtreme {
+  static_assert(std::is_integral<T>::value, "integer tensors only");
+  using Elem = T;
+  using Acc = ACC;
+  using Alpha = Acc;
+  Acc flip;
+  __device__ __forceinline__ explicit RedIntExtreme(int rk) : flip(rk == RK_MIN ? (Acc)-1 : (Acc)0) {}
+  __device__ __forceinline__ Acc identity() const { return std::numeric_limits<Acc>::min(); }
+  __device__ __forceinline__ Acc value(T x, Alpha alpha) const {
+    if constexpr (std::is_same<Acc, int32_t>::value) return w_mul((Acc)(T)alpha, (Acc)x) ^ flip;
+    else return w_mul(alpha, (Acc)x) ^ flip;
+  }
+  __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return a > b ? a : b; }
+  __device__ __forceinline__ T finish(Acc acc, int64_t) const { return jvm_cast<T>((Acc)(acc ^ flip)); }
+  static __device__ __forceinline__ Acc shfl(Acc v, int mask) {
+    if constexpr (std::is_same<Acc, int32_t>::value) return __shfl_xor(v, mask, 64);
+    else return (Acc)__shfl_xor((long long)v, mask, 64);
+  }
+};
+
+// sum / mean (SQUARES false) and magnitude-squared / magnitude (true): wrapping sums of the values or
+// of their squares, and the reference's final step per reduction (cpu/tensor_math.clj:610-622).
+template <class T, bool SQUARES, class ACC = typename acc_of<T>::type> struct RedIntSum {
+  static_assert(std::is_integral<T>::value, "integer tensors only");
+  using Elem = T;
+  using Acc = ACC;
+  using Alpha = Acc;
+  int rk;
+  __device__ __forceinline__ explicit RedIntSum(int rk_) : rk(rk_) {}
+  __device__ __forceinline__ Acc identity() const { return (Acc)0; }
+  __device__ __forceinline__ Acc value(T x, Alpha alpha) const {
+    Acc v;
+    if constexpr (std::is_same<Acc, int32_t>::value) v = w_mul((Acc)(T)alpha, (Acc)x);  // both in T's range: a 24-bit multiply
+    else v = w_mul(alpha, (Acc)x);
+    if constexpr (SQUARES) return w_mul(v, v);
+    else return v;
+  }
+  __device__ __forceinline__ Acc combine(Acc a, Acc b) const { return w_add(a, b); }
+  __device__ __forceinline__ T finish(Acc acc, int64_t count) const {
+    if constexpr (SQUARES) return rk == RK_MAG ? jvm_cast<T>(sqrt((double)acc)) : jvm_cast<T>(acc);
+    else return rk == RK_MEAN ? jvm_ratio_cast<T>((int64_t)acc, count) : jvm_cast<T>(acc);
+  }
+  static __device__ __forceinline__ Acc shfl(Acc v, int mask) {
+    if constexpr (std::is_same<Acc, int32_t>::value) return __shfl_xor(v, mask, 64);
+    else return (Acc)__shfl_xor((long long)v, mask, 64);
+  }
+};
+
 struct OutAddr {
   int32_t identity;  // output address == logical index
   int32_t accumulate;  // the result is added to what the output holds (the last pass of a staged binary-accum! :+)
+  int32_t rk;          // the reduction's ct_reduce_op_t code, for the policies that choose it at run time
   int32_t nd;
   GenOperand op;
   int64_t rmax[CT_MAX_DIMS];
@@ -178,11 +236,11 @@ __device__ __forceinline__ int64_t out_address(const OutAddr& o, int64_t p) {
 // Stores output p.  With oa.accumulate the stored value is old + result, formed as binary-op! :+
 // forms it (both widened, one rounding): what a separate in-place add of the result would leave.
 template <class P>
-__device__ __forceinline__ void store_output(void* out, const OutAddr& oa, int64_t p, const typename P::Acc& acc, int64_t k) {
+__device__ __forceinline__ void store_output(const P& pol, void* out, const OutAddr& oa, int64_t p, const typename P::Acc& acc, int64_t k) {
   using T = typename P::Elem;
   using W = typename acc_of<T>::type;
   T* const o = reinterpret_cast<T*>(out) + out_address(oa, p);
-  T r = P::finish(acc, k);
+  T r = pol.finish(acc, k);
   if (oa.accumulate) r = jvm_cast<T>(w_add((W)*o, (W)r));
   *o = r;
 }
@@ -217,6 +275,7 @@ struct RowArgs {
 // few rows to fill the chip (the norm of a whole parameter vector).
 template <class P, int VEC, int TPR, int BS = kBlock>
 __global__ void __launch_bounds__(BS) reduce_row_kernel(const RowArgs a, const typename P::Alpha alpha) {
+  const P pol(a.oa.rk);
   using T = typename P::Elem;
   using A = typename P::Acc;
   using V = Vec<T, VEC>;
@@ -234,7 +293,7 @@ __global__ void __launch_bounds__(BS) reduce_row_kernel(const RowArgs a, const t
   const bool live = vp < a.n_out * (int64_t)a.n_split;
   uint32_t p = (uint32_t)vp, seg = 0;
   if (a.n_split > 1) a.split_fd.divmod((uint32_t)vp, p, seg);
-  A acc0 = P::identity(), acc1 = P::identity();
+  A acc0 = pol.identity(), acc1 = pol.identity();
   if (live) {
     int64_t base = (int64_t)seg * a.chunk;
     int64_t len = a.k - base;
@@ -257,31 +316,31 @@ __global__ void __launch_bounds__(BS) reduce_row_kernel(const RowArgs a, const t
       const V x0 = nt_load(row + i), x1 = nt_load(row + i + TPR);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        acc0 = P::combine(acc0, P::value(x0.v[e], alpha));
-        acc1 = P::combine(acc1, P::value(x1.v[e], alpha));
+        acc0 = pol.combine(acc0, pol.value(x0.v[e], alpha));
+        acc1 = pol.combine(acc1, pol.value(x1.v[e], alpha));
       }
     }
     if (i < nv) {
       const V x0 = nt_load(row + i);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) acc0 = P::combine(acc0, P::value(x0.v[e], alpha));
+      for (int e = 0; e < VEC; ++e) acc0 = pol.combine(acc0, pol.value(x0.v[e], alpha));
     }
   }
-  A acc = P::combine(acc0, acc1);
+  A acc = pol.combine(acc0, acc1);
   constexpr int W = TPR < 64 ? TPR : 64;
 #pragma unroll
-  for (int m = W / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
+  for (int m = W / 2; m >= 1; m >>= 1) acc = pol.combine(acc, P::shfl(acc, m));
   if constexpr (TPR > 64) {
     if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = acc;
     __syncthreads();
     if (threadIdx.x == 0) {
       acc = lds[0];
 #pragma unroll
-      for (int w = 1; w < BS / 64; ++w) acc = P::combine(acc, lds[w]);
+      for (int w = 1; w < BS / 64; ++w) acc = pol.combine(acc, lds[w]);
     }
   }
   if (live && lane == 0) {
-    if (a.n_split == 1) store_output<P>(a.out, a.oa, p, acc, a.k);
+    if (a.n_split == 1) store_output<P>(pol, a.out, a.oa, p, acc, a.k);
     else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc;
   }
 }
@@ -293,6 +352,7 @@ __global__ void __launch_bounds__(BS) reduce_row_kernel(const RowArgs a, const t
 // instruction of a wave covers consecutive rows.
 template <class P, int VEC, int TPR, int L>
 __global__ void __launch_bounds__(kBlock) reduce_row_small_kernel(const RowArgs a, const typename P::Alpha alpha) {
+  const P pol(a.oa.rk);
   using T = typename P::Elem;
   using A = typename P::Acc;
   using V = Vec<T, VEC>;
@@ -323,18 +383,18 @@ __global__ void __launch_bounds__(kBlock) reduce_row_small_kernel(const RowArgs 
 #pragma unroll
   for (int r = 0; r < U; ++r) {
     const int64_t p = p0 + r * GPB;
-    A acc = P::identity();
+    A acc = pol.identity();
     if (p < a.n_out) {
 #pragma unroll
       for (int j = 0; j < L; ++j)
         if (lane + j * TPR < nv) {
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) acc = P::combine(acc, P::value(x[r][j].v[e], alpha));
+          for (int e = 0; e < VEC; ++e) acc = pol.combine(acc, pol.value(x[r][j].v[e], alpha));
         }
     }
 #pragma unroll
-    for (int m = TPR / 2; m >= 1; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
-    if (p < a.n_out && lane == 0) store_output<P>(a.out, a.oa, p, acc, a.k);
+    for (int m = TPR / 2; m >= 1; m >>= 1) acc = pol.combine(acc, P::shfl(acc, m));
+    if (p < a.n_out && lane == 0) store_output<P>(pol, a.out, a.oa, p, acc, a.k);
   }
 }
 
@@ -362,6 +422,7 @@ constexpr int64_t kRowSplitBytes = 16384;  // smallest chunk a split row is cut 
 
 template <class P, int VEC>
 __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, const typename P::Alpha alpha) {
+  const P pol(a.oa.rk);
   using T = typename P::Elem;
   using A = typename P::Acc;
   using V = Vec<T, VEC>;
@@ -383,7 +444,7 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
   const bool live = col < a.u;
   A acc[VEC];
 #pragma unroll
-  for (int e = 0; e < VEC; ++e) acc[e] = P::identity();
+  for (int e = 0; e < VEC; ++e) acc[e] = pol.identity();
   const int64_t r0 = (int64_t)seg * a.rows_per_seg;
   int64_t r1 = r0 + a.rows_per_seg;
   if (r1 > a.k) r1 = a.k;
@@ -400,7 +461,7 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
 #pragma unroll
       for (int j = 0; j < UN; ++j)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
+        for (int e = 0; e < VEC; ++e) acc[e] = pol.combine(acc[e], pol.value(x[j].v[e], alpha));
     }
     if (r < r1) {  // the last, partial batch: same depth, rows past the end skipped
       V x[UN];
@@ -411,7 +472,7 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
       for (int j = 0; j < UN; ++j)
         if (r + j * WAVES < r1) {
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
+          for (int e = 0; e < VEC; ++e) acc[e] = pol.combine(acc[e], pol.value(x[j].v[e], alpha));
         }
     }
   }
@@ -424,9 +485,9 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
 #pragma unroll
-      for (int w = 0; w < WAVES - 1; ++w) acc[e] = P::combine(acc[e], lds[w][e * 64 + lane]);
+      for (int w = 0; w < WAVES - 1; ++w) acc[e] = pol.combine(acc[e], lds[w][e * 64 + lane]);
       const int64_t p = pbase + (int64_t)(col + e) * a.u_pmul;
-      if (a.n_seg == 1) store_output<P>(a.out, a.oa, p, acc[e], a.k);
+      if (a.n_seg == 1) store_output<P>(pol, a.out, a.oa, p, acc[e], a.k);
       else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc[e];
     }
   }
@@ -441,6 +502,7 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
 // vec_out: the results of a lane are neighbours in the output and go out as one vector.
 template <class P, int VEC>
 __global__ void __launch_bounds__(kBlock) reduce_col_thin_kernel(const ColArgs a, const typename P::Alpha alpha, const int vec_out) {
+  const P pol(a.oa.rk);
   using T = typename P::Elem;
   using A = typename P::Acc;
   using V = Vec<T, VEC>;
@@ -458,7 +520,7 @@ __global__ void __launch_bounds__(kBlock) reduce_col_thin_kernel(const ColArgs a
   if (col >= a.u) return;
   A acc[VEC];
 #pragma unroll
-  for (int e = 0; e < VEC; ++e) acc[e] = P::identity();
+  for (int e = 0; e < VEC; ++e) acc[e] = pol.identity();
   const T* p = reinterpret_cast<const T*>(a.in) + base + col;
   constexpr int UN = 8;
   int64_t r = 0;
@@ -469,7 +531,7 @@ __global__ void __launch_bounds__(kBlock) reduce_col_thin_kernel(const ColArgs a
 #pragma unroll
     for (int j = 0; j < UN; ++j)
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
+      for (int e = 0; e < VEC; ++e) acc[e] = pol.combine(acc[e], pol.value(x[j].v[e], alpha));
   }
   if (r < a.k) {
     V x[UN];
@@ -480,17 +542,17 @@ __global__ void __launch_bounds__(kBlock) reduce_col_thin_kernel(const ColArgs a
     for (int j = 0; j < UN; ++j)
       if (r + j < a.k) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = P::combine(acc[e], P::value(x[j].v[e], alpha));
+        for (int e = 0; e < VEC; ++e) acc[e] = pol.combine(acc[e], pol.value(x[j].v[e], alpha));
       }
   }
   if (vec_out) {
     V out;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) out.v[e] = P::finish(acc[e], a.k);
+    for (int e = 0; e < VEC; ++e) out.v[e] = pol.finish(acc[e], a.k);
     *reinterpret_cast<V*>(reinterpret_cast<T*>(a.out) + pbase + col) = out;
   } else {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) store_output<P>(a.out, a.oa, pbase + (int64_t)(col + e) * a.u_pmul, acc[e], a.k);
+    for (int e = 0; e < VEC; ++e) store_output<P>(pol, a.out, a.oa, pbase + (int64_t)(col + e) * a.u_pmul, acc[e], a.k);
   }
 }
 
@@ -509,6 +571,7 @@ struct ShortRowsArgs {
 
 template <class P>
 __global__ void __launch_bounds__(kBlock) reduce_short_rows_kernel(const ShortRowsArgs a, const typename P::Alpha alpha) {
+  const P pol(a.oa.rk);
   using T = typename P::Elem;
   using A = typename P::Acc;
   constexpr int VEC = 16 / (int)sizeof(T);
@@ -528,9 +591,9 @@ __global__ void __launch_bounds__(kBlock) reduce_short_rows_kernel(const ShortRo
   __syncthreads();
   if (threadIdx.x < n_rows) {
     const T* row = tile + threadIdx.x * k;
-    A acc = P::identity();
-    for (uint32_t j = 0; j < k; ++j) acc = P::combine(acc, P::value(row[j], alpha));
-    store_output<P>(a.out, a.oa, row0 + threadIdx.x, acc, (int64_t)k);
+    A acc = pol.identity();
+    for (uint32_t j = 0; j < k; ++j) acc = pol.combine(acc, pol.value(row[j], alpha));
+    store_output<P>(pol, a.out, a.oa, row0 + threadIdx.x, acc, (int64_t)k);
   }
 }
 
@@ -546,6 +609,7 @@ constexpr int kFinishLoads = 4;
 
 template <class P, int LPO>
 __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs a) {
+  const P pol(a.oa.rk);
   using A = typename P::Acc;
   constexpr int PPW = 64 / LPO;  // outputs per wave
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -553,7 +617,7 @@ __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs 
   const int64_t p = ((int64_t)blockIdx.x * (kBlock / 64) + wave) * PPW + pl;
   const bool live = p < a.n_out;
   const A* part = reinterpret_cast<const A*>(a.partials);
-  A acc = P::identity();
+  A acc = pol.identity();
   if (live) {
     if (a.n_seg <= (uint32_t)(kFinishLoads * LPO)) {
       A x[kFinishLoads];
@@ -564,15 +628,15 @@ __global__ void __launch_bounds__(kBlock) reduce_finish_kernel(const FinishArgs 
       }
 #pragma unroll
       for (int j = 0; j < kFinishLoads; ++j)
-        if ((uint32_t)(sl + j * LPO) < a.n_seg) acc = P::combine(acc, x[j]);
+        if ((uint32_t)(sl + j * LPO) < a.n_seg) acc = pol.combine(acc, x[j]);
     } else {
 #pragma unroll 8
-      for (uint32_t s = sl; s < a.n_seg; s += LPO) acc = P::combine(acc, part[(int64_t)s * a.n_out + p]);
+      for (uint32_t s = sl; s < a.n_seg; s += LPO) acc = pol.combine(acc, part[(int64_t)s * a.n_out + p]);
     }
   }
 #pragma unroll
-  for (int m = 32; m >= PPW; m >>= 1) acc = P::combine(acc, P::shfl(acc, m));
-  if (live && sl == 0) store_output<P>(a.out, a.oa, p, acc, a.k);
+  for (int m = 32; m >= PPW; m >>= 1) acc = pol.combine(acc, P::shfl(acc, m));
+  if (live && sl == 0) store_output<P>(pol, a.out, a.oa, p, acc, a.k);
 }
 
 template <class P>
@@ -603,16 +667,17 @@ struct AnyArgs {
 // One lane per output, in the reference's own order (sequential accumulation).
 template <class P>
 __global__ void __launch_bounds__(kBlock) reduce_any_kernel(const AnyArgs a, const typename P::Alpha alpha) {
+  const P pol(a.oa.rk);
   using T = typename P::Elem;
   using A = typename P::Acc;
   const int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (p >= a.n_out) return;
   const T* in = reinterpret_cast<const T*>(a.in);
   const int64_t start = p * a.k;
-  A acc = P::value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start)], alpha);
+  A acc = pol.value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start)], alpha);
   for (int64_t i = 1; i < a.k; ++i)
-    acc = P::combine(acc, P::value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start + i)], alpha));
-  store_output<P>(a.out, a.oa, p, acc, a.k);
+    acc = pol.combine(acc, pol.value(in[ref_address(a.in_op, a.in_nd, a.in_rmax, start + i)], alpha));
+  store_output<P>(pol, a.out, a.oa, p, acc, a.k);
 }
 
 // ------------------------------------------------------------------ host planning
@@ -701,6 +766,7 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
   oa.nd = out_rank;
   oa.identity = oa.op.mode == 0;
   oa.accumulate = ps.accumulate ? 1 : 0;
+  oa.rk = op;
 
   constexpr int VMAX = 16 / (int)sizeof(T);
   const RedShape rs = analyse(*id, k);
@@ -901,18 +967,27 @@ int reduce_typed(hipStream_t st, const PartialStore& ps, void* out, const ct_dim
       return ct_unary_op(st, out, od, out, od, (double)a, CT_UOP_NOOP, sizeof(T) == 4 ? CT_F32 : CT_F64, dims_ecount(*od));
     }
   }
-  if constexpr (std::is_integral<T>::value && sizeof(T) <= 2) {
-    // the largest magnitude an element times the multiplier can have, and how many of them a sum adds
-    const int64_t a_abs = std::llabs((long long)jvm_cast<T>(alpha));
-    const int64_t x_abs = std::is_signed<T>::value ? (int64_t(1) << (8 * sizeof(T) - 1)) : (int64_t(1) << (8 * sizeof(T))) - 1;
-    const int64_t n_out = dims_ecount(*od), total = dims_ecount(*id);
-    const int64_t count = n_out > 0 ? total / n_out : 0;
-    const int64_t term = (RK == RK_SUMSQ || RK == RK_MAG) ? (a_abs * x_abs) * (a_abs * x_abs) : a_abs * x_abs;  // < 2^62
-    const bool fits = (RK == RK_MAX || RK == RK_MIN) ? term < (int64_t(1) << 31)
-                                                    : (count > 0 && term < (int64_t(1) << 31) / count);
-    if (fits) return reduce_run<RedWide<T, RK, int32_t>>(st, ps, out, od, alpha, in, id, op);
+  if constexpr (std::is_integral<T>::value) {
+    constexpr bool kExtreme = RK == RK_MAX || RK == RK_MIN;
+    constexpr bool kSquares = RK == RK_SUMSQ || RK == RK_MAG;
+    if constexpr (sizeof(T) <= 2) {
+      // the largest magnitude an element times the multiplier can have, and how many of them a sum adds
+      const int64_t a_abs = std::llabs((long long)jvm_cast<T>(alpha));
+      const int64_t x_abs = std::is_signed<T>::value ? (int64_t(1) << (8 * sizeof(T) - 1)) : (int64_t(1) << (8 * sizeof(T))) - 1;
+      const int64_t n_out = dims_ecount(*od), total = dims_ecount(*id);
+      const int64_t count = n_out > 0 ? total / n_out : 0;
+      const int64_t term = (RK == RK_SUMSQ || RK == RK_MAG) ? (a_abs * x_abs) * (a_abs * x_abs) : a_abs * x_abs;  // < 2^62
+      const bool fits = kExtreme ? term < (int64_t(1) << 31) : (count > 0 && term < (int64_t(1) << 31) / count);
+      if (fits) {
+        using Narrow = typename std::conditional<kExtreme, RedIntExtreme<T, int32_t>, RedIntSum<T, kSquares, int32_t>>::type;
+        return reduce_run<Narrow>(st, ps, out, od, alpha, in, id, op);
+      }
+    }
+    using Wide = typename std::conditional<kExtreme, RedIntExtreme<T>, RedIntSum<T, kSquares>>::type;
+    return reduce_run<Wide>(st, ps, out, od, alpha, in, id, op);
+  } else {
+    return reduce_run<RedWide<T, RK>>(st, ps, out, od, alpha, in, id, op);
   }
-  return reduce_run<RedWide<T, RK>>(st, ps, out, od, alpha, in, id, op);
 }
 
 template <class T>
