@@ -57,7 +57,8 @@ def ops_for(code):
     if code in FLOATS:
         return [("*", 1.0, 1.0, False), ("/", 1.0, 1.0, False), ("/", 1.0, -1.0, True), ("-", 1.0, 1.0, True),
                 ("+", 0.9, 1.0, False), ("*", 1.0, 0.5, True), ("min", 0.5, 1.0, False), ("max", 2.0, -1.0, True),
-                (">=", 1.0, 1.0, False), ("+", -1.0, 2.0, False)]
+                (">=", 1.0, 1.0, False), ("+", -1.0, 2.0, False), ("-", 0.5, 2.0, True), ("-", 0.75, -0.5, False),
+                ("+", 0.9, 3.0, True)]
     return [("*", 1.0, 1.0, False), ("/", 1.0, 1.0, False), ("-", 1.0, 1.0, True), ("+", 3.0, 1.0, False),
             ("bit-xor", 1.0, 1.0, False), ("bit-and", 1.0, 7.0, True), ("max", 1.0, 3.0, False), ("<", 1.0, 1.0, True)]
 
