@@ -229,7 +229,10 @@ int gemv_typed(hipStream_t s, void* y, int64_t incy, bool trans, double alpha, c
   // segment is a whole number of load rounds (16 waves x 8 rows)
   constexpr int64_t kRowQuantum = 128;
   const int64_t want_seg = std::max<int64_t>(1, std::min<int64_t>(512 / a.n_strips, rows / kRowQuantum));
-  const int64_t per = ((rows + want_seg - 1) / want_seg + kRowQuantum - 1) / kRowQuantum * kRowQuantum;
+  int64_t per = ((rows + want_seg - 1) / want_seg + kRowQuantum - 1) / kRowQuantum * kRowQuantum;
+  // eight rows more per segment, where that leaves their number alone: segment starts a power of
+  // two apart advance in step through the same memory channels (see the column reduction)
+  if (per < rows && (rows + per + 7) / (per + 8) == (rows + per - 1) / per) per += 8;
   a.rows_per_seg = (uint32_t)per;
   a.n_seg = (uint32_t)((rows + per - 1) / per);
   if (a.n_seg > 1) {

@@ -911,6 +911,11 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
     int64_t rows = ((k + want_seg - 1) / want_seg + kRowQuantum - 1) / kRowQuantum * kRowQuantum;
     const int64_t seg_cap = std::max<int64_t>(1, (int64_t(16) << 20) / (n_out * (int64_t)sizeof(A)));
     if ((k + rows - 1) / rows > seg_cap) rows = (k + seg_cap - 1) / seg_cap;
+    // Segments a power of two apart in memory advance in step through the same memory channels and
+    // banks: eight rows more per segment moves every segment's start off that grid without changing
+    // the number of segments (float [16384,4096]: 41.2 -> 38.5 us for the bare kernel, double
+    // [4096,4096] 20.0 -> 19.5, float [4096,4096] 10.0 -> 9.2).
+    if (rows < k && (k + rows + 7) / (rows + 8) == (k + rows - 1) / rows) rows += 8;
     int64_t seg = (k + rows - 1) / rows;
     a.n_seg = (uint32_t)seg;
     a.rows_per_seg = (uint32_t)rows;
