@@ -52,7 +52,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, published
-SECTIONS = ("headline", "others", "midsize", "variants", "patterns", "adjacent")
+SECTIONS = ("headline", "others", "midsize", "small", "variants", "patterns", "adjacent")
 
 
 def log(msg: str) -> None:
@@ -410,6 +410,63 @@ def build_midsize(b: Bench):
            lambda: s.ternary_op(d, sq, x, tr, 1.0, g, tr, 1.0, m, tr, 1.0, n, "select")),
         Op("m_softmax", "softmax! float32 [16384,1024]", 8 * n,
            lambda: s.softmax_eltwise(d, dims([16384, 1024]), x, dims([16384, 1024]))),
+    ]
+
+
+# ----------------------------------------------------------------------------- the reference's own sizes
+
+def build_small(b: Bench):
+    """The calls of one training step of the networks the reference trains itself (src/cortex/verify/nn/train.clj:185-187:
+    batches of 128 images of 784 pixels, ten classes; a [64,32,7,7] activation for the spatial forms).  Everything here is
+    bound by the launch: avg_call_us is what one call costs back to back, and c_caller holds the same calls from a
+    compiled loop."""
+    s = b.stream
+    rng = np.random.default_rng(12)
+    batch, pixels, classes = 128, 784, 10
+    n = batch * pixels
+    x = b.upload(rng.standard_normal(n, dtype=np.float32))
+    g = b.upload(rng.standard_normal(n, dtype=np.float32) * 1e-3)
+    d, m, v = b.alloc(n, "float"), b.alloc(n, "float"), b.alloc(n, "float")
+    s.memset(m, 0, 0.0, n)
+    s.memset(v, 0, 1e-6, n)
+    row = b.upload(rng.standard_normal(pixels, dtype=np.float32))
+    out = b.alloc(pixels, "float")
+    s.memset(out, 0, 0.0, pixels)
+    st = [b.upload(rng.uniform(0.5, 1.5, pixels).astype(np.float32)) for _ in range(8)]
+    act, act_t = dims([batch, pixels]), dims([pixels, batch], [1, pixels])
+    logits = dims([batch, classes])
+    sb, sc, se = 64, 32, 49
+    ns = sb * sc * se
+    pb1, pb2 = pow_betas()
+    it = 200
+    return [
+        Op("s_bias_add", f"binary-op! :+ float32 [{batch},{pixels}] + [{pixels}] row", 8 * n + 4 * pixels,
+           lambda: s.binary_op(d, act, x, act, 1.0, row, dims([pixels]), 1.0, n, "+"), iters=it),
+        Op("s_bias_gradient", f"binary-op! :+ accumulate (bias gradient): float32 [{pixels}] += rows of [{batch},{pixels}]",
+           4 * n + 8 * pixels, lambda: s.binary_accum(out, dims([pixels]), 1.0, x, act, 1.0, n, "+", False, True), iters=it),
+        Op("s_bias_gradient_classes", f"binary-op! :+ accumulate: float32 [{classes}] += rows of [{batch},{classes}]",
+           4 * batch * classes + 8 * classes,
+           lambda: s.binary_accum(out, dims([classes]), 1.0, x, logits, 1.0, batch * classes, "+", False, True), iters=it),
+        Op("s_sum_over_batch", f"unary-reduce! :sum axis 0 of float32 [{batch},{pixels}] (transposed view)", 4 * n + 4 * pixels,
+           lambda: s.unary_reduce(out, dims([pixels, 1]), 1.0, x, act_t, "sum"), iters=it),
+        Op("s_sum_rows", f"unary-reduce! :sum last axis of float32 [{batch},{pixels}]", 4 * n + 4 * batch,
+           lambda: s.unary_reduce(out, dims([batch, 1]), 1.0, x, act, "sum"), iters=it),
+        Op("s_softmax", f"softmax! float32 [{batch},{classes}]", 8 * batch * classes,
+           lambda: s.softmax_eltwise(d, logits, x, logits), iters=it),
+        Op("s_bn_update_eltwise", f"batch-normalize-update-and-apply! eltwise float32 [{batch},{pixels}]", 8 * n,
+           lambda: s.batch_normalize_update_and_apply_eltwise(d, x, st[0], st[1], st[4], st[5], 0.9, st[2], st[3], 1e-3,
+                                                              batch, pixels), iters=it),
+        Op("s_bn_gradients_eltwise", f"batch-normalize-gradients! eltwise float32 [{batch},{pixels}]", 12 * n,
+           lambda: s.batch_normalize_gradients_eltwise(d, st[6], st[7], g, d, x, st[0], st[1], st[2], st[3], 1e-3, batch,
+                                                       pixels), iters=it),
+        Op("s_bn_update_spatial", f"batch-normalize-update-and-apply! spatial float32 [{sb},{sc},7,7]", 8 * ns,
+           lambda: s.batch_normalize_update_and_apply_spatial(d, x, st[0], st[1], st[4], st[5], 0.9, st[2], st[3], 1e-3,
+                                                              sb, sc, se), iters=it),
+        Op("s_bn_gradients_spatial", f"batch-normalize-gradients! spatial float32 [{sb},{sc},7,7]", 12 * ns,
+           lambda: s.batch_normalize_gradients_spatial(d, st[6], st[7], g, d, x, st[0], st[1], st[2], st[3], 1e-3, sb, sc,
+                                                       se), iters=it),
+        Op("s_adam", f"Adam step, {n} float32 parameters (the weights of a [{pixels},{batch}] layer)", 28 * n,
+           lambda: s.adam_step(1e-3, 0.9, 0.999, 1e-8, pb1, pb2, 1.0, g, x, m, v, n), iters=it),
     ]
 
 
@@ -956,8 +1013,9 @@ def main() -> int:
     result = headline(args.steps, args.warmup, args.adam_n, step_bytes, ms_per_step, wall_ms / args.steps)
     result["roofline"] = roof
     result["ops"] = ops_out
-    builders = {"others": build_others, "midsize": build_midsize, "variants": build_variants, "patterns": build_patterns, "adjacent": build_adjacent}
-    for name in ("others", "midsize", "variants", "patterns", "adjacent"):
+    builders = {"others": build_others, "midsize": build_midsize, "small": build_small, "variants": build_variants,
+                "patterns": build_patterns, "adjacent": build_adjacent}
+    for name in ("others", "midsize", "small", "variants", "patterns", "adjacent"):
         if name not in sections:
             continue
         log(f"timing section '{name}' ...")

@@ -68,14 +68,35 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
+def _dependencies(depfile: Path):
+    """The files a make-style dependency file names, or None when it cannot be read."""
+    try:
+        text = depfile.read_text().replace("\\\n", " ")
+    except OSError:
+        return None
+    deps = []
+    for rule in text.splitlines():
+        _, sep, rest = rule.partition(":")
+        if sep:
+            deps.extend(Path(d) for d in rest.split())
+    return deps
+
+
 def _compile(src: str, force: bool) -> Path:
+    """Compiles one source; without `force`, only when it or a header it includes (as recorded by the compiler
+    in the object's dependency file at the last build) is newer than the object."""
     obj = CSRC / "build" / (Path(src).stem + ".o")
+    depfile = obj.with_suffix(".d")
     obj.parent.mkdir(exist_ok=True)
     path = CSRC / src
-    deps = [path] + list(CSRC.glob("*.h")) + [HERE.parent / "include" / "cortex_hip.h"]
-    if not force and obj.exists() and all(obj.stat().st_mtime >= d.stat().st_mtime for d in deps):
-        return obj
-    cmd = [_hipcc(), *FLAGS, "-x", "hip", "-c", str(path), "-o", str(obj)]
+    if not force and obj.exists():
+        deps = _dependencies(depfile)
+        if deps is None:
+            deps = [path] + list(CSRC.glob("*.h")) + [HERE.parent / "include" / "cortex_hip.h"]
+        own = [d for d in deps + [path] if CSRC in d.resolve().parents or d.resolve().parent == (HERE.parent / "include")]
+        if all(d.exists() and obj.stat().st_mtime >= d.stat().st_mtime for d in own):
+            return obj
+    cmd = [_hipcc(), *FLAGS, "-MD", "-MF", str(depfile), "-x", "hip", "-c", str(path), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)

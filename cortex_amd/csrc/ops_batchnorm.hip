@@ -857,6 +857,185 @@ void bn_launch_apply(hipStream_t s, const BnPlan& plan) {
 
 inline dim3 channel_grid(int64_t C, int per_block) { return dim3((uint32_t)((C + per_block - 1) / per_block)); }
 
+// ---------------------------------------------------------------- one launch for small tensors
+//
+// The networks the reference trains itself move batches of 128 x 784 through these methods
+// (src/cortex/verify/nn/train.clj:185-187): three launches cost three times what the arithmetic
+// does.  When a channel has at most kSmallChannelValues values (batch x elements) a block keeps
+// whole channels in registers: it reads its channels once, forms their statistics (the mean first,
+// then the squared distances from the rounded mean, exactly the CPU backend's two walks, or the
+// five sums of the gradients in one walk), finishes them as bn_finish_kernel does and applies them
+// to the values it holds.  One read, one write, one launch.
+//
+// A block of 256 lanes takes CG neighbouring channels with TPC = 256 / CG lanes each; lane t owns
+// channel t % CG and every TPC-th value of it.  CG is a power of two of at most 64, so the lanes
+// of one channel inside a wave are a fixed distance apart and combine with shuffles; the four
+// waves meet in LDS.
+constexpr int64_t kSmallChannelValues = 4096;
+constexpr int64_t kSmallTensorElements = int64_t(1) << 21;
+
+struct BnSmallArgs {
+  const void* x;
+  const void* og;
+  void* out;
+  const void* means;      // gradient mode: the batch statistics
+  const void* variances;
+  const void* scale;
+  const void* bias;
+  double epsilon;
+  int64_t C, E;
+  uint32_t count;         // values per channel: batch x elements
+  uint32_t cg, tpc, cg_shift;
+  FastDiv e_fd;
+  BnFinish f;
+};
+
+template <int NACC>
+__device__ __forceinline__ void bn_small_combine(double (&acc)[NACC], double (*lds)[kBlock / 64][64], uint32_t cg_count,
+                                                 int lane, int wave, int cg) {
+#pragma unroll
+  for (int k = 0; k < NACC; ++k)
+    for (uint32_t m = 32; m >= cg_count; m >>= 1) acc[k] += __shfl_xor(acc[k], (int)m, 64);
+  if ((uint32_t)lane < cg_count) {
+#pragma unroll
+    for (int k = 0; k < NACC; ++k) lds[k][wave][lane] = acc[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < NACC; ++k) {
+    double t = lds[k][0][cg];
+#pragma unroll
+    for (int w = 1; w < kBlock / 64; ++w) t += lds[k][w][cg];
+    acc[k] = t;
+  }
+}
+
+template <class T, int MODE, int R>
+__global__ void __launch_bounds__(kBlock) bn_small_kernel(const BnSmallArgs a) {
+  constexpr int NACC = bn_nacc<MODE>::value;
+  __shared__ double lds[NACC][kBlock / 64][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int cg = (int)(threadIdx.x & (a.cg - 1));
+  const uint32_t part = threadIdx.x >> a.cg_shift;
+  const int64_t c = (int64_t)blockIdx.x * a.cg + cg;
+  const bool live = c < a.C;
+  const T* xp = reinterpret_cast<const T*>(a.x);
+  const T* gp = reinterpret_cast<const T*>(a.og);
+  T x[R], g[MODE == kBnGradient ? R : 1];
+  int64_t off[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const uint32_t i = part + (uint32_t)r * a.tpc;
+    uint32_t b, e;
+    a.e_fd.divmod(i, b, e);
+    off[r] = live && i < a.count ? ((int64_t)b * a.C + c) * a.E + e : -1;
+    x[r] = (T)0;
+    if (off[r] >= 0) {
+      x[r] = xp[off[r]];
+      if constexpr (MODE == kBnGradient) g[r] = gp[off[r]];
+    }
+  }
+  double pm[kParamStride];
+  const int64_t count = a.count;
+  if constexpr (MODE == kBnGradient) {
+    const double mean = live ? (double)reinterpret_cast<const T*>(a.means)[c] : 0.0;
+    const T scale = live ? reinterpret_cast<const T*>(a.scale)[c] : (T)0;
+    double acc[NACC] = {0.0, 0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (off[r] >= 0) bn_accumulate_gradient<T>(acc, x[r], g[r], mean, scale);
+    bn_small_combine<NACC>(acc, lds, a.cg, lane, wave, cg);
+    if (!live) return;
+    // as bn_finish_kernel (cpu/tensor_math.clj:922-983)
+    const T eps = (T)a.epsilon;
+    const T pow_factor = (T)(-3.0 / 2.0);
+    const double variance = (double)eps + (double)reinterpret_cast<const T*>(a.variances)[c];
+    const double inv_std = 1.0 / sqrt(variance);
+    const double d_var = (double)(T)(-0.5 * pow(variance, (double)pow_factor));
+    const T d_var_d_out = (T)(d_var * acc[2]);
+    const T d_mean_d_out = (T)((-inv_std) * acc[3] + (double)d_var_d_out * ((-2.0 * acc[4]) / (double)count));
+    const double one_over_count = 1.0 / (double)count;
+    pm[0] = mean; pm[1] = inv_std; pm[2] = (double)scale; pm[3] = d_var;
+    pm[4] = (double)d_var_d_out * 2.0;
+    pm[5] = (double)d_mean_d_out * one_over_count;
+    pm[6] = one_over_count;
+    if (part == 0) {
+      reinterpret_cast<T*>(a.f.bias_gradient)[c] = (T)acc[0];
+      reinterpret_cast<T*>(a.f.scale_gradient)[c] = (T)(inv_std * acc[1]);
+    }
+  } else {
+    // batch-normalize-update-impl (cpu/tensor_math.clj:831-870): the mean, then the squared distances from it
+    double acc[NACC] = {0.0, 0.0};
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (off[r] >= 0) acc[0] += (double)x[r];
+    bn_small_combine<NACC>(acc, lds, a.cg, lane, wave, cg);
+    const double count_val = fmax(1.0, (double)count);
+    const double running_count_val = fmax(1.0, count_val - 1.0);
+    const T new_mean = (T)(acc[0] / count_val);
+    double sq = 0.0;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (off[r] >= 0) {
+        const double d = (double)new_mean - (double)x[r];
+        sq += d * d;
+      }
+    __syncthreads();  // every lane has read the sums before the table is written again
+    double acc2[NACC] = {sq, 0.0};
+    bn_small_combine<NACC>(acc2, lds, a.cg, lane, wave, cg);
+    if (!live) return;
+    const double new_var = acc2[0];
+    const T batch_variance = (T)(new_var / count_val);
+    const T eps = (T)a.epsilon;
+    pm[0] = (double)new_mean;
+    pm[1] = (double)(T)sqrt(1.0 / ((double)batch_variance + (double)eps));
+    pm[2] = (double)reinterpret_cast<const T*>(a.scale)[c];
+    pm[3] = (double)reinterpret_cast<const T*>(a.bias)[c];
+    if (part == 0) {
+      const T ave_factor = (T)a.f.average_factor;
+      const double ave_lerp = (double)(T)1.0 - (double)ave_factor;
+      T* running_means = reinterpret_cast<T*>(a.f.running_means);
+      T* running_variances = reinterpret_cast<T*>(a.f.running_variances);
+      const T mean = running_means[c], variance = running_variances[c];
+      reinterpret_cast<T*>(a.f.batch_means)[c] = new_mean;
+      reinterpret_cast<T*>(a.f.batch_variances)[c] = batch_variance;
+      running_means[c] = (T)((double)mean * ave_lerp + (double)new_mean * (double)ave_factor);
+      running_variances[c] =
+          (T)((double)variance * ave_lerp + (double)(T)(new_var / running_count_val) * (double)ave_factor);
+    }
+  }
+  T* op = reinterpret_cast<T*>(a.out);
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if (off[r] >= 0) op[off[r]] = bn_apply_one<T, MODE>(pm, x[r], MODE == kBnGradient ? g[r] : (T)0);
+}
+
+// Launches the one-launch form when the tensor qualifies; *taken says whether it did.
+template <class T, int MODE>
+int bn_small(hipStream_t s, BnSmallArgs& a, int64_t B, int64_t C, int64_t E, bool* taken) {
+  *taken = false;
+  const int64_t count = B * E;
+  if (count > kSmallChannelValues || count * C > kSmallTensorElements) return CT_OK;
+  // lanes per channel: enough that a lane holds at most eight values, at least four (the waves
+  // meet in LDS either way), at most the block
+  int64_t tpc = 4;
+  while (tpc < kBlock && tpc * 8 < count) tpc *= 2;
+  const int64_t per_lane = (count + tpc - 1) / tpc;
+  a.count = (uint32_t)count;
+  a.tpc = (uint32_t)tpc;
+  a.cg = (uint32_t)(kBlock / tpc);
+  a.cg_shift = 0;
+  while ((1u << a.cg_shift) < a.cg) ++a.cg_shift;
+  a.C = C; a.E = E;
+  a.e_fd = FastDiv((uint32_t)E);
+  const dim3 grid((uint32_t)((C + a.cg - 1) / a.cg));
+  if (per_lane <= 4) hipLaunchKernelGGL((bn_small_kernel<T, MODE, 4>), grid, dim3(kBlock), 0, s, a);
+  else if (per_lane <= 8) hipLaunchKernelGGL((bn_small_kernel<T, MODE, 8>), grid, dim3(kBlock), 0, s, a);
+  else hipLaunchKernelGGL((bn_small_kernel<T, MODE, 16>), grid, dim3(kBlock), 0, s, a);
+  *taken = true;
+  return CT_OK;
+}
+
 inline void bn_set_statistics(BnArgs* a, const void* means, const void* variances, const void* scale, const void* bias,
                               double epsilon) {
   a->means = means; a->variances = variances; a->scale = scale; a->bias = bias; a->epsilon = epsilon;
@@ -882,6 +1061,21 @@ template <class T>
 int bn_update_and_apply(hipStream_t s, void* output, const void* input, void* batch_means, void* batch_variances,
                         void* running_means, void* running_variances, double average_factor, const void* scale,
                         const void* bias, double epsilon, int64_t B, int64_t C, int64_t E) {
+  CT_REQUIRE(B >= 1 && C >= 1 && E >= 1, "batch-normalize: batch, channel and element counts must be positive");
+  {
+    BnSmallArgs sa;
+    std::memset(&sa, 0, sizeof(sa));
+    sa.x = input; sa.out = output; sa.scale = scale; sa.bias = bias; sa.epsilon = epsilon;
+    sa.f.batch_means = batch_means; sa.f.batch_variances = batch_variances;
+    sa.f.running_means = running_means; sa.f.running_variances = running_variances;
+    sa.f.average_factor = average_factor;
+    bool taken = false;
+    if (int rc = bn_small<T, kBnNormalize>(s, sa, B, C, E, &taken)) return rc;
+    if (taken) {
+      note_kernel("bn_update_small");
+      return after_launch(s);
+    }
+  }
   BnPlan plan;
   if (int rc = bn_plan<T, kBnNormalize>(s, B, C, E, input, nullptr, output, true, &plan)) return rc;
   // the apply pass normalizes with the batch statistics the finishing pass writes
@@ -903,6 +1097,20 @@ template <class T>
 int bn_gradients(hipStream_t s, void* input_gradient, void* scale_gradient, void* bias_gradient,
                  const void* output_gradient, const void* input, const void* batch_means, const void* batch_variances,
                  const void* scale, double epsilon, int64_t B, int64_t C, int64_t E) {
+  CT_REQUIRE(B >= 1 && C >= 1 && E >= 1, "batch-normalize: batch, channel and element counts must be positive");
+  {
+    BnSmallArgs sa;
+    std::memset(&sa, 0, sizeof(sa));
+    sa.x = input; sa.og = output_gradient; sa.out = input_gradient;
+    sa.means = batch_means; sa.variances = batch_variances; sa.scale = scale; sa.epsilon = epsilon;
+    sa.f.scale_gradient = scale_gradient; sa.f.bias_gradient = bias_gradient;
+    bool taken = false;
+    if (int rc = bn_small<T, kBnGradient>(s, sa, B, C, E, &taken)) return rc;
+    if (taken) {
+      note_kernel("bn_gradients_small");
+      return after_launch(s);
+    }
+  }
   BnPlan plan;
   if (int rc = bn_plan<T, kBnGradient>(s, B, C, E, input, output_gradient, input_gradient, true, &plan)) return rc;
   bn_set_statistics(&plan.a, batch_means, batch_variances, scale, nullptr, epsilon);

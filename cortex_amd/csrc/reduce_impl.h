@@ -418,6 +418,7 @@ struct ColArgs {
 // rows are in flight per block, 8 loads per lane.  Measured best among 1-16
 // waves and 32-512 rows per block for a [16384, 4096] float input.
 constexpr int kColBlock = 1024;
+constexpr int64_t kNarrowColBytes = int64_t(4) << 20;  // largest input the one-launch narrow-strip column kernel takes
 constexpr int64_t kRowSplitBytes = 16384;  // smallest chunk a split row is cut into
 
 template <class P, int VEC>
@@ -489,6 +490,73 @@ __global__ void __launch_bounds__(kColBlock) reduce_col_kernel(const ColArgs a, 
       const int64_t p = pbase + (int64_t)(col + e) * a.u_pmul;
       if (a.n_seg == 1) store_output<P>(pol, a.out, a.oa, p, acc[e], a.k);
       else reinterpret_cast<A*>(a.partials)[(int64_t)seg * a.n_out + p] = acc[e];
+    }
+  }
+}
+
+// A small matrix reduced down its columns (the [1024,1024] and [128,784] of a network's layer): cut
+// into row segments it needs the finishing launch, which costs more than the reduction; left whole
+// under 256-column strips it is four blocks.  Here a block owns a strip of LW * VEC columns (128
+// bytes) over all rows, so there are blocks enough without segments: LW lanes across, 64 / LW rows
+// per wave-load, eight loads in flight per lane; the lanes of a column combine with shuffles, the
+// waves in LDS.  One launch.  (Strips this narrow stream at half the rate of the wide ones, which
+// is why large matrices keep them.)
+template <class P, int VEC, int LW>
+__global__ void __launch_bounds__(kColBlock) reduce_col_narrow_kernel(const ColArgs a, const typename P::Alpha alpha) {
+  const P pol(a.oa.rk);
+  using T = typename P::Elem;
+  using A = typename P::Acc;
+  using V = Vec<T, VEC>;
+  constexpr int WAVES = kColBlock / 64, RW = 64 / LW, RB = RW * WAVES, UN = 8;
+  __shared__ A lds[WAVES - 1][LW * VEC];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lc = lane % LW, lr = lane / LW;
+  uint32_t rest, strip;
+  a.strips_fd.divmod(blockIdx.x, rest, strip);
+  int64_t base = 0, pbase = 0;
+  for (int d = 0; d < a.n_rest; ++d) {
+    uint32_t q, r;
+    a.rsize[d].divmod(rest, q, r);
+    rest = q;
+    base += (int64_t)r * a.rstride_in[d];
+    pbase += (int64_t)r * a.r_pmul[d];
+  }
+  const uint32_t col = (strip * LW + lc) * VEC;
+  const bool live = col < a.u;
+  A acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = pol.identity();
+  if (live) {
+    const T* p = reinterpret_cast<const T*>(a.in) + base + col;
+    for (int64_t r = wave * RW + lr; r < a.k; r += (int64_t)RB * UN) {
+      V x[UN];
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        if (r + j * RB < a.k) x[j] = nt_load(reinterpret_cast<const V*>(p + (r + j * RB) * a.rstride));
+#pragma unroll
+      for (int j = 0; j < UN; ++j)
+        if (r + j * RB < a.k) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[e] = pol.combine(acc[e], pol.value(x[j].v[e], alpha));
+        }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+#pragma unroll
+    for (int m = LW; m < 64; m <<= 1) acc[e] = pol.combine(acc[e], P::shfl(acc[e], m));
+  }
+  if (wave > 0 && lr == 0) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) lds[wave - 1][lc * VEC + e] = acc[e];
+  }
+  __syncthreads();
+  if (wave == 0 && lr == 0 && live) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+#pragma unroll
+      for (int w = 0; w < WAVES - 1; ++w) acc[e] = pol.combine(acc[e], lds[w][lc * VEC + e]);
+      store_output<P>(pol, a.out, a.oa, pbase + (int64_t)(col + e) * a.u_pmul, acc[e], a.k);
     }
   }
 }
@@ -858,10 +926,13 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
     return after_launch(st);
   }
 
+  // the unit-stride kept axis the column kernels run along: at least 16 columns, or any number when the
+  // input is small enough for the one-launch narrow-strip kernel (ten classes summed over a batch)
+  const int64_t min_unit = total * (int64_t)sizeof(T) <= kNarrowColBytes ? 2 : 16;
   int unit = -1;
   if (rs.fast && small_idx)
     for (int d = 0; d < rs.n_kept; ++d)
-      if (rs.kstride[d] == 1 && rs.ksize[d] >= 16) unit = d;
+      if (rs.kstride[d] == 1 && rs.ksize[d] >= min_unit) unit = d;
   if (unit >= 0) {
     ColArgs a;
     std::memset(&a, 0, sizeof(a));
@@ -917,6 +988,19 @@ int reduce_run(hipStream_t st, const PartialStore& ps, void* out, const ct_dims*
     // [4096,4096] 20.0 -> 19.5, float [4096,4096] 10.0 -> 9.2).
     if (rows < k && (k + rows + 7) / (rows + 8) == (k + rows - 1) / rows) rows += 8;
     int64_t seg = (k + rows - 1) / rows;
+    // a small matrix that the wide strips have to cut into row segments: narrow strips, one launch
+    constexpr int kNarrowLanes = 8;
+    const int64_t narrow_strips = ((int64_t)a.u + kNarrowLanes * vec - 1) / (kNarrowLanes * vec);
+    if (seg > 1 && total * (int64_t)sizeof(T) <= kNarrowColBytes) {
+      a.n_strips = (uint32_t)narrow_strips;
+      a.n_seg = 1;
+      a.strips_fd = FastDiv(a.n_strips);
+      note_kernel(vec_ok ? "reduce_col_narrow_vec" : "reduce_col_narrow");
+      const dim3 grid((uint32_t)(narrow_strips * rest_count));
+      if (vec_ok) hipLaunchKernelGGL((reduce_col_narrow_kernel<P, VMAX, kNarrowLanes>), grid, dim3(kColBlock), 0, st, a, alpha);
+      else hipLaunchKernelGGL((reduce_col_narrow_kernel<P, 1, kNarrowLanes>), grid, dim3(kColBlock), 0, st, a, alpha);
+      return after_launch(st);
+    }
     a.n_seg = (uint32_t)seg;
     a.rows_per_seg = (uint32_t)rows;
     a.strips_fd = FastDiv(a.n_strips);

@@ -1166,7 +1166,9 @@ def test_batch_normalize_update_and_gradients(P, code, shape):
     x64 = t["x"].init.astype(np.float64)
     k = P.run(H.batch_normalize_update_and_apply, V["out"], V["x"], V["means"], V["variances"], V["rmeans"],
               V["rvars"], 0.8, V["scale"], V["bias"], 1e-3, b, c, e)
-    assert k == ("bn_update_row" if (e or 1) * t["x"].init.itemsize >= 128 else "bn_update_col")
+    one_launch = b * (e or 1) <= 4096 and b * c * (e or 1) <= 1 << 21     # a channel fits a block's registers
+    assert k == ("bn_update_small" if one_launch else
+                 "bn_update_row" if (e or 1) * t["x"].init.itemsize >= 128 else "bn_update_col")
     what = f"batch-normalize-update-and-apply {shape} ({k})"
     bn_close(t["means"], what + " batch means", code, scale_by=np.max(np.abs(x64)))
     bn_close(t["variances"], what + " batch variances", code)
@@ -1178,6 +1180,7 @@ def test_batch_normalize_update_and_gradients(P, code, shape):
         t[name].upload(t[name].host)
     k = P.run(H.batch_normalize_gradients, V["ig"], V["sg"], V["bg"], V["og"], V["out"], V["x"], V["means"],
               V["variances"], V["scale"], V["bias"], 1e-3, b, c, e)
+    assert (k == "bn_gradients_small") == one_launch, k
     what = f"batch-normalize-gradients {shape} ({k})"
     og64 = np.abs(t["og"].init.astype(np.float64))
     per_channel = og64.reshape(b, c, e or 1).sum(axis=(0, 2)).max()

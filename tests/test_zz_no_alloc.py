@@ -62,7 +62,9 @@ def _check(pair, data: np.ndarray, shape, strides, op, alpha=1.0):
 def test_column_reduction_twice_second_smaller(pair_factory, dtype, op):
     rng = np.random.default_rng(11)
     with pair_factory() as pair:
-        for rows, cols in ((2048, 1024), (640, 384)):  # the second call is smaller and meets the first one's leftovers
+        # both calls are cut into row segments whose partials go through the fixed array (inputs above the 4 MiB
+        # that a single launch over narrow strips takes); the second is smaller and meets the first one's leftovers
+        for rows, cols in ((4096, 2048), (3072, 1536)):
             if np.dtype(dtype).kind == "f":
                 data = rng.standard_normal(rows * cols).astype(dtype)
             else:
