@@ -556,6 +556,19 @@ def build_patterns(b: Bench):
                                       "every 64-byte line of the matrix is fetched for one float: the memory system moves 8.5x these bytes)",
                   8 * rows_v,  # the elements asked for; the lines they sit in are 16 times that
                   lambda: s.assign(colv, dims([rows_v]), mat, dims([rows_v], [pitch]), rows_v)))
+    # blocks of a wider matrix copied out (ct/submatrix, tensor.clj:490-513): rows off the 16-byte grid
+    sub_rows, sub_w, sub_pitch = 65536, 999, 1024
+    wide = b.upload(rng.standard_normal(sub_rows * sub_pitch, dtype=np.float32))
+    block = b.alloc(sub_rows * sub_w, "float")
+    ops.append(Op("p_submatrix_copy", f"assign! float32 [{sub_rows},{sub_w}] <- block of a pitch-{sub_pitch} matrix", 8 * sub_rows * sub_w,
+                  lambda: s.assign(block, dims([sub_rows, sub_w]), wide, dims([sub_rows, sub_w], [sub_pitch, 1]), sub_rows * sub_w)))
+    ops.append(Op("p_submatrix_store", f"assign! block of a pitch-{sub_pitch} matrix <- float32 [{sub_rows},{sub_w}]", 8 * sub_rows * sub_w,
+                  lambda: s.assign(wide, dims([sub_rows, sub_w], [sub_pitch, 1]), block, dims([sub_rows, sub_w]), sub_rows * sub_w)))
+    short_rows, short_w, short_pitch = 1 << 22, 10, 16
+    ops.append(Op("p_short_rows_of_pitch", f"assign! float32 [{short_rows},{short_w}] <- rows of {short_w} out of a pitch of {short_pitch} "
+                                           "(the memory system moves whole 64-byte lines: 1.3x these bytes)", 8 * short_rows * short_w,
+                  lambda: s.assign(block, dims([short_rows, short_w]), wide, dims([short_rows, short_w], [short_pitch, 1]),
+                                   short_rows * short_w)))
     # planar <-> interleaved images (verify/tensor.clj:668-684, 785-805)
     nb, hh, ww, ch = 256, 224, 224, 3
     npx = nb * hh * ww * ch

@@ -258,8 +258,11 @@ bool prepare_ragged(const Plan& plan, const EwOperand* ops, int vmax, RaggedArgs
       if (dense) {
         if (((uintptr_t)ops[k].ptr % (uintptr_t)(vmax * ops[k].elem_size)) != 0) return false;
         a->dense_mask |= 1u << k;
-      } else if (!periodic || k == 0) {
+      } else if (k == 0) {
         return false;
+      } else if (!periodic) {
+        a->pitched_mask |= 1u << k;
+        for (int d = 1; d < c.nd; ++d) a->outer_stride[k][d - 1] = c.stride[k][d];
       }
     } else if (c.stride[k][0] == 0 && k != 0) {
       a->scalar_mask |= 1u << k;
@@ -269,6 +272,33 @@ bool prepare_ragged(const Plan& plan, const EwOperand* ops, int vmax, RaggedArgs
     }
   }
   return (a->dense_mask & 1u) != 0;
+}
+
+// A dense destination [rows, w] from unit-stride rows of a pitch of at most 128 bytes that leaves at least
+// a fifth of every pitch unused (otherwise reading each row where it lies moves about the same lines).
+bool prepare_span(const Plan& plan, const EwOperand* ops, int vmax, SpanArgs* a) {
+  const Canon& c = plan.canon;
+  if (c.any_index || c.nd != 2 || plan.n_ops != 2 || !ops[0].ptr || !ops[1].ptr) return false;
+  const int64_t w = c.size[0], rows = c.size[1], pitch = c.stride[1][1];
+  if (c.stride[0][0] != 1 || c.stride[0][1] != w || c.stride[1][0] != 1) return false;
+  if (w < 2 || pitch <= w || pitch * ops[1].elem_size > 128 || w * 5 > pitch * 4) return false;
+  if (plan.n < (int64_t(1) << 20) || plan.n >= kLim31 || rows * pitch >= kLim31) return false;
+  if (((uintptr_t)ops[0].ptr % 16) != 0 || ((uintptr_t)ops[1].ptr % 16) != 0) return false;
+  // a block's rows: a multiple of 16 (so that its span and its share of the destination start on the 16-byte
+  // grid whatever the element sizes) whose span fits the LDS budget
+  int64_t per = kSpanLdsBytes / (pitch * ops[1].elem_size) / 16 * 16;
+  if (per < 16) return false;
+  if (per > 256) per = 256;
+  (void)vmax;
+  std::memset(a, 0, sizeof(*a));
+  a->ptr[0] = (char*)ops[0].ptr;
+  a->ptr[1] = (char*)ops[1].ptr;
+  a->rows = (uint32_t)rows;
+  a->w = (uint32_t)w;
+  a->pitch = (uint32_t)pitch;
+  a->w_fd = FastDiv((uint32_t)w);
+  a->rows_per_block = (uint32_t)per;
+  return true;
 }
 
 bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* a, int* n_short, int* ppt, uint32_t* grid) {

@@ -446,7 +446,10 @@ __global__ void __launch_bounds__(kBlock) ew_vecu_kernel(const F f, const VecArg
 // a lane can take an aligned 16-byte vector of them that may straddle the end of a row: at most
 // one row boundary falls into a vector (rows are at least a vector long).  The small operands are
 // fetched per element: a per-row value (constant along the row: any outer strides) for the row or
-// the next one, a row vector (the same row for every outer index) at its column.
+// the next one, a row vector (the same row for every outer index) at its column.  An input whose
+// rows are unit-stride but lie a pitch apart (a [rows, 999] block of a pitch-1024 matrix copied
+// out, ct/submatrix) is read per destination vector from where its row lies, so that the stores,
+// which cost more than the loads when they straddle lines, stay aligned: 59 -> 7x % of peak.
 struct RaggedArgs {
   uint32_t n;                 // elements; < 2^31
   FastDiv inner_fd;           // row length
@@ -454,6 +457,7 @@ struct RaggedArgs {
   FastDiv outer_fd[CT_MAX_DIMS - 1];
   uint32_t dense_mask;        // bit k: operand k is dense (offset = element number)
   uint32_t scalar_mask;       // bit k: one value per row
+  uint32_t pitched_mask;      // bit k: unit-stride rows wherever the outer strides put them (a block of a wider matrix)
   uint32_t const_mask;        // bit k: a constant; every other input is a row vector
   uint32_t streaming;
   char* ptr[kMaxOps];
@@ -501,6 +505,19 @@ __global__ void __launch_bounds__(kBlock) ew_ragged_kernel(const F f, const Ragg
 #pragma unroll
         for (int i = 0; i < VEC; ++i) x.v[i] = e0 + i < a.n ? base[e0 + i] : T{};
       }
+    } else if ((a.pitched_mask >> k) & 1u) {
+      // the destination's aligned vector is the tail of one row of this operand and, past the row's end,
+      // the head of the next: a load that needs only the element's alignment when it stays inside the row
+      const T* rp = base + row_offset(k, row) + col;
+      if (in_row >= (uint32_t)VEC) {
+        const UVec<T, VEC> u = *reinterpret_cast<const UVec<T, VEC>*>(rp);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = u.v[i];
+      } else {
+        const T* np = e0 + in_row < a.n ? base + row_offset(k, row + 1) : rp;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) x.v[i] = (uint32_t)i < in_row ? rp[i] : (e0 + i < a.n ? np[(uint32_t)i - in_row] : T{});
+      }
     } else if ((a.scalar_mask >> k) & 1u) {
       const T cur = base[row_offset(k, row)];
       T next = cur;
@@ -539,6 +556,63 @@ __global__ void __launch_bounds__(kBlock) ew_ragged_kernel(const F f, const Ragg
 #pragma unroll
     for (int i = 0; i < VEC; ++i)
       if (e0 + i < a.n) dp[i] = r.v[i];
+  }
+}
+
+// ------------------------------------------------------------------ SHORT PITCHED ROWS
+//
+// A dense [rows, w] destination taken from rows of a small pitch (ten values out of every sixteen:
+// the first columns of a narrow matrix).  The memory system moves whole 64-byte lines whichever
+// bytes are asked for, so a block takes the contiguous span of memory that holds its rows, padding
+// included, with aligned 16-byte non-temporal loads, parks it in LDS and picks the values of its
+// destination vectors from there; the stores are aligned and dense.  assign! (with conversion) only.
+// (Per-vector loads from where the rows lie, as the ragged kernel does for longer rows, reach 52 % of
+// peak on float [4M, 10] of pitch 16; the lines that have to move bound it at 77 %.)
+struct SpanArgs {
+  char* ptr[2];
+  uint32_t rows;
+  uint32_t w, pitch;
+  FastDiv w_fd;
+  uint32_t rows_per_block;
+};
+
+constexpr int kSpanLdsBytes = 16384;
+
+template <class F, int VEC>
+__global__ void __launch_bounds__(kBlock) ew_span_kernel(const F f, const SpanArgs a) {
+  using Out = typename F::Out;
+  using In = typename F::In0;
+  constexpr int IV = 16 / (int)sizeof(In);
+  __shared__ __align__(16) char smem[kSpanLdsBytes];
+  In* tile = reinterpret_cast<In*>(smem);
+  const uint32_t row0 = blockIdx.x * a.rows_per_block;
+  const uint32_t n_rows = a.rows - row0 < a.rows_per_block ? a.rows - row0 : a.rows_per_block;
+  const In* src = reinterpret_cast<const In*>(a.ptr[1]) + (int64_t)row0 * a.pitch;
+  // the last row of the tensor ends with its last value: nothing behind it may be read
+  const uint32_t span = (n_rows - 1) * a.pitch + a.w;
+  const uint32_t span_vecs = span / IV;
+  for (uint32_t v = threadIdx.x; v < span_vecs; v += kBlock)
+    reinterpret_cast<Vec<In, IV>*>(tile)[v] = nt_load(reinterpret_cast<const Vec<In, IV>*>(src) + v);
+  for (uint32_t e = span_vecs * IV + threadIdx.x; e < span; e += kBlock) tile[e] = src[e];
+  __syncthreads();
+  const uint32_t count = n_rows * a.w;
+  Out* dst = reinterpret_cast<Out*>(a.ptr[0]) + (int64_t)row0 * a.w;
+  for (uint32_t e0 = threadIdx.x * VEC; e0 < count; e0 += kBlock * VEC) {
+    uint32_t r, c;
+    a.w_fd.divmod(e0, r, c);
+    Vec<Out, VEC> out;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      out.v[i] = f(tile[r * a.pitch + c], typename F::In1{}, typename F::In2{});
+      if (++c == a.w) { c = 0; ++r; }
+    }
+    if (e0 + VEC <= count) {
+      *reinterpret_cast<Vec<Out, VEC>*>(dst + e0) = out;
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i)
+        if (e0 + i < count) dst[e0 + i] = out.v[i];
+    }
   }
 }
 
@@ -1089,6 +1163,7 @@ int prepare_gen(const Plan& plan, const EwOperand* ops, GenArgs* args, bool* use
 bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* args, int* n_short, int* ppt, uint32_t* grid);
 bool prepare_ragged(const Plan& plan, const EwOperand* ops, int vmax, RaggedArgs* args);
 bool prepare_vecu(const Plan& plan, const EwOperand* ops, int vmax, VecArgs* args, uint32_t* inner_elems);
+bool prepare_span(const Plan& plan, const EwOperand* ops, int vmax, SpanArgs* args);
 
 // Functors that the lace kernel is built for declare `static constexpr bool kLace = true`.
 template <class F, class = void> struct has_lace : std::false_type {};
@@ -1235,6 +1310,14 @@ int launch_elementwise(hipStream_t s, const F& f, const EwOperand* ops, int64_t 
     int vec = 1;
     bool has_tail = false;
     if (int rc = prepare_vec(plan, ops, VMAX, &main_args, &vec, &tail_args, &has_tail)) return rc;
+    if constexpr (has_lace<F>::value && F::NIN == 1) {
+      SpanArgs sa;
+      if (prepare_span(plan, ops, VMAX, &sa)) {
+        note_kernel("span");
+        hipLaunchKernelGGL((ew_span_kernel<F, VMAX>), dim3((sa.rows + sa.rows_per_block - 1) / sa.rows_per_block), dim3(kBlock), 0, s, f, sa);
+        return after_launch(s);
+      }
+    }
     if constexpr (VMAX > 1) {
       RaggedArgs ra;
       if (vec == 1 && prepare_ragged(plan, ops, VMAX, &ra)) {

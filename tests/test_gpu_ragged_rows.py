@@ -112,7 +112,11 @@ def test_rows_off_the_vector_grid(P, code):
         sub = lambda b: View(b, [rows, width], [pitch, 1], offset=offset)
         k = P.run(H.assign, View(dense, [rows, width]), sub(src))
         exact(dense, f"copy out of a pitched block [{rows},{width}]/{pitch}+{offset} ({k})")
-        if n >= 4096 and (width % vmax or pitch % vmax or offset % vmax):
+        # a dense destination takes aligned vectors that may straddle a row end when the rows are no whole number of
+        # vectors; otherwise each row is walked in vectors that start wherever the row does
+        if n >= 4096 and width % vmax and pitch != width:
+            assert k == "ragged", (k, rows, width, pitch, offset)
+        elif n >= 4096 and (pitch % vmax or offset % vmax):
             assert k == "vecu", (k, rows, width, pitch, offset)
         k = P.run(H.binary_op, sub(pitched), sub(src), 1.0, sub(other), -1.0, "+")
         exact(pitched, f"pitched block minus pitched block ({k})")
@@ -132,7 +136,32 @@ def test_conversion_off_the_vector_grid(P):
     out = P.buf(np.zeros(rows * width, np.float32))
     k = P.run(H.assign, View(out, [rows, width]), View(pix, [rows, width], [pitch, 1], offset=1))
     exact(out, f"u8 block to float ({k})")
-    assert k == "vecu", k
+    assert k == "ragged", k
     back = P.buf(np.zeros(rows * pitch + 4, np.int16))
     k = P.run(H.assign, View(back, [rows, width], [pitch, 1], offset=3), View(out, [rows, width]))
     exact(back, f"float to a pitched short block ({k})")
+
+
+@pytest.mark.parametrize("pair", [(capi.F32, capi.F32), (capi.U8, capi.F32), (capi.F32, capi.I16), (capi.F64, capi.F32),
+                                  (capi.I8, capi.I64)])
+def test_short_rows_of_a_small_pitch(P, pair):
+    """A dense [rows, w] destination from rows of a pitch of at most 128 bytes (the first ten of every sixteen
+    values): a block stages the span of memory that holds its rows through LDS (ew_span_kernel).  assign!, with
+    conversion; a last block that is not full, and a width that leaves the padding of the last row unread."""
+    src_code, dst_code = pair
+    rng = np.random.default_rng(96)
+    item = NP[src_code]().itemsize
+    for rows, w, pitch in ((150000, 10, 16), (300017, 5, 8), (70001, 19, 128 // item)):
+        if pitch * item > 128 or w * 5 > pitch * 4 or pitch <= w:
+            continue
+        src = P.buf(values(rng, src_code, (rows - 1) * pitch + w))       # the buffer ends with the last row's last value
+        out = P.buf(np.zeros(rows * w, NP[dst_code]))
+        k = P.run(H.assign, View(out, [rows, w]), View(src, [rows, w], [pitch, 1]))
+        exact(out, f"short rows {w} of pitch {pitch}, {rows} rows ({k})")
+        assert k == "span", (k, rows, w, pitch)
+    # a destination that is not dense, or too small a call, keeps the other kernels
+    src = P.buf(values(rng, src_code, 4000 * 16))
+    out = P.buf(np.zeros(4000 * 12, NP[dst_code]))
+    k = P.run(H.assign, View(out, [4000, 10], [12, 1]), View(src, [4000, 10], [16, 1]))
+    exact(out, f"pitched destination ({k})")
+    assert k != "span", k
