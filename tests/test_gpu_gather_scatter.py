@@ -101,6 +101,8 @@ ACCUM_CASES = [
     (9000, 9000, 4, "accum_grouped_vec"),     # no duplicates at all
     (131075, 40000, 4, "accum_grouped_vec"),  # many entries, few duplicates, a count off every power of two
     (300, 1, 20, "accum_grouped_vec"),        # every row lands on one destination row
+    (30000, 70000, 4, "accum_grouped_vec"),   # index values beyond 16 bits: a third pass of the radix sort
+    (9001, 17000000, 1, "accum_grouped"),     # and beyond 24 bits: the fourth
 ]
 
 
