@@ -829,25 +829,37 @@ def summarize(prof_dir: str, out_dir: str) -> None:
         wcalls = plans["write"]["segments"][wi[0]]["calls"] if wi else 1
         per_call_us, per_call_bytes = 0.0, 0.0
         rows = []
+        call_sums = np.zeros(calls)     # kernel time of each call, when every kernel runs a whole number of times per call
         for name, durs in kernels.items():
             per = len(durs) / calls
             fk = float(np.sum(fseg.get(name, [0.0]))) / fcalls
             wk = float(np.sum(wseg.get(name, [0.0]))) / wcalls
             per_call_us += float(np.sum(durs)) / calls
             per_call_bytes += (fk * f_fac + wk * w_fac) * 1024
-            rows.append("      %-78s %6.2f/call %9.2f %9.2f %9.2f %12.1f %12.1f" % (
-                name[:78], per, float(np.mean(durs)), float(np.min(durs)), float(np.max(durs)), fk, wk))
+            if call_sums is not None and len(durs) % calls == 0:
+                call_sums = call_sums + np.asarray(durs).reshape(calls, -1).sum(axis=1)
+            else:
+                call_sums = None
+            rows.append("      %-70s %5.2f/call %9.2f %9.2f %9.2f %9.2f %12.1f %12.1f" % (
+                name[:70], per, float(np.mean(durs)), float(np.median(durs)), float(np.min(durs)), float(np.max(durs)), fk, wk))
         if key == "step":
-            lines.append("%s\n    %d steps; kernels of the timed region (avg / min / max us per dispatch; FETCH / WRITE KiB per step):" % (seg["label"], calls))
+            lines.append("%s\n    %d steps; kernels of the timed region (avg / median / best / max us per dispatch; FETCH / WRITE KiB per step):" % (seg["label"], calls))
             lines.extend(rows)
             continue
         rate = alg / per_call_us / 1e3 if per_call_us > 0 else 0.0
-        lines.append("%s\n    key %s: %d calls, kernel time %.2f us per call = %.0f GB/s = %.1f %% of 8 TB/s; HBM traffic %.0f bytes per call "
-                     "= %.4f x the %d algorithmic bytes" % (seg["label"], key, calls, per_call_us, rate, rate / 80,
+        spread = ""
+        if call_sums is not None and calls > 0:
+            med, best = float(np.median(call_sums)), float(np.min(call_sums))
+            spread = " (median %.2f us = %.1f %%, best %.2f us = %.1f %%)" % (med, alg / med / 8e4, best, alg / best / 8e4)
+        lines.append("%s\n    key %s: %d calls, kernel time %.2f us per call = %.0f GB/s = %.1f %% of 8 TB/s%s; HBM traffic %.0f bytes per call "
+                     "= %.4f x the %d algorithmic bytes" % (seg["label"], key, calls, per_call_us, rate, rate / 80, spread,
                                                             per_call_bytes, per_call_bytes / alg, alg))
         lines.extend(rows)
         traffic[key] = {"traffic": int(round(per_call_bytes)), "kernel_us": round(per_call_us, 2),
                         "kernels": [name[:100] for name in kernels], "algorithmic_bytes": alg}
+        if call_sums is not None and calls > 0:
+            traffic[key]["kernel_us_median"] = round(float(np.median(call_sums)), 2)
+            traffic[key]["kernel_us_best"] = round(float(np.min(call_sums)), 2)
 
     sha = shas.pop()
     head = f"""rocprofv3 summary of bench.py on one MI355X (gfx950): every workload of the step, the other BASELINE configs, the
@@ -862,8 +874,8 @@ Commands (from the repository root, one rocprofv3 run each; P = gpurun_out/prof)
 
 With --profile-plan every timed segment of the run starts with a one-byte fill, and the dispatches between two such markers
 belong to one workload: durations and counters are attributed by dispatch order, not by kernel name.
-Per kernel: launches per call, then avg / min / max duration in microseconds (kernel trace), then FETCH_SIZE and WRITE_SIZE
-in KiB per call.  HBM traffic = FETCH x {f_fac:.4f} + WRITE x {w_fac:.4f}: the factors make the calibration copy (exactly
+Per kernel: launches per call, then avg / median / best / max duration in microseconds (kernel trace), then FETCH_SIZE and
+WRITE_SIZE in KiB per call.  Per workload: the average kernel time of a call, and the median and the best call.  HBM traffic = FETCH x {f_fac:.4f} + WRITE x {w_fac:.4f}: the factors make the calibration copy (exactly
 {cal_kib:.0f} KiB each way) read {cal_kib:.0f}; FETCH_SIZE reported {f_raw:.1f} KiB for it (it counts half the bytes on this part),
 WRITE_SIZE {w_raw:.1f} KiB.  GB/s = algorithmic bytes / summed kernel time of one call; bench.py's own HIP-event figures
 (avg_call_us) also contain the gaps between dispatches.

@@ -287,8 +287,8 @@ int ct_unary_reduce(void* stream, void* output, const ct_dims* output_dims, doub
                     const void* input, const ct_dims* input_dims, int op, int dtype);
 
 /* The same reduction for callers that cannot allocate device memory while they
- * run: code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc.  No counterpart in the reference.  It runs ct_unary_reduce's
+ * run: tight serving loops, harnesses that forbid hipMalloc, code that records
+ * its calls into a graph.  No counterpart in the reference.  It runs ct_unary_reduce's
  * kernels with ct_unary_reduce's plan, so the results are the same bits, but
  * the partial accumulators of a split reduction (a column reduction through a
  * transposed view, a few very long rows) live in a fixed 2 MiB array that every
@@ -297,8 +297,11 @@ int ct_unary_reduce(void* stream, void* output, const ct_dims* output_dims, doub
  * than 2 MiB fails with CT_ERR_INVALID and launches nothing.  All calls on one
  * device share the array: calls that overlap in time on one device (two
  * streams, two host threads) race; calls on one stream are ordered and safe.
- * The first call on a device resolves the array's address; make that call
- * before a graph capture starts. */
+ * The first call on a device resolves the array's address.  The property is
+ * "allocates nothing"; recording the call into a HIP graph has not been tried,
+ * and a caller who does so must resolve the address with a call outside the
+ * capture first and leave debug-sync mode off (with ct_set_debug_sync(1) every
+ * call waits for its stream, which a capture does not allow). */
 int ct_unary_reduce_noalloc(void* stream, void* output, const ct_dims* output_dims,
                             double input_alpha, const void* input, const ct_dims* input_dims,
                             int op, int dtype);
