@@ -413,6 +413,89 @@ def test_broadcast_accumulates_at_benchmark_size():
         t.free()
 
 
+def test_streamed_accumulates_at_benchmark_size():
+    """[4096] <- the 16384 rows of a [16384, 4096] float matrix under operations that only the serial order
+    defines (:*, :/ reversed, :- reversed, :+ under a destination multiplier of 0.9): bit for bit against the
+    oracle's chain e = 0 .. n-1 (src/cortex/compute/cpu/tensor_math.clj:386-420)."""
+    rows, cols = 16384, 4096
+    rng = np.random.default_rng(84)
+    y = (1.0 + 0.01 * rng.standard_normal((rows, cols))).astype(np.float32)
+    y[77, 5] = np.nan
+    y[4000, 9] = 0.0
+    y[9000, 9] = -0.0
+    start = rng.standard_normal(cols).astype(np.float32)
+    d_y = Dev(y)
+    row_view, full = dims([rows, cols], [0, 1]), dims([rows, cols])
+    for op, dest_alpha, y_alpha, reverse, kernel in (("*", 1.0, 1.0, 0, "accum_stream_plain"), ("/", 1.0, 1.0, 1, "accum_stream_plain"),
+                                                     ("-", 1.0, 1.0, 1, "accum_stream_plain"), ("+", 0.9, 1.0, 0, "accum_stream"),
+                                                     ("max", 0.999, 0.5, 0, "accum_stream")):
+        d_acc = Dev(start)
+        capi.call("ct_binary_accum", None, d_acc.ptr, C.byref(row_view), dest_alpha, d_y.ptr, C.byref(full), y_alpha, rows * cols,
+                  capi.BINARY_OPS[op], reverse, 1, capi.F32)
+        assert capi.last_kernel() == kernel, (op, capi.last_kernel())
+        want = start.copy()
+        ob.call("binary_accum", want.ctypes.data, C.byref(row_view), dest_alpha, y.ctypes.data, C.byref(full), y_alpha, rows * cols,
+                capi.BINARY_OPS[op], reverse, 1, capi.F32)
+        assert bits_equal(d_acc.download(), want), op
+        d_acc.free()
+    # each row into one element: the chains lie along the unit-stride axis
+    col_view = dims([cols, rows], [1, 0])
+    yt = dims([cols, rows])
+    d_acc = Dev(start)
+    capi.call("ct_binary_accum", None, d_acc.ptr, C.byref(col_view), 1.0, d_y.ptr, C.byref(yt), 1.0, rows * cols,
+              capi.BINARY_OPS["*"], 0, 1, capi.F32)
+    assert capi.last_kernel() == "accum_stream_steps_plain", capi.last_kernel()
+    want = start.copy()
+    ob.call("binary_accum", want.ctypes.data, C.byref(col_view), 1.0, y.ctypes.data, C.byref(yt), 1.0, rows * cols,
+            capi.BINARY_OPS["*"], 0, 1, capi.F32)
+    assert bits_equal(d_acc.download(), want)
+    for t in (d_y, d_acc):
+        t.free()
+
+
+def test_blocks_of_a_wider_matrix_at_benchmark_size():
+    """ct/submatrix at the benchmark's sizes (tensor.clj:490-513): a [65536, 999] block of a pitch-1024 float
+    matrix copied out and written back (calls large enough for the stores to bypass the caches), rows of 10 out
+    of a pitch of 16 gathered into a dense matrix, and a block converted to double on the way.  numpy's slices
+    are the closed form; what lies between the rows of a pitched destination must stay as it was."""
+    rows, width, pitch = 65536, 999, 1024
+    rng = np.random.default_rng(85)
+    wide = rng.standard_normal((rows, pitch)).astype(np.float32)
+    d_wide, d_block = Dev(wide), Dev(np.zeros(rows * width, np.float32))
+    pitched, dense = dims([rows, width], [pitch, 1]), dims([rows, width])
+    capi.call("ct_assign", None, d_block.ptr, C.byref(dense), capi.F32, d_wide.ptr, C.byref(pitched), capi.F32, rows * width)
+    assert capi.last_kernel() == "ragged", capi.last_kernel()
+    assert bits_equal(d_block.download().reshape(rows, width), wide[:, :width])
+    fresh = rng.standard_normal((rows, width)).astype(np.float32)
+    d_fresh = Dev(fresh)
+    capi.call("ct_assign", None, d_wide.ptr, C.byref(pitched), capi.F32, d_fresh.ptr, C.byref(dense), capi.F32, rows * width)
+    assert capi.last_kernel() == "vecu", capi.last_kernel()
+    want = wide.copy()
+    want[:, :width] = fresh
+    assert bits_equal(d_wide.download().reshape(rows, pitch), want)
+    # a block that starts one element into the rows: nothing of it lies on the 16-byte grid
+    off_rows = rows - 1
+    d_block2 = Dev(np.zeros(off_rows * width, np.float32))
+    capi.call("ct_assign", None, d_block2.ptr, C.byref(dims([off_rows, width])), capi.F32, d_wide.ptr + 4 * 21,
+              C.byref(dims([off_rows, width], [pitch, 1])), capi.F32, off_rows * width)
+    flat = want.reshape(-1)
+    expect = np.lib.stride_tricks.as_strided(flat[21:], (off_rows, width), (4 * pitch, 4))
+    assert bits_equal(d_block2.download().reshape(off_rows, width), np.ascontiguousarray(expect))
+    d_double = Dev(np.zeros(rows * width, np.float64))
+    capi.call("ct_assign", None, d_double.ptr, C.byref(dense), capi.F64, d_wide.ptr, C.byref(pitched), capi.F32, rows * width)
+    assert bits_equal(d_double.download().reshape(rows, width), want[:, :width].astype(np.float64))
+    for t in (d_block, d_fresh, d_block2, d_double):
+        t.free()
+    short_rows, short_w, short_pitch = 1 << 22, 10, 16
+    d_short = Dev(np.zeros(short_rows * short_w, np.float32))
+    capi.call("ct_assign", None, d_short.ptr, C.byref(dims([short_rows, short_w])), capi.F32, d_wide.ptr,
+              C.byref(dims([short_rows, short_w], [short_pitch, 1])), capi.F32, short_rows * short_w)
+    assert capi.last_kernel() == "span", capi.last_kernel()
+    assert bits_equal(d_short.download().reshape(short_rows, short_w), want.reshape(short_rows, short_pitch)[:, :short_w])
+    for t in (d_wide, d_short):
+        t.free()
+
+
 def test_matrix_of_2_31_elements_built_and_reduced():
     """A float matrix of 65536 x 32768 (2^31 elements, 8 GiB: one element more than a 32-bit index
     counts) is built on the device as column[r] + row[c] (r % 5 and c % 7, so that every sum below is an
