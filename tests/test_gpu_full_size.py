@@ -403,6 +403,14 @@ def test_broadcast_accumulates_at_benchmark_size():
             scale = np.abs(start.astype(np.float64)) + np.abs(np.nan_to_num(y.astype(np.float64))).sum(axis=0)
             ok = np.abs(got.astype(np.float64) - want) <= 2e-6 * scale
             assert np.all(ok | (np.isnan(got) & np.isnan(want)))
+            # and against the sum itself.  The kernel leaves what unary-reduce! :sum followed by binary-op! :+ would:
+            # the column's sum (formed in double) rounded to float, added to the start, rounded again.  Half a unit
+            # in the last place for each rounding, plus what 16384 double additions can lose relative to the
+            # magnitudes they add
+            col_sum = y.astype(np.float64).sum(axis=0)
+            exact = start.astype(np.float64) + col_sum
+            near = np.abs(got.astype(np.float64) - exact) <= 6.0e-8 * (np.abs(col_sum) + np.abs(exact)) + 1e-11 * scale
+            assert np.all(near | (np.isnan(got) & np.isnan(exact)))
         d_acc.free()
     whole = rng.integers(-8, 9, (rows, cols)).astype(np.float32)
     d_whole, d_acc = Dev(whole), Dev(np.zeros(cols, np.float32))
