@@ -342,6 +342,7 @@ bool prepare_lace(const Plan& plan, const EwOperand* ops, int vmax, LaceArgs* a,
     }
   }
   if (!any_laced || !any_planar) return false;
+  a->streaming = streaming_level(plan, ops) > 0 ? 1u : 0u;
   int64_t rows = 1;
   int no = 0;
   for (int d = 0; d < c.nd; ++d) {

@@ -904,6 +904,7 @@ struct LaceArgs {
   int64_t plane_stride[kMaxOps];   // planar operands: stride along S
   uint32_t laced_mask;             // bit k: operand k is laced
   uint32_t const_mask;
+  uint32_t streaming;              // the call moves more than the caches hold: the stores bypass them
   uint64_t cbits[kMaxOps];
 };
 
@@ -1004,7 +1005,15 @@ __global__ void __launch_bounds__(kBlock) ew_lace_kernel(const F f, const LaceAr
   if (!(a.laced_mask & 1u)) {
     if (live) {
 #pragma unroll
-      for (int c = 0; c < S; ++c) *reinterpret_cast<Vec<Out, PPT>*>(dbase + c * a.plane_stride[0] + l_blk + lp) = o[c];
+      for (int c = 0; c < S; ++c) {
+        Vec<Out, PPT>* dp = reinterpret_cast<Vec<Out, PPT>*>(dbase + c * a.plane_stride[0] + l_blk + lp);
+        if (a.streaming) {
+          asm volatile("");  // keeps the two stores apart: merged into one, they lose the hint
+          nt_store(o[c], dp);
+        } else {
+          *dp = o[c];
+        }
+      }
     }
     return;
   }
@@ -1026,7 +1035,12 @@ __global__ void __launch_bounds__(kBlock) ew_lace_kernel(const F f, const LaceAr
         const uint32_t flat = vi * PPT + e;
         v.v[e] = *reinterpret_cast<const Out*>(smem + (flat % S) * kPlaneBytes + (flat / S) * sizeof(Out));
       }
-      run[vi] = v;
+      if (a.streaming) {
+        asm volatile("");
+        nt_store(v, run + vi);
+      } else {
+        run[vi] = v;
+      }
     }
   }
 }
