@@ -129,8 +129,9 @@ __device__ __forceinline__ void softmax_row_base(const SoftmaxArgs& a, int64_t r
 // it in registers: one read, one write.  VEC > 1 needs unit-stride, aligned rows.
 // The division by the row sum is a multiplication by its reciprocal (at most
 // one ulp from the quotient).
-// NT: the call moves more than the last-level cache holds, and the loads are non-temporal (rows of
-// 1024 floats, 1 GiB: +2 % of peak; 128 MiB: -7 %).
+// NT: the call moves more than the last-level cache holds, and the loads and stores are non-temporal
+// (rows of 1024 floats, 1 GiB: +2 % of peak for the loads, +2 to 3 for the stores; 128 MiB: -7 %).  The
+// same stores did nothing for the lane-per-row kernel of the spatial form.
 template <class T, int VEC, int TPR, int ITER, bool NT>
 __global__ void __launch_bounds__(kBlock) softmax_wave_kernel(const SoftmaxArgs a) {
   using V = Vec<T, VEC>;
@@ -177,8 +178,12 @@ __global__ void __launch_bounds__(kBlock) softmax_wave_kernel(const SoftmaxArgs 
     if (live && i < nv) {
 #pragma unroll
       for (int e = 0; e < VEC; ++e) x[j].v[e] *= inv;
-      if constexpr (VEC > 1) *reinterpret_cast<V*>(out + (int64_t)i * VEC) = x[j];
-      else out[(int64_t)i * a.out_k] = x[j].v[0];
+      if constexpr (VEC > 1) {
+        if constexpr (NT) nt_store(x[j], reinterpret_cast<V*>(out + (int64_t)i * VEC));
+        else *reinterpret_cast<V*>(out + (int64_t)i * VEC) = x[j];
+      } else {
+        out[(int64_t)i * a.out_k] = x[j].v[0];
+      }
     }
   }
 }
