@@ -149,3 +149,68 @@ def test_short_chains_keep_the_lane_per_element_kernel(P):
     k = P.run(H.binary_accum, View(d, [4096]), 1.0, View(y, [64, 4096]), 1.0, "*", requires_cas=True)
     assert k == "accum_owner", k
     exact(d, "64 updates per element")
+
+
+@pytest.mark.parametrize("seed", [301, 302])
+def test_random_broadcast_destinations(pair_factory, seed):
+    """A seeded sweep over destination and update layouts (dense, padded rows, permuted views, strided and
+    stride-0 destinations), every datatype, operations and multipliers of either sign, operands in either
+    order: whichever kernel takes the call (one lane per element, staged, streamed), the destination must hold
+    what the serial loop leaves, bit for bit; only a float :+ with dest_alpha 1 keeps the reference's 1e-4."""
+    rng = np.random.default_rng(seed)
+    kernels = {}
+
+    def fill(n, dt):
+        if np.issubdtype(dt, np.floating):
+            return (1.0 + 0.02 * rng.standard_normal(n)).astype(dt)
+        v = rng.integers(-3, 4, n)
+        return np.where(v == 0, 1, v).astype(dt)
+
+    for it in range(500):
+        with pair_factory() as P:
+            code = int(rng.choice(H.ALL_DTYPES))
+            dt = NP[code]
+            nd = int(rng.integers(2, 5))
+            yshape = [int(rng.choice([1, 2, 3, 5, 8, 17, 33, 64, 130, 257, 700])) for _ in range(nd)]
+            while np.prod(yshape) > 400_000:
+                yshape[int(np.argmax(yshape))] //= 2
+            dshape = [s if rng.random() < 0.4 else 1 for s in yshape]
+            mode = int(rng.integers(0, 3))
+            ystr = None
+            if mode == 1:
+                pad, run, ystr = int(rng.choice([0, 1, 4, 16])), 1, [0] * nd
+                for d in reversed(range(nd)):
+                    ystr[d] = run
+                    run *= yshape[d] + (pad if d == nd - 1 else 0)
+            elif mode == 2:
+                run, ystr = 1, [0] * nd
+                for d in rng.permutation(nd):
+                    ystr[d] = run
+                    run *= yshape[d]
+            y_elems = 1 + sum((s - 1) * st for s, st in zip(yshape, ystr)) if ystr else int(np.prod(yshape))
+            dstr = None
+            if rng.random() < 0.3:
+                mult, run, dstr = int(rng.choice([2, 3])), 1, [0] * nd
+                for d in reversed(range(nd)):
+                    dstr[d] = run * mult if dshape[d] > 1 else (0 if rng.random() < 0.5 else run * mult)
+                    run *= dshape[d]
+            d_elems = 1 + sum((s - 1) * st for s, st in zip(dshape, dstr)) if dstr else int(np.prod(dshape))
+            floating = code in FLOATS
+            ops = ["*", "/", "-", "+", "max", "min", ">=", "eq"] if floating else ["*", "-", "+", "bit-xor", "bit-and", "max", "<"]
+            op = str(rng.choice(ops))
+            da = float(rng.choice([1.0, 1.0, 0.9, -1.0, 2.0] if floating else [1.0, 1.0, 3.0, -1.0]))
+            ya = float(rng.choice([1.0, 1.0, -1.0, 0.5] if floating else [1.0, -1.0, 2.0]))
+            rev = bool(rng.integers(0, 2))
+            y = View(P.buf(fill(y_elems, dt)), yshape, ystr)
+            d = P.buf(fill(d_elems, dt))
+            what = f"case {it}: {op} dtype {code} y {yshape} {ystr} dest {dshape} {dstr} da={da} ya={ya} reverse={rev}"
+            k = P.run(H.binary_accum, View(d, dshape, dstr), da, y, ya, op, reverse=rev, requires_cas=True)
+            kernels[k] = kernels.get(k, 0) + 1
+            if k == "accum_staged_sum" and floating:
+                reps = np.prod(yshape) / max(1, np.prod(dshape))
+                got, want = d.download().astype(np.float64), d.host.astype(np.float64)
+                assert np.all(np.abs(got - want) <= 1e-4 * (np.abs(want) + reps)), what
+            else:
+                H.assert_bit_exact(d.download(), d.host, what + f" ({k})")
+    streamed = sum(v for k, v in kernels.items() if k.startswith("accum_stream"))
+    assert streamed >= 40 and kernels.get("accum_owner", 0) >= 100, kernels
