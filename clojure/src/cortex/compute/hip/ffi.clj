@@ -9,7 +9,7 @@
   UNEXERCISED: no JVM exists where this repository is built and tested.  The same entry points,
   in the same argument order, are driven through ctypes by cortex_amd/capi.py and
   cortex_amd/driver.py; tests/test_clojure_glue.py checks every ct_* call in these files
-  against the header (name and argument count)."
+  against the header (name, argument count, and the machine type each coercion yields)."
   (:require [think.datatype.core :as dtype]
             [clojure.core.matrix :as m])
   (:import [com.sun.jna Function NativeLibrary Pointer Memory]

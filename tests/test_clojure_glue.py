@@ -1,7 +1,7 @@
 """The Clojure glue under clojure/src cannot be executed here (no JVM).  What can be checked on
 the text is checked: every file reads as balanced Clojure forms, every `ct_*` entry point it
 invokes is declared in include/cortex_hip.h with exactly as many parameters as the call passes
-arguments, every TensorMath method of the reference's protocol is implemented with the protocol's
+arguments, each argument is coerced to the class that JNA marshals at the width the header declares, every TensorMath method of the reference's protocol is implemented with the protocol's
 arity, and every entry point of the header is reachable from the glue."""
 import re
 from pathlib import Path
@@ -107,6 +107,66 @@ def test_every_native_call_matches_the_header():
     for file, name, argc in calls:
         assert name in declared, f"{file}: {name} is not declared in include/cortex_hip.h"
         assert argc == declared[name], f"{file}: {name} is called with {argc} arguments, the header declares {declared[name]}"
+
+
+def header_parameter_kinds():
+    """Entry point -> the machine kind of each parameter: 'ptr', 'i32', 'i64', 'f64' or 'f32'."""
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:int|const char\*)\s+(ct_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        params = m.group(2).strip()
+        kinds = []
+        for p in ([] if params in ("", "void") else params.split(",")):
+            p = p.strip()
+            if "*" in p or "[" in p:
+                kinds.append("ptr")
+            elif re.match(r"(const\s+)?double\b", p):
+                kinds.append("f64")
+            elif re.match(r"(const\s+)?float\b", p):
+                kinds.append("f32")
+            elif re.match(r"(const\s+)?(u?int64_t|size_t)\b", p):
+                kinds.append("i64")
+            else:
+                assert re.match(r"(const\s+)?(int|u?int32_t|unsigned|ct_[a-z_]+_t)\b", p), (m.group(1), p)
+                kinds.append("i32")
+        out[m.group(1)] = kinds
+    return out
+
+
+# How JNA marshals what each coercion of the glue produces (Integer -> 32 bits, Long -> 64 bits, Double -> a double,
+# Pointer / Memory / ...ByReference / nil -> a pointer): the head of an argument form -> its machine kind.
+COERCIONS = {
+    "int": "i32", "dtype-code": "i32", "ffi/dtype-code": "i32", "op-code": "i32", "ffi/op-code": "i32",
+    "bool->int": "i32", "ffi/bool->int": "i32",
+    "long": "i64", "double": "f64", "float": "f32",
+    "->ptr": "ptr", "dims": "ptr", ":handle": "ptr", "ffi/conv-desc->native": "ptr", "ffi/pool-desc->native": "ptr",
+    "arg-indexes": "ptr", "when": "ptr",
+}
+
+
+def test_every_native_call_passes_the_headers_machine_types():
+    """JNA picks the native width from the Java class of each argument, so an (int ...) where the header says
+    int64_t, or a (long ...) where it says int, would put a wrong-sized value on the stack without any error.
+    Every argument of every call is a coercion form whose result class is known, or a bare symbol (a handle, a
+    pointer or a ...ByReference out-parameter): its kind must be the header's, parameter by parameter."""
+    declared = header_parameter_kinds()
+    checked = 0
+    for path in GLUE:
+        for form in walk(read_forms(path.read_text())):
+            if not (len(form) >= 3 and form[0] == "(" and form[1] == "call!" and isinstance(form[2], tuple)):
+                continue
+            name, args = form[2][1], form[3:]
+            for position, (arg, want) in enumerate(zip(args, declared[name])):
+                if isinstance(arg, str):
+                    assert not re.fullmatch(r"-?[0-9.]+", arg), f"{path.name}: {name} argument {position} is a bare number"
+                    got = "ptr"
+                else:
+                    assert isinstance(arg, list) and arg[0] == "(", f"{path.name}: {name} argument {position}: {arg!r}"
+                    assert arg[1] in COERCIONS, f"{path.name}: {name} argument {position} is built by {arg[1]!r}, whose class is unknown"
+                    got = COERCIONS[arg[1]]
+                assert got == want, f"{path.name}: {name} argument {position} is passed as {got}, the header declares {want}"
+                checked += 1
+    assert checked > 400
 
 
 def test_every_entry_point_is_bound():
