@@ -169,6 +169,51 @@ def test_every_native_call_passes_the_headers_machine_types():
     assert checked > 400
 
 
+def header_pointee_types():
+    """Entry point -> per parameter the C type a pointer parameter points to (None for values)."""
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:int|const char\*)\s+(ct_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        params = m.group(2).strip()
+        types = []
+        for p in ([] if params in ("", "void") else params.split(",")):
+            pm = re.match(r"\s*(?:const\s+)?([A-Za-z_0-9]+)\s*(\*+)", p)
+            types.append(pm.group(1) + pm.group(2)[1:] if pm else None)
+        out[m.group(1)] = types
+    return out
+
+
+BY_REFERENCE = {"IntByReference.": {"int", "int32_t"}, "LongByReference.": {"size_t", "int64_t", "uint64_t"},
+                "FloatByReference.": {"float"}, "PointerByReference.": {"void*"}}
+
+
+def test_out_parameters_use_the_reference_class_of_the_pointee():
+    """An out-parameter is a JNA ...ByReference object bound by an enclosing let: its class fixes how many bytes
+    the library's store may write (an IntByReference under a size_t* would be overrun)."""
+    pointees = header_pointee_types()
+    checked = 0
+    for path in GLUE:
+        for top in read_forms(path.read_text()):
+            bound = {}
+            for form in walk(top):
+                if len(form) >= 3 and form[0] == "(" and form[1] in ("let", "let*") and isinstance(form[2], list) and form[2][0] == "[":
+                    pairs = form[2][1:]
+                    for sym, init in zip(pairs[0::2], pairs[1::2]):
+                        if isinstance(sym, str) and isinstance(init, list) and len(init) >= 2 and isinstance(init[1], str):
+                            ctor = init[1].split(".")[-2] + "." if init[1].endswith("ByReference.") else None
+                            if ctor:
+                                bound[sym] = ctor
+            for form in walk(top):
+                if len(form) >= 3 and form[0] == "(" and form[1] == "call!" and isinstance(form[2], tuple):
+                    name = form[2][1]
+                    for position, (arg, pointee) in enumerate(zip(form[3:], pointees[name])):
+                        if isinstance(arg, str) and arg in bound:
+                            assert pointee in BY_REFERENCE[bound[arg]], \
+                                f"{path.name}: {name} argument {position} is a {bound[arg][:-1]}, the header declares {pointee}*"
+                            checked += 1
+    assert checked >= 10
+
+
 def test_every_entry_point_is_bound():
     declared = set(header_functions())
     text = "".join(p.read_text() for p in GLUE)
