@@ -214,6 +214,69 @@ def test_out_parameters_use_the_reference_class_of_the_pointee():
     assert checked >= 10
 
 
+LAYOUT_PROBE = r"""
+#include <stddef.h>
+#include <stdio.h>
+#include "cortex_hip.h"
+int main(void) {
+  printf("dims %zu %zu %zu %zu %zu\n", sizeof(ct_dims), offsetof(ct_dims, ndim), offsetof(ct_dims, shape),
+         offsetof(ct_dims, strides), offsetof(ct_dims, index));
+  printf("pool %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(ct_pool_desc), offsetof(ct_pool_desc, kernel_width),
+         offsetof(ct_pool_desc, kernel_height), offsetof(ct_pool_desc, pad_x), offsetof(ct_pool_desc, pad_y),
+         offsetof(ct_pool_desc, stride_x), offsetof(ct_pool_desc, stride_y), offsetof(ct_pool_desc, pool_op));
+  printf("conv %zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(ct_conv_desc), offsetof(ct_conv_desc, in_channels),
+         offsetof(ct_conv_desc, out_channels), offsetof(ct_conv_desc, kernel_width), offsetof(ct_conv_desc, kernel_height),
+         offsetof(ct_conv_desc, pad_x), offsetof(ct_conv_desc, pad_y), offsetof(ct_conv_desc, stride_x),
+         offsetof(ct_conv_desc, stride_y));
+  printf("max_dims %d\n", CT_MAX_DIMS);
+  return 0;
+}
+"""
+
+
+def test_struct_layouts_written_by_hand_are_the_compilers(tmp_path):
+    """ffi.clj fills ct_dims, ct_pool_desc and ct_conv_desc byte by byte into raw memory: the sizes and offsets
+    it uses are compared with what the C compiler makes of the header, field by field and in field order."""
+    import subprocess
+    src = tmp_path / "layout.c"
+    src.write_text(LAYOUT_PROBE)
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-I", str(HEADER.parent), str(src), "-o", str(exe)], check=True)
+    probe = {line.split()[0]: [int(v) for v in line.split()[1:]]
+             for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines()}
+    text = (ROOT / "clojure" / "src" / "cortex" / "compute" / "hip" / "ffi.clj").read_text()
+    const = lambda name: int(re.search(r"\(def \^:const " + re.escape(name) + r" (\d+)\)", text).group(1))
+    assert [const("dims-byte-size"), 0, const("dims-shape-offset"), const("dims-strides-offset"), const("dims-index-offset")] == probe["dims"]
+    assert const("ct-max-dims") == probe["max_dims"][0]
+    assert "(.setInt mem 0 (int (count shape)))" in text          # ndim at offset 0
+    forms = read_forms(text)
+
+    def descriptor(defn_name):
+        """(bytes allocated, [(offset, field symbol)] in the order written) of a `(doto (Memory. n) (.setInt off x) ...)`."""
+        body = [f for f in forms if f[:3] == ["(", "defn", defn_name]][0]
+        doto = [f for f in walk(body) if f[:2] == ["(", "doto"]][0]
+        size = int(doto[2][2])
+        writes = []
+        for f in doto[3:]:
+            assert f[1] == ".setInt", f
+            value = f[3]
+            writes.append((int(f[2]), value[2] if value[1] == "int" else value[-1]))
+        return size, writes
+
+    size, writes = descriptor("pool-desc->native")
+    assert [size] + [off for off, _ in writes] == probe["pool"]
+    assert [name for _, name in writes] == ["kernel-width", "kernel-height", "pad-x", "pad-y", "stride-x", "stride-y", "pool-op"]
+    size, writes = descriptor("conv-desc->native")
+    assert [size] + [off for off, _ in writes] == probe["conv"]
+    assert [name for _, name in writes] == ["in-channels", "out-channels", "kernel-width", "kernel-height", "pad-x", "pad-y",
+                                            "stride-x", "stride-y"]
+    # the ctypes mirror used by the Python side
+    import ctypes as C
+    from cortex_amd import capi
+    assert [C.sizeof(capi.CtDims), capi.CtDims.ndim.offset, capi.CtDims.shape.offset, capi.CtDims.strides.offset,
+            capi.CtDims.index.offset] == probe["dims"]
+
+
 def test_every_entry_point_is_bound():
     declared = set(header_functions())
     text = "".join(p.read_text() for p in GLUE)
