@@ -277,6 +277,51 @@ def test_struct_layouts_written_by_hand_are_the_compilers(tmp_path):
             capi.CtDims.index.offset] == probe["dims"]
 
 
+# keyword of the reference's API -> enumerator suffix of the header, per table
+ENUM_NAMES = {
+    ("datatype->code", "CT_"): {"byte": "I8", "short": "I16", "int": "I32", "long": "I64", "float": "F32", "double": "F64",
+                                "ubyte": "U8"},
+    ("unary-op->code", "CT_UOP_"): {"floor": "FLOOR", "ceil": "CEIL", "round": "ROUND", "-": "NEGATE", "tanh": "TANH",
+                                    "logistic": "LOGISTIC", "exp": "EXP", "sqrt": "SQRT", "noop": "NOOP"},
+    ("binary-op->code", "CT_BOP_"): {"+": "ADD", "-": "SUB", "*": "MUL", "/": "DIV", "min": "MIN", "max": "MAX",
+                                     "bit-and": "BIT_AND", "bit-xor": "BIT_XOR", "eq": "EQ", ">": "GT", ">=": "GE", "<": "LT",
+                                     "<=": "LE"},
+    ("ternary-op->code", "CT_TOP_"): {"select": "SELECT"},
+    ("reduce-op->code", "CT_ROP_"): {"max": "MAX", "min": "MIN", "sum": "SUM", "mean": "MEAN", "magnitude": "MAGNITUDE",
+                                     "magnitude-squared": "MAGNITUDE_SQUARED"},
+    ("activation-op->code", "CT_ACT_"): {"logistic": "LOGISTIC", "tanh": "TANH", "relu": "RELU"},
+    ("pool-op->code", "CT_POOL_"): {"max": "MAX", "avg": "AVG", "avg-exc-pad": "AVG_EXC_PAD"},
+    ("copy-kind", "CT_COPY_"): {"host->device": "HOST_TO_DEVICE", "device->host": "DEVICE_TO_HOST",
+                                "device->device": "DEVICE_TO_DEVICE"},
+}
+
+
+def test_code_tables_are_the_headers_enumerators():
+    """The keyword -> code maps of ffi.clj, and the tables of the Python side, against the enumerators of the header:
+    same keys, same numbers."""
+    header = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    enumerators = {m.group(1): int(m.group(2)) for m in re.finditer(r"\b(CT_[A-Z0-9_]+)\s*=\s*(\d+)", header)}
+    forms = read_forms((ROOT / "clojure" / "src" / "cortex" / "compute" / "hip" / "ffi.clj").read_text())
+    from cortex_amd import capi
+    python_tables = {"datatype->code": capi.DTYPE_CODES, "unary-op->code": capi.UNARY_OPS, "binary-op->code": capi.BINARY_OPS,
+                     "ternary-op->code": capi.TERNARY_OPS, "reduce-op->code": capi.REDUCE_OPS,
+                     "activation-op->code": capi.ACTIVATION_OPS, "pool-op->code": capi.POOL_OPS,
+                     "copy-kind": {"host->device": capi.COPY_H2D, "device->host": capi.COPY_D2H, "device->device": capi.COPY_D2D}}
+    for (table, prefix), names in ENUM_NAMES.items():
+        form = [f for f in forms if f[:3] == ["(", "def", table]][0]
+        literal = [x for x in form[3:] if isinstance(x, list) and x[0] == "{"][0][1:]
+        glue = {k.lstrip(":"): int(v) for k, v in zip(literal[0::2], literal[1::2])}
+        want = {key: enumerators[prefix + suffix] for key, suffix in names.items()}
+        assert glue == want, (table, glue, want)
+        assert python_tables[table] == want, (table, python_tables[table], want)
+        # and no enumerator of that family is left without a keyword
+        family = {n for n in enumerators if n.startswith(prefix) and (prefix != "CT_" or re.fullmatch(r"CT_[IUF]\d+", n))}
+        assert family == {prefix + suffix for suffix in names.values()}, (table, family)
+    assert capi.DISTRIBUTIONS == {"gaussian": enumerators["CT_DIST_GAUSSIAN"], "flat": enumerators["CT_DIST_FLAT"]}
+    tm = (ROOT / "clojure" / "src" / "cortex" / "compute" / "hip" / "tensor_math.clj").read_text()
+    assert re.search(r":gaussian \[%d " % enumerators["CT_DIST_GAUSSIAN"], tm) and re.search(r":flat \[%d " % enumerators["CT_DIST_FLAT"], tm)
+
+
 def test_every_entry_point_is_bound():
     declared = set(header_functions())
     text = "".join(p.read_text() for p in GLUE)
