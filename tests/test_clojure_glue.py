@@ -51,7 +51,10 @@ def read_forms(text: str):
             assert o == PAIR[ch], f"{o!r} opened at offset {where} is closed by {ch!r} at offset {pos}"
             stack.pop()
             pos += 1
-        elif ch in "'`~@^#":                   # reader macros: prefix the next form; #{ and #( open collections
+        elif ch == "^":                        # metadata: annotates the next form and is no form itself
+            stack[-1].append(META)
+            pos += 1
+        elif ch in "'`~@#":                    # reader macros: prefix the next form; #{ and #( open collections
             if ch == "#" and pos + 1 < n and text[pos + 1] == "_":
                 pos += 2
             else:
@@ -61,7 +64,23 @@ def read_forms(text: str):
             stack[-1].append(m.group(0))
             pos += len(m.group(0))
     assert not opened, f"{opened[-1][0]!r} opened at offset {opened[-1][1]} is never closed"
-    return stack[0]
+    return drop_metadata(stack[0])
+
+
+META = object()
+
+
+def drop_metadata(form):
+    """Removes every metadata marker together with the form it introduces (^String, ^:const, ^{:doc ...})."""
+    out, skip = [], False
+    for item in form:
+        if item is META:
+            skip = True
+        elif skip:
+            skip = False
+        else:
+            out.append(drop_metadata(item) if isinstance(item, list) else item)
+    return out
 
 
 def walk(form):
@@ -320,6 +339,99 @@ def test_code_tables_are_the_headers_enumerators():
     assert capi.DISTRIBUTIONS == {"gaussian": enumerators["CT_DIST_GAUSSIAN"], "flat": enumerators["CT_DIST_FLAT"]}
     tm = (ROOT / "clojure" / "src" / "cortex" / "compute" / "hip" / "tensor_math.clj").read_text()
     assert re.search(r":gaussian \[%d " % enumerators["CT_DIST_GAUSSIAN"], tm) and re.search(r":flat \[%d " % enumerators["CT_DIST_FLAT"], tm)
+
+
+DEFINERS = {"def", "defn", "defn-", "defmacro", "defmulti", "defonce", "declare", "defrecord", "deftype", "defprotocol"}
+
+
+def namespace_of(forms):
+    """(name, {alias: namespace}, {referred symbol: namespace}) of a file's ns form."""
+    ns = forms[0]
+    aliases, refers = {}, {}
+    for clause in ns[3:]:
+        if isinstance(clause, list) and len(clause) > 1 and clause[1] == ":require":
+            for spec in clause[2:]:
+                if not (isinstance(spec, list) and spec[0] == "["):
+                    continue
+                target, rest = spec[1], spec[2:]
+                for key, value in zip(rest[0::2], rest[1::2]):
+                    if key == ":as":
+                        aliases[value] = target
+                    elif key == ":refer" and isinstance(value, list):
+                        for sym in value[1:]:
+                            refers[sym] = target
+    return ns[2], aliases, refers
+
+
+def definitions(forms):
+    """Names a file defines at top level -> whether they are private; protocols also define their methods and
+    records their constructor functions."""
+    out = {}
+    for form in forms:
+        if not (isinstance(form, list) and len(form) > 2 and form[0] == "(" and form[1] in DEFINERS):
+            continue
+        names = form[2:] if form[1] == "declare" else [form[2]]
+        for name in names:
+            if not isinstance(name, str):
+                continue
+            out[name] = form[1] == "defn-"
+            if form[1] in ("defrecord", "deftype"):
+                out["->" + name] = False
+                out["map->" + name] = False
+            if form[1] == "defprotocol":
+                for method in form[3:]:
+                    if isinstance(method, list) and method[0] == "(" and isinstance(method[1], str):
+                        out[method[1]] = False
+    return out
+
+
+def symbols_with_namespace(form):
+    for item in form:
+        if isinstance(item, list):
+            yield from symbols_with_namespace(item)
+        elif isinstance(item, str) and "/" in item and not item.startswith((":", "\\")) and len(item) > 1:
+            alias, _, name = item.partition("/")
+            if alias and name:
+                yield alias, name
+
+
+def test_symbols_of_other_namespaces_exist_where_they_are_looked_up():
+    """No compiler has seen these files: every `alias/name` and every :refer that points into another file of the
+    glue must name something that file defines publicly, and, where the reference's sources are at hand, the same
+    for what points into the reference's namespaces (protocols, multimethods, helper functions)."""
+    files = {}
+    for path in GLUE:
+        forms = read_forms(path.read_text())
+        name, aliases, refers = namespace_of(forms)
+        files[name] = (path, forms, aliases, refers, definitions(forms))
+    reference_root = Path("/root/reference/src")
+    reference_cache = {}
+
+    def defined_in(namespace):
+        if namespace in files:
+            return {n for n, private in files[namespace][4].items() if not private}
+        source = reference_root / (namespace.replace(".", "/").replace("-", "_") + ".clj")
+        if not source.exists():
+            return None                      # a library that is not vendored, or no reference on this machine
+        if namespace not in reference_cache:
+            reference_cache[namespace] = {n for n, private in definitions(read_forms(source.read_text())).items() if not private}
+        return reference_cache[namespace]
+
+    checked = 0
+    for name, (path, forms, aliases, refers, _own) in files.items():
+        for sym, target in refers.items():
+            known = defined_in(target)
+            if known is not None:
+                assert sym in known, f"{path.name}: refers to {target}/{sym}, which {target} does not define"
+                checked += 1
+        for alias, sym in set(symbols_with_namespace(forms[1:])):
+            if alias not in aliases:
+                continue                     # a Java class with a static member, or a fully qualified name
+            known = defined_in(aliases[alias])
+            if known is not None:
+                assert sym in known, f"{path.name}: {alias}/{sym} is not defined in {aliases[alias]}"
+                checked += 1
+    assert checked > 20
 
 
 def test_every_entry_point_is_bound():
