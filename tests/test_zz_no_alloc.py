@@ -159,11 +159,12 @@ def test_allocates_nothing_on_a_fresh_stream(pair_factory):
             assert free1.value == free0.value, (free0.value, free1.value)
             want = data.reshape(rows, cols).max(axis=0)
             assert np.array_equal(out.download(), want)
-            # the probe does see an allocation of the size a stream's scratch starts with
+            # the probe does see allocations (a 64 MiB one: the runtime may serve a block as small as a stream's
+            # first scratch, 1 MiB, from a chunk it already holds, depending on what was freed before)
             block = C.c_void_p()
-            capi.call("ct_malloc", C.byref(block), 1 << 20)
+            capi.call("ct_malloc", C.byref(block), 64 << 20)
             capi.call("ct_memory_info", C.byref(free2), C.byref(total))
             capi.call("ct_free", block)
-            assert free2.value < free1.value, "ct_memory_info did not register a 1 MiB allocation"
+            assert free2.value < free1.value, "ct_memory_info did not register a 64 MiB allocation"
         finally:
             capi.call("ct_stream_destroy", fresh)
