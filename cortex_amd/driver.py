@@ -133,7 +133,34 @@ class Event:
             self.handle = None
 
 
+# ct_dims structs of directly addressed dimensions, by (shape, strides): building one costs 2 us of interpreter
+# time, three of them most of what a small call costs from Python.  The library reads a struct during the call
+# only and never writes it, so one struct serves every call with those dimensions, from any thread.
+_DIMS_CACHE: dict = {}
+_DIMS_CACHE_LIMIT = 4096
+
+
 def _dims_struct(dims: dict) -> capi.CtDims:
+    shape_in, strides_in = dims["shape"], dims["strides"]
+    direct = True
+    for entry in shape_in:
+        if type(entry) is not int:
+            direct = False
+            break
+    if direct:
+        key = (tuple(shape_in), tuple(strides_in))
+        try:
+            hit = _DIMS_CACHE.get(key)
+        except TypeError:       # a stride that does not hash: take the long way
+            hit, key = None, None
+        if hit is not None:
+            return hit
+        made = capi.make_dims(shape_in, strides_in, None)
+        if key is not None:
+            if len(_DIMS_CACHE) >= _DIMS_CACHE_LIMIT:
+                _DIMS_CACHE.clear()
+            _DIMS_CACHE[key] = made
+        return made
     shape, index = [], []
     for entry in dims["shape"]:
         if isinstance(entry, (int, np.integer)):
