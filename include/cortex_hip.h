@@ -297,11 +297,12 @@ int ct_unary_reduce(void* stream, void* output, const ct_dims* output_dims, doub
  * than 2 MiB fails with CT_ERR_INVALID and launches nothing.  All calls on one
  * device share the array: calls that overlap in time on one device (two
  * streams, two host threads) race; calls on one stream are ordered and safe.
- * The first call on a device resolves the array's address.  The property is
- * "allocates nothing"; recording the call into a HIP graph has not been tried,
- * and a caller who does so must resolve the address with a call outside the
- * capture first and leave debug-sync mode off (with ct_set_debug_sync(1) every
- * call waits for its stream, which a capture does not allow). */
+ * The first call on a device resolves the array's address.  A caller who
+ * records the call into a HIP graph (hipStreamBeginCapture on the stream it
+ * passes; replayed against the eager results in tests/test_gpu_graph_capture.py)
+ * makes one call outside the capture first, which resolves the address, and
+ * leaves debug-sync mode off (with ct_set_debug_sync(1) every call waits for
+ * its stream, which a capture does not allow). */
 int ct_unary_reduce_noalloc(void* stream, void* output, const ct_dims* output_dims,
                             double input_alpha, const void* input, const ct_dims* input_dims,
                             int op, int dtype);
